@@ -1,0 +1,198 @@
+/*
+ * trips_splat.h -- C ABI of the MI355X-native TRIPS point-splat rasterizer.
+ *
+ * Plain pointers and sizes only; no torch / C++ types cross this boundary.
+ * Every pointer named "device" is a HIP device pointer; every entry point
+ * enqueues its work on the hipStream_t passed as `stream` (given as void* so
+ * that this header needs no HIP include) and returns without synchronising.
+ * Nothing here allocates device memory: the caller passes outputs, a saved-
+ * state buffer and a workspace whose sizes come from the *_size queries.
+ *
+ * The entry points replace, for the pinhole / TILED_BILINEAR_BLEND "new impl"
+ * path of the reference, the following reference interfaces:
+ *
+ *   trips_splat_forward   <- BlendPointCloudForward   (src/lib/rendering/PointRenderer.cu:676-750,1139-1190)
+ *                            + PointRendererCache::RenderFast16 (src/lib/rendering/RenderForward.cu:1065-1394)
+ *   trips_splat_backward  <- BlendPointCloudBackward  (src/lib/rendering/PointRenderer.cu:1232-1427)
+ *                            + PointRendererCache::BlendBackwardsBilinearFast (src/lib/rendering/RenderBackward.cu:621-693)
+ *   trips_adam_step_fused <- torch::optim::MyAdam::step (src/lib/models/MyAdam.cu:164-345)
+ *   trips_apply_tangent   <- ApplyTangentToPose       (src/lib/rendering/PointRenderer.cu:1428-1456)
+ *   TripsView             <- ReducedImageInfo         (src/lib/data/SceneData.h:40-61)
+ *   TripsSplatDesc flags  <- RenderParams             (src/lib/data/Settings.h:19-83)
+ */
+#ifndef TRIPS_SPLAT_H
+#define TRIPS_SPLAT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRIPS_MAX_LAYERS 8 /* max_layers, src/lib/rendering/RenderConstants.h:38 */
+#define TRIPS_MAX_VIEWS 16
+#define TRIPS_ABI_VERSION 1
+
+/* status codes (the reference aborts through SAIGA_ASSERT instead) */
+enum {
+    TRIPS_OK                  = 0,
+    TRIPS_ERR_INVALID_ARG     = 1,
+    TRIPS_ERR_UNSUPPORTED     = 2,
+    TRIPS_ERR_WORKSPACE_SMALL = 3,
+    TRIPS_ERR_HIP             = 4,
+    TRIPS_ERR_LIST_OVERFLOW   = 5 /* reported by trips_splat_check only */
+};
+
+/* How the background is weighted in the forward pass.
+ * REFERENCE : transmittance *before* the last retained entry, as the forward kernel is
+ *             written (src/lib/rendering/RenderForward.cu:1002-1022).
+ * CONSISTENT: transmittance *after* the last retained entry, which is what the
+ *             reference's own backward differentiates (src/lib/rendering/RenderBackward.cu:302-308)
+ *             and what its older kernel computes (src/lib/rendering/RenderForward.cu:2955-2989). */
+enum { TRIPS_BG_REFERENCE = 0, TRIPS_BG_CONSISTENT = 1 };
+
+/* Output image layout. CHW: [B,C,H,W] (reference train==true). HWC: [B,H,W,C] (train==false,
+ * src/lib/rendering/PointRenderer.cu:458-475). */
+enum { TRIPS_LAYOUT_CHW = 0, TRIPS_LAYOUT_HWC = 1 };
+
+/* One rendered view; mirrors ReducedImageInfo (src/lib/data/SceneData.h:40-61).
+ * Only camera_model_type == 0 (PINHOLE_DISTORTION) is supported. */
+typedef struct TripsView {
+    int32_t w, h;
+    int32_t image_index;       /* row of poses_se3 / pose gradient */
+    int32_t camera_index;      /* row of intrinsics */
+    int32_t camera_model_type; /* must be 0 */
+    float crop_transform[5];   /* fx fy cx cy s */
+    float crop_rotation[4];    /* row-major 2x2: r00 r01 r10 r11 */
+} TripsView;
+
+typedef struct TripsSplatDesc {
+    int32_t abi_version;  /* TRIPS_ABI_VERSION */
+    int32_t num_points;   /* N */
+    int32_t num_texels;   /* columns of texture / confidence */
+    int32_t num_channels; /* C: 3, 4, 6, 8 or 16 (RenderForward.cu:1281-1331) */
+    int32_t num_layers;   /* L in 1..8 */
+    int32_t list_depth;   /* K: 8 or 16 (reference fixes 16, PointRenderer.h:178) */
+    int32_t num_views;    /* B in 1..TRIPS_MAX_VIEWS; all views share w,h */
+    int32_t num_images;   /* rows of poses_se3 */
+    int32_t num_cameras;  /* rows of intrinsics */
+    int32_t train;        /* 1: write saved state for backward, honour dropout */
+    int32_t layout;       /* TRIPS_LAYOUT_* of the output images */
+    int32_t floor_layer_sizes; /* 1: h/2 per level ("MultiScaleUnet2d"), 0: ceil (PointRenderer.cu:385-394) */
+    int32_t background_mode;   /* TRIPS_BG_* */
+    int32_t drop_out_points_by_radius;
+    float drop_out_radius_threshold;
+    float dist_cutoff;
+    int32_t viewer_only; /* 1: cull points whose confidence < stability_cutoff_value (RenderForward.cu:122-130,226-230) */
+    float stability_cutoff_value;
+    /* capacity, in entries, of the per-pixel list storage of ONE view; 0 = worst case 4*N*L */
+    int64_t max_list_entries;
+    TripsView views[TRIPS_MAX_VIEWS];
+} TripsSplatDesc;
+
+/* Scene tensors; device pointers, same layouts as the reference's tensors. */
+typedef struct TripsSplatIn {
+    const float* position;    /* [N,4]  xyz + drop-out radius (NeuralPointCloudCuda.cpp:62) */
+    const float* point_size;  /* [N]    raw value; softplus applied inside (RenderForward.cu:248) */
+    const int32_t* index;     /* [N]    column of texture / confidence */
+    const float* texture;     /* [C,T] */
+    const float* confidence;  /* [T]    already sigmoid(10 x) (NeuralTexture.h:40-43) */
+    const float* background;  /* [C] */
+    const double* poses_se3;  /* [F,8]  qx qy qz qw tx ty tz pad, world->camera (NeuralStructure.cpp:20-35) */
+    const float* intrinsics;  /* [Cam,13] fx fy cx cy s + 8 distortion (NeuralStructure.cpp:104-117) */
+    const float* dropout;     /* [B,N] or NULL; a point with value 1 is skipped (RenderForward.cu:240-244) */
+} TripsSplatIn;
+
+typedef struct TripsSplatOut {
+    float* image[TRIPS_MAX_LAYERS]; /* per layer [B,C,H_l,W_l] or [B,H_l,W_l,C] */
+    void* saved;                    /* trips_splat_saved_size bytes; may be NULL when train == 0 */
+} TripsSplatOut;
+
+/* Gradient outputs; the kernels ADD into these, the caller zeroes them first
+ * (PointRendererCache::Build(info,false), PointRenderer.cu:226-272). NULL = not requested, where allowed. */
+typedef struct TripsSplatGrads {
+    float* d_texture;     /* [C,T]   required */
+    float* d_confidence;  /* [T]     required */
+    float* d_background;  /* [C]     required */
+    float* d_position;    /* [N,4]   or NULL (xyz written, .w untouched) */
+    float* d_point_size;  /* [N]     or NULL; NULL also drops the layer factor from d_confidence and
+                                      d_position exactly as RenderBackward.cu:366-372 does */
+    double* d_pose;       /* [F,6]   or NULL; translation first, rotation last */
+    float* d_intrinsics;  /* [Cam,13] or NULL */
+} TripsSplatGrads;
+
+typedef struct TripsCtx TripsCtx;
+
+const char* trips_version(void);
+/* message of the last error raised on the calling thread */
+const char* trips_last_error_string(void);
+
+int trips_ctx_create(TripsCtx** out_ctx, int device);
+int trips_ctx_destroy(TripsCtx* ctx);
+
+/* Layer sizes of the pyramid for desc->width/height rules; w[l], h[l] for l < num_layers. Host only. */
+int trips_splat_layer_sizes(const TripsSplatDesc* desc, int32_t* w, int32_t* h);
+/* Bytes of workspace / saved-state the caller must provide. Host only. */
+int trips_splat_workspace_size(const TripsSplatDesc* desc, size_t* bytes);
+int trips_splat_saved_size(const TripsSplatDesc* desc, size_t* bytes);
+
+int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const void* saved,
+                         const float* const grad_image[TRIPS_MAX_LAYERS], const TripsSplatGrads* grads,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* Synchronises `stream` and reports a device-side list overflow of the last forward that used `workspace`
+ * (only possible when desc->max_list_entries was set below the worst case). */
+int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream);
+
+/* Counters of the last forward of view `view` kept in the saved state: [0]=valid points, [1]=E list entries,
+ * [2]=R retained entries, [3]=P pyramid pixels. Synchronises `stream`. */
+int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view, int64_t counters[4],
+                         void* stream);
+
+/* Debug / parity export: writes for view `view` the sorted, depth-limited per-pixel point-id lists as a dense
+ * [P,K] int32 array (-1 padded; all min(len,K) sorted entries), the per-pixel number of retained entries [P]
+ * (those the blend kept, transmittance >= 0.001) and the per-pixel list length [P] (before the top-K cut).
+ * Pixels are numbered layer by layer, row-major inside a layer. Any of the three may be NULL. */
+int trips_splat_export_lists(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view,
+                             int32_t* device_lists, int32_t* device_retained, int32_t* device_lengths, void* stream);
+
+/* Per-point projection records of view `view` from the saved state, as the reference keeps them in
+ * temp_full_buffer / temp_depth_buffer / temp_max_layer_buffer (RenderForward.cu:1077-1083):
+ * ip [N,2], depth [N] (-1 = culled), size_px [N], max_layer [N]. Any may be NULL. */
+int trips_splat_export_points(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view, float* device_ip,
+                              float* device_depth, float* device_size_px, int32_t* device_max_layer, void* stream);
+
+/* ---- fused Adam over several parameter tensors (MyAdam.cu:41-88) ---- */
+enum { TRIPS_DTYPE_F32 = 0, TRIPS_DTYPE_F64 = 1 };
+
+typedef struct TripsAdamTensor {
+    void* weights;        /* [n] f32 or f64 (master weights, updated in place) */
+    const void* grads;    /* [n] same dtype as weights */
+    float* first_moment;  /* [n] f32 */
+    float* second_moment; /* [n] f32 */
+    int64_t* steps;       /* [n] per-element step counter */
+    int64_t n;
+    int32_t dtype; /* TRIPS_DTYPE_* */
+    float lr;
+    float beta1, beta2, eps;
+    float relative_weight_decay, absolute_weight_decay;
+    float weight_clipping_magnitude; /* 0 = off */
+    float lower_lr_bound, upper_lr_bound; /* 0 and FLT_MAX unless adabound (MyAdam.cu:213-221) */
+    float loss_scale;                     /* 1 (MyAdam.cu:231) */
+} TripsAdamTensor;
+
+/* `tensors` is a HOST array of n_tensors descriptors; one launch covers all of them. */
+int trips_adam_step_fused(TripsCtx* ctx, const TripsAdamTensor* tensors, int n_tensors, void* stream);
+
+/* pose <- se3_exp(t with rotation part * 0.1) * pose; t <- 0   (PointRenderer.cu:1428-1447)
+ * tangent [F,6] f64 device, poses_se3 [F,8] f64 device. */
+int trips_apply_tangent(TripsCtx* ctx, double* tangent, double* poses_se3, int n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRIPS_SPLAT_H */
