@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Headline benchmark: forward + backward + fused Adam of the point splat on the 6M-point / 1920x1080 / 8-layer
+scene, inputs resident in HBM. Prints ONE JSON line.
+
+  python bench.py --gpus 1 --steps K --warmup W
+
+A step is one pass of the hot path over one synthetic view: trips_splat_forward, trips_splat_backward (dL/dimage ~
+N(0,1) on all layers, gradients to position, size, confidence, descriptors, background, pose, intrinsics) and one
+trips_adam_step_fused over position, size, descriptors and confidence. `value` = points / second of that whole step.
+Per-kernel times come from HIP events the library records on the launch stream (trips_profile_*); the roofline
+object is for the kernel with the largest share of the step.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0):
+    """Algorithmic HBM bytes per launch of each kernel, from the run's own counters
+    (N points, E list entries, R retained entries, P pyramid pixels)."""
+    N, E, R, P, C = n_points, c["E"], c["R"], c["P"], channels
+    return {
+        "project_count": 24 * N,                                  # position 16 + size 4 + index 4
+        "scatter_keys": 8 * E,                                    # one 64-bit key written per entry
+        "sort_blend": 8 * E + (20 + 4 + 4 * C + 28) * R + 4 * C * P,  # keys read, record+conf+descriptor, saved, image
+        "blend_backward": 4 * C * P + (76 + 8 * C) * R,
+        "adam_fused": 44 * adam_nonzero + 8 * adam_zero,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--points", type=int, default=6_000_000)
+    ap.add_argument("--cpu-steps", type=int, default=3, help="oracle steps for the cpu_baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across devices",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from trips_amd import abi, scenes
+    from trips_amd.adam import MyAdam
+    from trips_amd.renderer import SplatContext, get_context
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    ctx = get_context(0)
+    dev = ctx.device
+    sc = scenes.config3(n=args.points)
+    desc = abi.desc_for_scene(sc)
+    f = lambda a, dt=torch.float32: torch.as_tensor(np.ascontiguousarray(a), dtype=dt).to(dev).contiguous()
+    t = dict(position=f(sc.position), point_size=f(sc.point_size), index=f(sc.index, torch.int32),
+             texture=f(sc.texture), confidence=f(sc.confidence), background=f(sc.background),
+             poses_se3=f(sc.poses_se3, torch.float64), intrinsics=f(sc.intrinsics), dropout=None)
+    tin = SplatContext.make_in(**t)
+    workspace = ctx.alloc_bytes(ctx.workspace_size(desc))
+    saved = ctx.alloc_bytes(ctx.saved_size(desc))
+    images = ctx.alloc_images(desc)
+    sizes, _, P = abi.pyramid_pixels(desc)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    grad_images = [torch.randn(im.shape, generator=gen, device=dev, dtype=torch.float32) for im in images]
+    N, C = desc.num_points, desc.num_channels
+    grads = dict(d_texture=torch.zeros((C, N), device=dev), d_confidence=torch.zeros(N, device=dev),
+                 d_background=torch.zeros(C, device=dev), d_position=torch.zeros((N, 4), device=dev),
+                 d_point_size=torch.zeros(N, device=dev), d_pose=torch.zeros((1, 6), dtype=torch.float64, device=dev),
+                 d_intrinsics=torch.zeros((1, 13), device=dev))
+    params = [torch.nn.Parameter(t[k]) for k in ("position", "point_size", "texture", "confidence")]
+    gkeys = ("d_position", "d_point_size", "d_texture", "d_confidence")
+    for p, k in zip(params, gkeys):
+        p.grad = grads[k]
+    opt = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+
+    def step():
+        for g in grads.values():
+            g.zero_()
+        ctx.forward(desc, tin, images, saved, workspace)
+        ctx.backward(desc, tin, saved, grad_images, grads, workspace)
+        opt.step()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ctx.check(workspace)
+    counters = ctx.counters(desc, saved, 0)
+    nz = sum(int((grads[k] != 0).sum().item()) for k in gkeys)
+    total_el = sum(int(grads[k].numel()) for k in gkeys)
+
+    ctx.profile_enable(True)
+    ctx.profile_read()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    prof = ctx.profile_read()
+    ctx.profile_enable(False)
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    alg = algorithmic_bytes(counters, N, C, adam_nonzero=nz, adam_zero=total_el - nz)
+    kernels = {}
+    for name, (ms, launches) in prof.items():
+        avg = ms / max(launches, 1)
+        entry = {"avg_ms": round(avg, 4), "launches_per_step": launches / args.steps}
+        if name in alg and avg > 0:
+            entry["alg_bytes"] = int(alg[name])
+            entry["alg_GBs"] = round(alg[name] / (avg * 1e-3) / 1e9, 1)
+        kernels[name] = entry
+    dom = max((k for k in kernels if k in alg), key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
+    achieved = kernels[dom]["alg_GBs"]
+    kernel_ms = sum(v["avg_ms"] * v["launches_per_step"] for v in kernels.values())
+    fwd_bwd_ms = sum(v["avg_ms"] * v["launches_per_step"] for k, v in kernels.items() if k != "adam_fused")
+
+    cpu = None
+    if args.cpu_steps > 0:
+        from tests import oracle_lib
+        oracle = oracle_lib.load()
+        ref = oracle.forward(sc, desc, want_points=False)  # warm-up, also allocates
+        gi = [g.cpu().numpy() for g in grad_images]
+        c0 = time.perf_counter()
+        for _ in range(args.cpu_steps):
+            ref = oracle.forward(sc, desc, want_points=False)
+            oracle.backward(sc, desc, ref, gi)
+        c1 = time.perf_counter()
+        cpu_ms = (c1 - c0) * 1e3 / args.cpu_steps
+        cpu = {"value": round(N / (cpu_ms * 1e-3), 1), "unit": "points/s", "cores": oracle.num_threads(),
+               "kind": "port", "ms_per_step": round(cpu_ms, 1),
+               "sample": f"{args.cpu_steps} forward+backward passes (no Adam) of the same {N}-point 1920x1080 view "
+                         "with the OpenMP C++ oracle"}
+
+    out = {
+        "metric": "splatted points/s fwd+bwd (6M pts, 1080p); frame ms; % HBM peak",
+        "value": round(N / (ms_per_step * 1e-3), 1),
+        "unit": "points/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config3: 6M points (80% noisy ground plane, 20% box), 1920x1080, 8 layers, K=16, "
+                               "4-ch f32 descriptors; forward + backward + fused Adam, 1 view",
+                   "points": N, "width": sc.width, "height": sc.height, "layers": desc.num_layers,
+                   "list_depth": desc.list_depth, "counters": counters},
+        "frame_ms": {"fwd_bwd_kernels": round(fwd_bwd_ms, 4), "all_kernels": round(kernel_ms, 4),
+                     "wall_per_step": round(ms_per_step, 4)},
+        "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
+                                  HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
+        "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+        "kernels": kernels,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -192,6 +192,16 @@ int trips_adam_step_fused(TripsCtx* ctx, const TripsAdamTensor* tensors, int n_t
  * tangent [F,6] f64 device, poses_se3 [F,8] f64 device. */
 int trips_apply_tangent(TripsCtx* ctx, double* tangent, double* poses_se3, int n, void* stream);
 
+/* ---- per-kernel timing (stands in for the reference's CudaTimerSystem scopes "Count Render", "Splat",
+ * "FastSortAndBlendMore", "BlendBackwardsBilinearFast"; RenderForward.cu:1090,1238,1271, PointRenderer.cu:1338) ----
+ * While enabled, every kernel the library launches through `ctx` is bracketed by HIP events on its stream.
+ * trips_profile_read waits for those events, returns per kernel name the summed milliseconds and the number of
+ * launches since the last read, and resets the accumulation. names[i] point to static strings. */
+#define TRIPS_PROFILE_MAX_KERNELS 16
+int trips_profile_enable(TripsCtx* ctx, int enabled);
+int trips_profile_read(TripsCtx* ctx, int* n, const char* names[TRIPS_PROFILE_MAX_KERNELS],
+                       float ms[TRIPS_PROFILE_MAX_KERNELS], int launches[TRIPS_PROFILE_MAX_KERNELS]);
+
 #ifdef __cplusplus
 }
 #endif

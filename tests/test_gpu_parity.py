@@ -1,0 +1,206 @@
+"""Parity of the HIP path (called through the C ABI) with the CPU oracle on the same seeded inputs.
+
+Bars: per-point records and per-pixel index lists bit-exact; forward images within 1e-5 relative;
+gradients within 1e-4 of the largest gradient magnitude (float atomics sum in a different order)."""
+import numpy as np
+import pytest
+
+from trips_amd import abi, scenes
+
+pytestmark = pytest.mark.gpu
+
+IMG_RTOL = 1e-5
+GRAD_RTOL = 1e-4
+
+
+def _check_forward(oracle, sc, desc, dropout=None, views=None):
+    from tests.gpu_util import GpuRun
+    ref = oracle.forward(sc, desc, dropout=dropout)
+    run = GpuRun(sc, desc, dropout=dropout)
+    imgs = run.forward()
+    for l, (a, b) in enumerate(zip(imgs, ref["images"])):
+        assert not np.isnan(a).any(), f"layer {l}: unwritten pixels"
+        np.testing.assert_allclose(a, b, rtol=IMG_RTOL, atol=1e-6, err_msg=f"layer {l}")
+    if desc.train:
+        for b in range(desc.num_views):
+            lists, retained, lengths = run.lists(b)
+            np.testing.assert_array_equal(lengths, ref["lengths"][b])
+            np.testing.assert_array_equal(lists, ref["lists"][b])
+            np.testing.assert_array_equal(retained, ref["retained"][b])
+            ip, depth, size_px, max_layer = run.points(b)
+            np.testing.assert_array_equal(depth, ref["depth"][b])
+            np.testing.assert_array_equal(ip, ref["ip"][b])
+            np.testing.assert_array_equal(size_px, ref["size_px"][b])
+            np.testing.assert_array_equal(max_layer, ref["max_layer"][b])
+            c = run.ctx.counters(desc, run.saved, b)
+            assert [c["valid"], c["E"], c["R"], c["P"]] == list(ref["counters"][b])
+    return run, ref, imgs
+
+
+@pytest.mark.parametrize("L,K,bg", [(1, 16, 0), (3, 8, 0), (4, 16, 1), (8, 16, 0)])
+def test_forward_small(oracle, L, K, bg):
+    sc = scenes.tiny(n=4000, w=70, h=50, f=60.0, num_layers=L, list_depth=K, seed=100 + L, radius=(0.004, 0.5))
+    d = abi.desc_for_scene(sc, background_mode=bg)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert ref["lengths"].max() > 16
+
+
+def test_forward_views_crop_dropout(oracle):
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=7, views=3)
+    sc.views[1]["crop_transform"] = (1.5, 1.25, -10.0, 4.0, 0.0)
+    th = 0.3
+    sc.views[2]["crop_rotation"] = (float(np.cos(th)), float(-np.sin(th)), float(np.sin(th)), float(np.cos(th)))
+    sc.intrinsics[0, 4] = 0.5
+    d = abi.desc_for_scene(sc)
+    drop = (np.random.default_rng(0).random((3, 3000)) < 0.3).astype(np.float32)
+    _check_forward(oracle, sc, d, dropout=drop)
+
+
+def test_forward_eval_layout_and_viewer_cull(oracle):
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=8)
+    d = abi.desc_for_scene(sc, train=False, viewer_only=True, stability_cutoff_value=0.4)
+    assert d.layout == abi.TRIPS_LAYOUT_HWC
+    _check_forward(oracle, sc, d)
+
+
+def test_forward_radius_dropout_and_floor_layers(oracle):
+    sc = scenes.tiny(n=3000, w=63, h=47, f=60.0, num_layers=4, list_depth=16, seed=9, radius=(0.004, 0.3))
+    d = abi.desc_for_scene(sc, drop_out_points_by_radius=True, drop_out_radius_threshold=2.0, floor_layer_sizes=True)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert 0 < ref["counters"][0, 0] < 3000
+
+
+def test_forward_distortion(oracle):
+    # non-zero distortion: parity with Saiga's model is unpinned; this checks HIP == oracle for the restated model
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=10)
+    sc.intrinsics[0, 5:] = [0.1, -0.05, 0.01, 0.02, 0.01, -0.005, 0.003, -0.002]
+    d = abi.desc_for_scene(sc, dist_cutoff=0.45)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert 0 < ref["counters"][0, 0] < 3000
+
+
+@pytest.mark.parametrize("channels", [3, 6, 8, 16])
+def test_forward_other_channel_counts(oracle, channels):
+    sc = scenes.tiny(n=2000, w=48, h=40, f=45.0, num_layers=3, list_depth=16, seed=20 + channels, channels=channels)
+    d = abi.desc_for_scene(sc)
+    _check_forward(oracle, sc, d)
+
+
+def test_forward_edge_cases(oracle):
+    # all points behind the camera -> pure background; a single point; ties in depth
+    sc = scenes.tiny(n=5, w=16, h=12, f=30.0, num_layers=3, seed=8)
+    sc.position[:, 2] = -100.0
+    _check_forward(oracle, sc, abi.desc_for_scene(sc))
+    sc = scenes.tiny(n=40, w=16, h=16, f=30.0, num_layers=1, list_depth=16, seed=2)
+    sc.position[:, :3] = [0.01, 0.01, 0.0]  # 40 coincident points: tie-break by id, top-16 of 40
+    run, ref, _ = _check_forward(oracle, sc, abi.desc_for_scene(sc))
+    lists, _, _ = run.lists(0)
+    np.testing.assert_array_equal(lists[8 * 16 + 8], np.arange(16))
+
+
+def test_transmittance_cutoff_matches(oracle):
+    n = 12
+    sc = scenes.tiny(n=n, w=16, h=16, f=30.0, num_layers=1, list_depth=16, seed=3, background=0.5)
+    sc.position[:, :3] = [[0.0, 0.0, 0.1 * i] for i in range(n)]
+    sc.confidence[:] = 0.95
+    sc.point_size[:] = scenes.inverse_softplus((3.0 + 0.1 * np.arange(n)) / 30.0)
+    for mode in (0, 1):
+        run, ref, _ = _check_forward(oracle, sc, abi.desc_for_scene(sc, background_mode=mode))
+        assert ref["retained"][0][8 * 16 + 8] == 3
+
+
+def _check_backward(oracle, sc, desc, seed=0, **want):
+    from tests.gpu_util import GpuRun, rel_err
+    ref = oracle.forward(sc, desc)
+    rng = np.random.default_rng(seed)
+    shape = (lambda w, h: (desc.num_views, desc.num_channels, h, w)) if desc.layout == abi.TRIPS_LAYOUT_CHW else \
+        (lambda w, h: (desc.num_views, h, w, desc.num_channels))
+    grads = [rng.normal(0, 1, shape(w, h)).astype(np.float32) for (w, h) in ref["sizes"]]
+    g_ref = oracle.backward(sc, desc, ref, grads, **want)
+    run = GpuRun(sc, desc)
+    run.forward()
+    g = run.backward(grads, **want)
+    errs = {}
+    for k, v in g_ref.items():
+        if v is None:
+            assert g[k] is None
+            continue
+        errs[k] = rel_err(g[k], v)
+        assert errs[k] < GRAD_RTOL, f"{k}: {errs[k]:.3e}"
+    return errs, g, g_ref
+
+
+@pytest.mark.parametrize("L,K,bg", [(1, 16, 1), (3, 8, 0), (4, 16, 1), (8, 16, 0)])
+def test_backward_small(oracle, L, K, bg):
+    radius = (0.004, 0.5) if L > 1 else (0.004, 0.03)
+    sc = scenes.tiny(n=4000, w=70, h=50, f=60.0, num_layers=L, list_depth=K, seed=200 + L, radius=radius)
+    sc.confidence = (sc.confidence ** 0.3).astype(np.float32)
+    sc.intrinsics[0, 4] = 0.7
+    d = abi.desc_for_scene(sc, background_mode=bg)
+    errs, g, _ = _check_backward(oracle, sc, d)
+    assert np.abs(g["d_pose"]).max() > 0 and np.abs(g["d_intrinsics"]).max() > 0
+
+
+def test_backward_views_crop_distortion_optional_outputs(oracle):
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=31, views=2)
+    sc.views[1]["crop_transform"] = (1.5, 1.25, -10.0, 4.0, 0.0)
+    th = 0.3
+    sc.views[1]["crop_rotation"] = (float(np.cos(th)), float(-np.sin(th)), float(np.sin(th)), float(np.cos(th)))
+    sc.intrinsics[0, 5:] = [0.1, -0.05, 0.01, 0.02, 0.01, -0.005, 0.003, -0.002]
+    d = abi.desc_for_scene(sc)
+    _check_backward(oracle, sc, d)
+    _check_backward(oracle, sc, d, want_point_size=False)
+    _check_backward(oracle, sc, d, want_position=False, want_pose=False, want_intrinsics=False)
+
+
+def test_config1_forward_full(oracle):
+    sc = scenes.config1()
+    _check_forward(oracle, sc, abi.desc_for_scene(sc, train=True))
+    _check_forward(oracle, sc, abi.desc_for_scene(sc, train=False))
+
+
+def test_config2_forward_backward_full(oracle):
+    sc = scenes.config2()
+    d = abi.desc_for_scene(sc)
+    _check_forward(oracle, sc, d)
+    _check_backward(oracle, sc, d, seed=2)
+
+
+def test_config4_contention_reduced(oracle):
+    # same shape as the contention config (64 tight clusters, 4 views, K = 16) at a tenth of the points
+    sc = scenes.config4(n=400_000)
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert ref["lengths"].max() > 200
+    _check_backward(oracle, sc, d, seed=4)
+
+
+def test_list_overflow_is_reported(oracle):
+    from tests.gpu_util import GpuRun
+    from trips_amd._lib import TripsError
+    sc = scenes.tiny(n=4000, w=70, h=50, f=60.0, num_layers=3, list_depth=16, seed=103)
+    d_ok = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d_ok)
+    E = int(ref["counters"][0, 1])
+    run = GpuRun(sc, abi.desc_for_scene(sc, max_list_entries=E))
+    run.forward()
+    run.ctx.check(run.workspace)  # exactly enough: fine
+    run = GpuRun(sc, abi.desc_for_scene(sc, max_list_entries=E // 2))
+    run.forward()
+    with pytest.raises(TripsError) as ei:
+        run.ctx.check(run.workspace)
+    assert ei.value.code == abi.TRIPS_ERR_LIST_OVERFLOW
+
+
+def test_forward_is_deterministic_and_repeatable(oracle):
+    from tests.gpu_util import GpuRun
+    sc = scenes.tiny(n=20000, w=160, h=120, f=120.0, num_layers=5, list_depth=16, seed=77)
+    run = GpuRun(sc, abi.desc_for_scene(sc))
+    a = run.forward()
+    la = run.lists(0)
+    b = run.forward()
+    lb = run.lists(0)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+    for x, y in zip(la, lb):
+        np.testing.assert_array_equal(x, y)

@@ -1,0 +1,280 @@
+// Fused multi-tensor Adam, pose update, and the small export / reduction kernels of the C ABI (gfx950).
+//
+//   adam_fused_kernel    <- adam_step      src/lib/models/MyAdam.cu:41-88 (one launch for all tensors instead of
+//                                          one 128-thread launch per tensor, :226-288)
+//   apply_tangent_kernel <- ApplyTangent   src/lib/rendering/PointRenderer.cu:1428-1447
+#include <float.h>
+
+#include "splat_internal.h"
+#include "trips_math.h"
+
+#pragma clang fp contract(off)
+
+namespace trips
+{
+constexpr int kAdamMaxTensors = 16;
+constexpr int kAdamPerBlock   = 1024;  // 256 threads x 4 consecutive elements
+
+struct AdamTable
+{
+    TripsAdamTensor t[kAdamMaxTensors];
+    long long block_start[kAdamMaxTensors + 1];
+    int32_t vec_ok[kAdamMaxTensors];
+    int32_t n;
+};
+
+struct AdamScalars
+{
+    float lr, beta1, beta2, eps, rel_wd, abs_wd, clip, lo, hi, loss_scale;
+};
+
+__device__ __forceinline__ bool adam_element(const AdamScalars& h, float gradient_raw, float weight_fp, float& m,
+                                             float& v, long long& step, float& new_weight)
+{
+    float gradient = gradient_raw / h.loss_scale;
+    if (gradient == 0.f) return false;  // parameter not seen in this step (MyAdam.cu:57-61)
+    const float gradient_sq   = gradient * gradient;
+    const float first_moment  = h.beta1 * m + (1 - h.beta1) * gradient;
+    const float second_moment = h.beta2 * v + (1 - h.beta2) * gradient_sq;
+    m                         = first_moment;
+    v                         = second_moment;
+    step                      = step + 1;
+    const uint32_t current_step = (uint32_t)step;
+    float learning_rate         = h.lr;
+    learning_rate *= sqrtf(1 - powf(h.beta2, (float)current_step)) / (1 - powf(h.beta1, (float)current_step));
+    const float effective_learning_rate =
+        fminf(fmaxf(learning_rate / (sqrtf(second_moment) + h.eps), h.lo), h.hi);
+    const float rel            = h.rel_wd * learning_rate;
+    const float ab             = h.abs_wd * learning_rate;
+    const float decayed_weight = (1 - rel) * weight_fp - copysignf(ab, weight_fp);
+    float w                    = decayed_weight - effective_learning_rate * first_moment;
+    if (h.clip != 0.0f)
+    {
+        const float lo = -h.clip, hi = h.clip;
+        w = w < lo ? lo : (hi < w ? hi : w);
+    }
+    new_weight = w;
+    return true;
+}
+
+__global__ __launch_bounds__(256) void adam_fused_kernel(const AdamTable tab)
+{
+    int ti = 0;
+    while (ti + 1 < tab.n && (long long)blockIdx.x >= tab.block_start[ti + 1]) ++ti;
+    const TripsAdamTensor& T = tab.t[ti];
+    const AdamScalars h      = {T.lr, T.beta1, T.beta2, T.eps, T.relative_weight_decay, T.absolute_weight_decay,
+                                T.weight_clipping_magnitude, T.lower_lr_bound, T.upper_lr_bound, T.loss_scale};
+    const long long i0 = ((long long)blockIdx.x - tab.block_start[ti]) * kAdamPerBlock + (long long)threadIdx.x * 4;
+    if (i0 >= T.n) return;
+    float* mo      = T.first_moment;
+    float* vo      = T.second_moment;
+    long long* st  = reinterpret_cast<long long*>(T.steps);
+
+    if (T.dtype == TRIPS_DTYPE_F32 && tab.vec_ok[ti] && i0 + 4 <= T.n)
+    {
+        float* w       = reinterpret_cast<float*>(T.weights);
+        const float* g = reinterpret_cast<const float*>(T.grads);
+        const float4 g4 = *reinterpret_cast<const float4*>(g + i0);
+        if (g4.x == 0.f && g4.y == 0.f && g4.z == 0.f && g4.w == 0.f) return;
+        float4 w4 = *reinterpret_cast<const float4*>(w + i0);
+        float4 m4 = *reinterpret_cast<const float4*>(mo + i0);
+        float4 v4 = *reinterpret_cast<const float4*>(vo + i0);
+        longlong2 s01 = *reinterpret_cast<const longlong2*>(st + i0);
+        longlong2 s23 = *reinterpret_cast<const longlong2*>(st + i0 + 2);
+        float nw;
+        if (adam_element(h, g4.x, w4.x, m4.x, v4.x, s01.x, nw)) w4.x = nw;
+        if (adam_element(h, g4.y, w4.y, m4.y, v4.y, s01.y, nw)) w4.y = nw;
+        if (adam_element(h, g4.z, w4.z, m4.z, v4.z, s23.x, nw)) w4.z = nw;
+        if (adam_element(h, g4.w, w4.w, m4.w, v4.w, s23.y, nw)) w4.w = nw;
+        *reinterpret_cast<float4*>(w + i0)        = w4;
+        *reinterpret_cast<float4*>(mo + i0)       = m4;
+        *reinterpret_cast<float4*>(vo + i0)       = v4;
+        *reinterpret_cast<longlong2*>(st + i0)     = s01;
+        *reinterpret_cast<longlong2*>(st + i0 + 2) = s23;
+        return;
+    }
+    for (int k = 0; k < 4; ++k)
+    {
+        const long long i = i0 + k;
+        if (i >= T.n) break;
+        float gr, wf;
+        if (T.dtype == TRIPS_DTYPE_F64)
+        {
+            gr = (float)reinterpret_cast<const double*>(T.grads)[i];
+            wf = (float)reinterpret_cast<double*>(T.weights)[i];
+        }
+        else
+        {
+            gr = reinterpret_cast<const float*>(T.grads)[i];
+            wf = reinterpret_cast<float*>(T.weights)[i];
+        }
+        float m = mo[i], v = vo[i], nw;
+        long long s = st[i];
+        if (adam_element(h, gr, wf, m, v, s, nw))
+        {
+            mo[i] = m;
+            vo[i] = v;
+            st[i] = s;
+            if (T.dtype == TRIPS_DTYPE_F64)
+                reinterpret_cast<double*>(T.weights)[i] = nw;
+            else
+                reinterpret_cast<float*>(T.weights)[i] = nw;
+        }
+    }
+}
+
+hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_t stream, Profiler* prof)
+{
+    ProfScope ps(prof, "adam_fused", stream);
+    int done = 0;
+    while (done < n_tensors)
+    {
+        AdamTable tab;
+        tab.n           = 0;
+        long long block = 0;
+        while (done < n_tensors && tab.n < kAdamMaxTensors)
+        {
+            const TripsAdamTensor& T = tensors[done++];
+            if (T.n <= 0) continue;
+            tab.t[tab.n]           = T;
+            tab.block_start[tab.n] = block;
+            auto al16              = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+            tab.vec_ok[tab.n] = al16(T.weights) && al16(T.grads) && al16(T.first_moment) && al16(T.second_moment) &&
+                                al16(T.steps);
+            block += (T.n + kAdamPerBlock - 1) / kAdamPerBlock;
+            tab.n += 1;
+        }
+        tab.block_start[tab.n] = block;
+        if (tab.n == 0 || block == 0) continue;
+        if (block > 0x7fffffffll) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(adam_fused_kernel, dim3((unsigned)block), dim3(256), 0, stream, tab);
+    }
+    return hipGetLastError();
+}
+
+// pose <- se3_exp(t with rotation * 0.1) * pose; t <- 0. Sophus' exp restated (quaternion half-angle form,
+// V = I + (1-cos)/th^2 W + (th-sin)/th^3 W^2, first-order renormalisation of the product quaternion).
+__global__ __launch_bounds__(128) void apply_tangent_kernel(double* tangent, double* poses, int n)
+{
+    const int i = blockIdx.x * 128 + threadIdx.x;
+    if (i >= n) return;
+    double* t = tangent + 6 * (size_t)i;
+    double* p = poses + 8 * (size_t)i;
+    const double u[3] = {t[0], t[1], t[2]};
+    const double w[3] = {t[3] * 0.1, t[4] * 0.1, t[5] * 0.1};
+    const double th2  = w[0] * w[0] + w[1] * w[1] + w[2] * w[2];
+    const double th   = sqrt(th2);
+    double imag, real;
+    if (th < 1e-10)
+    {
+        const double th4 = th2 * th2;
+        imag             = 0.5 - th2 / 48.0 + th4 / 3840.0;
+        real             = 1.0 - th2 / 8.0 + th4 / 384.0;
+    }
+    else
+    {
+        imag = sin(0.5 * th) / th;
+        real = cos(0.5 * th);
+    }
+    const double x1 = imag * w[0], y1 = imag * w[1], z1 = imag * w[2], w1 = real;
+    const double W[9] = {0, -w[2], w[1], w[2], 0, -w[0], -w[1], w[0], 0};
+    double W2[9];
+    for (int r = 0; r < 3; ++r)
+        for (int c = 0; c < 3; ++c)
+        {
+            double s = 0;
+            for (int k = 0; k < 3; ++k) s += W[3 * r + k] * W[3 * k + c];
+            W2[3 * r + c] = s;
+        }
+    const double R1[9] = {1 - 2 * (y1 * y1 + z1 * z1), 2 * (x1 * y1 - z1 * w1),     2 * (x1 * z1 + y1 * w1),
+                          2 * (x1 * y1 + z1 * w1),     1 - 2 * (x1 * x1 + z1 * z1), 2 * (y1 * z1 - x1 * w1),
+                          2 * (x1 * z1 - y1 * w1),     2 * (y1 * z1 + x1 * w1),     1 - 2 * (x1 * x1 + y1 * y1)};
+    double Vm[9];
+    if (th < 1e-10)
+    {
+        for (int k = 0; k < 9; ++k) Vm[k] = R1[k];
+    }
+    else
+    {
+        const double a = (1 - cos(th)) / th2, b = (th - sin(th)) / (th2 * th);
+        for (int k = 0; k < 9; ++k) Vm[k] = (k % 4 == 0 ? 1.0 : 0.0) + a * W[k] + b * W2[k];
+    }
+    double t1[3];
+    for (int r = 0; r < 3; ++r) t1[r] = Vm[3 * r] * u[0] + Vm[3 * r + 1] * u[1] + Vm[3 * r + 2] * u[2];
+    const double x2 = p[0], y2 = p[1], z2 = p[2], w2 = p[3];
+    double q[4] = {w1 * x2 + x1 * w2 + y1 * z2 - z1 * y2, w1 * y2 - x1 * z2 + y1 * w2 + z1 * x2,
+                   w1 * z2 + x1 * y2 - y1 * x2 + z1 * w2, w1 * w2 - x1 * x2 - y1 * y2 - z1 * z2};
+    const double sn = q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3];
+    if (sn != 1.0)
+    {
+        const double sc = 2.0 / (1.0 + sn);
+        for (int k = 0; k < 4; ++k) q[k] *= sc;
+    }
+    double tn[3];
+    for (int r = 0; r < 3; ++r) tn[r] = t1[r] + R1[3 * r] * p[4] + R1[3 * r + 1] * p[5] + R1[3 * r + 2] * p[6];
+    for (int k = 0; k < 4; ++k) p[k] = q[k];
+    for (int k = 0; k < 3; ++k) p[4 + k] = tn[k];
+    for (int k = 0; k < 6; ++k) t[k] = 0.0;
+}
+
+hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(apply_tangent_kernel, dim3((n + 127) / 128), dim3(128), 0, stream, tangent, poses, n);
+    return hipGetLastError();
+}
+
+// ---- exports from the saved state ----
+__global__ __launch_bounds__(256) void export_points_kernel(const float* __restrict__ rec, int rec_floats, int n,
+                                                            float* ip, float* depth, float* size_px,
+                                                            int32_t* max_layer)
+{
+    const int pid = blockIdx.x * 256 + threadIdx.x;
+    if (pid >= n) return;
+    const float* r  = rec + (size_t)pid * rec_floats;
+    const float4 tl = *reinterpret_cast<const float4*>(r + rec_floats - 4);  // {tex, depth, max_layer, -}
+    const bool ok   = tl.y > 0.f;
+    if (ip)
+    {
+        ip[2 * (size_t)pid]     = ok ? r[0] : 0.f;
+        ip[2 * (size_t)pid + 1] = ok ? r[1] : 0.f;
+    }
+    if (depth) depth[pid] = tl.y;
+    if (size_px) size_px[pid] = ok ? r[2] : 0.f;
+    if (max_layer) max_layer[pid] = ok ? __float_as_int(tl.z) : 0;
+}
+
+hipError_t launch_export_points(const float* rec, int rec_floats, int n, float* ip, float* depth, float* size_px,
+                                int32_t* max_layer, hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(export_points_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, rec, rec_floats, n, ip,
+                       depth, size_px, max_layer);
+    return hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void sum_i32_kernel(const int32_t* __restrict__ v, long long n,
+                                                      unsigned long long* out)
+{
+    __shared__ unsigned long long s[4];
+    unsigned long long acc = 0;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+        acc += (unsigned long long)(unsigned)v[i];
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+    if ((threadIdx.x & 63) == 0) s[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(out, s[0] + s[1] + s[2] + s[3]);
+}
+
+hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream)
+{
+    hipError_t e = hipMemsetAsync(out, 0, sizeof(unsigned long long), stream);
+    if (e != hipSuccess) return e;
+    if (n <= 0) return hipSuccess;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(sum_i32_kernel, dim3(blocks), dim3(256), 0, stream, v, n, out);
+    return hipGetLastError();
+}
+
+}  // namespace trips

@@ -1,0 +1,191 @@
+// Internal structures shared by the host-side C ABI and the HIP kernels of the splat path.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/trips_splat.h"
+
+#include <vector>
+
+namespace trips
+{
+// Optional HIP-event bracket around every kernel launch (host side only).
+struct Profiler
+{
+    struct Span
+    {
+        const char* name;
+        hipEvent_t a, b;
+    };
+    bool enabled = false;
+    std::vector<Span> spans;
+    std::vector<hipEvent_t> pool;
+
+    hipEvent_t get_event()
+    {
+        if (!pool.empty())
+        {
+            hipEvent_t e = pool.back();
+            pool.pop_back();
+            return e;
+        }
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) return nullptr;
+        return e;
+    }
+    void begin(const char* name, hipStream_t s)
+    {
+        if (!enabled) return;
+        Span sp{name, get_event(), get_event()};
+        if (!sp.a || !sp.b) return;
+        (void)hipEventRecord(sp.a, s);
+        spans.push_back(sp);
+    }
+    void end(hipStream_t s)
+    {
+        if (!enabled || spans.empty()) return;
+        (void)hipEventRecord(spans.back().b, s);
+    }
+    ~Profiler()
+    {
+        for (auto& sp : spans)
+        {
+            (void)hipEventDestroy(sp.a);
+            (void)hipEventDestroy(sp.b);
+        }
+        for (auto e : pool) (void)hipEventDestroy(e);
+    }
+};
+
+struct ProfScope
+{
+    Profiler* p;
+    hipStream_t s;
+    ProfScope(Profiler* p_, const char* name, hipStream_t s_) : p(p_), s(s_)
+    {
+        if (p) p->begin(name, s);
+    }
+    ~ProfScope()
+    {
+        if (p) p->end(s);
+    }
+};
+
+// Per-point record written by the projection pass and gathered by blend / backward.
+// First 4 + Cpad floats: {ip.x, ip.y, size_px, confidence, descriptor[0..C)} -- everything the blend needs,
+// one aligned gather instead of three scattered reads (reference: 5-float record + confidence + [C,N] texture,
+// src/lib/rendering/RenderForward.cu:875-899,952). In train mode 8 more floats follow for the backward:
+// {view.x, view.y, view.z, softplus'(raw size), texture index, depth (-1 = culled), layers written, -}.
+__host__ __device__ inline int record_floats(int channels, bool train)
+{
+    int cpad = (channels + 3) & ~3;
+    return 4 + cpad + (train ? 8 : 0);
+}
+
+struct PyramidGeom
+{
+    int32_t num_layers;
+    int32_t w[TRIPS_MAX_LAYERS];
+    int32_t h[TRIPS_MAX_LAYERS];
+    int32_t off[TRIPS_MAX_LAYERS + 1];  // first pixel number of each layer; off[L] = P
+};
+
+// Header at the start of each view's saved state (and of the workspace status block).
+struct ViewHeader
+{
+    unsigned long long n_valid;     // points that passed the validity test
+    unsigned long long n_entries;   // E: total list entries (from the scan)
+    unsigned long long overflow;    // entries dropped because the list storage was too small
+    unsigned long long reserved[5];
+};
+
+// Layout of one view's saved state (all offsets in bytes, 256-aligned)
+struct SavedLayout
+{
+    size_t header;    // ViewHeader
+    size_t rec;       // float [N * record_floats]
+    size_t lists;     // int32 [P, K]
+    size_t retained;  // int32 [P]
+    size_t lengths;   // int32 [P]
+    size_t bytes_per_view;
+};
+
+struct WorkspaceLayout
+{
+    size_t ptk;         // float4 [N]   {ip.x, ip.y, depth (-1 culled), max_layer bits}
+    size_t counts;      // int32 [P]
+    size_t cursor;      // int32 [P]
+    size_t block_sums;  // int32 [scan blocks + 1]
+    size_t keys;        // uint64 [capacity]
+    size_t capacity;    // entries
+    size_t bytes;
+};
+
+constexpr int kScanTile = 4096;  // elements per scan block (256 threads x 16)
+
+inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
+struct ForwardParams
+{
+    // scene
+    const float4* position;
+    const float* point_size;
+    const int32_t* index;
+    const float* texture;
+    const float* confidence;
+    const float* background;
+    const double* pose;      // 8 doubles of this view's image
+    const float* intrinsics; // 13 floats of this view's camera
+    const float* dropout;    // this view's row or nullptr
+    // geometry
+    PyramidGeom geom;
+    TripsView view;
+    int32_t num_points, num_texels, num_layers, list_depth;
+    int32_t view_index, num_views;
+    int32_t layout, background_mode;
+    int32_t drop_out_points_by_radius, viewer_only;
+    float drop_out_radius_threshold, dist_cutoff, stability_cutoff_value;
+    // buffers
+    float4* ptk;
+    int32_t* counts;
+    int32_t* cursor;
+    int32_t* block_sums;
+    unsigned long long* keys;
+    long long capacity;
+    float* rec;
+    int32_t rec_floats;
+    int32_t* lists;
+    int32_t* retained;
+    int32_t* lengths;
+    ViewHeader* header;  // counters of this view
+    ViewHeader* status;  // overflow flag of the whole forward call (start of the workspace)
+    float* image[TRIPS_MAX_LAYERS];
+};
+
+struct BackwardParams
+{
+    const float* background;
+    const double* pose;
+    const float* intrinsics;
+    const float* point_size;
+    PyramidGeom geom;
+    TripsView view;
+    int32_t num_points, num_texels, num_layers, list_depth;
+    int32_t view_index, num_views, layout;
+    float dist_cutoff;
+    const float* rec;
+    int32_t rec_floats;
+    const int32_t* lists;
+    const int32_t* retained;
+    const float* grad_image[TRIPS_MAX_LAYERS];
+    float* d_texture;
+    float* d_confidence;
+    float* d_background;
+    float* d_position;
+    float* d_point_size;
+    double* d_pose;       // row of this view's image or nullptr
+    float* d_intrinsics;  // row of this view's camera or nullptr
+};
+
+}  // namespace trips

@@ -1,0 +1,554 @@
+// Host side of the C ABI declared in include/trips_splat.h: argument checks, buffer carving, launches.
+// Nothing here allocates device memory or synchronises, except the calls documented as synchronising
+// (trips_splat_check, trips_splat_counters).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "splat_internal.h"
+
+namespace trips
+{
+hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train, bool first_view, hipStream_t stream,
+                               Profiler* prof);
+hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof);
+hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_t stream, Profiler* prof);
+hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t stream);
+hipError_t launch_export_points(const float* rec, int rec_floats, int n, float* ip, float* depth, float* size_px,
+                                int32_t* max_layer, hipStream_t stream);
+hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream);
+}  // namespace trips
+
+using namespace trips;
+
+struct TripsCtx
+{
+    int device;
+    Profiler prof;
+};
+
+namespace
+{
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    return fail(TRIPS_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool channels_ok(int c) { return c == 3 || c == 4 || c == 6 || c == 8 || c == 16; }
+
+int check_desc(const TripsSplatDesc* d)
+{
+    if (!d) return fail(TRIPS_ERR_INVALID_ARG, "desc is NULL");
+    if (d->abi_version != TRIPS_ABI_VERSION)
+        return fail(TRIPS_ERR_INVALID_ARG, "abi_version %d, library has %d", d->abi_version, TRIPS_ABI_VERSION);
+    if (d->num_points < 0) return fail(TRIPS_ERR_INVALID_ARG, "num_points < 0");
+    if (d->num_texels < 0) return fail(TRIPS_ERR_INVALID_ARG, "num_texels < 0");
+    if (!channels_ok(d->num_channels))
+        return fail(TRIPS_ERR_UNSUPPORTED, "num_channels %d not in {3,4,6,8,16}", d->num_channels);
+    if (d->num_layers < 1 || d->num_layers > TRIPS_MAX_LAYERS)
+        return fail(TRIPS_ERR_INVALID_ARG, "num_layers %d not in 1..%d", d->num_layers, TRIPS_MAX_LAYERS);
+    if (d->list_depth != 8 && d->list_depth != 16)
+        return fail(TRIPS_ERR_UNSUPPORTED, "list_depth %d not in {8,16}", d->list_depth);
+    if (d->num_views < 1 || d->num_views > TRIPS_MAX_VIEWS)
+        return fail(TRIPS_ERR_INVALID_ARG, "num_views %d not in 1..%d", d->num_views, TRIPS_MAX_VIEWS);
+    if (d->num_images < 1 || d->num_cameras < 1) return fail(TRIPS_ERR_INVALID_ARG, "num_images / num_cameras < 1");
+    if (d->layout != TRIPS_LAYOUT_CHW && d->layout != TRIPS_LAYOUT_HWC) return fail(TRIPS_ERR_INVALID_ARG, "layout");
+    if (d->background_mode != TRIPS_BG_REFERENCE && d->background_mode != TRIPS_BG_CONSISTENT)
+        return fail(TRIPS_ERR_INVALID_ARG, "background_mode");
+    if (d->max_list_entries < 0) return fail(TRIPS_ERR_INVALID_ARG, "max_list_entries < 0");
+    const int w = d->views[0].w, h = d->views[0].h;
+    if (w < 1 || h < 1 || w > 32768 || h > 32768) return fail(TRIPS_ERR_INVALID_ARG, "view size %dx%d", w, h);
+    for (int b = 0; b < d->num_views; ++b)
+    {
+        const TripsView& v = d->views[b];
+        if (v.w != w || v.h != h) return fail(TRIPS_ERR_INVALID_ARG, "views must share one size");
+        if (v.camera_model_type != 0)
+            return fail(TRIPS_ERR_UNSUPPORTED, "camera_model_type %d: only pinhole+distortion (0)", v.camera_model_type);
+        if (v.image_index < 0 || v.image_index >= d->num_images)
+            return fail(TRIPS_ERR_INVALID_ARG, "view %d: image_index %d out of range", b, v.image_index);
+        if (v.camera_index < 0 || v.camera_index >= d->num_cameras)
+            return fail(TRIPS_ERR_INVALID_ARG, "view %d: camera_index %d out of range", b, v.camera_index);
+    }
+    // list entries are addressed with 32-bit offsets
+    if (4ll * d->num_points * d->num_layers > 0x7fffffffll && d->max_list_entries == 0)
+        return fail(TRIPS_ERR_UNSUPPORTED, "4*N*L exceeds 2^31-1; set max_list_entries");
+    if (d->max_list_entries > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "max_list_entries exceeds 2^31-1");
+    return TRIPS_OK;
+}
+
+void make_geom(const TripsSplatDesc& d, PyramidGeom& g)
+{
+    int cw = d.views[0].w, ch = d.views[0].h;
+    g.num_layers = d.num_layers;
+    g.off[0]     = 0;
+    for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
+    {
+        if (l < d.num_layers)
+        {
+            g.w[l]       = cw;
+            g.h[l]       = ch;
+            g.off[l + 1] = g.off[l] + cw * ch;
+            if (!d.floor_layer_sizes)
+            {
+                // PointRenderer.cu:385-389
+                ch = (int)std::ceil(float(ch) / 2.f);
+                cw = (int)std::ceil(float(cw) / 2.f);
+            }
+            else
+            {
+                ch = ch / 2;
+                cw = cw / 2;
+            }
+        }
+        else
+        {
+            g.w[l]       = 0;
+            g.h[l]       = 0;
+            g.off[l + 1] = g.off[l];
+        }
+    }
+}
+
+long long pyramid_pixels_checked(const TripsSplatDesc& d)
+{
+    long long P = 0;
+    int cw = d.views[0].w, ch = d.views[0].h;
+    for (int l = 0; l < d.num_layers; ++l)
+    {
+        P += (long long)cw * ch;
+        if (!d.floor_layer_sizes)
+        {
+            ch = (int)std::ceil(float(ch) / 2.f);
+            cw = (int)std::ceil(float(cw) / 2.f);
+        }
+        else
+        {
+            ch = ch / 2;
+            cw = cw / 2;
+        }
+    }
+    return P;
+}
+
+SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
+{
+    SavedLayout s;
+    const size_t N = (size_t)d.num_points, P = (size_t)g.off[d.num_layers], K = (size_t)d.list_depth;
+    const size_t rf = (size_t)record_floats(d.num_channels, true);
+    size_t o        = 0;
+    s.header        = o;
+    o += align256(sizeof(ViewHeader));
+    s.rec = o;
+    o += align256(N * rf * sizeof(float));
+    s.lists = o;
+    o += align256(P * K * sizeof(int32_t));
+    s.retained = o;
+    o += align256(P * sizeof(int32_t));
+    s.lengths = o;
+    o += align256(P * sizeof(int32_t));
+    s.bytes_per_view = o;
+    return s;
+}
+
+WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
+{
+    WorkspaceLayout w;
+    const size_t N = (size_t)d.num_points, P = (size_t)g.off[d.num_layers];
+    const size_t nb = (P + kScanTile - 1) / kScanTile;
+    w.capacity      = d.max_list_entries > 0 ? (size_t)d.max_list_entries : 4 * N * (size_t)d.num_layers;
+    size_t o        = 0;
+    // status header (overflow flag of the whole call), then for eval mode, which has no saved state to live
+    // in, the per-view counters and the per-point records
+    o += align256(sizeof(ViewHeader));
+    o += align256(sizeof(ViewHeader));
+    o += align256(N * (size_t)record_floats(d.num_channels, false) * sizeof(float));
+    w.ptk = o;
+    o += align256(N * sizeof(float4));
+    w.counts = o;
+    o += align256(P * sizeof(int32_t));
+    w.cursor = o;
+    o += align256(P * sizeof(int32_t));
+    w.block_sums = o;
+    o += align256((nb + 1) * sizeof(int32_t));
+    w.keys = o;
+    o += align256(w.capacity * sizeof(unsigned long long));
+    w.bytes = o;
+    return w;
+}
+}  // namespace
+
+extern "C" {
+
+const char* trips_version(void) { return "trips_splat 0.1 (gfx950)"; }
+const char* trips_last_error_string(void) { return g_error; }
+
+int trips_ctx_create(TripsCtx** out_ctx, int device)
+{
+    if (!out_ctx) return fail(TRIPS_ERR_INVALID_ARG, "out_ctx is NULL");
+    int count    = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDeviceCount");
+    if (device < 0 || device >= count) return fail(TRIPS_ERR_INVALID_ARG, "device %d of %d", device, count);
+    TripsCtx* c = new TripsCtx;
+    c->device   = device;
+    *out_ctx    = c;
+    return TRIPS_OK;
+}
+
+int trips_ctx_destroy(TripsCtx* ctx)
+{
+    delete ctx;
+    return TRIPS_OK;
+}
+
+int trips_splat_layer_sizes(const TripsSplatDesc* desc, int32_t* w, int32_t* h)
+{
+    if (int e = check_desc(desc)) return e;
+    if (!w || !h) return fail(TRIPS_ERR_INVALID_ARG, "w / h is NULL");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    for (int l = 0; l < desc->num_layers; ++l)
+    {
+        w[l] = g.w[l];
+        h[l] = g.h[l];
+    }
+    return TRIPS_OK;
+}
+
+int trips_splat_workspace_size(const TripsSplatDesc* desc, size_t* bytes)
+{
+    if (int e = check_desc(desc)) return e;
+    if (!bytes) return fail(TRIPS_ERR_INVALID_ARG, "bytes is NULL");
+    if (pyramid_pixels_checked(*desc) > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "pyramid has more than 2^31-1 pixels");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    *bytes = workspace_layout(*desc, g).bytes;
+    return TRIPS_OK;
+}
+
+int trips_splat_saved_size(const TripsSplatDesc* desc, size_t* bytes)
+{
+    if (int e = check_desc(desc)) return e;
+    if (!bytes) return fail(TRIPS_ERR_INVALID_ARG, "bytes is NULL");
+    if (pyramid_pixels_checked(*desc) > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "pyramid has more than 2^31-1 pixels");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    *bytes = saved_layout(*desc, g).bytes_per_view * (size_t)desc->num_views;
+    return TRIPS_OK;
+}
+
+int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
+                        void* workspace, size_t workspace_bytes, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_desc(desc)) return e;
+    if (!in || !out) return fail(TRIPS_ERR_INVALID_ARG, "in / out is NULL");
+    if (pyramid_pixels_checked(*desc) > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "pyramid has more than 2^31-1 pixels");
+    const TripsSplatDesc& d = *desc;
+    if (d.num_points > 0 && (!in->position || !in->point_size || !in->index))
+        return fail(TRIPS_ERR_INVALID_ARG, "position / point_size / index is NULL");
+    if (!in->texture || !in->confidence || !in->background || !in->poses_se3 || !in->intrinsics)
+        if (d.num_points > 0 || !in->background || !in->poses_se3 || !in->intrinsics)
+            return fail(TRIPS_ERR_INVALID_ARG, "texture / confidence / background / poses_se3 / intrinsics is NULL");
+    for (int l = 0; l < d.num_layers; ++l)
+        if (!out->image[l]) return fail(TRIPS_ERR_INVALID_ARG, "image[%d] is NULL", l);
+    const bool train = d.train != 0;
+    if (train && !out->saved) return fail(TRIPS_ERR_INVALID_ARG, "saved is NULL in train mode");
+    if (!workspace) return fail(TRIPS_ERR_INVALID_ARG, "workspace is NULL");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255) || (train && (reinterpret_cast<uintptr_t>(out->saved) & 255)))
+        return fail(TRIPS_ERR_INVALID_ARG, "workspace / saved must be 256-byte aligned");
+
+    PyramidGeom g;
+    make_geom(d, g);
+    const WorkspaceLayout wl = workspace_layout(d, g);
+    if (workspace_bytes < wl.bytes)
+        return fail(TRIPS_ERR_WORKSPACE_SMALL, "workspace has %zu bytes, %zu needed", workspace_bytes, wl.bytes);
+    const SavedLayout sl = saved_layout(d, g);
+    hipStream_t stream   = reinterpret_cast<hipStream_t>(stream_);
+    char* ws             = reinterpret_cast<char*>(workspace);
+
+    for (int b = 0; b < d.num_views; ++b)
+    {
+        ForwardParams p;
+        std::memset(&p, 0, sizeof(p));
+        p.position   = reinterpret_cast<const float4*>(in->position);
+        p.point_size = in->point_size;
+        p.index      = in->index;
+        p.texture    = in->texture;
+        p.confidence = in->confidence;
+        p.background = in->background;
+        p.pose       = in->poses_se3 + 8 * (size_t)d.views[b].image_index;
+        p.intrinsics = in->intrinsics + 13 * (size_t)d.views[b].camera_index;
+        p.dropout    = (train && in->dropout) ? in->dropout + (size_t)b * d.num_points : nullptr;
+        p.geom       = g;
+        p.view       = d.views[b];
+        p.num_points = d.num_points;
+        p.num_texels = d.num_texels;
+        p.num_layers = d.num_layers;
+        p.list_depth = d.list_depth;
+        p.view_index = b;
+        p.num_views  = d.num_views;
+        p.layout     = d.layout;
+        p.background_mode           = d.background_mode;
+        p.drop_out_points_by_radius = d.drop_out_points_by_radius;
+        p.viewer_only               = d.viewer_only;
+        p.drop_out_radius_threshold = d.drop_out_radius_threshold;
+        p.dist_cutoff               = d.dist_cutoff;
+        p.stability_cutoff_value    = d.stability_cutoff_value;
+        p.ptk        = reinterpret_cast<float4*>(ws + wl.ptk);
+        p.counts     = reinterpret_cast<int32_t*>(ws + wl.counts);
+        p.cursor     = reinterpret_cast<int32_t*>(ws + wl.cursor);
+        p.block_sums = reinterpret_cast<int32_t*>(ws + wl.block_sums);
+        p.keys       = reinterpret_cast<unsigned long long*>(ws + wl.keys);
+        p.capacity   = (long long)wl.capacity;
+        if (train)
+        {
+            char* sv     = reinterpret_cast<char*>(out->saved) + sl.bytes_per_view * (size_t)b;
+            p.header     = reinterpret_cast<ViewHeader*>(sv + sl.header);
+            p.rec        = reinterpret_cast<float*>(sv + sl.rec);
+            p.rec_floats = record_floats(d.num_channels, true);
+            p.lists      = reinterpret_cast<int32_t*>(sv + sl.lists);
+            p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
+            p.lengths    = reinterpret_cast<int32_t*>(sv + sl.lengths);
+        }
+        else
+        {
+            p.header     = reinterpret_cast<ViewHeader*>(ws + align256(sizeof(ViewHeader)));
+            p.rec        = reinterpret_cast<float*>(ws + 2 * align256(sizeof(ViewHeader)));
+            p.rec_floats = record_floats(d.num_channels, false);
+        }
+        p.status = reinterpret_cast<ViewHeader*>(ws);
+        for (int l = 0; l < d.num_layers; ++l) p.image[l] = out->image[l];
+        hipError_t e = launch_forward_view(p, d.num_channels, train, b == 0, stream, ctx->prof.enabled ? &ctx->prof : nullptr);
+        if (e != hipSuccess) return hip_fail(e, "forward launch");
+    }
+    return TRIPS_OK;
+}
+
+int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const void* saved,
+                         const float* const grad_image[TRIPS_MAX_LAYERS], const TripsSplatGrads* grads,
+                         void* workspace, size_t workspace_bytes, void* stream_)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_desc(desc)) return e;
+    const TripsSplatDesc& d = *desc;
+    if (!d.train) return fail(TRIPS_ERR_INVALID_ARG, "backward needs a forward run with train = 1");
+    if (!in || !saved || !grad_image || !grads) return fail(TRIPS_ERR_INVALID_ARG, "in / saved / grad_image / grads is NULL");
+    if (!in->background || !in->poses_se3 || !in->intrinsics)
+        return fail(TRIPS_ERR_INVALID_ARG, "background / poses_se3 / intrinsics is NULL");
+    if (!grads->d_texture || !grads->d_confidence || !grads->d_background)
+        return fail(TRIPS_ERR_INVALID_ARG, "d_texture / d_confidence / d_background is required");
+    for (int l = 0; l < d.num_layers; ++l)
+        if (!grad_image[l]) return fail(TRIPS_ERR_INVALID_ARG, "grad_image[%d] is NULL", l);
+    if (reinterpret_cast<uintptr_t>(saved) & 255) return fail(TRIPS_ERR_INVALID_ARG, "saved must be 256-byte aligned");
+
+    PyramidGeom g;
+    make_geom(d, g);
+    const SavedLayout sl = saved_layout(d, g);
+    hipStream_t stream   = reinterpret_cast<hipStream_t>(stream_);
+    for (int b = 0; b < d.num_views; ++b)
+    {
+        BackwardParams p;
+        std::memset(&p, 0, sizeof(p));
+        const char* sv = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)b;
+        p.background   = in->background;
+        p.pose         = in->poses_se3 + 8 * (size_t)d.views[b].image_index;
+        p.intrinsics   = in->intrinsics + 13 * (size_t)d.views[b].camera_index;
+        p.point_size   = in->point_size;
+        p.geom         = g;
+        p.view         = d.views[b];
+        p.num_points   = d.num_points;
+        p.num_texels   = d.num_texels;
+        p.num_layers   = d.num_layers;
+        p.list_depth   = d.list_depth;
+        p.view_index   = b;
+        p.num_views    = d.num_views;
+        p.layout       = d.layout;
+        p.dist_cutoff  = d.dist_cutoff;
+        p.rec          = reinterpret_cast<const float*>(sv + sl.rec);
+        p.rec_floats   = record_floats(d.num_channels, true);
+        p.lists        = reinterpret_cast<const int32_t*>(sv + sl.lists);
+        p.retained     = reinterpret_cast<const int32_t*>(sv + sl.retained);
+        for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
+        p.d_texture    = grads->d_texture;
+        p.d_confidence = grads->d_confidence;
+        p.d_background = grads->d_background;
+        p.d_position   = grads->d_position;
+        p.d_point_size = grads->d_point_size;
+        p.d_pose       = grads->d_pose ? grads->d_pose + 6 * (size_t)d.views[b].image_index : nullptr;
+        p.d_intrinsics = grads->d_intrinsics ? grads->d_intrinsics + 13 * (size_t)d.views[b].camera_index : nullptr;
+        hipError_t e   = launch_backward_view(p, d.num_channels, stream, ctx->prof.enabled ? &ctx->prof : nullptr);
+        if (e != hipSuccess) return hip_fail(e, "backward launch");
+    }
+    return TRIPS_OK;
+}
+
+int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
+{
+    const void* header_owner = workspace;
+    if (!ctx || !header_owner) return fail(TRIPS_ERR_INVALID_ARG, "ctx / workspace is NULL");
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    ViewHeader h;
+    hipError_t e = hipMemcpyAsync(&h, header_owner, sizeof(h), hipMemcpyDeviceToHost, stream);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync");
+    e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    if (h.overflow) return fail(TRIPS_ERR_LIST_OVERFLOW, "%llu list entries dropped: max_list_entries too small", h.overflow);
+    return TRIPS_OK;
+}
+
+int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view, int64_t counters[4],
+                         void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_desc(desc)) return e;
+    if (!saved || !counters) return fail(TRIPS_ERR_INVALID_ARG, "saved / counters is NULL");
+    if (view < 0 || view >= desc->num_views) return fail(TRIPS_ERR_INVALID_ARG, "view out of range");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    const SavedLayout sl = saved_layout(*desc, g);
+    hipStream_t stream   = reinterpret_cast<hipStream_t>(stream_);
+    char* sv             = const_cast<char*>(reinterpret_cast<const char*>(saved)) + sl.bytes_per_view * (size_t)view;
+    ViewHeader* hd       = reinterpret_cast<ViewHeader*>(sv + sl.header);
+    const long long P    = g.off[desc->num_layers];
+    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), P, &hd->reserved[0], stream);
+    if (e != hipSuccess) return hip_fail(e, "retained sum");
+    ViewHeader h;
+    e = hipMemcpyAsync(&h, hd, sizeof(h), hipMemcpyDeviceToHost, stream);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync");
+    e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    counters[0] = (int64_t)h.n_valid;
+    counters[1] = (int64_t)h.n_entries;
+    counters[2] = (int64_t)h.reserved[0];
+    counters[3] = (int64_t)P;
+    return TRIPS_OK;
+}
+
+int trips_splat_export_lists(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view,
+                             int32_t* device_lists, int32_t* device_retained, int32_t* device_lengths, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_desc(desc)) return e;
+    if (!saved) return fail(TRIPS_ERR_INVALID_ARG, "saved is NULL");
+    if (view < 0 || view >= desc->num_views) return fail(TRIPS_ERR_INVALID_ARG, "view out of range");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    const SavedLayout sl = saved_layout(*desc, g);
+    hipStream_t stream   = reinterpret_cast<hipStream_t>(stream_);
+    const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
+    const size_t P = (size_t)g.off[desc->num_layers], K = (size_t)desc->list_depth;
+    hipError_t e = hipSuccess;
+    if (device_lists && P)
+        e = hipMemcpyAsync(device_lists, sv + sl.lists, P * K * sizeof(int32_t), hipMemcpyDeviceToDevice, stream);
+    if (e == hipSuccess && device_retained && P)
+        e = hipMemcpyAsync(device_retained, sv + sl.retained, P * sizeof(int32_t), hipMemcpyDeviceToDevice, stream);
+    if (e == hipSuccess && device_lengths && P)
+        e = hipMemcpyAsync(device_lengths, sv + sl.lengths, P * sizeof(int32_t), hipMemcpyDeviceToDevice, stream);
+    if (e != hipSuccess) return hip_fail(e, "export copy");
+    return TRIPS_OK;
+}
+
+int trips_splat_export_points(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view, float* device_ip,
+                              float* device_depth, float* device_size_px, int32_t* device_max_layer, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_desc(desc)) return e;
+    if (!saved) return fail(TRIPS_ERR_INVALID_ARG, "saved is NULL");
+    if (view < 0 || view >= desc->num_views) return fail(TRIPS_ERR_INVALID_ARG, "view out of range");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    const SavedLayout sl = saved_layout(*desc, g);
+    const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
+    hipError_t e = launch_export_points(reinterpret_cast<const float*>(sv + sl.rec), record_floats(desc->num_channels, true),
+                                        desc->num_points, device_ip, device_depth, device_size_px, device_max_layer,
+                                        reinterpret_cast<hipStream_t>(stream_));
+    if (e != hipSuccess) return hip_fail(e, "export points");
+    return TRIPS_OK;
+}
+
+int trips_adam_step_fused(TripsCtx* ctx, const TripsAdamTensor* tensors, int n_tensors, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (n_tensors < 0 || (n_tensors > 0 && !tensors)) return fail(TRIPS_ERR_INVALID_ARG, "tensors");
+    for (int i = 0; i < n_tensors; ++i)
+    {
+        const TripsAdamTensor& t = tensors[i];
+        if (t.n < 0) return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: n < 0", i);
+        if (t.n == 0) continue;
+        if (!t.weights || !t.grads || !t.first_moment || !t.second_moment || !t.steps)
+            return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: NULL pointer", i);
+        if (t.dtype != TRIPS_DTYPE_F32 && t.dtype != TRIPS_DTYPE_F64)
+            return fail(TRIPS_ERR_UNSUPPORTED, "tensor %d: dtype %d", i, t.dtype);
+        if (!(t.loss_scale != 0.f)) return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: loss_scale is 0", i);
+    }
+    hipError_t e = launch_adam(tensors, n_tensors, reinterpret_cast<hipStream_t>(stream_), ctx->prof.enabled ? &ctx->prof : nullptr);
+    if (e != hipSuccess) return hip_fail(e, "adam launch");
+    return TRIPS_OK;
+}
+
+int trips_apply_tangent(TripsCtx* ctx, double* tangent, double* poses_se3, int n, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (n < 0 || (n > 0 && (!tangent || !poses_se3))) return fail(TRIPS_ERR_INVALID_ARG, "tangent / poses_se3");
+    hipError_t e = launch_apply_tangent(tangent, poses_se3, n, reinterpret_cast<hipStream_t>(stream_));
+    if (e != hipSuccess) return hip_fail(e, "apply_tangent launch");
+    return TRIPS_OK;
+}
+
+int trips_profile_enable(TripsCtx* ctx, int enabled)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    ctx->prof.enabled = enabled != 0;
+    return TRIPS_OK;
+}
+
+int trips_profile_read(TripsCtx* ctx, int* n, const char* names[TRIPS_PROFILE_MAX_KERNELS],
+                       float ms[TRIPS_PROFILE_MAX_KERNELS], int launches[TRIPS_PROFILE_MAX_KERNELS])
+{
+    if (!ctx || !n || !names || !ms || !launches) return fail(TRIPS_ERR_INVALID_ARG, "NULL argument");
+    int count = 0;
+    for (auto& sp : ctx->prof.spans)
+    {
+        hipError_t e = hipEventSynchronize(sp.b);
+        if (e != hipSuccess) return hip_fail(e, "hipEventSynchronize");
+        float t = 0.f;
+        e       = hipEventElapsedTime(&t, sp.a, sp.b);
+        if (e != hipSuccess) return hip_fail(e, "hipEventElapsedTime");
+        int k = 0;
+        while (k < count && std::strcmp(names[k], sp.name) != 0) ++k;
+        if (k == count)
+        {
+            if (count == TRIPS_PROFILE_MAX_KERNELS) continue;
+            names[k]    = sp.name;
+            ms[k]       = 0.f;
+            launches[k] = 0;
+            ++count;
+        }
+        ms[k] += t;
+        launches[k] += 1;
+        ctx->prof.pool.push_back(sp.a);
+        ctx->prof.pool.push_back(sp.b);
+    }
+    ctx->prof.spans.clear();
+    *n = count;
+    return TRIPS_OK;
+}
+
+}  // extern "C"
