@@ -1,0 +1,105 @@
+"""The reference-shaped operator surface (BlendPointCloud / PointRender autograd function) on the GPU."""
+import numpy as np
+import pytest
+import torch
+
+from trips_amd import abi, scenes
+
+pytestmark = pytest.mark.gpu
+
+
+def _info(sc, ns, train=True, **params):
+    from trips_amd.renderer import NeuralRenderInfo, PointRendererCache, ReducedImageInfo, RenderParams
+    p = RenderParams(dropout=0.0, drop_out_points_by_radius=False, max_pixels_per_list=sc.list_depth, **params)
+    images = [ReducedImageInfo(w=v["w"], h=v["h"], image_index=v["image_index"], camera_index=v["camera_index"])
+              for v in sc.views]
+    return NeuralRenderInfo(scene=ns, images=images, params=p, num_layers=sc.num_layers, train=train,
+                            cache=PointRendererCache())
+
+
+def test_blend_point_cloud_forward_backward_matches_oracle(oracle):
+    from tests.gpu_util import rel_err
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=5000, w=80, h=60, f=70.0, num_layers=4, list_depth=16, seed=41, views=2, radius=(0.004, 0.4))
+    ns = NeuralScene.from_arrays(sc, requires_grad=True)
+    info = _info(sc, ns)
+    outs = BlendPointCloud(info)
+    assert len(outs) == 4 and outs[0].shape == (2, 4, 60, 80) and outs[3].shape == (2, 4, 8, 10)
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    for a, b in zip(outs, ref["images"]):
+        np.testing.assert_allclose(a.detach().cpu().numpy(), b, rtol=1e-5, atol=1e-6)
+    rng = np.random.default_rng(0)
+    grads = [rng.normal(0, 1, o.shape).astype(np.float32) for o in outs]
+    loss = sum((o * torch.as_tensor(g).cuda()).sum() for o, g in zip(outs, grads))
+    loss.backward()
+    g_ref = oracle.backward(sc, d, ref, grads)
+    pairs = [(ns.texture.texture.grad, g_ref["d_texture"]), (ns.texture.background_color.grad, g_ref["d_background"]),
+             (ns.point_cloud_cuda.t_position.grad, g_ref["d_position"]),
+             (ns.poses.tangent_poses.grad, g_ref["d_pose"]), (ns.intrinsics.intrinsics.grad, g_ref["d_intrinsics"]),
+             (ns.texture.confidence_value_of_point.grad.reshape(-1), g_ref["d_confidence"]),
+             (ns.point_cloud_cuda.t_point_size.grad.reshape(-1), g_ref["d_point_size"])]
+    for got, want in pairs:
+        assert rel_err(got.cpu().numpy(), want) < 1e-4
+    assert ns.texture.confidence_value_of_point.grad.shape == (1, 5000)
+    assert ns.point_cloud_cuda.t_point_size.grad.shape == (5000, 1)
+    assert ns.poses.tangent_poses.grad.dtype == torch.float64
+
+
+def test_eval_mode_returns_permuted_views_and_no_graph(oracle):
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=42)
+    ns = NeuralScene.from_arrays(sc)
+    info = _info(sc, ns, train=False)
+    with torch.no_grad():
+        outs = BlendPointCloud(info)
+    assert outs[0].shape == (1, 4, 48, 64) and not outs[0].is_contiguous()  # [B,H,W,C] storage, permuted view
+    d = abi.desc_for_scene(sc, train=False)
+    ref = oracle.forward(sc, d)
+    for a, b in zip(outs, ref["images"]):
+        np.testing.assert_allclose(a.permute(0, 2, 3, 1).cpu().numpy(), b, rtol=1e-5, atol=1e-6)
+
+
+def test_only_requested_gradients_are_produced(oracle):
+    from tests.gpu_util import rel_err
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=43)
+    ns = NeuralScene.from_arrays(sc)
+    ns.texture.texture.requires_grad_(True)
+    ns.texture.confidence_value_of_point.requires_grad_(True)
+    info = _info(sc, ns)
+    outs = BlendPointCloud(info)
+    sum(o.sum() for o in outs).backward()
+    assert ns.point_cloud_cuda.t_position.grad is None and ns.point_cloud_cuda.t_point_size.grad is None
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    ones = [np.ones(o.shape, np.float32) for o in outs]
+    g_ref = oracle.backward(sc, d, ref, ones, want_position=False, want_point_size=False, want_pose=False,
+                            want_intrinsics=False)
+    assert rel_err(ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
+    assert rel_err(ns.texture.confidence_value_of_point.grad.cpu().numpy().reshape(-1), g_ref["d_confidence"]) < 1e-4
+
+
+def test_dropout_is_drawn_per_forward_in_train_mode():
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=2, list_depth=16, seed=44)
+    ns = NeuralScene.from_arrays(sc)
+    info = _info(sc, ns)
+    info.params.dropout = 0.5
+    torch.manual_seed(0)
+    a = BlendPointCloud(info)[0].clone()
+    b = BlendPointCloud(info)[0].clone()
+    assert not torch.equal(a, b)
+    assert info.cache.dropout_points.shape == (1, 3000)
+    frac = float(info.cache.dropout_points.mean())
+    assert 0.4 < frac < 0.6
+
+
+def test_unsupported_render_modes_raise():
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=100)
+    ns = NeuralScene.from_arrays(sc)
+    info = _info(sc, ns)
+    info.params.render_mode = 1
+    with pytest.raises(NotImplementedError):
+        BlendPointCloud(info)

@@ -1,6 +1,6 @@
 """Seeded synthetic scenes for tests and bench.py.
 
-All inputs come from numpy's counter-based Philox generator, so the CPU oracle and the GPU path
+All inputs come from numpy's counter-based Philox generator, so a CPU check and the GPU path
 consume bit-identical host arrays. Layouts follow the reference's tensors:
   position   [N,4] f32  xyz + drop-out radius        (src/lib/rendering/NeuralPointCloudCuda.cpp:62)
   point_size [N]   f32  raw, softplus applied inside (NeuralPointCloudCuda.cpp:19-24,50)
