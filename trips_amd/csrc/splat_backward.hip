@@ -1,13 +1,23 @@
-// Backward kernel of the splat path for gfx950 (wave64).
+// Backward kernels of the splat path for gfx950 (wave64).
 //
-//   blend_backward_kernel <- BlendBackwardsBilinearTiled  src/lib/rendering/RenderBackward.cu:90-618
+//   backward_pixels_kernel + backward_points_kernel <- BlendBackwardsBilinearTiled
+//                                                      src/lib/rendering/RenderBackward.cu:90-618
 //
-// The reference walks one pixel list per thread, sequentially, re-reading 7 saved floats per entry. Here a
-// 16-lane row owns a pixel and each lane owns one retained entry: alpha and transmittance are recomputed from
-// the per-point record exactly as the forward computed them, the "all later entries" sum of
-// RenderBackward.cu:284-301 becomes a suffix sum across the row, and pose / intrinsics / background partials
-// stay in registers (double) over a grid-stride loop before one block-level reduction and one atomic per value
-// and block (the reference keeps them in shared double arrays, :160-187,546-617).
+// The reference walks one pixel list per thread and scatters every entry's gradient with float atomics
+// (3 position + 1 size + 1 confidence + C descriptor atomics per retained entry). Scattered atomics run at
+// about 2e10 per second on this GPU while scattered loads run at 5e10 and cost the same for 4 or 64 bytes,
+// so the work is split in two passes without atomics on the per-point arrays:
+//   1. pixels: a 16-lane row owns a pixel, each lane one retained entry. Alpha and transmittance are recomputed
+//      from the per-point record exactly as the forward computed them; the "all later entries" sum of
+//      RenderBackward.cu:284-301 is a suffix sum across the row. Per entry it writes {dL/dalpha, T*alpha*dL/dimage}
+//      into the pixel's row of a [P,K] table and one byte, the entry's rank, into the point's 32-slot table
+//      (slot = layer * 4 + footprint corner).
+//   2. points: one thread per point walks its slots, gathers those records (one aligned load each), sums the image-space gradient of all its entries and runs the projection chain ONCE
+//      (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then adds its gradients
+//      with plain read-modify-writes. Pose / intrinsics partials stay in double registers over a grid-stride
+//      loop before one block-level reduction and one atomic per value and block (the reference keeps them in
+//      shared double arrays, :160-187,546-617).
+// Gradients are therefore summed in a fixed order and are bit-reproducible from run to run.
 #include "splat_internal.h"
 #include "trips_math.h"
 
@@ -47,30 +57,27 @@ __device__ __forceinline__ double wave_sum(double v)
     return v;
 }
 
+
+// ---------------------------------------------------------------------------------------------------------
+// Pass 1: per pixel row. Writes entry_grad[pix*K + j] = {dL/dalpha_j, T_j alpha_j g[0..C)} and rank[pid*32 + slot] = j.
 template <int C>
-__global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParams p)
+__global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardParams p)
 {
     constexpr int CPAD = (C + 3) & ~3;
-    constexpr int NACC = 6 + 5 + 8 + C;  // pose, K, distortion, background
+    constexpr int EF   = (1 + C + 3) & ~3;  // floats per entry of entry_grad
     const int lane     = threadIdx.x & 63;
     const int sub      = lane & 15;
     const int grp      = lane >> 4;
     const int P        = p.geom.off[p.num_layers];
     const int K        = p.list_depth;
-    const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
-    float R[9];
-    rotation_matrix(cam.V, R);
-    const bool want_pose = p.d_pose != nullptr;
-    const bool want_intr = p.d_intrinsics != nullptr;
-    const bool want_size = p.d_point_size != nullptr;
 
-    double acc[NACC];
+    double acc_bg[C];
 #pragma unroll
-    for (int i = 0; i < NACC; ++i) acc[i] = 0.0;
+    for (int i = 0; i < C; ++i) acc_bg[i] = 0.0;
 
-    const long long total_waves  = ((long long)P + 3) / 4;
-    const long long wave0        = ((long long)blockIdx.x * 256 + threadIdx.x) >> 6;
-    const long long wave_stride  = (long long)gridDim.x * 4;
+    const long long total_waves = ((long long)P + 3) / 4;
+    const long long wave0       = ((long long)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const long long wave_stride = (long long)gridDim.x * 4;
 
     for (long long wv = wave0; wv < total_waves; wv += wave_stride)
     {
@@ -105,17 +112,16 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
         }
 
         int pid = 0;
-        float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), rv = make_float4(0.f, 0.f, 1.f, 0.f);
-        int tex = 0;
         float desc[CPAD];
 #pragma unroll
         for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
-        float a = 0.f, ux = 0.f, uy = 0.f;
+        float a = 0.f;
+        int slot = 0;
         if (has)
         {
             pid               = p.lists[(size_t)pix * K + sub];
             const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
-            r0                = rec[0];
+            const float4 r0   = rec[0];
 #pragma unroll
             for (int q = 0; q < CPAD / 4; ++q)
             {
@@ -125,15 +131,15 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
                 desc[4 * q + 2] = t.z;
                 desc[4 * q + 3] = t.w;
             }
-            rv                = rec[1 + CPAD / 4];
-            tex               = __float_as_int(rec[2 + CPAD / 4].x);
-            const float mfac  = 1.f / float(1 << layer);
-            ux                = r0.x * mfac;
-            uy                = r0.y * mfac;
-            float w           = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
+            const float mfac = 1.f / float(1 << layer);
+            const float ux = r0.x * mfac, uy = r0.y * mfac;
+            float w = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
             if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
             a = w * r0.w;
             a *= layer_factor(r0.z, layer, p.num_layers, nullptr);
+            // which of the point's four footprint pixels this one is
+            const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
+            slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
         }
 
         // exclusive transmittance, same chain as the forward
@@ -144,14 +150,13 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
             pre = __shfl_up(pre * (1.f - a), 1, 16);
             if (sub == s) T = pre;
         }
-        // transmittance after the m retained entries: decides whether the background is reached
+        // transmittance after the m retained entries decides whether the background is reached
         // (RenderBackward.cu:205-210,302-308)
         float T_after = T * (1.f - a);
         T_after       = __shfl(T_after, max(m - 1, 0), 16);
         if (m == 0) T_after = 1.f;
         const bool bg_reached = live && (T_after >= 0.001f);
 
-        // s_j = sum_c colour_c * grad_c ; q_j = T_j a_j s_j
         float s = 0.f, sbg = 0.f;
 #pragma unroll
         for (int c = 0; c < C; ++c)
@@ -159,9 +164,9 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
             s += desc[c] * g[c];
             sbg += p.background[c] * g[c];
         }
-        const float q = has ? (T * a) * s : 0.f;
-        // suffix sum over later entries of the row
-        float later = __shfl_down(q, 1, 16);  // entries i > j
+        const float ta = T * a;
+        const float q  = has ? ta * s : 0.f;
+        float later    = __shfl_down(q, 1, 16);  // entries i > j
         if (sub == 15) later = 0.f;
 #pragma unroll
         for (int o = 1; o < 16; o <<= 1)
@@ -176,72 +181,190 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
         if (bg_reached && sub == 0)
         {
 #pragma unroll
-            for (int c = 0; c < C; ++c) acc[19 + c] += (double)(T_after * g[c]);
+            for (int c = 0; c < C; ++c) acc_bg[c] += (double)(T_after * g[c]);
         }
-
         if (has)
         {
-            // colour gradient (RenderBackward.cu:262-267)
-            const float ta = T * a;
+            // {dL/dalpha, T*alpha*g[0..C)} padded to a multiple of 4 floats: one aligned gather for pass 2
+            float e[EF];
+            e[0] = grad_alpha;
 #pragma unroll
-            for (int c = 0; c < C; ++c) unsafeAtomicAdd(p.d_texture + (size_t)c * p.num_texels + tex, ta * g[c]);
-
-            // geometric part (RenderBackward.cu:334-465)
-            const float sx = ux - floorf(ux), sy = uy - floorf(uy);
-            const int x_i  = float(gx) < ux ? 0 : 1;
-            const int y_i  = float(gy) < uy ? 0 : 2;
-            const int bi   = y_i + x_i;
-            float blend, J0, J1;
-            switch (bi)
-            {
-                case 0: blend = (1.f - sx) * (1.f - sy); J0 = sy - 1.f; J1 = sx - 1.f; break;
-                case 1: blend = sx * (1.f - sy); J0 = 1.f - sy; J1 = -sx; break;
-                case 2: blend = (1.f - sx) * sy; J0 = -sy; J1 = 1.f - sx; break;
-                default: blend = sx * sy; J0 = sy; J1 = sx; break;
-            }
-            if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
-            const float conf = r0.w;
-            float lfac = 1.f, J_lf = 0.f;
-            if (want_size) lfac = layer_factor(r0.z, layer, p.num_layers, &J_lf);
-            unsafeAtomicAdd(p.d_confidence + tex, blend * lfac * grad_alpha);
-
-            const float gbs = conf * lfac * grad_alpha;
-            float g_point[3], g_pose[6], g_k[5], g_dis[8];
-            project_backward(cam, R, rv.x, rv.y, rv.z, J0 * gbs, J1 * gbs, g_point, g_pose, g_k, g_dis, want_intr);
-            if (want_size)
-            {
-                const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
-                const float grad_layer_ps  = rv.w * J_softmax_proj * J_lf * grad_alpha;
-                unsafeAtomicAdd(p.d_point_size + pid, blend * conf * grad_layer_ps);
-            }
-            if (p.d_position)
-            {
-                float* dp = p.d_position + 4 * (size_t)pid;
-                unsafeAtomicAdd(dp + 0, g_point[0]);
-                unsafeAtomicAdd(dp + 1, g_point[1]);
-                unsafeAtomicAdd(dp + 2, g_point[2]);
-            }
-            if (want_pose)
-            {
+            for (int c = 0; c < C; ++c) e[1 + c] = ta * g[c];
 #pragma unroll
-                for (int k = 0; k < 6; ++k) acc[k] += (double)g_pose[k];
-            }
-            if (want_intr)
-            {
+            for (int c = 1 + C; c < EF; ++c) e[c] = 0.f;
+            float4* dst = reinterpret_cast<float4*>(p.entry_grad + ((size_t)pix * K + sub) * EF);
 #pragma unroll
-                for (int k = 0; k < 5; ++k) acc[6 + k] += (double)g_k[k];
-#pragma unroll
-                for (int k = 0; k < 8; ++k) acc[11 + k] += (double)g_dis[k];
-            }
+            for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
+            p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
         }
     }
 
-    // block reduction, one atomic per value and block
+    __shared__ double s_acc[4][C];
+#pragma unroll
+    for (int i = 0; i < C; ++i)
+    {
+        double v = wave_sum(acc_bg[i]);
+        if (lane == 0) s_acc[threadIdx.x >> 6][i] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < C)
+    {
+        const int i = threadIdx.x;
+        double v    = s_acc[0][i] + s_acc[1][i] + s_acc[2][i] + s_acc[3][i];
+        if (v != 0.0) unsafeAtomicAdd(p.d_background + i, (float)v);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Pass 2: per point.
+template <int C>
+__global__ __launch_bounds__(256) void backward_points_kernel(const BackwardParams p)
+{
+    constexpr int CPAD = (C + 3) & ~3;
+    constexpr int EF   = (1 + C + 3) & ~3;
+    constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
+    const int lane     = threadIdx.x & 63;
+    const int K        = p.list_depth;
+    const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
+    float R[9];
+    rotation_matrix(cam.V, R);
+    const bool want_pose = p.d_pose != nullptr;
+    const bool want_intr = p.d_intrinsics != nullptr;
+    const bool want_size = p.d_point_size != nullptr;
+    const bool identity  = p.header->reserved[1] == 0;  // index[pid] == pid for every point
+
+    double acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i] = 0.0;
+
+    for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
+    {
+        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
+        const float4 tail = rec[2 + CPAD / 4];  // {texture index, depth, layers written, -}
+        if (!(tail.y > 0.f)) continue;
+        const int tex       = __float_as_int(tail.x);
+        const int max_layer = __float_as_int(tail.z);
+        const float4 r0     = rec[0];          // ip.x ip.y size_px conf
+        const float4 rv     = rec[1 + CPAD / 4];  // view xyz, softplus'(raw size)
+        const uint4* rk     = reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 32);
+        const uint4 rk0 = rk[0], rk1 = rk[1];
+        const unsigned words[8] = {rk0.x, rk0.y, rk0.z, rk0.w, rk1.x, rk1.y, rk1.z, rk1.w};
+
+        float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;
+        float tex_grad[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) tex_grad[c] = 0.f;
+        const float conf = r0.w;
+        bool any         = false;
+
+        for (int layer = 0; layer < max_layer; ++layer)
+        {
+            const unsigned word = words[layer];
+            if (word == 0xFFFFFFFFu) continue;
+            const float mfac = 1.f / float(1 << layer);
+            const float ux = r0.x * mfac, uy = r0.y * mfac;
+            const float fx = floorf(ux), fy = floorf(uy);
+            const int px = (int)fx, py = (int)fy;
+            const float sx = ux - fx, sy = uy - fy;
+            const int lw = p.geom.w[layer];
+            float lfac = 1.f, J_lf = 0.f;
+            if (want_size) lfac = layer_factor(r0.z, layer, p.num_layers, &J_lf);
+            const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
+#pragma unroll
+            for (int corner = 0; corner < 4; ++corner)
+            {
+                const unsigned j = (word >> (8 * corner)) & 0xFFu;
+                if (j == 0xFFu) continue;
+                any          = true;
+                const int gx = px + (corner & 1), gy = py + (corner >> 1);
+                const int pix = p.geom.off[layer] + gy * lw + gx;
+                float e[EF];
+                {
+                    const float4* src = reinterpret_cast<const float4*>(p.entry_grad + ((size_t)pix * K + j) * EF);
+#pragma unroll
+                    for (int q = 0; q < EF / 4; ++q)
+                    {
+                        const float4 t = src[q];
+                        e[4 * q]       = t.x;
+                        e[4 * q + 1]   = t.y;
+                        e[4 * q + 2]   = t.z;
+                        e[4 * q + 3]   = t.w;
+                    }
+                }
+                const float grad_alpha = e[0];
+#pragma unroll
+                for (int c = 0; c < C; ++c) tex_grad[c] += e[1 + c];
+                // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
+                const int x_i = float(gx) < ux ? 0 : 1;
+                const int y_i = float(gy) < uy ? 0 : 2;
+                const int bi  = y_i + x_i;
+                float blend, J0, J1;
+                switch (bi)
+                {
+                    case 0: blend = (1.f - sx) * (1.f - sy); J0 = sy - 1.f; J1 = sx - 1.f; break;
+                    case 1: blend = sx * (1.f - sy); J0 = 1.f - sy; J1 = -sx; break;
+                    case 2: blend = (1.f - sx) * sy; J0 = -sy; J1 = 1.f - sx; break;
+                    default: blend = sx * sy; J0 = sy; J1 = sx; break;
+                }
+                if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
+                conf_grad += blend * lfac * grad_alpha;
+                const float gbs = conf * lfac * grad_alpha;
+                d0 += J0 * gbs;
+                d1 += J1 * gbs;
+                if (want_size)
+                {
+                    const float grad_layer_ps = rv.w * J_softmax_proj * J_lf * grad_alpha;
+                    size_grad += blend * conf * grad_layer_ps;
+                }
+            }
+        }
+        if (!any) continue;
+
+        float g_point[3], g_pose[6], g_k[5], g_dis[8];
+        project_backward(cam, R, rv.x, rv.y, rv.z, d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
+
+        if (identity)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c) p.d_texture[(size_t)c * p.num_texels + tex] += tex_grad[c];
+            p.d_confidence[tex] += conf_grad;
+        }
+        else
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c) unsafeAtomicAdd(p.d_texture + (size_t)c * p.num_texels + tex, tex_grad[c]);
+            unsafeAtomicAdd(p.d_confidence + tex, conf_grad);
+        }
+        if (want_size) p.d_point_size[pid] += size_grad;
+        if (p.d_position)
+        {
+            float4* dp = reinterpret_cast<float4*>(p.d_position) + pid;
+            float4 v   = *dp;
+            v.x += g_point[0];
+            v.y += g_point[1];
+            v.z += g_point[2];
+            *dp = v;
+        }
+        if (want_pose)
+        {
+#pragma unroll
+            for (int k = 0; k < 6; ++k) acc[k] += (double)g_pose[k];
+        }
+        if (want_intr)
+        {
+#pragma unroll
+            for (int k = 0; k < 5; ++k) acc[6 + k] += (double)g_k[k];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[11 + k] += (double)g_dis[k];
+        }
+    }
+
+    if (!want_pose && !want_intr) return;
     __shared__ double s_acc[4][NACC];
 #pragma unroll
     for (int i = 0; i < NACC; ++i)
     {
-        const bool used = (i < 6) ? want_pose : (i < 19 ? want_intr : true);
+        const bool used = (i < 6) ? want_pose : want_intr;
         if (!used) continue;
         double v = wave_sum(acc[i]);
         if (lane == 0) s_acc[threadIdx.x >> 6][i] = v;
@@ -250,7 +373,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
     if (threadIdx.x < NACC)
     {
         const int i     = threadIdx.x;
-        const bool used = (i < 6) ? want_pose : (i < 19 ? want_intr : true);
+        const bool used = (i < 6) ? want_pose : want_intr;
         if (used)
         {
             double v = s_acc[0][i] + s_acc[1][i] + s_acc[2][i] + s_acc[3][i];
@@ -258,30 +381,61 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(const BackwardParam
             {
                 if (i < 6)
                     unsafeAtomicAdd(p.d_pose + i, v);
-                else if (i < 19)
-                    unsafeAtomicAdd(p.d_intrinsics + (i - 6), (float)v);
                 else
-                    unsafeAtomicAdd(p.d_background + (i - 19), (float)v);
+                    unsafeAtomicAdd(p.d_intrinsics + (i - 6), (float)v);
             }
         }
     }
 }
 
+__global__ __launch_bounds__(256) void fill_u32_kernel(unsigned* __restrict__ p, unsigned v, long long n)
+{
+    long long i      = (long long)blockIdx.x * 256 + threadIdx.x;
+    long long stride = (long long)gridDim.x * 256;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+#define TRIPS_BW_DISPATCH(KERNEL, BLOCKS)                                                                      \
+    switch (channels)                                                                                          \
+    {                                                                                                          \
+        case 3: hipLaunchKernelGGL((KERNEL<3>), dim3(BLOCKS), dim3(256), 0, stream, p); break;                 \
+        case 4: hipLaunchKernelGGL((KERNEL<4>), dim3(BLOCKS), dim3(256), 0, stream, p); break;                 \
+        case 6: hipLaunchKernelGGL((KERNEL<6>), dim3(BLOCKS), dim3(256), 0, stream, p); break;                 \
+        case 8: hipLaunchKernelGGL((KERNEL<8>), dim3(BLOCKS), dim3(256), 0, stream, p); break;                 \
+        case 16: hipLaunchKernelGGL((KERNEL<16>), dim3(BLOCKS), dim3(256), 0, stream, p); break;               \
+        default: return hipErrorInvalidValue;                                                                  \
+    }
+
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof)
 {
-    ProfScope ps(prof, "blend_backward", stream);
-    const int P            = p.geom.off[p.num_layers];
-    const long long waves  = ((long long)P + 3) / 4;
-    long long blocks_ll    = (waves + 3) / 4;
-    const int blocks       = (int)(blocks_ll < 2048 ? (blocks_ll < 1 ? 1 : blocks_ll) : 2048);
-    switch (channels)
+    const int P           = p.geom.off[p.num_layers];
+    const int N           = p.num_points;
+    if (N <= 0) 
     {
-        case 3: hipLaunchKernelGGL((blend_backward_kernel<3>), dim3(blocks), dim3(256), 0, stream, p); break;
-        case 4: hipLaunchKernelGGL((blend_backward_kernel<4>), dim3(blocks), dim3(256), 0, stream, p); break;
-        case 6: hipLaunchKernelGGL((blend_backward_kernel<6>), dim3(blocks), dim3(256), 0, stream, p); break;
-        case 8: hipLaunchKernelGGL((blend_backward_kernel<8>), dim3(blocks), dim3(256), 0, stream, p); break;
-        case 16: hipLaunchKernelGGL((blend_backward_kernel<16>), dim3(blocks), dim3(256), 0, stream, p); break;
-        default: return hipErrorInvalidValue;
+        // no points: only the background receives gradient
+    }
+    {
+        ProfScope ps(prof, "fill_rank", stream);
+        const long long words = (long long)N * 8;  // 32 bytes per point
+        if (words > 0)
+        {
+            int blocks = (int)min((words + 255) / 256, 8192ll);
+            hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks), dim3(256), 0, stream,
+                               reinterpret_cast<unsigned*>(p.rank), 0xFFFFFFFFu, words);
+        }
+    }
+    {
+        ProfScope ps(prof, "backward_pixels", stream);
+        const long long waves = ((long long)P + 3) / 4;
+        long long blocks_ll   = (waves + 3) / 4;
+        const int blocks      = (int)(blocks_ll < 4096 ? (blocks_ll < 1 ? 1 : blocks_ll) : 4096);
+        TRIPS_BW_DISPATCH(backward_pixels_kernel, blocks);
+    }
+    if (N > 0)
+    {
+        ProfScope ps(prof, "backward_points", stream);
+        const int blocks = min((N + 255) / 256, 4096);
+        TRIPS_BW_DISPATCH(backward_points_kernel, blocks);
     }
     return hipGetLastError();
 }

@@ -72,12 +72,14 @@ __global__ __launch_bounds__(256) void project_count_kernel(const ForwardParams 
     const Camera cam   = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L        = p.num_layers;
     unsigned my_valid  = 0;
+    bool not_identity  = false;  // some point's descriptor column differs from its own index
 
     for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
     {
         float4 ptk  = make_float4(0.f, 0.f, -1.f, 0.f);
         bool skip   = false;
         const int tex = p.index[pid];
+        not_identity |= (tex != pid);
         if (p.viewer_only)
         {
             if (p.confidence[tex] < p.stability_cutoff_value) skip = true;
@@ -165,6 +167,7 @@ __global__ __launch_bounds__(256) void project_count_kernel(const ForwardParams 
         unsigned t = s_valid[0] + s_valid[1] + s_valid[2] + s_valid[3];
         if (t) atomicAdd(&p.header->n_valid, (u64)t);
     }
+    if (__ballot(not_identity) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.header->reserved[1], 1ull);
 }
 
 // ---------------------------------------------------------------------------------------------------------

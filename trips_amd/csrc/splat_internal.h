@@ -111,6 +111,13 @@ struct SavedLayout
     size_t bytes_per_view;
 };
 
+struct BackwardWorkspaceLayout
+{
+    size_t entry_grad;  // float [P, K, EF]
+    size_t rank;        // uint8 [N, 32]
+    size_t bytes;
+};
+
 struct WorkspaceLayout
 {
     size_t ptk;         // float4 [N]   {ip.x, ip.y, depth (-1 culled), max_layer bits}
@@ -178,7 +185,10 @@ struct BackwardParams
     int32_t rec_floats;
     const int32_t* lists;
     const int32_t* retained;
+    const ViewHeader* header;
     const float* grad_image[TRIPS_MAX_LAYERS];
+    float* entry_grad;    // [P, K, EF] {dL/dalpha, T alpha dL/dimage[0..C)}, EF = (1+C) rounded up to 4 (workspace)
+    unsigned char* rank;  // [N, 32] rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
     float* d_texture;
     float* d_confidence;
     float* d_background;

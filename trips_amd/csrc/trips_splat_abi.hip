@@ -189,6 +189,18 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     w.bytes = o;
     return w;
 }
+BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
+{
+    BackwardWorkspaceLayout w;
+    const size_t N = (size_t)d.num_points, P = (size_t)g.off[d.num_layers], K = (size_t)d.list_depth;
+    size_t o       = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
+    w.entry_grad   = o;
+    o += align256(P * K * (size_t)((1 + d.num_channels + 3) & ~3) * sizeof(float));
+    w.rank = o;
+    o += align256(N * 32);
+    w.bytes = o;
+    return w;
+}
 }  // namespace
 
 extern "C" {
@@ -236,7 +248,9 @@ int trips_splat_workspace_size(const TripsSplatDesc* desc, size_t* bytes)
     if (pyramid_pixels_checked(*desc) > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "pyramid has more than 2^31-1 pixels");
     PyramidGeom g;
     make_geom(*desc, g);
-    *bytes = workspace_layout(*desc, g).bytes;
+    const size_t fwd = workspace_layout(*desc, g).bytes;
+    const size_t bwd = desc->train ? backward_workspace_layout(*desc, g).bytes : 0;
+    *bytes           = fwd > bwd ? fwd : bwd;
     return TRIPS_OK;
 }
 
@@ -343,8 +357,6 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
                          const float* const grad_image[TRIPS_MAX_LAYERS], const TripsSplatGrads* grads,
                          void* workspace, size_t workspace_bytes, void* stream_)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
     if (int e = check_desc(desc)) return e;
     const TripsSplatDesc& d = *desc;
@@ -361,6 +373,12 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
     PyramidGeom g;
     make_geom(d, g);
     const SavedLayout sl = saved_layout(d, g);
+    const BackwardWorkspaceLayout bl = backward_workspace_layout(d, g);
+    if (!workspace) return fail(TRIPS_ERR_INVALID_ARG, "workspace is NULL");
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return fail(TRIPS_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
+    if (workspace_bytes < bl.bytes)
+        return fail(TRIPS_ERR_WORKSPACE_SMALL, "workspace has %zu bytes, %zu needed", workspace_bytes, bl.bytes);
+    char* ws             = reinterpret_cast<char*>(workspace);
     hipStream_t stream   = reinterpret_cast<hipStream_t>(stream_);
     for (int b = 0; b < d.num_views; ++b)
     {
@@ -385,6 +403,9 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.rec_floats   = record_floats(d.num_channels, true);
         p.lists        = reinterpret_cast<const int32_t*>(sv + sl.lists);
         p.retained     = reinterpret_cast<const int32_t*>(sv + sl.retained);
+        p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
+        p.entry_grad   = reinterpret_cast<float*>(ws + bl.entry_grad);
+        p.rank         = reinterpret_cast<unsigned char*>(ws + bl.rank);
         for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
         p.d_texture    = grads->d_texture;
         p.d_confidence = grads->d_confidence;
