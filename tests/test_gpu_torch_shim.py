@@ -1,0 +1,109 @@
+"""The C++ libtorch host side (trips_amd/csrc/torch_shim): BlendPointCloud / PointRender / MyAdam / ApplyTangent
+driven through its pybind11 test module, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from trips_amd import abi, scenes
+
+
+def _load():
+    from trips_amd import _trips_torch  # noqa: built by trips_amd.build.build_torch_shim
+    return _trips_torch
+
+
+def test_shim_module_imports_without_gpu():
+    m = _load()
+    assert hasattr(m, "Session")
+    s = m.Session()
+    assert hasattr(s, "blend_point_cloud") and hasattr(s, "adam_step") and hasattr(s, "apply_tangent")
+
+
+def _session(sc, requires_grad=True):
+    m = _load()
+    f = lambda a, dt=torch.float32: torch.as_tensor(np.ascontiguousarray(a), dtype=dt).cuda().contiguous()
+    t = dict(texture=f(sc.texture), background=f(sc.background), confidence=f(sc.confidence).reshape(1, -1),
+             position=f(sc.position), point_size=f(sc.point_size).reshape(-1, 1),
+             index=f(sc.index, torch.int32).reshape(-1, 1), poses_se3=f(sc.poses_se3, torch.float64),
+             tangent_poses=torch.zeros((sc.poses_se3.shape[0], 6), dtype=torch.float64, device="cuda"),
+             intrinsics=f(sc.intrinsics))
+    if requires_grad:
+        for k in ("texture", "background", "confidence", "position", "point_size", "tangent_poses", "intrinsics"):
+            t[k].requires_grad_(True)
+    s = m.Session()
+    s.set_scene(t["texture"], t["background"], t["confidence"], t["position"], t["point_size"], t["index"],
+                t["poses_se3"], t["tangent_poses"], t["intrinsics"])
+    return s, t
+
+
+@pytest.mark.gpu
+def test_cpp_blend_point_cloud_forward_backward(oracle):
+    from tests.gpu_util import rel_err
+    sc = scenes.tiny(n=5000, w=80, h=60, f=70.0, num_layers=4, list_depth=16, seed=51, views=2, radius=(0.004, 0.4))
+    s, t = _session(sc)
+    views = [[v["w"], v["h"], v["image_index"], v["camera_index"]] for v in sc.views]
+    outs = s.blend_point_cloud(views, sc.num_layers, True, 0.0, 0, 16)
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    assert len(outs) == 4
+    for a, b in zip(outs, ref["images"]):
+        np.testing.assert_allclose(a.detach().cpu().numpy(), b, rtol=1e-5, atol=1e-6)
+    rng = np.random.default_rng(0)
+    grads = [rng.normal(0, 1, o.shape).astype(np.float32) for o in outs]
+    sum((o * torch.as_tensor(g).cuda()).sum() for o, g in zip(outs, grads)).backward()
+    g_ref = oracle.backward(sc, d, ref, grads)
+    pairs = [(t["texture"].grad, g_ref["d_texture"]), (t["background"].grad, g_ref["d_background"]),
+             (t["position"].grad, g_ref["d_position"]), (t["tangent_poses"].grad, g_ref["d_pose"]),
+             (t["intrinsics"].grad, g_ref["d_intrinsics"]), (t["confidence"].grad.reshape(-1), g_ref["d_confidence"]),
+             (t["point_size"].grad.reshape(-1), g_ref["d_point_size"])]
+    for got, want in pairs:
+        assert rel_err(got.cpu().numpy(), want) < 1e-4
+
+
+@pytest.mark.gpu
+def test_cpp_eval_mode_and_crop(oracle):
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=52)
+    sc.views[0]["crop_transform"] = (1.5, 1.25, -10.0, 4.0, 0.0)
+    s, t = _session(sc, requires_grad=False)
+    v = sc.views[0]
+    views = [[v["w"], v["h"], 0, 0, *v["crop_transform"], 1.0, 0.0, 0.0, 1.0]]
+    with torch.no_grad():
+        outs = s.blend_point_cloud(views, sc.num_layers, False, 0.0, 0, 16)
+    assert outs[0].shape == (1, 4, 48, 64)
+    ref = oracle.forward(sc, abi.desc_for_scene(sc, train=False))
+    for a, b in zip(outs, ref["images"]):
+        np.testing.assert_allclose(a.permute(0, 2, 3, 1).cpu().numpy(), b, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_cpp_myadam_and_apply_tangent(oracle):
+    sc = scenes.tiny(n=2000, w=48, h=40, f=45.0, num_layers=2, list_depth=16, seed=53)
+    s, t = _session(sc)
+    rng = np.random.default_rng(3)
+    gpos = rng.normal(0, 1, sc.position.shape).astype(np.float32)
+    gpos[::3] = 0
+    gtan = rng.normal(0, 1, (1, 6))
+    w0 = t["position"].detach().cpu().numpy().copy()
+    p0 = t["tangent_poses"].detach().cpu().numpy().copy()
+    s.make_adam([t["position"], t["tangent_poses"]], 1e-2)
+    ref_w = dict(w=w0.reshape(-1).copy(), g=gpos.reshape(-1), m=np.zeros(w0.size, np.float32),
+                 v=np.zeros(w0.size, np.float32), steps=np.zeros(w0.size, np.int64), n=w0.size, lr=1e-2)
+    ref_p = dict(w=p0.reshape(-1).copy(), g=gtan.reshape(-1), m=np.zeros(6, np.float32), v=np.zeros(6, np.float32),
+                 steps=np.zeros(6, np.int64), n=6, lr=1e-2, dtype=abi.TRIPS_DTYPE_F64)
+    for _ in range(2):
+        t["position"].grad = torch.as_tensor(gpos).cuda()
+        t["tangent_poses"].grad = torch.as_tensor(gtan).cuda()
+        s.adam_step()
+        oracle.adam_step([ref_w, ref_p])
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(t["position"].detach().cpu().numpy().reshape(-1), ref_w["w"], rtol=2e-6, atol=1e-7)
+    np.testing.assert_allclose(t["tangent_poses"].detach().cpu().numpy().reshape(-1), ref_p["w"], rtol=2e-6, atol=1e-9)
+    # pose <- exp(tangent) * pose, tangent <- 0
+    poses = sc.poses_se3.copy()
+    tang = t["tangent_poses"].detach().cpu().numpy().copy()
+    with torch.no_grad():
+        s.apply_tangent()
+    torch.cuda.synchronize()
+    oracle.apply_tangent(tang, poses)
+    np.testing.assert_allclose(t["poses_se3"].cpu().numpy(), poses, atol=1e-13)
+    assert float(t["tangent_poses"].detach().abs().max()) == 0.0

@@ -31,6 +31,34 @@ def build(verbose=False):
     return LIB
 
 
+SHIM_DIR = os.path.join(CSRC, "torch_shim")
+SHIM_LIB = os.path.join(HERE, "_trips_torch.so")
+
+
+def build_torch_shim(verbose=False):
+    """Builds the libtorch host side (PointRender / NeuralRenderInfo / MyAdam in C++) with a pybind11 test driver.
+    Plain g++: the shim holds no device code, it only calls the C ABI of libtrips_splat.so."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = ce.library_paths()[0]
+    inc = [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include"]
+    abi_flag = f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"
+    cmd = (["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-variable", abi_flag,
+            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_trips_torch",
+            "-DTORCH_API_INCLUDE_EXTENSION_H"] + inc +
+           [os.path.join(SHIM_DIR, "trips_torch.cpp"), os.path.join(SHIM_DIR, "trips_torch_py.cpp"),
+            f"-L{tlib}", f"-L{HERE}", "-ltrips_splat", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+            "-ltorch_python", f"-Wl,-rpath,{tlib}", "-Wl,-rpath,$ORIGIN", "-o", SHIM_LIB])
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return SHIM_LIB
+
+
 if __name__ == "__main__":
     build(verbose=True)
     print(LIB)
+    if "--shim" in sys.argv:
+        print(build_torch_shim(verbose=True))

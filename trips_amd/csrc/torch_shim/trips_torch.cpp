@@ -1,0 +1,392 @@
+// Implementation of trips_torch.h: marshals libtorch tensors into the C ABI. No kernels here.
+#include "trips_torch.h"
+
+#include <c10/hip/HIPStream.h>
+#include <torch/custom_class.h>
+#include <torch/library.h>
+
+#include <cfloat>
+#include <stdexcept>
+#include <string>
+
+namespace
+{
+struct Ctx
+{
+    TripsCtx* ctx = nullptr;
+    int device    = -1;
+};
+
+TripsCtx* context_for(const torch::Tensor& t)
+{
+    static thread_local Ctx cached;
+    TORCH_CHECK(t.is_cuda(), "trips: tensors must live on the GPU (there is no CPU implementation of the splat path)");
+    const int dev = t.get_device();
+    if (cached.ctx && cached.device == dev) return cached.ctx;
+    TripsCtx* c = nullptr;
+    int rc      = trips_ctx_create(&c, dev);
+    TORCH_CHECK(rc == TRIPS_OK, "trips_ctx_create: ", trips_last_error_string());
+    cached.ctx    = c;
+    cached.device = dev;
+    return c;
+}
+
+void* current_stream(const torch::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
+
+void check(int rc, const char* what)
+{
+    TORCH_CHECK(rc == TRIPS_OK, what, ": ", trips_last_error_string());
+}
+
+TripsSplatDesc make_desc(const NeuralRenderInfo& info, const torch::Tensor& texture)
+{
+    const RenderParams& p = info.params;
+    TORCH_CHECK(p.render_mode == 4 && p.use_layer_point_size && p.render_points_in_all_lower_resolutions &&
+                    !p.combine_lists,
+                "trips: only render_mode 4 (TILED_BILINEAR_BLEND) with use_layer_point_size, "
+                "render_points_in_all_lower_resolutions and !combine_lists is implemented");
+    TORCH_CHECK(info.scene, "NeuralRenderInfo::scene is null");
+    TORCH_CHECK(!info.images.empty() && info.images.size() <= TRIPS_MAX_VIEWS, "1..", TRIPS_MAX_VIEWS, " images per call");
+    TripsSplatDesc d{};
+    d.abi_version               = TRIPS_ABI_VERSION;
+    d.num_points                = info.scene->point_cloud_cuda->Size();
+    d.num_texels                = (int)texture.size(1);
+    d.num_channels              = (int)texture.size(0);
+    d.num_layers                = info.num_layers;
+    d.list_depth                = p.max_pixels_per_list;
+    d.num_views                 = (int)info.images.size();
+    d.num_images                = (int)info.scene->poses->poses_se3.size(0);
+    d.num_cameras               = (int)info.scene->intrinsics->intrinsics.size(0);
+    d.train                     = info.train ? 1 : 0;
+    d.layout                    = info.train ? TRIPS_LAYOUT_CHW : TRIPS_LAYOUT_HWC;
+    d.floor_layer_sizes         = p.floor_layer_sizes ? 1 : 0;
+    d.background_mode           = p.background_mode;
+    d.drop_out_points_by_radius = p.drop_out_points_by_radius ? 1 : 0;
+    d.drop_out_radius_threshold = p.drop_out_radius_threshold;
+    d.dist_cutoff               = p.dist_cutoff;
+    d.viewer_only               = p.viewer_only ? 1 : 0;
+    d.stability_cutoff_value    = p.stability_cutoff_value;
+    d.max_list_entries          = 0;
+    for (size_t i = 0; i < info.images.size(); ++i)
+    {
+        const ReducedImageInfo& im = info.images[i];
+        TripsView& v               = d.views[i];
+        v.w                        = im.w;
+        v.h                        = im.h;
+        v.image_index              = im.image_index;
+        v.camera_index             = im.camera_index;
+        v.camera_model_type        = im.camera_model_type;
+        for (int k = 0; k < 5; ++k) v.crop_transform[k] = im.crop_transform[k];
+        for (int k = 0; k < 4; ++k) v.crop_rotation[k] = im.crop_rotation[k];
+    }
+    return d;
+}
+
+torch::Tensor alloc_bytes(size_t n, const torch::Device& dev)
+{
+    return torch::empty({(int64_t)std::max<size_t>(n, 256)}, torch::TensorOptions().dtype(torch::kUInt8).device(dev));
+}
+
+struct SavedForBackward : public torch::CustomClassHolder
+{
+    TripsSplatDesc desc;
+    torch::Tensor saved_state;
+    torch::Tensor position, point_size, index, texture, confidence, background, poses_se3, intrinsics, dropout;
+};
+
+TripsSplatIn make_in(const SavedForBackward& s)
+{
+    TripsSplatIn in{};
+    in.position   = s.position.data_ptr<float>();
+    in.point_size = s.point_size.data_ptr<float>();
+    in.index      = s.index.data_ptr<int32_t>();
+    in.texture    = s.texture.data_ptr<float>();
+    in.confidence = s.confidence.data_ptr<float>();
+    in.background = s.background.data_ptr<float>();
+    in.poses_se3  = s.poses_se3.data_ptr<double>();
+    in.intrinsics = s.intrinsics.data_ptr<float>();
+    in.dropout    = s.dropout.defined() ? s.dropout.data_ptr<float>() : nullptr;
+    return in;
+}
+}  // namespace
+
+// custom classes travel through IValue / saved_data, as in the reference (RenderInfo.cpp:14-18)
+TORCH_LIBRARY(trips_amd, m)
+{
+    m.class_<NeuralRenderInfo>("NeuralRenderInfo").def(torch::init());
+    m.class_<SavedForBackward>("SavedForBackward").def(torch::init());
+}
+
+void PointRendererCache::Build(NeuralRenderInfo* info, const TripsSplatDesc& d, size_t workspace_bytes)
+{
+    std::vector<int64_t> key = {d.num_channels, d.num_points, d.num_layers, d.num_views,
+                                d.views[0].h,   d.views[0].w, d.list_depth, d.train};
+    const auto dev           = info->scene->texture->texture.device();
+    if (key != cache_size || !workspace.defined() || (size_t)workspace.numel() < workspace_bytes)
+    {
+        workspace      = alloc_bytes(workspace_bytes, dev);
+        cache_size     = key;
+        dropout_points = torch::Tensor();
+    }
+    if (info->train && info->params.dropout > 0)
+    {
+        if (!dropout_points.defined())
+            dropout_points = torch::empty({d.num_views, d.num_points}, torch::TensorOptions().dtype(torch::kFloat32).device(dev));
+        dropout_points.bernoulli_(info->params.dropout);
+    }
+    else
+    {
+        dropout_points = torch::Tensor();
+    }
+}
+
+namespace torch::autograd
+{
+variable_list PointRender::forward(AutogradContext* ctx, Variable texture, Variable background_color, Variable points,
+                                   Variable pose_tangents, Variable intrinsics, Variable confidence,
+                                   Variable dynamic_refinement, Variable layer_of_point, IValue info_v)
+{
+    (void)dynamic_refinement;
+    ctx->saved_data["render_info"] = info_v;
+    NeuralRenderInfo* info         = info_v.toCustomClass<NeuralRenderInfo>().get();
+    TORCH_CHECK(info->cache, "NeuralRenderInfo::cache is null");
+    TripsCtx* tc = context_for(texture);
+
+    auto s          = c10::make_intrusive<SavedForBackward>();
+    s->desc         = make_desc(*info, texture);
+    s->position     = points.contiguous();
+    s->point_size   = layer_of_point.contiguous();
+    s->index        = info->scene->point_cloud_cuda->t_index.contiguous();
+    s->texture      = texture.contiguous();
+    s->confidence   = confidence.contiguous();
+    s->background   = background_color.contiguous();
+    s->poses_se3    = info->scene->poses->poses_se3.contiguous();
+    s->intrinsics   = intrinsics.contiguous();
+    TORCH_CHECK(s->index.scalar_type() == torch::kInt32 && s->poses_se3.scalar_type() == torch::kFloat64 &&
+                    pose_tangents.scalar_type() == torch::kFloat64,
+                "t_index must be int32, poses_se3 / tangent_poses float64");
+    const TripsSplatDesc& d = s->desc;
+
+    size_t ws_bytes = 0, saved_bytes = 0;
+    check(trips_splat_workspace_size(&d, &ws_bytes), "trips_splat_workspace_size");
+    check(trips_splat_saved_size(&d, &saved_bytes), "trips_splat_saved_size");
+    info->cache->Build(info, d, ws_bytes);
+    s->dropout = info->cache->dropout_points;
+    if (info->train) s->saved_state = alloc_bytes(saved_bytes, texture.device());
+
+    int32_t lw[TRIPS_MAX_LAYERS], lh[TRIPS_MAX_LAYERS];
+    check(trips_splat_layer_sizes(&d, lw, lh), "trips_splat_layer_sizes");
+    variable_list images;
+    TripsSplatOut out{};
+    for (int l = 0; l < d.num_layers; ++l)
+    {
+        auto opt = torch::TensorOptions().dtype(torch::kFloat32).device(texture.device());
+        images.push_back(info->train ? torch::empty({d.num_views, d.num_channels, lh[l], lw[l]}, opt)
+                                     : torch::empty({d.num_views, lh[l], lw[l], d.num_channels}, opt));
+        out.image[l] = images.back().data_ptr<float>();
+    }
+    out.saved       = info->train ? s->saved_state.data_ptr() : nullptr;
+    TripsSplatIn in = make_in(*s);
+    check(trips_splat_forward(tc, &d, &in, &out, info->cache->workspace.data_ptr(), (size_t)info->cache->workspace.numel(),
+                              current_stream(texture)),
+          "trips_splat_forward");
+    ctx->saved_data["trips_saved"] = IValue(s);
+    if (!info->train)
+        for (auto& im : images) im = im.permute({0, 3, 1, 2});  // PointRenderer.cu:747-749
+    return images;
+}
+
+variable_list PointRender::backward(AutogradContext* ctx, variable_list grad_output)
+{
+    IValue info_v          = ctx->saved_data["render_info"];
+    NeuralRenderInfo* info = info_v.toCustomClass<NeuralRenderInfo>().get();
+    auto s                 = ctx->saved_data["trips_saved"].toCustomClass<SavedForBackward>();
+    TORCH_CHECK(s->saved_state.defined(), "PointRender::backward needs a forward with info->train == true");
+    const TripsSplatDesc& d = s->desc;
+    TripsCtx* tc            = context_for(s->texture);
+    const auto dev          = s->texture.device();
+
+    // zero-initialised outputs as PointRendererCache::Build(info, false) creates them (PointRenderer.cu:226-272)
+    torch::Tensor g_texture    = torch::zeros_like(s->texture);
+    torch::Tensor g_confidence = torch::zeros_like(s->confidence);
+    torch::Tensor g_background = torch::zeros_like(s->background);
+    torch::Tensor g_points, g_layer, g_pose, g_intrinsics;
+    if (ctx->needs_input_grad(2)) g_points = torch::zeros_like(s->position);
+    if (ctx->needs_input_grad(7)) g_layer = torch::zeros_like(s->point_size);
+    if (ctx->needs_input_grad(3))
+        g_pose = torch::zeros({d.num_images, 6}, torch::TensorOptions().dtype(torch::kFloat64).device(dev));
+    if (ctx->needs_input_grad(4)) g_intrinsics = torch::zeros_like(s->intrinsics);
+
+    std::vector<torch::Tensor> gi;
+    const float* gptr[TRIPS_MAX_LAYERS] = {};
+    for (int l = 0; l < d.num_layers; ++l)
+    {
+        TORCH_CHECK(grad_output[l].defined() && grad_output[l].scalar_type() == torch::kFloat32, "image gradient ", l);
+        gi.push_back(grad_output[l].contiguous());
+        gptr[l] = gi.back().data_ptr<float>();
+    }
+    TripsSplatGrads g{};
+    g.d_texture     = g_texture.data_ptr<float>();
+    g.d_confidence  = g_confidence.data_ptr<float>();
+    g.d_background  = g_background.data_ptr<float>();
+    g.d_position    = g_points.defined() ? g_points.data_ptr<float>() : nullptr;
+    g.d_point_size  = g_layer.defined() ? g_layer.data_ptr<float>() : nullptr;
+    g.d_pose        = g_pose.defined() ? g_pose.data_ptr<double>() : nullptr;
+    g.d_intrinsics  = g_intrinsics.defined() ? g_intrinsics.data_ptr<float>() : nullptr;
+    TripsSplatIn in = make_in(*s);
+    check(trips_splat_backward(tc, &d, &in, s->saved_state.data_ptr(), gptr, &g, info->cache->workspace.data_ptr(),
+                               (size_t)info->cache->workspace.numel(), current_stream(s->texture)),
+          "trips_splat_backward");
+    // order of PointRenderer.cu:1423-1426 (dynamic-refinement gradient undefined), then one for `info`
+    return {g_texture, g_background, g_points, g_pose, g_intrinsics, g_confidence, Variable(), g_layer, Variable()};
+}
+}  // namespace torch::autograd
+
+std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info)
+{
+    torch::intrusive_ptr<NeuralRenderInfo> render_data = torch::make_intrusive<NeuralRenderInfo>(*info);
+    TORCH_CHECK(render_data->scene && render_data->scene->texture, "scene / texture missing");
+    if (!render_data->scene->dynamic_refinement_t.defined())
+        render_data->scene->dynamic_refinement_t = torch::zeros({1}, render_data->scene->texture->texture.options());
+    return torch::autograd::PointRender::apply(
+        render_data->scene->texture->texture, render_data->scene->texture->background_color,
+        render_data->scene->point_cloud_cuda->t_position, render_data->scene->poses->tangent_poses,
+        render_data->scene->intrinsics->intrinsics, render_data->scene->texture->confidence_value_of_point,
+        render_data->scene->dynamic_refinement_t, render_data->scene->point_cloud_cuda->t_point_size,
+        torch::IValue(render_data));
+}
+
+void ApplyTangentToPose(torch::Tensor tangent, torch::Tensor pose)
+{
+    TORCH_CHECK(tangent.is_contiguous() && pose.is_contiguous(), "tangent / pose must be contiguous");
+    TORCH_CHECK(tangent.scalar_type() == torch::kFloat64 && pose.scalar_type() == torch::kFloat64, "float64 expected");
+    check(trips_apply_tangent(context_for(pose), tangent.data_ptr<double>(), pose.data_ptr<double>(), (int)tangent.size(0),
+                              current_stream(pose)),
+          "trips_apply_tangent");
+}
+
+void PoseModule_::ApplyTangent() { ApplyTangentToPose(tangent_poses, poses_se3); }
+
+namespace torch::optim
+{
+MyAdam::MyAdam(std::vector<OptimizerParamGroup> param_groups, MyAdamOptions defaults)
+    : Optimizer(std::move(param_groups), std::make_unique<MyAdamOptions>(defaults))
+{
+    TORCH_CHECK(defaults.lr() >= 0, "Invalid learning rate: ", defaults.lr());
+    TORCH_CHECK(defaults.eps() >= 0, "Invalid epsilon value: ", defaults.eps());
+    auto betas = defaults.betas();
+    TORCH_CHECK(0 <= std::get<0>(betas) && std::get<0>(betas) < 1.0, "Invalid beta parameter at index 0: ", std::get<0>(betas));
+    TORCH_CHECK(0 <= std::get<1>(betas) && std::get<1>(betas) < 1.0, "Invalid beta parameter at index 1: ", std::get<1>(betas));
+    TORCH_CHECK(defaults.relative_weight_decay() >= 0, "Invalid relative_weight_decay value: ", defaults.relative_weight_decay());
+    TORCH_CHECK(defaults.absolute_weight_decay() >= 0, "Invalid absolute_weight_decay value: ", defaults.absolute_weight_decay());
+}
+
+torch::Tensor MyAdam::step(LossClosure closure)
+{
+    NoGradGuard no_grad;
+    Tensor loss = {};
+    if (closure != nullptr)
+    {
+        at::AutoGradMode enable_grad(true);
+        loss = closure();
+    }
+    std::vector<TripsAdamTensor> descs;
+    std::vector<Tensor> keep;
+    Tensor any;
+    for (auto& group : param_groups_)
+    {
+        for (auto& p : group.params())
+        {
+            if (!p.grad().defined()) continue;
+            auto grad = p.grad();
+            TORCH_CHECK(!grad.is_sparse(), "Adam does not support sparse gradients");
+            TORCH_CHECK(p.is_contiguous(), "MyAdam needs contiguous parameters");
+            TORCH_CHECK(p.scalar_type() == torch::kFloat || p.scalar_type() == torch::kDouble, "float32 / float64 only");
+            auto& options = static_cast<MyAdamOptions&>(group.options());
+            auto it       = state_.find(p.unsafeGetTensorImpl());
+            if (it == state_.end())
+            {
+                auto st = std::make_unique<MyAdamParamState>();
+                st->param_steps(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kInt64));
+                st->first_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
+                st->second_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
+                st->current_step(0);
+                state_[p.unsafeGetTensorImpl()] = std::move(st);
+            }
+            auto& st = static_cast<MyAdamParamState&>(*state_[p.unsafeGetTensorImpl()]);
+            st.current_step(st.current_step() + 1);
+            const double beta1 = std::get<0>(options.betas()), beta2 = std::get<1>(options.betas());
+            float lower = 0, upper = FLT_MAX;
+            if (options.adabound())
+            {
+                // AdaBound bounds, MyAdam.cu:213-221
+                lower = 0.1f - 0.1f / ((1 - (float)beta2) * (float)st.current_step() + 1);
+                upper = 0.1f + 0.1f / ((1 - (float)beta2) * (float)st.current_step());
+            }
+            Tensor g = grad.contiguous();
+            keep.push_back(g);
+            TripsAdamTensor t{};
+            t.weights                   = p.data_ptr();
+            t.grads                     = g.data_ptr();
+            t.first_moment              = st.first_moments().data_ptr<float>();
+            t.second_moment             = st.second_moments().data_ptr<float>();
+            t.steps                     = st.param_steps().data_ptr<int64_t>();
+            t.n                         = p.numel();
+            t.dtype                     = p.scalar_type() == torch::kDouble ? TRIPS_DTYPE_F64 : TRIPS_DTYPE_F32;
+            t.lr                        = (float)options.lr();
+            t.beta1                     = (float)beta1;
+            t.beta2                     = (float)beta2;
+            t.eps                       = (float)options.eps();
+            t.relative_weight_decay     = (float)options.relative_weight_decay();
+            t.absolute_weight_decay     = (float)options.absolute_weight_decay();
+            t.weight_clipping_magnitude = (float)options.weight_clipping_magnitude();
+            t.lower_lr_bound            = lower;
+            t.upper_lr_bound            = upper;
+            t.loss_scale                = 1.f;
+            descs.push_back(t);
+            any = p;
+        }
+    }
+    if (!descs.empty())
+        check(trips_adam_step_fused(context_for(any), descs.data(), (int)descs.size(), current_stream(any)),
+              "trips_adam_step_fused");
+    return loss;
+}
+
+// state follows the last dimension of the parameter (MyAdam.cu:346-415)
+void MyAdam::shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep)
+{
+    TORCH_CHECK(param_group_index < (int)param_groups_.size());
+    for (auto& p : param_groups_[param_group_index].params())
+    {
+        auto it = state_.find(p.unsafeGetTensorImpl());
+        if (it == state_.end()) continue;
+        auto& st   = static_cast<MyAdamParamState&>(*it->second);
+        auto keepf = [&](torch::Tensor t)
+        { return t.index_select(t.dim() - 1, indices_to_keep.squeeze().to(t.device())).contiguous(); };
+        st.first_moments(keepf(st.first_moments()));
+        st.second_moments(keepf(st.second_moments()));
+        st.param_steps(keepf(st.param_steps()));
+    }
+}
+
+void MyAdam::appendToInternalState(int param_group_index, int new_size)
+{
+    TORCH_CHECK(param_group_index < (int)param_groups_.size());
+    for (auto& p : param_groups_[param_group_index].params())
+    {
+        auto it = state_.find(p.unsafeGetTensorImpl());
+        if (it == state_.end()) continue;
+        auto& st  = static_cast<MyAdamParamState&>(*it->second);
+        auto grow = [&](torch::Tensor t)
+        {
+            std::vector<int64_t> sizes(t.sizes().begin(), t.sizes().end());
+            sizes.back() = new_size - t.size(-1);
+            return torch::cat({t, torch::zeros(sizes, t.options())}, -1).contiguous();
+        };
+        st.first_moments(grow(st.first_moments()));
+        st.second_moments(grow(st.second_moments()));
+        st.param_steps(grow(st.param_steps()));
+    }
+}
+}  // namespace torch::optim

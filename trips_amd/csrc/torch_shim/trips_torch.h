@@ -1,0 +1,173 @@
+// libtorch host side of the splat path: the reference's operator surface over the C ABI (include/trips_splat.h).
+//
+// Same names, argument order and return arity as the reference so that its callers compile unchanged against
+// this header for the render path (paths relative to the reference checkout):
+//   ReducedImageInfo             src/lib/data/SceneData.h:40-61
+//   RenderParams (subset)        src/lib/data/Settings.h:19-83
+//   NeuralRenderInfo             src/lib/rendering/PointRenderer.h:23-34
+//   PointRendererCache           src/lib/rendering/PointRenderer.h:120-232
+//   torch::autograd::PointRender src/lib/rendering/PointRenderer.h:39-47, RenderInfo.cpp:44-80
+//   BlendPointCloud              src/lib/rendering/PointRenderer.h:53, RenderInfo.cpp:27-40
+//   ApplyTangentToPose           src/lib/rendering/PointRenderer.h:64, PointRenderer.cu:1449-1456
+//   torch::optim::MyAdam         src/lib/models/MyAdam.h:28-85
+// Saiga / Sophus types of the reference (IntrinsicsPinholef, Matrix<float,2,2>, CudaTimerSystem) are replaced by
+// plain arrays and an opaque pointer; NeuralScene is reduced to the tensors the operator reads.
+#pragma once
+#include <torch/torch.h>
+
+#include <array>
+#include <memory>
+#include <vector>
+
+#include "../../../include/trips_splat.h"
+
+struct ReducedImageInfo
+{
+    int w = 0, h = 0;
+    int image_index          = -1;
+    int camera_index         = -1;
+    int camera_model_type    = 0;                        // CameraModel::PINHOLE_DISTORTION
+    std::array<float, 5> crop_transform = {1, 1, 0, 0, 0};  // fx fy cx cy s
+    std::array<float, 4> crop_rotation  = {1, 0, 0, 1};     // row-major 2x2
+};
+
+struct RenderParams
+{
+    float dropout                               = 0.25f;
+    float drop_out_radius_threshold             = 0.6f;
+    bool drop_out_points_by_radius              = true;
+    int num_texture_channels                    = -1;
+    float dist_cutoff                           = 20.f;
+    float stability_cutoff_value                = 10000.f;
+    bool viewer_only                            = false;
+    int render_mode                             = 4;  // TILED_BILINEAR_BLEND, the only mode implemented
+    bool use_layer_point_size                   = true;
+    bool combine_lists                          = false;
+    bool render_points_in_all_lower_resolutions = true;
+    bool normalize_grads                        = false;
+    // not in the reference
+    int background_mode     = TRIPS_BG_REFERENCE;
+    int max_pixels_per_list = 16;  // PointRenderer.h:178
+    bool floor_layer_sizes  = false;  // network_version == "MultiScaleUnet2d", PointRenderer.cu:385-394
+};
+
+// The tensors of the reference's NeuralScene that the operator reads, under the same member paths.
+struct NeuralTexture_
+{
+    torch::Tensor texture;                    // [C,N]
+    torch::Tensor background_color;           // [C]
+    torch::Tensor confidence_value_of_point;  // [1,N]
+};
+struct NeuralPointCloudCuda_
+{
+    torch::Tensor t_position;    // [N,4]
+    torch::Tensor t_point_size;  // [N,1]
+    torch::Tensor t_index;       // [N,1] int32
+    int Size() const { return (int)t_position.size(0); }
+};
+struct PoseModule_
+{
+    torch::Tensor poses_se3;      // [F,8] f64
+    torch::Tensor tangent_poses;  // [F,6] f64
+    void ApplyTangent();
+};
+struct IntrinsicsModule_
+{
+    torch::Tensor intrinsics;  // [Cam,13]
+};
+struct NeuralScene
+{
+    std::shared_ptr<NeuralTexture_> texture                 = std::make_shared<NeuralTexture_>();
+    std::shared_ptr<NeuralPointCloudCuda_> point_cloud_cuda = std::make_shared<NeuralPointCloudCuda_>();
+    std::shared_ptr<PoseModule_> poses                      = std::make_shared<PoseModule_>();
+    std::shared_ptr<IntrinsicsModule_> intrinsics           = std::make_shared<IntrinsicsModule_>();
+    torch::Tensor dynamic_refinement_t;  // dummy [1] tensor when no displacement is optimised
+};
+
+class PointRendererCache;
+
+class NeuralRenderInfo : public torch::CustomClassHolder
+{
+   public:
+    NeuralScene* scene = nullptr;
+    std::vector<ReducedImageInfo> images;
+    RenderParams params;
+    int num_layers            = 1;
+    bool train                = true;
+    int current_epoch         = 0;
+    void* timer_system        = nullptr;  // accepted for interface parity (CUDA::CudaTimerSystem* in the reference)
+    PointRendererCache* cache = nullptr;
+};
+
+class PointRendererCache
+{
+   public:
+    // (Re)allocates the workspace when the size key changes and draws the drop-out mask (PointRenderer.cu:285-309,516-521)
+    void Build(NeuralRenderInfo* info, const TripsSplatDesc& desc, size_t workspace_bytes);
+
+    torch::Tensor workspace;       // uint8
+    torch::Tensor dropout_points;  // [batch, num_points] or undefined
+    std::vector<int64_t> cache_size;
+};
+
+namespace torch::autograd
+{
+struct PointRender : public Function<PointRender>
+{
+    // returns a tensor for every layer
+    static variable_list forward(AutogradContext* ctx, Variable texture, Variable background_color, Variable points,
+                                 Variable pose_tangents, Variable intrinsics, Variable confidence,
+                                 Variable dynamic_refinement, Variable layer_value_of_point, IValue info);
+    static variable_list backward(AutogradContext* ctx, variable_list grad_output);
+};
+}  // namespace torch::autograd
+
+// Render the scene into a batch of images; every image is a pyramid of layers in different resolutions
+std::vector<torch::Tensor> BlendPointCloud(NeuralRenderInfo* info);
+
+void ApplyTangentToPose(torch::Tensor tangent, torch::Tensor pose);
+
+namespace torch::optim
+{
+struct MyAdamOptions : public OptimizerCloneableOptions<MyAdamOptions>
+{
+    MyAdamOptions(double lr = 1e-3) { set_lr(lr); }
+    TORCH_ARG(double, lr) = 1e-3;
+    typedef std::tuple<double, double> betas_t;
+    TORCH_ARG(betas_t, betas)                    = std::make_tuple(0.9, 0.999);
+    TORCH_ARG(double, eps)                       = 1e-8;
+    TORCH_ARG(double, relative_weight_decay)     = 0;
+    TORCH_ARG(double, absolute_weight_decay)     = 0;
+    TORCH_ARG(double, weight_clipping_magnitude) = 0;
+    TORCH_ARG(bool, adabound)                    = false;
+
+   public:
+    ~MyAdamOptions() override = default;
+    double get_lr() const override { return lr(); }
+    void set_lr(const double lr) override { this->lr(lr); }
+};
+
+struct MyAdamParamState : public OptimizerCloneableParamState<MyAdamParamState>
+{
+    TORCH_ARG(torch::Tensor, param_steps);
+    TORCH_ARG(torch::Tensor, first_moments);
+    TORCH_ARG(torch::Tensor, second_moments);
+    TORCH_ARG(int64_t, current_step) = 0;
+
+   public:
+    ~MyAdamParamState() override = default;
+};
+
+class MyAdam : public Optimizer
+{
+   public:
+    explicit MyAdam(std::vector<OptimizerParamGroup> param_groups, MyAdamOptions defaults = {});
+    explicit MyAdam(std::vector<Tensor> params, MyAdamOptions defaults = {})
+        : MyAdam({OptimizerParamGroup(std::move(params))}, defaults)
+    {
+    }
+    torch::Tensor step(LossClosure closure = nullptr) override;
+    void shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep);
+    void appendToInternalState(int param_group_index, int new_size);
+};
+}  // namespace torch::optim
