@@ -42,6 +42,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--points", type=int, default=6_000_000)
     ap.add_argument("--cpu-steps", type=int, default=3, help="oracle steps for the cpu_baseline sample (0 = skip)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); nothing here shards across devices",
@@ -124,6 +126,13 @@ def main():
     achieved = kernels[dom]["alg_GBs"]
     kernel_ms = sum(v["avg_ms"] * v["launches_per_step"] for v in kernels.values())
     fwd_bwd_ms = sum(v["avg_ms"] * v["launches_per_step"] for k, v in kernels.items() if k != "adam_fused")
+
+    if args.calibration_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     cpu = None
     if args.cpu_steps > 0:

@@ -1,0 +1,79 @@
+"""Committed fixture tests/golden/splat_small.npz (inputs + expected outputs, made by tests/golden/make_golden.py):
+the oracle must keep reproducing it (CPU) and the HIP path must match it without the oracle in the loop (GPU)."""
+import os
+
+import numpy as np
+import pytest
+
+from trips_amd import abi, scenes
+
+PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "splat_small.npz")
+
+
+def _scene(z):
+    poses = z["poses_se3"]
+    views = [dict(w=48, h=40, image_index=i, camera_index=0) for i in range(poses.shape[0])]
+    views[1]["crop_transform"] = tuple(float(x) for x in z["crop_transform_1"])
+    return scenes.Scene(name="golden", position=z["position"], point_size=z["point_size"], index=z["index"],
+                        texture=z["texture"], confidence=z["confidence"], background=z["background"],
+                        poses_se3=poses, intrinsics=z["intrinsics"], views=views, num_layers=3, list_depth=16)
+
+
+def test_oracle_reproduces_golden(oracle):
+    z = np.load(PATH)
+    sc = _scene(z)
+    for mode, tag in ((abi.TRIPS_BG_REFERENCE, "ref"), (abi.TRIPS_BG_CONSISTENT, "con")):
+        d = abi.desc_for_scene(sc, background_mode=mode)
+        fwd = oracle.forward(sc, d)
+        for l, im in enumerate(fwd["images"]):
+            np.testing.assert_allclose(im, z[f"image_{tag}_{l}"], rtol=1e-6, atol=1e-7)
+        if tag == "ref":
+            for k in ("depth", "ip", "size_px", "max_layer", "lengths", "lists", "retained", "counters"):
+                np.testing.assert_array_equal(fwd[k], z[k], err_msg=k)
+            g = oracle.backward(sc, d, fwd, [z[f"grad_image_{l}"] for l in range(3)])
+            for k, v in g.items():
+                scale = np.abs(z[k]).max() + 1e-30
+                assert np.abs(v - z[k]).max() / scale < 1e-5, k
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_golden():
+    import torch
+    from tests.gpu_util import GpuRun, rel_err
+    from trips_amd.renderer import get_context
+    z = np.load(PATH)
+    sc = _scene(z)
+    for mode, tag in ((abi.TRIPS_BG_REFERENCE, "ref"), (abi.TRIPS_BG_CONSISTENT, "con")):
+        run = GpuRun(sc, abi.desc_for_scene(sc, background_mode=mode))
+        imgs = run.forward()
+        for l, im in enumerate(imgs):
+            np.testing.assert_allclose(im, z[f"image_{tag}_{l}"], rtol=1e-5, atol=1e-6)
+        if tag == "ref":
+            for b in range(2):
+                lists, retained, lengths = run.lists(b)
+                np.testing.assert_array_equal(lists, z["lists"][b])
+                np.testing.assert_array_equal(retained, z["retained"][b])
+                np.testing.assert_array_equal(lengths, z["lengths"][b])
+                ip, depth, size_px, max_layer = run.points(b)
+                np.testing.assert_array_equal(depth, z["depth"][b])
+                np.testing.assert_array_equal(ip, z["ip"][b])
+                np.testing.assert_array_equal(max_layer, z["max_layer"][b])
+            g = run.backward([z[f"grad_image_{l}"] for l in range(3)])
+            for k, v in g.items():
+                assert rel_err(v, z[k]) < 1e-4, k
+            # one Adam step on the positions with the golden gradient
+            ctx = get_context(0)
+            n = sc.position.size
+            w = torch.as_tensor(sc.position.reshape(-1).copy()).cuda()
+            gt = torch.as_tensor(z["d_position"].reshape(-1)).cuda()
+            m, v2 = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+            steps = torch.zeros(n, dtype=torch.int64, device="cuda")
+            t = abi.TripsAdamTensor()
+            t.weights, t.grads, t.first_moment, t.second_moment, t.steps = (w.data_ptr(), gt.data_ptr(), m.data_ptr(),
+                                                                          v2.data_ptr(), steps.data_ptr())
+            t.n, t.dtype, t.lr, t.beta1, t.beta2, t.eps = n, abi.TRIPS_DTYPE_F32, 1e-3, 0.9, 0.999, 1e-8
+            t.lower_lr_bound, t.upper_lr_bound, t.loss_scale = 0.0, abi.FLT_MAX, 1.0
+            ctx.adam_step([t])
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(steps.cpu().numpy(), z["adam_steps"])
+            np.testing.assert_allclose(w.cpu().numpy(), z["adam_position"], rtol=2e-6, atol=1e-7)
