@@ -27,10 +27,11 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0):
     (N points, E list entries, R retained entries, P pyramid pixels)."""
     N, E, R, P, C = n_points, c["E"], c["R"], c["P"], channels
     return {
-        "project_count": 24 * N,                                  # position 16 + size 4 + index 4
-        "scatter_keys": 8 * E,                                    # one 64-bit key written per entry
+        "project_bin": 24 * N,                                    # position 16 + size 4 + index 4
+        "tile_scatter": 8 * E,                                    # one 64-bit key written per entry
         "sort_blend": 8 * E + (20 + 4 + 4 * C + 28) * R + 4 * C * P,  # keys read, record+conf+descriptor, saved, image
-        "blend_backward": 4 * C * P + (76 + 8 * C) * R,
+        "backward_pixels": 4 * C * P + (28 + 4 * C + 4 + 20) * R,  # dL/dimage, saved entry, descriptor+conf+record
+        "backward_points": (4 * C + 4 + 12 + 4) * R,              # one write per accumulated gradient float
         "adam_fused": 44 * adam_nonzero + 8 * adam_zero,
     }
 

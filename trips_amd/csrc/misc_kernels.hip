@@ -253,6 +253,37 @@ hipError_t launch_export_points(const float* rec, int rec_floats, int n, float* 
     return hipGetLastError();
 }
 
+// saved tables are tile-major (padded); the exports are row-major, layer by layer
+__global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, int K, const int32_t* __restrict__ lists,
+                                                           const int32_t* __restrict__ retained,
+                                                           const int32_t* __restrict__ lengths, int32_t* out_lists,
+                                                           int32_t* out_retained, int32_t* out_lengths)
+{
+    const int P = g.off[g.num_layers];
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= P) return;
+    int layer = 0;
+    while (layer + 1 < g.num_layers && r >= g.off[layer + 1]) ++layer;
+    const int local = r - g.off[layer];
+    const int x = local % g.w[layer], y = local / g.w[layer];
+    const int ip = pix_index(g, layer, x, y);
+    if (out_retained) out_retained[r] = retained[ip];
+    if (out_lengths) out_lengths[r] = lengths[ip];
+    if (out_lists)
+        for (int k = 0; k < K; ++k) out_lists[(size_t)r * K + k] = lists[(size_t)ip * K + k];
+}
+
+hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
+                               const int32_t* lengths, int32_t* out_lists, int32_t* out_retained, int32_t* out_lengths,
+                               hipStream_t stream)
+{
+    const int P = g.off[g.num_layers];
+    if (P <= 0) return hipSuccess;
+    hipLaunchKernelGGL(export_lists_kernel, dim3((P + 255) / 256), dim3(256), 0, stream, g, K, lists, retained, lengths,
+                       out_lists, out_retained, out_lengths);
+    return hipGetLastError();
+}
+
 __global__ __launch_bounds__(256) void sum_i32_kernel(const int32_t* __restrict__ v, long long n,
                                                       unsigned long long* out)
 {

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
     const int lane     = threadIdx.x & 63;
     const int sub      = lane & 15;
     const int grp      = lane >> 4;
-    const int P        = p.geom.off[p.num_layers];
+    const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
 
     double acc_bg[C];
@@ -82,13 +82,10 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
     for (long long wv = wave0; wv < total_waves; wv += wave_stride)
     {
         const long long pix_ll = wv * 4 + grp;
-        const bool live        = pix_ll < P;
-        const int pix          = live ? (int)pix_ll : 0;
-        int layer              = 0;
-        while (layer + 1 < p.num_layers && pix >= p.geom.off[layer + 1]) ++layer;
-        const int local = pix - p.geom.off[layer];
+        const int pix          = pix_ll < P ? (int)pix_ll : 0;
+        int layer, gx, gy;
+        const bool live = pix_decode(p.geom, pix, layer, gx, gy) && pix_ll < P;
         const int lw = p.geom.w[layer], lh = p.geom.h[layer];
-        const int gx = local % lw, gy = local / lw;
 
         const int m    = live ? p.retained[pix] : 0;
         const bool has = sub < m;
@@ -266,7 +263,6 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             const float fx = floorf(ux), fy = floorf(uy);
             const int px = (int)fx, py = (int)fy;
             const float sx = ux - fx, sy = uy - fy;
-            const int lw = p.geom.w[layer];
             float lfac = 1.f, J_lf = 0.f;
             if (want_size) lfac = layer_factor(r0.z, layer, p.num_layers, &J_lf);
             const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
@@ -277,7 +273,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
                 if (j == 0xFFu) continue;
                 any          = true;
                 const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                const int pix = p.geom.off[layer] + gy * lw + gx;
+                const int pix = pix_index(p.geom, layer, gx, gy);
                 float e[EF];
                 {
                     const float4* src = reinterpret_cast<const float4*>(p.entry_grad + ((size_t)pix * K + j) * EF);
@@ -408,7 +404,7 @@ __global__ __launch_bounds__(256) void fill_u32_kernel(unsigned* __restrict__ p,
 
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof)
 {
-    const int P           = p.geom.off[p.num_layers];
+    const int P           = p.geom.bin_off[p.num_layers] * kTilePixels;
     const int N           = p.num_points;
     if (N <= 0) 
     {

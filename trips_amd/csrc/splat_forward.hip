@@ -1,15 +1,20 @@
 // Forward kernels of the splat path for gfx950 (wave64).
 //
-//   project_count_kernel   <- CountAndCollectTiled     src/lib/rendering/RenderForward.cu:168-366
-//   scan_*_kernel          <- cub ExclusiveSum section src/lib/rendering/RenderForward.cu:1155-1232
-//   scatter_keys_kernel    <- SplattingPass            src/lib/rendering/RenderForward.cu:368-436
-//   sort_blend_kernel      <- FastSortFusedNew         src/lib/rendering/RenderForward.cu:474-1059
+//   project_bin_kernel   <- CountAndCollectTiled (projection, validity, layer selection)
+//                           src/lib/rendering/RenderForward.cu:168-366
+//   bin_scan / bin_scatter / tile_count / tile_scatter
+//                        <- per-pixel counting (:355-361), cub ExclusiveSum section (:1155-1232) and
+//                           SplattingPass (:368-436)
+//   sort_blend_kernel    <- FastSortFusedNew    src/lib/rendering/RenderForward.cu:474-1059
 //
-// Differences in shape, not in result: all pyramid layers share ONE counter array and ONE scan (the reference
-// scans layer by layer with two blocking read-backs each); a wavefront holds four pixel lists of 16 lanes
-// (one DPP row each) instead of two per 32-lane warp; the per-point record gathered by the blend carries
-// position, size, confidence and descriptor together; what is kept for the backward is the sorted id list
-// per pixel (64 B) instead of 16 x 7 floats.
+// Differences in shape, not in result. The reference increments one global counter per (point, layer, corner),
+// scans layer by layer with two blocking read-backs each, and takes one more global atomic per entry to place
+// its key. Scattered global atomics run at about 2.7e10 per second on this GPU, so here a point is first binned
+// into 32 x 32 pixel tiles (one global atomic per (point, layer), a second one for the few footprints that cross
+// a tile border); a workgroup per tile then counts, scans and places the keys of its 1024 pixels with LDS
+// atomics. A wavefront of the sort holds four pixel lists of 16 lanes (one DPP row each) instead of two per
+// 32-lane warp; the per-point record gathered by the blend carries position, size, confidence and descriptor
+// together; what is kept for the backward is the sorted id list per pixel (64 B) instead of 16 x 7 floats.
 #include "splat_internal.h"
 #include "trips_math.h"
 
@@ -64,17 +69,24 @@ __global__ void clear_header_kernel(ViewHeader* h)
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Projection, validity, layer selection, per-pixel counting. One point per thread, grid-stride.
+// Projection, validity, layer selection, tile binning. One point per thread, grid-stride.
 template <int C, bool TRAIN>
-__global__ __launch_bounds__(256) void project_count_kernel(const ForwardParams p)
+__global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardParams p)
 {
     constexpr int CPAD = (C + 3) & ~3;
+    extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
     const Camera cam   = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L        = p.num_layers;
+    const int NB       = p.geom.bin_off[L];
     unsigned my_valid  = 0;
     bool not_identity  = false;  // some point's descriptor column differs from its own index
+    for (int i = threadIdx.x; i < NB; i += kBinThreads) s_hist[i] = 0;
+    __syncthreads();
 
-    for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
+    // a workgroup owns one contiguous chunk of points; bin_scatter_kernel walks the same chunks
+    const int chunk_begin = min(p.num_points, (int)blockIdx.x * p.points_per_block);
+    const int chunk_end   = min(p.num_points, chunk_begin + p.points_per_block);
+    for (int pid = chunk_begin + threadIdx.x; pid < chunk_end; pid += kBinThreads)
     {
         float4 ptk  = make_float4(0.f, 0.f, -1.f, 0.f);
         bool skip   = false;
@@ -124,11 +136,15 @@ __global__ __launch_bounds__(256) void project_count_kernel(const ForwardParams 
                 {
                     const int px = (int)floorf(lx), py = (int)floorf(ly);
                     if (!valid(float(px), float(py), layer, radius_px)) break;
-                    int32_t* base = p.counts + p.geom.off[layer] + py * p.geom.w[layer] + px;
-                    atomicAdd(base, 1);
-                    atomicAdd(base + 1, 1);
-                    atomicAdd(base + p.geom.w[layer], 1);
-                    atomicAdd(base + p.geom.w[layer] + 1, 1);
+                    // the 2 x 2 footprint (px..px+1, py..py+1) touches 1, 2 or 4 tiles; px+1 and py+1 are inside
+                    // the image because px < w-1 and py < h-1
+                    const int tsx = p.geom.tiles_x[layer];
+                    int* bc       = s_hist + p.geom.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
+                    const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
+                    atomicAdd(bc, 1);
+                    if (cx) atomicAdd(bc + 1, 1);
+                    if (cy) atomicAdd(bc + tsx, 1);
+                    if (cx && cy) atomicAdd(bc + tsx + 1, 1);
                 }
                 ptk = make_float4(ipx, ipy, z, __int_as_float(layer));
 
@@ -156,61 +172,43 @@ __global__ __launch_bounds__(256) void project_count_kernel(const ForwardParams 
         p.ptk[pid] = ptk;
     }
 
+    // this workgroup's row of the histogram matrix [workgroup][bin]
+    __syncthreads();
+    int32_t* row = p.bin_hist + (size_t)blockIdx.x * NB;
+    for (int i = threadIdx.x; i < NB; i += kBinThreads) row[i] = s_hist[i];
+
     // one counter update per block
-    __shared__ unsigned s_valid[4];
+    __shared__ unsigned s_valid[kBinThreads / 64];
     unsigned v = my_valid;
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
     if ((threadIdx.x & 63) == 0) s_valid[threadIdx.x >> 6] = v;
     __syncthreads();
     if (threadIdx.x == 0)
     {
-        unsigned t = s_valid[0] + s_valid[1] + s_valid[2] + s_valid[3];
+        unsigned t = 0;
+        for (int i = 0; i < kBinThreads / 64; ++i) t += s_valid[i];
         if (t) atomicAdd(&p.header->n_valid, (u64)t);
     }
     if (__ballot(not_identity) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.header->reserved[1], 1ull);
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Exclusive scan of the P per-pixel counts (all layers concatenated): reduce, spine, apply.
-__device__ __forceinline__ int block_reduce_sum(int v, int* smem)
-{
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
-    __syncthreads();
-    int t = 0;
-    for (unsigned i = 0; i < blockDim.x / 64; ++i) t += smem[i];
-    __syncthreads();
-    return t;
-}
-
-__global__ __launch_bounds__(256) void scan_reduce_kernel(const int32_t* __restrict__ counts, int32_t* __restrict__ block_sums,
-                                                          int n)
-{
-    __shared__ int smem[4];
-    const int base = blockIdx.x * kScanTile;
-    int s          = 0;
-    for (int i = threadIdx.x; i < kScanTile; i += 256)
-    {
-        int idx = base + i;
-        if (idx < n) s += counts[idx];
-    }
-    s = block_reduce_sum(s, smem);
-    if (threadIdx.x == 0) block_sums[blockIdx.x] = s;
-}
-
-// single block: exclusive scan of the block sums in place, total to the header
-__global__ __launch_bounds__(1024) void scan_spine_kernel(int32_t* __restrict__ block_sums, int nb, ViewHeader* header)
+// Exclusive scan of a short int array by ONE workgroup: out[i] = sum_{k<i} in[i], out[n] = total; optionally a
+// copy of the scan (the running slots of the scatter) and the total as a counter in the header.
+__global__ __launch_bounds__(1024) void small_scan_kernel(const int32_t* __restrict__ in, int32_t* __restrict__ out,
+                                                          int32_t* __restrict__ out_copy, int n,
+                                                          unsigned long long* total_out)
 {
     __shared__ int s_wave[16];
     __shared__ int s_carry;
     if (threadIdx.x == 0) s_carry = 0;
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int base = 0; base < nb; base += 1024)
+    for (int base = 0; base < n; base += 1024)
     {
-        int idx = base + threadIdx.x;
-        int v   = idx < nb ? block_sums[idx] : 0;
-        int inc = v;
+        const int idx = base + threadIdx.x;
+        const int v   = idx < n ? in[idx] : 0;
+        int inc       = v;
         for (int o = 1; o < 64; o <<= 1)
         {
             int t = __shfl_up(inc, o);
@@ -220,29 +218,163 @@ __global__ __launch_bounds__(1024) void scan_spine_kernel(int32_t* __restrict__ 
         __syncthreads();
         int wave_prefix = 0;
         for (int w = 0; w < wave; ++w) wave_prefix += s_wave[w];
-        int carry = s_carry;
-        if (idx < nb) block_sums[idx] = carry + wave_prefix + inc - v;
+        const int carry = s_carry;
+        if (idx < n)
+        {
+            const int ex = carry + wave_prefix + inc - v;
+            out[idx]     = ex;
+            if (out_copy) out_copy[idx] = ex;
+        }
         __syncthreads();
         if (threadIdx.x == 1023) s_carry = carry + wave_prefix + inc;
         __syncthreads();
     }
-    if (threadIdx.x == 0) header->n_entries = (u64)(unsigned)s_carry;
+    if (threadIdx.x == 0)
+    {
+        out[n] = s_carry;
+        if (total_out) *total_out = (u64)(unsigned)s_carry;
+    }
 }
 
-__global__ __launch_bounds__(256) void scan_apply_kernel(const int32_t* __restrict__ counts,
-                                                         const int32_t* __restrict__ block_sums,
-                                                         int32_t* __restrict__ cursor, int n)
+// ---------------------------------------------------------------------------------------------------------
+// Column-wise exclusive prefix of the histogram matrix [workgroup][bin]: afterwards hist[g][bin] = entries of
+// `bin` that come from workgroups before g, and bin_count[bin] = the column total. One thread per bin (rows are
+// read coalesced); no atomics anywhere in the binning, since atomics on a few thousand hot counters serialise.
+__global__ __launch_bounds__(256) void bin_column_scan_kernel(int32_t* __restrict__ hist, int32_t* __restrict__ bin_count,
+                                                              int NB, int G)
 {
-    __shared__ int s_wave[4];
-    constexpr int PER = kScanTile / 256;  // 16 consecutive elements per thread
-    const int base    = blockIdx.x * kScanTile + threadIdx.x * PER;
-    int v[PER];
-    int sum = 0;
-#pragma unroll
-    for (int i = 0; i < PER; ++i)
+    const int bin = blockIdx.x * 256 + threadIdx.x;
+    if (bin >= NB) return;
+    int run = 0;
+    int32_t* col = hist + bin;
+    for (int g = 0; g < G; g += 8)
     {
-        int idx = base + i;
-        v[i]    = idx < n ? counts[idx] : 0;
+        int v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = (g + k < G) ? col[(size_t)(g + k) * NB] : 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+        {
+            if (g + k < G) col[(size_t)(g + k) * NB] = run;
+            run += v[k];
+        }
+    }
+    bin_count[bin] = run;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// One bin entry {depth bits, point id, px | py << 16} per (point, layer, touched tile). A workgroup walks the same
+// chunk of points as in project_bin_kernel; its slots inside every bin are contiguous and start at
+// bin_start[bin] + hist[workgroup][bin].
+__global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardParams p)
+{
+    extern __shared__ int s_cur[];
+    const int NB       = p.geom.bin_off[p.num_layers];
+    const int32_t* row = p.bin_hist + (size_t)blockIdx.x * NB;
+    for (int i = threadIdx.x; i < NB; i += kBinThreads) s_cur[i] = p.bin_start[i] + row[i];
+    __syncthreads();
+    const int chunk_begin = min(p.num_points, (int)blockIdx.x * p.points_per_block);
+    const int chunk_end   = min(p.num_points, chunk_begin + p.points_per_block);
+    unsigned dropped      = 0;
+    for (int pid = chunk_begin + threadIdx.x; pid < chunk_end; pid += kBinThreads)
+    {
+        const float4 k = p.ptk[pid];
+        const float z  = k.z;
+        if (!(z > 0.f)) continue;
+        const int max_layer = __float_as_int(k.w);
+        float lx = k.x, ly = k.y;
+        for (int layer = 0; layer < max_layer; ++layer)
+        {
+            const int px = (int)floorf(lx), py = (int)floorf(ly);
+            const int tsx = p.geom.tiles_x[layer];
+            int* bc       = s_cur + p.geom.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
+            const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
+            const uint4 e = make_uint4(__float_as_uint(z), (unsigned)pid, (unsigned)px | ((unsigned)py << 16), 0u);
+            auto put = [&](int* c)
+            {
+                const int slot = atomicAdd(c, 1);
+                if ((long long)slot < p.capacity)
+                    p.bin_entries[slot] = e;
+                else
+                    dropped += 1;
+            };
+            put(bc);
+            if (cx) put(bc + 1);
+            if (cy) put(bc + tsx);
+            if (cx && cy) put(bc + tsx + 1);
+            lx *= 0.5f;
+            ly *= 0.5f;
+        }
+    }
+    if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// One workgroup per tile. Pass `SCATTER == false`: count the list length of the tile's 1024 pixels in LDS and
+// write them (plus the tile total). Pass `SCATTER == true` (after the scan of the tile totals): exclusive scan of
+// the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 | point id) into their lists.
+__device__ __forceinline__ void tile_of_bin(const PyramidGeom& g, int bin, int& layer, int& tx, int& ty)
+{
+    layer = 0;
+    while (layer + 1 < g.num_layers && bin >= g.bin_off[layer + 1]) ++layer;
+    const int t = bin - g.bin_off[layer];
+    ty          = t / g.tiles_x[layer];
+    tx          = t - ty * g.tiles_x[layer];
+}
+
+template <bool SCATTER>
+__global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
+{
+    __shared__ int s_cnt[kTilePixels];
+    __shared__ int s_wave[4];
+    const int bin = blockIdx.x;
+    int layer, tx, ty;
+    tile_of_bin(p.geom, bin, layer, tx, ty);
+    const long long first = p.bin_start[bin];
+    long long last        = p.bin_start[bin + 1];
+    if (last > p.capacity) last = p.capacity;  // entries beyond the capacity were dropped by the scatter
+    const int n           = first < last ? (int)(last - first) : 0;
+    const uint4* entries  = p.bin_entries + first;
+    int32_t* counts       = p.counts + (size_t)bin * kTilePixels;
+
+    if (!SCATTER)
+    {
+        for (int i = threadIdx.x; i < kTilePixels; i += 256) s_cnt[i] = 0;
+        __syncthreads();
+        for (int i = threadIdx.x; i < n; i += 256)
+        {
+            const uint4 e = entries[i];
+            const int px = (int)(e.z & 0xffffu), py = (int)(e.z >> 16);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+            {
+                const int x = px + (c & 1), y = py + (c >> 1);
+                if ((x >> kTileShift) == tx && (y >> kTileShift) == ty)
+                    atomicAdd(&s_cnt[((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1))], 1);
+            }
+        }
+        __syncthreads();
+        int sum = 0;
+        for (int i = threadIdx.x; i < kTilePixels; i += 256)
+        {
+            const int c = s_cnt[i];
+            counts[i]   = c;
+            sum += c;
+        }
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+        if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = sum;
+        __syncthreads();
+        if (threadIdx.x == 0) p.bin_total[bin] = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+        return;
+    }
+
+    // exclusive scan of the tile's 1024 lengths: 4 consecutive pixels per thread
+    const int base4 = threadIdx.x * 4;
+    int v[4], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        v[i] = counts[base4 + i];
         sum += v[i];
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -254,43 +386,37 @@ __global__ __launch_bounds__(256) void scan_apply_kernel(const int32_t* __restri
     }
     if (lane == 63) s_wave[wave] = inc;
     __syncthreads();
-    int prefix = block_sums[blockIdx.x] + inc - sum;
+    int prefix = inc - sum;
     for (int w = 0; w < wave; ++w) prefix += s_wave[w];
+    const int key_start = p.bin_key_start[bin];
+    int32_t* cursor     = p.cursor + (size_t)bin * kTilePixels;
 #pragma unroll
-    for (int i = 0; i < PER; ++i)
+    for (int i = 0; i < 4; ++i)
     {
-        int idx = base + i;
-        if (idx < n) cursor[idx] = prefix;
+        s_cnt[base4 + i]  = key_start + prefix;  // running slot of the pixel
+        cursor[base4 + i] = key_start + prefix;
         prefix += v[i];
     }
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// 64-bit keys (depth bits << 32 | point id) into the pixel lists. Thread = (point, corner).
-__global__ __launch_bounds__(256) void scatter_keys_kernel(const ForwardParams p)
-{
-    const long long tid = (long long)blockIdx.x * 256 + threadIdx.x;
-    const int pid       = int(tid >> 2);
-    const int sub       = int(tid & 3);
-    if (pid >= p.num_points) return;
-    const float4 k = p.ptk[pid];
-    const float z  = k.z;
-    if (!(z > 0.f)) return;
-    const int max_layer = __float_as_int(k.w);
-    const u64 key       = ((u64)__float_as_uint(z) << 32) | (u64)(unsigned)pid;
-    float lx = k.x, ly = k.y;
+    __syncthreads();
     unsigned dropped = 0;
-    for (int layer = 0; layer < max_layer; ++layer)
+    for (int i = threadIdx.x; i < n; i += 256)
     {
-        const int px = (int)floorf(lx) + (sub & 1), py = (int)floorf(ly) + (sub >> 1);
-        const int pix  = p.geom.off[layer] + py * p.geom.w[layer] + px;
-        const int slot = atomicAdd(p.cursor + pix, 1);
-        if ((long long)slot < p.capacity)
-            p.keys[slot] = key;
-        else
-            dropped += 1;
-        lx *= 0.5f;
-        ly *= 0.5f;
+        const uint4 e = entries[i];
+        const int px = (int)(e.z & 0xffffu), py = (int)(e.z >> 16);
+        const u64 key = ((u64)e.x << 32) | (u64)e.y;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+        {
+            const int x = px + (c & 1), y = py + (c >> 1);
+            if ((x >> kTileShift) == tx && (y >> kTileShift) == ty)
+            {
+                const int slot = atomicAdd(&s_cnt[((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1))], 1);
+                if ((long long)slot < p.capacity)
+                    p.keys[slot] = key;
+                else
+                    dropped += 1;
+            }
+        }
     }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
 }
@@ -355,20 +481,22 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     const int lane     = threadIdx.x & 63;
     const int sub      = lane & 15;
     const int grp      = lane >> 4;
-    const int P        = p.geom.off[p.num_layers];
+    const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
     const long long wave_global = ((long long)blockIdx.x * 256 + threadIdx.x) >> 6;
     const long long pix_ll      = wave_global * 4 + grp;
-    const bool live             = pix_ll < P;
-    const int pix               = live ? (int)pix_ll : 0;
+    const bool in_range         = pix_ll < P;
+    const int pix               = in_range ? (int)pix_ll : 0;
+    int layer, gx, gy;
+    const bool live = pix_decode(p.geom, pix, layer, gx, gy) && in_range;  // false for the padding of partial tiles
 
-    int len = 0, end = 0;
+    int len = 0;
+    long long start = 0;
     if (live)
     {
-        len = p.counts[pix];
-        end = p.cursor[pix];
+        len   = p.counts[pix];
+        start = p.cursor[pix];
     }
-    const long long start = (long long)end - len;
     // entries beyond the capacity were never written
     int readable = len;
     if (start + len > p.capacity) readable = (int)max(0ll, p.capacity - start);
@@ -403,11 +531,7 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     }
 
     // ---- blend (RenderForward.cu:820-1048) ----
-    int layer = 0;
-    while (layer + 1 < p.num_layers && pix >= p.geom.off[layer + 1]) ++layer;
-    const int local = pix - p.geom.off[layer];
     const int lw = p.geom.w[layer], lh = p.geom.h[layer];
-    const int gx = local % lw, gy = local / lw;
 
     const int n    = min(min(len, readable), K);
     const bool has = live && sub < n;
@@ -488,13 +612,17 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
 #pragma unroll
             for (int c = 0; c < C; ++c) o[c] = col[c];
         }
-        if (TRAIN)
-        {
-            p.retained[pix] = ret;
-            p.lengths[pix]  = len;
-        }
     }
-    if (TRAIN && live && sub < K) p.lists[(size_t)pix * K + sub] = has ? pid : -1;
+    // saved state, also for padding pixels (empty) so that every row of the tables is defined
+    if (TRAIN && in_range)
+    {
+        if (sub == 0)
+        {
+            p.retained[pix] = live ? ret : 0;
+            p.lengths[pix]  = live ? len : 0;
+        }
+        if (sub < K) p.lists[(size_t)pix * K + sub] = has ? pid : -1;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -513,42 +641,46 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
 hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train, bool first_view, hipStream_t stream,
                                Profiler* prof)
 {
-    const int P  = p.geom.off[p.num_layers];
-    const int N  = p.num_points;
-    const int nb = (P + kScanTile - 1) / kScanTile;
+    const int NB = p.geom.bin_off[p.num_layers];
+    const int P  = NB * kTilePixels;
 
     if (first_view) hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.status);
     hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header);
+    const int G          = p.bin_groups;
+    const size_t lds_hist = (size_t)NB * sizeof(int);
     {
-        ProfScope ps(prof, "fill_counts", stream);
-        int blocks = (int)min((long long)(P + 255) / 256, 4096ll);
-        hipLaunchKernelGGL(fill_i32_kernel, dim3(max(blocks, 1)), dim3(256), 0, stream, p.counts, 0, (long long)P);
-    }
-    if (N > 0)
-    {
-        ProfScope ps(prof, "project_count", stream);
-        int blocks = min((N + 255) / 256, 2048);
+        ProfScope ps(prof, "project_bin", stream);
         if (train)
         {
-            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((project_count_kernel<CC, true>), dim3(blocks), dim3(256), 0, stream, p));
+            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((project_bin_kernel<CC, true>), dim3(G), dim3(kBinThreads), lds_hist, stream, p));
         }
         else
         {
-            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((project_count_kernel<CC, false>), dim3(blocks), dim3(256), 0, stream, p));
+            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((project_bin_kernel<CC, false>), dim3(G), dim3(kBinThreads), lds_hist, stream, p));
         }
     }
     {
-        ProfScope ps(prof, "scan", stream);
-        hipLaunchKernelGGL(scan_reduce_kernel, dim3(nb), dim3(256), 0, stream, p.counts, p.block_sums, P);
-        hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(1024), 0, stream, p.block_sums, nb, p.header);
-        hipLaunchKernelGGL(scan_apply_kernel, dim3(nb), dim3(256), 0, stream, p.counts, p.block_sums, p.cursor, P);
+        ProfScope ps(prof, "bin_scan", stream);
+        hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + 255) / 256), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
+        hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_count, p.bin_start,
+                           (int32_t*)nullptr, NB, (unsigned long long*)nullptr);
     }
-    if (N > 0)
     {
-        ProfScope ps(prof, "scatter_keys", stream);
-        long long threads = 4ll * N;
-        int blocks        = (int)((threads + 255) / 256);
-        hipLaunchKernelGGL(scatter_keys_kernel, dim3(blocks), dim3(256), 0, stream, p);
+        ProfScope ps(prof, "bin_scatter", stream);
+        hipLaunchKernelGGL(bin_scatter_kernel, dim3(G), dim3(kBinThreads), lds_hist, stream, p);
+    }
+    {
+        ProfScope ps(prof, "tile_count", stream);
+        hipLaunchKernelGGL((tile_lists_kernel<false>), dim3(NB), dim3(256), 0, stream, p);
+    }
+    {
+        ProfScope ps(prof, "tile_scan", stream);
+        hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_total, p.bin_key_start,
+                           (int32_t*)nullptr, NB, &p.header->n_entries);
+    }
+    {
+        ProfScope ps(prof, "tile_scatter", stream);
+        hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB), dim3(256), 0, stream, p);
     }
     {
         ProfScope ps(prof, "sort_blend", stream);

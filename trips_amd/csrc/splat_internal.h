@@ -83,13 +83,46 @@ __host__ __device__ inline int record_floats(int channels, bool train)
     return 4 + cpad + (train ? 8 : 0);
 }
 
+// Pixels are binned into 32 x 32 tiles per layer. Internally a pixel is numbered tile-major:
+// (bin << 10) | (y & 31) << 5 | (x & 31), bin = bin_off[layer] + tile_y * tiles_x[layer] + tile_x, so that a
+// tile's 1024 counters, list offsets and saved lists are contiguous (partial tiles are padded with empty pixels).
+// The exports of the C ABI translate back to the row-major numbering (off[]).
+constexpr int kTileShift  = 5;
+constexpr int kTile       = 1 << kTileShift;
+constexpr int kTilePixels = kTile * kTile;
+constexpr int kBinThreads = 512;    // workgroup size of the two binning kernels
+constexpr int kBinGroups  = 512;    // workgroups (= contiguous chunks of points) of the two binning kernels
+constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
+
 struct PyramidGeom
 {
     int32_t num_layers;
     int32_t w[TRIPS_MAX_LAYERS];
     int32_t h[TRIPS_MAX_LAYERS];
-    int32_t off[TRIPS_MAX_LAYERS + 1];  // first pixel number of each layer; off[L] = P
+    int32_t off[TRIPS_MAX_LAYERS + 1];  // row-major numbering: first pixel of each layer; off[L] = P
+    int32_t tiles_x[TRIPS_MAX_LAYERS];
+    int32_t tiles_y[TRIPS_MAX_LAYERS];
+    int32_t bin_off[TRIPS_MAX_LAYERS + 1];  // first bin of each layer; bin_off[L] = number of bins
 };
+
+__host__ __device__ inline int pix_index(const PyramidGeom& g, int layer, int x, int y)
+{
+    const int bin = g.bin_off[layer] + (y >> kTileShift) * g.tiles_x[layer] + (x >> kTileShift);
+    return (bin << (2 * kTileShift)) | ((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1));
+}
+
+// internal pixel number -> (layer, x, y); false for the padding of partial tiles
+__host__ __device__ inline bool pix_decode(const PyramidGeom& g, int ipix, int& layer, int& x, int& y)
+{
+    const int bin = ipix >> (2 * kTileShift), loc = ipix & (kTilePixels - 1);
+    layer         = 0;
+    while (layer + 1 < g.num_layers && bin >= g.bin_off[layer + 1]) ++layer;
+    const int t  = bin - g.bin_off[layer];
+    const int ty = t / g.tiles_x[layer], tx = t - ty * g.tiles_x[layer];
+    x            = (tx << kTileShift) + (loc & (kTile - 1));
+    y            = (ty << kTileShift) + (loc >> kTileShift);
+    return x < g.w[layer] && y < g.h[layer];
+}
 
 // Header at the start of each view's saved state (and of the workspace status block).
 struct ViewHeader
@@ -105,9 +138,9 @@ struct SavedLayout
 {
     size_t header;    // ViewHeader
     size_t rec;       // float [N * record_floats]
-    size_t lists;     // int32 [P, K]
-    size_t retained;  // int32 [P]
-    size_t lengths;   // int32 [P]
+    size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded)
+    size_t retained;  // int32 [Pi]
+    size_t lengths;   // int32 [Pi]
     size_t bytes_per_view;
 };
 
@@ -120,16 +153,19 @@ struct BackwardWorkspaceLayout
 
 struct WorkspaceLayout
 {
-    size_t ptk;         // float4 [N]   {ip.x, ip.y, depth (-1 culled), max_layer bits}
-    size_t counts;      // int32 [P]
-    size_t cursor;      // int32 [P]
-    size_t block_sums;  // int32 [scan blocks + 1]
-    size_t keys;        // uint64 [capacity]
-    size_t capacity;    // entries
+    size_t ptk;          // float4 [N]   {ip.x, ip.y, depth (-1 culled), max_layer bits}
+    size_t counts;       // int32 [Pi]   list length per pixel
+    size_t cursor;       // int32 [Pi]   first key of each pixel's list
+    size_t bin_count;    // int32 [NB]   bin entries per tile
+    size_t bin_start;    // int32 [NB+1] exclusive scan of bin_count
+    size_t bin_hist;     // int32 [G, NB] bin entries per (workgroup, tile), then its column-wise exclusive prefix
+    size_t bin_total;    // int32 [NB]   list entries per tile
+    size_t bin_key_start;  // int32 [NB+1] exclusive scan of bin_total
+    size_t bin_entries;  // uint4 [capacity] {depth bits, point id, px | py << 16, -}
+    size_t keys;         // uint64 [capacity]
+    size_t capacity;     // entries
     size_t bytes;
 };
-
-constexpr int kScanTile = 4096;  // elements per scan block (256 threads x 16)
 
 inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
@@ -157,7 +193,13 @@ struct ForwardParams
     float4* ptk;
     int32_t* counts;
     int32_t* cursor;
-    int32_t* block_sums;
+    int32_t* bin_count;
+    int32_t* bin_start;
+    int32_t* bin_hist;
+    int32_t bin_groups, points_per_block;
+    int32_t* bin_total;
+    int32_t* bin_key_start;
+    uint4* bin_entries;
     unsigned long long* keys;
     long long capacity;
     float* rec;

@@ -20,6 +20,9 @@ hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream
 hipError_t launch_export_points(const float* rec, int rec_floats, int n, float* ip, float* depth, float* size_px,
                                 int32_t* max_layer, hipStream_t stream);
 hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream);
+hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
+                               const int32_t* lengths, int32_t* out_lists, int32_t* out_retained, int32_t* out_lengths,
+                               hipStream_t stream);
 }  // namespace trips
 
 using namespace trips;
@@ -87,6 +90,27 @@ int check_desc(const TripsSplatDesc* d)
     if (4ll * d->num_points * d->num_layers > 0x7fffffffll && d->max_list_entries == 0)
         return fail(TRIPS_ERR_UNSUPPORTED, "4*N*L exceeds 2^31-1; set max_list_entries");
     if (d->max_list_entries > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "max_list_entries exceeds 2^31-1");
+    {
+        // one LDS counter per 32 x 32 tile of the pyramid in the binning kernels
+        long long bins = 0;
+        int cw = w, ch = h;
+        for (int l = 0; l < d->num_layers; ++l)
+        {
+            bins += (long long)((cw + kTile - 1) / kTile) * ((ch + kTile - 1) / kTile);
+            if (!d->floor_layer_sizes)
+            {
+                ch = (int)std::ceil(float(ch) / 2.f);
+                cw = (int)std::ceil(float(cw) / 2.f);
+            }
+            else
+            {
+                ch = ch / 2;
+                cw = cw / 2;
+            }
+        }
+        if (bins > kMaxBins)
+            return fail(TRIPS_ERR_UNSUPPORTED, "%lld tiles of 32x32 pixels, at most %d (about 4096 x 2700 pixels)", bins, kMaxBins);
+    }
     return TRIPS_OK;
 }
 
@@ -95,13 +119,17 @@ void make_geom(const TripsSplatDesc& d, PyramidGeom& g)
     int cw = d.views[0].w, ch = d.views[0].h;
     g.num_layers = d.num_layers;
     g.off[0]     = 0;
+    g.bin_off[0] = 0;
     for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
     {
         if (l < d.num_layers)
         {
-            g.w[l]       = cw;
-            g.h[l]       = ch;
-            g.off[l + 1] = g.off[l] + cw * ch;
+            g.w[l]           = cw;
+            g.h[l]           = ch;
+            g.off[l + 1]     = g.off[l] + cw * ch;
+            g.tiles_x[l]     = (cw + kTile - 1) / kTile;
+            g.tiles_y[l]     = (ch + kTile - 1) / kTile;
+            g.bin_off[l + 1] = g.bin_off[l] + g.tiles_x[l] * g.tiles_y[l];
             if (!d.floor_layer_sizes)
             {
                 // PointRenderer.cu:385-389
@@ -116,20 +144,24 @@ void make_geom(const TripsSplatDesc& d, PyramidGeom& g)
         }
         else
         {
-            g.w[l]       = 0;
-            g.h[l]       = 0;
-            g.off[l + 1] = g.off[l];
+            g.w[l]           = 0;
+            g.h[l]           = 0;
+            g.off[l + 1]     = g.off[l];
+            g.tiles_x[l]     = 0;
+            g.tiles_y[l]     = 0;
+            g.bin_off[l + 1] = g.bin_off[l];
         }
     }
 }
 
+// number of internally numbered pixels (tiles padded to 32 x 32), as a 64-bit value for the range check
 long long pyramid_pixels_checked(const TripsSplatDesc& d)
 {
     long long P = 0;
     int cw = d.views[0].w, ch = d.views[0].h;
     for (int l = 0; l < d.num_layers; ++l)
     {
-        P += (long long)cw * ch;
+        P += (long long)((cw + kTile - 1) / kTile) * ((ch + kTile - 1) / kTile) * kTilePixels;
         if (!d.floor_layer_sizes)
         {
             ch = (int)std::ceil(float(ch) / 2.f);
@@ -147,7 +179,7 @@ long long pyramid_pixels_checked(const TripsSplatDesc& d)
 SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     SavedLayout s;
-    const size_t N = (size_t)d.num_points, P = (size_t)g.off[d.num_layers], K = (size_t)d.list_depth;
+    const size_t N = (size_t)d.num_points, P = (size_t)g.bin_off[d.num_layers] * kTilePixels, K = (size_t)d.list_depth;
     const size_t rf = (size_t)record_floats(d.num_channels, true);
     size_t o        = 0;
     s.header        = o;
@@ -167,10 +199,9 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     WorkspaceLayout w;
-    const size_t N = (size_t)d.num_points, P = (size_t)g.off[d.num_layers];
-    const size_t nb = (P + kScanTile - 1) / kScanTile;
-    w.capacity      = d.max_list_entries > 0 ? (size_t)d.max_list_entries : 4 * N * (size_t)d.num_layers;
-    size_t o        = 0;
+    const size_t N = (size_t)d.num_points, NB = (size_t)g.bin_off[d.num_layers], P = NB * kTilePixels;
+    w.capacity     = d.max_list_entries > 0 ? (size_t)d.max_list_entries : 4 * N * (size_t)d.num_layers;
+    size_t o       = 0;
     // status header (overflow flag of the whole call), then for eval mode, which has no saved state to live
     // in, the per-view counters and the per-point records
     o += align256(sizeof(ViewHeader));
@@ -182,17 +213,31 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(P * sizeof(int32_t));
     w.cursor = o;
     o += align256(P * sizeof(int32_t));
-    w.block_sums = o;
-    o += align256((nb + 1) * sizeof(int32_t));
+    w.bin_count = o;
+    o += align256(NB * sizeof(int32_t));
+    w.bin_start = o;
+    o += align256((NB + 1) * sizeof(int32_t));
+    w.bin_hist = o;
+    o += align256((size_t)kBinGroups * NB * sizeof(int32_t));
+    w.bin_total = o;
+    o += align256(NB * sizeof(int32_t));
+    w.bin_key_start = o;
+    o += align256((NB + 1) * sizeof(int32_t));
+    w.bin_entries = o;
+    o += align256(w.capacity * sizeof(uint4));
     w.keys = o;
     o += align256(w.capacity * sizeof(unsigned long long));
     w.bytes = o;
     return w;
 }
+}  // namespace
+
+namespace
+{
 BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     BackwardWorkspaceLayout w;
-    const size_t N = (size_t)d.num_points, P = (size_t)g.off[d.num_layers], K = (size_t)d.list_depth;
+    const size_t N = (size_t)d.num_points, P = (size_t)g.bin_off[d.num_layers] * kTilePixels, K = (size_t)d.list_depth;
     size_t o       = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
     w.entry_grad   = o;
     o += align256(P * K * (size_t)((1 + d.num_channels + 3) & ~3) * sizeof(float));
@@ -326,7 +371,14 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
         p.ptk        = reinterpret_cast<float4*>(ws + wl.ptk);
         p.counts     = reinterpret_cast<int32_t*>(ws + wl.counts);
         p.cursor     = reinterpret_cast<int32_t*>(ws + wl.cursor);
-        p.block_sums = reinterpret_cast<int32_t*>(ws + wl.block_sums);
+        p.bin_count  = reinterpret_cast<int32_t*>(ws + wl.bin_count);
+        p.bin_start  = reinterpret_cast<int32_t*>(ws + wl.bin_start);
+        p.bin_hist   = reinterpret_cast<int32_t*>(ws + wl.bin_hist);
+        p.bin_groups = kBinGroups;
+        p.points_per_block = (d.num_points + kBinGroups - 1) / kBinGroups;
+        p.bin_total  = reinterpret_cast<int32_t*>(ws + wl.bin_total);
+        p.bin_key_start = reinterpret_cast<int32_t*>(ws + wl.bin_key_start);
+        p.bin_entries   = reinterpret_cast<uint4*>(ws + wl.bin_entries);
         p.keys       = reinterpret_cast<unsigned long long*>(ws + wl.keys);
         p.capacity   = (long long)wl.capacity;
         if (train)
@@ -448,7 +500,8 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
     char* sv             = const_cast<char*>(reinterpret_cast<const char*>(saved)) + sl.bytes_per_view * (size_t)view;
     ViewHeader* hd       = reinterpret_cast<ViewHeader*>(sv + sl.header);
     const long long P    = g.off[desc->num_layers];
-    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), P, &hd->reserved[0], stream);
+    const long long Pi   = (long long)g.bin_off[desc->num_layers] * kTilePixels;  // padding rows hold 0
+    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, &hd->reserved[0], stream);
     if (e != hipSuccess) return hip_fail(e, "retained sum");
     ViewHeader h;
     e = hipMemcpyAsync(&h, hd, sizeof(h), hipMemcpyDeviceToHost, stream);
@@ -474,14 +527,10 @@ int trips_splat_export_lists(TripsCtx* ctx, const TripsSplatDesc* desc, const vo
     const SavedLayout sl = saved_layout(*desc, g);
     hipStream_t stream   = reinterpret_cast<hipStream_t>(stream_);
     const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
-    const size_t P = (size_t)g.off[desc->num_layers], K = (size_t)desc->list_depth;
-    hipError_t e = hipSuccess;
-    if (device_lists && P)
-        e = hipMemcpyAsync(device_lists, sv + sl.lists, P * K * sizeof(int32_t), hipMemcpyDeviceToDevice, stream);
-    if (e == hipSuccess && device_retained && P)
-        e = hipMemcpyAsync(device_retained, sv + sl.retained, P * sizeof(int32_t), hipMemcpyDeviceToDevice, stream);
-    if (e == hipSuccess && device_lengths && P)
-        e = hipMemcpyAsync(device_lengths, sv + sl.lengths, P * sizeof(int32_t), hipMemcpyDeviceToDevice, stream);
+    hipError_t e = launch_export_lists(g, desc->list_depth, reinterpret_cast<const int32_t*>(sv + sl.lists),
+                                       reinterpret_cast<const int32_t*>(sv + sl.retained),
+                                       reinterpret_cast<const int32_t*>(sv + sl.lengths), device_lists, device_retained,
+                                       device_lengths, stream);
     if (e != hipSuccess) return hip_fail(e, "export copy");
     return TRIPS_OK;
 }
