@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void export_points_kernel(const float* __restr
         ip[2 * (size_t)pid + 1] = ok ? r[1] : 0.f;
     }
     if (depth) depth[pid] = tl.y;
-    if (size_px) size_px[pid] = ok ? r[2] : 0.f;
+    if (size_px) size_px[pid] = ok ? tl.w : 0.f;
     if (max_layer) max_layer[pid] = ok ? __float_as_int(tl.z) : 0;
 }
 

@@ -18,6 +18,7 @@
 //      loop before one block-level reduction and one atomic per value and block (the reference keeps them in
 //      shared double arrays, :160-187,546-617).
 // Gradients are therefore summed in a fixed order and are bit-reproducible from run to run.
+#include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"
 
@@ -75,12 +76,16 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
 #pragma unroll
     for (int i = 0; i < C; ++i) acc_bg[i] = 0.0;
 
+    // a workgroup walks whole tiles (256 pixel quads each), 4 workgroups per tile, all on one XCD
+    constexpr int kPerTile      = 4;
     const long long total_waves = ((long long)P + 3) / 4;
-    const long long wave0       = ((long long)blockIdx.x * 256 + threadIdx.x) >> 6;
-    const long long wave_stride = (long long)gridDim.x * 4;
+    const long long num_tiles   = p.geom.bin_off[p.num_layers];
+    const long long tile_stride = (long long)(gridDim.x / (kPerTile * kNumXcd)) * kNumXcd;
 
-    for (long long wv = wave0; wv < total_waves; wv += wave_stride)
+    for (long long lb = xcd_tile_block(blockIdx.x, kPerTile); lb < num_tiles * kPerTile; lb += tile_stride * kPerTile)
+    for (long long wv = lb * (kTilePixels / 4 / kPerTile) + (threadIdx.x >> 6); wv < (lb + 1) * (kTilePixels / 4 / kPerTile); wv += 4)
     {
+        if (wv >= total_waves) break;
         const long long pix_ll = wv * 4 + grp;
         const int pix          = pix_ll < P ? (int)pix_ll : 0;
         int layer, gx, gy;
@@ -133,20 +138,18 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
             float w = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
             if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
             a = w * r0.w;
-            a *= layer_factor(r0.z, layer, p.num_layers, nullptr);
+            a *= layer_factor_encoded(r0.z, layer, p.num_layers);
             // which of the point's four footprint pixels this one is
             const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
             slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
         }
 
         // exclusive transmittance, same chain as the forward
-        float pre = 1.f, T = 1.f;
-#pragma unroll
-        for (int s = 1; s < 16; ++s)
-        {
-            pre = __shfl_up(pre * (1.f - a), 1, 16);
-            if (sub == s) T = pre;
-        }
+        int mmax = m;
+        mmax     = max(mmax, __shfl_xor(mmax, 16));
+        mmax     = max(mmax, __shfl_xor(mmax, 32));
+        mmax     = __builtin_amdgcn_readfirstlane(mmax);
+        const float T = row_exclusive_product(1.f - a, mmax);
         // transmittance after the m retained entries decides whether the background is reached
         // (RenderBackward.cu:205-210,302-308)
         float T_after = T * (1.f - a);
@@ -163,14 +166,7 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
         }
         const float ta = T * a;
         const float q  = has ? ta * s : 0.f;
-        float later    = __shfl_down(q, 1, 16);  // entries i > j
-        if (sub == 15) later = 0.f;
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1)
-        {
-            float t = __shfl_down(later, o, 16);
-            if (sub + o < 16) later += t;
-        }
+        float later    = row_exclusive_suffix_sum(q);  // entries i > j
         if (bg_reached) later += T_after * sbg;
         const float dem        = 1.f / (1.f - a + 1e-9f);
         const float grad_alpha = T * s - later * dem;
@@ -264,7 +260,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             const int px = (int)fx, py = (int)fy;
             const float sx = ux - fx, sy = uy - fy;
             float lfac = 1.f, J_lf = 0.f;
-            if (want_size) lfac = layer_factor(r0.z, layer, p.num_layers, &J_lf);
+            if (want_size) lfac = layer_factor_encoded_grad(r0.z, tail.w, layer, p.num_layers, &J_lf);
             const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
 #pragma unroll
             for (int corner = 0; corner < 4; ++corner)
@@ -424,7 +420,8 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
         ProfScope ps(prof, "backward_pixels", stream);
         const long long waves = ((long long)P + 3) / 4;
         long long blocks_ll   = (waves + 3) / 4;
-        const int blocks      = (int)(blocks_ll < 4096 ? (blocks_ll < 1 ? 1 : blocks_ll) : 4096);
+        int blocks            = (int)(blocks_ll < 8192 ? (blocks_ll < 1 ? 1 : blocks_ll) : 8192);
+        blocks                = ((blocks + 4 * kNumXcd - 1) / (4 * kNumXcd)) * (4 * kNumXcd);  // whole groups of 8 tiles x 4
         TRIPS_BW_DISPATCH(backward_pixels_kernel, blocks);
     }
     if (N > 0)

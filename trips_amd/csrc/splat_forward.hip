@@ -15,6 +15,7 @@
 // atomics. A wavefront of the sort holds four pixel lists of 16 lanes (one DPP row each) instead of two per
 // 32-lane warp; the per-point record gathered by the blend carries position, size, confidence and descriptor
 // together; what is kept for the backward is the sorted id list per pixel (64 B) instead of 16 x 7 floats.
+#include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"
 
@@ -22,7 +23,6 @@
 
 namespace trips
 {
-using u64 = unsigned long long;
 
 __device__ __forceinline__ Camera load_camera(const double* pose, const float* intr, const TripsView& v,
                                               float dist_cutoff)
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
 
                 // record for blend (+ backward)
                 float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)pid * p.rec_floats);
-                rec[0]      = make_float4(ipx, ipy, size_px, p.confidence[tex]);
+                rec[0]      = make_float4(ipx, ipy, encode_size_field(size_px, L), p.confidence[tex]);
                 float d[CPAD];
 #pragma unroll
                 for (int c = 0; c < CPAD; ++c) d[c] = c < C ? p.texture[(size_t)c * p.num_texels + tex] : 0.f;
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 if (TRAIN)
                 {
                     rec[1 + CPAD / 4] = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
-                    rec[2 + CPAD / 4] = make_float4(__int_as_float(tex), z, __int_as_float(layer), 0.f);
+                    rec[2 + CPAD / 4] = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
                 }
             }
         }
@@ -398,7 +398,12 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
         prefix += v[i];
     }
     __syncthreads();
-    unsigned dropped = 0;
+    // Keys of a tile whose lists fit into LDS are staged there and copied out with full-line stores; the keys of
+    // bigger tiles go to their lists directly (8-byte stores scattered over the tile's region).
+    extern __shared__ u64 s_keys[];
+    const int tile_total = p.bin_key_start[bin + 1] - key_start;
+    const bool staged    = tile_total <= kStageKeys && (long long)key_start + tile_total <= p.capacity;
+    unsigned dropped     = 0;
     for (int i = threadIdx.x; i < n; i += 256)
     {
         const uint4 e = entries[i];
@@ -411,66 +416,31 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
             if ((x >> kTileShift) == tx && (y >> kTileShift) == ty)
             {
                 const int slot = atomicAdd(&s_cnt[((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1))], 1);
-                if ((long long)slot < p.capacity)
+                if (staged)
+                    s_keys[slot - key_start] = key;
+                else if ((long long)slot < p.capacity)
                     p.keys[slot] = key;
                 else
                     dropped += 1;
             }
         }
     }
+    if (staged)
+    {
+        __syncthreads();
+        u64* dst = p.keys + key_start;
+        for (int i = threadIdx.x; i < tile_total; i += 256) dst[i] = s_keys[i];
+    }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// 16-lane (one DPP row) primitives. Every group of 16 lanes is either fully active or fully inactive
-// wherever these are called.
-__device__ __forceinline__ u64 shfl_xor16(u64 v, int m)
-{
-    unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
-    lo = __shfl_xor(lo, m, 16);
-    hi = __shfl_xor(hi, m, 16);
-    return ((u64)hi << 32) | lo;
-}
-
 __device__ __forceinline__ u64 shfl16(u64 v, int src)
 {
     unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
     lo = __shfl(lo, src, 16);
     hi = __shfl(hi, src, 16);
     return ((u64)hi << 32) | lo;
-}
-
-// ascending bitonic sort of 16 keys, one per lane of the row
-__device__ __forceinline__ u64 sort16(u64 v, int sub)
-{
-#pragma unroll
-    for (int k = 2; k <= 16; k <<= 1)
-    {
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1)
-        {
-            const u64 o      = shfl_xor16(v, j);
-            const bool up    = (sub & k) == 0 || k == 16;
-            const bool lower = (sub & j) == 0;
-            const u64 mn = v < o ? v : o, mx = v < o ? o : v;
-            v = (lower == up) ? mn : mx;
-        }
-    }
-    return v;
-}
-
-// v is bitonic over the row: ascending merge
-__device__ __forceinline__ u64 merge16(u64 v, int sub)
-{
-#pragma unroll
-    for (int j = 8; j > 0; j >>= 1)
-    {
-        const u64 o      = shfl_xor16(v, j);
-        const bool lower = (sub & j) == 0;
-        const u64 mn = v < o ? v : o, mx = v < o ? o : v;
-        v = lower ? mn : mx;
-    }
-    return v;
 }
 
 // Top-16 of each pixel list by key, then the alpha blend. One wavefront = four pixels, 16 lanes each.
@@ -483,9 +453,11 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     const int grp      = lane >> 4;
     const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
-    const long long wave_global = ((long long)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const long long nblocks     = ((long long)P + 15) / 16;  // 16 pixels per workgroup, 64 workgroups per tile
+    const long long lblock      = xcd_tile_block(blockIdx.x, kTilePixels / 16);
+    const long long wave_global = lblock * 4 + (threadIdx.x >> 6);
     const long long pix_ll      = wave_global * 4 + grp;
-    const bool in_range         = pix_ll < P;
+    const bool in_range         = pix_ll < P && lblock < nblocks;
     const int pix               = in_range ? (int)pix_ll : 0;
     int layer, gx, gy;
     const bool live = pix_decode(p.geom, pix, layer, gx, gy) && in_range;  // false for the padding of partial tiles
@@ -514,7 +486,7 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
         if (base + sub < readable) k = p.keys[start + base + sub];
         if (base == 0)
         {
-            best = sort16(k, sub);
+            best = row_sort16(k);
         }
         else
         {
@@ -522,10 +494,10 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
             const bool need = k < worst;
             if (__ballot(need) & grp_mask)
             {
-                k           = sort16(k, sub);
-                const u64 r = shfl_xor16(k, 15);  // reversed: lane i sees the (15-i)-th smallest new key
+                k           = row_sort16(k);
+                const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
                 best        = best < r ? best : r;
-                best        = merge16(best, sub);
+                best        = row_merge16(best);
             }
         }
     }
@@ -559,17 +531,16 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
         float w        = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
         if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
         a = w * r0.w;
-        a *= layer_factor(r0.z, layer, p.num_layers, nullptr);
+        a *= layer_factor_encoded(r0.z, layer, p.num_layers);
     }
 
     // exclusive transmittance: lane j latches prod_{k<j} (1 - a_k), built left to right
-    float pre = 1.f, T = 1.f;
-#pragma unroll
-    for (int s = 1; s < 16; ++s)
-    {
-        pre = __shfl_up(pre * (1.f - a), 1, 16);
-        if (sub == s) T = pre;
-    }
+    // only the first n positions of a row matter; n <= K
+    int nmax = n;
+    nmax     = max(nmax, __shfl_xor(nmax, 16));
+    nmax     = max(nmax, __shfl_xor(nmax, 32));
+    nmax     = __builtin_amdgcn_readfirstlane(nmax);
+    const float T     = row_exclusive_product(1.f - a, nmax);
     const float Tc    = (T >= kAlphaDestCutoff) ? T : 0.f;
     const bool kept   = has && Tc >= kAlphaDestCutoff;
     const unsigned kb = (unsigned)((__ballot(kept) >> (grp * 16)) & 0xFFFFull);
@@ -580,11 +551,7 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
 #pragma unroll
     for (int c = 0; c < C; ++c) col[c] = wgt * desc[c];
 #pragma unroll
-    for (int o = 1; o < 16; o <<= 1)
-    {
-#pragma unroll
-        for (int c = 0; c < C; ++c) col[c] = col[c] + __shfl_xor(col[c], o, 16);
-    }
+    for (int c = 0; c < C; ++c) col[c] = row_sum_to_lane0(col[c]);
 
     // background weight (RenderForward.cu:1002-1022); empty list -> 1
     float bgw_lane = (p.background_mode == TRIPS_BG_REFERENCE) ? Tc : T * (1.f - a);
@@ -642,7 +609,6 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
                                Profiler* prof)
 {
     const int NB = p.geom.bin_off[p.num_layers];
-    const int P  = NB * kTilePixels;
 
     if (first_view) hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.status);
     hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header);
@@ -680,12 +646,12 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     }
     {
         ProfScope ps(prof, "tile_scatter", stream);
-        hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB), dim3(256), kStageKeys * sizeof(u64), stream, p);
     }
     {
         ProfScope ps(prof, "sort_blend", stream);
-        long long waves = ((long long)P + 3) / 4;
-        int blocks      = (int)((waves + 3) / 4);
+        const long long tiles8 = (((long long)NB + kNumXcd - 1) / kNumXcd) * kNumXcd;  // tiles rounded up to 8
+        int blocks             = (int)(tiles8 * (kTilePixels / 16));
         if (train)
         {
             TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((sort_blend_kernel<CC, true>), dim3(blocks), dim3(256), 0, stream, p));

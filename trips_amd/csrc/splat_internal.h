@@ -73,10 +73,11 @@ struct ProfScope
 };
 
 // Per-point record written by the projection pass and gathered by blend / backward.
-// First 4 + Cpad floats: {ip.x, ip.y, size_px, confidence, descriptor[0..C)} -- everything the blend needs,
+// First 4 + Cpad floats: {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)} --
+// everything the blend needs,
 // one aligned gather instead of three scattered reads (reference: 5-float record + confidence + [C,N] texture,
 // src/lib/rendering/RenderForward.cu:875-899,952). In train mode 8 more floats follow for the backward:
-// {view.x, view.y, view.z, softplus'(raw size), texture index, depth (-1 = culled), layers written, -}.
+// {view.x, view.y, view.z, softplus'(raw size), texture index, depth (-1 = culled), layers written, size_px}.
 __host__ __device__ inline int record_floats(int channels, bool train)
 {
     int cpad = (channels + 3) & ~3;
@@ -93,6 +94,7 @@ constexpr int kTilePixels = kTile * kTile;
 constexpr int kBinThreads = 512;    // workgroup size of the two binning kernels
 constexpr int kBinGroups  = 512;    // workgroups (= contiguous chunks of points) of the two binning kernels
 constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
+constexpr int kStageKeys  = 7168;   // keys of one tile staged in LDS before they are written (56 KB)
 
 struct PyramidGeom
 {
@@ -104,6 +106,19 @@ struct PyramidGeom
     int32_t tiles_y[TRIPS_MAX_LAYERS];
     int32_t bin_off[TRIPS_MAX_LAYERS + 1];  // first bin of each layer; bin_off[L] = number of bins
 };
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Kernels that walk pixels remap their
+// workgroup number so that all workgroups of one 32 x 32 tile run on the same XCD (the records a tile's pixels
+// share are then fetched once per tile instead of once per workgroup), while consecutive tiles go to different
+// XCDs (layers differ a lot in list length, so a contiguous range per XCD would be unbalanced).
+// `per_tile` = workgroups per tile; the result may be >= the number of real workgroups (no work then).
+constexpr int kNumXcd = 8;
+__device__ inline long long xcd_tile_block(long long block, int per_tile)
+{
+    const long long xcd = block % kNumXcd, k = block / kNumXcd;
+    const long long tile = (k / per_tile) * kNumXcd + xcd;
+    return tile * per_tile + k % per_tile;
+}
 
 __host__ __device__ inline int pix_index(const PyramidGeom& g, int layer, int x, int y)
 {

@@ -98,6 +98,35 @@ __device__ __forceinline__ float layer_factor(float s, int layer, int max_layers
     return f;
 }
 
+// The "small point" branch of the layer factor (layer_higher == 0, i.e. size <= 1 pixel or a single layer) is the
+// only one that needs exp(), and it does not depend on the layer (such a point lands in layer 0 only). The
+// projection kernel evaluates it once per point and stores it NEGATED in the size slot of the per-point record;
+// the blend and the backward then read the factor instead of re-evaluating a double-precision exp per list entry.
+__device__ __forceinline__ float encode_size_field(float size_px, int max_layers)
+{
+    const bool small_branch = !(size_px > 1.f) || max_layers == 1;
+    return small_branch ? -(0.75f * exp_rn(size_px - 1.f) + 0.25f) : size_px;
+}
+
+// layer factor from the encoded size field; identical in value to layer_factor(size_px, ...)
+__device__ __forceinline__ float layer_factor_encoded(float field, int layer, int max_layers)
+{
+    if (field < 0.f) return -field;
+    return layer_factor(field, layer, max_layers, nullptr);
+}
+
+// same with the reference's gradient; true_size is the un-encoded projected size
+__device__ __forceinline__ float layer_factor_encoded_grad(float field, float true_size, int layer, int max_layers,
+                                                           float* grad)
+{
+    if (field < 0.f)
+    {
+        *grad = 0.27591f * true_size;
+        return -field;
+    }
+    return layer_factor(field, layer, max_layers, grad);
+}
+
 struct Pose
 {
     float qx, qy, qz, qw, tx, ty, tz;
