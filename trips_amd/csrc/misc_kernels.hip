@@ -225,14 +225,14 @@ hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream
 }
 
 // ---- exports from the saved state ----
-__global__ __launch_bounds__(256) void export_points_kernel(const float* __restrict__ rec, int rec_floats, int n,
-                                                            float* ip, float* depth, float* size_px,
-                                                            int32_t* max_layer)
+__global__ __launch_bounds__(256) void export_points_kernel(const float* __restrict__ rec, int rec_floats,
+                                                            const float* __restrict__ prec, int n, float* ip,
+                                                            float* depth, float* size_px, int32_t* max_layer)
 {
     const int pid = blockIdx.x * 256 + threadIdx.x;
     if (pid >= n) return;
     const float* r  = rec + (size_t)pid * rec_floats;
-    const float4 tl = *reinterpret_cast<const float4*>(r + rec_floats - 4);  // {tex, depth, max_layer, -}
+    const float4 tl = *reinterpret_cast<const float4*>(prec + (size_t)pid * kPointRecordFloats + 4);  // {tex, depth, max_layer, size_px}
     const bool ok   = tl.y > 0.f;
     if (ip)
     {
@@ -244,11 +244,11 @@ __global__ __launch_bounds__(256) void export_points_kernel(const float* __restr
     if (max_layer) max_layer[pid] = ok ? __float_as_int(tl.z) : 0;
 }
 
-hipError_t launch_export_points(const float* rec, int rec_floats, int n, float* ip, float* depth, float* size_px,
-                                int32_t* max_layer, hipStream_t stream)
+hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, int n, float* ip, float* depth,
+                                float* size_px, int32_t* max_layer, hipStream_t stream)
 {
     if (n <= 0) return hipSuccess;
-    hipLaunchKernelGGL(export_points_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, rec, rec_floats, n, ip,
+    hipLaunchKernelGGL(export_points_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, rec, rec_floats, prec, n, ip,
                        depth, size_px, max_layer);
     return hipGetLastError();
 }

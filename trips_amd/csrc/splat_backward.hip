@@ -94,6 +94,10 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
 
         const int m    = live ? p.retained[pix] : 0;
         const bool has = sub < m;
+        int mmax       = m;
+        mmax           = max(mmax, __shfl_xor(mmax, 16));
+        mmax           = max(mmax, __shfl_xor(mmax, 32));
+        mmax           = __builtin_amdgcn_readfirstlane(mmax);
 
         float g[C];
         {
@@ -145,10 +149,6 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
         }
 
         // exclusive transmittance, same chain as the forward
-        int mmax = m;
-        mmax     = max(mmax, __shfl_xor(mmax, 16));
-        mmax     = max(mmax, __shfl_xor(mmax, 32));
-        mmax     = __builtin_amdgcn_readfirstlane(mmax);
         const float T = row_exclusive_product(1.f - a, mmax);
         // transmittance after the m retained entries decides whether the background is reached
         // (RenderBackward.cu:205-210,302-308)
@@ -232,16 +232,15 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 
     for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
     {
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
-        const float4 tail = rec[2 + CPAD / 4];  // {texture index, depth, layers written, -}
+        const float4* prec = reinterpret_cast<const float4*>(p.prec + (size_t)pid * kPointRecordFloats);
+        const float4 tail  = prec[1];  // {texture index, depth, layers written, size_px}
         if (!(tail.y > 0.f)) continue;
         const int tex       = __float_as_int(tail.x);
         const int max_layer = __float_as_int(tail.z);
-        const float4 r0     = rec[0];          // ip.x ip.y size_px conf
-        const float4 rv     = rec[1 + CPAD / 4];  // view xyz, softplus'(raw size)
+        const float4 r0     = *reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);  // ip.x ip.y size field conf
+        const float4 rv     = prec[0];  // view xyz, softplus'(raw size)
         const uint4* rk     = reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 32);
         const uint4 rk0 = rk[0], rk1 = rk[1];
-        const unsigned words[8] = {rk0.x, rk0.y, rk0.z, rk0.w, rk1.x, rk1.y, rk1.z, rk1.w};
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;
         float tex_grad[C];
@@ -249,11 +248,13 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         for (int c = 0; c < C; ++c) tex_grad[c] = 0.f;
         const float conf = r0.w;
         bool any         = false;
+        const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
 
-        for (int layer = 0; layer < max_layer; ++layer)
+        // one layer: the four gathers are issued together, then consumed in corner order
+        auto do_layer = [&](const int layer, const unsigned word)
         {
-            const unsigned word = words[layer];
-            if (word == 0xFFFFFFFFu) continue;
+            if (layer >= max_layer || word == 0xFFFFFFFFu) return;
+            any              = true;
             const float mfac = 1.f / float(1 << layer);
             const float ux = r0.x * mfac, uy = r0.y * mfac;
             const float fx = floorf(ux), fy = floorf(uy);
@@ -261,31 +262,35 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             const float sx = ux - fx, sy = uy - fy;
             float lfac = 1.f, J_lf = 0.f;
             if (want_size) lfac = layer_factor_encoded_grad(r0.z, tail.w, layer, p.num_layers, &J_lf);
-            const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
+            float4 e[4][EF / 4];
+#pragma unroll
+            for (int corner = 0; corner < 4; ++corner)
+            {
+                const unsigned j = (word >> (8 * corner)) & 0xFFu;
+                const int gx = px + (corner & 1), gy = py + (corner >> 1);
+                const int pix = pix_index(p.geom, layer, gx, gy);
+                const float4* src = reinterpret_cast<const float4*>(p.entry_grad + ((size_t)pix * K + (j & 15u)) * EF);
+#pragma unroll
+                for (int q = 0; q < EF / 4; ++q) e[corner][q] = (j != 0xFFu) ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
 #pragma unroll
             for (int corner = 0; corner < 4; ++corner)
             {
                 const unsigned j = (word >> (8 * corner)) & 0xFFu;
                 if (j == 0xFFu) continue;
-                any          = true;
                 const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                const int pix = pix_index(p.geom, layer, gx, gy);
-                float e[EF];
+                float ev[EF];
+#pragma unroll
+                for (int q = 0; q < EF / 4; ++q)
                 {
-                    const float4* src = reinterpret_cast<const float4*>(p.entry_grad + ((size_t)pix * K + j) * EF);
-#pragma unroll
-                    for (int q = 0; q < EF / 4; ++q)
-                    {
-                        const float4 t = src[q];
-                        e[4 * q]       = t.x;
-                        e[4 * q + 1]   = t.y;
-                        e[4 * q + 2]   = t.z;
-                        e[4 * q + 3]   = t.w;
-                    }
+                    ev[4 * q]     = e[corner][q].x;
+                    ev[4 * q + 1] = e[corner][q].y;
+                    ev[4 * q + 2] = e[corner][q].z;
+                    ev[4 * q + 3] = e[corner][q].w;
                 }
-                const float grad_alpha = e[0];
+                const float grad_alpha = ev[0];
 #pragma unroll
-                for (int c = 0; c < C; ++c) tex_grad[c] += e[1 + c];
+                for (int c = 0; c < C; ++c) tex_grad[c] += ev[1 + c];
                 // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
                 const int x_i = float(gx) < ux ? 0 : 1;
                 const int y_i = float(gy) < uy ? 0 : 2;
@@ -309,7 +314,15 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
                     size_grad += blend * conf * grad_layer_ps;
                 }
             }
-        }
+        };
+        do_layer(0, rk0.x);
+        do_layer(1, rk0.y);
+        do_layer(2, rk0.z);
+        do_layer(3, rk0.w);
+        do_layer(4, rk1.x);
+        do_layer(5, rk1.y);
+        do_layer(6, rk1.z);
+        do_layer(7, rk1.w);
         if (!any) continue;
 
         float g_point[3], g_pose[6], g_k[5], g_dis[8];

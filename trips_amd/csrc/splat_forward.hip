@@ -158,16 +158,17 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 for (int q = 0; q < CPAD / 4; ++q) rec[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
                 if (TRAIN)
                 {
-                    rec[1 + CPAD / 4] = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
-                    rec[2 + CPAD / 4] = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
+                    float4* prec = reinterpret_cast<float4*>(p.prec + (size_t)pid * kPointRecordFloats);
+                    prec[0]      = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
+                    prec[1]      = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
                 }
             }
         }
         if (TRAIN && !(ptk.z > 0.f))
         {
             // culled: only the tail {texture index, depth = -1, layers = 0} is defined
-            float4* rec       = reinterpret_cast<float4*>(p.rec + (size_t)pid * p.rec_floats);
-            rec[2 + CPAD / 4] = make_float4(__int_as_float(tex), -1.f, __int_as_float(0), 0.f);
+            float4* prec = reinterpret_cast<float4*>(p.prec + (size_t)pid * kPointRecordFloats);
+            prec[1]      = make_float4(__int_as_float(tex), -1.f, __int_as_float(0), 0.f);
         }
         p.ptk[pid] = ptk;
     }

@@ -72,17 +72,16 @@ struct ProfScope
     }
 };
 
-// Per-point record written by the projection pass and gathered by blend / backward.
-// First 4 + Cpad floats: {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)} --
-// everything the blend needs,
-// one aligned gather instead of three scattered reads (reference: 5-float record + confidence + [C,N] texture,
-// src/lib/rendering/RenderForward.cu:875-899,952). In train mode 8 more floats follow for the backward:
-// {view.x, view.y, view.z, softplus'(raw size), texture index, depth (-1 = culled), layers written, size_px}.
-__host__ __device__ inline int record_floats(int channels, bool train)
-{
-    int cpad = (channels + 3) & ~3;
-    return 4 + cpad + (train ? 8 : 0);
-}
+// Per-point records written by the projection pass.
+//   rec[pid]   4 + Cpad floats {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)}:
+//              everything the blend and the pixel pass of the backward need in one aligned gather of 32 bytes at
+//              C = 4 (the reference reads a 5-float record, the confidence and C descriptor planes,
+//              src/lib/rendering/RenderForward.cu:875-899,952). Kept apart from the rest because a scattered gather
+//              costs the bytes of the whole aligned block it touches.
+//   prec[pid]  8 floats {view.x, view.y, view.z, softplus'(raw size), texture index, depth (-1 = culled), layers
+//              written, size_px}: read in point order by the point pass of the backward (training only).
+__host__ __device__ inline int record_floats(int channels) { return 4 + ((channels + 3) & ~3); }
+constexpr int kPointRecordFloats = 8;
 
 // Pixels are binned into 32 x 32 tiles per layer. Internally a pixel is numbered tile-major:
 // (bin << 10) | (y & 31) << 5 | (x & 31), bin = bin_off[layer] + tile_y * tiles_x[layer] + tile_x, so that a
@@ -153,6 +152,7 @@ struct SavedLayout
 {
     size_t header;    // ViewHeader
     size_t rec;       // float [N * record_floats]
+    size_t prec;      // float [N * kPointRecordFloats]
     size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded)
     size_t retained;  // int32 [Pi]
     size_t lengths;   // int32 [Pi]
@@ -218,6 +218,7 @@ struct ForwardParams
     unsigned long long* keys;
     long long capacity;
     float* rec;
+    float* prec;  // training only
     int32_t rec_floats;
     int32_t* lists;
     int32_t* retained;
@@ -239,6 +240,7 @@ struct BackwardParams
     int32_t view_index, num_views, layout;
     float dist_cutoff;
     const float* rec;
+    const float* prec;
     int32_t rec_floats;
     const int32_t* lists;
     const int32_t* retained;

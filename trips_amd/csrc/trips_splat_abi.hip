@@ -17,8 +17,8 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof);
 hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_t stream, Profiler* prof);
 hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t stream);
-hipError_t launch_export_points(const float* rec, int rec_floats, int n, float* ip, float* depth, float* size_px,
-                                int32_t* max_layer, hipStream_t stream);
+hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, int n, float* ip, float* depth,
+                                float* size_px, int32_t* max_layer, hipStream_t stream);
 hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream);
 hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
                                const int32_t* lengths, int32_t* out_lists, int32_t* out_retained, int32_t* out_lengths,
@@ -180,12 +180,14 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     SavedLayout s;
     const size_t N = (size_t)d.num_points, P = (size_t)g.bin_off[d.num_layers] * kTilePixels, K = (size_t)d.list_depth;
-    const size_t rf = (size_t)record_floats(d.num_channels, true);
+    const size_t rf = (size_t)record_floats(d.num_channels);
     size_t o        = 0;
     s.header        = o;
     o += align256(sizeof(ViewHeader));
     s.rec = o;
     o += align256(N * rf * sizeof(float));
+    s.prec = o;
+    o += align256(N * kPointRecordFloats * sizeof(float));
     s.lists = o;
     o += align256(P * K * sizeof(int32_t));
     s.retained = o;
@@ -206,7 +208,7 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     // in, the per-view counters and the per-point records
     o += align256(sizeof(ViewHeader));
     o += align256(sizeof(ViewHeader));
-    o += align256(N * (size_t)record_floats(d.num_channels, false) * sizeof(float));
+    o += align256(N * (size_t)record_floats(d.num_channels) * sizeof(float));
     w.ptk = o;
     o += align256(N * sizeof(float4));
     w.counts = o;
@@ -386,7 +388,8 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
             char* sv     = reinterpret_cast<char*>(out->saved) + sl.bytes_per_view * (size_t)b;
             p.header     = reinterpret_cast<ViewHeader*>(sv + sl.header);
             p.rec        = reinterpret_cast<float*>(sv + sl.rec);
-            p.rec_floats = record_floats(d.num_channels, true);
+            p.prec       = reinterpret_cast<float*>(sv + sl.prec);
+            p.rec_floats = record_floats(d.num_channels);
             p.lists      = reinterpret_cast<int32_t*>(sv + sl.lists);
             p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
             p.lengths    = reinterpret_cast<int32_t*>(sv + sl.lengths);
@@ -395,7 +398,7 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
         {
             p.header     = reinterpret_cast<ViewHeader*>(ws + align256(sizeof(ViewHeader)));
             p.rec        = reinterpret_cast<float*>(ws + 2 * align256(sizeof(ViewHeader)));
-            p.rec_floats = record_floats(d.num_channels, false);
+            p.rec_floats = record_floats(d.num_channels);
         }
         p.status = reinterpret_cast<ViewHeader*>(ws);
         for (int l = 0; l < d.num_layers; ++l) p.image[l] = out->image[l];
@@ -452,7 +455,8 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.layout       = d.layout;
         p.dist_cutoff  = d.dist_cutoff;
         p.rec          = reinterpret_cast<const float*>(sv + sl.rec);
-        p.rec_floats   = record_floats(d.num_channels, true);
+        p.prec         = reinterpret_cast<const float*>(sv + sl.prec);
+        p.rec_floats   = record_floats(d.num_channels);
         p.lists        = reinterpret_cast<const int32_t*>(sv + sl.lists);
         p.retained     = reinterpret_cast<const int32_t*>(sv + sl.retained);
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
@@ -546,7 +550,8 @@ int trips_splat_export_points(TripsCtx* ctx, const TripsSplatDesc* desc, const v
     make_geom(*desc, g);
     const SavedLayout sl = saved_layout(*desc, g);
     const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
-    hipError_t e = launch_export_points(reinterpret_cast<const float*>(sv + sl.rec), record_floats(desc->num_channels, true),
+    hipError_t e = launch_export_points(reinterpret_cast<const float*>(sv + sl.rec), record_floats(desc->num_channels),
+                                        reinterpret_cast<const float*>(sv + sl.prec),
                                         desc->num_points, device_ip, device_depth, device_size_px, device_max_layer,
                                         reinterpret_cast<hipStream_t>(stream_));
     if (e != hipSuccess) return hip_fail(e, "export points");
