@@ -20,6 +20,32 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+DEFAULT_POINTS = 6_000_000
+
+# HBM traffic per launch on the default workload, measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# (KiB per dispatch, one counter per run, same bench.py command with --steps 2 --warmup 1 --cpu-steps 0
+# --calibration-copy). A plain 256 MiB device copy reads FETCH_SIZE = 131084 and WRITE_SIZE = 262144 for
+# 262144 KiB each way, hence the scale factors. bench.py cannot run the profiler on itself; these are the figures
+# of the committed summary of those two runs and apply to the default --points only.
+PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
+PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
+    "project_bin": (131589, 407187),
+    "bin_scatter": (50029, 203344),
+    "tile_count": (51795, 11061),
+    "tile_scatter": (57559, 511718),
+    "sort_blend": (358645, 240802),
+    "fill_rank": (10, 187500),
+    "backward_pixels": (525044, 647669),
+    "backward_points": (1405460, 566754),
+    "adam_fused": (688600, 912211),
+}
+
+
+def measured_traffic_bytes(kernel):
+    if kernel not in PMC_KIB_DEFAULT_WORKLOAD:
+        return None
+    f, w = PMC_KIB_DEFAULT_WORKLOAD[kernel]
+    return int((f * PMC_FETCH_SCALE + w * PMC_WRITE_SCALE) * 1024)
 
 
 def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0):
@@ -41,7 +67,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--points", type=int, default=6_000_000)
+    ap.add_argument("--points", type=int, default=DEFAULT_POINTS)
     ap.add_argument("--cpu-steps", type=int, default=3, help="oracle steps for the cpu_baseline sample (0 = skip)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three plain 256 MiB device copies, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
@@ -169,7 +195,9 @@ def main():
         "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic_bytes(dom) if args.points == DEFAULT_POINTS else None,
+                     "algorithmic_bytes": int(alg[dom]), "avg_ms": kernels[dom]["avg_ms"]},
         "kernels": kernels,
         "cpu_baseline": cpu,
     }
