@@ -175,6 +175,67 @@ def test_config4_contention_reduced(oracle):
     _check_backward(oracle, sc, d, seed=4)
 
 
+def test_config3_forward_backward_full(oracle):
+    # the configuration the benchmark is quoted on: 6M points, 1920x1080, 8 layers, K = 16
+    sc = scenes.config3()
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert int(ref["counters"][0, 1]) > 20_000_000
+    _check_backward(oracle, sc, d, seed=3)
+
+
+def test_config4_contention_full(oracle):
+    # 4M points in 64 tight clusters, 4 views, 1245x825 (odd sizes: ceil halving), K = 16
+    sc = scenes.config4()
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert ref["lengths"].max() > 2000
+    _check_backward(oracle, sc, d, seed=5)
+
+
+def test_point_order_does_not_matter_at_full_size():
+    """Size-independent property at the benchmark's size: shuffling the point order permutes the per-point
+    gradients and leaves the images unchanged (depth ties aside, which break by point id)."""
+    import dataclasses
+    from tests.gpu_util import GpuRun
+    sc = scenes.config3()
+    rng = np.random.Generator(np.random.Philox(99))
+    perm = rng.permutation(sc.num_points)
+    sc2 = dataclasses.replace(sc, position=sc.position[perm], point_size=sc.point_size[perm],
+                              texture=np.ascontiguousarray(sc.texture[:, perm]), confidence=sc.confidence[perm])
+    d = abi.desc_for_scene(sc)
+    grad_rng = np.random.Generator(np.random.Philox(100))
+    sizes, _, _ = abi.pyramid_pixels(d)
+    gi = [grad_rng.normal(0, 1, (1, d.num_channels, h, w)).astype(np.float32) for (w, h) in sizes]
+    a = GpuRun(sc, d)
+    ia = a.forward()
+    ga = a.backward(gi)
+    ca = a.ctx.counters(d, a.saved, 0)
+    del a
+    b = GpuRun(sc2, d)
+    ib = b.forward()
+    gb = b.backward(gi)
+    cb = b.ctx.counters(d, b.saved, 0)
+    assert ca == cb
+    for x, y in zip(ia, ib):
+        # pixels whose two front-most entries tie in depth may order differently
+        assert (np.abs(x - y) > 1e-5 * (1 + np.abs(y))).mean() < 1e-4
+
+    def off(got, want):
+        # fraction of elements further apart than the gradient bar; a depth tie reorders two entries of a pixel
+        # and moves the gradients of those two points
+        got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+        return float((np.abs(got - want) > GRAD_RTOL * np.abs(want).max()).mean())
+
+    assert off(gb["d_position"], ga["d_position"][perm]) < 1e-4
+    assert off(gb["d_point_size"], ga["d_point_size"][perm]) < 1e-4
+    assert off(gb["d_confidence"], ga["d_confidence"][perm]) < 1e-4
+    assert off(gb["d_texture"], ga["d_texture"][:, perm]) < 1e-4
+    from tests.gpu_util import rel_err
+    assert rel_err(gb["d_pose"], ga["d_pose"]) < 1e-3
+    assert rel_err(gb["d_background"], ga["d_background"]) < 1e-3
+
+
 def test_list_overflow_is_reported(oracle):
     from tests.gpu_util import GpuRun
     from trips_amd._lib import TripsError
