@@ -69,6 +69,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--points", type=int, default=DEFAULT_POINTS)
     ap.add_argument("--cpu-steps", type=int, default=3, help="oracle steps for the cpu_baseline sample (0 = skip)")
+    ap.add_argument("--no-net", action="store_true", help="skip the reconstruction-net forward that is reported beside the splat")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three plain 256 MiB device copies, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -161,6 +162,33 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
 
+    # The reconstruction net that consumes the pyramid (next row after the splat): forward only, on the images
+    # the splat just rendered. 4 levels, filters 16/32/64/64, fp16 operands on the matrix cores.
+    unet = None
+    if not args.no_net:
+        from trips_amd.unet import MultiScaleUnet2dDecOnlySmallFixed, MultiScaleUnet2dParams
+        np_ = MultiScaleUnet2dParams(num_input_layers=desc.num_layers, num_layers=4, filters_network=[16, 32, 64, 64])
+        net = MultiScaleUnet2dDecOnlySmallFixed(np_).he_normal_(torch.Generator().manual_seed(5)).to(dev)
+        with torch.no_grad():
+            for _ in range(3):
+                rgb = net.forward(images)
+            torch.cuda.synchronize()
+            ctx.profile_enable(True)
+            ctx.profile_read()
+            for _ in range(args.steps):
+                rgb = net.forward(images)
+            torch.cuda.synchronize()
+            nprof = ctx.profile_read()
+            ctx.profile_enable(False)
+        net_ms = sum(ms for ms, _ in nprof.values()) / args.steps
+        flops = net.flops(images)
+        unet = {"workload": "MultiScaleUnet2dDecOnlySmallFixed forward, 4 levels 16/32/64/64, 1920x1080, fp16 operands / "
+                            "fp32 accumulate, He-normal weights, input = the splat's pyramid",
+                "ms_forward": round(net_ms, 4), "gflop": round(flops / 1e9, 2),
+                "tflops": round(flops / (net_ms * 1e-3) / 1e12, 1),
+                "mfma_frac_of_fp16_dense_peak": round(flops / (net_ms * 1e-3) / 2.5e15, 4),
+                "kernels": {k: round(ms / max(n, 1), 4) for k, (ms, n) in nprof.items()}}
+
     cpu = None
     if args.cpu_steps > 0:
         from tests import oracle_lib
@@ -199,6 +227,7 @@ def main():
                      "traffic": measured_traffic_bytes(dom) if args.points == DEFAULT_POINTS else None,
                      "algorithmic_bytes": int(alg[dom]), "avg_ms": kernels[dom]["avg_ms"]},
         "kernels": kernels,
+        "unet": unet,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

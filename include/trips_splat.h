@@ -197,7 +197,7 @@ int trips_apply_tangent(TripsCtx* ctx, double* tangent, double* poses_se3, int n
  * While enabled, every kernel the library launches through `ctx` is bracketed by HIP events on its stream.
  * trips_profile_read waits for those events, returns per kernel name the summed milliseconds and the number of
  * launches since the last read, and resets the accumulation. names[i] point to static strings. */
-#define TRIPS_PROFILE_MAX_KERNELS 16
+#define TRIPS_PROFILE_MAX_KERNELS 32
 int trips_profile_enable(TripsCtx* ctx, int enabled);
 int trips_profile_read(TripsCtx* ctx, int* n, const char* names[TRIPS_PROFILE_MAX_KERNELS],
                        float ms[TRIPS_PROFILE_MAX_KERNELS], int launches[TRIPS_PROFILE_MAX_KERNELS]);

@@ -1,0 +1,73 @@
+/* C ABI of the reconstruction net that consumes the splat's image pyramid: TRIPS' decoder-only multi-scale
+ * gated-convolution U-Net on the MI355X matrix cores (fp16 operands, fp32 accumulation). Same library and context
+ * as trips_splat.h.
+ *
+ * Replaces, for inference, MultiScaleUnet2dDecOnlySmallFixedImpl::forward
+ * (src/lib/models/Networks.h:1080-1208 of the reference) with its blocks
+ *   SmallDecStartBlockImpl                 (Networks.h:751-787)
+ *   UpsampleDecOnlySmallBlockFixedImpl     (Networks.h:999-1098)
+ * for upsample_mode = bilinear, conv_block_up = gated, norm_layer_up = id, activation = elu, last_act = id
+ * (configs/train_normalnet.ini:200-219).
+ *
+ * Network (L = num_levels, C = num_input_channels, F = filters):
+ *   x_{L-1}  = cat(in[L-1], gated3x3(in[L-1]; C -> F[L-1] - 2C))
+ *   x_i      = cat(in[i], gated3x3(cat(in[i], up2(x_{i+1})); F[i+1] -> F[i] - 2C))   for i = L-2 .. 1
+ *   x_0      = cat(in[0], gated3x3(cat(in[0], up2(x_1)); F[1] -> F[0] - C))
+ *   out      = conv1x1(x_0; F[0] -> num_output_channels)
+ * gated3x3(x) = elu(conv_f(x)) * sigmoid(conv_m(x)), 3x3, stride 1, zero padding 1; up2 = bilinear, scale 2,
+ * align_corners = false, centre-cropped to the size of in[i] when 2*size(x_{i+1}) is larger.
+ * The gated block itself lives in a dependency the reference does not vendor (Saiga, PartialConvUnet2d.h); its
+ * form here is the published one of gated convolutions.
+ */
+#ifndef TRIPS_UNET_H
+#define TRIPS_UNET_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "trips_splat.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRIPS_UNET_MAX_LEVELS 8
+
+typedef struct TripsUnetDesc {
+    int32_t abi_version;          /* TRIPS_ABI_VERSION */
+    int32_t num_levels;           /* L, 1..8: in[0..L-1] are consumed (MultiScaleUnet2dParams::num_layers) */
+    int32_t num_input_channels;   /* C, 1..8 (4 in every shipped config) */
+    int32_t num_output_channels;  /* 1..4 (3) */
+    int32_t batch;                /* images per call */
+    int32_t filters[TRIPS_UNET_MAX_LEVELS];  /* F[0..L-1] (filters_network); conv outputs must be >= 1 and <= 64 */
+    int32_t level_w[TRIPS_UNET_MAX_LEVELS];  /* size of in[i]; level i+1 must be ceil or floor of half of level i */
+    int32_t level_h[TRIPS_UNET_MAX_LEVELS];
+} TripsUnetDesc;
+
+/* Weights in the reference's tensor layouts (torch::nn::Conv2d): weight [Cout, Cin, 3, 3] and bias [Cout], fp32,
+ * device pointers. Block i < L-1 is up[i], block L-1 is the start block. */
+typedef struct TripsUnetWeights {
+    const float* feature_weight[TRIPS_UNET_MAX_LEVELS];
+    const float* feature_bias[TRIPS_UNET_MAX_LEVELS];
+    const float* mask_weight[TRIPS_UNET_MAX_LEVELS];
+    const float* mask_bias[TRIPS_UNET_MAX_LEVELS];
+    const float* final_weight; /* [num_output_channels, F[0], 1, 1] */
+    const float* final_bias;   /* [num_output_channels] */
+} TripsUnetWeights;
+
+/* Bytes of scratch trips_unet_forward needs (packed fp16 weights and the fp16 activations of every level). */
+int trips_unet_workspace_size(const TripsUnetDesc* desc, size_t* bytes);
+
+/* inputs[i]: [batch, C, level_h[i], level_w[i]] fp32 (the splat's output layout TRIPS_LAYOUT_CHW);
+ * output: [batch, num_output_channels, level_h[0], level_w[0]] fp32. Stream-ordered, allocates nothing. */
+int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
+                       const float* const inputs[TRIPS_UNET_MAX_LEVELS], float* output, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/* Multiply-accumulate operations (2 flops each) of one forward call, for utilisation figures. */
+int trips_unet_flops(const TripsUnetDesc* desc, double* flops);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -30,6 +30,40 @@ def test_library_exports_every_declared_symbol():
     assert b"gfx950" in lib.trips_version()
 
 
+def test_library_exports_every_unet_symbol():
+    lib = _lib.load()
+    src = open(os.path.join(ROOT, "include", "trips_unet.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    names = sorted(set(re.findall(r"\b(trips_unet_[a-z0-9_]+)\s*\(", src)))
+    assert names == sorted(_lib.UNET_SYMBOLS)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in trips_unet.h but not exported"
+
+
+def test_unet_ctypes_mirrors_and_host_checks(tmp_path):
+    prog = tmp_path / "sizes.c"
+    prog.write_text('#include <stdio.h>\n#include "trips_unet.h"\nint main(){printf("%zu %zu %zu\\n",'
+                    "sizeof(TripsUnetDesc),sizeof(TripsUnetWeights),offsetof(TripsUnetDesc,level_w));return 0;}\n")
+    exe = tmp_path / "sizes"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(prog), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert got == [C.sizeof(abi.TripsUnetDesc), C.sizeof(abi.TripsUnetWeights), abi.TripsUnetDesc.level_w.offset]
+    lib = _lib.load()
+    d = abi.make_unet_desc([16, 32, 64, 64], abi.layer_sizes(1920, 1080, 4))
+    b, f = C.c_size_t(0), C.c_double(0)
+    assert lib.trips_unet_workspace_size(C.byref(d), C.byref(b)) == 0
+    assert b.value >= 1920 * 1080 * 16 * 2  # fp16 activations of the finest level
+    assert lib.trips_unet_flops(C.byref(d), C.byref(f)) == 0
+    # two 3x3 convolutions per level, 2 flops per multiply-accumulate, plus the 1x1
+    want = sum(2 * 2 * 9 * cin * cout * w * h for (cin, cout, (w, h)) in
+               zip([32, 64, 64, 4], [12, 24, 56, 56], abi.layer_sizes(1920, 1080, 4))) + 2 * 16 * 3 * 1920 * 1080
+    assert abs(f.value - want) < 1e-6 * want
+    d.filters[0] = 200  # more convolution outputs than the kernels are built for
+    assert lib.trips_unet_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_UNSUPPORTED
+    d = abi.make_unet_desc([16, 32], [(100, 60), (40, 30)])  # level 1 is not half of level 0
+    assert lib.trips_unet_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_UNSUPPORTED
+
+
 def test_ctypes_mirrors_have_c_sizes(tmp_path):
     prog = tmp_path / "sizes.c"
     prog.write_text('#include <stdio.h>\n#include "trips_splat.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu\\n",'

@@ -1,0 +1,88 @@
+"""The gated-convolution U-Net forward on the matrix cores against a plain-torch fp32 restatement.
+
+Tolerance: operands are fp16 (weights, block inputs, activations between blocks), accumulation fp32. The torch
+restatement rounds at the same places, so what remains is summation order inside a 9 x Cin dot product and the fast
+exp of the device epilogue: 2e-3 of the largest output magnitude. Against the unrounded fp32 network the bar is the
+fp16 one, 2e-2."""
+import numpy as np
+import pytest
+import torch
+
+from trips_amd import abi
+
+pytestmark = pytest.mark.gpu
+
+
+def _pyramid(w, h, levels, channels, batch, seed):
+    g = torch.Generator().manual_seed(seed)
+    sizes = abi.layer_sizes(w, h, levels)
+    return [torch.rand((batch, channels, hh, ww), generator=g) for (ww, hh) in sizes]
+
+
+def _net(filters, levels, seed, cin=4):
+    from trips_amd.unet import MultiScaleUnet2dDecOnlySmallFixed, MultiScaleUnet2dParams
+    p = MultiScaleUnet2dParams(num_input_layers=levels, num_layers=levels, num_input_channels=cin,
+                               filters_network=list(filters))
+    net = MultiScaleUnet2dDecOnlySmallFixed(p)
+    g = torch.Generator().manual_seed(seed)
+    net.he_normal_(g)
+    with torch.no_grad():
+        for m in net.modules():
+            if isinstance(m, torch.nn.Conv2d):
+                m.bias.normal_(0.0, 0.1, generator=g)
+    return net
+
+
+def _compare(net, inputs, tol_rounded=2e-3, tol_fp32=2e-2):
+    from tests.ref_unet import unet_forward
+    with torch.no_grad():
+        want = unet_forward(net, inputs, half_rounding=True).numpy()
+        want32 = unet_forward(net, inputs, half_rounding=False).numpy()
+        got = net.forward([t.cuda() for t in inputs]).cpu().numpy()
+    assert got.shape == want.shape
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() < tol_rounded * scale, np.abs(got - want).max() / scale
+    assert np.abs(got - want32).max() < tol_fp32 * scale
+
+
+@pytest.mark.parametrize("filters,levels,w,h", [
+    ([16, 32, 64, 64], 4, 96, 72),      # the benchmark's channel plan; sizes halve exactly
+    ([32, 32, 32, 32, 32], 5, 100, 60),  # the shipped configuration's filters; odd sizes -> centre crop
+    ([16, 24], 2, 37, 29),               # partial tiles everywhere
+    ([20], 1, 40, 24),                   # start block only
+])
+def test_unet_forward_matches_torch(filters, levels, w, h):
+    net = _net(filters, levels, seed=levels)
+    inputs = _pyramid(w, h, levels, 4, batch=2, seed=10 + levels)
+    if levels == 1:
+        # a one-level net feeds the final 1x1 with F[0] - C channels; the reference's final expects F[0]
+        net.final = torch.nn.Conv2d(filters[0] - 4, 3, 1)
+    _compare(net, inputs)
+
+
+def test_unet_forward_three_input_channels():
+    net = _net([16, 32, 32], 3, seed=5, cin=3)
+    inputs = _pyramid(64, 48, 3, 3, batch=1, seed=6)
+    _compare(net, inputs)
+
+
+def test_unet_extra_input_layers_are_ignored():
+    # the splat renders 8 layers, the net may consume fewer (num_input_layers > num_layers)
+    from trips_amd.unet import MultiScaleUnet2dDecOnlySmallFixed, MultiScaleUnet2dParams
+    p = MultiScaleUnet2dParams(num_input_layers=4, num_layers=2, filters_network=[16, 32])
+    net = MultiScaleUnet2dDecOnlySmallFixed(p).he_normal_(torch.Generator().manual_seed(1))
+    inputs = _pyramid(64, 32, 4, 4, batch=1, seed=2)
+    from tests.ref_unet import unet_forward
+    with torch.no_grad():
+        want = unet_forward(net, inputs).numpy()
+        got = net.forward([t.cuda() for t in inputs]).cpu().numpy()
+    assert np.abs(got - want).max() < 2e-3 * np.abs(want).max()
+
+
+def test_unet_refuses_autograd_and_cpu_tensors():
+    net = _net([16, 32], 2, seed=1)
+    inputs = _pyramid(32, 32, 2, 4, batch=1, seed=2)
+    with pytest.raises(NotImplementedError):
+        net.forward([t.cuda() for t in inputs])
+    with torch.no_grad(), pytest.raises(RuntimeError):
+        net.forward(inputs)

@@ -17,6 +17,8 @@ SYMBOLS = [
     "trips_splat_check", "trips_splat_counters", "trips_splat_export_lists", "trips_splat_export_points",
     "trips_adam_step_fused", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
 ]
+# every symbol include/trips_unet.h declares
+UNET_SYMBOLS = ["trips_unet_workspace_size", "trips_unet_forward", "trips_unet_flops"]
 
 
 class TripsError(RuntimeError):
@@ -55,6 +57,10 @@ def load():
     lib.trips_splat_export_points.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), vp, i32, vp, vp, vp, vp, vp]
     lib.trips_adam_step_fused.argtypes = [vp, C.POINTER(abi.TripsAdamTensor), i32, vp]
     lib.trips_apply_tangent.argtypes = [vp, vp, vp, i32, vp]
+    lib.trips_unet_workspace_size.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_size_t)]
+    lib.trips_unet_flops.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_double)]
+    lib.trips_unet_forward.argtypes = [vp, C.POINTER(abi.TripsUnetDesc), C.POINTER(abi.TripsUnetWeights),
+                                       C.POINTER(vp), vp, vp, C.c_size_t, vp]
     lib.trips_profile_enable.argtypes = [vp, i32]
     lib.trips_profile_read.argtypes = [vp, C.POINTER(i32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
                                        C.POINTER(i32)]

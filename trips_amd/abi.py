@@ -8,6 +8,8 @@ import ctypes as C
 TRIPS_MAX_LAYERS = 8
 TRIPS_MAX_VIEWS = 16
 TRIPS_ABI_VERSION = 1
+TRIPS_PROFILE_MAX_KERNELS = 32
+TRIPS_UNET_MAX_LEVELS = 8
 
 TRIPS_OK = 0
 TRIPS_ERR_INVALID_ARG = 1
@@ -114,6 +116,46 @@ class TripsAdamTensor(C.Structure):
         ("upper_lr_bound", C.c_float),
         ("loss_scale", C.c_float),
     ]
+
+
+class TripsUnetDesc(C.Structure):
+    """include/trips_unet.h"""
+    _fields_ = [
+        ("abi_version", C.c_int32),
+        ("num_levels", C.c_int32),
+        ("num_input_channels", C.c_int32),
+        ("num_output_channels", C.c_int32),
+        ("batch", C.c_int32),
+        ("filters", C.c_int32 * TRIPS_UNET_MAX_LEVELS),
+        ("level_w", C.c_int32 * TRIPS_UNET_MAX_LEVELS),
+        ("level_h", C.c_int32 * TRIPS_UNET_MAX_LEVELS),
+    ]
+
+
+class TripsUnetWeights(C.Structure):
+    _fields_ = [
+        ("feature_weight", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("feature_bias", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("mask_weight", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("mask_bias", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("final_weight", C.c_void_p),
+        ("final_bias", C.c_void_p),
+    ]
+
+
+def make_unet_desc(filters, level_sizes, num_input_channels=4, num_output_channels=3, batch=1):
+    """level_sizes: [(w, h)] of the pyramid levels the net consumes, finest first."""
+    d = TripsUnetDesc()
+    d.abi_version = TRIPS_ABI_VERSION
+    d.num_levels = len(level_sizes)
+    d.num_input_channels = num_input_channels
+    d.num_output_channels = num_output_channels
+    d.batch = batch
+    for i, (w, h) in enumerate(level_sizes):
+        d.filters[i] = int(filters[i])
+        d.level_w[i] = int(w)
+        d.level_h[i] = int(h)
+    return d
 
 
 FLT_MAX = 3.4028234663852886e38

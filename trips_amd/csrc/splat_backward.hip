@@ -213,7 +213,6 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
 template <int C>
 __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardParams p)
 {
-    constexpr int CPAD = (C + 3) & ~3;
     constexpr int EF   = (1 + C + 3) & ~3;
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
     const int lane     = threadIdx.x & 63;

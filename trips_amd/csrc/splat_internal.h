@@ -72,6 +72,20 @@ struct ProfScope
     }
 };
 
+// records the message trips_last_error_string() returns on this thread; returns `code`
+int set_error(int code, const char* fmt, ...);
+
+}  // namespace trips
+
+// The opaque context of the C ABI.
+struct TripsCtx
+{
+    int device;
+    trips::Profiler prof;
+};
+
+namespace trips
+{
 // Per-point records written by the projection pass.
 //   rec[pid]   4 + Cpad floats {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)}:
 //              everything the blend and the pixel pass of the backward need in one aligned gather of 32 bytes at

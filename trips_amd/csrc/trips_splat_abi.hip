@@ -27,23 +27,29 @@ hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists
 
 using namespace trips;
 
-struct TripsCtx
-{
-    int device;
-    Profiler prof;
-};
-
 namespace
 {
 thread_local char g_error[512] = "";
+}
 
-int fail(int code, const char* fmt, ...)
+namespace trips
+{
+int set_error(int code, const char* fmt, ...)
 {
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
     va_end(ap);
     return code;
+}
+}  // namespace trips
+
+namespace
+{
+template <typename... A>
+int fail(int code, const char* fmt, A... a)
+{
+    return trips::set_error(code, fmt, a...);
 }
 
 int hip_fail(hipError_t e, const char* what)

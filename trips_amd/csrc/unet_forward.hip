@@ -1,0 +1,549 @@
+// Forward of the decoder-only gated-convolution U-Net on the gfx950 matrix cores.
+//
+//   gated_conv3x3_kernel <- SmallDecStartBlockImpl::forward / UpsampleDecOnlySmallBlockFixedImpl::forward
+//                           src/lib/models/Networks.h:751-787, 999-1098
+//   final_conv1x1_kernel <- the `final` Sequential of MultiScaleUnet2dDecOnlySmallFixedImpl, Networks.h:1129-1131
+//
+// The reference runs, per level, upsample -> cat -> two 3x3 convolutions -> elu / sigmoid -> multiply -> cat as
+// separate libtorch ops on NCHW tensors, materialising every intermediate. Here one kernel per level does all of
+// it as an implicit GEMM: M = 256 output pixels of an 8 x 32 patch, N = feature and mask outputs side by side,
+// K = 9 taps x input channels. The input patch (with its one-pixel halo) is assembled in LDS, channels innermost:
+// channels [0, C) come straight from this level's splat image, the others are the bilinear 2x upsampling of the
+// level below (its splat image, then its convolution outputs), computed while loading, so neither the upsampled
+// tensor nor the concatenations ever exist in memory. Activations between levels are fp16, channels innermost.
+// MFMA: v_mfma_f32_16x16x32_f16; lane l holds, of A, row l % 16 and the 8 consecutive K values (l / 16) * 8 ..,
+// of B the same for column l % 16, and of the 16 x 16 result rows (l / 16) * 4 .. + 3 of column l % 16.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "../../include/trips_unet.h"
+#include "splat_internal.h"
+
+namespace trips
+{
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kConvTileH   = 8;
+constexpr int kConvTileW   = 32;
+constexpr int kConvPatchH  = kConvTileH + 2;
+constexpr int kConvPatchW  = kConvTileW + 2;
+constexpr int kBelowH      = kConvTileH / 2 + 2;  // rows / columns of the level below that an upsampled patch touches
+constexpr int kBelowW      = kConvTileW / 2 + 2;
+constexpr int kLdsChanPad  = 8;  // halves added to every LDS row so that 16 lanes reading 16 bytes hit 64 distinct banks
+
+struct ConvParams
+{
+    int H, W;            // this level
+    int Hb, Wb;          // level below (0 x 0 for the start block)
+    int c_feat;          // channels of the splat images (C)
+    int cb_store;        // halves per pixel of act_below (multiple of 8; channels past the real ones hold zero)
+    int cout;            // real outputs of each of the two convolutions
+    int cout_store;      // halves per pixel of `out` (multiple of 8)
+    const float* feat;        // [C][H][W]
+    const float* feat_below;  // [C][Hb][Wb]
+    const _Float16* act_below;  // [Hb][Wb][cb_store]
+    const _Float16* wpack;    // [9][NPAD][CIN]
+    const float* bias;        // [NPAD]: feature biases, then mask biases, each padded to NPAD / 2
+    _Float16* out;            // [H][W][cout_store]
+};
+
+// source row / column and weight of torch's bilinear upsampling with scale_factor 2, align_corners = false
+// (area_pixel_compute_source_index: src = max(0, (dst + 0.5) * 0.5 - 0.5))
+__device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i1, float& lambda)
+{
+    float src = (float(dst) + 0.5f) * 0.5f - 0.5f;
+    src       = src < 0.f ? 0.f : src;
+    i0        = (int)src;
+    i0        = i0 < in_size - 1 ? i0 : in_size - 1;
+    i1        = i0 + 1 < in_size ? i0 + 1 : in_size - 1;
+    lambda    = src - float(i0);
+}
+
+template <int CIN, int NPAD>
+__global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
+{
+    constexpr int ROW  = CIN + kLdsChanPad;  // halves per patch pixel in LDS
+    constexpr int NB   = NPAD / 16;          // 16-column blocks; the first half are feature outputs
+    constexpr int HB   = NB / 2;
+    constexpr int KB   = CIN / 32;
+    extern __shared__ _Float16 smem[];
+    _Float16* s_patch = smem;  // [kConvPatchH * kConvPatchW][ROW]
+
+    const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
+    const bool has_below = p.Hb > 0;
+
+    // ---- stage 1: everything the patch needs from memory, all loads of a thread in flight together ----
+    // (a) this level's image -> channels [0, C) of the patch; (b) the level below, x_{i+1} = cat(image, activations),
+    // as a (TILE/2 + 2)^2 patch in the same row format, channel k of the concatenated input at row position k.
+    constexpr int GROUPS = CIN / 8;
+    _Float16* s_below    = s_patch + kConvPatchH * kConvPatchW * ROW;  // [kBelowH * kBelowW][ROW]
+    const int by0 = y0 / 2 - 1, bx0 = x0 / 2 - 1;
+    const int C   = p.c_feat;
+    {
+        const size_t plane = (size_t)p.H * p.W;
+        for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW; item += 256)
+        {
+            const int py = item / kConvPatchW, px = item - py * kConvPatchW;
+            const int y = y0 + py - 1, x = x0 + px - 1;
+            const bool in = y >= 0 && y < p.H && x >= 0 && x < p.W;
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            if (in)
+                for (int c = 0; c < C; ++c) v[c] = p.feat[c * plane + (size_t)y * p.W + x];
+            _Float16* row = s_patch + (size_t)item * ROW;
+            for (int c = 0; c < C; ++c) row[c] = _Float16(v[c]);
+            if (!has_below)
+            {
+                // start block: the image is the whole input
+                for (int c = C; c < CIN; ++c) row[c] = _Float16(0.f);
+            }
+        }
+    }
+    if (has_below)
+    {
+        const size_t pb = (size_t)p.Hb * p.Wb;
+        const int act_groups = p.cb_store / 8;
+        const int per_pixel  = 1 + act_groups;  // item 0 of a pixel: the image below; others: 8 activations each
+        for (int item = threadIdx.x; item < kBelowH * kBelowW * per_pixel; item += 256)
+        {
+            const int q = item % per_pixel, bp = item / per_pixel;
+            const int r = bp / kBelowW, c0 = bp - r * kBelowW;
+            const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
+            _Float16* row = s_below + (size_t)bp * ROW;
+            if (q == 0)
+            {
+                for (int c = 0; c < C; ++c) row[C + c] = _Float16(p.feat_below[c * pb + (size_t)yy * p.Wb + xx]);
+                for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);  // padding channels
+            }
+            else
+            {
+                const half8 a = *reinterpret_cast<const half8*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+                const int pos = 2 * C + 8 * (q - 1);
+                if (C == 4)
+                    *reinterpret_cast<half8*>(row + pos) = a;
+                else
+                    for (int i = 0; i < 8; ++i)
+                        if (pos + i < CIN) row[pos + i] = a[i];
+            }
+        }
+        __syncthreads();
+        // ---- stage 2: bilinear 2x upsampling from the below patch into channels [C, CIN) of the patch ----
+        for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
+        {
+            const int g = item % GROUPS, pp = item / GROUPS;
+            const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
+            const int y = y0 + py - 1, x = x0 + px - 1;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = 0.f;
+            if (y >= 0 && y < p.H && x >= 0 && x < p.W)
+            {
+                int ya, yb, xa, xb;
+                float ly, lx;
+                up2_source(y, p.Hb, ya, yb, ly);
+                up2_source(x, p.Wb, xa, xb, lx);
+                const float w00 = (1.f - ly) * (1.f - lx), w01 = (1.f - ly) * lx, w10 = ly * (1.f - lx), w11 = ly * lx;
+                const half8 a = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
+                const half8 b = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
+                const half8 c = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
+                const half8 d = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = w00 * float(a[i]) + w01 * float(b[i]) + w10 * float(c[i]) + w11 * float(d[i]);
+            }
+            _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
+            if (g == 0)
+            {
+                for (int i = C; i < 8; ++i) dst[i] = _Float16(v[i]);  // [0, C) holds this level's image
+            }
+            else
+            {
+                half8 h;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = _Float16(v[i]);
+                *reinterpret_cast<half8*>(dst) = h;
+            }
+        }
+    }
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lrow = lane & 15, lk = (lane >> 4) * 8;
+    floatx4 acc[4][NB];
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int n = 0; n < NB; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // B fragments come straight from memory: the packed weights are a few tens of KB that every wavefront of
+    // every workgroup reads at the same addresses, so they stay in L2 / L1, and the tap loop needs no barrier.
+    // The fragments of the next tap are requested before the current tap's MFMAs are issued.
+    __syncthreads();  // patch complete
+    const _Float16* wlane = p.wpack + (size_t)lrow * CIN + lk;
+    half8 bcur[KB][NB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int n = 0; n < NB; ++n) bcur[kb][n] = *reinterpret_cast<const half8*>(wlane + (size_t)(n * 16) * CIN + kb * 32);
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap)
+    {
+        const int dy = tap / 3, dx = tap - dy * 3;  // patch coordinates already include the halo
+        half8 bnext[KB][NB];
+        if (tap + 1 < 9)
+        {
+            const _Float16* wt = wlane + (size_t)(tap + 1) * NPAD * CIN;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int n = 0; n < NB; ++n) bnext[kb][n] = *reinterpret_cast<const half8*>(wt + (size_t)(n * 16) * CIN + kb * 32);
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+        {
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+            {
+                const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
+                const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
+#pragma unroll
+                for (int n = 0; n < NB; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[kb][n], acc[m][n], 0, 0, 0);
+            }
+        }
+        if (tap + 1 < 9)
+        {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int n = 0; n < NB; ++n) bcur[kb][n] = bnext[kb][n];
+        }
+    }
+
+    // ---- epilogue: elu(feature) * sigmoid(mask), fp16, channels innermost ----
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+    {
+        const int y = y0 + 2 * wave + (m >> 1);
+#pragma unroll
+        for (int j = 0; j < HB; ++j)
+        {
+            const int ch = 16 * j + lrow;
+            if (ch >= p.cout_store) continue;
+            const float bf = p.bias[ch], bm = p.bias[NPAD / 2 + ch];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                const int x = x0 + (m & 1) * 16 + (lane >> 4) * 4 + i;
+                if (y >= p.H || x >= p.W) continue;
+                const float f = acc[m][j][i] + bf, g = acc[m][HB + j][i] + bm;
+                const float e = f > 0.f ? f : (__expf(f) - 1.f);
+                const float s = 1.f / (1.f + __expf(-g));
+                p.out[((size_t)y * p.W + x) * p.cout_store + ch] = ch < p.cout ? _Float16(e * s) : _Float16(0.f);
+            }
+        }
+    }
+}
+
+// wpack[tap][n][c]: n < NPAD/2 feature output n, else mask output n - NPAD/2; zero outside the real ranges
+__global__ __launch_bounds__(256) void pack_conv_weights_kernel(const float* __restrict__ wf, const float* __restrict__ bf,
+                                                                const float* __restrict__ wm, const float* __restrict__ bm,
+                                                                int cout, int cin_real, int cin_pad, int npad,
+                                                                _Float16* __restrict__ wpack, float* __restrict__ bias)
+{
+    const int total = 9 * npad * cin_pad;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256)
+    {
+        const int c = i % cin_pad, n = (i / cin_pad) % npad, tap = i / (cin_pad * npad);
+        const int half = npad / 2;
+        const int o    = n < half ? n : n - half;
+        float v        = 0.f;
+        if (o < cout && c < cin_real) v = (n < half ? wf : wm)[((size_t)o * cin_real + c) * 9 + tap];
+        wpack[i] = _Float16(v);
+    }
+    for (int n = blockIdx.x * 256 + threadIdx.x; n < npad; n += gridDim.x * 256)
+    {
+        const int half = npad / 2;
+        const int o    = n < half ? n : n - half;
+        bias[n]        = o < cout ? (n < half ? bf : bm)[o] : 0.f;
+    }
+}
+
+struct FinalParams
+{
+    int H, W, c_feat, cact, cact_store, cout;
+    const float* feat;      // [C][H][W]
+    const _Float16* act;    // [H][W][cact_store]
+    const float* weight;    // [cout][c_feat + cact]
+    const float* bias;      // [cout]
+    float* out;             // [cout][H][W]
+};
+
+__global__ __launch_bounds__(256) void final_conv1x1_kernel(const FinalParams p)
+{
+    __shared__ float s_w[4 * 80];
+    __shared__ float s_b[4];
+    const int cin = p.c_feat + p.cact;
+    for (int i = threadIdx.x; i < p.cout * cin; i += 256) s_w[i] = float(_Float16(p.weight[i]));
+    if (threadIdx.x < p.cout) s_b[threadIdx.x] = p.bias[threadIdx.x];
+    __syncthreads();
+    const size_t plane = (size_t)p.H * p.W;
+    for (size_t pix = (size_t)blockIdx.x * 256 + threadIdx.x; pix < plane; pix += (size_t)gridDim.x * 256)
+    {
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < p.c_feat; ++c)
+        {
+            const float v = float(_Float16(p.feat[c * plane + pix]));
+            for (int k = 0; k < p.cout; ++k) o[k] += s_w[k * cin + c] * v;
+        }
+        const _Float16* a = p.act + pix * p.cact_store;
+        for (int c = 0; c < p.cact; ++c)
+        {
+            const float v = float(a[c]);
+            for (int k = 0; k < p.cout; ++k) o[k] += s_w[k * cin + p.c_feat + c] * v;
+        }
+        for (int k = 0; k < p.cout; ++k) p.out[k * plane + pix] = o[k] + s_b[k];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+namespace
+{
+int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+struct LevelPlan
+{
+    int H, W, cin_real, cin_pad, cout, npad, cout_store;
+    size_t wpack_off, bias_off, act_off;  // bytes into the workspace
+};
+
+struct NetPlan
+{
+    LevelPlan lv[TRIPS_UNET_MAX_LEVELS];
+    size_t bytes;
+};
+
+int check_unet_desc(const TripsUnetDesc* d)
+{
+    if (!d) return set_error(TRIPS_ERR_INVALID_ARG, "desc is NULL");
+    if (d->abi_version != TRIPS_ABI_VERSION)
+        return set_error(TRIPS_ERR_INVALID_ARG, "abi_version %d, library has %d", d->abi_version, TRIPS_ABI_VERSION);
+    if (d->num_levels < 1 || d->num_levels > TRIPS_UNET_MAX_LEVELS)
+        return set_error(TRIPS_ERR_INVALID_ARG, "num_levels %d not in 1..%d", d->num_levels, TRIPS_UNET_MAX_LEVELS);
+    if (d->num_input_channels < 1 || d->num_input_channels > 4)
+        return set_error(TRIPS_ERR_UNSUPPORTED, "num_input_channels %d not in 1..4", d->num_input_channels);
+    if (d->num_output_channels < 1 || d->num_output_channels > 4)
+        return set_error(TRIPS_ERR_UNSUPPORTED, "num_output_channels %d not in 1..4", d->num_output_channels);
+    if (d->batch < 1) return set_error(TRIPS_ERR_INVALID_ARG, "batch < 1");
+    const int C = d->num_input_channels, L = d->num_levels;
+    for (int i = 0; i < L; ++i)
+    {
+        if (d->level_w[i] < 1 || d->level_h[i] < 1 || d->level_w[i] > 32768 || d->level_h[i] > 32768)
+            return set_error(TRIPS_ERR_INVALID_ARG, "level %d size %dx%d", i, d->level_w[i], d->level_h[i]);
+        if (i > 0)
+        {
+            const int w = d->level_w[i - 1], h = d->level_h[i - 1];
+            const bool okw = d->level_w[i] == w / 2 || d->level_w[i] == (w + 1) / 2;
+            const bool okh = d->level_h[i] == h / 2 || d->level_h[i] == (h + 1) / 2;
+            if (!okw || !okh || 2 * d->level_w[i] < w || 2 * d->level_h[i] < h)
+                return set_error(TRIPS_ERR_UNSUPPORTED, "level %d (%dx%d) must be half of level %d (%dx%d), rounded up", i,
+                                 d->level_w[i], d->level_h[i], i - 1, w, h);
+        }
+        const int cout = d->filters[i] - ((i == 0 && L > 1) ? C : 2 * C);
+        if (cout < 1 || cout > 64)
+            return set_error(TRIPS_ERR_UNSUPPORTED, "filters[%d] = %d gives %d convolution outputs (1..64 supported)", i,
+                             d->filters[i], cout);
+        if (i + 1 < L && d->filters[i + 1] > 64)
+            return set_error(TRIPS_ERR_UNSUPPORTED, "filters[%d] = %d input channels (at most 64 supported)", i + 1,
+                             d->filters[i + 1]);
+    }
+    return TRIPS_OK;
+}
+
+// Block i convolves cat(in[i], up2(x_{i+1})) (F[i+1] channels; C for the start block) to F[i] - 2C outputs
+// (F[0] - C for the last block when it is not also the start block), Networks.h:1034-1037,1104-1118.
+NetPlan make_plan(const TripsUnetDesc& d)
+{
+    NetPlan np;
+    const int C = d.num_input_channels, L = d.num_levels;
+    size_t o = 0;
+    for (int i = 0; i < L; ++i)
+    {
+        LevelPlan& lv = np.lv[i];
+        lv.H          = d.level_h[i];
+        lv.W          = d.level_w[i];
+        lv.cin_real   = (i == L - 1) ? C : d.filters[i + 1];
+        lv.cin_pad    = lv.cin_real <= 32 ? 32 : 64;
+        lv.cout       = d.filters[i] - ((i == 0 && L > 1) ? C : 2 * C);
+        lv.npad       = 2 * round_up(lv.cout, 16);
+        lv.cout_store = round_up(lv.cout, 8);
+        lv.wpack_off  = o;
+        o += align256((size_t)9 * lv.npad * lv.cin_pad * sizeof(_Float16));
+        lv.bias_off = o;
+        o += align256((size_t)lv.npad * sizeof(float));
+    }
+    for (int i = 0; i < L; ++i)
+    {
+        np.lv[i].act_off = o;
+        o += align256((size_t)d.batch * np.lv[i].H * np.lv[i].W * np.lv[i].cout_store * sizeof(_Float16));
+    }
+    np.bytes = o;
+    return np;
+}
+
+template <int CIN, int NPAD>
+hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
+{
+    constexpr int ROW  = CIN + kLdsChanPad;
+    const size_t lds   = (size_t)((kConvPatchH * kConvPatchW + kBelowH * kBelowW) * ROW) * sizeof(_Float16);  // 36 or 65 KB
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    dim3 grid((p.W + kConvTileW - 1) / kConvTileW, (p.H + kConvTileH - 1) / kConvTileH);
+    hipLaunchKernelGGL((gated_conv3x3_kernel<CIN, NPAD>), grid, dim3(256), lds, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t dispatch_conv(const ConvParams& p, int cin_pad, int npad, hipStream_t stream)
+{
+    if (cin_pad == 32)
+    {
+        if (npad == 32) return launch_conv<32, 32>(p, stream);
+        if (npad == 64) return launch_conv<32, 64>(p, stream);
+        if (npad == 96) return launch_conv<32, 96>(p, stream);
+        if (npad == 128) return launch_conv<32, 128>(p, stream);
+    }
+    else
+    {
+        if (npad == 32) return launch_conv<64, 32>(p, stream);
+        if (npad == 64) return launch_conv<64, 64>(p, stream);
+        if (npad == 96) return launch_conv<64, 96>(p, stream);
+        if (npad == 128) return launch_conv<64, 128>(p, stream);
+    }
+    return hipErrorInvalidValue;
+}
+}  // namespace
+}  // namespace trips
+
+using namespace trips;
+
+extern "C" {
+
+int trips_unet_workspace_size(const TripsUnetDesc* desc, size_t* bytes)
+{
+    if (int e = check_unet_desc(desc)) return e;
+    if (!bytes) return set_error(TRIPS_ERR_INVALID_ARG, "bytes is NULL");
+    *bytes = make_plan(*desc).bytes;
+    return TRIPS_OK;
+}
+
+int trips_unet_flops(const TripsUnetDesc* desc, double* flops)
+{
+    if (int e = check_unet_desc(desc)) return e;
+    if (!flops) return set_error(TRIPS_ERR_INVALID_ARG, "flops is NULL");
+    const NetPlan np = make_plan(*desc);
+    double f         = 0.0;
+    for (int i = 0; i < desc->num_levels; ++i)
+        f += 2.0 * 2.0 * 9.0 * np.lv[i].cin_real * np.lv[i].cout * (double)np.lv[i].H * np.lv[i].W;
+    f += 2.0 * desc->filters[0] * desc->num_output_channels * (double)desc->level_h[0] * desc->level_w[0];
+    *flops = f * desc->batch;
+    return TRIPS_OK;
+}
+
+int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
+                       const float* const inputs[TRIPS_UNET_MAX_LEVELS], float* output, void* workspace,
+                       size_t workspace_bytes, void* stream_)
+{
+    if (!ctx) return set_error(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_unet_desc(desc)) return e;
+    if (!weights || !inputs || !output || !workspace) return set_error(TRIPS_ERR_INVALID_ARG, "NULL argument");
+    const TripsUnetDesc& d = *desc;
+    const int C = d.num_input_channels, L = d.num_levels;
+    for (int i = 0; i < L; ++i)
+    {
+        if (!inputs[i]) return set_error(TRIPS_ERR_INVALID_ARG, "inputs[%d] is NULL", i);
+        if (!weights->feature_weight[i] || !weights->feature_bias[i] || !weights->mask_weight[i] || !weights->mask_bias[i])
+            return set_error(TRIPS_ERR_INVALID_ARG, "weights of block %d are NULL", i);
+    }
+    if (!weights->final_weight || !weights->final_bias) return set_error(TRIPS_ERR_INVALID_ARG, "final weights are NULL");
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return set_error(TRIPS_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
+    const NetPlan np = make_plan(d);
+    if (workspace_bytes < np.bytes)
+        return set_error(TRIPS_ERR_WORKSPACE_SMALL, "workspace has %zu bytes, %zu needed", workspace_bytes, np.bytes);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    char* ws           = reinterpret_cast<char*>(workspace);
+    Profiler* prof     = ctx->prof.enabled ? &ctx->prof : nullptr;
+
+    {
+        ProfScope ps(prof, "unet_pack_weights", stream);
+        for (int i = 0; i < L; ++i)
+        {
+            const LevelPlan& lv = np.lv[i];
+            const int total     = 9 * lv.npad * lv.cin_pad;
+            hipLaunchKernelGGL(pack_conv_weights_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
+                               weights->feature_weight[i], weights->feature_bias[i], weights->mask_weight[i],
+                               weights->mask_bias[i], lv.cout, lv.cin_real, lv.cin_pad, lv.npad,
+                               reinterpret_cast<_Float16*>(ws + lv.wpack_off), reinterpret_cast<float*>(ws + lv.bias_off));
+        }
+    }
+    static const char* const kLevelNames[TRIPS_UNET_MAX_LEVELS] = {"unet_conv_l0", "unet_conv_l1", "unet_conv_l2", "unet_conv_l3",
+                                                                   "unet_conv_l4", "unet_conv_l5", "unet_conv_l6", "unet_conv_l7"};
+    for (int i = L - 1; i >= 0; --i)
+    {
+        const LevelPlan& lv = np.lv[i];
+        ProfScope ps(prof, kLevelNames[i], stream);
+        for (int b = 0; b < d.batch; ++b)
+        {
+            ConvParams p;
+            std::memset(&p, 0, sizeof(p));
+            p.H          = lv.H;
+            p.W          = lv.W;
+            p.c_feat     = C;
+            p.cout       = lv.cout;
+            p.cout_store = lv.cout_store;
+            p.feat       = inputs[i] + (size_t)b * C * lv.H * lv.W;
+            p.wpack      = reinterpret_cast<const _Float16*>(ws + lv.wpack_off);
+            p.bias       = reinterpret_cast<const float*>(ws + lv.bias_off);
+            p.out        = reinterpret_cast<_Float16*>(ws + lv.act_off) + (size_t)b * lv.H * lv.W * lv.cout_store;
+            if (i < L - 1)
+            {
+                const LevelPlan& lb = np.lv[i + 1];
+                p.Hb         = lb.H;
+                p.Wb         = lb.W;
+                p.cb_store   = lb.cout_store;
+                p.feat_below = inputs[i + 1] + (size_t)b * C * lb.H * lb.W;
+                p.act_below  = reinterpret_cast<const _Float16*>(ws + lb.act_off) + (size_t)b * lb.H * lb.W * lb.cout_store;
+            }
+            hipError_t e = dispatch_conv(p, lv.cin_pad, lv.npad, stream);
+            if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "gated conv launch (level %d): %s", i, hipGetErrorString(e));
+        }
+    }
+    {
+        ProfScope ps(prof, "unet_final_1x1", stream);
+        const LevelPlan& lv = np.lv[0];
+        for (int b = 0; b < d.batch; ++b)
+        {
+            FinalParams p;
+            p.H          = lv.H;
+            p.W          = lv.W;
+            p.c_feat     = C;
+            p.cact       = lv.cout;
+            p.cact_store = lv.cout_store;
+            p.cout       = d.num_output_channels;
+            p.feat       = inputs[0] + (size_t)b * C * lv.H * lv.W;
+            p.act        = reinterpret_cast<const _Float16*>(ws + lv.act_off) + (size_t)b * lv.H * lv.W * lv.cout_store;
+            p.weight     = weights->final_weight;
+            p.bias       = weights->final_bias;
+            p.out        = output + (size_t)b * d.num_output_channels * lv.H * lv.W;
+            const size_t plane = (size_t)lv.H * lv.W;
+            const int blocks   = (int)std::min<size_t>((plane + 255) / 256, 65535);
+            hipLaunchKernelGGL(final_conv1x1_kernel, dim3(blocks), dim3(256), 0, stream, p);
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "final conv launch: %s", hipGetErrorString(e));
+    }
+    return TRIPS_OK;
+}
+
+}  // extern "C"

@@ -145,9 +145,9 @@ class SplatContext:
     def profile_read(self):
         """{kernel name: (milliseconds summed over launches, launches)} since the last read."""
         n = C.c_int(0)
-        names = (C.c_char_p * 16)()
-        ms = (C.c_float * 16)()
-        launches = (C.c_int * 16)()
+        names = (C.c_char_p * abi.TRIPS_PROFILE_MAX_KERNELS)()
+        ms = (C.c_float * abi.TRIPS_PROFILE_MAX_KERNELS)()
+        launches = (C.c_int * abi.TRIPS_PROFILE_MAX_KERNELS)()
         _lib.check(self.lib.trips_profile_read(self.ctx, C.byref(n), names, ms, launches))
         return {names[i].decode(): (float(ms[i]), int(launches[i])) for i in range(n.value)}
 
