@@ -55,14 +55,42 @@ typedef struct TripsUnetWeights {
     const float* final_bias;   /* [num_output_channels] */
 } TripsUnetWeights;
 
-/* Bytes of scratch trips_unet_forward needs (packed fp16 weights and the fp16 activations of every level). */
+/* Gradients of one backward call, fp32, the reference's layouts, device pointers. Everything is written, not
+ * accumulated; NULL members are skipped. */
+typedef struct TripsUnetGrads {
+    float* feature_weight[TRIPS_UNET_MAX_LEVELS];
+    float* feature_bias[TRIPS_UNET_MAX_LEVELS];
+    float* mask_weight[TRIPS_UNET_MAX_LEVELS];
+    float* mask_bias[TRIPS_UNET_MAX_LEVELS];
+    float* final_weight;
+    float* final_bias;
+    float* inputs[TRIPS_UNET_MAX_LEVELS]; /* dL/d in[i]: the splat's grad_image of level i; required for i < L */
+} TripsUnetGrads;
+
+/* Bytes of scratch trips_unet_forward needs (packed fp16 weights and, without a saved state, the fp16 block
+ * outputs of every level). */
 int trips_unet_workspace_size(const TripsUnetDesc* desc, size_t* bytes);
+/* Bytes of the state a training forward keeps for the backward (fp16 block outputs and pre-activations). */
+int trips_unet_saved_size(const TripsUnetDesc* desc, size_t* bytes);
+/* Bytes of scratch trips_unet_backward needs. */
+int trips_unet_backward_workspace_size(const TripsUnetDesc* desc, size_t* bytes);
 
 /* inputs[i]: [batch, C, level_h[i], level_w[i]] fp32 (the splat's output layout TRIPS_LAYOUT_CHW);
- * output: [batch, num_output_channels, level_h[0], level_w[0]] fp32. Stream-ordered, allocates nothing. */
+ * output: [batch, num_output_channels, level_h[0], level_w[0]] fp32; saved: NULL for inference, else
+ * trips_unet_saved_size bytes, 256-byte aligned. Stream-ordered, allocates nothing. */
 int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
-                       const float* const inputs[TRIPS_UNET_MAX_LEVELS], float* output, void* workspace,
+                       const float* const inputs[TRIPS_UNET_MAX_LEVELS], float* output, void* saved, void* workspace,
                        size_t workspace_bytes, void* stream);
+
+/* Backward of the forward that wrote `saved` (same desc, weights and inputs). d_output: [batch, out, H, W] fp32.
+ * Intermediate gradients are fp16: they are carried multiplied by grad_scale (a power of two such as 65536 keeps
+ * dL/doutput ~ 1e-7 of a mean loss over millions of pixels in range) and every fp32 result is divided by it again.
+ * Replaces what autograd does for MultiScaleUnet2dDecOnlySmallFixedImpl::forward in the reference
+ * (src/lib/models/Networks.h:1139-1191). Only num_input_channels = 4. Stream-ordered, allocates nothing. */
+int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
+                        const float* const inputs[TRIPS_UNET_MAX_LEVELS], const void* saved, const float* d_output,
+                        float grad_scale, const TripsUnetGrads* grads, void* workspace, size_t workspace_bytes,
+                        void* stream);
 
 /* Multiply-accumulate operations (2 flops each) of one forward call, for utilisation figures. */
 int trips_unet_flops(const TripsUnetDesc* desc, double* flops);

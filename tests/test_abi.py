@@ -42,12 +42,14 @@ def test_library_exports_every_unet_symbol():
 
 def test_unet_ctypes_mirrors_and_host_checks(tmp_path):
     prog = tmp_path / "sizes.c"
-    prog.write_text('#include <stdio.h>\n#include "trips_unet.h"\nint main(){printf("%zu %zu %zu\\n",'
-                    "sizeof(TripsUnetDesc),sizeof(TripsUnetWeights),offsetof(TripsUnetDesc,level_w));return 0;}\n")
+    prog.write_text('#include <stdio.h>\n#include "trips_unet.h"\nint main(){printf("%zu %zu %zu %zu\\n",'
+                    "sizeof(TripsUnetDesc),sizeof(TripsUnetWeights),offsetof(TripsUnetDesc,level_w),"
+                    "sizeof(TripsUnetGrads));return 0;}\n")
     exe = tmp_path / "sizes"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(prog), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
-    assert got == [C.sizeof(abi.TripsUnetDesc), C.sizeof(abi.TripsUnetWeights), abi.TripsUnetDesc.level_w.offset]
+    assert got == [C.sizeof(abi.TripsUnetDesc), C.sizeof(abi.TripsUnetWeights), abi.TripsUnetDesc.level_w.offset,
+                   C.sizeof(abi.TripsUnetGrads)]
     lib = _lib.load()
     d = abi.make_unet_desc([16, 32, 64, 64], abi.layer_sizes(1920, 1080, 4))
     b, f = C.c_size_t(0), C.c_double(0)

@@ -79,10 +79,72 @@ def test_unet_extra_input_layers_are_ignored():
     assert np.abs(got - want).max() < 2e-3 * np.abs(want).max()
 
 
-def test_unet_refuses_autograd_and_cpu_tensors():
+def test_unet_refuses_cpu_tensors():
     net = _net([16, 32], 2, seed=1)
     inputs = _pyramid(32, 32, 2, 4, batch=1, seed=2)
-    with pytest.raises(NotImplementedError):
-        net.forward([t.cuda() for t in inputs])
     with torch.no_grad(), pytest.raises(RuntimeError):
         net.forward(inputs)
+
+
+# Gradients: fp16 operands in every GEMM of the backward as well (pre-activation gradients, block-input gradients),
+# fp32 accumulation; compared with torch autograd through the restatement that rounds where the forward rounds.
+# Bar: 2e-2 of the largest magnitude of each gradient tensor.
+GRAD_TOL = 2e-2
+
+
+@pytest.mark.parametrize("filters,levels,w,h,batch", [
+    ([16, 32, 64, 64], 4, 96, 72, 1),      # the benchmark's channel plan
+    ([32, 32, 32, 32, 32], 5, 100, 60, 2),  # shipped filters, odd sizes, two images
+    ([16, 24], 2, 37, 29, 1),               # partial tiles
+])
+def test_unet_backward_matches_torch_autograd(filters, levels, w, h, batch):
+    import copy
+    from tests.ref_unet import unet_forward
+    net = _net(filters, levels, seed=20 + levels)
+    ref = copy.deepcopy(net)
+    inputs = _pyramid(w, h, levels, 4, batch=batch, seed=30 + levels)
+    g = torch.Generator().manual_seed(7)
+    upstream = torch.randn((batch, 3, h, w), generator=g) * 1e-3
+
+    ins_ref = [t.clone().requires_grad_(True) for t in inputs]
+    (unet_forward(ref, ins_ref, half_rounding=True) * upstream).sum().backward()
+
+    net = net.cuda()
+    ins = [t.cuda().requires_grad_(True) for t in inputs]
+    out = net.forward(ins)
+    (out * upstream.cuda()).sum().backward()
+
+    def check(name, got, want):
+        got, want = got.detach().cpu().numpy(), want.detach().numpy()
+        scale = np.abs(want).max()
+        err = np.abs(got - want).max()
+        assert err < GRAD_TOL * scale, f"{name}: {err / scale:.3e}"
+
+    for i in range(levels):
+        check(f"d inputs[{i}]", ins[i].grad, ins_ref[i].grad)
+    for (n1, p1), (n2, p2) in zip(net.named_parameters(), ref.named_parameters()):
+        assert n1 == n2
+        check(n1, p1.grad, p2.grad)
+
+
+def test_unet_backward_small_gradients_survive_fp16():
+    """dL/doutput of a mean loss over a full-HD image is ~1e-7, below fp16's smallest normal number: the scale the
+    gradients are carried with must keep them."""
+    import copy
+    from tests.ref_unet import unet_forward
+    net = _net([16, 32], 2, seed=3)
+    ref = copy.deepcopy(net)
+    inputs = _pyramid(64, 48, 2, 4, batch=1, seed=4)
+    upstream = torch.full((1, 3, 48, 64), 1.0 / 6_220_800)
+    ins_ref = [t.clone().requires_grad_(True) for t in inputs]
+    # the unrounded fp32 network: torch's own fp16 casts would flush these gradients in the restatement itself
+    (unet_forward(ref, ins_ref, half_rounding=False) * upstream).sum().backward()
+    net = net.cuda()
+    ins = [t.cuda().requires_grad_(True) for t in inputs]
+    (net.forward(ins) * upstream.cuda()).sum().backward()
+    for a, b in zip(ins, ins_ref):
+        want = b.grad.numpy()
+        assert np.abs(want).max() < 1e-6
+        assert np.abs(a.grad.cpu().numpy() - want).max() < 3e-2 * np.abs(want).max()
+    want = ref.up1.feature_transform.weight.grad.numpy()
+    assert np.abs(net.up1.feature_transform.weight.grad.cpu().numpy() - want).max() < 3e-2 * np.abs(want).max()

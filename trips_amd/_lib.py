@@ -18,7 +18,8 @@ SYMBOLS = [
     "trips_adam_step_fused", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
 ]
 # every symbol include/trips_unet.h declares
-UNET_SYMBOLS = ["trips_unet_workspace_size", "trips_unet_forward", "trips_unet_flops"]
+UNET_SYMBOLS = ["trips_unet_workspace_size", "trips_unet_saved_size", "trips_unet_backward_workspace_size",
+                "trips_unet_forward", "trips_unet_backward", "trips_unet_flops"]
 
 
 class TripsError(RuntimeError):
@@ -59,8 +60,13 @@ def load():
     lib.trips_apply_tangent.argtypes = [vp, vp, vp, i32, vp]
     lib.trips_unet_workspace_size.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_size_t)]
     lib.trips_unet_flops.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_double)]
+    lib.trips_unet_saved_size.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_size_t)]
+    lib.trips_unet_backward_workspace_size.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_size_t)]
     lib.trips_unet_forward.argtypes = [vp, C.POINTER(abi.TripsUnetDesc), C.POINTER(abi.TripsUnetWeights),
-                                       C.POINTER(vp), vp, vp, C.c_size_t, vp]
+                                       C.POINTER(vp), vp, vp, vp, C.c_size_t, vp]
+    lib.trips_unet_backward.argtypes = [vp, C.POINTER(abi.TripsUnetDesc), C.POINTER(abi.TripsUnetWeights),
+                                        C.POINTER(vp), vp, vp, C.c_float, C.POINTER(abi.TripsUnetGrads), vp,
+                                        C.c_size_t, vp]
     lib.trips_profile_enable.argtypes = [vp, i32]
     lib.trips_profile_read.argtypes = [vp, C.POINTER(i32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
                                        C.POINTER(i32)]

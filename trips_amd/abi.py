@@ -143,6 +143,18 @@ class TripsUnetWeights(C.Structure):
     ]
 
 
+class TripsUnetGrads(C.Structure):
+    _fields_ = [
+        ("feature_weight", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("feature_bias", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("mask_weight", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("mask_bias", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+        ("final_weight", C.c_void_p),
+        ("final_bias", C.c_void_p),
+        ("inputs", C.c_void_p * TRIPS_UNET_MAX_LEVELS),
+    ]
+
+
 def make_unet_desc(filters, level_sizes, num_input_channels=4, num_output_channels=3, batch=1):
     """level_sizes: [(w, h)] of the pyramid levels the net consumes, finest first."""
     d = TripsUnetDesc()

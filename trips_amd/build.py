@@ -7,7 +7,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtrips_splat.so")
-SOURCES = ["trips_splat_abi.hip", "splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "unet_forward.hip"]
+SOURCES = ["trips_splat_abi.hip", "splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "unet_forward.hip",
+           "unet_backward.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
     # packed FP32 instructions are kept out of the generated code on purpose

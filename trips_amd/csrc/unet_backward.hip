@@ -1,0 +1,798 @@
+// Backward of the decoder-only gated-convolution U-Net on the gfx950 matrix cores: what libtorch's autograd does
+// for MultiScaleUnet2dDecOnlySmallFixedImpl::forward in the reference (src/lib/models/Networks.h:1139-1191, blocks
+// at :751-787 and :999-1098), as hand-written kernels over the state the training forward saved.
+//
+//   final_backward_kernel     1x1 output convolution: gradient of x_0, split into dL/d in[0] and, through the gate,
+//                             the gradient of the finest block's pre-activations
+//   final_weight_grad_kernel  its weight and bias gradients
+//   conv_bwd_data_kernel      gradient of a block's input: the forward's implicit GEMM with flipped, transposed
+//                             weights (M = 256 pixels, N = input channels, K = 9 taps x pre-activations)
+//   up2_adjoint_gate_kernel   adjoint of the bilinear 2x upsampling (a gather over <= 4 x 4 finer pixels), then
+//                             dL/d in[i+1] and the gate of the coarser block
+//   conv_bwd_weight_kernel    weight gradients: GEMM with the pixels as the reduction dimension. Both operands are
+//                             needed pixel-contiguous, so the tiles are written to LDS transposed ([channel][pixel]);
+//                             persistent workgroups keep their partial sums in registers over many tiles
+//   bias_grad_kernel, reduce_weight_grad_kernel
+//
+// Intermediate gradients are fp16 and carried multiplied by grad_scale; every fp32 result is divided by it again.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "unet_common.h"
+
+namespace trips
+{
+typedef half8 half8_unaligned __attribute__((aligned(2)));
+
+// d(elu(f) * sigmoid(m)) for an incoming gradient da
+__device__ __forceinline__ void gate_backward(float da, float f, float m, float& df, float& dm)
+{
+    const float s  = 1.f / (1.f + __expf(-m));
+    const float ex = __expf(f);
+    const float e  = f > 0.f ? f : ex - 1.f;
+    const float de = f > 0.f ? 1.f : ex;
+    df             = da * s * de;
+    dm             = da * e * s * (1.f - s);
+}
+
+// wt[tap'][c][n] = W[n][c][8 - tap']: the data gradient is a correlation of the pre-activation gradient with the
+// spatially flipped kernel, input and output channels exchanged
+__global__ __launch_bounds__(256) void pack_conv_weights_T_kernel(const float* __restrict__ wf, const float* __restrict__ wm,
+                                                                  int cout, int cin_real, int cin_pad, int npad,
+                                                                  _Float16* __restrict__ wt)
+{
+    const int total = 9 * cin_pad * npad;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256)
+    {
+        const int n = i % npad, c = (i / npad) % cin_pad, tap = i / (npad * cin_pad);
+        const int half = npad / 2;
+        const int o    = n < half ? n : n - half;
+        float v        = 0.f;
+        if (o < cout && c < cin_real) v = (n < half ? wf : wm)[((size_t)o * cin_real + c) * 9 + (8 - tap)];
+        wt[i] = _Float16(v);
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ p, float v, int n)
+{
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) p[i] = v;
+}
+
+struct FinalBwdParams
+{
+    int H, W, c_feat, cact, cact_store, cout, npad;
+    float scale;
+    const float* feat;        // [C][H][W]
+    const _Float16* act;      // [H][W][cact_store]
+    const _Float16* pre;      // [H][W][npad]
+    const float* weight;      // [cout][c_feat + cact]
+    const float* d_out;       // [cout][H][W]
+    float* d_feat;            // [C][H][W], written
+    _Float16* dpre;           // [H][W][npad], written
+    float* d_weight;          // [cout][c_feat + cact], accumulated (zeroed by the caller)
+    float* d_bias;            // [cout]
+};
+
+__global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParams p)
+{
+    __shared__ float s_w[4 * 80];
+    const int cin = p.c_feat + p.cact;
+    for (int i = threadIdx.x; i < p.cout * cin; i += 256) s_w[i] = float(_Float16(p.weight[i]));
+    __syncthreads();
+    const size_t plane = (size_t)p.H * p.W;
+    const int half     = p.npad / 2;
+    for (size_t pix = (size_t)blockIdx.x * 256 + threadIdx.x; pix < plane; pix += (size_t)gridDim.x * 256)
+    {
+        float g[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < p.cout; ++k) g[k] = p.d_out[k * plane + pix];
+        for (int c = 0; c < p.c_feat; ++c)
+        {
+            float d = 0.f;
+            for (int k = 0; k < p.cout; ++k) d += s_w[k * cin + c] * g[k];
+            p.d_feat[c * plane + pix] = d;
+        }
+        const _Float16* pr = p.pre + pix * p.npad;
+        _Float16* dp       = p.dpre + pix * p.npad;
+        for (int j0 = 0; j0 < half; j0 += 8)
+        {
+            const half8 f8 = *reinterpret_cast<const half8*>(pr + j0);
+            const half8 m8 = *reinterpret_cast<const half8*>(pr + half + j0);
+            half8 of, om;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+            {
+                const int j = j0 + i;
+                float da    = 0.f;
+                if (j < p.cact)
+                {
+                    for (int k = 0; k < p.cout; ++k) da += s_w[k * cin + p.c_feat + j] * g[k];
+                    da *= p.scale;
+                }
+                float df, dm;
+                gate_backward(da, float(f8[i]), float(m8[i]), df, dm);
+                of[i] = _Float16(df);
+                om[i] = _Float16(dm);
+            }
+            *reinterpret_cast<half8*>(dp + j0)        = of;
+            *reinterpret_cast<half8*>(dp + half + j0) = om;
+        }
+    }
+}
+
+// thread t <-> one (output k, input c) pair, or a bias; a block sums a chunk of pixels and adds it once
+constexpr int kFinalChunk = 2048;
+__global__ __launch_bounds__(256) void final_weight_grad_kernel(const FinalBwdParams p)
+{
+    const int cin      = p.c_feat + p.cact;
+    const size_t plane = (size_t)p.H * p.W;
+    const size_t p0 = (size_t)blockIdx.x * kFinalChunk, p1 = std::min(plane, p0 + kFinalChunk);
+    for (int t = threadIdx.x; t < p.cout * cin + p.cout; t += 256)
+    {
+        float sum = 0.f;
+        if (t < p.cout * cin)
+        {
+            const int k = t / cin, c = t - k * cin;
+            const float* g = p.d_out + k * plane;
+            if (c < p.c_feat)
+            {
+                const float* x = p.feat + c * plane;
+                for (size_t pix = p0; pix < p1; ++pix) sum += g[pix] * float(_Float16(x[pix]));
+            }
+            else
+            {
+                const _Float16* x = p.act + (c - p.c_feat);
+                for (size_t pix = p0; pix < p1; ++pix) sum += g[pix] * float(x[pix * p.cact_store]);
+            }
+            atomicAdd(p.d_weight + t, sum);
+        }
+        else
+        {
+            const float* g = p.d_out + (size_t)(t - p.cout * cin) * plane;
+            for (size_t pix = p0; pix < p1; ++pix) sum += g[pix];
+            atomicAdd(p.d_bias + (t - p.cout * cin), sum);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+struct BwdDataParams
+{
+    int H, W, c_feat;
+    float scale_inv;
+    const _Float16* dpre;  // [H][W][KC]
+    const _Float16* wt;    // [9][NN][KC]
+    float* d_feat;         // [C][H][W], accumulated
+    _Float16* d_in;        // [H][W][NN] or nullptr (start block: nothing below)
+};
+
+template <int KC, int NN>
+__global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams p)
+{
+    constexpr int ROW    = KC + kLdsChanPad;
+    constexpr int GROUPS = KC / 8;
+    constexpr int NB     = NN / 16;
+    extern __shared__ _Float16 smem[];
+    _Float16* s_patch = smem;
+    const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
+    for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
+    {
+        const int g = item % GROUPS, pp = item / GROUPS;
+        const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
+        const int y = y0 + py - 1, x = x0 + px - 1;
+        half8 v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = _Float16(0.f);
+        if (y >= 0 && y < p.H && x >= 0 && x < p.W) v = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * KC + 8 * g);
+        *reinterpret_cast<half8*>(s_patch + (size_t)pp * ROW + 8 * g) = v;
+    }
+    __syncthreads();
+    floatx4 acc[4][NB];
+    conv_taps_mfma<KC, NN>(s_patch, p.wt, acc);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lrow = lane & 15;
+    const size_t plane = (size_t)p.H * p.W;
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+    {
+        const int y = y0 + 2 * wave + (m >> 1);
+#pragma unroll
+        for (int n = 0; n < NB; ++n)
+        {
+            const int c = 16 * n + lrow;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                const int x = x0 + (m & 1) * 16 + (lane >> 4) * 4 + i;
+                if (y >= p.H || x >= p.W) continue;
+                const float v = acc[m][n][i];
+                if (p.d_in) p.d_in[((size_t)y * p.W + x) * NN + c] = _Float16(v);
+                if (c < p.c_feat) p.d_feat[c * plane + (size_t)y * p.W + x] += v * p.scale_inv;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+struct UpAdjointParams
+{
+    int H, W;      // finer level, whose block input gradient is given
+    int Hb, Wb;    // this (coarser) level
+    int cin_fine;  // halves per pixel of d_in
+    int c_feat, cout, npad;
+    float scale_inv;
+    const _Float16* d_in;  // [H][W][cin_fine]: position k = channel k of cat(in, up2(x))
+    const _Float16* pre;   // [Hb][Wb][npad]
+    float* d_feat;         // [C][Hb][Wb], written
+    _Float16* dpre;        // [Hb][Wb][npad], written
+};
+
+// weight with which finer row / column `dst` reads coarser row / column `src`
+__device__ __forceinline__ float up2_weight(int dst, int fine_size, int src, int coarse_size)
+{
+    if (dst < 0 || dst >= fine_size) return 0.f;
+    int i0, i1;
+    float l;
+    up2_source(dst, coarse_size, i0, i1, l);
+    return (i0 == src ? 1.f - l : 0.f) + (i1 == src ? l : 0.f);
+}
+
+__global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointParams p)
+{
+    const int half   = p.npad / 2;
+    const int groups = 1 + half / 8;  // group 0: the image below; group q: 8 block outputs
+    const size_t pb  = (size_t)p.Hb * p.Wb;
+    for (size_t item = (size_t)blockIdx.x * 256 + threadIdx.x; item < pb * groups; item += (size_t)gridDim.x * 256)
+    {
+        const int q     = (int)(item % groups);
+        const size_t bp = item / groups;
+        const int Y = (int)(bp / p.Wb), X = (int)(bp - (size_t)Y * p.Wb);
+        float a[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = 0.f;
+        const int pos = 8 * q;  // position in the finer block's input: [0, C) its own image, then x of this level
+        if (pos < p.cin_fine)
+        {
+            float wy[4], wx[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                wy[k] = up2_weight(2 * Y - 1 + k, p.H, Y, p.Hb);
+                wx[k] = up2_weight(2 * X - 1 + k, p.W, X, p.Wb);
+            }
+#pragma unroll
+            for (int ky = 0; ky < 4; ++ky)
+            {
+                if (wy[ky] == 0.f) continue;
+                const int y = 2 * Y - 1 + ky;
+#pragma unroll
+                for (int kx = 0; kx < 4; ++kx)
+                {
+                    if (wx[kx] == 0.f) continue;
+                    const int x   = 2 * X - 1 + kx;
+                    const half8 v = *reinterpret_cast<const half8*>(p.d_in + ((size_t)y * p.W + x) * p.cin_fine + pos);
+                    const float w = wy[ky] * wx[kx];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) a[i] += w * float(v[i]);
+                }
+            }
+        }
+        if (q == 0)
+        {
+            // positions [C, 2C) are this level's image (C = 4: a[4..7])
+            for (int c = 0; c < p.c_feat; ++c) p.d_feat[c * pb + bp] = a[p.c_feat + c] * p.scale_inv;
+        }
+        else
+        {
+            const int ch0       = 8 * (q - 1);
+            const _Float16* pr  = p.pre + bp * p.npad;
+            _Float16* dp        = p.dpre + bp * p.npad;
+            const half8 f8 = *reinterpret_cast<const half8*>(pr + ch0);
+            const half8 m8 = *reinterpret_cast<const half8*>(pr + half + ch0);
+            half8 of, om;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+            {
+                float df, dm;
+                gate_backward(ch0 + i < p.cout ? a[i] : 0.f, float(f8[i]), float(m8[i]), df, dm);
+                of[i] = _Float16(df);
+                om[i] = _Float16(dm);
+            }
+            *reinterpret_cast<half8*>(dp + ch0)        = of;
+            *reinterpret_cast<half8*>(dp + half + ch0) = om;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+struct BiasGradParams
+{
+    size_t pixels;
+    int npad, cout;
+    float scale_inv;
+    const _Float16* dpre;  // [pixels][npad]
+    float* d_bias_f;       // [cout], accumulated (zeroed by the caller)
+    float* d_bias_m;
+};
+
+constexpr int kBiasChunk = 8192;
+__global__ __launch_bounds__(256) void bias_grad_kernel(const BiasGradParams p)
+{
+    __shared__ float s_sum[128];
+    if (threadIdx.x < 128) s_sum[threadIdx.x] = 0.f;
+    __syncthreads();
+    const int groups = p.npad / 8;
+    const int lanes  = 256 / groups;  // pixels in flight per block
+    const int g = threadIdx.x % groups, sub = threadIdx.x / groups;
+    if (sub < lanes)
+    {
+        float a[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = 0.f;
+        const size_t p0 = (size_t)blockIdx.x * kBiasChunk, p1 = std::min(p.pixels, p0 + kBiasChunk);
+        for (size_t pix = p0 + sub; pix < p1; pix += lanes)
+        {
+            const half8 v = *reinterpret_cast<const half8*>(p.dpre + pix * p.npad + 8 * g);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[i] += float(v[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) atomicAdd(&s_sum[8 * g + i], a[i]);
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < p.npad)
+    {
+        const int n = threadIdx.x, half = p.npad / 2;
+        const int o = n < half ? n : n - half;
+        if (o < p.cout)
+        {
+            float* dst = n < half ? p.d_bias_f : p.d_bias_m;
+            if (dst) atomicAdd(dst + o, s_sum[n] * p.scale_inv);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+struct BwdWeightParams
+{
+    int H, W, Hb, Wb;
+    int c_feat, cb_store;
+    int tiles_x, tiles;
+    const float* feat;
+    const float* feat_below;
+    const _Float16* act_below;
+    const _Float16* dpre;  // [H][W][NPAD]
+    float* part;           // [gridDim.x][9][NPAD][CIN]
+};
+
+constexpr int kXtRow   = 40;                          // halves per patch row in the transposed input tile
+constexpr int kXtChan  = kConvPatchH * kXtRow + 8;    // halves per channel (padding spreads the 16 channels of a read over the banks)
+constexpr int kDtChan  = kConvTileH * kConvTileW + 8;  // halves per pre-activation channel in the transposed gradient tile
+
+template <int CIN, int NPAD>
+__global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightParams p)
+{
+    constexpr int ROW    = CIN + kLdsChanPad;
+    constexpr int GROUPS = CIN / 8;
+    constexpr int NB     = NPAD / 16;
+    constexpr int CB     = CIN / 16;
+    constexpr int UNITS  = 9 * NB;            // (tap, 16 pre-activation channels) pairs, dealt round-robin to the 4 wavefronts
+    constexpr int U      = (UNITS + 3) / 4;
+    extern __shared__ _Float16 smem[];
+    _Float16* s_below = smem;                                  // [kBelowH * kBelowW][ROW]
+    _Float16* s_xt    = s_below + kBelowH * kBelowW * ROW;     // [CIN][kXtChan]
+    _Float16* s_dt    = s_xt + CIN * kXtChan;                  // [NPAD][kDtChan]
+    const bool has_below = p.Hb > 0;
+    const int C          = p.c_feat;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lrow = lane & 15, lk = (lane >> 4) * 8;
+
+    floatx4 acc[U][CB];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int c = 0; c < CB; ++c) acc[u][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // channels that no stage writes stay zero for every tile
+    for (int i = threadIdx.x; i < CIN * kXtChan; i += 256) s_xt[i] = _Float16(0.f);
+
+    for (int tile = blockIdx.x; tile < p.tiles; tile += gridDim.x)
+    {
+        const int ty = tile / p.tiles_x, tx = tile - ty * p.tiles_x;
+        const int x0 = tx * kConvTileW, y0 = ty * kConvTileH;
+        const int by0 = y0 / 2 - 1, bx0 = x0 / 2 - 1;
+        __syncthreads();  // the previous tile's operands have been consumed (and the zero fill is done)
+        // ---- stage 1: this level's image (transposed), the patch of the level below, the gradient tile (transposed) ----
+        {
+            const size_t plane = (size_t)p.H * p.W;
+            for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW; item += 256)
+            {
+                const int py = item / kConvPatchW, px = item - py * kConvPatchW;
+                const int y = y0 + py - 1, x = x0 + px - 1;
+                const bool in = y >= 0 && y < p.H && x >= 0 && x < p.W;
+                for (int c = 0; c < C; ++c)
+                    s_xt[c * kXtChan + py * kXtRow + px] = in ? _Float16(p.feat[c * plane + (size_t)y * p.W + x]) : _Float16(0.f);
+            }
+        }
+        if (has_below)
+        {
+            const size_t pb      = (size_t)p.Hb * p.Wb;
+            const int act_groups = p.cb_store / 8;
+            const int per_pixel  = 1 + act_groups;
+            for (int item = threadIdx.x; item < kBelowH * kBelowW * per_pixel; item += 256)
+            {
+                const int q = item % per_pixel, bp = item / per_pixel;
+                const int r = bp / kBelowW, c0 = bp - r * kBelowW;
+                const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
+                _Float16* row = s_below + (size_t)bp * ROW;
+                if (q == 0)
+                {
+                    for (int c = 0; c < C; ++c) row[C + c] = _Float16(p.feat_below[c * pb + (size_t)yy * p.Wb + xx]);
+                    for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
+                }
+                else
+                {
+                    *reinterpret_cast<half8*>(row + 2 * C + 8 * (q - 1)) =
+                        *reinterpret_cast<const half8*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+                }
+            }
+        }
+        for (int item = threadIdx.x; item < kConvTileH * kConvTileW * (NPAD / 8); item += 256)
+        {
+            const int tp = item % (kConvTileH * kConvTileW), g = item / (kConvTileH * kConvTileW);
+            const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
+            half8 v;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = _Float16(0.f);
+            if (y < p.H && x < p.W) v = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * NPAD + 8 * g);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s_dt[(8 * g + i) * kDtChan + tp] = v[i];
+        }
+        if (has_below)
+        {
+            __syncthreads();
+            // ---- stage 2: bilinear 2x upsampling from the below patch, written transposed ----
+            for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
+            {
+                const int pp = item % (kConvPatchH * kConvPatchW), g = item / (kConvPatchH * kConvPatchW);
+                const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
+                const int y = y0 + py - 1, x = x0 + px - 1;
+                float v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = 0.f;
+                if (y >= 0 && y < p.H && x >= 0 && x < p.W)
+                {
+                    int ya, yb, xa, xb;
+                    float ly, lx;
+                    up2_source(y, p.Hb, ya, yb, ly);
+                    up2_source(x, p.Wb, xa, xb, lx);
+                    const float w00 = (1.f - ly) * (1.f - lx), w01 = (1.f - ly) * lx, w10 = ly * (1.f - lx), w11 = ly * lx;
+                    const half8 a = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
+                    const half8 b = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
+                    const half8 c = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
+                    const half8 d = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = w00 * float(a[i]) + w01 * float(b[i]) + w10 * float(c[i]) + w11 * float(d[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (8 * g + i >= C) s_xt[(8 * g + i) * kXtChan + py * kXtRow + px] = _Float16(v[i]);
+            }
+        }
+        __syncthreads();
+        // ---- dW[tap][n][c] += sum over the tile's pixels of dpre[pixel][n] * x[pixel + tap][c] ----
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu)
+        {
+            const int u = wave + 4 * uu;
+            if (u < UNITS)
+            {
+                const int tap = u / NB, nb = u - tap * NB;
+                const int dy = tap / 3, dx = tap - dy * 3;
+#pragma unroll
+                for (int r = 0; r < kConvTileH; ++r)
+                {
+                    const half8 a = *reinterpret_cast<const half8*>(s_dt + (nb * 16 + lrow) * kDtChan + r * kConvTileW + lk);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+                    {
+                        const half8 b = *reinterpret_cast<const half8_unaligned*>(s_xt + (cb * 16 + lrow) * kXtChan + (r + dy) * kXtRow + lk + dx);
+                        acc[uu][cb]   = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[uu][cb], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    float* part = p.part + (size_t)blockIdx.x * 9 * NPAD * CIN;
+#pragma unroll
+    for (int uu = 0; uu < U; ++uu)
+    {
+        const int u = wave + 4 * uu;
+        if (u < UNITS)
+        {
+            const int tap = u / NB, nb = u - tap * NB;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    part[((size_t)tap * NPAD + nb * 16 + (lane >> 4) * 4 + i) * CIN + cb * 16 + lrow] = acc[uu][cb][i];
+        }
+    }
+}
+
+// sums the partial weight gradients of all workgroups (and images) into the reference's [Cout][Cin][3][3] layout
+__global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const float* __restrict__ part, int groups, int cout,
+                                                                 int cin_real, int cin_pad, int npad, float scale_inv,
+                                                                 float* __restrict__ d_wf, float* __restrict__ d_wm)
+{
+    const int total = 9 * npad * cin_pad;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256)
+    {
+        const int c = i % cin_pad, n = (i / cin_pad) % npad, tap = i / (cin_pad * npad);
+        const int half = npad / 2;
+        const int o    = n < half ? n : n - half;
+        if (o >= cout || c >= cin_real) continue;
+        float* dst = n < half ? d_wf : d_wm;
+        if (!dst) continue;
+        float s = 0.f;
+        for (int g = 0; g < groups; ++g) s += part[(size_t)g * total + i];
+        dst[((size_t)o * cin_real + c) * 9 + tap] = s * scale_inv;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+namespace
+{
+template <int KC, int NN>
+hipError_t launch_bwd_data(const BwdDataParams& p, hipStream_t stream)
+{
+    const size_t lds = (size_t)kConvPatchH * kConvPatchW * (KC + kLdsChanPad) * sizeof(_Float16);  // up to 92 KB
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    dim3 grid((p.W + kConvTileW - 1) / kConvTileW, (p.H + kConvTileH - 1) / kConvTileH);
+    hipLaunchKernelGGL((conv_bwd_data_kernel<KC, NN>), grid, dim3(256), lds, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipStream_t stream)
+{
+#define TRIPS_BD(KC_, NN_) \
+    if (npad == KC_ && cin_pad == NN_) return launch_bwd_data<KC_, NN_>(p, stream);
+    TRIPS_BD(32, 32) TRIPS_BD(64, 32) TRIPS_BD(96, 32) TRIPS_BD(128, 32)
+    TRIPS_BD(32, 64) TRIPS_BD(64, 64) TRIPS_BD(96, 64) TRIPS_BD(128, 64)
+#undef TRIPS_BD
+    return hipErrorInvalidValue;
+}
+
+template <int CIN, int NPAD>
+hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
+{
+    const size_t lds = ((size_t)kBelowH * kBelowW * (CIN + kLdsChanPad) + (size_t)CIN * kXtChan + (size_t)NPAD * kDtChan) *
+                       sizeof(_Float16);  // up to 133 KB
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD>), dim3(groups), dim3(256), lds, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t dispatch_bwd_weight(const BwdWeightParams& p, int cin_pad, int npad, int groups, hipStream_t stream)
+{
+#define TRIPS_BW(CIN_, NPAD_) \
+    if (cin_pad == CIN_ && npad == NPAD_) return launch_bwd_weight<CIN_, NPAD_>(p, groups, stream);
+    TRIPS_BW(32, 32) TRIPS_BW(32, 64) TRIPS_BW(32, 96) TRIPS_BW(32, 128)
+    TRIPS_BW(64, 32) TRIPS_BW(64, 64) TRIPS_BW(64, 96) TRIPS_BW(64, 128)
+#undef TRIPS_BW
+    return hipErrorInvalidValue;
+}
+}  // namespace
+}  // namespace trips
+
+using namespace trips;
+
+extern "C" {
+
+int trips_unet_backward_workspace_size(const TripsUnetDesc* desc, size_t* bytes)
+{
+    if (int e = check_unet_desc(desc)) return e;
+    if (!bytes) return set_error(TRIPS_ERR_INVALID_ARG, "bytes is NULL");
+    *bytes = make_plan(*desc).backward_bytes;
+    return TRIPS_OK;
+}
+
+int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
+                        const float* const inputs[TRIPS_UNET_MAX_LEVELS], const void* saved, const float* d_output,
+                        float grad_scale, const TripsUnetGrads* grads, void* workspace, size_t workspace_bytes,
+                        void* stream_)
+{
+    if (!ctx) return set_error(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (int e = check_unet_desc(desc)) return e;
+    if (!weights || !inputs || !saved || !d_output || !grads || !workspace) return set_error(TRIPS_ERR_INVALID_ARG, "NULL argument");
+    const TripsUnetDesc& d = *desc;
+    const int C = d.num_input_channels, L = d.num_levels;
+    if (C != 4) return set_error(TRIPS_ERR_UNSUPPORTED, "the backward is built for num_input_channels = 4 (got %d)", C);
+    if (!(grad_scale > 0.f) || !std::isfinite(grad_scale)) return set_error(TRIPS_ERR_INVALID_ARG, "grad_scale must be positive");
+    for (int i = 0; i < L; ++i)
+    {
+        if (!inputs[i]) return set_error(TRIPS_ERR_INVALID_ARG, "inputs[%d] is NULL", i);
+        if (!grads->inputs[i]) return set_error(TRIPS_ERR_INVALID_ARG, "grads->inputs[%d] is NULL", i);
+        if (!weights->feature_weight[i] || !weights->mask_weight[i])
+            return set_error(TRIPS_ERR_INVALID_ARG, "weights of block %d are NULL", i);
+    }
+    if (!weights->final_weight) return set_error(TRIPS_ERR_INVALID_ARG, "final weights are NULL");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255) || (reinterpret_cast<uintptr_t>(saved) & 255))
+        return set_error(TRIPS_ERR_INVALID_ARG, "workspace / saved must be 256-byte aligned");
+    const NetPlan np = make_plan(d);
+    if (workspace_bytes < np.backward_bytes)
+        return set_error(TRIPS_ERR_WORKSPACE_SMALL, "workspace has %zu bytes, %zu needed", workspace_bytes, np.backward_bytes);
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    char* ws           = reinterpret_cast<char*>(workspace);
+    const char* sv     = reinterpret_cast<const char*>(saved);
+    Profiler* prof     = ctx->prof.enabled ? &ctx->prof : nullptr;
+    const float scale_inv = 1.f / grad_scale;
+    const int K           = d.num_output_channels;
+
+    auto act_ptr = [&](int level, int b)
+    {
+        const LevelPlan& l = np.lv[level];
+        return reinterpret_cast<const _Float16*>(sv + l.saved_act_off) + (size_t)b * l.H * l.W * l.cout_store;
+    };
+    auto pre_ptr = [&](int level, int b)
+    {
+        const LevelPlan& l = np.lv[level];
+        return reinterpret_cast<const _Float16*>(sv + l.saved_pre_off) + (size_t)b * l.H * l.W * l.npad;
+    };
+    auto dpre_ptr = [&](int level, int b)
+    {
+        const LevelPlan& l = np.lv[level];
+        return reinterpret_cast<_Float16*>(ws + l.dpre_off) + (size_t)b * l.H * l.W * l.npad;
+    };
+    auto din_ptr = [&](int level, int b)
+    {
+        const LevelPlan& l = np.lv[level];
+        return reinterpret_cast<_Float16*>(ws + l.din_off) + (size_t)b * l.H * l.W * l.cin_pad;
+    };
+    auto fill = [&](float* p, int n)
+    {
+        if (p && n > 0) hipLaunchKernelGGL(fill_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, p, 0.f, n);
+    };
+
+    {
+        ProfScope ps(prof, "unet_bwd_prepare", stream);
+        for (int i = 0; i < L; ++i)
+        {
+            const LevelPlan& lv = np.lv[i];
+            const int total     = 9 * lv.npad * lv.cin_pad;
+            hipLaunchKernelGGL(pack_conv_weights_T_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
+                               weights->feature_weight[i], weights->mask_weight[i], lv.cout, lv.cin_real, lv.cin_pad, lv.npad,
+                               reinterpret_cast<_Float16*>(ws + lv.wt_off));
+            fill(grads->feature_bias[i], lv.cout);
+            fill(grads->mask_bias[i], lv.cout);
+        }
+        fill(grads->final_weight, K * (C + np.lv[0].cout));
+        fill(grads->final_bias, K);
+    }
+    {
+        ProfScope ps(prof, "unet_bwd_final", stream);
+        const LevelPlan& lv = np.lv[0];
+        const size_t plane  = (size_t)lv.H * lv.W;
+        // the weight-gradient kernel needs somewhere to add to even when the caller does not want the result
+        for (int b = 0; b < d.batch; ++b)
+        {
+            FinalBwdParams p;
+            std::memset(&p, 0, sizeof(p));
+            p.H = lv.H, p.W = lv.W, p.c_feat = C, p.cact = lv.cout, p.cact_store = lv.cout_store, p.cout = K, p.npad = lv.npad;
+            p.scale    = grad_scale;
+            p.feat     = inputs[0] + (size_t)b * C * plane;
+            p.act      = act_ptr(0, b);
+            p.pre      = pre_ptr(0, b);
+            p.weight   = weights->final_weight;
+            p.d_out    = d_output + (size_t)b * K * plane;
+            p.d_feat   = grads->inputs[0] + (size_t)b * C * plane;
+            p.dpre     = dpre_ptr(0, b);
+            p.d_weight = grads->final_weight;
+            p.d_bias   = grads->final_bias;
+            const int blocks = (int)std::min<size_t>((plane + 255) / 256, 65535);
+            hipLaunchKernelGGL(final_backward_kernel, dim3(blocks), dim3(256), 0, stream, p);
+            if (p.d_weight && p.d_bias)
+            {
+                const int chunks = (int)((plane + kFinalChunk - 1) / kFinalChunk);
+                hipLaunchKernelGGL(final_weight_grad_kernel, dim3(chunks), dim3(256), 0, stream, p);
+            }
+        }
+    }
+    static const char* const kDataNames[TRIPS_UNET_MAX_LEVELS]   = {"unet_bwd_data_l0", "unet_bwd_data_l1", "unet_bwd_data_l2", "unet_bwd_data_l3",
+                                                                    "unet_bwd_data_l4", "unet_bwd_data_l5", "unet_bwd_data_l6", "unet_bwd_data_l7"};
+    static const char* const kWeightNames[TRIPS_UNET_MAX_LEVELS] = {"unet_bwd_weight_l0", "unet_bwd_weight_l1", "unet_bwd_weight_l2", "unet_bwd_weight_l3",
+                                                                    "unet_bwd_weight_l4", "unet_bwd_weight_l5", "unet_bwd_weight_l6", "unet_bwd_weight_l7"};
+    for (int i = 0; i < L; ++i)
+    {
+        const LevelPlan& lv = np.lv[i];
+        const size_t plane  = (size_t)lv.H * lv.W;
+        const bool below    = i < L - 1;
+        {
+            ProfScope ps(prof, kWeightNames[i], stream);
+            for (int b = 0; b < d.batch; ++b)
+            {
+                BiasGradParams bp;
+                bp.pixels    = plane;
+                bp.npad      = lv.npad;
+                bp.cout      = lv.cout;
+                bp.scale_inv = scale_inv;
+                bp.dpre      = dpre_ptr(i, b);
+                bp.d_bias_f  = grads->feature_bias[i];
+                bp.d_bias_m  = grads->mask_bias[i];
+                if (bp.d_bias_f || bp.d_bias_m)
+                    hipLaunchKernelGGL(bias_grad_kernel, dim3((unsigned)((plane + kBiasChunk - 1) / kBiasChunk)), dim3(256), 0, stream, bp);
+
+                BwdWeightParams wp;
+                std::memset(&wp, 0, sizeof(wp));
+                wp.H = lv.H, wp.W = lv.W, wp.c_feat = C;
+                wp.tiles_x = (lv.W + kConvTileW - 1) / kConvTileW;
+                wp.tiles   = wp.tiles_x * ((lv.H + kConvTileH - 1) / kConvTileH);
+                wp.feat    = inputs[i] + (size_t)b * C * plane;
+                wp.dpre    = dpre_ptr(i, b);
+                wp.part    = reinterpret_cast<float*>(ws + lv.part_off) + (size_t)b * lv.groups * 9 * lv.npad * lv.cin_pad;
+                if (below)
+                {
+                    const LevelPlan& lb = np.lv[i + 1];
+                    wp.Hb = lb.H, wp.Wb = lb.W, wp.cb_store = lb.cout_store;
+                    wp.feat_below = inputs[i + 1] + (size_t)b * C * lb.H * lb.W;
+                    wp.act_below  = act_ptr(i + 1, b);
+                }
+                if (grads->feature_weight[i] || grads->mask_weight[i])
+                {
+                    hipError_t e = dispatch_bwd_weight(wp, lv.cin_pad, lv.npad, lv.groups, stream);
+                    if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "weight gradient launch (level %d): %s", i, hipGetErrorString(e));
+                }
+            }
+            if (grads->feature_weight[i] || grads->mask_weight[i])
+            {
+                const int total = 9 * lv.npad * lv.cin_pad;
+                hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
+                                   reinterpret_cast<const float*>(ws + lv.part_off), d.batch * lv.groups, lv.cout, lv.cin_real,
+                                   lv.cin_pad, lv.npad, scale_inv, grads->feature_weight[i], grads->mask_weight[i]);
+            }
+        }
+        {
+            ProfScope ps(prof, kDataNames[i], stream);
+            for (int b = 0; b < d.batch; ++b)
+            {
+                BwdDataParams dp;
+                dp.H = lv.H, dp.W = lv.W, dp.c_feat = C;
+                dp.scale_inv = scale_inv;
+                dp.dpre      = dpre_ptr(i, b);
+                dp.wt        = reinterpret_cast<const _Float16*>(ws + lv.wt_off);
+                dp.d_feat    = grads->inputs[i] + (size_t)b * C * plane;
+                dp.d_in      = below ? din_ptr(i, b) : nullptr;
+                hipError_t e = dispatch_bwd_data(dp, lv.npad, lv.cin_pad, stream);
+                if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "data gradient launch (level %d): %s", i, hipGetErrorString(e));
+                if (below)
+                {
+                    const LevelPlan& lb = np.lv[i + 1];
+                    UpAdjointParams up;
+                    up.H = lv.H, up.W = lv.W, up.Hb = lb.H, up.Wb = lb.W;
+                    up.cin_fine  = lv.cin_pad;
+                    up.c_feat    = C;
+                    up.cout      = lb.cout;
+                    up.npad      = lb.npad;
+                    up.scale_inv = scale_inv;
+                    up.d_in      = din_ptr(i, b);
+                    up.pre       = pre_ptr(i + 1, b);
+                    up.d_feat    = grads->inputs[i + 1] + (size_t)b * C * lb.H * lb.W;
+                    up.dpre      = dpre_ptr(i + 1, b);
+                    const size_t items = (size_t)lb.H * lb.W * (1 + lb.npad / 16);
+                    const int blocks   = (int)std::min<size_t>((items + 255) / 256, 1u << 20);
+                    hipLaunchKernelGGL(up2_adjoint_gate_kernel, dim3(blocks), dim3(256), 0, stream, up);
+                }
+            }
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "backward launch (level %d): %s", i, hipGetErrorString(e));
+    }
+    return TRIPS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,209 @@
+// Pieces shared by the forward and backward kernels of the reconstruction net (gfx950).
+#pragma once
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "../../include/trips_unet.h"
+#include "splat_internal.h"
+
+namespace trips
+{
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kConvTileH   = 8;
+constexpr int kConvTileW   = 32;
+constexpr int kConvPatchH  = kConvTileH + 2;
+constexpr int kConvPatchW  = kConvTileW + 2;
+constexpr int kBelowH      = kConvTileH / 2 + 2;  // rows / columns of the level below that an upsampled patch touches
+constexpr int kBelowW      = kConvTileW / 2 + 2;
+constexpr int kLdsChanPad  = 8;  // halves added to every LDS row so that 16 lanes reading 16 bytes hit 64 distinct banks
+
+// source row / column and weight of torch's bilinear upsampling with scale_factor 2, align_corners = false
+// (area_pixel_compute_source_index: src = max(0, (dst + 0.5) * 0.5 - 0.5))
+__device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i1, float& lambda)
+{
+    float src = (float(dst) + 0.5f) * 0.5f - 0.5f;
+    src       = src < 0.f ? 0.f : src;
+    i0        = (int)src;
+    i0        = i0 < in_size - 1 ? i0 : in_size - 1;
+    i1        = i0 + 1 < in_size ? i0 + 1 : in_size - 1;
+    lambda    = src - float(i0);
+}
+
+
+// The 9-tap implicit-GEMM core shared by the forward convolution and the data gradient: A operands are 16-byte
+// LDS reads from a (8+2) x (32+2) pixel patch with KIN channels innermost (row stride KIN + 8 halves), B operands
+// (packed weights [tap][NOUT][KIN], L2-resident) are loaded from memory directly, the next tap's fragments
+// requested before the current tap's MFMAs issue, so the tap loop has no barrier. A wavefront owns two rows of the
+// 8 x 32 output tile = four 16-pixel row blocks; acc[m][n] is the 16 x 16 block of pixels m, outputs 16n .. 16n+15.
+template <int KIN, int NOUT>
+__device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, const _Float16* __restrict__ wpack,
+                                               floatx4 (&acc)[4][NOUT / 16])
+{
+    constexpr int ROW = KIN + kLdsChanPad;
+    constexpr int NB  = NOUT / 16;
+    constexpr int KB  = KIN / 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lrow = lane & 15, lk = (lane >> 4) * 8;
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int n = 0; n < NB; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const _Float16* wlane = wpack + (size_t)lrow * KIN + lk;
+    half8 bcur[KB][NB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int n = 0; n < NB; ++n) bcur[kb][n] = *reinterpret_cast<const half8*>(wlane + (size_t)(n * 16) * KIN + kb * 32);
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap)
+    {
+        const int dy = tap / 3, dx = tap - dy * 3;  // patch coordinates already include the halo
+        half8 bnext[KB][NB];
+        if (tap + 1 < 9)
+        {
+            const _Float16* wt = wlane + (size_t)(tap + 1) * NOUT * KIN;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int n = 0; n < NB; ++n) bnext[kb][n] = *reinterpret_cast<const half8*>(wt + (size_t)(n * 16) * KIN + kb * 32);
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+        {
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+            {
+                const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
+                const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
+#pragma unroll
+                for (int n = 0; n < NB; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[kb][n], acc[m][n], 0, 0, 0);
+            }
+        }
+        if (tap + 1 < 9)
+        {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int n = 0; n < NB; ++n) bcur[kb][n] = bnext[kb][n];
+        }
+    }
+}
+
+// ---- host-side plan of a network: per level the padded GEMM sizes and where its buffers live ----
+inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+struct LevelPlan
+{
+    int H, W, cin_real, cin_pad, cout, npad, cout_store;
+    size_t wpack_off, bias_off, act_off;  // bytes into the forward workspace
+    size_t saved_act_off, saved_pre_off;  // bytes into the saved state (training)
+    // bytes into the backward workspace
+    size_t wt_off;      // packed transposed weights [9][cin_pad][npad] fp16
+    size_t dpre_off;    // gradient of the pre-activations [B][H][W][npad] fp16
+    size_t din_off;     // gradient of the block input [B][H][W][cin_pad] fp16
+    size_t part_off;    // partial weight gradients [groups][9][npad][cin_pad] fp32
+    int groups;         // persistent workgroups of the weight-gradient kernel (per image)
+};
+
+struct NetPlan
+{
+    LevelPlan lv[TRIPS_UNET_MAX_LEVELS];
+    size_t bytes;           // forward workspace
+    size_t saved_bytes;     // saved state
+    size_t backward_bytes;  // backward workspace
+};
+
+inline int check_unet_desc(const TripsUnetDesc* d)
+{
+    if (!d) return set_error(TRIPS_ERR_INVALID_ARG, "desc is NULL");
+    if (d->abi_version != TRIPS_ABI_VERSION)
+        return set_error(TRIPS_ERR_INVALID_ARG, "abi_version %d, library has %d", d->abi_version, TRIPS_ABI_VERSION);
+    if (d->num_levels < 1 || d->num_levels > TRIPS_UNET_MAX_LEVELS)
+        return set_error(TRIPS_ERR_INVALID_ARG, "num_levels %d not in 1..%d", d->num_levels, TRIPS_UNET_MAX_LEVELS);
+    if (d->num_input_channels < 1 || d->num_input_channels > 4)
+        return set_error(TRIPS_ERR_UNSUPPORTED, "num_input_channels %d not in 1..4", d->num_input_channels);
+    if (d->num_output_channels < 1 || d->num_output_channels > 4)
+        return set_error(TRIPS_ERR_UNSUPPORTED, "num_output_channels %d not in 1..4", d->num_output_channels);
+    if (d->batch < 1) return set_error(TRIPS_ERR_INVALID_ARG, "batch < 1");
+    const int C = d->num_input_channels, L = d->num_levels;
+    for (int i = 0; i < L; ++i)
+    {
+        if (d->level_w[i] < 1 || d->level_h[i] < 1 || d->level_w[i] > 32768 || d->level_h[i] > 32768)
+            return set_error(TRIPS_ERR_INVALID_ARG, "level %d size %dx%d", i, d->level_w[i], d->level_h[i]);
+        if (i > 0)
+        {
+            const int w = d->level_w[i - 1], h = d->level_h[i - 1];
+            const bool okw = d->level_w[i] == w / 2 || d->level_w[i] == (w + 1) / 2;
+            const bool okh = d->level_h[i] == h / 2 || d->level_h[i] == (h + 1) / 2;
+            if (!okw || !okh || 2 * d->level_w[i] < w || 2 * d->level_h[i] < h)
+                return set_error(TRIPS_ERR_UNSUPPORTED, "level %d (%dx%d) must be half of level %d (%dx%d), rounded up", i,
+                                 d->level_w[i], d->level_h[i], i - 1, w, h);
+        }
+        const int cout = d->filters[i] - ((i == 0 && L > 1) ? C : 2 * C);
+        if (cout < 1 || cout > 64)
+            return set_error(TRIPS_ERR_UNSUPPORTED, "filters[%d] = %d gives %d convolution outputs (1..64 supported)", i,
+                             d->filters[i], cout);
+        if (i + 1 < L && d->filters[i + 1] > 64)
+            return set_error(TRIPS_ERR_UNSUPPORTED, "filters[%d] = %d input channels (at most 64 supported)", i + 1,
+                             d->filters[i + 1]);
+    }
+    return TRIPS_OK;
+}
+
+// Block i convolves cat(in[i], up2(x_{i+1})) (F[i+1] channels; C for the start block) to F[i] - 2C outputs
+// (F[0] - C for the last block when it is not also the start block), Networks.h:1034-1037,1104-1118.
+inline NetPlan make_plan(const TripsUnetDesc& d)
+{
+    NetPlan np;
+    const int C = d.num_input_channels, L = d.num_levels;
+    size_t o = 0;
+    for (int i = 0; i < L; ++i)
+    {
+        LevelPlan& lv = np.lv[i];
+        lv.H          = d.level_h[i];
+        lv.W          = d.level_w[i];
+        lv.cin_real   = (i == L - 1) ? C : d.filters[i + 1];
+        lv.cin_pad    = lv.cin_real <= 32 ? 32 : 64;
+        lv.cout       = d.filters[i] - ((i == 0 && L > 1) ? C : 2 * C);
+        lv.npad       = 2 * round_up(lv.cout, 16);
+        lv.cout_store = round_up(lv.cout, 8);
+        lv.wpack_off  = o;
+        o += align256((size_t)9 * lv.npad * lv.cin_pad * sizeof(_Float16));
+        lv.bias_off = o;
+        o += align256((size_t)lv.npad * sizeof(float));
+    }
+    for (int i = 0; i < L; ++i)
+    {
+        np.lv[i].act_off = o;
+        o += align256((size_t)d.batch * np.lv[i].H * np.lv[i].W * np.lv[i].cout_store * sizeof(_Float16));
+    }
+    np.bytes = o;
+    size_t sv = 0, bw = 0;
+    for (int i = 0; i < L; ++i)
+    {
+        LevelPlan& lv       = np.lv[i];
+        const size_t pixels = (size_t)d.batch * lv.H * lv.W;
+        lv.saved_act_off    = sv;
+        sv += align256(pixels * lv.cout_store * sizeof(_Float16));
+        lv.saved_pre_off = sv;
+        sv += align256(pixels * lv.npad * sizeof(_Float16));
+        lv.wt_off = bw;
+        bw += align256((size_t)9 * lv.cin_pad * lv.npad * sizeof(_Float16));
+        lv.dpre_off = bw;
+        bw += align256(pixels * lv.npad * sizeof(_Float16));
+        lv.din_off = bw;
+        bw += align256(pixels * lv.cin_pad * sizeof(_Float16));
+        const int tiles = ((lv.W + kConvTileW - 1) / kConvTileW) * ((lv.H + kConvTileH - 1) / kConvTileH);
+        lv.groups       = tiles < 512 ? tiles : 512;
+        lv.part_off     = bw;
+        bw += align256((size_t)d.batch * lv.groups * 9 * lv.npad * lv.cin_pad * sizeof(float));
+    }
+    np.saved_bytes    = sv;
+    np.backward_bytes = bw;
+    return np;
+}
+
+
+}  // namespace trips

@@ -20,22 +20,10 @@
 #include <cmath>
 #include <cstring>
 
-#include "../../include/trips_unet.h"
-#include "splat_internal.h"
+#include "unet_common.h"
 
 namespace trips
 {
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-constexpr int kConvTileH   = 8;
-constexpr int kConvTileW   = 32;
-constexpr int kConvPatchH  = kConvTileH + 2;
-constexpr int kConvPatchW  = kConvTileW + 2;
-constexpr int kBelowH      = kConvTileH / 2 + 2;  // rows / columns of the level below that an upsampled patch touches
-constexpr int kBelowW      = kConvTileW / 2 + 2;
-constexpr int kLdsChanPad  = 8;  // halves added to every LDS row so that 16 lanes reading 16 bytes hit 64 distinct banks
-
 struct ConvParams
 {
     int H, W;            // this level
@@ -50,19 +38,8 @@ struct ConvParams
     const _Float16* wpack;    // [9][NPAD][CIN]
     const float* bias;        // [NPAD]: feature biases, then mask biases, each padded to NPAD / 2
     _Float16* out;            // [H][W][cout_store]
+    _Float16* pre;            // [H][W][NPAD] pre-activations (feature | mask) for the backward, or nullptr
 };
-
-// source row / column and weight of torch's bilinear upsampling with scale_factor 2, align_corners = false
-// (area_pixel_compute_source_index: src = max(0, (dst + 0.5) * 0.5 - 0.5))
-__device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i1, float& lambda)
-{
-    float src = (float(dst) + 0.5f) * 0.5f - 0.5f;
-    src       = src < 0.f ? 0.f : src;
-    i0        = (int)src;
-    i0        = i0 < in_size - 1 ? i0 : in_size - 1;
-    i1        = i0 + 1 < in_size ? i0 + 1 : in_size - 1;
-    lambda    = src - float(i0);
-}
 
 template <int CIN, int NPAD>
 __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
@@ -169,57 +146,11 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         }
     }
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lrow = lane & 15, lk = (lane >> 4) * 8;
-    floatx4 acc[4][NB];
-#pragma unroll
-    for (int m = 0; m < 4; ++m)
-#pragma unroll
-        for (int n = 0; n < NB; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    // B fragments come straight from memory: the packed weights are a few tens of KB that every wavefront of
-    // every workgroup reads at the same addresses, so they stay in L2 / L1, and the tap loop needs no barrier.
-    // The fragments of the next tap are requested before the current tap's MFMAs are issued.
     __syncthreads();  // patch complete
-    const _Float16* wlane = p.wpack + (size_t)lrow * CIN + lk;
-    half8 bcur[KB][NB];
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int n = 0; n < NB; ++n) bcur[kb][n] = *reinterpret_cast<const half8*>(wlane + (size_t)(n * 16) * CIN + kb * 32);
-#pragma unroll
-    for (int tap = 0; tap < 9; ++tap)
-    {
-        const int dy = tap / 3, dx = tap - dy * 3;  // patch coordinates already include the halo
-        half8 bnext[KB][NB];
-        if (tap + 1 < 9)
-        {
-            const _Float16* wt = wlane + (size_t)(tap + 1) * NPAD * CIN;
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int n = 0; n < NB; ++n) bnext[kb][n] = *reinterpret_cast<const half8*>(wt + (size_t)(n * 16) * CIN + kb * 32);
-        }
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-        {
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-            {
-                const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
-                const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
-#pragma unroll
-                for (int n = 0; n < NB; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[kb][n], acc[m][n], 0, 0, 0);
-            }
-        }
-        if (tap + 1 < 9)
-        {
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int n = 0; n < NB; ++n) bcur[kb][n] = bnext[kb][n];
-        }
-    }
+    floatx4 acc[4][NB];
+    conv_taps_mfma<CIN, NPAD>(s_patch, p.wpack, acc);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lrow = lane & 15;
 
     // ---- epilogue: elu(feature) * sigmoid(mask), fp16, channels innermost ----
 #pragma unroll
@@ -230,14 +161,20 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         for (int j = 0; j < HB; ++j)
         {
             const int ch = 16 * j + lrow;
-            if (ch >= p.cout_store) continue;
             const float bf = p.bias[ch], bm = p.bias[NPAD / 2 + ch];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
                 const int x = x0 + (m & 1) * 16 + (lane >> 4) * 4 + i;
                 if (y >= p.H || x >= p.W) continue;
-                const float f = acc[m][j][i] + bf, g = acc[m][HB + j][i] + bm;
+                const float f = acc[m][j][i] + bf, g = acc[m][HB + j][i] + bm;  // both 0 for padding channels
+                if (p.pre)
+                {
+                    _Float16* pr        = p.pre + ((size_t)y * p.W + x) * NPAD;
+                    pr[ch]              = _Float16(f);
+                    pr[NPAD / 2 + ch]   = _Float16(g);
+                }
+                if (ch >= p.cout_store) continue;
                 const float e = f > 0.f ? f : (__expf(f) - 1.f);
                 const float s = 1.f / (1.f + __expf(-g));
                 p.out[((size_t)y * p.W + x) * p.cout_store + ch] = ch < p.cout ? _Float16(e * s) : _Float16(0.f);
@@ -310,88 +247,6 @@ __global__ __launch_bounds__(256) void final_conv1x1_kernel(const FinalParams p)
 // ---------------------------------------------------------------------------------------------------------
 namespace
 {
-int round_up(int v, int m) { return (v + m - 1) / m * m; }
-
-struct LevelPlan
-{
-    int H, W, cin_real, cin_pad, cout, npad, cout_store;
-    size_t wpack_off, bias_off, act_off;  // bytes into the workspace
-};
-
-struct NetPlan
-{
-    LevelPlan lv[TRIPS_UNET_MAX_LEVELS];
-    size_t bytes;
-};
-
-int check_unet_desc(const TripsUnetDesc* d)
-{
-    if (!d) return set_error(TRIPS_ERR_INVALID_ARG, "desc is NULL");
-    if (d->abi_version != TRIPS_ABI_VERSION)
-        return set_error(TRIPS_ERR_INVALID_ARG, "abi_version %d, library has %d", d->abi_version, TRIPS_ABI_VERSION);
-    if (d->num_levels < 1 || d->num_levels > TRIPS_UNET_MAX_LEVELS)
-        return set_error(TRIPS_ERR_INVALID_ARG, "num_levels %d not in 1..%d", d->num_levels, TRIPS_UNET_MAX_LEVELS);
-    if (d->num_input_channels < 1 || d->num_input_channels > 4)
-        return set_error(TRIPS_ERR_UNSUPPORTED, "num_input_channels %d not in 1..4", d->num_input_channels);
-    if (d->num_output_channels < 1 || d->num_output_channels > 4)
-        return set_error(TRIPS_ERR_UNSUPPORTED, "num_output_channels %d not in 1..4", d->num_output_channels);
-    if (d->batch < 1) return set_error(TRIPS_ERR_INVALID_ARG, "batch < 1");
-    const int C = d->num_input_channels, L = d->num_levels;
-    for (int i = 0; i < L; ++i)
-    {
-        if (d->level_w[i] < 1 || d->level_h[i] < 1 || d->level_w[i] > 32768 || d->level_h[i] > 32768)
-            return set_error(TRIPS_ERR_INVALID_ARG, "level %d size %dx%d", i, d->level_w[i], d->level_h[i]);
-        if (i > 0)
-        {
-            const int w = d->level_w[i - 1], h = d->level_h[i - 1];
-            const bool okw = d->level_w[i] == w / 2 || d->level_w[i] == (w + 1) / 2;
-            const bool okh = d->level_h[i] == h / 2 || d->level_h[i] == (h + 1) / 2;
-            if (!okw || !okh || 2 * d->level_w[i] < w || 2 * d->level_h[i] < h)
-                return set_error(TRIPS_ERR_UNSUPPORTED, "level %d (%dx%d) must be half of level %d (%dx%d), rounded up", i,
-                                 d->level_w[i], d->level_h[i], i - 1, w, h);
-        }
-        const int cout = d->filters[i] - ((i == 0 && L > 1) ? C : 2 * C);
-        if (cout < 1 || cout > 64)
-            return set_error(TRIPS_ERR_UNSUPPORTED, "filters[%d] = %d gives %d convolution outputs (1..64 supported)", i,
-                             d->filters[i], cout);
-        if (i + 1 < L && d->filters[i + 1] > 64)
-            return set_error(TRIPS_ERR_UNSUPPORTED, "filters[%d] = %d input channels (at most 64 supported)", i + 1,
-                             d->filters[i + 1]);
-    }
-    return TRIPS_OK;
-}
-
-// Block i convolves cat(in[i], up2(x_{i+1})) (F[i+1] channels; C for the start block) to F[i] - 2C outputs
-// (F[0] - C for the last block when it is not also the start block), Networks.h:1034-1037,1104-1118.
-NetPlan make_plan(const TripsUnetDesc& d)
-{
-    NetPlan np;
-    const int C = d.num_input_channels, L = d.num_levels;
-    size_t o = 0;
-    for (int i = 0; i < L; ++i)
-    {
-        LevelPlan& lv = np.lv[i];
-        lv.H          = d.level_h[i];
-        lv.W          = d.level_w[i];
-        lv.cin_real   = (i == L - 1) ? C : d.filters[i + 1];
-        lv.cin_pad    = lv.cin_real <= 32 ? 32 : 64;
-        lv.cout       = d.filters[i] - ((i == 0 && L > 1) ? C : 2 * C);
-        lv.npad       = 2 * round_up(lv.cout, 16);
-        lv.cout_store = round_up(lv.cout, 8);
-        lv.wpack_off  = o;
-        o += align256((size_t)9 * lv.npad * lv.cin_pad * sizeof(_Float16));
-        lv.bias_off = o;
-        o += align256((size_t)lv.npad * sizeof(float));
-    }
-    for (int i = 0; i < L; ++i)
-    {
-        np.lv[i].act_off = o;
-        o += align256((size_t)d.batch * np.lv[i].H * np.lv[i].W * np.lv[i].cout_store * sizeof(_Float16));
-    }
-    np.bytes = o;
-    return np;
-}
-
 template <int CIN, int NPAD>
 hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
 {
@@ -438,6 +293,14 @@ int trips_unet_workspace_size(const TripsUnetDesc* desc, size_t* bytes)
     return TRIPS_OK;
 }
 
+int trips_unet_saved_size(const TripsUnetDesc* desc, size_t* bytes)
+{
+    if (int e = check_unet_desc(desc)) return e;
+    if (!bytes) return set_error(TRIPS_ERR_INVALID_ARG, "bytes is NULL");
+    *bytes = make_plan(*desc).saved_bytes;
+    return TRIPS_OK;
+}
+
 int trips_unet_flops(const TripsUnetDesc* desc, double* flops)
 {
     if (int e = check_unet_desc(desc)) return e;
@@ -452,7 +315,7 @@ int trips_unet_flops(const TripsUnetDesc* desc, double* flops)
 }
 
 int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
-                       const float* const inputs[TRIPS_UNET_MAX_LEVELS], float* output, void* workspace,
+                       const float* const inputs[TRIPS_UNET_MAX_LEVELS], float* output, void* saved, void* workspace,
                        size_t workspace_bytes, void* stream_)
 {
     if (!ctx) return set_error(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
@@ -467,13 +330,22 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
             return set_error(TRIPS_ERR_INVALID_ARG, "weights of block %d are NULL", i);
     }
     if (!weights->final_weight || !weights->final_bias) return set_error(TRIPS_ERR_INVALID_ARG, "final weights are NULL");
-    if (reinterpret_cast<uintptr_t>(workspace) & 255) return set_error(TRIPS_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255) || (reinterpret_cast<uintptr_t>(saved) & 255))
+        return set_error(TRIPS_ERR_INVALID_ARG, "workspace / saved must be 256-byte aligned");
     const NetPlan np = make_plan(d);
     if (workspace_bytes < np.bytes)
         return set_error(TRIPS_ERR_WORKSPACE_SMALL, "workspace has %zu bytes, %zu needed", workspace_bytes, np.bytes);
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     char* ws           = reinterpret_cast<char*>(workspace);
+    char* sv           = reinterpret_cast<char*>(saved);
     Profiler* prof     = ctx->prof.enabled ? &ctx->prof : nullptr;
+    // block outputs live in the saved state when there is one (the backward reads them), else in the workspace
+    auto act_ptr = [&](int level, int b)
+    {
+        const LevelPlan& l = np.lv[level];
+        char* base         = sv ? sv + l.saved_act_off : ws + l.act_off;
+        return reinterpret_cast<_Float16*>(base) + (size_t)b * l.H * l.W * l.cout_store;
+    };
 
     {
         ProfScope ps(prof, "unet_pack_weights", stream);
@@ -505,7 +377,8 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
             p.feat       = inputs[i] + (size_t)b * C * lv.H * lv.W;
             p.wpack      = reinterpret_cast<const _Float16*>(ws + lv.wpack_off);
             p.bias       = reinterpret_cast<const float*>(ws + lv.bias_off);
-            p.out        = reinterpret_cast<_Float16*>(ws + lv.act_off) + (size_t)b * lv.H * lv.W * lv.cout_store;
+            p.out        = act_ptr(i, b);
+            p.pre        = sv ? reinterpret_cast<_Float16*>(sv + lv.saved_pre_off) + (size_t)b * lv.H * lv.W * lv.npad : nullptr;
             if (i < L - 1)
             {
                 const LevelPlan& lb = np.lv[i + 1];
@@ -513,7 +386,7 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
                 p.Wb         = lb.W;
                 p.cb_store   = lb.cout_store;
                 p.feat_below = inputs[i + 1] + (size_t)b * C * lb.H * lb.W;
-                p.act_below  = reinterpret_cast<const _Float16*>(ws + lb.act_off) + (size_t)b * lb.H * lb.W * lb.cout_store;
+                p.act_below  = act_ptr(i + 1, b);
             }
             hipError_t e = dispatch_conv(p, lv.cin_pad, lv.npad, stream);
             if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "gated conv launch (level %d): %s", i, hipGetErrorString(e));
@@ -532,7 +405,7 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
             p.cact_store = lv.cout_store;
             p.cout       = d.num_output_channels;
             p.feat       = inputs[0] + (size_t)b * C * lv.H * lv.W;
-            p.act        = reinterpret_cast<const _Float16*>(ws + lv.act_off) + (size_t)b * lv.H * lv.W * lv.cout_store;
+            p.act        = act_ptr(0, b);
             p.weight     = weights->final_weight;
             p.bias       = weights->final_bias;
             p.out        = output + (size_t)b * d.num_output_channels * lv.H * lv.W;
