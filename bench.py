@@ -189,6 +189,51 @@ def main():
                 "mfma_frac_of_fp16_dense_peak": round(flops / (net_ms * 1e-3) / 2.5e15, 4),
                 "kernels": {k: round(ms / max(n, 1), 4) for k, (ms, n) in nprof.items()}}
 
+        # The full training step of the fifth configuration: splat forward, net forward, L1 loss against a uniform
+        # target, net backward, splat backward with the net's input gradients, fused Adam over point and net
+        # parameters.
+        target = torch.rand(rgb.shape, generator=gen, device=dev)
+        net_params = [q for q in net.parameters()]
+        net_opt = MyAdam(net_params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+        zero_tail = [torch.zeros_like(im) for im in images[np_.num_layers:]]
+
+        def train_step():
+            for g in grads.values():
+                g.zero_()
+            net_opt.zero_grad(set_to_none=True)
+            ctx.forward(desc, tin, images, saved, workspace)
+            ins = [im.detach().requires_grad_(True) for im in images]
+            loss = (net.forward(ins) - target).abs().mean()
+            loss.backward()
+            gi = [t.grad for t in ins[:np_.num_layers]] + zero_tail
+            ctx.backward(desc, tin, saved, gi, grads, workspace)
+            opt.step()
+            net_opt.step()
+            return loss
+
+        for _ in range(3):
+            train_step()
+        torch.cuda.synchronize()
+        ctx.profile_enable(True)
+        ctx.profile_read()
+        c0 = time.perf_counter()
+        for _ in range(args.steps):
+            train_step()
+        torch.cuda.synchronize()
+        c1 = time.perf_counter()
+        tprof = ctx.profile_read()
+        ctx.profile_enable(False)
+        net_bwd_ms = sum(ms for k, (ms, _) in tprof.items() if k.startswith("unet_bwd")) / args.steps
+        net_fwd_ms = sum(ms for k, (ms, _) in tprof.items() if k.startswith("unet_") and not k.startswith("unet_bwd")) / args.steps
+        unet["train_step"] = {
+            "workload": "config5: splat forward + net forward + L1 loss + net backward + splat backward + fused Adam "
+                        "(point parameters and net weights), 6M points, 1920x1080",
+            "ms_per_step_wall": round((c1 - c0) * 1e3 / args.steps, 4),
+            "ms_all_kernels": round(sum(ms for ms, _ in tprof.values()) / args.steps, 4),
+            "ms_net_forward": round(net_fwd_ms, 4), "ms_net_backward": round(net_bwd_ms, 4),
+            "net_backward_tflops": round(2 * flops / (net_bwd_ms * 1e-3) / 1e12, 1) if net_bwd_ms > 0 else None,
+            "kernels": {k: round(ms / max(n, 1), 4) for k, (ms, n) in tprof.items() if k.startswith("unet_bwd")}}
+
     cpu = None
     if args.cpu_steps > 0:
         from tests import oracle_lib

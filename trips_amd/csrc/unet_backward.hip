@@ -120,39 +120,63 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
     }
 }
 
-// thread t <-> one (output k, input c) pair, or a bias; a block sums a chunk of pixels and adds it once
-constexpr int kFinalChunk = 2048;
+// Weight and bias gradients of the 1x1 convolution: every thread keeps the cout x cin products of its pixels in
+// registers, a block folds them through LDS and adds its sums once. CS = halves per pixel of the block output.
+constexpr int kFinalPixelsPerBlock = 4096;
+template <int CS>
 __global__ __launch_bounds__(256) void final_weight_grad_kernel(const FinalBwdParams p)
 {
-    const int cin      = p.c_feat + p.cact;
+    constexpr int MAXC = 4 + CS;
+    __shared__ float s_sum[4 * MAXC + 4];
+    for (int i = threadIdx.x; i < 4 * MAXC + 4; i += 256) s_sum[i] = 0.f;
+    __syncthreads();
     const size_t plane = (size_t)p.H * p.W;
-    const size_t p0 = (size_t)blockIdx.x * kFinalChunk, p1 = std::min(plane, p0 + kFinalChunk);
-    for (int t = threadIdx.x; t < p.cout * cin + p.cout; t += 256)
+    const size_t p0 = (size_t)blockIdx.x * kFinalPixelsPerBlock, p1 = std::min(plane, p0 + kFinalPixelsPerBlock);
+    float acc[4][MAXC];
+    float accb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) acc[k][c] = 0.f;
+    for (size_t pix = p0 + threadIdx.x; pix < p1; pix += 256)
     {
-        float sum = 0.f;
-        if (t < p.cout * cin)
+        float g[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < p.cout; ++k) g[k] = p.d_out[k * plane + pix];
+        float x[MAXC];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) x[c] = c < p.c_feat ? float(_Float16(p.feat[c * plane + pix])) : 0.f;
+#pragma unroll
+        for (int q = 0; q < CS / 8; ++q)
         {
-            const int k = t / cin, c = t - k * cin;
-            const float* g = p.d_out + k * plane;
-            if (c < p.c_feat)
-            {
-                const float* x = p.feat + c * plane;
-                for (size_t pix = p0; pix < p1; ++pix) sum += g[pix] * float(_Float16(x[pix]));
-            }
-            else
-            {
-                const _Float16* x = p.act + (c - p.c_feat);
-                for (size_t pix = p0; pix < p1; ++pix) sum += g[pix] * float(x[pix * p.cact_store]);
-            }
-            atomicAdd(p.d_weight + t, sum);
+            const half8 v = *reinterpret_cast<const half8*>(p.act + pix * CS + 8 * q);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[4 + 8 * q + i] = float(v[i]);
         }
-        else
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
         {
-            const float* g = p.d_out + (size_t)(t - p.cout * cin) * plane;
-            for (size_t pix = p0; pix < p1; ++pix) sum += g[pix];
-            atomicAdd(p.d_bias + (t - p.cout * cin), sum);
+            accb[k] += g[k];
+#pragma unroll
+            for (int c = 0; c < MAXC; ++c) acc[k][c] += g[k] * x[c];
         }
     }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        atomicAdd(&s_sum[4 * MAXC + k], accb[k]);
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) atomicAdd(&s_sum[k * MAXC + c], acc[k][c]);
+    }
+    __syncthreads();
+    // registers are laid out [k][4 image channels | CS block outputs]; the weight is [k][c_feat + cact]
+    const int cin = p.c_feat + p.cact;
+    for (int t = threadIdx.x; t < p.cout * cin; t += 256)
+    {
+        const int k = t / cin, c = t - k * cin;
+        const int r = c < p.c_feat ? c : 4 + (c - p.c_feat);
+        atomicAdd(p.d_weight + t, s_sum[k * MAXC + r]);
+    }
+    if ((int)threadIdx.x < p.cout) atomicAdd(p.d_bias + threadIdx.x, s_sum[4 * MAXC + threadIdx.x]);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -315,7 +339,7 @@ struct BiasGradParams
     float* d_bias_m;
 };
 
-constexpr int kBiasChunk = 8192;
+constexpr int kBiasChunk = 1024;
 __global__ __launch_bounds__(256) void bias_grad_kernel(const BiasGradParams p)
 {
     __shared__ float s_sum[128];
@@ -521,24 +545,29 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     }
 }
 
-// sums the partial weight gradients of all workgroups (and images) into the reference's [Cout][Cin][3][3] layout
+// sums the partial weight gradients of all workgroups (and images) into the reference's [Cout][Cin][3][3] layout;
+// 8 lanes share an element and split the partials between them
 __global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const float* __restrict__ part, int groups, int cout,
                                                                  int cin_real, int cin_pad, int npad, float scale_inv,
                                                                  float* __restrict__ d_wf, float* __restrict__ d_wm)
 {
     const int total = 9 * npad * cin_pad;
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256)
-    {
-        const int c = i % cin_pad, n = (i / cin_pad) % npad, tap = i / (cin_pad * npad);
-        const int half = npad / 2;
-        const int o    = n < half ? n : n - half;
-        if (o >= cout || c >= cin_real) continue;
-        float* dst = n < half ? d_wf : d_wm;
-        if (!dst) continue;
-        float s = 0.f;
-        for (int g = 0; g < groups; ++g) s += part[(size_t)g * total + i];
-        dst[((size_t)o * cin_real + c) * 9 + tap] = s * scale_inv;
-    }
+    const int sub   = threadIdx.x & 7;
+    // consecutive elements (c fastest) sit in consecutive 8-lane groups: a wavefront reads 8 x 32 bytes per step
+    const int i = (blockIdx.x * 256 + threadIdx.x) >> 3;
+    float s     = 0.f;
+    if (i < total)
+        for (int g = sub; g < groups; g += 8) s += part[(size_t)g * total + i];
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 4);
+    if (i >= total || sub != 0) return;
+    const int c = i % cin_pad, n = (i / cin_pad) % npad, tap = i / (cin_pad * npad);
+    const int half = npad / 2;
+    const int o    = n < half ? n : n - half;
+    if (o >= cout || c >= cin_real) return;
+    float* dst = n < half ? d_wf : d_wm;
+    if (dst) dst[((size_t)o * cin_real + c) * 9 + tap] = s * scale_inv;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -698,8 +727,15 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             hipLaunchKernelGGL(final_backward_kernel, dim3(blocks), dim3(256), 0, stream, p);
             if (p.d_weight && p.d_bias)
             {
-                const int chunks = (int)((plane + kFinalChunk - 1) / kFinalChunk);
-                hipLaunchKernelGGL(final_weight_grad_kernel, dim3(chunks), dim3(256), 0, stream, p);
+                const int chunks = (int)((plane + kFinalPixelsPerBlock - 1) / kFinalPixelsPerBlock);
+                switch (lv.cout_store)
+                {
+#define TRIPS_FW(CS_) \
+    case CS_: hipLaunchKernelGGL((final_weight_grad_kernel<CS_>), dim3(chunks), dim3(256), 0, stream, p); break;
+                    TRIPS_FW(8) TRIPS_FW(16) TRIPS_FW(24) TRIPS_FW(32) TRIPS_FW(40) TRIPS_FW(48) TRIPS_FW(56) TRIPS_FW(64)
+#undef TRIPS_FW
+                    default: return set_error(TRIPS_ERR_UNSUPPORTED, "block output stride %d", lv.cout_store);
+                }
             }
         }
     }
@@ -751,7 +787,7 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             if (grads->feature_weight[i] || grads->mask_weight[i])
             {
                 const int total = 9 * lv.npad * lv.cin_pad;
-                hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
+                hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total * 8 + 255) / 256), dim3(256), 0, stream,
                                    reinterpret_cast<const float*>(ws + lv.part_off), d.batch * lv.groups, lv.cout, lv.cin_real,
                                    lv.cin_pad, lv.npad, scale_inv, grads->feature_weight[i], grads->mask_weight[i]);
             }

@@ -196,7 +196,7 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
         lv.din_off = bw;
         bw += align256(pixels * lv.cin_pad * sizeof(_Float16));
         const int tiles = ((lv.W + kConvTileW - 1) / kConvTileW) * ((lv.H + kConvTileH - 1) / kConvTileH);
-        lv.groups       = tiles < 512 ? tiles : 512;
+        lv.groups       = tiles < 1024 ? tiles : 1024;
         lv.part_off     = bw;
         bw += align256((size_t)d.batch * lv.groups * 9 * lv.npad * lv.cin_pad * sizeof(float));
     }
