@@ -20,8 +20,8 @@ def _center_crop(t, h, w):
 
 
 def gated(x, blk, half_rounding):
-    wf, bf = _r(blk.feature_transform.weight, half_rounding), blk.feature_transform.bias
-    wm, bm = _r(blk.mask_transform.weight, half_rounding), blk.mask_transform.bias
+    wf, bf = _r(blk.feature_conv.weight, half_rounding), blk.feature_conv.bias
+    wm, bm = _r(blk.mask_conv.weight, half_rounding), blk.mask_conv.bias
     x = _r(x, half_rounding)
     f = F.elu(F.conv2d(x, wf, bf, padding=1))
     m = torch.sigmoid(F.conv2d(x, wm, bm, padding=1))
@@ -41,4 +41,4 @@ def unet_forward(net, inputs, half_rounding=True):
         up = _center_crop(up, feats.shape[2], feats.shape[3])
         comb = torch.cat([feats, up], 1)
         cur = torch.cat([_r(feats, half_rounding), gated(comb, net.block(i), half_rounding)], 1)
-    return F.conv2d(cur, _r(net.final.weight, half_rounding), net.final.bias)
+    return F.conv2d(cur, _r(net.final_conv.weight, half_rounding), net.final_conv.bias)

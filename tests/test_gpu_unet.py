@@ -56,7 +56,7 @@ def test_unet_forward_matches_torch(filters, levels, w, h):
     inputs = _pyramid(w, h, levels, 4, batch=2, seed=10 + levels)
     if levels == 1:
         # a one-level net feeds the final 1x1 with F[0] - C channels; the reference's final expects F[0]
-        net.final = torch.nn.Conv2d(filters[0] - 4, 3, 1)
+        net.final = torch.nn.Sequential(torch.nn.Conv2d(filters[0] - 4, 3, 1), torch.nn.Identity())
     _compare(net, inputs)
 
 
@@ -146,5 +146,5 @@ def test_unet_backward_small_gradients_survive_fp16():
         want = b.grad.numpy()
         assert np.abs(want).max() < 1e-6
         assert np.abs(a.grad.cpu().numpy() - want).max() < 3e-2 * np.abs(want).max()
-    want = ref.up1.feature_transform.weight.grad.numpy()
-    assert np.abs(net.up1.feature_transform.weight.grad.cpu().numpy() - want).max() < 3e-2 * np.abs(want).max()
+    want = ref.up1.convolution.feature_conv.weight.grad.numpy()
+    assert np.abs(net.up1.convolution.feature_conv.weight.grad.cpu().numpy() - want).max() < 3e-2 * np.abs(want).max()

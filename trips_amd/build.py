@@ -46,15 +46,27 @@ def build_torch_shim(verbose=False):
     tlib = ce.library_paths()[0]
     inc = [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include"]
     abi_flag = f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"
-    cmd = (["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-variable", abi_flag,
-            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_trips_torch",
-            "-DTORCH_API_INCLUDE_EXTENSION_H"] + inc +
-           [os.path.join(SHIM_DIR, "trips_torch.cpp"), os.path.join(SHIM_DIR, "trips_torch_py.cpp"),
-            f"-L{tlib}", f"-L{HERE}", "-ltrips_splat", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
-            "-ltorch_python", f"-Wl,-rpath,{tlib}", "-Wl,-rpath,$ORIGIN", "-o", SHIM_LIB])
+    flags = (["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-variable", abi_flag, "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+              "-DTORCH_EXTENSION_NAME=_trips_torch", "-DTORCH_API_INCLUDE_EXTENSION_H"] + inc)
+    sources = ("trips_torch.cpp", "trips_unet_torch.cpp", "trips_scene_io.cpp", "trips_torch_py.cpp")
+    objdir = os.path.join(SHIM_DIR, "_obj")
+    os.makedirs(objdir, exist_ok=True)
+    procs = []
+    for f in sources:  # one compiler process per translation unit, side by side
+        obj = os.path.join(objdir, f.replace(".cpp", ".o"))
+        cmd = ["g++"] + flags + ["-c", os.path.join(SHIM_DIR, f), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((cmd, obj, subprocess.Popen(cmd)))
+    for cmd, obj, pr in procs:
+        if pr.wait() != 0:
+            raise subprocess.CalledProcessError(pr.returncode, cmd)
+    link = (["g++", "-shared"] + [obj for _, obj, _ in procs] +
+            [f"-L{tlib}", f"-L{HERE}", "-ltrips_splat", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+             "-ltorch_python", f"-Wl,-rpath,{tlib}", "-Wl,-rpath,$ORIGIN", "-o", SHIM_LIB])
     if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+        print(" ".join(link), flush=True)
+    subprocess.check_call(link)
     return SHIM_LIB
 
 

@@ -1,7 +1,9 @@
 // pybind11 entry points that drive the C++ operator surface from Python tests.
 #include <torch/extension.h>
 
+#include "trips_scene_io.h"
 #include "trips_torch.h"
+#include "trips_unet_torch.h"
 
 namespace
 {
@@ -43,8 +45,119 @@ std::vector<torch::Tensor> blend_point_cloud(Session& s, std::vector<std::vector
 }
 }  // namespace
 
+namespace
+{
+struct UnetSession
+{
+    MultiScaleUnet2dDecOnlySmallFixed net = nullptr;
+    UnetSession(std::vector<int> filters, int num_layers, int num_input_layers, int num_input_channels)
+    {
+        MultiScaleUnet2dParams p;
+        p.filters_network    = filters;
+        p.num_layers         = num_layers;
+        p.num_input_layers   = num_input_layers;
+        p.num_input_channels = num_input_channels;
+        net                  = MultiScaleUnet2dDecOnlySmallFixed(p);
+    }
+    std::vector<std::pair<std::string, torch::Tensor>> named_parameters()
+    {
+        std::vector<std::pair<std::string, torch::Tensor>> out;
+        for (auto& kv : net->named_parameters()) out.emplace_back(kv.key(), kv.value());
+        return out;
+    }
+};
+
+SceneModules make_modules(torch::Tensor position, torch::Tensor point_size, torch::Tensor index, torch::Tensor color,
+                          torch::Tensor texture, torch::Tensor background, torch::Tensor confidence, torch::Tensor poses_se3,
+                          torch::Tensor intrinsics)
+{
+    SceneModules s;
+    s.point_cloud_cuda = NeuralPointCloudCudaModule(position, point_size, index, color);
+    s.texture          = NeuralTextureModule(texture, background, confidence);
+    s.poses            = PoseModule(poses_se3);
+    s.intrinsics       = IntrinsicsModule(intrinsics);
+    return s;
+}
+
+py::dict modules_to_dict(const SceneModules& s)
+{
+    py::dict d;
+    auto put = [&](const char* prefix, const torch::nn::Module& m)
+    {
+        for (auto& kv : m.named_parameters()) d[py::str(std::string(prefix) + "." + kv.key())] = kv.value();
+        for (auto& kv : m.named_buffers()) d[py::str(std::string(prefix) + "." + kv.key())] = kv.value();
+    };
+    put("points", *s.point_cloud_cuda);
+    put("texture", *s.texture);
+    put("poses", *s.poses);
+    put("intrinsics", *s.intrinsics);
+    d["texture.prepared_confidence"] = s.texture->confidence_value_of_point;
+    return d;
+}
+}  // namespace
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
+    py::class_<UnetSession>(m, "UnetSession")
+        .def(py::init<std::vector<int>, int, int, int>(), py::arg("filters"), py::arg("num_layers"), py::arg("num_input_layers"),
+             py::arg("num_input_channels") = 4)
+        .def("named_parameters", &UnetSession::named_parameters)
+        .def("cuda", [](UnetSession& s) { s.net->to(torch::kCUDA); })
+        .def("forward", [](UnetSession& s, std::vector<torch::Tensor> inputs) { return s.net->forward(inputs); })
+        .def("save", [](UnetSession& s, const std::string& file) { torch::save(s.net, file); })
+        .def("load", [](UnetSession& s, const std::string& file) { torch::load(s.net, file); });
+
+    m.def("save_checkpoint",
+          [](const std::string& dir, const std::string& name, torch::Tensor position, torch::Tensor point_size, torch::Tensor index,
+             torch::Tensor color, torch::Tensor texture, torch::Tensor background, torch::Tensor confidence, torch::Tensor poses_se3,
+             torch::Tensor intrinsics, bool reduced)
+          { SaveCheckpoint(make_modules(position, point_size, index, color, texture, background, confidence, poses_se3, intrinsics), dir, name, reduced); });
+    m.def("load_checkpoint",
+          [](const std::string& dir, const std::string& name, int64_t num_points, int64_t channels, int64_t frames, int64_t cameras)
+          {
+              // modules of the right shapes, as a TRIPS build has after constructing the scene; the archives overwrite them
+              auto f32 = torch::kFloat32;
+              SceneModules s = make_modules(torch::zeros({num_points, 4}, f32), torch::zeros({num_points, 1}, f32),
+                                            torch::zeros({num_points, 1}, torch::kInt32), torch::zeros({num_points, 4}, f32),
+                                            torch::zeros({channels, num_points}, f32), torch::zeros({channels}, f32),
+                                            torch::zeros({1, num_points}, f32), torch::zeros({frames, 8}, torch::kFloat64),
+                                            torch::zeros({cameras, 13}, f32));
+              const int n = LoadCheckpoint(s, dir, name);
+              py::dict d  = modules_to_dict(s);
+              d["archives_loaded"] = n;
+              return d;
+          });
+    m.def("load_scene",
+          [](const std::string& dir)
+          {
+              SceneData s = LoadScene(dir);
+              py::dict d;
+              d["scene_name"]     = s.scene_name;
+              d["image_names"]    = s.image_names;
+              d["camera_indices"] = s.camera_indices;
+              d["poses_se3"]      = PosesToSe3(s.poses);
+              d["intrinsics"]     = CamerasToIntrinsics(s.scene_cameras);
+              std::vector<std::pair<int, int>> sizes;
+              for (auto& c : s.scene_cameras) sizes.emplace_back(c.w, c.h);
+              d["camera_sizes"] = sizes;
+              if (s.point_position.defined()) d["point_position"] = s.point_position;
+              if (s.point_normal.defined()) d["point_normal"] = s.point_normal;
+              if (s.point_color.defined()) d["point_color"] = s.point_color;
+              return d;
+          });
+    m.def("save_camera",
+          [](const std::string& file, int w, int h, std::vector<float> K, std::vector<float> distortion)
+          {
+              SceneCameraParams c;
+              c.w = w, c.h = h;
+              for (size_t i = 0; i < 5; ++i) c.K[i] = K.at(i);
+              for (size_t i = 0; i < 8; ++i) c.distortion[i] = distortion.at(i);
+              SaveSceneCameraParams(c, file);
+          });
+    m.def("save_poses",
+          [](const std::string& file, std::vector<std::array<double, 7>> poses) { SavePoses(poses, file); });
+    m.def("load_poses", [](const std::string& file) { return LoadPoses(file); });
+
     py::class_<Session>(m, "Session")
         .def(py::init<>())
         .def("set_scene",

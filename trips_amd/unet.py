@@ -2,8 +2,9 @@
 
 Names follow src/lib/models/Networks.h of the reference: MultiScaleUnet2dParams (ini section
 [MultiScaleUnet2dParams], configs/train_normalnet.ini:200-219) and MultiScaleUnet2dDecOnlySmallFixed
-(Networks.h:1080-1208) with the registered module names `start`, `up1` .. `up<L-1>`, `final`. The gated block's
-own parameter names come from an un-vendored dependency; `feature_transform` / `mask_transform` are used here.
+(Networks.h:1080-1208) with the registered module names `start.conv`, `up<i>.up`, `up<i>.convolution`, `final`.
+The gated block's own parameter names come from an un-vendored dependency; Sequentials `feature_transform` /
+`mask_transform` (convolution at index 0) are used here.
 
 forward() runs the HIP kernels (fp16 operands on the matrix cores, fp32 accumulation); with autograd enabled it
 records one graph node whose backward is the device backward. There is no CPU path.
@@ -36,12 +37,38 @@ class MultiScaleUnet2dParams:
 
 
 class GatedBlock(torch.nn.Module):
-    """elu(conv_f(x)) * sigmoid(conv_m(x)), 3x3, stride 1, zero padding 1; holds the parameters only."""
+    """elu(conv_f(x)) * sigmoid(conv_m(x)), 3x3, stride 1, zero padding 1; holds the parameters only.
+    The two branches are Sequentials (convolution, activation), so a parameter is `feature_transform.0.weight`."""
 
     def __init__(self, in_channels, out_channels):
         super().__init__()
-        self.feature_transform = torch.nn.Conv2d(in_channels, out_channels, 3, padding=1)
-        self.mask_transform = torch.nn.Conv2d(in_channels, out_channels, 3, padding=1)
+        self.feature_transform = torch.nn.Sequential(torch.nn.Conv2d(in_channels, out_channels, 3, padding=1), torch.nn.ELU())
+        self.mask_transform = torch.nn.Sequential(torch.nn.Conv2d(in_channels, out_channels, 3, padding=1), torch.nn.Sigmoid())
+
+    @property
+    def feature_conv(self):
+        return self.feature_transform[0]
+
+    @property
+    def mask_conv(self):
+        return self.mask_transform[0]
+
+
+class SmallDecStartBlock(torch.nn.Module):
+    """Networks.h:751-787: registers its gated block as `conv`."""
+
+    def __init__(self, in_channels, out_channels):
+        super().__init__()
+        self.conv = GatedBlock(in_channels, out_channels)
+
+
+class UpsampleDecOnlySmallBlockFixed(torch.nn.Module):
+    """Networks.h:999-1098: registers `up` (the bilinear upsampling) and `convolution` (the gated block)."""
+
+    def __init__(self, in_channels, conv_out_channels):
+        super().__init__()
+        self.up = torch.nn.Sequential(torch.nn.Upsample(scale_factor=2.0, mode="bilinear", align_corners=False))
+        self.convolution = GatedBlock(in_channels, conv_out_channels)
 
 
 class _UnetFunction(torch.autograd.Function):
@@ -77,25 +104,29 @@ class MultiScaleUnet2dDecOnlySmallFixed(torch.nn.Module):
         self.grad_scale = float(grad_scale)  # factor the fp16 gradients inside the backward are carried with
         L, Cin, F = p.num_layers, p.num_input_channels, list(p.filters_network)
         # Networks.h:1104-1118: start block outputs F[L-1] - 2C, block i outputs F[i] - 2C (F[0] - C for the last)
-        self.start = GatedBlock(Cin, F[L - 1] - 2 * Cin)
+        self.start = SmallDecStartBlock(Cin, F[L - 1] - 2 * Cin)
         for i in range(L - 2, -1, -1):
             out = F[i] - (Cin if i == 0 else 2 * Cin)
-            self.add_module(f"up{i + 1}", GatedBlock(F[i + 1], out))
-        self.final = torch.nn.Conv2d(F[0], p.num_output_channels, 1)
+            self.add_module(f"up{i + 1}", UpsampleDecOnlySmallBlockFixed(F[i + 1], out))
+        self.final = torch.nn.Sequential(torch.nn.Conv2d(F[0], p.num_output_channels, 1), torch.nn.Identity())
         self._buffers_dev = {}
 
     def block(self, i):
-        """Gated block of pyramid level i (the start block for the coarsest level)."""
+        """Gated block of pyramid level i (the start block's for the coarsest level)."""
         L = self.params.num_layers
-        return self.start if i == L - 1 else getattr(self, f"up{i + 1}")
+        return self.start.conv if i == L - 1 else getattr(self, f"up{i + 1}").convolution
+
+    @property
+    def final_conv(self):
+        return self.final[0]
 
     def ordered_parameters(self):
         """Parameters in the order of the C structs: per level feature weight, bias, mask weight, bias; then final."""
         out = []
         for i in range(self.params.num_layers):
             b = self.block(i)
-            out += [b.feature_transform.weight, b.feature_transform.bias, b.mask_transform.weight, b.mask_transform.bias]
-        return out + [self.final.weight, self.final.bias]
+            out += [b.feature_conv.weight, b.feature_conv.bias, b.mask_conv.weight, b.mask_conv.bias]
+        return out + [self.final_conv.weight, self.final_conv.bias]
 
     def he_normal_(self, generator=None):
         """He-normal weights, zero biases (the initialisation the benchmark configuration names)."""
