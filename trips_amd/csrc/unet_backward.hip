@@ -160,12 +160,25 @@ __global__ __launch_bounds__(256) void final_weight_grad_kernel(const FinalBwdPa
             for (int c = 0; c < MAXC; ++c) acc[k][c] += g[k] * x[c];
         }
     }
+    // fold the wavefront with a butterfly first: 64 lanes adding to one LDS address would be serialised
+    auto wave_sum = [](float v)
+    {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        return v;
+    };
+    const bool first_lane = (threadIdx.x & 63) == 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k)
     {
-        atomicAdd(&s_sum[4 * MAXC + k], accb[k]);
+        const float b = wave_sum(accb[k]);
+        if (first_lane) atomicAdd(&s_sum[4 * MAXC + k], b);
 #pragma unroll
-        for (int c = 0; c < MAXC; ++c) atomicAdd(&s_sum[k * MAXC + c], acc[k][c]);
+        for (int c = 0; c < MAXC; ++c)
+        {
+            const float v = wave_sum(acc[k][c]);
+            if (first_lane) atomicAdd(&s_sum[k * MAXC + c], v);
+        }
     }
     __syncthreads();
     // registers are laid out [k][4 image channels | CS block outputs]; the weight is [k][c_feat + cact]
@@ -400,8 +413,14 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     constexpr int GROUPS = CIN / 8;
     constexpr int NB     = NPAD / 16;
     constexpr int CB     = CIN / 16;
-    constexpr int UNITS  = 9 * NB;            // (tap, 16 pre-activation channels) pairs, dealt round-robin to the 4 wavefronts
-    constexpr int U      = (UNITS + 3) / 4;
+    // The 4 wavefronts split the NPAD x CIN result: CBW ways over the 16-channel input blocks, NBW ways over the
+    // 16-channel pre-activation blocks; each keeps all 9 taps of its blocks. Per tile row a wavefront reads its A
+    // fragments (pre-activation gradients, the same for every tap) once and one B fragment per tap and input block.
+    constexpr int CBW    = CB < 4 ? CB : 4;
+    constexpr int NBW    = 4 / CBW;
+    constexpr int MYCB   = CB / CBW;
+    constexpr int MYNB   = NB / NBW;
+    static_assert(CB % CBW == 0 && NB % NBW == 0, "block split");
     extern __shared__ _Float16 smem[];
     _Float16* s_below = smem;                                  // [kBelowH * kBelowW][ROW]
     _Float16* s_xt    = s_below + kBelowH * kBelowW * ROW;     // [CIN][kXtChan]
@@ -411,11 +430,14 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
-    floatx4 acc[U][CB];
+    const int cb0 = (wave % CBW) * MYCB, nb0 = (wave / CBW) * MYNB;
+    floatx4 acc[9][MYNB][MYCB];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int t = 0; t < 9; ++t)
 #pragma unroll
-        for (int c = 0; c < CB; ++c) acc[u][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int n = 0; n < MYNB; ++n)
+#pragma unroll
+            for (int c = 0; c < MYCB; ++c) acc[t][n][c] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // channels that no stage writes stay zero for every tile
     for (int i = threadIdx.x; i < CIN * kXtChan; i += 256) s_xt[i] = _Float16(0.f);
@@ -506,23 +528,22 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         __syncthreads();
         // ---- dW[tap][n][c] += sum over the tile's pixels of dpre[pixel][n] * x[pixel + tap][c] ----
 #pragma unroll
-        for (int uu = 0; uu < U; ++uu)
+        for (int r = 0; r < kConvTileH; ++r)
         {
-            const int u = wave + 4 * uu;
-            if (u < UNITS)
+            half8 a[MYNB];
+#pragma unroll
+            for (int n = 0; n < MYNB; ++n)
+                a[n] = *reinterpret_cast<const half8*>(s_dt + ((nb0 + n) * 16 + lrow) * kDtChan + r * kConvTileW + lk);
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap)
             {
-                const int tap = u / NB, nb = u - tap * NB;
                 const int dy = tap / 3, dx = tap - dy * 3;
 #pragma unroll
-                for (int r = 0; r < kConvTileH; ++r)
+                for (int c = 0; c < MYCB; ++c)
                 {
-                    const half8 a = *reinterpret_cast<const half8*>(s_dt + (nb * 16 + lrow) * kDtChan + r * kConvTileW + lk);
+                    const half8 b = *reinterpret_cast<const half8_unaligned*>(s_xt + ((cb0 + c) * 16 + lrow) * kXtChan + (r + dy) * kXtRow + lk + dx);
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb)
-                    {
-                        const half8 b = *reinterpret_cast<const half8_unaligned*>(s_xt + (cb * 16 + lrow) * kXtChan + (r + dy) * kXtRow + lk + dx);
-                        acc[uu][cb]   = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[uu][cb], 0, 0, 0);
-                    }
+                    for (int n = 0; n < MYNB; ++n) acc[tap][n][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[n], b, acc[tap][n][c], 0, 0, 0);
                 }
             }
         }
@@ -530,44 +551,57 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 
     float* part = p.part + (size_t)blockIdx.x * 9 * NPAD * CIN;
 #pragma unroll
-    for (int uu = 0; uu < U; ++uu)
-    {
-        const int u = wave + 4 * uu;
-        if (u < UNITS)
-        {
-            const int tap = u / NB, nb = u - tap * NB;
+    for (int tap = 0; tap < 9; ++tap)
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
+        for (int n = 0; n < MYNB; ++n)
+#pragma unroll
+            for (int c = 0; c < MYCB; ++c)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    part[((size_t)tap * NPAD + nb * 16 + (lane >> 4) * 4 + i) * CIN + cb * 16 + lrow] = acc[uu][cb][i];
-        }
-    }
+                    part[((size_t)tap * NPAD + (nb0 + n) * 16 + (lane >> 4) * 4 + i) * CIN + (cb0 + c) * 16 + lrow] = acc[tap][n][c][i];
 }
 
-// sums the partial weight gradients of all workgroups (and images) into the reference's [Cout][Cin][3][3] layout;
-// 8 lanes share an element and split the partials between them
-__global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const float* __restrict__ part, int groups, int cout,
-                                                                 int cin_real, int cin_pad, int npad, float scale_inv,
+// Sum of the partial weight gradients of all workgroups (and images), in two steps so that many loads are in
+// flight and every load is a full line: slice y of kReduceSlices sums its share of the partials element by element
+// (consecutive threads = consecutive elements), then the slices are summed into the reference's [Cout][Cin][3][3].
+constexpr int kReduceSlices = 16;
+__global__ __launch_bounds__(256) void reduce_weight_grad_slices_kernel(const float* __restrict__ part, int groups, int total,
+                                                                        float* __restrict__ sliced)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int per = (groups + kReduceSlices - 1) / kReduceSlices;
+    const int g0 = blockIdx.y * per, g1 = min(groups, g0 + per);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int g = g0;
+    for (; g + 4 <= g1; g += 4)
+    {
+        s0 += part[(size_t)g * total + i];
+        s1 += part[(size_t)(g + 1) * total + i];
+        s2 += part[(size_t)(g + 2) * total + i];
+        s3 += part[(size_t)(g + 3) * total + i];
+    }
+    for (; g < g1; ++g) s0 += part[(size_t)g * total + i];
+    sliced[(size_t)blockIdx.y * total + i] = (s0 + s1) + (s2 + s3);
+}
+
+__global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const float* __restrict__ sliced, int cout, int cin_real,
+                                                                 int cin_pad, int npad, float scale_inv,
                                                                  float* __restrict__ d_wf, float* __restrict__ d_wm)
 {
     const int total = 9 * npad * cin_pad;
-    const int sub   = threadIdx.x & 7;
-    // consecutive elements (c fastest) sit in consecutive 8-lane groups: a wavefront reads 8 x 32 bytes per step
-    const int i = (blockIdx.x * 256 + threadIdx.x) >> 3;
-    float s     = 0.f;
-    if (i < total)
-        for (int g = sub; g < groups; g += 8) s += part[(size_t)g * total + i];
-    s += __shfl_xor(s, 1);
-    s += __shfl_xor(s, 2);
-    s += __shfl_xor(s, 4);
-    if (i >= total || sub != 0) return;
+    const int i     = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
     const int c = i % cin_pad, n = (i / cin_pad) % npad, tap = i / (cin_pad * npad);
     const int half = npad / 2;
     const int o    = n < half ? n : n - half;
     if (o >= cout || c >= cin_real) return;
     float* dst = n < half ? d_wf : d_wm;
-    if (dst) dst[((size_t)o * cin_real + c) * 9 + tap] = s * scale_inv;
+    if (!dst) return;
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < kReduceSlices; ++k) s += sliced[(size_t)k * total + i];
+    dst[((size_t)o * cin_real + c) * 9 + tap] = s * scale_inv;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -787,9 +821,11 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             if (grads->feature_weight[i] || grads->mask_weight[i])
             {
                 const int total = 9 * lv.npad * lv.cin_pad;
-                hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total * 8 + 255) / 256), dim3(256), 0, stream,
-                                   reinterpret_cast<const float*>(ws + lv.part_off), d.batch * lv.groups, lv.cout, lv.cin_real,
-                                   lv.cin_pad, lv.npad, scale_inv, grads->feature_weight[i], grads->mask_weight[i]);
+                float* sliced   = reinterpret_cast<float*>(ws + lv.sliced_off);
+                hipLaunchKernelGGL(reduce_weight_grad_slices_kernel, dim3((total + 255) / 256, kReduceSlices), dim3(256), 0, stream,
+                                   reinterpret_cast<const float*>(ws + lv.part_off), d.batch * lv.groups, total, sliced);
+                hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, sliced, lv.cout,
+                                   lv.cin_real, lv.cin_pad, lv.npad, scale_inv, grads->feature_weight[i], grads->mask_weight[i]);
             }
         }
         {

@@ -91,6 +91,22 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, const _F
     }
 }
 
+// Copies `groups` x 8 halves per pixel of an 8 x 32 tile staged in LDS ([256][lds_stride]) to a channels-innermost
+// image ([H][W][dst_stride]) with 16-byte stores: consecutive lanes write consecutive 16 bytes, so a tile row leaves
+// as whole lines (2-byte stores straight from the MFMA result layout cost twice the memory requests).
+__device__ __forceinline__ void store_tile_nhwc(const _Float16* s_tile, int lds_stride, int groups, _Float16* dst,
+                                                int dst_stride, int x0, int y0, int W, int H)
+{
+    for (int item = threadIdx.x; item < kConvTileH * kConvTileW * groups; item += 256)
+    {
+        const int g = item % groups, tp = item / groups;
+        const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
+        if (y < H && x < W)
+            *reinterpret_cast<half8*>(dst + ((size_t)y * W + x) * dst_stride + 8 * g) =
+                *reinterpret_cast<const half8*>(s_tile + (size_t)tp * lds_stride + 8 * g);
+    }
+}
+
 // ---- host-side plan of a network: per level the padded GEMM sizes and where its buffers live ----
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
@@ -104,6 +120,7 @@ struct LevelPlan
     size_t dpre_off;    // gradient of the pre-activations [B][H][W][npad] fp16
     size_t din_off;     // gradient of the block input [B][H][W][cin_pad] fp16
     size_t part_off;    // partial weight gradients [groups][9][npad][cin_pad] fp32
+    size_t sliced_off;  // partial sums of the partials [16][9][npad][cin_pad] fp32
     int groups;         // persistent workgroups of the weight-gradient kernel (per image)
 };
 
@@ -199,6 +216,8 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
         lv.groups       = tiles < 1024 ? tiles : 1024;
         lv.part_off     = bw;
         bw += align256((size_t)d.batch * lv.groups * 9 * lv.npad * lv.cin_pad * sizeof(float));
+        lv.sliced_off = bw;
+        bw += align256((size_t)16 * 9 * lv.npad * lv.cin_pad * sizeof(float));
     }
     np.saved_bytes    = sv;
     np.backward_bytes = bw;

@@ -152,11 +152,15 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
 
-    // ---- epilogue: elu(feature) * sigmoid(mask), fp16, channels innermost ----
+    // ---- epilogue: elu(feature) * sigmoid(mask) in fp16, staged in LDS (the patch is no longer needed) and
+    // written channels innermost with full-line stores; the pre-activations too when the backward needs them ----
+    constexpr int AS = NPAD / 2 + kLdsChanPad, PS = NPAD + kLdsChanPad;
+    _Float16* s_act = smem;                                      // [256][AS]
+    _Float16* s_pre = smem + kConvTileH * kConvTileW * AS;       // [256][PS]
+    __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
     for (int m = 0; m < 4; ++m)
     {
-        const int y = y0 + 2 * wave + (m >> 1);
 #pragma unroll
         for (int j = 0; j < HB; ++j)
         {
@@ -165,22 +169,22 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
-                const int x = x0 + (m & 1) * 16 + (lane >> 4) * 4 + i;
-                if (y >= p.H || x >= p.W) continue;
+                const int tp  = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + (lane >> 4) * 4 + i;
                 const float f = acc[m][j][i] + bf, g = acc[m][HB + j][i] + bm;  // both 0 for padding channels
                 if (p.pre)
                 {
-                    _Float16* pr        = p.pre + ((size_t)y * p.W + x) * NPAD;
-                    pr[ch]              = _Float16(f);
-                    pr[NPAD / 2 + ch]   = _Float16(g);
+                    s_pre[tp * PS + ch]            = _Float16(f);
+                    s_pre[tp * PS + NPAD / 2 + ch] = _Float16(g);
                 }
-                if (ch >= p.cout_store) continue;
                 const float e = f > 0.f ? f : (__expf(f) - 1.f);
                 const float s = 1.f / (1.f + __expf(-g));
-                p.out[((size_t)y * p.W + x) * p.cout_store + ch] = ch < p.cout ? _Float16(e * s) : _Float16(0.f);
+                s_act[tp * AS + ch] = ch < p.cout ? _Float16(e * s) : _Float16(0.f);
             }
         }
     }
+    __syncthreads();
+    store_tile_nhwc(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
+    if (p.pre) store_tile_nhwc(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
 }
 
 // wpack[tap][n][c]: n < NPAD/2 feature output n, else mask output n - NPAD/2; zero outside the real ranges
@@ -251,7 +255,9 @@ template <int CIN, int NPAD>
 hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
 {
     constexpr int ROW  = CIN + kLdsChanPad;
-    const size_t lds   = (size_t)((kConvPatchH * kConvPatchW + kBelowH * kBelowW) * ROW) * sizeof(_Float16);  // 36 or 65 KB
+    const size_t lds_in  = (size_t)((kConvPatchH * kConvPatchW + kBelowH * kBelowW) * ROW) * sizeof(_Float16);  // 36 or 65 KB
+    const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NPAD / 2 + kLdsChanPad) + (p.pre ? NPAD + kLdsChanPad : 0)) * sizeof(_Float16);
+    const size_t lds     = std::max(lds_in, lds_out);  // up to 104 KB when the largest block saves its pre-activations
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
