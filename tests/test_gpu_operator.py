@@ -103,3 +103,27 @@ def test_unsupported_render_modes_raise():
     info.params.render_mode = 1
     with pytest.raises(NotImplementedError):
         BlendPointCloud(info)
+
+
+def test_unused_layers_and_extra_outputs(oracle):
+    """A consumer that reads only some pyramid layers leaves the others without a gradient; add_depth_to_network /
+    output_background_mask append L zero tensors each, as the reference's path does (PointRenderer.cu:482-505)."""
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=4, list_depth=16, seed=9)
+    ns = NeuralScene.from_arrays(sc, requires_grad=True)
+    info = _info(sc, ns, add_depth_to_network=True, output_background_mask=True)
+    outs = BlendPointCloud(info)
+    assert len(outs) == 12
+    for l in range(4):
+        assert outs[4 + l].shape == (1, 1) + outs[l].shape[2:] and float(outs[4 + l].abs().max()) == 0.0
+        assert outs[8 + l].shape == outs[4 + l].shape and float(outs[8 + l].abs().max()) == 0.0
+    rng = np.random.default_rng(1)
+    g0, g1 = [torch.as_tensor(rng.normal(0, 1, outs[l].shape).astype(np.float32)).cuda() for l in range(2)]
+    ((outs[0] * g0).sum() + (outs[1] * g1).sum()).backward()
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    grads = [g0.cpu().numpy(), g1.cpu().numpy()] + [np.zeros_like(ref["images"][l]) for l in (2, 3)]
+    g_ref = oracle.backward(sc, d, ref, grads)
+    from tests.gpu_util import rel_err
+    assert rel_err(ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
+    assert rel_err(ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"]) < 1e-4

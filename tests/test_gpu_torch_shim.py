@@ -144,3 +144,21 @@ def test_cpp_unet_forward_backward_matches_python_mirror():
         assert cpp_params[n].grad is not None, n
         # bias and 1x1 gradients are summed with float atomics: same values up to summation order
         assert torch.allclose(cpp_params[n].grad, q.grad, rtol=1e-4, atol=1e-7 * float(q.grad.abs().max())), n
+
+
+@pytest.mark.gpu
+def test_cpp_unused_layers_and_extra_outputs(oracle):
+    from tests.gpu_util import rel_err
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=4, list_depth=16, seed=9)
+    s, t = _session(sc)
+    views = [[v["w"], v["h"], v["image_index"], v["camera_index"]] for v in sc.views]
+    outs = s.blend_point_cloud(views, sc.num_layers, True, 0.0, 0, 16, True, True)
+    assert len(outs) == 12 and all(float(o.abs().max()) == 0.0 and o.shape[1] == 1 for o in outs[4:])
+    rng = np.random.default_rng(1)
+    g0 = rng.normal(0, 1, outs[0].shape).astype(np.float32)
+    (outs[0] * torch.as_tensor(g0).cuda()).sum().backward()  # layers 1..3 get no gradient
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    g_ref = oracle.backward(sc, d, ref, [g0] + [np.zeros_like(ref["images"][l]) for l in (1, 2, 3)])
+    assert rel_err(t["texture"].grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
+    assert rel_err(t["position"].grad.cpu().numpy(), g_ref["d_position"]) < 1e-4

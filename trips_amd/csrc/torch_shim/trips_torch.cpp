@@ -193,6 +193,14 @@ variable_list PointRender::forward(AutogradContext* ctx, Variable texture, Varia
     ctx->saved_data["trips_saved"] = IValue(s);
     if (!info->train)
         for (auto& im : images) im = im.permute({0, 3, 1, 2});  // PointRenderer.cu:747-749
+    // depth buffers, then background masks: allocated and zero in the reference's path too
+    auto zeros_like_layers = [&]()
+    {
+        for (int l = 0; l < d.num_layers; ++l)
+            images.push_back(torch::zeros({d.num_views, 1, lh[l], lw[l]}, torch::TensorOptions().dtype(torch::kFloat32).device(texture.device())));
+    };
+    if (info->params.add_depth_to_network) zeros_like_layers();
+    if (info->params.output_background_mask) zeros_like_layers();
     return images;
 }
 
@@ -221,8 +229,18 @@ variable_list PointRender::backward(AutogradContext* ctx, variable_list grad_out
     const float* gptr[TRIPS_MAX_LAYERS] = {};
     for (int l = 0; l < d.num_layers; ++l)
     {
-        TORCH_CHECK(grad_output[l].defined() && grad_output[l].scalar_type() == torch::kFloat32, "image gradient ", l);
-        gi.push_back(grad_output[l].contiguous());
+        if (grad_output[l].defined())
+        {
+            TORCH_CHECK(grad_output[l].scalar_type() == torch::kFloat32, "image gradient ", l, " must be float32");
+            gi.push_back(grad_output[l].contiguous());
+        }
+        else
+        {
+            // a layer nobody consumed (a net with fewer levels than the pyramid) arrives without a gradient
+            int32_t lw[TRIPS_MAX_LAYERS], lh[TRIPS_MAX_LAYERS];
+            check(trips_splat_layer_sizes(&d, lw, lh), "trips_splat_layer_sizes");
+            gi.push_back(torch::zeros({d.num_views, d.num_channels, lh[l], lw[l]}, torch::TensorOptions().dtype(torch::kFloat32).device(dev)));
+        }
         gptr[l] = gi.back().data_ptr<float>();
     }
     TripsSplatGrads g{};

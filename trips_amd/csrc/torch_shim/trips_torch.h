@@ -45,6 +45,11 @@ struct RenderParams
     bool combine_lists                          = false;
     bool render_points_in_all_lower_resolutions = true;
     bool normalize_grads                        = false;
+    // The path implemented here never writes these two outputs in the reference either (RenderForward.cu:43 keeps
+    // blend_out commented out, no kernel of the new path takes the depth buffers): they come back as zeros, after
+    // the L images, so that the output arity matches (PointRenderer.cu:482-505,1183-1190)
+    bool add_depth_to_network   = false;
+    bool output_background_mask = false;
     // not in the reference
     int background_mode     = TRIPS_BG_REFERENCE;
     int max_pixels_per_list = 16;  // PointRenderer.h:178

@@ -15,7 +15,8 @@ struct Session
 };
 
 std::vector<torch::Tensor> blend_point_cloud(Session& s, std::vector<std::vector<double>> views, int num_layers, bool train,
-                                             double dropout, int background_mode, int list_depth)
+                                             double dropout, int background_mode, int list_depth, bool add_depth,
+                                             bool background_mask)
 {
     NeuralRenderInfo info;
     info.scene      = &s.scene;
@@ -26,6 +27,8 @@ std::vector<torch::Tensor> blend_point_cloud(Session& s, std::vector<std::vector
     info.params.drop_out_points_by_radius = false;
     info.params.background_mode           = background_mode;
     info.params.max_pixels_per_list       = list_depth;
+    info.params.add_depth_to_network      = add_depth;
+    info.params.output_background_mask    = background_mask;
     info.params.num_texture_channels      = (int)s.scene.texture->texture.size(0);
     for (auto& v : views)
     {
@@ -176,7 +179,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                  s.scene.intrinsics->intrinsics             = intrinsics;
              })
         .def("blend_point_cloud", &blend_point_cloud, py::arg("views"), py::arg("num_layers"), py::arg("train") = true,
-             py::arg("dropout") = 0.0, py::arg("background_mode") = 0, py::arg("list_depth") = 16)
+             py::arg("dropout") = 0.0, py::arg("background_mode") = 0, py::arg("list_depth") = 16,
+             py::arg("add_depth_to_network") = false, py::arg("output_background_mask") = false)
         .def("apply_tangent", [](Session& s) { s.scene.poses->ApplyTangent(); })
         .def("make_adam",
              [](Session& s, std::vector<torch::Tensor> params, double lr)

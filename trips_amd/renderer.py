@@ -210,6 +210,10 @@ class RenderParams:
     combine_lists: bool = False
     render_points_in_all_lower_resolutions: bool = True
     normalize_grads: bool = False
+    # never written by the reference's kernels on this path either (RenderForward.cu:43): returned as zeros after
+    # the L images so that the output arity matches (PointRenderer.cu:482-505,1183-1190)
+    add_depth_to_network: bool = False
+    output_background_mask: bool = False
     # not in the reference: see TRIPS_BG_* in include/trips_splat.h; list depth is fixed to 16 there
     background_mode: int = abi.TRIPS_BG_REFERENCE
     max_pixels_per_list: int = 16
@@ -300,9 +304,15 @@ class PointRender(torch.autograd.Function):
         ctx.saved_state = saved
         ctx.shapes = dict(points=points.shape, layer=layer_value_of_point.shape, confidence=confidence.shape,
                           pose=pose_tangents.shape)
+        ctx.image_shapes = [tuple(im.shape) for im in images]
         if not info.train:
             images = [im.permute(0, 3, 1, 2) for im in images]  # PointRenderer.cu:747-749
-        return tuple(images)
+        extra = []
+        for flag in (info.params.add_depth_to_network, info.params.output_background_mask):
+            if flag:
+                extra += [torch.zeros((im.shape[0], 1, im.shape[2], im.shape[3]), dtype=torch.float32, device=im.device)
+                          for im in images]
+        return tuple(images) + tuple(extra)
 
     @staticmethod
     def backward(ctx, *grad_output):
@@ -321,7 +331,9 @@ class PointRender(torch.autograd.Function):
             d_pose=torch.zeros((desc.num_images, 6), dtype=torch.float64, device=dev) if need[3] else None,
             d_intrinsics=torch.zeros_like(t["intrinsics"]) if need[4] else None,
         )
-        gi = [g.contiguous() for g in grad_output[:desc.num_layers]]
+        # a layer nobody consumed (a net with fewer levels than the pyramid) arrives without a gradient
+        gi = [g.contiguous() if g is not None else torch.zeros(shape, dtype=torch.float32, device=dev)
+              for g, shape in zip(grad_output[:desc.num_layers], ctx.image_shapes)]
         tin = SplatContext.make_in(**t)
         sctx.backward(desc, tin, ctx.saved_state, gi, grads, info.cache.workspace if info.cache else None)
         d_layer = grads["d_point_size"].reshape(ctx.shapes["layer"]) if need[7] else None
