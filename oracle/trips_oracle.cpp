@@ -906,8 +906,11 @@ int oracle_adam_step(const TripsAdamTensor* tensors, int n_tensors)
             float first_moment        = T.first_moment[i] = T.beta1 * T.first_moment[i] + (1 - T.beta1) * gradient;
             const float second_moment = T.second_moment[i] =
                 T.beta2 * T.second_moment[i] + (1 - T.beta2) * gradient_sq;
-            T.steps[i]                  = T.steps[i] + 1;
-            const uint32_t current_step = (uint32_t)T.steps[i];
+            uint32_t current_step;
+            if (T.steps_dtype == TRIPS_STEPS_I32)
+                current_step = (uint32_t)(((int32_t*)T.steps)[i] += 1);
+            else
+                current_step = (uint32_t)(((int64_t*)T.steps)[i] += 1);
             float learning_rate         = T.lr;
             learning_rate *= std::sqrt(1 - std::pow(T.beta2, (float)current_step)) /
                              (1 - std::pow(T.beta1, (float)current_step));

@@ -209,6 +209,7 @@ def fill_adam_tensor(dst, t, addr):
     dst.lower_lr_bound = t.get("lower_lr_bound", 0.0)
     dst.upper_lr_bound = t.get("upper_lr_bound", abi.FLT_MAX)
     dst.loss_scale = t.get("loss_scale", 1.0)
+    dst.steps_dtype = int(t.get("steps_dtype", abi.TRIPS_STEPS_I64))
 
 
 _cached = None

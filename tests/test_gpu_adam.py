@@ -26,6 +26,11 @@ def test_fused_adam_matches_oracle(oracle):
              _mk(4 * 6001 + 3, rng, lr=1e-2, absolute_weight_decay=0.01, weight_clipping_magnitude=1.5),
              _mk(6001, rng, lr=1e-3, lower_lr_bound=0.0, upper_lr_bound=0.02),
              _mk(37 * 6, rng, dtype=np.float64, lr=1e-4, zero_frac=0.0), _mk(1, rng), _mk(0, rng)]
+    # the same with 32-bit step counters
+    for extra in (_mk(6001 * 4, rng, lr=1e-3), _mk(4 * 6001 + 3, rng, lr=2e-3), _mk(50, rng, dtype=np.float64)):
+        extra["steps"] = np.zeros(extra["n"], np.int32)
+        extra["steps_dtype"] = abi.TRIPS_STEPS_I32
+        specs.append(extra)
     dev = ctx.device
     gpu = []
     for s in specs:

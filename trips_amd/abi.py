@@ -8,6 +8,7 @@ import ctypes as C
 TRIPS_MAX_LAYERS = 8
 TRIPS_MAX_VIEWS = 16
 TRIPS_ABI_VERSION = 1
+TRIPS_STEPS_I64, TRIPS_STEPS_I32 = 0, 1
 TRIPS_PROFILE_MAX_KERNELS = 32
 TRIPS_UNET_MAX_LEVELS = 8
 
@@ -115,6 +116,7 @@ class TripsAdamTensor(C.Structure):
         ("lower_lr_bound", C.c_float),
         ("upper_lr_bound", C.c_float),
         ("loss_scale", C.c_float),
+        ("steps_dtype", C.c_int32),
     ]
 
 

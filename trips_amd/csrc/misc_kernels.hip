@@ -57,18 +57,18 @@ __device__ __forceinline__ bool adam_element(const AdamScalars& h, float gradien
     return true;
 }
 
-__global__ __launch_bounds__(256) void adam_fused_kernel(const AdamTable tab)
+// STEP = long long (the reference's state tensor) or int
+template <typename STEP>
+__device__ __forceinline__ void adam_block(const AdamTable& tab, int ti)
 {
-    int ti = 0;
-    while (ti + 1 < tab.n && (long long)blockIdx.x >= tab.block_start[ti + 1]) ++ti;
     const TripsAdamTensor& T = tab.t[ti];
     const AdamScalars h      = {T.lr, T.beta1, T.beta2, T.eps, T.relative_weight_decay, T.absolute_weight_decay,
                                 T.weight_clipping_magnitude, T.lower_lr_bound, T.upper_lr_bound, T.loss_scale};
     const long long i0 = ((long long)blockIdx.x - tab.block_start[ti]) * kAdamPerBlock + (long long)threadIdx.x * 4;
     if (i0 >= T.n) return;
-    float* mo      = T.first_moment;
-    float* vo      = T.second_moment;
-    long long* st  = reinterpret_cast<long long*>(T.steps);
+    float* mo = T.first_moment;
+    float* vo = T.second_moment;
+    STEP* st  = reinterpret_cast<STEP*>(T.steps);
 
     if (T.dtype == TRIPS_DTYPE_F32 && tab.vec_ok[ti] && i0 + 4 <= T.n)
     {
@@ -79,18 +79,31 @@ __global__ __launch_bounds__(256) void adam_fused_kernel(const AdamTable tab)
         float4 w4 = *reinterpret_cast<const float4*>(w + i0);
         float4 m4 = *reinterpret_cast<const float4*>(mo + i0);
         float4 v4 = *reinterpret_cast<const float4*>(vo + i0);
-        longlong2 s01 = *reinterpret_cast<const longlong2*>(st + i0);
-        longlong2 s23 = *reinterpret_cast<const longlong2*>(st + i0 + 2);
+        STEP s[4];
+        if (sizeof(STEP) == 8)
+        {
+            *reinterpret_cast<longlong2*>(&s[0]) = *reinterpret_cast<const longlong2*>(st + i0);
+            *reinterpret_cast<longlong2*>(&s[2]) = *reinterpret_cast<const longlong2*>(st + i0 + 2);
+        }
+        else
+            *reinterpret_cast<int4*>(&s[0]) = *reinterpret_cast<const int4*>(st + i0);
+        long long s0 = s[0], s1 = s[1], s2 = s[2], s3 = s[3];
         float nw;
-        if (adam_element(h, g4.x, w4.x, m4.x, v4.x, s01.x, nw)) w4.x = nw;
-        if (adam_element(h, g4.y, w4.y, m4.y, v4.y, s01.y, nw)) w4.y = nw;
-        if (adam_element(h, g4.z, w4.z, m4.z, v4.z, s23.x, nw)) w4.z = nw;
-        if (adam_element(h, g4.w, w4.w, m4.w, v4.w, s23.y, nw)) w4.w = nw;
-        *reinterpret_cast<float4*>(w + i0)        = w4;
-        *reinterpret_cast<float4*>(mo + i0)       = m4;
-        *reinterpret_cast<float4*>(vo + i0)       = v4;
-        *reinterpret_cast<longlong2*>(st + i0)     = s01;
-        *reinterpret_cast<longlong2*>(st + i0 + 2) = s23;
+        if (adam_element(h, g4.x, w4.x, m4.x, v4.x, s0, nw)) w4.x = nw;
+        if (adam_element(h, g4.y, w4.y, m4.y, v4.y, s1, nw)) w4.y = nw;
+        if (adam_element(h, g4.z, w4.z, m4.z, v4.z, s2, nw)) w4.z = nw;
+        if (adam_element(h, g4.w, w4.w, m4.w, v4.w, s3, nw)) w4.w = nw;
+        s[0] = (STEP)s0, s[1] = (STEP)s1, s[2] = (STEP)s2, s[3] = (STEP)s3;
+        *reinterpret_cast<float4*>(w + i0)  = w4;
+        *reinterpret_cast<float4*>(mo + i0) = m4;
+        *reinterpret_cast<float4*>(vo + i0) = v4;
+        if (sizeof(STEP) == 8)
+        {
+            *reinterpret_cast<longlong2*>(st + i0)     = *reinterpret_cast<longlong2*>(&s[0]);
+            *reinterpret_cast<longlong2*>(st + i0 + 2) = *reinterpret_cast<longlong2*>(&s[2]);
+        }
+        else
+            *reinterpret_cast<int4*>(st + i0) = *reinterpret_cast<int4*>(&s[0]);
         return;
     }
     for (int k = 0; k < 4; ++k)
@@ -114,13 +127,23 @@ __global__ __launch_bounds__(256) void adam_fused_kernel(const AdamTable tab)
         {
             mo[i] = m;
             vo[i] = v;
-            st[i] = s;
+            st[i] = (STEP)s;
             if (T.dtype == TRIPS_DTYPE_F64)
                 reinterpret_cast<double*>(T.weights)[i] = nw;
             else
                 reinterpret_cast<float*>(T.weights)[i] = nw;
         }
     }
+}
+
+__global__ __launch_bounds__(256) void adam_fused_kernel(const AdamTable tab)
+{
+    int ti = 0;
+    while (ti + 1 < tab.n && (long long)blockIdx.x >= tab.block_start[ti + 1]) ++ti;
+    if (tab.t[ti].steps_dtype == TRIPS_STEPS_I32)
+        adam_block<int>(tab, ti);
+    else
+        adam_block<long long>(tab, ti);
 }
 
 hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_t stream, Profiler* prof)

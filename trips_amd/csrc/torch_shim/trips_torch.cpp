@@ -325,7 +325,7 @@ torch::Tensor MyAdam::step(LossClosure closure)
             if (it == state_.end())
             {
                 auto st = std::make_unique<MyAdamParamState>();
-                st->param_steps(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kInt64));
+                st->param_steps(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kInt32));
                 st->first_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
                 st->second_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
                 st->current_step(0);
@@ -348,7 +348,8 @@ torch::Tensor MyAdam::step(LossClosure closure)
             t.grads                     = g.data_ptr();
             t.first_moment              = st.first_moments().data_ptr<float>();
             t.second_moment             = st.second_moments().data_ptr<float>();
-            t.steps                     = st.param_steps().data_ptr<int64_t>();
+            t.steps                     = st.param_steps().data_ptr();
+            t.steps_dtype               = st.param_steps().scalar_type() == torch::kInt32 ? TRIPS_STEPS_I32 : TRIPS_STEPS_I64;
             t.n                         = p.numel();
             t.dtype                     = p.scalar_type() == torch::kDouble ? TRIPS_DTYPE_F64 : TRIPS_DTYPE_F32;
             t.lr                        = (float)options.lr();

@@ -578,6 +578,8 @@ int trips_adam_step_fused(TripsCtx* ctx, const TripsAdamTensor* tensors, int n_t
         if (t.dtype != TRIPS_DTYPE_F32 && t.dtype != TRIPS_DTYPE_F64)
             return fail(TRIPS_ERR_UNSUPPORTED, "tensor %d: dtype %d", i, t.dtype);
         if (!(t.loss_scale != 0.f)) return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: loss_scale is 0", i);
+        if (t.steps_dtype != TRIPS_STEPS_I64 && t.steps_dtype != TRIPS_STEPS_I32)
+            return fail(TRIPS_ERR_UNSUPPORTED, "tensor %d: steps_dtype %d", i, t.steps_dtype);
     }
     hipError_t e = launch_adam(tensors, n_tensors, reinterpret_cast<hipStream_t>(stream_), ctx->prof.enabled ? &ctx->prof : nullptr);
     if (e != hipSuccess) return hip_fail(e, "adam launch");
