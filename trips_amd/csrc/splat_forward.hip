@@ -239,28 +239,49 @@ __global__ __launch_bounds__(1024) void small_scan_kernel(const int32_t* __restr
 
 // ---------------------------------------------------------------------------------------------------------
 // Column-wise exclusive prefix of the histogram matrix [workgroup][bin]: afterwards hist[g][bin] = entries of
-// `bin` that come from workgroups before g, and bin_count[bin] = the column total. One thread per bin (rows are
-// read coalesced); no atomics anywhere in the binning, since atomics on a few thousand hot counters serialise.
+// `bin` that come from workgroups before g, and bin_count[bin] = the column total. No atomics anywhere in the
+// binning, since atomics on a few thousand hot counters serialise. A workgroup owns 16 columns; its 16 row
+// segments are summed side by side, prefixed through LDS, then each segment writes its rows' prefixes (one thread
+// walking a whole column is a chain of G dependent-latency steps).
+constexpr int kScanCols = 16, kScanSegs = 16;
 __global__ __launch_bounds__(256) void bin_column_scan_kernel(int32_t* __restrict__ hist, int32_t* __restrict__ bin_count,
                                                               int NB, int G)
 {
-    const int bin = blockIdx.x * 256 + threadIdx.x;
-    if (bin >= NB) return;
+    __shared__ int s_seg[kScanSegs][kScanCols];
+    const int c = threadIdx.x % kScanCols, seg = threadIdx.x / kScanCols;
+    const int bin = blockIdx.x * kScanCols + c;
+    const int rows = (G + kScanSegs - 1) / kScanSegs;
+    const int g0 = seg * rows, g1 = min(G, g0 + rows);
+    const bool live = bin < NB;
+    int32_t* col    = hist + bin;
+    int sum         = 0;
+    if (live)
+        for (int g = g0; g < g1; g += 8)
+        {
+            int v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = (g + k < g1) ? col[(size_t)(g + k) * NB] : 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) sum += v[k];
+        }
+    s_seg[seg][c] = sum;
+    __syncthreads();
     int run = 0;
-    int32_t* col = hist + bin;
-    for (int g = 0; g < G; g += 8)
+    for (int k = 0; k < seg; ++k) run += s_seg[k][c];
+    if (!live) return;
+    for (int g = g0; g < g1; g += 8)
     {
         int v[8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = (g + k < G) ? col[(size_t)(g + k) * NB] : 0;
+        for (int k = 0; k < 8; ++k) v[k] = (g + k < g1) ? col[(size_t)(g + k) * NB] : 0;
 #pragma unroll
         for (int k = 0; k < 8; ++k)
         {
-            if (g + k < G) col[(size_t)(g + k) * NB] = run;
+            if (g + k < g1) col[(size_t)(g + k) * NB] = run;
             run += v[k];
         }
     }
-    bin_count[bin] = run;
+    if (seg == kScanSegs - 1) bin_count[bin] = run;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -628,7 +649,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     }
     {
         ProfScope ps(prof, "bin_scan", stream);
-        hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + 255) / 256), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
+        hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + kScanCols - 1) / kScanCols), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
         hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_count, p.bin_start,
                            (int32_t*)nullptr, NB, (unsigned long long*)nullptr);
     }
