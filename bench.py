@@ -29,15 +29,15 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (131589, 407187),
-    "bin_scatter": (50029, 203344),
-    "tile_count": (51795, 11061),
-    "tile_scatter": (57559, 511718),
-    "sort_blend": (358645, 240802),
-    "fill_rank": (10, 187500),
-    "backward_pixels": (525044, 647669),
-    "backward_points": (1405460, 566754),
-    "adam_fused": (688600, 912211),
+    "project_bin": (132310, 407399),
+    "bin_scatter": (50074, 203361),
+    "tile_count": (51807, 11061),
+    "tile_scatter": (57591, 512632),
+    "sort_blend": (359430, 240809),
+    "fill_rank": (13, 187500),
+    "backward_pixels": (525426, 648202),
+    "backward_points": (1407066, 567129),
+    "adam_fused": (582978, 792823),
 }
 
 

@@ -115,8 +115,8 @@ def test_unused_layers_and_extra_outputs(oracle):
     outs = BlendPointCloud(info)
     assert len(outs) == 12
     for l in range(4):
-        assert outs[4 + l].shape == (1, 1) + outs[l].shape[2:] and float(outs[4 + l].abs().max()) == 0.0
-        assert outs[8 + l].shape == outs[4 + l].shape and float(outs[8 + l].abs().max()) == 0.0
+        assert outs[4 + l].shape == (1, 1) + outs[l].shape[2:] and float(outs[4 + l].detach().abs().max()) == 0.0
+        assert outs[8 + l].shape == outs[4 + l].shape and float(outs[8 + l].detach().abs().max()) == 0.0
     rng = np.random.default_rng(1)
     g0, g1 = [torch.as_tensor(rng.normal(0, 1, outs[l].shape).astype(np.float32)).cuda() for l in range(2)]
     ((outs[0] * g0).sum() + (outs[1] * g1).sum()).backward()
