@@ -108,6 +108,44 @@ __device__ __forceinline__ u64 row_merge16(u64 v)
     return v;
 }
 
+// ---- the same row split into two independent lists of 8 lanes (two short pixel lists per DPP row) ----
+// final merge stage of an ascending sort of 8: every 8-lane group ascends, so position i keeps the larger key
+// when its bit J is set
+template <int J>
+__device__ __forceinline__ u64 bitonic_step_half_ascending(u64 v)
+{
+    static_assert(J == 1 || J == 2 || J == 4, "inside 8 lanes");
+    const u64 o = row_xor_u64<J>(v);
+    unsigned m  = 0;
+    for (int i = 0; i < 16; ++i)
+        if (i & J) m |= 1u << i;
+    const u64 kMax  = rows4(m);
+    const u64 lt    = __builtin_amdgcn_ballot_w64(o < v);
+    const bool take = __builtin_amdgcn_inverse_ballot_w64(lt ^ kMax);
+    return take ? o : v;
+}
+
+// ascending sort of the 8 keys of each half row (the 2- and 4-stages of the sort of 16 already treat the halves alike)
+__device__ __forceinline__ u64 half_sort8(u64 v)
+{
+    v = bitonic_step<2, 1>(v);
+    v = bitonic_step<4, 2>(v);
+    v = bitonic_step<4, 1>(v);
+    v = bitonic_step_half_ascending<4>(v);
+    v = bitonic_step_half_ascending<2>(v);
+    v = bitonic_step_half_ascending<1>(v);
+    return v;
+}
+
+// sum over each half row, valid in its lane 0; same pairing as row_sum_to_lane0 without the last step
+__device__ __forceinline__ float half_sum_to_lane0(float v)
+{
+    v = v + dpp_f<kDppXor1>(v);
+    v = v + dpp_f<kDppXor2>(v);
+    v = v + dpp_f<kDppHalfMirror>(v);
+    return v;
+}
+
 // lane i reads lane i-1 of the row; lane 0 of the row reads `fill`
 __device__ __forceinline__ float row_shr1(float v, float fill)
 {
@@ -142,6 +180,22 @@ __device__ __forceinline__ float row_exclusive_product(float f, int steps)
     {
         pre = row_shr1(pre * f, 1.f);
         T   = __builtin_amdgcn_inverse_ballot_w64(latch) ? pre : T;  // position s latches its product
+        latch <<= 1;
+    }
+    return T;
+}
+
+// the same per half row (steps 1..8): positions 0 and 8 of a row start a chain
+__device__ __forceinline__ float half_exclusive_product(float f, int steps)
+{
+    float pre = 1.f, T = 1.f;
+    u64 latch = rows4((1u << 1) | (1u << 9));
+    constexpr u64 kFirst = rows4(0x0101u);
+    for (int s = 1; s < steps; ++s)
+    {
+        pre = row_shr1(pre * f, 1.f);
+        pre = __builtin_amdgcn_inverse_ballot_w64(kFirst) ? 1.f : pre;  // position 8 must not see position 7
+        T   = __builtin_amdgcn_inverse_ballot_w64(latch) ? pre : T;
         latch <<= 1;
     }
     return T;

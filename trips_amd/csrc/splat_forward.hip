@@ -465,22 +465,22 @@ __device__ __forceinline__ u64 shfl16(u64 v, int src)
     return ((u64)hi << 32) | lo;
 }
 
-// Top-16 of each pixel list by key, then the alpha blend. One wavefront = four pixels, 16 lanes each.
-template <int C, bool TRAIN>
-__global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
+// Top-16 of each pixel list by key, then the alpha blend, for 64 / ROW consecutive pixels starting at `pix_first`:
+// ROW = 16 lanes per pixel (one DPP row; lists of any length stream through in chunks of 16), or ROW = 8 when no
+// list of the group is longer than 8 (two thirds of the pixels of a typical view have at most 4 entries: half the
+// lanes of a 16-lane row would idle through every instruction).
+template <int C, bool TRAIN, int ROW>
+__device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long long pix_first, bool group_in_range)
 {
     constexpr int CPAD = (C + 3) & ~3;
     const int lane     = threadIdx.x & 63;
-    const int sub      = lane & 15;
-    const int grp      = lane >> 4;
+    const int sub      = lane & (ROW - 1);
+    const int grp      = lane / ROW;
     const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
-    const long long nblocks     = ((long long)P + 15) / 16;  // 16 pixels per workgroup, 64 workgroups per tile
-    const long long lblock      = xcd_tile_block(blockIdx.x, kTilePixels / 16);
-    const long long wave_global = lblock * 4 + (threadIdx.x >> 6);
-    const long long pix_ll      = wave_global * 4 + grp;
-    const bool in_range         = pix_ll < P && lblock < nblocks;
-    const int pix               = in_range ? (int)pix_ll : 0;
+    const long long pix_ll = pix_first + grp;
+    const bool in_range    = pix_ll < P && group_in_range;
+    const int pix          = in_range ? (int)pix_ll : 0;
     int layer, gx, gy;
     const bool live = pix_decode(p.geom, pix, layer, gx, gy) && in_range;  // false for the padding of partial tiles
 
@@ -495,13 +495,19 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     int readable = len;
     if (start + len > p.capacity) readable = (int)max(0ll, p.capacity - start);
 
+    const u64 kInf = ~0ull;
+    u64 best       = kInf;
+    if (ROW == 8)
+    {
+        if (sub < readable) best = p.keys[start + sub];
+        best = half_sort8(best);
+    }
+    else
+    {
     int maxlen = readable;
     maxlen     = max(maxlen, __shfl_xor(maxlen, 16));
     maxlen     = max(maxlen, __shfl_xor(maxlen, 32));
-
-    const u64 kInf      = ~0ull;
-    const u64 grp_mask  = 0xFFFFull << (grp * 16);
-    u64 best            = kInf;
+    const u64 grp_mask = 0xFFFFull << (grp * 16);
     for (int base = 0; base < maxlen; base += 16)
     {
         u64 k = kInf;
@@ -522,6 +528,7 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
                 best        = row_merge16(best);
             }
         }
+    }
     }
 
     // ---- blend (RenderForward.cu:820-1048) ----
@@ -559,25 +566,26 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     // exclusive transmittance: lane j latches prod_{k<j} (1 - a_k), built left to right
     // only the first n positions of a row matter; n <= K
     int nmax = n;
+    if (ROW == 8) nmax = max(nmax, __shfl_xor(nmax, 8));
     nmax     = max(nmax, __shfl_xor(nmax, 16));
     nmax     = max(nmax, __shfl_xor(nmax, 32));
     nmax     = __builtin_amdgcn_readfirstlane(nmax);
-    const float T     = row_exclusive_product(1.f - a, nmax);
+    const float T     = ROW == 8 ? half_exclusive_product(1.f - a, nmax) : row_exclusive_product(1.f - a, nmax);
     const float Tc    = (T >= kAlphaDestCutoff) ? T : 0.f;
     const bool kept   = has && Tc >= kAlphaDestCutoff;
-    const unsigned kb = (unsigned)((__ballot(kept) >> (grp * 16)) & 0xFFFFull);
-    const int ret     = __ffs(~kb) - 1;  // length of the leading run of kept entries (kb has at most 16 bits)
+    const unsigned kb = (unsigned)((__ballot(kept) >> (grp * ROW)) & ((1u << ROW) - 1u));
+    const int ret     = __ffs(~kb) - 1;  // length of the leading run of kept entries (kb has at most ROW bits)
 
     float col[C];
     const float wgt = has ? Tc * a : 0.f;
 #pragma unroll
     for (int c = 0; c < C; ++c) col[c] = wgt * desc[c];
 #pragma unroll
-    for (int c = 0; c < C; ++c) col[c] = row_sum_to_lane0(col[c]);
+    for (int c = 0; c < C; ++c) col[c] = ROW == 8 ? half_sum_to_lane0(col[c]) : row_sum_to_lane0(col[c]);
 
     // background weight (RenderForward.cu:1002-1022); empty list -> 1
     float bgw_lane = (p.background_mode == TRIPS_BG_REFERENCE) ? Tc : T * (1.f - a);
-    float bgw      = __shfl(bgw_lane, max(n - 1, 0), 16);
+    float bgw      = __shfl(bgw_lane, max(n - 1, 0), ROW);
     if (n == 0) bgw = 1.f;
 
     if (live && sub == 0)
@@ -611,8 +619,47 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
             p.lengths[pix]  = live ? len : 0;
         }
         if (sub < K) p.lists[(size_t)pix * K + sub] = has ? pid : -1;
+        if (ROW == 8 && sub + 8 < K) p.lists[(size_t)pix * K + sub + 8] = -1;
     }
 }
+
+// One wavefront = eight consecutive pixels: all at once in 8-lane rows when none of their lists is longer than 8,
+// else four and four in 16-lane rows.
+template <int C, bool TRAIN>
+__global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
+{
+    const int lane = threadIdx.x & 63;
+    const int P    = p.geom.bin_off[p.num_layers] * kTilePixels;
+    const long long nblocks     = ((long long)P + 31) / 32;  // 32 pixels per workgroup, 32 workgroups per tile
+    const long long lblock      = xcd_tile_block(blockIdx.x, kTilePixels / 32);
+    const long long pix_first   = (lblock * 4 + (threadIdx.x >> 6)) * 8;
+    const bool group_in_range   = lblock < nblocks;
+    // longest list of the eight pixels (lists that ran past the key storage count with what was written)
+    int len8 = 0;
+    if (lane < 8 && group_in_range && pix_first + lane < P)
+    {
+        const int pix = (int)(pix_first + lane);
+        int layer, gx, gy;
+        if (pix_decode(p.geom, pix, layer, gx, gy))
+        {
+            len8 = p.counts[pix];
+            const long long start = p.cursor[pix];
+            if (start + len8 > p.capacity) len8 = (int)max(0ll, p.capacity - start);
+        }
+    }
+    len8 = max(len8, __shfl_xor(len8, 1));
+    len8 = max(len8, __shfl_xor(len8, 2));
+    len8 = max(len8, __shfl_xor(len8, 4));
+    len8 = __builtin_amdgcn_readfirstlane(len8);
+    if (len8 <= 8)
+        sort_blend_rows<C, TRAIN, 8>(p, pix_first, group_in_range);
+    else
+    {
+        sort_blend_rows<C, TRAIN, 16>(p, pix_first, group_in_range);
+        sort_blend_rows<C, TRAIN, 16>(p, pix_first + 4, group_in_range);
+    }
+}
+
 
 // ---------------------------------------------------------------------------------------------------------
 // host-side launchers
@@ -673,7 +720,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     {
         ProfScope ps(prof, "sort_blend", stream);
         const long long tiles8 = (((long long)NB + kNumXcd - 1) / kNumXcd) * kNumXcd;  // tiles rounded up to 8
-        int blocks             = (int)(tiles8 * (kTilePixels / 16));
+        int blocks             = (int)(tiles8 * (kTilePixels / 32));
         if (train)
         {
             TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((sort_blend_kernel<CC, true>), dim3(blocks), dim3(256), 0, stream, p));
