@@ -102,6 +102,9 @@ typedef struct TripsSplatIn {
     const double* poses_se3;  /* [F,8]  qx qy qz qw tx ty tz pad, world->camera (NeuralStructure.cpp:20-35) */
     const float* intrinsics;  /* [Cam,13] fx fy cx cy s + 8 distortion (NeuralStructure.cpp:104-117) */
     const float* dropout;     /* [B,N] or NULL; a point with value 1 is skipped (RenderForward.cu:240-244) */
+    const float* displacement; /* [B,N,3] or NULL; view b renders xyz + displacement[b] (dynamic_refinement_t,
+                                  PointRenderer.cu:703-713, NeuralPointCloudCuda.h:260-270); no gradient is
+                                  returned for it, as in the reference (PointRenderer.cu:243-252 is compiled out) */
 } TripsSplatIn;
 
 typedef struct TripsSplatOut {

@@ -161,6 +161,26 @@ inline Pose load_pose(const double* p)
     return P;
 }
 
+// GetPointWoNormal (NeuralPointCloudCuda.h:240-273): xyz of the point, plus view b's displacement when the scene
+// optimises one (PointRenderer.cu:703-713); .w is the drop-out radius
+struct PointPos
+{
+    float v[4];
+    operator const float*() const { return v; }
+};
+inline PointPos load_point(const TripsSplatIn* in, int N, int b, int pid)
+{
+    PointPos p;
+    const float* src = in->position + 4 * int64_t(pid);
+    for (int k = 0; k < 4; ++k) p.v[k] = src[k];
+    if (in->displacement)
+    {
+        const float* dsp = in->displacement + (int64_t(b) * N + pid) * 3;
+        for (int k = 0; k < 3; ++k) p.v[k] += dsp[k];
+    }
+    return p;
+}
+
 // SE3f * point. Rotation as Eigen's QuaternionBase::_transformVector does it:
 //   uv = 2 * (q.vec x v);  v' = v + w * uv + q.vec x uv
 inline void transform_point(const Pose& V, const float p[3], float out[3])
@@ -505,8 +525,8 @@ int oracle_splat_forward(const TripsSplatDesc* desc, const TripsSplatIn* in, con
             }
             if (drop && drop[pid] == 1.f) continue;
             float size         = softplus(in->point_size[pid]);
-            const float* pos   = in->position + 4 * int64_t(pid);
-            float drop_radius  = pos[3];
+            const PointPos pos = load_point(in, N, b, pid);
+            float drop_radius  = pos.v[3];
             Projected pr       = project(V, intr, cam, d.dist_cutoff, pos);
             float z            = pr.z;
             float radius_px    = pr.scale * drop_radius / z;
@@ -715,8 +735,8 @@ int oracle_splat_backward(const TripsSplatDesc* desc, const TripsSplatIn* in, co
 #pragma omp parallel for schedule(static)
         for (int pid = 0; pid < N; ++pid)
         {
-            const float* pos = in->position + 4 * int64_t(pid);
-            Projected pr     = project(V, intr, cam, d.dist_cutoff, pos);
+            const PointPos pos = load_point(in, N, b, pid);
+            Projected pr       = project(V, intr, cam, d.dist_cutoff, pos);
             PointRec r;
             r.ipx       = pr.ipx;
             r.ipy       = pr.ipy;
@@ -829,7 +849,7 @@ int oracle_splat_backward(const TripsSplatDesc* desc, const TripsSplatIn* in, co
                     }
                     float grad_blend_single = confidence_val * lfac * grad_alpha;
                     float dR_dp[2]          = {J[2 * bi] * grad_blend_single, J[2 * bi + 1] * grad_blend_single};
-                    const float* pos        = in->position + 4 * int64_t(pid);
+                    const PointPos pos      = load_point(in, N, b, pid);
                     float g_point[3], g_pose[6], g_k[5], g_dis[8];
                     oracle_project_point_backward(pose, intr, &cam, d.dist_cutoff, pos, dR_dp, g_point, g_pose, g_k,
                                                   g_dis);

@@ -15,7 +15,8 @@ class GpuRun:
         self.t = dict(position=f(scene.position), point_size=f(scene.point_size), index=f(scene.index, torch.int32),
                       texture=f(scene.texture), confidence=f(scene.confidence), background=f(scene.background),
                       poses_se3=f(scene.poses_se3, torch.float64), intrinsics=f(scene.intrinsics),
-                      dropout=None if dropout is None else f(dropout))
+                      dropout=None if dropout is None else f(dropout),
+                      displacement=None if getattr(scene, "displacement", None) is None else f(scene.displacement))
         self.tin = SplatContext.make_in(**self.t)
         self.workspace = self.ctx.alloc_bytes(self.ctx.workspace_size(desc))
         self.saved = self.ctx.alloc_bytes(self.ctx.saved_size(desc)) if desc.train else None

@@ -97,6 +97,7 @@ class Oracle:
     # ---- full passes ----
     @staticmethod
     def _inputs(scene, dropout=None):
+        disp = getattr(scene, "displacement", None)
         arrs = dict(
             position=np.ascontiguousarray(scene.position, dtype=np.float32),
             point_size=np.ascontiguousarray(scene.point_size, dtype=np.float32),
@@ -107,6 +108,7 @@ class Oracle:
             poses_se3=np.ascontiguousarray(scene.poses_se3, dtype=np.float64),
             intrinsics=np.ascontiguousarray(scene.intrinsics, dtype=np.float32),
             dropout=None if dropout is None else np.ascontiguousarray(dropout, dtype=np.float32),
+            displacement=None if disp is None else np.ascontiguousarray(disp, dtype=np.float32),
         )
         tin = abi.TripsSplatIn()
         for k, v in arrs.items():

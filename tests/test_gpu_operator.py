@@ -127,3 +127,29 @@ def test_unused_layers_and_extra_outputs(oracle):
     from tests.gpu_util import rel_err
     assert rel_err(ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
     assert rel_err(ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"]) < 1e-4
+
+
+def test_dynamic_refinement_displaces_points_per_view(oracle):
+    """A [B,N,3] dynamic_refinement_t moves the points of view b; the [1] dummy does nothing; no gradient comes back
+    for it (the reference never allocates one, PointRenderer.cu:243-252)."""
+    from tests.gpu_util import rel_err
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=43, views=2)
+    sc.displacement = np.random.default_rng(6).normal(0, 0.05, (2, 3000, 3)).astype(np.float32)
+    ns = NeuralScene.from_arrays(sc, requires_grad=True)
+    ns.dynamic_refinement_t = torch.as_tensor(sc.displacement).cuda().requires_grad_(True)
+    outs = BlendPointCloud(_info(sc, ns))
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    for a, b in zip(outs, ref["images"]):
+        np.testing.assert_allclose(a.detach().cpu().numpy(), b, rtol=1e-5, atol=1e-6)
+    rng = np.random.default_rng(0)
+    grads = [rng.normal(0, 1, o.shape).astype(np.float32) for o in outs]
+    sum((o * torch.as_tensor(g).cuda()).sum() for o, g in zip(outs, grads)).backward()
+    g_ref = oracle.backward(sc, d, ref, grads)
+    assert rel_err(ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"]) < 1e-4
+    assert rel_err(ns.poses.tangent_poses.grad.cpu().numpy(), g_ref["d_pose"]) < 1e-4
+    assert ns.dynamic_refinement_t.grad is None
+    ns.dynamic_refinement_t = torch.zeros((2, 5, 3), device="cuda")
+    with pytest.raises(ValueError):
+        BlendPointCloud(_info(sc, ns))

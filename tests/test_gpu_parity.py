@@ -153,6 +153,15 @@ def test_backward_views_crop_distortion_optional_outputs(oracle):
     _check_backward(oracle, sc, d, want_position=False, want_pose=False, want_intrinsics=False)
 
 
+def test_displacement_forward_backward(oracle):
+    """Per-view displacements of the point positions (dynamic_refinement_t, PointRenderer.cu:703-713)."""
+    sc = scenes.tiny(n=4000, w=70, h=50, f=60.0, num_layers=4, list_depth=16, seed=77, views=3, radius=(0.004, 0.4))
+    sc.displacement = np.random.default_rng(5).normal(0, 0.05, (3, 4000, 3)).astype(np.float32)
+    d = abi.desc_for_scene(sc)
+    _check_forward(oracle, sc, d)
+    _check_backward(oracle, sc, d)
+
+
 def test_config1_forward_full(oracle):
     sc = scenes.config1()
     _check_forward(oracle, sc, abi.desc_for_scene(sc, train=True))

@@ -162,3 +162,17 @@ def test_cpp_unused_layers_and_extra_outputs(oracle):
     g_ref = oracle.backward(sc, d, ref, [g0] + [np.zeros_like(ref["images"][l]) for l in (1, 2, 3)])
     assert rel_err(t["texture"].grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
     assert rel_err(t["position"].grad.cpu().numpy(), g_ref["d_position"]) < 1e-4
+
+
+@pytest.mark.gpu
+def test_cpp_dynamic_refinement(oracle):
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=44, views=2)
+    sc.displacement = np.random.default_rng(7).normal(0, 0.05, (2, 3000, 3)).astype(np.float32)
+    s, t = _session(sc, requires_grad=False)
+    s.set_dynamic_refinement(torch.as_tensor(sc.displacement).cuda())
+    views = [[v["w"], v["h"], v["image_index"], v["camera_index"]] for v in sc.views]
+    with torch.no_grad():
+        outs = s.blend_point_cloud(views, sc.num_layers, True, 0.0, 0, 16)
+    ref = oracle.forward(sc, abi.desc_for_scene(sc))
+    for a, b in zip(outs, ref["images"]):
+        np.testing.assert_allclose(a.cpu().numpy(), b, rtol=1e-5, atol=1e-6)

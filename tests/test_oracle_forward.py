@@ -243,6 +243,42 @@ def test_dropout_and_viewer_cull(oracle):
     np.testing.assert_array_equal(r_view["depth"][0][sc.confidence >= 0.5], r0["depth"][0][sc.confidence >= 0.5])
 
 
+def test_displacement_equals_moved_points_per_view(oracle):
+    """View b renders xyz + displacement[b] (NeuralPointCloudCuda.h:260-270): the same bits as a single-view render
+    of a cloud whose positions were moved beforehand, forward and backward."""
+    import copy
+    sc = scenes.tiny(n=600, w=40, h=30, f=38.0, num_layers=3, list_depth=16, seed=21, views=2)
+    rng = np.random.default_rng(2)
+    sc.displacement = rng.normal(0, 0.05, (2, 600, 3)).astype(np.float32)
+    d = abi.desc_for_scene(sc)
+    r = oracle.forward(sc, d)
+    grads = [rng.normal(0, 1, im.shape).astype(np.float32) for im in r["images"]]
+    g = oracle.backward(sc, d, r, grads)
+    d_pos = np.zeros_like(g["d_position"])
+    for b in range(2):
+        one = copy.copy(sc)
+        one.displacement = None
+        one.position = sc.position.copy()
+        one.position[:, :3] = sc.position[:, :3] + sc.displacement[b]
+        one.views = [sc.views[b]]
+        d1 = abi.desc_for_scene(one)
+        r1 = oracle.forward(one, d1)
+        for l in range(3):
+            np.testing.assert_array_equal(r["images"][l][b], r1["images"][l][0])
+        np.testing.assert_array_equal(r["lists"][b], r1["lists"][0])
+        g1 = oracle.backward(one, d1, r1, [x[b:b + 1] for x in grads])
+        d_pos += g1["d_position"]
+    assert np.abs(r["images"][0][0] - oracle.forward(_without_displacement(sc), d)["images"][0][0]).max() > 1e-3
+    np.testing.assert_allclose(g["d_position"], d_pos, rtol=1e-5, atol=1e-6 * np.abs(d_pos).max())
+
+
+def _without_displacement(sc):
+    import copy
+    out = copy.copy(sc)
+    out.displacement = None
+    return out
+
+
 def test_empty_scene_is_background(oracle):
     sc = scenes.tiny(n=4, w=16, h=12, f=30.0, num_layers=3, seed=8)
     sc.position[:, 2] = -100.0  # everything behind the camera

@@ -75,6 +75,7 @@ class TripsSplatIn(C.Structure):
         ("poses_se3", C.c_void_p),
         ("intrinsics", C.c_void_p),
         ("dropout", C.c_void_p),
+        ("displacement", C.c_void_p),
     ]
 
 

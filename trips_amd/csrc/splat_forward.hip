@@ -102,7 +102,14 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         }
         if (!skip)
         {
-            const float4 pos = p.position[pid];
+            float4 pos = p.position[pid];
+            if (p.displacement)
+            {
+                const float* dsp = p.displacement + (size_t)pid * 3;
+                pos.x += dsp[0];
+                pos.y += dsp[1];
+                pos.z += dsp[2];
+            }
             const float size = softplus(p.point_size[pid]);
             const Projected pr = project(cam, pos.x, pos.y, pos.z);
             const float z      = pr.z;

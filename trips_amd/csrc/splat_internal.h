@@ -210,6 +210,7 @@ struct ForwardParams
     const double* pose;      // 8 doubles of this view's image
     const float* intrinsics; // 13 floats of this view's camera
     const float* dropout;    // this view's row or nullptr
+    const float* displacement;  // this view's [N,3] or nullptr
     // geometry
     PyramidGeom geom;
     TripsView view;

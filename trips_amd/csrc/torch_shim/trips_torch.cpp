@@ -92,6 +92,7 @@ struct SavedForBackward : public torch::CustomClassHolder
     TripsSplatDesc desc;
     torch::Tensor saved_state;
     torch::Tensor position, point_size, index, texture, confidence, background, poses_se3, intrinsics, dropout;
+    torch::Tensor displacement;  // [B,N,3] when the scene optimises per-view displacements
 };
 
 TripsSplatIn make_in(const SavedForBackward& s)
@@ -106,6 +107,7 @@ TripsSplatIn make_in(const SavedForBackward& s)
     in.poses_se3  = s.poses_se3.data_ptr<double>();
     in.intrinsics = s.intrinsics.data_ptr<float>();
     in.dropout    = s.dropout.defined() ? s.dropout.data_ptr<float>() : nullptr;
+    in.displacement = s.displacement.defined() ? s.displacement.data_ptr<float>() : nullptr;
     return in;
 }
 }  // namespace
@@ -146,7 +148,6 @@ variable_list PointRender::forward(AutogradContext* ctx, Variable texture, Varia
                                    Variable pose_tangents, Variable intrinsics, Variable confidence,
                                    Variable dynamic_refinement, Variable layer_of_point, IValue info_v)
 {
-    (void)dynamic_refinement;
     ctx->saved_data["render_info"] = info_v;
     NeuralRenderInfo* info         = info_v.toCustomClass<NeuralRenderInfo>().get();
     TORCH_CHECK(info->cache, "NeuralRenderInfo::cache is null");
@@ -166,6 +167,13 @@ variable_list PointRender::forward(AutogradContext* ctx, Variable texture, Varia
                     pose_tangents.scalar_type() == torch::kFloat64,
                 "t_index must be int32, poses_se3 / tangent_poses float64");
     const TripsSplatDesc& d = s->desc;
+    if (dynamic_refinement.defined() && dynamic_refinement.dim() > 1)  // a [1] dummy otherwise, PointRenderer.cu:705-706
+    {
+        TORCH_CHECK(dynamic_refinement.dim() == 3 && dynamic_refinement.size(0) == d.num_views &&
+                        dynamic_refinement.size(1) == d.num_points && dynamic_refinement.size(2) == 3,
+                    "dynamic_refinement must be [views, points, 3]");
+        s->displacement = dynamic_refinement.detach().to(torch::kFloat32).contiguous();
+    }
 
     size_t ws_bytes = 0, saved_bytes = 0;
     check(trips_splat_workspace_size(&d, &ws_bytes), "trips_splat_workspace_size");

@@ -178,6 +178,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                  s.scene.poses->tangent_poses               = tangent_poses;
                  s.scene.intrinsics->intrinsics             = intrinsics;
              })
+        .def("set_dynamic_refinement", [](Session& s, torch::Tensor t) { s.scene.dynamic_refinement_t = t; })
         .def("blend_point_cloud", &blend_point_cloud, py::arg("views"), py::arg("num_layers"), py::arg("train") = true,
              py::arg("dropout") = 0.0, py::arg("background_mode") = 0, py::arg("list_depth") = 16,
              py::arg("add_depth_to_network") = false, py::arg("output_background_mask") = false)

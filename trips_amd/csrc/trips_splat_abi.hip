@@ -361,6 +361,7 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
         p.pose       = in->poses_se3 + 8 * (size_t)d.views[b].image_index;
         p.intrinsics = in->intrinsics + 13 * (size_t)d.views[b].camera_index;
         p.dropout    = (train && in->dropout) ? in->dropout + (size_t)b * d.num_points : nullptr;
+        p.displacement = in->displacement ? in->displacement + (size_t)b * d.num_points * 3 : nullptr;
         p.geom       = g;
         p.view       = d.views[b];
         p.num_points = d.num_points;

@@ -75,7 +75,8 @@ class SplatContext:
 
     # ---- forward / backward ----
     @staticmethod
-    def make_in(position, point_size, index, texture, confidence, background, poses_se3, intrinsics, dropout=None):
+    def make_in(position, point_size, index, texture, confidence, background, poses_se3, intrinsics, dropout=None,
+                displacement=None):
         tin = abi.TripsSplatIn()
         tin.position = _ptr(position)
         tin.point_size = _ptr(point_size)
@@ -86,6 +87,7 @@ class SplatContext:
         tin.poses_se3 = _ptr(poses_se3)
         tin.intrinsics = _ptr(intrinsics)
         tin.dropout = _ptr(dropout)
+        tin.displacement = _ptr(displacement)
         return tin
 
     def forward(self, desc, tin, images, saved, workspace):
@@ -289,11 +291,17 @@ class PointRender(torch.autograd.Function):
             info.cache = PointRendererCache()
         cache = info.cache
         cache.build(sctx, desc, info.train, info.params.dropout if info.train else 0.0)
+        displacement = None
+        if dynamic_refinement is not None and dynamic_refinement.dim() > 1:  # a [1] dummy otherwise, PointRenderer.cu:705-706
+            if tuple(dynamic_refinement.shape) != (desc.num_views, desc.num_points, 3):
+                raise ValueError(f"dynamic_refinement: expected [{desc.num_views}, {desc.num_points}, 3], "
+                                 f"got {tuple(dynamic_refinement.shape)}")
+            displacement = dynamic_refinement.detach().to(torch.float32).contiguous()
         tensors = dict(position=points.contiguous(), point_size=layer_value_of_point.contiguous(),
                        index=sc.point_cloud_cuda.t_index.contiguous(), texture=texture.contiguous(),
                        confidence=confidence.contiguous(), background=background_color.contiguous(),
                        poses_se3=sc.poses.poses_se3.contiguous(), intrinsics=intrinsics.contiguous(),
-                       dropout=cache.dropout_points)
+                       dropout=cache.dropout_points, displacement=displacement)
         tin = SplatContext.make_in(**tensors)
         images = sctx.alloc_images(desc)
         saved = sctx.alloc_bytes(sctx.saved_size(desc)) if info.train else None
