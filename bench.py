@@ -68,6 +68,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--points", type=int, default=DEFAULT_POINTS)
+    ap.add_argument("--point-order", choices=("random", "morton_blocks"), default="random",
+                    help="memory order of the synthetic cloud: random (default, the workload the metric is quoted on) or "
+                         "the order the reference's scene preprocessing produces")
+    ap.add_argument("--no-order-variant", action="store_true",
+                    help="skip the second splat measurement with the points in the reference's preprocessing order")
     ap.add_argument("--cpu-steps", type=int, default=3, help="oracle steps for the cpu_baseline sample (0 = skip)")
     ap.add_argument("--no-net", action="store_true", help="skip the reconstruction-net forward that is reported beside the splat")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -89,57 +94,80 @@ def main():
         sys.exit(1)
     ctx = get_context(0)
     dev = ctx.device
-    sc = scenes.config3(n=args.points)
-    desc = abi.desc_for_scene(sc)
-    f = lambda a, dt=torch.float32: torch.as_tensor(np.ascontiguousarray(a), dtype=dt).to(dev).contiguous()
-    t = dict(position=f(sc.position), point_size=f(sc.point_size), index=f(sc.index, torch.int32),
-             texture=f(sc.texture), confidence=f(sc.confidence), background=f(sc.background),
-             poses_se3=f(sc.poses_se3, torch.float64), intrinsics=f(sc.intrinsics), dropout=None)
-    tin = SplatContext.make_in(**t)
-    workspace = ctx.alloc_bytes(ctx.workspace_size(desc))
-    saved = ctx.alloc_bytes(ctx.saved_size(desc))
-    images = ctx.alloc_images(desc)
-    sizes, _, P = abi.pyramid_pixels(desc)
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(1234)
-    grad_images = [torch.randn(im.shape, generator=gen, device=dev, dtype=torch.float32) for im in images]
+    def splat_run(order):
+        """Builds config 3 with the given memory order of the points and times warm-up + steps of the splat step."""
+        sc = scenes.config3(n=args.points, order=order)
+        desc = abi.desc_for_scene(sc)
+        f = lambda a, dt=torch.float32: torch.as_tensor(np.ascontiguousarray(a), dtype=dt).to(dev).contiguous()
+        t = dict(position=f(sc.position), point_size=f(sc.point_size), index=f(sc.index, torch.int32),
+                 texture=f(sc.texture), confidence=f(sc.confidence), background=f(sc.background),
+                 poses_se3=f(sc.poses_se3, torch.float64), intrinsics=f(sc.intrinsics), dropout=None)
+        tin = SplatContext.make_in(**t)
+        workspace = ctx.alloc_bytes(ctx.workspace_size(desc))
+        saved = ctx.alloc_bytes(ctx.saved_size(desc))
+        images = ctx.alloc_images(desc)
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(1234)
+        grad_images = [torch.randn(im.shape, generator=gen, device=dev, dtype=torch.float32) for im in images]
+        N, C = desc.num_points, desc.num_channels
+        grads = dict(d_texture=torch.zeros((C, N), device=dev), d_confidence=torch.zeros(N, device=dev),
+                     d_background=torch.zeros(C, device=dev), d_position=torch.zeros((N, 4), device=dev),
+                     d_point_size=torch.zeros(N, device=dev), d_pose=torch.zeros((1, 6), dtype=torch.float64, device=dev),
+                     d_intrinsics=torch.zeros((1, 13), device=dev))
+        params = [torch.nn.Parameter(t[k]) for k in ("position", "point_size", "texture", "confidence")]
+        gkeys = ("d_position", "d_point_size", "d_texture", "d_confidence")
+        for p, k in zip(params, gkeys):
+            p.grad = grads[k]
+        opt = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+
+        def step():
+            for g in grads.values():
+                g.zero_()
+            ctx.forward(desc, tin, images, saved, workspace)
+            ctx.backward(desc, tin, saved, grad_images, grads, workspace)
+            opt.step()
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        ctx.check(workspace)
+        counters = ctx.counters(desc, saved, 0)
+        nz = sum(int((grads[k] != 0).sum().item()) for k in gkeys)
+        total_el = sum(int(grads[k].numel()) for k in gkeys)
+
+        ctx.profile_enable(True)
+        ctx.profile_read()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        prof = ctx.profile_read()
+        ctx.profile_enable(False)
+        ms_per_step = (t1 - t0) * 1e3 / args.steps
+        return dict(sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
+                    grad_images=grad_images, grads=grads, opt=opt, counters=counters, nz=nz, total_el=total_el,
+                    prof=prof, ms_per_step=ms_per_step)
+
+    other_order = None
+    if args.point_order == "random" and not args.no_order_variant:
+        # the same cloud in the memory order real TRIPS scenes have after the reference's preprocessing
+        r = splat_run("morton_blocks")
+        ms_k = {k: ms / max(n, 1) * (n / args.steps) for k, (ms, n) in r["prof"].items()}
+        other_order = {"point_order": "morton_blocks (Morton curve, blocks of 256 shuffled: SceneData.cpp:115-116)",
+                       "ms_per_step": round(r["ms_per_step"], 4),
+                       "fwd_bwd_kernels_ms": round(sum(v for k, v in ms_k.items() if k != "adam_fused"), 4),
+                       "points_per_s": round(r["desc"].num_points / (r["ms_per_step"] * 1e-3), 1),
+                       "kernels_ms": {k: round(v, 4) for k, v in ms_k.items()}}
+        del r
+        torch.cuda.empty_cache()
+
+    r = splat_run(args.point_order)
+    sc, desc, t, tin, workspace, saved, images = (r[k] for k in ("sc", "desc", "t", "tin", "workspace", "saved", "images"))
+    gen, grad_images, grads, opt, counters = (r[k] for k in ("gen", "grad_images", "grads", "opt", "counters"))
+    nz, total_el, prof, ms_per_step = r["nz"], r["total_el"], r["prof"], r["ms_per_step"]
     N, C = desc.num_points, desc.num_channels
-    grads = dict(d_texture=torch.zeros((C, N), device=dev), d_confidence=torch.zeros(N, device=dev),
-                 d_background=torch.zeros(C, device=dev), d_position=torch.zeros((N, 4), device=dev),
-                 d_point_size=torch.zeros(N, device=dev), d_pose=torch.zeros((1, 6), dtype=torch.float64, device=dev),
-                 d_intrinsics=torch.zeros((1, 13), device=dev))
-    params = [torch.nn.Parameter(t[k]) for k in ("position", "point_size", "texture", "confidence")]
-    gkeys = ("d_position", "d_point_size", "d_texture", "d_confidence")
-    for p, k in zip(params, gkeys):
-        p.grad = grads[k]
-    opt = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
-
-    def step():
-        for g in grads.values():
-            g.zero_()
-        ctx.forward(desc, tin, images, saved, workspace)
-        ctx.backward(desc, tin, saved, grad_images, grads, workspace)
-        opt.step()
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ctx.check(workspace)
-    counters = ctx.counters(desc, saved, 0)
-    nz = sum(int((grads[k] != 0).sum().item()) for k in gkeys)
-    total_el = sum(int(grads[k].numel()) for k in gkeys)
-
-    ctx.profile_enable(True)
-    ctx.profile_read()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    prof = ctx.profile_read()
-    ctx.profile_enable(False)
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
 
     alg = algorithmic_bytes(counters, N, C, adam_nonzero=nz, adam_zero=total_el - nz)
     kernels = {}
@@ -261,7 +289,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config3: 6M points (80% noisy ground plane, 20% box), 1920x1080, 8 layers, K=16, "
                                "4-ch f32 descriptors; forward + backward + fused Adam, 1 view",
-                   "points": N, "width": sc.width, "height": sc.height, "layers": desc.num_layers,
+                   "point_order": args.point_order, "points": N, "width": sc.width, "height": sc.height, "layers": desc.num_layers,
                    "list_depth": desc.list_depth, "counters": counters},
         "frame_ms": {"fwd_bwd_kernels": round(fwd_bwd_ms, 4), "all_kernels": round(kernel_ms, 4),
                      "wall_per_step": round(ms_per_step, 4)},
@@ -269,9 +297,10 @@ def main():
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic_bytes(dom) if args.points == DEFAULT_POINTS else None,
+                     "traffic": measured_traffic_bytes(dom) if args.points == DEFAULT_POINTS and args.point_order == "random" else None,
                      "algorithmic_bytes": int(alg[dom]), "avg_ms": kernels[dom]["avg_ms"]},
         "kernels": kernels,
+        "other_point_order": other_order,
         "unet": unet,
         "cpu_baseline": cpu,
     }

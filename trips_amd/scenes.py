@@ -157,9 +157,33 @@ def config2(n=1_000_000, seed=2, w=1920, h=1080, f=1400.0):
                    background=0.0, seed=seed)
 
 
-def config3(n=6_000_000, seed=3, w=1920, h=1080, f=1400.0):
+def _morton_blocks(xyz, rng, block=256):
+    """Order of a point cloud after the reference's one-time preprocessing (SceneData.cpp:115-116): sorted along a
+    3D Morton curve (21 bits per axis), then blocks of `block` consecutive points shuffled."""
+    lo, hi = xyz.min(axis=0), xyz.max(axis=0)
+    q = ((xyz - lo) / np.maximum(hi - lo, 1e-30) * (2 ** 21 - 1)).astype(np.uint64)
+
+    def spread(v):  # 21 bits -> every third bit
+        v = (v | (v << np.uint64(32))) & np.uint64(0x1F00000000FFFF)
+        v = (v | (v << np.uint64(16))) & np.uint64(0x1F0000FF0000FF)
+        v = (v | (v << np.uint64(8))) & np.uint64(0x100F00F00F00F00F)
+        v = (v | (v << np.uint64(4))) & np.uint64(0x10C30C30C30C30C3)
+        v = (v | (v << np.uint64(2))) & np.uint64(0x1249249249249249)
+        return v
+
+    code = spread(q[:, 0]) | (spread(q[:, 1]) << np.uint64(1)) | (spread(q[:, 2]) << np.uint64(2))
+    order = np.argsort(code, kind="stable")
+    nb = (len(order) + block - 1) // block
+    blocks = rng.permutation(nb)
+    idx = (blocks[:, None] * block + np.arange(block)[None, :]).reshape(-1)
+    return order[idx[idx < len(order)]]
+
+
+def config3(n=6_000_000, seed=3, w=1920, h=1080, f=1400.0, order="random"):
     """6M points: 80% on a noisy ground plane (y ~ N(0,0.02^2), x,z uniform over 20x20), 20% uniform in a
-    20x20x5 box above it; camera 1.5 above the plane at its edge, looking at the centre; 8 layers, K=16."""
+    20x20x5 box above it; camera 1.5 above the plane at its edge, looking at the centre; 8 layers, K=16.
+    order: "random" (points in no spatial order) or "morton_blocks" (the order the reference's scene
+    preprocessing leaves a cloud in)."""
     rng = _rng(seed)
     n_ground = int(round(0.8 * n))
     n_box = n - n_ground
@@ -174,6 +198,10 @@ def config3(n=6_000_000, seed=3, w=1920, h=1080, f=1400.0):
     xyz = np.concatenate([ground, box], axis=0)
     perm = rng.permutation(n)
     xyz = xyz[perm]
+    if order == "morton_blocks":
+        xyz = xyz[_morton_blocks(xyz, _rng(seed + 1000))]
+    elif order != "random":
+        raise ValueError(f"order {order!r}")
     radius = _log_uniform(rng, 5e-4, 5e-2, n)
     pose = look_at_pose((0.0, -1.5, -10.0), (0.0, 0.0, 0.0))
     return _finish("config3", xyz, radius, rng, w=w, h=h, f=f, poses=[pose], num_layers=8, list_depth=16, seed=seed)
