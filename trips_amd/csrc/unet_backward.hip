@@ -3,8 +3,7 @@
 // at :751-787 and :999-1098), as hand-written kernels over the state the training forward saved.
 //
 //   final_backward_kernel     1x1 output convolution: gradient of x_0, split into dL/d in[0] and, through the gate,
-//                             the gradient of the finest block's pre-activations
-//   final_weight_grad_kernel  its weight and bias gradients
+//                             the gradient of the finest block's pre-activations; its weight and bias gradients
 //   conv_bwd_data_kernel      gradient of a block's input: the forward's implicit GEMM with flipped, transposed
 //                             weights (M = 256 pixels, N = input channels, K = 9 taps x pre-activations)
 //   up2_adjoint_gate_kernel   adjoint of the bilinear 2x upsampling (a gather over <= 4 x 4 finer pixels), then
@@ -12,7 +11,9 @@
 //   conv_bwd_weight_kernel    weight gradients: GEMM with the pixels as the reduction dimension. Both operands are
 //                             needed pixel-contiguous, so the tiles are written to LDS transposed ([channel][pixel]);
 //                             persistent workgroups keep their partial sums in registers over many tiles
-//   bias_grad_kernel, reduce_weight_grad_kernel
+//                             and sum the pre-activation gradients of their tiles for the bias gradients
+//   bias_grad_kernel          bias gradients alone, when no weight gradient is asked for
+//   reduce_weight_grad_kernel
 //
 // Intermediate gradients are fp16 and carried multiplied by grad_scale; every fp32 result is divided by it again.
 #include <algorithm>
@@ -70,126 +71,206 @@ struct FinalBwdParams
     const float* d_out;       // [cout][H][W]
     float* d_feat;            // [C][H][W], written
     _Float16* dpre;           // [H][W][npad], written
-    float* d_weight;          // [cout][c_feat + cact], accumulated (zeroed by the caller)
-    float* d_bias;            // [cout]
+    float* part;              // [gridDim.x][4 * (4 + CS) + 4] sums of this launch's workgroups (WGRAD)
+    int chunks;               // ceil(pixels / kFinalPixelsPerBlock)
 };
 
+// One pass over the pixels of the finest level: dL/d in[0], the gated block's pre-activation gradients and, when
+// WGRAD, the weight and bias gradients of the 1x1 convolution. Every thread keeps the cout x cin products of its
+// pixels in registers, a workgroup folds them through LDS and writes its sums once (final_reduce_kernel adds the
+// workgroups up: atomics of a thousand workgroups on these few addresses would serialise in one L2 channel).
+// CS = halves per pixel of the block output.
+template <int CS, bool WGRAD>
 __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParams p)
 {
-    __shared__ float s_w[4 * 80];
-    const int cin = p.c_feat + p.cact;
-    for (int i = threadIdx.x; i < p.cout * cin; i += 256) s_w[i] = float(_Float16(p.weight[i]));
-    __syncthreads();
-    const size_t plane = (size_t)p.H * p.W;
-    const int half     = p.npad / 2;
-    for (size_t pix = (size_t)blockIdx.x * 256 + threadIdx.x; pix < plane; pix += (size_t)gridDim.x * 256)
-    {
-        float g[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int k = 0; k < p.cout; ++k) g[k] = p.d_out[k * plane + pix];
-        for (int c = 0; c < p.c_feat; ++c)
-        {
-            float d = 0.f;
-            for (int k = 0; k < p.cout; ++k) d += s_w[k * cin + c] * g[k];
-            p.d_feat[c * plane + pix] = d;
-        }
-        const _Float16* pr = p.pre + pix * p.npad;
-        _Float16* dp       = p.dpre + pix * p.npad;
-        for (int j0 = 0; j0 < half; j0 += 8)
-        {
-            const half8 f8 = *reinterpret_cast<const half8*>(pr + j0);
-            const half8 m8 = *reinterpret_cast<const half8*>(pr + half + j0);
-            half8 of, om;
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-            {
-                const int j = j0 + i;
-                float da    = 0.f;
-                if (j < p.cact)
-                {
-                    for (int k = 0; k < p.cout; ++k) da += s_w[k * cin + p.c_feat + j] * g[k];
-                    da *= p.scale;
-                }
-                float df, dm;
-                gate_backward(da, float(f8[i]), float(m8[i]), df, dm);
-                of[i] = _Float16(df);
-                om[i] = _Float16(dm);
-            }
-            *reinterpret_cast<half8*>(dp + j0)        = of;
-            *reinterpret_cast<half8*>(dp + half + j0) = om;
-        }
-    }
-}
-
-// Weight and bias gradients of the 1x1 convolution: every thread keeps the cout x cin products of its pixels in
-// registers, a block folds them through LDS and adds its sums once. CS = halves per pixel of the block output.
-constexpr int kFinalPixelsPerBlock = 4096;
-template <int CS>
-__global__ __launch_bounds__(256) void final_weight_grad_kernel(const FinalBwdParams p)
-{
     constexpr int MAXC = 4 + CS;
+    // LPP lanes share a pixel, one per 16 bytes of its pre-activation row (feature groups first, then mask groups),
+    // so that a wavefront reads and writes whole lines of the channels-innermost arrays. The feature and the mask
+    // lane of a channel group exchange their values with one cross-lane read.
+    constexpr int LPP = CS <= 16 ? 4 : CS <= 32 ? 8 : 16;
+    constexpr int PPW = 64 / LPP;  // pixels per wavefront and iteration
+    __shared__ float s_w[4 * MAXC];
     __shared__ float s_sum[4 * MAXC + 4];
+    const int cin = p.c_feat + p.cact;
+    // weights as the forward used them (fp16), laid out [k][4 image channels | CS block outputs], zero where unused
+    for (int i = threadIdx.x; i < 4 * MAXC; i += 256)
+    {
+        const int k = i / MAXC, r = i - k * MAXC;
+        const int c = r < 4 ? (r < p.c_feat ? r : -1) : (r - 4 < p.cact ? p.c_feat + r - 4 : -1);
+        s_w[i]      = (k < p.cout && c >= 0) ? float(_Float16(p.weight[k * cin + c])) : 0.f;
+    }
     for (int i = threadIdx.x; i < 4 * MAXC + 4; i += 256) s_sum[i] = 0.f;
     __syncthreads();
     const size_t plane = (size_t)p.H * p.W;
-    const size_t p0 = (size_t)blockIdx.x * kFinalPixelsPerBlock, p1 = std::min(plane, p0 + kFinalPixelsPerBlock);
-    float acc[4][MAXC];
-    float accb[4] = {0.f, 0.f, 0.f, 0.f};
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane % LPP, sub = lane / LPP;
+    const int hg       = p.npad / 16;                    // 16-byte groups in each half of a pre-activation row
+    const bool is_f    = g < hg;
+    const bool in_row  = g < 2 * hg;                     // lanes past the row idle (rows of 96 halves on 16 lanes)
+    const int ch0      = 8 * (is_f ? g : g - hg);        // first of this lane's 8 channels
+    const int partner  = is_f ? lane + hg : lane - hg;   // the lane with the other half of the same channels
+    const bool has_act = is_f && ch0 < CS;               // this lane also reads the block output of its channels
+    const bool has_img = g < p.c_feat;                   // ... and image channel g
+    float wj[4][8], wimg[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        wimg[k] = has_img ? s_w[k * MAXC + g] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wj[k][i] = (in_row && ch0 + i < CS) ? s_w[k * MAXC + 4 + ch0 + i] : 0.f;
+    }
+    float acc[4][8];
+    float acc_img[4] = {0.f, 0.f, 0.f, 0.f}, accb[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < 4; ++k)
 #pragma unroll
-        for (int c = 0; c < MAXC; ++c) acc[k][c] = 0.f;
-    for (size_t pix = p0 + threadIdx.x; pix < p1; pix += 256)
+        for (int i = 0; i < 8; ++i) acc[k][i] = 0.f;
+
+    struct Loaded
     {
-        float g[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int k = 0; k < p.cout; ++k) g[k] = p.d_out[k * plane + pix];
-        float x[MAXC];
+        float g[4], x;
+        half8 v, mine;
+    };
+    auto load = [&](size_t pix, bool valid)
+    {
+        Loaded l;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) x[c] = c < p.c_feat ? float(_Float16(p.feat[c * plane + pix])) : 0.f;
+        for (int k = 0; k < 4; ++k) l.g[k] = (valid && k < p.cout) ? p.d_out[k * plane + pix] : 0.f;
+        l.x = (WGRAD && valid && has_img) ? p.feat[g * plane + pix] : 0.f;
 #pragma unroll
-        for (int q = 0; q < CS / 8; ++q)
+        for (int i = 0; i < 8; ++i) l.v[i] = l.mine[i] = _Float16(0.f);
+        if (WGRAD && valid && has_act) l.v = *reinterpret_cast<const half8*>(p.act + pix * CS + ch0);
+        if (valid && in_row) l.mine = *reinterpret_cast<const half8*>(p.pre + pix * p.npad + 8 * g);
+        return l;
+    };
+    constexpr int STEP = 4 * PPW;  // pixels per iteration of the workgroup
+    for (int chunk = blockIdx.x; chunk < p.chunks; chunk += gridDim.x)
+    {
+        const size_t p1 = std::min(plane, (size_t)(chunk + 1) * kFinalPixelsPerBlock);
+        size_t base     = (size_t)chunk * kFinalPixelsPerBlock + wave * PPW;
+        Loaded next     = load(base + sub, base + sub < p1);
+        for (; base < p1; base += STEP)
         {
-            const half8 v = *reinterpret_cast<const half8*>(p.act + pix * CS + 8 * q);
+            const size_t pix = base + sub;
+            const bool valid = pix < p1;
+            const Loaded cur = next;
+            if (base + STEP < p1) next = load(pix + STEP, pix + STEP < p1);  // in flight while this pixel is worked on
+            // the other half (mask values for a feature lane and the reverse) of the same 8 channels
+            typedef int intx4 __attribute__((ext_vector_type(4)));
+            intx4 raw = __builtin_bit_cast(intx4, cur.mine), oth;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[4 + 8 * q + i] = float(v[i]);
-        }
+            for (int q = 0; q < 4; ++q) oth[q] = __shfl(raw[q], partner);
+            const half8 other = __builtin_bit_cast(half8, oth);
+            const half8 f8 = is_f ? cur.mine : other, m8 = is_f ? other : cur.mine;
+            half8 out;
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-        {
-            accb[k] += g[k];
+            for (int i = 0; i < 8; ++i)
+            {
+                float da = 0.f;
 #pragma unroll
-            for (int c = 0; c < MAXC; ++c) acc[k][c] += g[k] * x[c];
+                for (int k = 0; k < 4; ++k) da += wj[k][i] * cur.g[k];
+                float df, dm;
+                gate_backward(da * p.scale, float(f8[i]), float(m8[i]), df, dm);
+                out[i] = _Float16(is_f ? df : dm);
+            }
+            if (valid && in_row) *reinterpret_cast<half8*>(p.dpre + pix * p.npad + 8 * g) = out;
+            if (valid && has_img)
+            {
+                float d = 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) d += wimg[k] * cur.g[k];
+                p.d_feat[g * plane + pix] = d;
+            }
+            if (WGRAD)
+            {
+                const float xr = float(_Float16(cur.x));
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                {
+                    accb[k] += cur.g[k];
+                    acc_img[k] += cur.g[k] * xr;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[k][i] += cur.g[k] * float(cur.v[i]);
+                }
+            }
         }
     }
-    // fold the wavefront with a butterfly first: 64 lanes adding to one LDS address would be serialised
-    auto wave_sum = [](float v)
+    if (!WGRAD) return;
+    // fold the lanes that hold the same channels with a butterfly first: many lanes adding to one LDS address would
+    // be serialised
+    auto fold = [](float v)
     {
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        for (int o = 32; o >= LPP; o >>= 1) v += __shfl_xor(v, o);
         return v;
     };
-    const bool first_lane = (threadIdx.x & 63) == 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k)
     {
-        const float b = wave_sum(accb[k]);
-        if (first_lane) atomicAdd(&s_sum[4 * MAXC + k], b);
+        const float b = fold(accb[k]);
+        if (lane == 0) atomicAdd(&s_sum[4 * MAXC + k], b);
+        const float im = fold(acc_img[k]);
+        if (lane < LPP && has_img) atomicAdd(&s_sum[k * MAXC + g], im);
 #pragma unroll
-        for (int c = 0; c < MAXC; ++c)
+        for (int i = 0; i < 8; ++i)
         {
-            const float v = wave_sum(acc[k][c]);
-            if (first_lane) atomicAdd(&s_sum[k * MAXC + c], v);
+            const float v = fold(acc[k][i]);
+            if (lane < LPP && has_act && ch0 + i < CS) atomicAdd(&s_sum[k * MAXC + 4 + ch0 + i], v);
         }
     }
     __syncthreads();
-    // registers are laid out [k][4 image channels | CS block outputs]; the weight is [k][c_feat + cact]
-    const int cin = p.c_feat + p.cact;
-    for (int t = threadIdx.x; t < p.cout * cin; t += 256)
+    float* part = p.part + (size_t)blockIdx.x * (4 * MAXC + 4);
+    for (int t = threadIdx.x; t < 4 * MAXC + 4; t += 256) part[t] = s_sum[t];
+}
+
+// Adds up `rows` partial-sum rows of `cols` floats: workgroup c sums column c, thread 0 holds the result.
+__device__ __forceinline__ float block_column_sum(const float* __restrict__ part, int rows, int cols, int c)
+{
+    __shared__ float s_red[4];
+    float s = 0.f;
+    for (int r = threadIdx.x; r < rows; r += 256) s += part[(size_t)r * cols + c];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    return (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+}
+
+// d_weight [cout][c_feat + cact] and d_bias [cout] of the 1x1 convolution from final_backward_kernel's partial sums
+// (row layout [k][4 image channels | CS block outputs], then 4 biases); one workgroup per result
+__global__ __launch_bounds__(256) void final_reduce_kernel(const float* __restrict__ part, int rows, int maxc, int c_feat, int cact,
+                                                           int cout, float* __restrict__ d_weight, float* __restrict__ d_bias)
+{
+    const int cin = c_feat + cact;
+    const int t   = blockIdx.x;  // < cout * cin + cout
+    int col;
+    float* dst;
+    if (t < cout * cin)
     {
         const int k = t / cin, c = t - k * cin;
-        const int r = c < p.c_feat ? c : 4 + (c - p.c_feat);
-        atomicAdd(p.d_weight + t, s_sum[k * MAXC + r]);
+        col = k * maxc + (c < c_feat ? c : 4 + (c - c_feat));
+        dst = d_weight + t;
     }
-    if ((int)threadIdx.x < p.cout) atomicAdd(p.d_bias + threadIdx.x, s_sum[4 * MAXC + threadIdx.x]);
+    else
+    {
+        col = 4 * maxc + (t - cout * cin);
+        dst = d_bias + (t - cout * cin);
+    }
+    if (!(t < cout * cin ? d_weight : d_bias)) return;  // the caller asked for one of the two only
+    const float s = block_column_sum(part, rows, 4 * maxc + 4, col);
+    if (threadIdx.x == 0) *dst = s;
+}
+
+// feature and mask bias gradients of a block from the weight-gradient kernel's per-workgroup sums [rows][npad]
+__global__ __launch_bounds__(256) void bias_reduce_kernel(const float* __restrict__ part, int rows, int npad, int cout, float scale_inv,
+                                                          float* __restrict__ d_bias_f, float* __restrict__ d_bias_m)
+{
+    const int n = blockIdx.x, half = npad / 2;
+    const int o = n < half ? n : n - half;
+    float* dst  = n < half ? d_bias_f : d_bias_m;
+    if (o >= cout || !dst) return;
+    const float s = block_column_sum(part, rows, npad, n);
+    if (threadIdx.x == 0) dst[o] = s * scale_inv;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -400,15 +481,22 @@ struct BwdWeightParams
     const _Float16* act_below;
     const _Float16* dpre;  // [H][W][NPAD]
     float* part;           // [gridDim.x][9][NPAD][CIN]
+    // bias gradients = sums of dpre over the pixels, taken from the transposed tile while it is in LDS
+    float* bias_part;      // [gridDim.x][NPAD] or nullptr
 };
 
 constexpr int kXtRow   = 40;                          // halves per patch row in the transposed input tile
 constexpr int kXtChan  = kConvPatchH * kXtRow + 8;    // halves per channel (padding spreads the 16 channels of a read over the banks)
 constexpr int kDtChan  = kConvTileH * kConvTileW + 8;  // halves per pre-activation channel in the transposed gradient tile
 
-template <int CIN, int NPAD>
+template <int CIN, int NPAD, bool BIAS>
 __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightParams p)
 {
+    // bias sums: thread t adds up segment t / NPAD (kBiasSegLen pixels) of row t % NPAD of the gradient tile
+    constexpr int kBiasSegs   = 256 / NPAD;
+    constexpr int kBiasSegLen = kConvTileH * kConvTileW / kBiasSegs;
+    const int bias_n = threadIdx.x % NPAD, bias_seg = threadIdx.x / NPAD;
+    float bias_acc = 0.f;
     constexpr int ROW    = CIN + kLdsChanPad;
     constexpr int GROUPS = CIN / 8;
     constexpr int NB     = NPAD / 16;
@@ -526,6 +614,19 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
             }
         }
         __syncthreads();
+        if (BIAS && (int)threadIdx.x < kBiasSegs * NPAD)
+        {
+            const _Float16* src = s_dt + bias_n * kDtChan + bias_seg * kBiasSegLen;
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int q = 0; q < kBiasSegLen / 8; ++q)
+            {
+                const half8 v = *reinterpret_cast<const half8*>(src + 8 * q);
+                s0 += (float(v[0]) + float(v[1])) + (float(v[2]) + float(v[3]));
+                s1 += (float(v[4]) + float(v[5])) + (float(v[6]) + float(v[7]));
+            }
+            bias_acc += s0 + s1;
+        }
         // ---- dW[tap][n][c] += sum over the tile's pixels of dpre[pixel][n] * x[pixel + tap][c] ----
 #pragma unroll
         for (int r = 0; r < kConvTileH; ++r)
@@ -549,6 +650,16 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         }
     }
 
+    if (BIAS)
+    {
+        __syncthreads();  // all tiles consumed: the tile memory is free
+        float* s_bias = reinterpret_cast<float*>(smem);
+        if ((int)threadIdx.x < NPAD) s_bias[threadIdx.x] = 0.f;
+        __syncthreads();
+        if ((int)threadIdx.x < kBiasSegs * NPAD) atomicAdd(&s_bias[bias_n], bias_acc);
+        __syncthreads();
+        if ((int)threadIdx.x < NPAD) p.bias_part[(size_t)blockIdx.x * NPAD + threadIdx.x] = s_bias[threadIdx.x];
+    }
     float* part = p.part + (size_t)blockIdx.x * 9 * NPAD * CIN;
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)
@@ -629,22 +740,24 @@ hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipS
     return hipErrorInvalidValue;
 }
 
-template <int CIN, int NPAD>
+template <int CIN, int NPAD, bool BIAS>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
     const size_t lds = ((size_t)kBelowH * kBelowW * (CIN + kLdsChanPad) + (size_t)CIN * kXtChan + (size_t)NPAD * kDtChan) *
                        sizeof(_Float16);  // up to 133 KB
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD, BIAS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD>), dim3(groups), dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD, BIAS>), dim3(groups), dim3(256), lds, stream, p);
     return hipGetLastError();
 }
 
 hipError_t dispatch_bwd_weight(const BwdWeightParams& p, int cin_pad, int npad, int groups, hipStream_t stream)
 {
-#define TRIPS_BW(CIN_, NPAD_) \
-    if (cin_pad == CIN_ && npad == NPAD_) return launch_bwd_weight<CIN_, NPAD_>(p, groups, stream);
+#define TRIPS_BW(CIN_, NPAD_)                                                                  \
+    if (cin_pad == CIN_ && npad == NPAD_)                                                      \
+        return p.bias_part ? launch_bwd_weight<CIN_, NPAD_, true>(p, groups, stream) \
+                                          : launch_bwd_weight<CIN_, NPAD_, false>(p, groups, stream);
     TRIPS_BW(32, 32) TRIPS_BW(32, 64) TRIPS_BW(32, 96) TRIPS_BW(32, 128)
     TRIPS_BW(64, 32) TRIPS_BW(64, 64) TRIPS_BW(64, 96) TRIPS_BW(64, 128)
 #undef TRIPS_BW
@@ -731,17 +844,17 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             hipLaunchKernelGGL(pack_conv_weights_T_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
                                weights->feature_weight[i], weights->mask_weight[i], lv.cout, lv.cin_real, lv.cin_pad, lv.npad,
                                reinterpret_cast<_Float16*>(ws + lv.wt_off));
-            fill(grads->feature_bias[i], lv.cout);
-            fill(grads->mask_bias[i], lv.cout);
+            if (!grads->feature_weight[i] && !grads->mask_weight[i])  // bias_grad_kernel accumulates; otherwise they are written
+            {
+                fill(grads->feature_bias[i], lv.cout);
+                fill(grads->mask_bias[i], lv.cout);
+            }
         }
-        fill(grads->final_weight, K * (C + np.lv[0].cout));
-        fill(grads->final_bias, K);
     }
     {
         ProfScope ps(prof, "unet_bwd_final", stream);
         const LevelPlan& lv = np.lv[0];
         const size_t plane  = (size_t)lv.H * lv.W;
-        // the weight-gradient kernel needs somewhere to add to even when the caller does not want the result
         for (int b = 0; b < d.batch; ++b)
         {
             FinalBwdParams p;
@@ -755,22 +868,29 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             p.d_out    = d_output + (size_t)b * K * plane;
             p.d_feat   = grads->inputs[0] + (size_t)b * C * plane;
             p.dpre     = dpre_ptr(0, b);
-            p.d_weight = grads->final_weight;
-            p.d_bias   = grads->final_bias;
-            const int blocks = (int)std::min<size_t>((plane + 255) / 256, 65535);
-            hipLaunchKernelGGL(final_backward_kernel, dim3(blocks), dim3(256), 0, stream, p);
-            if (p.d_weight && p.d_bias)
+            p.chunks   = (int)((plane + kFinalPixelsPerBlock - 1) / kFinalPixelsPerBlock);
+            p.part     = reinterpret_cast<float*>(ws + np.final_part_off) + (size_t)b * np.final_groups * (4 * (4 + lv.cout_store) + 4);
+            const bool wgrad = grads->final_weight || grads->final_bias;
+            const int chunks = wgrad ? np.final_groups : p.chunks;
+            switch (lv.cout_store)
             {
-                const int chunks = (int)((plane + kFinalPixelsPerBlock - 1) / kFinalPixelsPerBlock);
-                switch (lv.cout_store)
-                {
-#define TRIPS_FW(CS_) \
-    case CS_: hipLaunchKernelGGL((final_weight_grad_kernel<CS_>), dim3(chunks), dim3(256), 0, stream, p); break;
-                    TRIPS_FW(8) TRIPS_FW(16) TRIPS_FW(24) TRIPS_FW(32) TRIPS_FW(40) TRIPS_FW(48) TRIPS_FW(56) TRIPS_FW(64)
+#define TRIPS_FW(CS_)                                                                                         \
+    case CS_:                                                                                                 \
+        if (wgrad)                                                                                            \
+            hipLaunchKernelGGL((final_backward_kernel<CS_, true>), dim3(chunks), dim3(256), 0, stream, p);    \
+        else                                                                                                  \
+            hipLaunchKernelGGL((final_backward_kernel<CS_, false>), dim3(chunks), dim3(256), 0, stream, p);   \
+        break;
+                TRIPS_FW(8) TRIPS_FW(16) TRIPS_FW(24) TRIPS_FW(32) TRIPS_FW(40) TRIPS_FW(48) TRIPS_FW(56) TRIPS_FW(64)
 #undef TRIPS_FW
-                    default: return set_error(TRIPS_ERR_UNSUPPORTED, "block output stride %d", lv.cout_store);
-                }
+                default: return set_error(TRIPS_ERR_UNSUPPORTED, "block output stride %d", lv.cout_store);
             }
+        }
+        if (grads->final_weight || grads->final_bias)
+        {
+            hipLaunchKernelGGL(final_reduce_kernel, dim3(K * (C + lv.cout) + K), dim3(256), 0, stream,
+                               reinterpret_cast<const float*>(ws + np.final_part_off), d.batch * np.final_groups, 4 + lv.cout_store, C,
+                               lv.cout, K, grads->final_weight, grads->final_bias);
         }
     }
     static const char* const kDataNames[TRIPS_UNET_MAX_LEVELS]   = {"unet_bwd_data_l0", "unet_bwd_data_l1", "unet_bwd_data_l2", "unet_bwd_data_l3",
@@ -794,7 +914,8 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
                 bp.dpre      = dpre_ptr(i, b);
                 bp.d_bias_f  = grads->feature_bias[i];
                 bp.d_bias_m  = grads->mask_bias[i];
-                if (bp.d_bias_f || bp.d_bias_m)
+                const bool want_w = grads->feature_weight[i] || grads->mask_weight[i];
+                if ((bp.d_bias_f || bp.d_bias_m) && !want_w)  // otherwise the weight-gradient kernel sums them on its way
                     hipLaunchKernelGGL(bias_grad_kernel, dim3((unsigned)((plane + kBiasChunk - 1) / kBiasChunk)), dim3(256), 0, stream, bp);
 
                 BwdWeightParams wp;
@@ -805,6 +926,8 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
                 wp.feat    = inputs[i] + (size_t)b * C * plane;
                 wp.dpre    = dpre_ptr(i, b);
                 wp.part    = reinterpret_cast<float*>(ws + lv.part_off) + (size_t)b * lv.groups * 9 * lv.npad * lv.cin_pad;
+                if (bp.d_bias_f || bp.d_bias_m)
+                    wp.bias_part = reinterpret_cast<float*>(ws + lv.bias_part_off) + (size_t)b * lv.groups * lv.npad;
                 if (below)
                 {
                     const LevelPlan& lb = np.lv[i + 1];
@@ -826,6 +949,10 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
                                    reinterpret_cast<const float*>(ws + lv.part_off), d.batch * lv.groups, total, sliced);
                 hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, sliced, lv.cout,
                                    lv.cin_real, lv.cin_pad, lv.npad, scale_inv, grads->feature_weight[i], grads->mask_weight[i]);
+                if (grads->feature_bias[i] || grads->mask_bias[i])
+                    hipLaunchKernelGGL(bias_reduce_kernel, dim3(lv.npad), dim3(256), 0, stream,
+                                       reinterpret_cast<const float*>(ws + lv.bias_part_off), d.batch * lv.groups, lv.npad, lv.cout,
+                                       scale_inv, grads->feature_bias[i], grads->mask_bias[i]);
             }
         }
         {

@@ -17,6 +17,8 @@ constexpr int kConvPatchH  = kConvTileH + 2;
 constexpr int kConvPatchW  = kConvTileW + 2;
 constexpr int kBelowH      = kConvTileH / 2 + 2;  // rows / columns of the level below that an upsampled patch touches
 constexpr int kBelowW      = kConvTileW / 2 + 2;
+constexpr int kFinalPixelsPerBlock = 2048;  // pixels a workgroup of the 1x1 convolution's backward takes at a time
+constexpr int kFinalPartFloats     = 4 * (4 + 64) + 4;  // its partial sums: [4 outputs][4 image + <= 64 block channels], 4 biases
 constexpr int kLdsChanPad  = 8;  // halves added to every LDS row so that 16 lanes reading 16 bytes hit 64 distinct banks
 
 // source row / column and weight of torch's bilinear upsampling with scale_factor 2, align_corners = false
@@ -121,6 +123,7 @@ struct LevelPlan
     size_t din_off;     // gradient of the block input [B][H][W][cin_pad] fp16
     size_t part_off;    // partial weight gradients [groups][9][npad][cin_pad] fp32
     size_t sliced_off;  // partial sums of the partials [16][9][npad][cin_pad] fp32
+    size_t bias_part_off;  // per-workgroup sums of the pre-activation gradients [batch * groups][npad] fp32
     int groups;         // persistent workgroups of the weight-gradient kernel (per image)
 };
 
@@ -130,6 +133,8 @@ struct NetPlan
     size_t bytes;           // forward workspace
     size_t saved_bytes;     // saved state
     size_t backward_bytes;  // backward workspace
+    size_t final_part_off;  // backward workspace: per-workgroup sums of the 1x1 convolution's weight and bias gradients
+    int final_groups;       // persistent workgroups of the finest level's first backward kernel (per image)
 };
 
 inline int check_unet_desc(const TripsUnetDesc* d)
@@ -218,6 +223,14 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
         bw += align256((size_t)d.batch * lv.groups * 9 * lv.npad * lv.cin_pad * sizeof(float));
         lv.sliced_off = bw;
         bw += align256((size_t)16 * 9 * lv.npad * lv.cin_pad * sizeof(float));
+        lv.bias_part_off = bw;
+        bw += align256((size_t)d.batch * lv.groups * lv.npad * sizeof(float));
+    }
+    {
+        const size_t chunks = ((size_t)np.lv[0].H * np.lv[0].W + kFinalPixelsPerBlock - 1) / kFinalPixelsPerBlock;
+        np.final_groups     = chunks < 1024 ? (int)chunks : 1024;
+        np.final_part_off   = bw;
+        bw += align256((size_t)d.batch * np.final_groups * kFinalPartFloats * sizeof(float));
     }
     np.saved_bytes    = sv;
     np.backward_bytes = bw;

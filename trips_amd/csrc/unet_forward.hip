@@ -2,7 +2,8 @@
 //
 //   gated_conv3x3_kernel <- SmallDecStartBlockImpl::forward / UpsampleDecOnlySmallBlockFixedImpl::forward
 //                           src/lib/models/Networks.h:751-787, 999-1098
-//   final_conv1x1_kernel <- the `final` Sequential of MultiScaleUnet2dDecOnlySmallFixedImpl, Networks.h:1129-1131
+//                           and, in the finest block's epilogue, the `final` 1x1 Sequential of
+//                           MultiScaleUnet2dDecOnlySmallFixedImpl, Networks.h:1129-1131
 //
 // The reference runs, per level, upsample -> cat -> two 3x3 convolutions -> elu / sigmoid -> multiply -> cat as
 // separate libtorch ops on NCHW tensors, materialising every intermediate. Here one kernel per level does all of
@@ -39,6 +40,11 @@ struct ConvParams
     const float* bias;        // [NPAD]: feature biases, then mask biases, each padded to NPAD / 2
     _Float16* out;            // [H][W][cout_store]
     _Float16* pre;            // [H][W][NPAD] pre-activations (feature | mask) for the backward, or nullptr
+    // the finest block also applies the net's 1x1 output convolution to x_0 = cat(image, block output)
+    const float* final_w;     // [final_cout][C + cout] or nullptr
+    const float* final_b;     // [final_cout]
+    float* final_out;         // [final_cout][H][W]
+    int final_cout;
 };
 
 template <int CIN, int NPAD>
@@ -47,12 +53,19 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     constexpr int ROW  = CIN + kLdsChanPad;  // halves per patch pixel in LDS
     constexpr int NB   = NPAD / 16;          // 16-column blocks; the first half are feature outputs
     constexpr int HB   = NB / 2;
-    constexpr int KB   = CIN / 32;
     extern __shared__ _Float16 smem[];
     _Float16* s_patch = smem;  // [kConvPatchH * kConvPatchW][ROW]
 
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
     const bool has_below = p.Hb > 0;
+    // weights and biases of the 1x1 output convolution, rounded to fp16 like every other operand
+    __shared__ float s_fw[4 * (4 + 64) + 4];
+    if (p.final_out)
+    {
+        const int cin = p.c_feat + p.cout;
+        for (int i = threadIdx.x; i < p.final_cout * cin; i += 256) s_fw[i] = float(_Float16(p.final_w[i]));
+        if ((int)threadIdx.x < p.final_cout) s_fw[4 * (4 + 64) + threadIdx.x] = p.final_b[threadIdx.x];
+    }
 
     // ---- stage 1: everything the patch needs from memory, all loads of a thread in flight together ----
     // (a) this level's image -> channels [0, C) of the patch; (b) the level below, x_{i+1} = cat(image, activations),
@@ -157,6 +170,12 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     constexpr int AS = NPAD / 2 + kLdsChanPad, PS = NPAD + kLdsChanPad;
     _Float16* s_act = smem;                                      // [256][AS]
     _Float16* s_pre = smem + kConvTileH * kConvTileW * AS;       // [256][PS]
+    float my_feat[4] = {0.f, 0.f, 0.f, 0.f};  // this thread's pixel of the image, as the convolution saw it (fp16)
+    if (p.final_out)
+    {
+        const _Float16* row = s_patch + (size_t)((threadIdx.x / kConvTileW + 1) * kConvPatchW + threadIdx.x % kConvTileW + 1) * ROW;
+        for (int c = 0; c < C; ++c) my_feat[c] = float(row[c]);
+    }
     __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
     for (int m = 0; m < 4; ++m)
@@ -185,6 +204,33 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     __syncthreads();
     store_tile_nhwc(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
     if (p.pre) store_tile_nhwc(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
+    if (p.final_out)
+    {
+        // `final` of the net (Networks.h:1129-1131): one thread per pixel of the tile, weights rounded to fp16 like
+        // every other operand
+        const int y = y0 + threadIdx.x / kConvTileW, x = x0 + threadIdx.x % kConvTileW;
+        if (y < p.H && x < p.W)
+        {
+            const int cin           = C + p.cout;
+            const _Float16* a       = s_act + (size_t)threadIdx.x * AS;
+            const size_t plane      = (size_t)p.H * p.W;
+            float o[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (k < p.final_cout) o[k] += s_fw[k * cin + c] * my_feat[c];
+            for (int c = 0; c < p.cout; ++c)
+            {
+                const float v = float(a[c]);
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (k < p.final_cout) o[k] += s_fw[k * cin + C + c] * v;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (k < p.final_cout) p.final_out[k * plane + (size_t)y * p.W + x] = o[k] + s_fw[4 * (4 + 64) + k];
+        }
+    }
 }
 
 // wpack[tap][n][c]: n < NPAD/2 feature output n, else mask output n - NPAD/2; zero outside the real ranges
@@ -208,43 +254,6 @@ __global__ __launch_bounds__(256) void pack_conv_weights_kernel(const float* __r
         const int half = npad / 2;
         const int o    = n < half ? n : n - half;
         bias[n]        = o < cout ? (n < half ? bf : bm)[o] : 0.f;
-    }
-}
-
-struct FinalParams
-{
-    int H, W, c_feat, cact, cact_store, cout;
-    const float* feat;      // [C][H][W]
-    const _Float16* act;    // [H][W][cact_store]
-    const float* weight;    // [cout][c_feat + cact]
-    const float* bias;      // [cout]
-    float* out;             // [cout][H][W]
-};
-
-__global__ __launch_bounds__(256) void final_conv1x1_kernel(const FinalParams p)
-{
-    __shared__ float s_w[4 * 80];
-    __shared__ float s_b[4];
-    const int cin = p.c_feat + p.cact;
-    for (int i = threadIdx.x; i < p.cout * cin; i += 256) s_w[i] = float(_Float16(p.weight[i]));
-    if (threadIdx.x < p.cout) s_b[threadIdx.x] = p.bias[threadIdx.x];
-    __syncthreads();
-    const size_t plane = (size_t)p.H * p.W;
-    for (size_t pix = (size_t)blockIdx.x * 256 + threadIdx.x; pix < plane; pix += (size_t)gridDim.x * 256)
-    {
-        float o[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int c = 0; c < p.c_feat; ++c)
-        {
-            const float v = float(_Float16(p.feat[c * plane + pix]));
-            for (int k = 0; k < p.cout; ++k) o[k] += s_w[k * cin + c] * v;
-        }
-        const _Float16* a = p.act + pix * p.cact_store;
-        for (int c = 0; c < p.cact; ++c)
-        {
-            const float v = float(a[c]);
-            for (int k = 0; k < p.cout; ++k) o[k] += s_w[k * cin + p.c_feat + c] * v;
-        }
-        for (int k = 0; k < p.cout; ++k) p.out[k * plane + pix] = o[k] + s_b[k];
     }
 }
 
@@ -394,33 +403,16 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
                 p.feat_below = inputs[i + 1] + (size_t)b * C * lb.H * lb.W;
                 p.act_below  = act_ptr(i + 1, b);
             }
+            if (i == 0)
+            {
+                p.final_w    = weights->final_weight;
+                p.final_b    = weights->final_bias;
+                p.final_out  = output + (size_t)b * d.num_output_channels * lv.H * lv.W;
+                p.final_cout = d.num_output_channels;
+            }
             hipError_t e = dispatch_conv(p, lv.cin_pad, lv.npad, stream);
             if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "gated conv launch (level %d): %s", i, hipGetErrorString(e));
         }
-    }
-    {
-        ProfScope ps(prof, "unet_final_1x1", stream);
-        const LevelPlan& lv = np.lv[0];
-        for (int b = 0; b < d.batch; ++b)
-        {
-            FinalParams p;
-            p.H          = lv.H;
-            p.W          = lv.W;
-            p.c_feat     = C;
-            p.cact       = lv.cout;
-            p.cact_store = lv.cout_store;
-            p.cout       = d.num_output_channels;
-            p.feat       = inputs[0] + (size_t)b * C * lv.H * lv.W;
-            p.act        = act_ptr(0, b);
-            p.weight     = weights->final_weight;
-            p.bias       = weights->final_bias;
-            p.out        = output + (size_t)b * d.num_output_channels * lv.H * lv.W;
-            const size_t plane = (size_t)lv.H * lv.W;
-            const int blocks   = (int)std::min<size_t>((plane + 255) / 256, 65535);
-            hipLaunchKernelGGL(final_conv1x1_kernel, dim3(blocks), dim3(256), 0, stream, p);
-        }
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "final conv launch: %s", hipGetErrorString(e));
     }
     return TRIPS_OK;
 }
