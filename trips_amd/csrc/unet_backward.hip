@@ -309,11 +309,15 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     conv_taps_mfma<KC, NN>(s_patch, p.wt, acc);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
-    const size_t plane = (size_t)p.H * p.W;
+    // ---- epilogue: the tile staged in LDS (the patch is no longer needed) and written channels innermost with
+    // 16-byte stores, whole lines at a time; the image channels' share kept in fp32 beside it ----
+    constexpr int OS   = NN + kLdsChanPad;
+    _Float16* s_out    = smem;                                                                   // [256][OS]
+    float* s_img       = reinterpret_cast<float*>(smem + kConvTileH * kConvTileW * OS);          // [4][256]
+    __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
     for (int m = 0; m < 4; ++m)
     {
-        const int y = y0 + 2 * wave + (m >> 1);
 #pragma unroll
         for (int n = 0; n < NB; ++n)
         {
@@ -321,12 +325,24 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
 #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
-                const int x = x0 + (m & 1) * 16 + (lane >> 4) * 4 + i;
-                if (y >= p.H || x >= p.W) continue;
+                const int tp  = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + (lane >> 4) * 4 + i;
                 const float v = acc[m][n][i];
-                if (p.d_in) p.d_in[((size_t)y * p.W + x) * NN + c] = _Float16(v);
-                if (c < p.c_feat) p.d_feat[c * plane + (size_t)y * p.W + x] += v * p.scale_inv;
+                s_out[tp * OS + c] = _Float16(v);
+                if (n == 0 && c < 4) s_img[c * (kConvTileH * kConvTileW) + tp] = v;
             }
+        }
+    }
+    __syncthreads();
+    if (p.d_in) store_tile_nhwc(s_out, OS, NN / 8, p.d_in, NN, x0, y0, p.W, p.H);
+    {
+        const size_t plane = (size_t)p.H * p.W;
+        const int y = y0 + threadIdx.x / kConvTileW, x = x0 + threadIdx.x % kConvTileW;
+        if (y < p.H && x < p.W)
+        {
+            float old[4];
+            for (int c = 0; c < p.c_feat; ++c) old[c] = p.d_feat[c * plane + (size_t)y * p.W + x];
+            for (int c = 0; c < p.c_feat; ++c)
+                p.d_feat[c * plane + (size_t)y * p.W + x] = old[c] + s_img[c * (kConvTileH * kConvTileW) + threadIdx.x] * p.scale_inv;
         }
     }
 }
@@ -721,7 +737,9 @@ namespace
 template <int KC, int NN>
 hipError_t launch_bwd_data(const BwdDataParams& p, hipStream_t stream)
 {
-    const size_t lds = (size_t)kConvPatchH * kConvPatchW * (KC + kLdsChanPad) * sizeof(_Float16);  // up to 92 KB
+    const size_t lds_in  = (size_t)kConvPatchH * kConvPatchW * (KC + kLdsChanPad) * sizeof(_Float16);  // up to 92 KB
+    const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NN + kLdsChanPad) * sizeof(_Float16) + 4 * sizeof(float));
+    const size_t lds     = std::max(lds_in, lds_out);
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
