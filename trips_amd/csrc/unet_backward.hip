@@ -293,6 +293,8 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     extern __shared__ _Float16 smem[];
     _Float16* s_patch = smem;
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
+    ConvTapRing<KC, NN> ring;
+    conv_taps_prefetch(ring, p.wt);  // in flight while the patch is loaded
     for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
     {
         const int g = item % GROUPS, pp = item / GROUPS;
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     }
     __syncthreads();
     floatx4 acc[4][NB];
-    conv_taps_mfma<KC, NN>(s_patch, p.wt, acc);
+    conv_taps_mfma<KC, NN>(s_patch, p.wt, ring, acc);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
     // ---- epilogue: the tile staged in LDS (the patch is no longer needed) and written channels innermost with

@@ -36,41 +36,60 @@ __device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i
 
 // The 9-tap implicit-GEMM core shared by the forward convolution and the data gradient: A operands are 16-byte
 // LDS reads from a (8+2) x (32+2) pixel patch with KIN channels innermost (row stride KIN + 8 halves), B operands
-// (packed weights [tap][NOUT][KIN], L2-resident) are loaded from memory directly, the next tap's fragments
-// requested before the current tap's MFMAs issue, so the tap loop has no barrier. A wavefront owns two rows of the
-// 8 x 32 output tile = four 16-pixel row blocks; acc[m][n] is the 16 x 16 block of pixels m, outputs 16n .. 16n+15.
+// (packed weights [tap][NOUT][KIN], L2-resident) are loaded from memory directly into a ring of registers, DEPTH taps
+// ahead of their use: the first DEPTH taps are requested by conv_taps_prefetch, which a kernel calls before it
+// assembles its patch, so their latency (a tap's fragments are one dependent L2 round trip) hides behind that work;
+// the tap loop has no barrier. A wavefront owns two rows of the 8 x 32 output tile = four 16-pixel row blocks;
+// acc[m][n] is the 16 x 16 block of pixels m, outputs 16n .. 16n+15.
+template <int KIN, int NOUT>
+struct ConvTapRing
+{
+    static constexpr int NB = NOUT / 16;
+    static constexpr int KB = KIN / 32;
+    // three taps ahead while that costs at most 128 registers, else one (registers decide how many workgroups share a CU)
+    static constexpr int DEPTH = KB * NB <= 8 ? 3 : 1;
+    half8 b[DEPTH + 1][KB][NB];
+};
+
+template <int KIN, int NOUT>
+__device__ __forceinline__ void conv_taps_load(ConvTapRing<KIN, NOUT>& ring, const _Float16* __restrict__ wpack, int tap)
+{
+    using R = ConvTapRing<KIN, NOUT>;
+    const int lane = threadIdx.x & 63;
+    const _Float16* wt = wpack + (size_t)tap * NOUT * KIN + (size_t)(lane & 15) * KIN + (lane >> 4) * 8;
+#pragma unroll
+    for (int kb = 0; kb < R::KB; ++kb)
+#pragma unroll
+        for (int n = 0; n < R::NB; ++n)
+            ring.b[tap % (R::DEPTH + 1)][kb][n] = *reinterpret_cast<const half8*>(wt + (size_t)(n * 16) * KIN + kb * 32);
+}
+
+template <int KIN, int NOUT>
+__device__ __forceinline__ void conv_taps_prefetch(ConvTapRing<KIN, NOUT>& ring, const _Float16* __restrict__ wpack)
+{
+#pragma unroll
+    for (int tap = 0; tap < ConvTapRing<KIN, NOUT>::DEPTH; ++tap) conv_taps_load(ring, wpack, tap);
+}
+
 template <int KIN, int NOUT>
 __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, const _Float16* __restrict__ wpack,
-                                               floatx4 (&acc)[4][NOUT / 16])
+                                               ConvTapRing<KIN, NOUT>& ring, floatx4 (&acc)[4][NOUT / 16])
 {
+    using R = ConvTapRing<KIN, NOUT>;
     constexpr int ROW = KIN + kLdsChanPad;
-    constexpr int NB  = NOUT / 16;
-    constexpr int KB  = KIN / 32;
+    constexpr int NB  = R::NB;
+    constexpr int KB  = R::KB;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 #pragma unroll
     for (int m = 0; m < 4; ++m)
 #pragma unroll
         for (int n = 0; n < NB; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
-    const _Float16* wlane = wpack + (size_t)lrow * KIN + lk;
-    half8 bcur[KB][NB];
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int n = 0; n < NB; ++n) bcur[kb][n] = *reinterpret_cast<const half8*>(wlane + (size_t)(n * 16) * KIN + kb * 32);
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)
     {
         const int dy = tap / 3, dx = tap - dy * 3;  // patch coordinates already include the halo
-        half8 bnext[KB][NB];
-        if (tap + 1 < 9)
-        {
-            const _Float16* wt = wlane + (size_t)(tap + 1) * NOUT * KIN;
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int n = 0; n < NB; ++n) bnext[kb][n] = *reinterpret_cast<const half8*>(wt + (size_t)(n * 16) * KIN + kb * 32);
-        }
+        if (tap + R::DEPTH < 9) conv_taps_load(ring, wpack, tap + R::DEPTH);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
         {
@@ -80,15 +99,9 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, const _F
                 const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
                 const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
 #pragma unroll
-                for (int n = 0; n < NB; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[kb][n], acc[m][n], 0, 0, 0);
+                for (int n = 0; n < NB; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ring.b[tap % (R::DEPTH + 1)][kb][n], acc[m][n], 0, 0, 0);
             }
-        }
-        if (tap + 1 < 9)
-        {
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int n = 0; n < NB; ++n) bcur[kb][n] = bnext[kb][n];
         }
     }
 }

@@ -58,6 +58,8 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
     const bool has_below = p.Hb > 0;
+    ConvTapRing<CIN, NPAD> ring;
+    conv_taps_prefetch(ring, p.wpack);  // in flight while the patch is assembled
     // weights and biases of the 1x1 output convolution, rounded to fp16 like every other operand
     __shared__ float s_fw[4 * (4 + 64) + 4];
     if (p.final_out)
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 
     __syncthreads();  // patch complete
     floatx4 acc[4][NB];
-    conv_taps_mfma<CIN, NPAD>(s_patch, p.wpack, acc);
+    conv_taps_mfma<CIN, NPAD>(s_patch, p.wpack, ring, acc);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
 
