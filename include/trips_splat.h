@@ -147,8 +147,10 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
                          const float* const grad_image[TRIPS_MAX_LAYERS], const TripsSplatGrads* grads,
                          void* workspace, size_t workspace_bytes, void* stream);
 
-/* Synchronises `stream` and reports a device-side list overflow of the last forward that used `workspace`
- * (only possible when desc->max_list_entries was set below the worst case). */
+/* Synchronises `stream` and reports what the last forward that used `workspace` found on the device: a list
+ * overflow (TRIPS_ERR_LIST_OVERFLOW, only possible when desc->max_list_entries was set below the worst case) or
+ * values of `index` outside [0, num_texels) (TRIPS_ERR_INVALID_ARG; such points are left out of the image, the
+ * reference reads past its tables). */
 int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream);
 
 /* Counters of the last forward of view `view` kept in the saved state: [0]=valid points, [1]=E list entries,

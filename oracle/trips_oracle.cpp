@@ -518,6 +518,8 @@ int oracle_splat_forward(const TripsSplatDesc* desc, const TripsSplatIn* in, con
             r.tex         = in->index[pid];
             r.max_layer   = 0;
             rec[pid]      = r;
+            // a descriptor column outside the table: the reference would read past it; the build leaves the point out
+            if ((unsigned)r.tex >= (unsigned)d.num_texels) continue;
             if (d.viewer_only)
             {
                 // discard_point_for_confidence, RenderForward.cu:122-130

@@ -162,6 +162,24 @@ def test_displacement_forward_backward(oracle):
     _check_backward(oracle, sc, d)
 
 
+def test_index_outside_the_descriptor_table_is_left_out_and_reported(oracle):
+    import ctypes as C
+    from tests.gpu_util import GpuRun
+    from trips_amd import _lib
+    sc = scenes.tiny(n=2000, w=48, h=40, f=45.0, num_layers=3, list_depth=16, seed=12)
+    sc.index = sc.index.copy()
+    sc.index[::7] = -1
+    sc.index[3::11] = sc.texture.shape[1]
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    bad = (sc.index < 0) | (sc.index >= sc.texture.shape[1])
+    assert np.all(ref["depth"][0][bad] == -1)
+    rc = run.ctx.lib.trips_splat_check(run.ctx.ctx, C.c_void_p(run.workspace.data_ptr()), None)
+    assert rc == abi.TRIPS_ERR_INVALID_ARG and b"index" in _lib.load().trips_last_error_string()
+    with pytest.raises(RuntimeError):
+        run.ctx.check(run.workspace)
+
+
 def test_config1_forward_full(oracle):
     sc = scenes.config1()
     _check_forward(oracle, sc, abi.desc_for_scene(sc, train=True))

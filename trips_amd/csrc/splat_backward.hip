@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     const bool want_pose = p.d_pose != nullptr;
     const bool want_intr = p.d_intrinsics != nullptr;
     const bool want_size = p.d_point_size != nullptr;
-    const bool identity  = p.header->reserved[1] == 0;  // index[pid] == pid for every point
+    const bool identity  = p.header->not_identity == 0;  // index[pid] == pid for every point
 
     double acc[NACC];
 #pragma unroll

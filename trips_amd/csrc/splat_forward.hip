@@ -64,7 +64,8 @@ __global__ void clear_header_kernel(ViewHeader* h)
         h->n_valid   = 0;
         h->n_entries = 0;
         h->overflow  = 0;
-        for (int i = 0; i < 5; ++i) h->reserved[i] = 0;
+        h->retained = h->not_identity = h->bad_index = 0;
+        h->reserved[0] = h->reserved[1] = 0;
     }
 }
 
@@ -80,6 +81,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     const int NB       = p.geom.bin_off[L];
     unsigned my_valid  = 0;
     bool not_identity  = false;  // some point's descriptor column differs from its own index
+    bool bad_index     = false;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) s_hist[i] = 0;
     __syncthreads();
 
@@ -92,7 +94,14 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         bool skip   = false;
         const int tex = p.index[pid];
         not_identity |= (tex != pid);
-        if (p.viewer_only)
+        if ((unsigned)tex >= (unsigned)p.num_texels)
+        {
+            // a column outside the descriptor table: leave the point out (reported by the status query) rather
+            // than read past the tables
+            bad_index = true;
+            skip      = true;
+        }
+        if (p.viewer_only && !skip)
         {
             if (p.confidence[tex] < p.stability_cutoff_value) skip = true;
         }
@@ -197,7 +206,8 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         for (int i = 0; i < kBinThreads / 64; ++i) t += s_valid[i];
         if (t) atomicAdd(&p.header->n_valid, (u64)t);
     }
-    if (__ballot(not_identity) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.header->reserved[1], 1ull);
+    if (__ballot(not_identity) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.header->not_identity, 1ull);
+    if (__ballot(bad_index) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.status->bad_index, 1ull);
 }
 
 // ---------------------------------------------------------------------------------------------------------

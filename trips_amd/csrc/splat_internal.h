@@ -158,7 +158,10 @@ struct ViewHeader
     unsigned long long n_valid;     // points that passed the validity test
     unsigned long long n_entries;   // E: total list entries (from the scan)
     unsigned long long overflow;    // entries dropped because the list storage was too small
-    unsigned long long reserved[5];
+    unsigned long long retained;    // R: sum of the retained entries (filled by the counters query)
+    unsigned long long not_identity;  // some point's descriptor column differs from its own index
+    unsigned long long bad_index;   // some point's descriptor column lies outside [0, num_texels): the point was skipped
+    unsigned long long reserved[2];
 };
 
 // Layout of one view's saved state (all offsets in bytes, 256-aligned)

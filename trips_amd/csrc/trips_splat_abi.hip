@@ -493,6 +493,7 @@ int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
     if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync");
     e = hipStreamSynchronize(stream);
     if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    if (h.bad_index) return fail(TRIPS_ERR_INVALID_ARG, "index holds values outside [0, num_texels): those points were left out");
     if (h.overflow) return fail(TRIPS_ERR_LIST_OVERFLOW, "%llu list entries dropped: max_list_entries too small", h.overflow);
     return TRIPS_OK;
 }
@@ -512,7 +513,7 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
     ViewHeader* hd       = reinterpret_cast<ViewHeader*>(sv + sl.header);
     const long long P    = g.off[desc->num_layers];
     const long long Pi   = (long long)g.bin_off[desc->num_layers] * kTilePixels;  // padding rows hold 0
-    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, &hd->reserved[0], stream);
+    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, &hd->retained, stream);
     if (e != hipSuccess) return hip_fail(e, "retained sum");
     ViewHeader h;
     e = hipMemcpyAsync(&h, hd, sizeof(h), hipMemcpyDeviceToHost, stream);
@@ -521,7 +522,7 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
     if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
     counters[0] = (int64_t)h.n_valid;
     counters[1] = (int64_t)h.n_entries;
-    counters[2] = (int64_t)h.reserved[0];
+    counters[2] = (int64_t)h.retained;
     counters[3] = (int64_t)P;
     return TRIPS_OK;
 }
