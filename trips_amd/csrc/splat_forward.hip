@@ -57,6 +57,11 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ p, 
     for (; i < n; i += stride) p[i] = v;
 }
 
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint4* __restrict__ p, long long n)
+{
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
 __global__ void clear_header_kernel(ViewHeader* h)
 {
     if (threadIdx.x == 0)
@@ -349,9 +354,57 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// One workgroup per tile. Pass `SCATTER == false`: count the list length of the tile's 1024 pixels in LDS and
-// write them (plus the tile total). Pass `SCATTER == true` (after the scan of the tile totals): exclusive scan of
-// the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 | point id) into their lists.
+// Slices of split tiles: a tile with more than kSliceEntries bin entries (hundreds of points per pixel, e.g. tight
+// clusters) would keep a single workgroup busy for milliseconds; it is cut into slices of kSliceEntries entries,
+// each a workgroup of its own. slice_start[t] = number of slices of split tiles before tile t (ONE workgroup).
+// Also clears the per-tile key totals, which the slices of a split tile accumulate with atomics.
+__global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restrict__ bin_start, long long capacity, int NB,
+                                                          int32_t* __restrict__ slice_start, int32_t* __restrict__ bin_total)
+{
+    __shared__ int s_wave[16];
+    __shared__ int s_carry;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int base = 0; base < NB; base += 1024)
+    {
+        const int idx = base + threadIdx.x;
+        int v         = 0;
+        if (idx < NB)
+        {
+            const long long first = bin_start[idx];
+            long long last        = bin_start[idx + 1];
+            if (last > capacity) last = capacity;
+            const long long n = last > first ? last - first : 0;
+            v                 = n > kSliceEntries ? (int)((n + kSliceEntries - 1) / kSliceEntries) : 0;
+            bin_total[idx]    = 0;
+        }
+        int inc = v;
+        for (int o = 1; o < 64; o <<= 1)
+        {
+            int t = __shfl_up(inc, o);
+            if (lane >= o) inc += t;
+        }
+        if (lane == 63) s_wave[wave] = inc;
+        __syncthreads();
+        int wave_prefix = 0;
+        for (int w = 0; w < wave; ++w) wave_prefix += s_wave[w];
+        const int carry = s_carry;
+        if (idx < NB) slice_start[idx] = carry + wave_prefix + inc - v;
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = carry + wave_prefix + inc;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) slice_start[NB] = s_carry;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// One workgroup per tile (blocks [0, NB)) plus one per slice of a split tile (blocks from NB on; those past the
+// number of slices the plan found return at once). Pass `SCATTER == false`: count the list length of the tile's
+// 1024 pixels in LDS and write them (plus the tile total). Pass `SCATTER == true` (after the scan of the tile
+// totals): exclusive scan of the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 |
+// point id) into their lists. A slice adds its counts to the tile's with atomics; when it places its keys it first
+// counts its own entries per pixel again and claims that many slots of each pixel's list with one atomic.
 __device__ __forceinline__ void tile_of_bin(const PyramidGeom& g, int bin, int& layer, int& tx, int& ty)
 {
     layer = 0;
@@ -361,49 +414,104 @@ __device__ __forceinline__ void tile_of_bin(const PyramidGeom& g, int bin, int& 
     tx          = t - ty * g.tiles_x[layer];
 }
 
+// Calls f(local pixel index) for each of the entry's 2 x 2 pixels that lie in tile (tx, ty).
+template <typename F>
+__device__ __forceinline__ void for_corners_in_tile(const uint4& e, int tx, int ty, F&& f)
+{
+    const int px = (int)(e.z & 0xffffu), py = (int)(e.z >> 16);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+    {
+        const int x = px + (c & 1), y = py + (c >> 1);
+        if ((x >> kTileShift) == tx && (y >> kTileShift) == ty) f(((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1)));
+    }
+}
+
+// Walks entries [0, n) with the workgroup, four loads of a thread in flight together.
+template <typename F>
+__device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, int n, F&& f)
+{
+    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * 256)
+    {
+        uint4 e[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (i0 + 256 * j < n) e[j] = entries[i0 + 256 * j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (i0 + 256 * j < n) f(e[j]);
+    }
+}
+
 template <bool SCATTER>
 __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
 {
     __shared__ int s_cnt[kTilePixels];
+    __shared__ int s_mine[SCATTER ? kTilePixels : 1];
     __shared__ int s_wave[4];
-    const int bin = blockIdx.x;
+    const int NB = p.geom.bin_off[p.num_layers];
+    int bin      = blockIdx.x;
+    int slice    = -1;  // -1: the tile's own workgroup
+    if (bin >= NB)
+    {
+        const int e = bin - NB;
+        if (e >= p.slice_start[NB]) return;
+        // the tile with slice_start[t] <= e < slice_start[t + 1]: a split one, tiles without slices have empty ranges
+        int lo = 0, hi = NB;
+        while (hi - lo > 1)
+        {
+            const int mid = (lo + hi) >> 1;
+            if (p.slice_start[mid] <= e)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        bin   = lo;
+        slice = e - p.slice_start[bin];
+    }
     int layer, tx, ty;
     tile_of_bin(p.geom, bin, layer, tx, ty);
-    const long long first = p.bin_start[bin];
-    long long last        = p.bin_start[bin + 1];
+    long long first = p.bin_start[bin];
+    long long last  = p.bin_start[bin + 1];
     if (last > p.capacity) last = p.capacity;  // entries beyond the capacity were dropped by the scatter
-    const int n           = first < last ? (int)(last - first) : 0;
-    const uint4* entries  = p.bin_entries + first;
-    int32_t* counts       = p.counts + (size_t)bin * kTilePixels;
+    const bool split = last - first > kSliceEntries;
+    if (slice >= 0)
+    {
+        first += (long long)slice * kSliceEntries;
+        last = min(last, first + kSliceEntries);
+    }
+    const int n          = first < last ? (int)(last - first) : 0;
+    const uint4* entries = p.bin_entries + first;
+    int32_t* counts      = p.counts + (size_t)bin * kTilePixels;
 
     if (!SCATTER)
     {
+        if (split && slice < 0) return;  // the slices do the counting
         for (int i = threadIdx.x; i < kTilePixels; i += 256) s_cnt[i] = 0;
         __syncthreads();
-        for (int i = threadIdx.x; i < n; i += 256)
-        {
-            const uint4 e = entries[i];
-            const int px = (int)(e.z & 0xffffu), py = (int)(e.z >> 16);
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-            {
-                const int x = px + (c & 1), y = py + (c >> 1);
-                if ((x >> kTileShift) == tx && (y >> kTileShift) == ty)
-                    atomicAdd(&s_cnt[((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1))], 1);
-            }
-        }
+        for_entries(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&s_cnt[i], 1); }); });
         __syncthreads();
         int sum = 0;
         for (int i = threadIdx.x; i < kTilePixels; i += 256)
         {
             const int c = s_cnt[i];
-            counts[i]   = c;
+            if (slice < 0)
+                counts[i] = c;
+            else if (c)
+                atomicAdd(&counts[i], c);  // cleared before this kernel
             sum += c;
         }
         for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
         if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = sum;
         __syncthreads();
-        if (threadIdx.x == 0) p.bin_total[bin] = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+        if (threadIdx.x == 0)
+        {
+            const int total = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+            if (slice < 0)
+                p.bin_total[bin] = total;
+            else
+                atomicAdd(&p.bin_total[bin], total);
+        }
         return;
     }
 
@@ -424,6 +532,8 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
         if (lane >= o) inc += t;
     }
     if (lane == 63) s_wave[wave] = inc;
+    if (slice >= 0)
+        for (int i = threadIdx.x; i < kTilePixels; i += 256) s_mine[SCATTER ? i : 0] = 0;
     __syncthreads();
     int prefix = inc - sum;
     for (int w = 0; w < wave; ++w) prefix += s_wave[w];
@@ -432,38 +542,63 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
 #pragma unroll
     for (int i = 0; i < 4; ++i)
     {
-        s_cnt[base4 + i]  = key_start + prefix;  // running slot of the pixel
-        cursor[base4 + i] = key_start + prefix;
+        s_cnt[base4 + i] = key_start + prefix;  // running slot of the pixel
+        if (slice < 0) cursor[base4 + i] = key_start + prefix;
         prefix += v[i];
     }
+    if (split && slice < 0) return;  // the slices place the keys
     __syncthreads();
+    unsigned dropped = 0;
+    if (slice >= 0)
+    {
+        // this slice's share of every pixel's list: count, then claim the slots with one atomic per pixel
+        int32_t* run = p.run + (size_t)bin * kTilePixels;
+        for_entries(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&s_mine[SCATTER ? i : 0], 1); }); });
+        __syncthreads();
+        for (int i = threadIdx.x; i < kTilePixels; i += 256)
+        {
+            const int c = s_mine[SCATTER ? i : 0];
+            if (c) s_cnt[i] += atomicAdd(&run[i], c);  // cleared before the counting kernel
+        }
+        __syncthreads();
+        for_entries(entries, n,
+                    [&](const uint4& e)
+                    {
+                        const u64 key = ((u64)e.x << 32) | (u64)e.y;
+                        for_corners_in_tile(e, tx, ty,
+                                            [&](int i)
+                                            {
+                                                const int slot = atomicAdd(&s_cnt[i], 1);
+                                                if ((long long)slot < p.capacity)
+                                                    p.keys[slot] = key;
+                                                else
+                                                    dropped += 1;
+                                            });
+                    });
+        if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
+        return;
+    }
     // Keys of a tile whose lists fit into LDS are staged there and copied out with full-line stores; the keys of
     // bigger tiles go to their lists directly (8-byte stores scattered over the tile's region).
     extern __shared__ u64 s_keys[];
     const int tile_total = p.bin_key_start[bin + 1] - key_start;
     const bool staged    = tile_total <= kStageKeys && (long long)key_start + tile_total <= p.capacity;
-    unsigned dropped     = 0;
-    for (int i = threadIdx.x; i < n; i += 256)
-    {
-        const uint4 e = entries[i];
-        const int px = (int)(e.z & 0xffffu), py = (int)(e.z >> 16);
-        const u64 key = ((u64)e.x << 32) | (u64)e.y;
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-        {
-            const int x = px + (c & 1), y = py + (c >> 1);
-            if ((x >> kTileShift) == tx && (y >> kTileShift) == ty)
-            {
-                const int slot = atomicAdd(&s_cnt[((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1))], 1);
-                if (staged)
-                    s_keys[slot - key_start] = key;
-                else if ((long long)slot < p.capacity)
-                    p.keys[slot] = key;
-                else
-                    dropped += 1;
-            }
-        }
-    }
+    for_entries(entries, n,
+                [&](const uint4& e)
+                {
+                    const u64 key = ((u64)e.x << 32) | (u64)e.y;
+                    for_corners_in_tile(e, tx, ty,
+                                        [&](int i)
+                                        {
+                                            const int slot = atomicAdd(&s_cnt[i], 1);
+                                            if (staged)
+                                                s_keys[slot - key_start] = key;
+                                            else if ((long long)slot < p.capacity)
+                                                p.keys[slot] = key;
+                                            else
+                                                dropped += 1;
+                                        });
+                });
     if (staged)
     {
         __syncthreads();
@@ -525,25 +660,48 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     maxlen     = max(maxlen, __shfl_xor(maxlen, 16));
     maxlen     = max(maxlen, __shfl_xor(maxlen, 32));
     const u64 grp_mask = 0xFFFFull << (grp * 16);
-    for (int base = 0; base < maxlen; base += 16)
+    maxlen             = __builtin_amdgcn_readfirstlane(maxlen);
     {
         u64 k = kInf;
-        if (base + sub < readable) k = p.keys[start + base + sub];
-        if (base == 0)
+        if (sub < readable) k = p.keys[start + sub];
+        best = row_sort16(k);
+    }
+    // A chunk of 16 further keys is sorted and merged only if one of them beats the current 16th; most chunks of a
+    // long list are passed over, so the loop runs at the latency of its loads: four chunks are requested together
+    // and the next four are in flight while these are looked at.
+    auto load4 = [&](int base, u64 (&kk)[4])
+    {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
         {
-            best = row_sort16(k);
+            const int i = base + 16 * j + sub;
+            kk[j]       = i < readable ? p.keys[start + i] : kInf;
         }
-        else
+    };
+    if (maxlen > 16)
+    {
+        u64 cur[4], nxt[4];
+        load4(16, cur);
+        for (int base = 16; base < maxlen; base += 64)
         {
-            const u64 worst = shfl16(best, 15);
-            const bool need = k < worst;
-            if (__ballot(need) & grp_mask)
+            if (base + 64 < maxlen) load4(base + 64, nxt);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
             {
-                k           = row_sort16(k);
-                const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
-                best        = best < r ? best : r;
-                best        = row_merge16(best);
+                if (base + 16 * j >= maxlen) break;
+                u64 k           = cur[j];
+                const u64 worst = shfl16(best, 15);
+                const bool need = k < worst;
+                if (__ballot(need) & grp_mask)
+                {
+                    k           = row_sort16(k);
+                    const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
+                    best        = best < r ? best : r;
+                    best        = row_merge16(best);
+                }
             }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
         }
     }
     }
@@ -721,9 +879,17 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         ProfScope ps(prof, "bin_scatter", stream);
         hipLaunchKernelGGL(bin_scatter_kernel, dim3(G), dim3(kBinThreads), lds_hist, stream, p);
     }
+    // workgroups for the slices of split tiles: at most capacity / kSliceEntries full slices plus one partial slice
+    // per split tile
+    const int max_slices = (int)std::min<long long>(2 * (p.capacity / kSliceEntries) + 1, 1 << 20);
     {
         ProfScope ps(prof, "tile_count", stream);
-        hipLaunchKernelGGL((tile_lists_kernel<false>), dim3(NB), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(slice_plan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_start, p.capacity, NB, p.slice_start, p.bin_total);
+        // counts and run are neighbours in the workspace: one fill clears both
+        const long long words = 2ll * NB * kTilePixels;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)std::min<long long>((words / 4 + 255) / 256, 4096)), dim3(256), 0, stream,
+                           reinterpret_cast<uint4*>(p.counts), words / 4);
+        hipLaunchKernelGGL((tile_lists_kernel<false>), dim3(NB + max_slices), dim3(256), 0, stream, p);
     }
     {
         ProfScope ps(prof, "tile_scan", stream);
@@ -732,7 +898,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     }
     {
         ProfScope ps(prof, "tile_scatter", stream);
-        hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB), dim3(256), kStageKeys * sizeof(u64), stream, p);
+        hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB + max_slices), dim3(256), kStageKeys * sizeof(u64), stream, p);
     }
     {
         ProfScope ps(prof, "sort_blend", stream);

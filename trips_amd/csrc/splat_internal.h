@@ -107,6 +107,8 @@ constexpr int kTilePixels = kTile * kTile;
 constexpr int kBinThreads = 512;    // workgroup size of the two binning kernels
 constexpr int kBinGroups  = 512;    // workgroups (= contiguous chunks of points) of the two binning kernels
 constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
+// bin entries of a tile above which the tile is split into slices of that many entries, one workgroup each
+constexpr int kSliceEntries = 8192;
 constexpr int kStageKeys  = 7168;   // keys of one tile staged in LDS before they are written (56 KB)
 
 struct PyramidGeom
@@ -188,6 +190,8 @@ struct WorkspaceLayout
     size_t ptk;          // float4 [N]   {ip.x, ip.y, depth (-1 culled), max_layer bits}
     size_t counts;       // int32 [Pi]   list length per pixel
     size_t cursor;       // int32 [Pi]   first key of each pixel's list
+    size_t run;          // int32 [Pi]   keys of a pixel already claimed by slices of a split tile (zeroed per view)
+    size_t slice_start;  // int32 [NB+1] exclusive scan of the slices of split tiles (0 for a tile that is not split)
     size_t bin_count;    // int32 [NB]   bin entries per tile
     size_t bin_start;    // int32 [NB+1] exclusive scan of bin_count
     size_t bin_hist;     // int32 [G, NB] bin entries per (workgroup, tile), then its column-wise exclusive prefix
@@ -232,6 +236,8 @@ struct ForwardParams
     int32_t bin_groups, points_per_block;
     int32_t* bin_total;
     int32_t* bin_key_start;
+    int32_t* run;
+    int32_t* slice_start;
     uint4* bin_entries;
     unsigned long long* keys;
     long long capacity;

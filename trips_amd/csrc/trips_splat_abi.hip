@@ -219,8 +219,12 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(N * sizeof(float4));
     w.counts = o;
     o += align256(P * sizeof(int32_t));
+    w.run = o;  // directly behind counts: one fill clears both
+    o += align256(P * sizeof(int32_t));
     w.cursor = o;
     o += align256(P * sizeof(int32_t));
+    w.slice_start = o;
+    o += align256((NB + 1) * sizeof(int32_t));
     w.bin_count = o;
     o += align256(NB * sizeof(int32_t));
     w.bin_start = o;
@@ -387,6 +391,8 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
         p.points_per_block = (d.num_points + kBinGroups - 1) / kBinGroups;
         p.bin_total  = reinterpret_cast<int32_t*>(ws + wl.bin_total);
         p.bin_key_start = reinterpret_cast<int32_t*>(ws + wl.bin_key_start);
+        p.run         = reinterpret_cast<int32_t*>(ws + wl.run);
+        p.slice_start = reinterpret_cast<int32_t*>(ws + wl.slice_start);
         p.bin_entries   = reinterpret_cast<uint4*>(ws + wl.bin_entries);
         p.keys       = reinterpret_cast<unsigned long long*>(ws + wl.keys);
         p.capacity   = (long long)wl.capacity;
