@@ -180,6 +180,29 @@ def test_index_outside_the_descriptor_table_is_left_out_and_reported(oracle):
         run.ctx.check(run.workspace)
 
 
+def test_tight_cluster_long_lists_and_split_tiles(oracle):
+    """Thousands of points on a handful of pixels: lists far longer than the segment length of the long-list
+    reduction (1024 / 512 keys) and tiles with more bin entries than a slice (8192), with exact depth ties."""
+    sc = scenes.tiny(n=30000, w=96, h=64, f=80.0, num_layers=4, list_depth=16, seed=91, radius=(0.004, 0.2))
+    rng = np.random.default_rng(3)
+    sc.position[:, :3] = (rng.normal(0, 0.004, (30000, 3)) + np.array([0.05, -0.02, 0.0])).astype(np.float32)
+    sc.position[:2000, 2] = sc.position[0, 2]  # equal depths: the tie-break by point id decides
+    sc.position[5000:5600, :3] = rng.uniform(-1, 1, (600, 3)).astype(np.float32)  # some ordinary pixels too
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert ref["lengths"].max() > 3000
+    c = run.ctx.counters(d, run.saved, 0)
+    assert c["E"] > 4 * 8192
+    _check_backward(oracle, sc, d)
+    # the same with a list storage that is too small: no fault, the overflow is reported
+    d_small = abi.desc_for_scene(sc, max_list_entries=20000)
+    from tests.gpu_util import GpuRun
+    small = GpuRun(sc, d_small)
+    small.forward()
+    with pytest.raises(RuntimeError):
+        small.ctx.check(small.workspace)
+
+
 def test_config1_forward_full(oracle):
     sc = scenes.config1()
     _check_forward(oracle, sc, abi.desc_for_scene(sc, train=True))

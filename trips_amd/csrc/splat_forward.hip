@@ -359,8 +359,10 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
 // each a workgroup of its own. slice_start[t] = number of slices of split tiles before tile t (ONE workgroup).
 // Also clears the per-tile key totals, which the slices of a split tile accumulate with atomics.
 __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restrict__ bin_start, long long capacity, int NB,
-                                                          int32_t* __restrict__ slice_start, int32_t* __restrict__ bin_total)
+                                                          int32_t* __restrict__ slice_start, int32_t* __restrict__ bin_total,
+                                                          int32_t* __restrict__ long_count)
 {
+    if (threadIdx.x == 0) *long_count = 0;
     __shared__ int s_wave[16];
     __shared__ int s_carry;
     if (threadIdx.x == 0) s_carry = 0;
@@ -543,7 +545,23 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     for (int i = 0; i < 4; ++i)
     {
         s_cnt[base4 + i] = key_start + prefix;  // running slot of the pixel
-        if (slice < 0) cursor[base4 + i] = key_start + prefix;
+        if (slice < 0)
+        {
+            int where = key_start + prefix;
+            if (v[i] > kLongList && (long long)key_start + prefix + v[i] <= p.capacity)
+            {
+                // a long list: hand its segments to the reduction pass and point the pixel at their results
+                const int nseg = (v[i] + kLongSegment - 1) / kLongSegment;
+                const int base = atomicAdd(p.long_count, nseg);
+                if (base + nseg <= p.max_long_items)
+                {
+                    for (int sg = 0; sg < nseg; ++sg)
+                        p.long_items[base + sg] = make_int2(key_start + prefix + sg * kLongSegment, min(kLongSegment, v[i] - sg * kLongSegment));
+                    where = -1 - base;
+                }
+            }
+            cursor[base4 + i] = where;
+        }
         prefix += v[i];
     }
     if (split && slice < 0) return;  // the slices place the keys
@@ -617,6 +635,83 @@ __device__ __forceinline__ u64 shfl16(u64 v, int src)
     return ((u64)hi << 32) | lo;
 }
 
+// The 16 smallest of keys[start, start + readable) for each of the wavefront's four 16-lane rows, ascending over
+// the row's lanes (all-ones where the list is shorter).
+__device__ __forceinline__ u64 row_top16(const u64* __restrict__ keys, long long start, int readable)
+{
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & 15, grp = lane >> 4;
+    const u64 kInf = ~0ull;
+    u64 best;
+    int maxlen = readable;
+    maxlen     = max(maxlen, __shfl_xor(maxlen, 16));
+    maxlen     = max(maxlen, __shfl_xor(maxlen, 32));
+    const u64 grp_mask = 0xFFFFull << (grp * 16);
+    maxlen             = __builtin_amdgcn_readfirstlane(maxlen);
+    {
+        u64 k = kInf;
+        if (sub < readable) k = keys[start + sub];
+        best = row_sort16(k);
+    }
+    // A chunk of 16 further keys is sorted and merged only if one of them beats the current 16th; most chunks of a
+    // long list are passed over, so the loop runs at the latency of its loads: four chunks are requested together
+    // and the next four are in flight while these are looked at.
+    auto load4 = [&](int base, u64 (&kk)[4])
+    {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const int i = base + 16 * j + sub;
+            kk[j]       = i < readable ? keys[start + i] : kInf;
+        }
+    };
+    if (maxlen > 16)
+    {
+        u64 cur[4], nxt[4];
+        load4(16, cur);
+        for (int base = 16; base < maxlen; base += 64)
+        {
+            if (base + 64 < maxlen) load4(base + 64, nxt);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                if (base + 16 * j >= maxlen) break;
+                u64 k           = cur[j];
+                const u64 worst = shfl16(best, 15);
+                const bool need = k < worst;
+                if (__ballot(need) & grp_mask)
+                {
+                    k           = row_sort16(k);
+                    const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
+                    best        = best < r ? best : r;
+                    best        = row_merge16(best);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
+        }
+    }
+    return best;
+}
+
+// Reduction pass over the segments of long lists (tile_lists_kernel hands them out): a 16-lane row keeps the 16
+// smallest keys of a segment. Persistent workgroups, the four rows of a wavefront take consecutive segments.
+__global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardParams p)
+{
+    const int n    = min(*p.long_count, p.max_long_items);
+    const int lane = threadIdx.x & 63;
+    const int rows = gridDim.x * 16;
+    for (int first = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 4; first < n; first += rows)
+    {
+        const int item = first + (lane >> 4);
+        int2 seg       = make_int2(0, 0);
+        if (item < n) seg = p.long_items[item];
+        if (seg.x < 0 || seg.y < 0 || seg.y > kLongSegment || (long long)seg.x + seg.y > p.capacity) seg = make_int2(0, 0);
+        const u64 best = row_top16(p.keys, seg.x, seg.y);
+        if (item < n) p.cand[(size_t)item * 16 + (lane & 15)] = best;
+    }
+}
+
 // Top-16 of each pixel list by key, then the alpha blend, for 64 / ROW consecutive pixels starting at `pix_first`:
 // ROW = 16 lanes per pixel (one DPP row; lists of any length stream through in chunks of 16), or ROW = 8 when no
 // list of the group is longer than 8 (two thirds of the pixels of a typical view have at most 4 entries: half the
@@ -656,54 +751,15 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     }
     else
     {
-    int maxlen = readable;
-    maxlen     = max(maxlen, __shfl_xor(maxlen, 16));
-    maxlen     = max(maxlen, __shfl_xor(maxlen, 32));
-    const u64 grp_mask = 0xFFFFull << (grp * 16);
-    maxlen             = __builtin_amdgcn_readfirstlane(maxlen);
+    const u64* src = p.keys;
+    if (start < 0)
     {
-        u64 k = kInf;
-        if (sub < readable) k = p.keys[start + sub];
-        best = row_sort16(k);
+        // a long list: the reduction pass left the 16 smallest keys of each of its segments
+        src      = p.cand;
+        start    = (-1 - start) * 16ll;
+        readable = ((len + kLongSegment - 1) / kLongSegment) * 16;
     }
-    // A chunk of 16 further keys is sorted and merged only if one of them beats the current 16th; most chunks of a
-    // long list are passed over, so the loop runs at the latency of its loads: four chunks are requested together
-    // and the next four are in flight while these are looked at.
-    auto load4 = [&](int base, u64 (&kk)[4])
-    {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-        {
-            const int i = base + 16 * j + sub;
-            kk[j]       = i < readable ? p.keys[start + i] : kInf;
-        }
-    };
-    if (maxlen > 16)
-    {
-        u64 cur[4], nxt[4];
-        load4(16, cur);
-        for (int base = 16; base < maxlen; base += 64)
-        {
-            if (base + 64 < maxlen) load4(base + 64, nxt);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-            {
-                if (base + 16 * j >= maxlen) break;
-                u64 k           = cur[j];
-                const u64 worst = shfl16(best, 15);
-                const bool need = k < worst;
-                if (__ballot(need) & grp_mask)
-                {
-                    k           = row_sort16(k);
-                    const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
-                    best        = best < r ? best : r;
-                    best        = row_merge16(best);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
-        }
-    }
+    best = row_top16(src, start, readable);
     }
 
     // ---- blend (RenderForward.cu:820-1048) ----
@@ -884,7 +940,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     const int max_slices = (int)std::min<long long>(2 * (p.capacity / kSliceEntries) + 1, 1 << 20);
     {
         ProfScope ps(prof, "tile_count", stream);
-        hipLaunchKernelGGL(slice_plan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_start, p.capacity, NB, p.slice_start, p.bin_total);
+        hipLaunchKernelGGL(slice_plan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_start, p.capacity, NB, p.slice_start, p.bin_total, p.long_count);
         // counts and run are neighbours in the workspace: one fill clears both
         const long long words = 2ll * NB * kTilePixels;
         hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)std::min<long long>((words / 4 + 255) / 256, 4096)), dim3(256), 0, stream,
@@ -899,6 +955,11 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     {
         ProfScope ps(prof, "tile_scatter", stream);
         hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB + max_slices), dim3(256), kStageKeys * sizeof(u64), stream, p);
+    }
+    {
+        ProfScope ps(prof, "long_lists", stream);
+        const int blocks = std::min((p.max_long_items + 15) / 16, 2048);
+        hipLaunchKernelGGL(long_list_reduce_kernel, dim3(blocks), dim3(256), 0, stream, p);
     }
     {
         ProfScope ps(prof, "sort_blend", stream);

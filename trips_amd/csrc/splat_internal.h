@@ -109,6 +109,10 @@ constexpr int kBinGroups  = 512;    // workgroups (= contiguous chunks of points
 constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
 // bin entries of a tile above which the tile is split into slices of that many entries, one workgroup each
 constexpr int kSliceEntries = 8192;
+// A pixel list longer than kLongList keys is cut into segments of kLongSegment keys; a pass of its own keeps the 16
+// smallest keys of every segment (a 16-lane row each), and the blend kernel then sorts those instead of the list.
+constexpr int kLongList    = 1024;
+constexpr int kLongSegment = 512;
 constexpr int kStageKeys  = 7168;   // keys of one tile staged in LDS before they are written (56 KB)
 
 struct PyramidGeom
@@ -192,6 +196,10 @@ struct WorkspaceLayout
     size_t cursor;       // int32 [Pi]   first key of each pixel's list
     size_t run;          // int32 [Pi]   keys of a pixel already claimed by slices of a split tile (zeroed per view)
     size_t slice_start;  // int32 [NB+1] exclusive scan of the slices of split tiles (0 for a tile that is not split)
+    size_t long_count;   // int32 [1]    segments of long lists handed out so far
+    size_t long_items;   // int2  [max_long_items] {first key, number of keys} of each segment of a long list
+    size_t cand;         // uint64 [max_long_items * 16] the 16 smallest keys of each segment
+    size_t max_long_items;
     size_t bin_count;    // int32 [NB]   bin entries per tile
     size_t bin_start;    // int32 [NB+1] exclusive scan of bin_count
     size_t bin_hist;     // int32 [G, NB] bin entries per (workgroup, tile), then its column-wise exclusive prefix
@@ -238,6 +246,10 @@ struct ForwardParams
     int32_t* bin_key_start;
     int32_t* run;
     int32_t* slice_start;
+    int32_t* long_count;
+    int2* long_items;
+    unsigned long long* cand;
+    int32_t max_long_items;
     uint4* bin_entries;
     unsigned long long* keys;
     long long capacity;

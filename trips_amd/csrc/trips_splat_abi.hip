@@ -225,6 +225,14 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(P * sizeof(int32_t));
     w.slice_start = o;
     o += align256((NB + 1) * sizeof(int32_t));
+    // every long list has at least kLongList / kLongSegment full segments, so the partial ones add at most half
+    w.max_long_items = std::min<size_t>(w.capacity / kLongSegment * 3 / 2 + 16, (size_t)1 << 27);
+    w.long_count     = o;
+    o += align256(sizeof(int32_t));
+    w.long_items = o;
+    o += align256(w.max_long_items * sizeof(int2));
+    w.cand = o;
+    o += align256(w.max_long_items * 16 * sizeof(unsigned long long));
     w.bin_count = o;
     o += align256(NB * sizeof(int32_t));
     w.bin_start = o;
@@ -393,6 +401,10 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
         p.bin_key_start = reinterpret_cast<int32_t*>(ws + wl.bin_key_start);
         p.run         = reinterpret_cast<int32_t*>(ws + wl.run);
         p.slice_start = reinterpret_cast<int32_t*>(ws + wl.slice_start);
+        p.long_count  = reinterpret_cast<int32_t*>(ws + wl.long_count);
+        p.long_items  = reinterpret_cast<int2*>(ws + wl.long_items);
+        p.cand        = reinterpret_cast<unsigned long long*>(ws + wl.cand);
+        p.max_long_items = (int32_t)wl.max_long_items;
         p.bin_entries   = reinterpret_cast<uint4*>(ws + wl.bin_entries);
         p.keys       = reinterpret_cast<unsigned long long*>(ws + wl.keys);
         p.capacity   = (long long)wl.capacity;
