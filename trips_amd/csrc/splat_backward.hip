@@ -225,9 +225,10 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     const bool want_size = p.d_point_size != nullptr;
     const bool identity  = p.header->not_identity == 0;  // index[pid] == pid for every point
 
-    double acc[NACC];
+    // a thread sees a handful of points: its own sums stay in single precision, everything across threads is double
+    float acc[NACC];
 #pragma unroll
-    for (int i = 0; i < NACC; ++i) acc[i] = 0.0;
+    for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
 
     for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
     {
@@ -352,14 +353,14 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         if (want_pose)
         {
 #pragma unroll
-            for (int k = 0; k < 6; ++k) acc[k] += (double)g_pose[k];
+            for (int k = 0; k < 6; ++k) acc[k] += g_pose[k];
         }
         if (want_intr)
         {
 #pragma unroll
-            for (int k = 0; k < 5; ++k) acc[6 + k] += (double)g_k[k];
+            for (int k = 0; k < 5; ++k) acc[6 + k] += g_k[k];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) acc[11 + k] += (double)g_dis[k];
+            for (int k = 0; k < 8; ++k) acc[11 + k] += g_dis[k];
         }
     }
 
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     {
         const bool used = (i < 6) ? want_pose : want_intr;
         if (!used) continue;
-        double v = wave_sum(acc[i]);
+        double v = wave_sum((double)acc[i]);
         if (lane == 0) s_acc[threadIdx.x >> 6][i] = v;
     }
     __syncthreads();

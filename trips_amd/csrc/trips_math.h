@@ -294,7 +294,7 @@ __device__ __forceinline__ void project_backward(const Camera& cam, const float 
     float nx = vx * iz, ny = vy * iz;
     float Jp[4], Jd[16];
     float dx, dy;
-    distort(nx, ny, cam.dist, cam.dist_cutoff, dx, dy, Jp, want_intrinsics ? Jd : nullptr);
+    distort(nx, ny, cam.dist, cam.dist_cutoff, dx, dy, Jp, Jd);  // a pointer chosen at run time would put the arrays in scratch memory
     float gr0 = cam.r00 * g0 + cam.r10 * g1;
     float gr1 = cam.r01 * g0 + cam.r11 * g1;
     float a   = cam.cfx * gr0;
