@@ -212,4 +212,21 @@ __device__ __forceinline__ float row_exclusive_suffix_sum(float v)
     return s;
 }
 
+// the same per half row
+__device__ __forceinline__ float half_exclusive_suffix_sum(float v)
+{
+    // positions whose source (i + S) lies in the same half: S = 1 -> all but 7 and 15, S = 2 -> 0..5 and 8..13,
+    // S = 4 -> 0..3 and 8..11
+    constexpr u64 k1 = rows4(0x7F7Fu), k2 = rows4(0x3F3Fu), k4 = rows4(0x0F0Fu);
+    float t = row_shl0<1>(v);
+    float s = __builtin_amdgcn_inverse_ballot_w64(k1) ? t : 0.f;
+    t       = row_shl0<1>(s);
+    s += __builtin_amdgcn_inverse_ballot_w64(k1) ? t : 0.f;
+    t = row_shl0<2>(s);
+    s += __builtin_amdgcn_inverse_ballot_w64(k2) ? t : 0.f;
+    t = row_shl0<4>(s);
+    s += __builtin_amdgcn_inverse_ballot_w64(k4) ? t : 0.f;
+    return s;
+}
+
 }  // namespace trips

@@ -7,7 +7,7 @@
 // (3 position + 1 size + 1 confidence + C descriptor atomics per retained entry). Scattered atomics run at
 // about 2e10 per second on this GPU while scattered loads run at 5e10 and cost the same for 4 or 64 bytes,
 // so the work is split in two passes without atomics on the per-point arrays:
-//   1. pixels: a 16-lane row owns a pixel, each lane one retained entry. Alpha and transmittance are recomputed
+//   1. pixels: a 16-lane row (an 8-lane half row for short lists) owns a pixel, each lane one retained entry. Alpha and transmittance are recomputed
 //      from the per-point record exactly as the forward computed them; the "all later entries" sum of
 //      RenderBackward.cu:284-301 is a suffix sum across the row. Per entry it writes {dL/dalpha, T*alpha*dL/dimage}
 //      into the pixel's row of a [P,K] table and one byte, the entry's rank, into the point's 32-slot table
@@ -61,40 +61,29 @@ __device__ __forceinline__ double wave_sum(double v)
 
 // ---------------------------------------------------------------------------------------------------------
 // Pass 1: per pixel row. Writes entry_grad[pix*K + j] = {dL/dalpha_j, T_j alpha_j g[0..C)} and rank[pid*32 + slot] = j.
-template <int C>
-__global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardParams p)
+// 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
+// than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
+template <int C, int ROW>
+__device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, long long pix_first, int m_in, double (&acc_bg)[C])
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int EF   = (1 + C + 3) & ~3;  // floats per entry of entry_grad
     const int lane     = threadIdx.x & 63;
-    const int sub      = lane & 15;
-    const int grp      = lane >> 4;
+    const int sub      = lane & (ROW - 1);
+    const int grp      = lane / ROW;
     const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
-
-    double acc_bg[C];
-#pragma unroll
-    for (int i = 0; i < C; ++i) acc_bg[i] = 0.0;
-
-    // a workgroup walks whole tiles (256 pixel quads each), 4 workgroups per tile, all on one XCD
-    constexpr int kPerTile      = 4;
-    const long long total_waves = ((long long)P + 3) / 4;
-    const long long num_tiles   = p.geom.bin_off[p.num_layers];
-    const long long tile_stride = (long long)(gridDim.x / (kPerTile * kNumXcd)) * kNumXcd;
-
-    for (long long lb = xcd_tile_block(blockIdx.x, kPerTile); lb < num_tiles * kPerTile; lb += tile_stride * kPerTile)
-    for (long long wv = lb * (kTilePixels / 4 / kPerTile) + (threadIdx.x >> 6); wv < (lb + 1) * (kTilePixels / 4 / kPerTile); wv += 4)
     {
-        if (wv >= total_waves) break;
-        const long long pix_ll = wv * 4 + grp;
+        const long long pix_ll = pix_first + grp;
         const int pix          = pix_ll < P ? (int)pix_ll : 0;
         int layer, gx, gy;
         const bool live = pix_decode(p.geom, pix, layer, gx, gy) && pix_ll < P;
         const int lw = p.geom.w[layer], lh = p.geom.h[layer];
 
-        const int m    = live ? p.retained[pix] : 0;
+        const int m    = live ? m_in : 0;
         const bool has = sub < m;
         int mmax       = m;
+        if (ROW == 8) mmax = max(mmax, __shfl_xor(mmax, 8));
         mmax           = max(mmax, __shfl_xor(mmax, 16));
         mmax           = max(mmax, __shfl_xor(mmax, 32));
         mmax           = __builtin_amdgcn_readfirstlane(mmax);
@@ -149,11 +138,11 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
         }
 
         // exclusive transmittance, same chain as the forward
-        const float T = row_exclusive_product(1.f - a, mmax);
+        const float T = ROW == 8 ? half_exclusive_product(1.f - a, mmax) : row_exclusive_product(1.f - a, mmax);
         // transmittance after the m retained entries decides whether the background is reached
         // (RenderBackward.cu:205-210,302-308)
         float T_after = T * (1.f - a);
-        T_after       = __shfl(T_after, max(m - 1, 0), 16);
+        T_after       = __shfl(T_after, max(m - 1, 0), ROW);
         if (m == 0) T_after = 1.f;
         const bool bg_reached = live && (T_after >= 0.001f);
 
@@ -166,7 +155,7 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
         }
         const float ta = T * a;
         const float q  = has ? ta * s : 0.f;
-        float later    = row_exclusive_suffix_sum(q);  // entries i > j
+        float later    = ROW == 8 ? half_exclusive_suffix_sum(q) : row_exclusive_suffix_sum(q);  // entries i > j
         if (bg_reached) later += T_after * sbg;
         const float dem        = 1.f / (1.f - a + 1e-9f);
         const float grad_alpha = T * s - later * dem;
@@ -189,6 +178,50 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
 #pragma unroll
             for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
             p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
+        }
+    }
+
+}
+
+template <int C>
+__global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardParams p)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int P    = p.geom.bin_off[p.num_layers] * kTilePixels;
+    double acc_bg[C];
+#pragma unroll
+    for (int i = 0; i < C; ++i) acc_bg[i] = 0.0;
+
+    // A workgroup walks quarters of tiles (256 pixels = 32 groups of eight), 4 workgroups per tile, all on one XCD.
+    // A wavefront takes every fourth group; it reads the retained counts of all its 64 pixels with one load, so the
+    // choice of the row width and the rows' own lengths cost no further memory round trip.
+    constexpr int kPerTile      = 4;
+    constexpr int kQuarter      = kTilePixels / kPerTile;
+    const long long num_tiles   = p.geom.bin_off[p.num_layers];
+    const long long tile_stride = (long long)(gridDim.x / (kPerTile * kNumXcd)) * kNumXcd;
+
+    for (long long lb = xcd_tile_block(blockIdx.x, kPerTile); lb < num_tiles * kPerTile; lb += tile_stride * kPerTile)
+    {
+        // lane -> pixel (lane % 8) of this wavefront's group number lane / 8
+        const long long my_pix = lb * kQuarter + ((lane >> 3) * 4 + wave) * 8 + (lane & 7);
+        int m_all              = my_pix < P ? p.retained[my_pix] : 0;  // 0 for the padding of partial tiles
+        int m_grp              = m_all;
+        m_grp                  = max(m_grp, __shfl_xor(m_grp, 1));
+        m_grp                  = max(m_grp, __shfl_xor(m_grp, 2));
+        m_grp                  = max(m_grp, __shfl_xor(m_grp, 4));
+#pragma unroll 1
+        for (int it = 0; it < 8; ++it)
+        {
+            const long long pix_first = lb * kQuarter + (it * 4 + wave) * 8;
+            if (pix_first >= P) break;
+            const int m8 = __builtin_amdgcn_readfirstlane(__shfl(m_grp, it * 8));
+            if (m8 <= 8)
+                backward_pixel_rows<C, 8>(p, pix_first, __shfl(m_all, it * 8 + (lane >> 3)), acc_bg);
+            else
+            {
+                backward_pixel_rows<C, 16>(p, pix_first, __shfl(m_all, it * 8 + (lane >> 4)), acc_bg);
+                backward_pixel_rows<C, 16>(p, pix_first + 4, __shfl(m_all, it * 8 + 4 + (lane >> 4)), acc_bg);
+            }
         }
     }
 

@@ -717,7 +717,8 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
 // list of the group is longer than 8 (two thirds of the pixels of a typical view have at most 4 entries: half the
 // lanes of a 16-lane row would idle through every instruction).
 template <int C, bool TRAIN, int ROW>
-__device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long long pix_first, bool group_in_range)
+__device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long long pix_first, bool group_in_range, int len_in,
+                                                int start_in)
 {
     constexpr int CPAD = (C + 3) & ~3;
     const int lane     = threadIdx.x & 63;
@@ -731,13 +732,9 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     int layer, gx, gy;
     const bool live = pix_decode(p.geom, pix, layer, gx, gy) && in_range;  // false for the padding of partial tiles
 
-    int len = 0;
-    long long start = 0;
-    if (live)
-    {
-        len   = p.counts[pix];
-        start = p.cursor[pix];
-    }
+    // length and first key of this lane's list: the caller has read them for the whole group
+    const int len   = live ? len_in : 0;
+    long long start = live ? start_in : 0;
     // entries beyond the capacity were never written
     int readable = len;
     if (start + len > p.capacity) readable = (int)max(0ll, p.capacity - start);
@@ -866,28 +863,26 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     const long long pix_first   = (lblock * 4 + (threadIdx.x >> 6)) * 8;
     const bool group_in_range   = lblock < nblocks;
     // longest list of the eight pixels (lists that ran past the key storage count with what was written)
-    int len8 = 0;
+    int len8 = 0, my_len = 0, my_start = 0;  // lanes 0..7: one pixel of the group each
     if (lane < 8 && group_in_range && pix_first + lane < P)
     {
         const int pix = (int)(pix_first + lane);
-        int layer, gx, gy;
-        if (pix_decode(p.geom, pix, layer, gx, gy))
-        {
-            len8 = p.counts[pix];
-            const long long start = p.cursor[pix];
-            if (start + len8 > p.capacity) len8 = (int)max(0ll, p.capacity - start);
-        }
+        my_len        = p.counts[pix];  // 0 for the padding of partial tiles
+        my_start      = p.cursor[pix];
+        len8          = my_len;
+        if (my_start >= 0 && (long long)my_start + len8 > p.capacity) len8 = (int)max(0ll, p.capacity - my_start);
     }
     len8 = max(len8, __shfl_xor(len8, 1));
     len8 = max(len8, __shfl_xor(len8, 2));
     len8 = max(len8, __shfl_xor(len8, 4));
     len8 = __builtin_amdgcn_readfirstlane(len8);
+    // the rows take their pixel's length and list start from these lanes: no second memory round trip
     if (len8 <= 8)
-        sort_blend_rows<C, TRAIN, 8>(p, pix_first, group_in_range);
+        sort_blend_rows<C, TRAIN, 8>(p, pix_first, group_in_range, __shfl(my_len, lane >> 3), __shfl(my_start, lane >> 3));
     else
     {
-        sort_blend_rows<C, TRAIN, 16>(p, pix_first, group_in_range);
-        sort_blend_rows<C, TRAIN, 16>(p, pix_first + 4, group_in_range);
+        sort_blend_rows<C, TRAIN, 16>(p, pix_first, group_in_range, __shfl(my_len, lane >> 4), __shfl(my_start, lane >> 4));
+        sort_blend_rows<C, TRAIN, 16>(p, pix_first + 4, group_in_range, __shfl(my_len, 4 + (lane >> 4)), __shfl(my_start, 4 + (lane >> 4)));
     }
 }
 
