@@ -325,17 +325,12 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 #pragma unroll
                 for (int c = 0; c < C; ++c) tex_grad[c] += ev[1 + c];
                 // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
-                const int x_i = float(gx) < ux ? 0 : 1;
-                const int y_i = float(gy) < uy ? 0 : 2;
-                const int bi  = y_i + x_i;
-                float blend, J0, J1;
-                switch (bi)
-                {
-                    case 0: blend = (1.f - sx) * (1.f - sy); J0 = sy - 1.f; J1 = sx - 1.f; break;
-                    case 1: blend = sx * (1.f - sy); J0 = 1.f - sy; J1 = -sx; break;
-                    case 2: blend = (1.f - sx) * sy; J0 = -sy; J1 = 1.f - sx; break;
-                    default: blend = sx * sy; J0 = sy; J1 = sx; break;
-                }
+                // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
+                const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
+                const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
+                float blend    = wx * wy;
+                const float J0 = x_hi ? wy : -wy;
+                const float J1 = y_hi ? wx : -wx;
                 if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
                 conf_grad += blend * lfac * grad_alpha;
                 const float gbs = conf * lfac * grad_alpha;
