@@ -29,15 +29,15 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (131670, 407415),
-    "bin_scatter": (50072, 203416),
-    "tile_count": (51807, 11061),
-    "tile_scatter": (57577, 512573),
-    "sort_blend": (376542, 254199),
-    "fill_rank": (13, 187500),
-    "backward_pixels": (525380, 647968),
-    "backward_points": (1408001, 567159),
-    "adam_fused": (582978, 792823),
+    "project_bin": (132821, 406727),
+    "bin_scatter": (50064, 203516),
+    "tile_count": (51861, 12443 + 21944),
+    "tile_scatter": (87096, 451131),
+    "sort_blend": (374740, 254823),
+    "fill_rank": (12, 187500),
+    "backward_pixels": (504759, 652866),
+    "backward_points": (1223724, 198835),
+    "adam_fused": (582967, 792823),
 }
 
 
