@@ -50,13 +50,6 @@ __device__ __forceinline__ Camera load_camera(const double* pose, const float* i
     return c;
 }
 
-__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ p, int32_t v, long long n)
-{
-    long long i      = (long long)blockIdx.x * 256 + threadIdx.x;
-    long long stride = (long long)gridDim.x * 256;
-    for (; i < n; i += stride) p[i] = v;
-}
-
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint4* __restrict__ p, long long n)
 {
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = make_uint4(0u, 0u, 0u, 0u);
