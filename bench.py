@@ -73,6 +73,7 @@ def main():
                          "the order the reference's scene preprocessing produces")
     ap.add_argument("--no-order-variant", action="store_true",
                     help="skip the second splat measurement with the points in the reference's preprocessing order")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the step that is reported beside the eager one")
     ap.add_argument("--cpu-steps", type=int, default=3, help="oracle steps for the cpu_baseline sample (0 = skip)")
     ap.add_argument("--no-net", action="store_true", help="skip the reconstruction-net forward that is reported beside the splat")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -146,7 +147,25 @@ def main():
         prof = ctx.profile_read()
         ctx.profile_enable(False)
         ms_per_step = (t1 - t0) * 1e3 / args.steps
-        return dict(sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
+        # the same step captured once into a HIP graph and replayed: the launch gaps of the eager loop are gone
+        graph_ms = None
+        if not args.no_graph:
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    step()
+            torch.cuda.synchronize()
+            for _ in range(2):
+                graph.replay()
+            torch.cuda.synchronize()
+            g0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
+            del graph
+        return dict(graph_ms=graph_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
                     grad_images=grad_images, grads=grads, opt=opt, counters=counters, nz=nz, total_el=total_el,
                     prof=prof, ms_per_step=ms_per_step)
 
@@ -157,6 +176,7 @@ def main():
         ms_k = {k: ms / max(n, 1) * (n / args.steps) for k, (ms, n) in r["prof"].items()}
         other_order = {"point_order": "morton_blocks (Morton curve, blocks of 256 shuffled: SceneData.cpp:115-116)",
                        "ms_per_step": round(r["ms_per_step"], 4),
+                       "ms_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4),
                        "fwd_bwd_kernels_ms": round(sum(v for k, v in ms_k.items() if k != "adam_fused"), 4),
                        "points_per_s": round(r["desc"].num_points / (r["ms_per_step"] * 1e-3), 1),
                        "kernels_ms": {k: round(v, 4) for k, v in ms_k.items()}}
@@ -292,7 +312,8 @@ def main():
                    "point_order": args.point_order, "points": N, "width": sc.width, "height": sc.height, "layers": desc.num_layers,
                    "list_depth": desc.list_depth, "counters": counters},
         "frame_ms": {"fwd_bwd_kernels": round(fwd_bwd_ms, 4), "all_kernels": round(kernel_ms, 4),
-                     "wall_per_step": round(ms_per_step, 4)},
+                     "wall_per_step": round(ms_per_step, 4),
+                     "wall_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4)},
         "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

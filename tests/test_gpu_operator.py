@@ -153,3 +153,66 @@ def test_dynamic_refinement_displaces_points_per_view(oracle):
     ns.dynamic_refinement_t = torch.zeros((2, 5, 3), device="cuda")
     with pytest.raises(ValueError):
         BlendPointCloud(_info(sc, ns))
+
+
+def test_step_replays_from_a_hip_graph(oracle):
+    """The C ABI is stream-ordered and allocates nothing, so a caller can capture forward + backward + fused Adam
+    once and replay it. Every replay is checked against the eager step it stands for, with eager work between the
+    replays."""
+    from trips_amd.adam import MyAdam
+    from trips_amd.renderer import SplatContext, get_context
+    sc = scenes.tiny(n=6000, w=96, h=64, f=80.0, num_layers=4, list_depth=16, seed=61, views=2, radius=(0.004, 0.4))
+    d = abi.desc_for_scene(sc)
+    ctx = get_context(0)
+    dev = ctx.device
+    f = lambda a, dt=torch.float32: torch.as_tensor(np.ascontiguousarray(a), dtype=dt).to(dev).contiguous()
+
+    def make():
+        t = dict(position=f(sc.position), point_size=f(sc.point_size), index=f(sc.index, torch.int32),
+                 texture=f(sc.texture), confidence=f(sc.confidence), background=f(sc.background),
+                 poses_se3=f(sc.poses_se3, torch.float64), intrinsics=f(sc.intrinsics), dropout=None)
+        N, C = d.num_points, d.num_channels
+        grads = dict(d_texture=torch.zeros((C, N), device=dev), d_confidence=torch.zeros(N, device=dev),
+                     d_background=torch.zeros(C, device=dev), d_position=torch.zeros((N, 4), device=dev),
+                     d_point_size=torch.zeros(N, device=dev), d_pose=torch.zeros((d.num_images, 6), dtype=torch.float64, device=dev),
+                     d_intrinsics=torch.zeros((d.num_cameras, 13), device=dev))
+        params = [torch.nn.Parameter(t[k]) for k in ("position", "point_size", "texture", "confidence")]
+        for p, k in zip(params, ("d_position", "d_point_size", "d_texture", "d_confidence")):
+            p.grad = grads[k]
+        state = dict(t=t, grads=grads, tin=SplatContext.make_in(**t), opt=MyAdam(params, lr=1e-2),
+                     ws=ctx.alloc_bytes(ctx.workspace_size(d)), saved=ctx.alloc_bytes(ctx.saved_size(d)),
+                     images=ctx.alloc_images(d))
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(7)
+        state["gi"] = [torch.randn(im.shape, generator=gen, device=dev) for im in state["images"]]
+        return state
+
+    def step(s):
+        for g in s["grads"].values():
+            g.zero_()
+        ctx.forward(d, s["tin"], s["images"], s["saved"], s["ws"])
+        ctx.backward(d, s["tin"], s["saved"], s["gi"], s["grads"], s["ws"])
+        s["opt"].step()
+
+    eager, graphed = make(), make()
+    step(eager)
+    step(graphed)  # the optimiser's state tensors exist before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(graphed)
+    torch.cuda.synchronize()
+    step(eager)  # the capture itself does not run the step; the first replay does
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for k in ("position", "texture", "confidence", "point_size"):
+            assert torch.equal(graphed["t"][k], eager["t"][k]), k
+        for a, b in zip(graphed["images"], eager["images"]):
+            assert torch.equal(a, b)
+        # summed with double atomics over workgroups: equal up to the order of the additions
+        assert torch.allclose(graphed["grads"]["d_pose"], eager["grads"]["d_pose"], rtol=1e-9, atol=1e-12)
+        (eager["images"][0].sum() + graphed["images"][0].sum()).item()  # eager work and a synchronisation in between
+        step(eager)
