@@ -91,6 +91,12 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         float4 ptk  = make_float4(0.f, 0.f, -1.f, 0.f);
         bool skip   = false;
         const int tex = p.index[pid];
+        constexpr int NREC = 1 + CPAD / 4;  // float4 per blend record
+        float4 recv[NREC], precv[2];
+#pragma unroll
+        for (int q = 0; q < NREC; ++q) recv[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+        precv[0] = make_float4(0.f, 0.f, 0.f, 0.f);
+        precv[1] = make_float4(__int_as_float(tex), -1.f, __int_as_float(0), 0.f);
         not_identity |= (tex != pid);
         if ((unsigned)tex >= (unsigned)p.num_texels)
         {
@@ -163,26 +169,29 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 ptk = make_float4(ipx, ipy, z, __int_as_float(layer));
 
                 // record for blend (+ backward)
-                float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)pid * p.rec_floats);
-                rec[0]      = make_float4(ipx, ipy, encode_size_field(size_px, L), p.confidence[tex]);
+                recv[0] = make_float4(ipx, ipy, encode_size_field(size_px, L), p.confidence[tex]);
                 float d[CPAD];
 #pragma unroll
                 for (int c = 0; c < CPAD; ++c) d[c] = c < C ? p.texture[(size_t)c * p.num_texels + tex] : 0.f;
 #pragma unroll
-                for (int q = 0; q < CPAD / 4; ++q) rec[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
+                for (int q = 0; q < CPAD / 4; ++q) recv[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
                 if (TRAIN)
                 {
-                    float4* prec = reinterpret_cast<float4*>(p.prec + (size_t)pid * kPointRecordFloats);
-                    prec[0]      = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
-                    prec[1]      = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
+                    precv[0] = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
+                    precv[1] = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
                 }
             }
         }
-        if (TRAIN && !(ptk.z > 0.f))
+        // The records of culled points are written too (zeros; tail {texture index, depth = -1, layers = 0}): whole
+        // lines leave the chip faster than lines with holes
+        float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)pid * p.rec_floats);
+#pragma unroll
+        for (int q = 0; q < NREC; ++q) rec[q] = recv[q];
+        if (TRAIN)
         {
-            // culled: only the tail {texture index, depth = -1, layers = 0} is defined
             float4* prec = reinterpret_cast<float4*>(p.prec + (size_t)pid * kPointRecordFloats);
-            prec[1]      = make_float4(__int_as_float(tex), -1.f, __int_as_float(0), 0.f);
+            prec[0]      = precv[0];
+            prec[1]      = precv[1];
         }
         p.ptk[pid] = ptk;
     }
