@@ -29,15 +29,15 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (132821, 406727),
-    "bin_scatter": (50064, 203516),
-    "tile_count": (51861, 12443 + 21944),
-    "tile_scatter": (87096, 451131),
-    "sort_blend": (374740, 254823),
+    "project_bin": (134008, 477943),
+    "bin_scatter": (50060, 203347),
+    "tile_count": (51864, 34387),
+    "tile_scatter": (87152, 451113),
+    "sort_blend": (374727, 254802),
     "fill_rank": (12, 187500),
-    "backward_pixels": (504759, 652866),
-    "backward_points": (1223724, 198835),
-    "adam_fused": (582967, 792823),
+    "backward_pixels": (504725, 652902),
+    "backward_points": (1223729, 198835),
+    "adam_fused": (582969, 792823),
 }
 
 
