@@ -141,6 +141,14 @@ def test_backward_small(oracle, L, K, bg):
     assert np.abs(g["d_pose"]).max() > 0 and np.abs(g["d_intrinsics"]).max() > 0
 
 
+@pytest.mark.parametrize("channels,K", [(3, 16), (8, 8), (16, 16)])
+def test_backward_other_channel_counts(oracle, channels, K):
+    sc = scenes.tiny(n=2500, w=56, h=40, f=50.0, num_layers=3, list_depth=K, seed=60 + channels, channels=channels,
+                     radius=(0.004, 0.4))
+    sc.confidence = (sc.confidence ** 0.3).astype(np.float32)
+    _check_backward(oracle, sc, abi.desc_for_scene(sc))
+
+
 def test_backward_views_crop_distortion_optional_outputs(oracle):
     sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=31, views=2)
     sc.views[1]["crop_transform"] = (1.5, 1.25, -10.0, 4.0, 0.0)
