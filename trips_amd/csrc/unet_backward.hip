@@ -383,6 +383,16 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
         const int q     = (int)(item % groups);
         const size_t bp = item / groups;
         const int Y = (int)(bp / p.Wb), X = (int)(bp - (size_t)Y * p.Wb);
+        // the pre-activations first: in flight during the gather
+        const int ch0 = 8 * (q - 1);
+        half8 f8, m8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f8[i] = m8[i] = _Float16(0.f);
+        if (q > 0)
+        {
+            f8 = *reinterpret_cast<const half8*>(p.pre + bp * p.npad + ch0);
+            m8 = *reinterpret_cast<const half8*>(p.pre + bp * p.npad + half + ch0);
+        }
         float a[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) a[i] = 0.f;
@@ -420,11 +430,7 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
         }
         else
         {
-            const int ch0       = 8 * (q - 1);
-            const _Float16* pr  = p.pre + bp * p.npad;
-            _Float16* dp        = p.dpre + bp * p.npad;
-            const half8 f8 = *reinterpret_cast<const half8*>(pr + ch0);
-            const half8 m8 = *reinterpret_cast<const half8*>(pr + half + ch0);
+            _Float16* dp = p.dpre + bp * p.npad;
             half8 of, om;
 #pragma unroll
             for (int i = 0; i < 8; ++i)
