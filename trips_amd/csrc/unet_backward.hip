@@ -554,13 +554,123 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     // channels that no stage writes stay zero for every tile
     for (int i = threadIdx.x; i < CIN * kXtChan; i += 256) s_xt[i] = _Float16(0.f);
 
-    for (int tile = blockIdx.x; tile < p.tiles; tile += gridDim.x)
+    // ---- stage 1 in two halves: every global load of a tile is issued into registers (a thread's loads are all in
+    // flight together), and written to LDS (transposed) one tile later, so that the loads of tile t + 1 travel while
+    // tile t is upsampled and multiplied ----
+    constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + 255) / 256;
+    constexpr int kMaxPerPix  = 1 + (CIN - 8) / 8;  // image below + groups of 8 block outputs (C = 4)
+    constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + 255) / 256;
+    constexpr int kDpreItems  = NPAD / 8;
+    struct TileLoads
+    {
+        float feat[kFeatItems][4];
+        uint4 below[kBelowItems];
+        half8 dpre[kDpreItems];
+    };
+    const int act_groups = p.cb_store / 8;
+    const int per_pixel  = 1 + act_groups;
+    auto issue_loads = [&](int tile, TileLoads& r)
     {
         const int ty = tile / p.tiles_x, tx = tile - ty * p.tiles_x;
         const int x0 = tx * kConvTileW, y0 = ty * kConvTileH;
         const int by0 = y0 / 2 - 1, bx0 = x0 / 2 - 1;
-        __syncthreads();  // the previous tile's operands have been consumed (and the zero fill is done)
-        // ---- stage 1: this level's image (transposed), the patch of the level below, the gradient tile (transposed) ----
+        const size_t plane = (size_t)p.H * p.W;
+#pragma unroll
+        for (int k = 0; k < kFeatItems; ++k)
+        {
+            const int item = threadIdx.x + 256 * k;
+            const int py = item / kConvPatchW, px = item - py * kConvPatchW;
+            const int y = y0 + py - 1, x = x0 + px - 1;
+            const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) r.feat[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+        }
+        if (has_below)
+        {
+            const size_t pb = (size_t)p.Hb * p.Wb;
+#pragma unroll
+            for (int k = 0; k < kBelowItems; ++k)
+            {
+                const int item = threadIdx.x + 256 * k;
+                r.below[k]     = make_uint4(0u, 0u, 0u, 0u);
+                if (item < kBelowH * kBelowW * per_pixel)
+                {
+                    const int q = item % per_pixel, bp = item / per_pixel;
+                    const int rr = bp / kBelowW, c0 = bp - rr * kBelowW;
+                    const int yy = min(max(by0 + rr, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
+                    if (q == 0)
+                    {
+                        float f[4];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) f[c] = c < C ? p.feat_below[c * pb + (size_t)yy * p.Wb + xx] : 0.f;
+                        r.below[k] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+                    }
+                    else
+                        r.below[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kDpreItems; ++k)
+        {
+            const int item = threadIdx.x + 256 * k;
+            const int tp = item % (kConvTileH * kConvTileW), g = item / (kConvTileH * kConvTileW);
+            const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) r.dpre[k][i] = _Float16(0.f);
+            if (y < p.H && x < p.W) r.dpre[k] = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * NPAD + 8 * g);
+        }
+    };
+    auto commit_loads = [&](const TileLoads& r)
+    {
+#pragma unroll
+        for (int k = 0; k < kFeatItems; ++k)
+        {
+            const int item = threadIdx.x + 256 * k;
+            if (item < kConvPatchH * kConvPatchW)
+            {
+                const int py = item / kConvPatchW, px = item - py * kConvPatchW;
+#pragma unroll
+                for (int c = 0; c < 4; ++c)  // a run-time bound would put the register array into scratch memory
+                    if (c < C) s_xt[c * kXtChan + py * kXtRow + px] = _Float16(r.feat[k][c]);
+            }
+        }
+        if (has_below)
+        {
+#pragma unroll
+            for (int k = 0; k < kBelowItems; ++k)
+            {
+                const int item = threadIdx.x + 256 * k;
+                if (item < kBelowH * kBelowW * per_pixel)
+                {
+                    const int q = item % per_pixel, bp = item / per_pixel;
+                    _Float16* row = s_below + (size_t)bp * ROW;
+                    if (q == 0)
+                    {
+                        const unsigned f[4] = {r.below[k].x, r.below[k].y, r.below[k].z, r.below[k].w};
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            if (c < C) row[C + c] = _Float16(__uint_as_float(f[c]));
+                        for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
+                    }
+                    else
+                        *reinterpret_cast<uint4*>(row + 2 * C + 8 * (q - 1)) = r.below[k];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kDpreItems; ++k)
+        {
+            const int item = threadIdx.x + 256 * k;
+            const int tp = item % (kConvTileH * kConvTileW), g = item / (kConvTileH * kConvTileW);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s_dt[(8 * g + i) * kDtChan + tp] = r.dpre[k][i];
+        }
+    };
+
+    // the same without registers in between, for the shapes that have none to spare
+    auto stream_stage1 = [&](int x0, int y0, int by0, int bx0)
+    {
         {
             const size_t plane = (size_t)p.H * p.W;
             for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW; item += 256)
@@ -606,6 +716,23 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
             for (int i = 0; i < 8; ++i) s_dt[(8 * g + i) * kDtChan + tp] = v[i];
         }
+    };
+
+    // with 64 input channels and more than 64 pre-activations the accumulators leave no registers for a tile in flight
+    constexpr bool kPrefetch = !(CIN == 64 && NPAD > 64);
+    TileLoads cur;
+    if (kPrefetch && (int)blockIdx.x < p.tiles) issue_loads(blockIdx.x, cur);
+    for (int tile = blockIdx.x; tile < p.tiles; tile += gridDim.x)
+    {
+        const int ty = tile / p.tiles_x, tx = tile - ty * p.tiles_x;
+        const int x0 = tx * kConvTileW, y0 = ty * kConvTileH;
+        const int by0 = y0 / 2 - 1, bx0 = x0 / 2 - 1;
+        __syncthreads();  // the previous tile's operands have been consumed (and the zero fill is done)
+        if (!kPrefetch)
+            stream_stage1(x0, y0, by0, bx0);
+        else
+            commit_loads(cur);
+        if (kPrefetch && tile + (int)gridDim.x < p.tiles) issue_loads(tile + gridDim.x, cur);  // travels during stage 2 and the taps
         if (has_below)
         {
             __syncthreads();
