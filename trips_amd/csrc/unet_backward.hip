@@ -295,16 +295,29 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
     ConvTapRing<KC, NN> ring;
     conv_taps_prefetch(ring, p.wt);  // in flight while the patch is loaded
-    for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
+    // the patch of pre-activation gradients, four 16-byte loads of a thread in flight together
+    constexpr int kItems = kConvPatchH * kConvPatchW * GROUPS;
+    for (int item0 = threadIdx.x; item0 < kItems; item0 += 4 * 256)
     {
-        const int g = item % GROUPS, pp = item / GROUPS;
-        const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
-        const int y = y0 + py - 1, x = x0 + px - 1;
-        half8 v;
+        half8 v[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = _Float16(0.f);
-        if (y >= 0 && y < p.H && x >= 0 && x < p.W) v = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * KC + 8 * g);
-        *reinterpret_cast<half8*>(s_patch + (size_t)pp * ROW + 8 * g) = v;
+        for (int j = 0; j < 4; ++j)
+        {
+            const int item = item0 + 256 * j;
+            const int g = item % GROUPS, pp = item / GROUPS;
+            const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
+            const int y = y0 + py - 1, x = x0 + px - 1;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[j][i] = _Float16(0.f);
+            if (item < kItems && y >= 0 && y < p.H && x >= 0 && x < p.W)
+                v[j] = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * KC + 8 * g);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const int item = item0 + 256 * j;
+            if (item < kItems) *reinterpret_cast<half8*>(s_patch + (size_t)(item / GROUPS) * ROW + 8 * (item % GROUPS)) = v[j];
+        }
     }
     __syncthreads();
     floatx4 acc[4][NB];
