@@ -419,20 +419,33 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
                 wy[k] = up2_weight(2 * Y - 1 + k, p.H, Y, p.Hb);
                 wx[k] = up2_weight(2 * X - 1 + k, p.W, X, p.Wb);
             }
+            // all 16 gathers are issued before the first one is used (a load inside a branch on its weight would be
+            // waited for there: 16 memory round trips in a row); pixels outside the image have weight 0 and are read
+            // at a clamped position instead
+            half8 v[4][4];
 #pragma unroll
             for (int ky = 0; ky < 4; ++ky)
             {
-                if (wy[ky] == 0.f) continue;
-                const int y = 2 * Y - 1 + ky;
+                const int y = min(max(2 * Y - 1 + ky, 0), p.H - 1);
 #pragma unroll
                 for (int kx = 0; kx < 4; ++kx)
                 {
-                    if (wx[kx] == 0.f) continue;
-                    const int x   = 2 * X - 1 + kx;
-                    const half8 v = *reinterpret_cast<const half8*>(p.d_in + ((size_t)y * p.W + x) * p.cin_fine + pos);
-                    const float w = wy[ky] * wx[kx];
+                    const int x = min(max(2 * X - 1 + kx, 0), p.W - 1);
+                    v[ky][kx]   = *reinterpret_cast<const half8*>(p.d_in + ((size_t)y * p.W + x) * p.cin_fine + pos);
+                }
+            }
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) a[i] += w * float(v[i]);
+            for (int ky = 0; ky < 4; ++ky)
+            {
+#pragma unroll
+                for (int kx = 0; kx < 4; ++kx)
+                {
+                    const float w = wy[ky] * wx[kx];
+                    if (w != 0.f)
+                    {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) a[i] += w * float(v[ky][kx][i]);
+                    }
                 }
             }
         }
