@@ -73,114 +73,111 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
     const int grp      = lane / ROW;
     const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
+    const long long pix_ll = pix_first + grp;
+    const int pix          = pix_ll < P ? (int)pix_ll : 0;
+    int layer, gx, gy;
+    const bool live = pix_decode(p.geom, pix, layer, gx, gy) && pix_ll < P;
+    const int lw = p.geom.w[layer], lh = p.geom.h[layer];
+
+    const int m    = live ? m_in : 0;
+    const bool has = sub < m;
+    int mmax       = m;
+    if (ROW == 8) mmax = max(mmax, __shfl_xor(mmax, 8));
+    mmax           = max(mmax, __shfl_xor(mmax, 16));
+    mmax           = max(mmax, __shfl_xor(mmax, 32));
+    mmax           = __builtin_amdgcn_readfirstlane(mmax);
+
+    float g[C];
     {
-        const long long pix_ll = pix_first + grp;
-        const int pix          = pix_ll < P ? (int)pix_ll : 0;
-        int layer, gx, gy;
-        const bool live = pix_decode(p.geom, pix, layer, gx, gy) && pix_ll < P;
-        const int lw = p.geom.w[layer], lh = p.geom.h[layer];
-
-        const int m    = live ? m_in : 0;
-        const bool has = sub < m;
-        int mmax       = m;
-        if (ROW == 8) mmax = max(mmax, __shfl_xor(mmax, 8));
-        mmax           = max(mmax, __shfl_xor(mmax, 16));
-        mmax           = max(mmax, __shfl_xor(mmax, 32));
-        mmax           = __builtin_amdgcn_readfirstlane(mmax);
-
-        float g[C];
+        const float* gi = p.grad_image[layer];
+        if (p.layout == TRIPS_LAYOUT_CHW)
         {
-            const float* gi = p.grad_image[layer];
-            if (p.layout == TRIPS_LAYOUT_CHW)
-            {
-                const size_t plane = (size_t)lw * lh;
-                const float* o     = gi + ((size_t)p.view_index * C) * plane + (size_t)gy * lw + gx;
+            const size_t plane = (size_t)lw * lh;
+            const float* o     = gi + ((size_t)p.view_index * C) * plane + (size_t)gy * lw + gx;
 #pragma unroll
-                for (int c = 0; c < C; ++c) g[c] = live ? o[c * plane] : 0.f;
-            }
-            else
-            {
-                const float* o = gi + (((size_t)p.view_index * lh + gy) * lw + gx) * C;
-#pragma unroll
-                for (int c = 0; c < C; ++c) g[c] = live ? o[c] : 0.f;
-            }
+            for (int c = 0; c < C; ++c) g[c] = live ? o[c * plane] : 0.f;
         }
-
-        int pid = 0;
-        float desc[CPAD];
-#pragma unroll
-        for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
-        float a = 0.f;
-        int slot = 0;
-        if (has)
+        else
         {
-            pid               = p.lists[(size_t)pix * K + sub];
-            const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
-            const float4 r0   = rec[0];
+            const float* o = gi + (((size_t)p.view_index * lh + gy) * lw + gx) * C;
 #pragma unroll
-            for (int q = 0; q < CPAD / 4; ++q)
-            {
-                const float4 t  = rec[1 + q];
-                desc[4 * q]     = t.x;
-                desc[4 * q + 1] = t.y;
-                desc[4 * q + 2] = t.z;
-                desc[4 * q + 3] = t.w;
-            }
-            const float mfac = 1.f / float(1 << layer);
-            const float ux = r0.x * mfac, uy = r0.y * mfac;
-            float w = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
-            if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
-            a = w * r0.w;
-            a *= layer_factor_encoded(r0.z, layer, p.num_layers);
-            // which of the point's four footprint pixels this one is
-            const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
-            slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
-        }
-
-        // exclusive transmittance, same chain as the forward
-        const float T = ROW == 8 ? half_exclusive_product(1.f - a, mmax) : row_exclusive_product(1.f - a, mmax);
-        // transmittance after the m retained entries decides whether the background is reached
-        // (RenderBackward.cu:205-210,302-308)
-        float T_after = T * (1.f - a);
-        T_after       = __shfl(T_after, max(m - 1, 0), ROW);
-        if (m == 0) T_after = 1.f;
-        const bool bg_reached = live && (T_after >= 0.001f);
-
-        float s = 0.f, sbg = 0.f;
-#pragma unroll
-        for (int c = 0; c < C; ++c)
-        {
-            s += desc[c] * g[c];
-            sbg += p.background[c] * g[c];
-        }
-        const float ta = T * a;
-        const float q  = has ? ta * s : 0.f;
-        float later    = ROW == 8 ? half_exclusive_suffix_sum(q) : row_exclusive_suffix_sum(q);  // entries i > j
-        if (bg_reached) later += T_after * sbg;
-        const float dem        = 1.f / (1.f - a + 1e-9f);
-        const float grad_alpha = T * s - later * dem;
-
-        if (bg_reached && sub == 0)
-        {
-#pragma unroll
-            for (int c = 0; c < C; ++c) acc_bg[c] += (double)(T_after * g[c]);
-        }
-        if (has)
-        {
-            // {dL/dalpha, T*alpha*g[0..C)} padded to a multiple of 4 floats: one aligned gather for pass 2
-            float e[EF];
-            e[0] = grad_alpha;
-#pragma unroll
-            for (int c = 0; c < C; ++c) e[1 + c] = ta * g[c];
-#pragma unroll
-            for (int c = 1 + C; c < EF; ++c) e[c] = 0.f;
-            float4* dst = reinterpret_cast<float4*>(p.entry_grad + ((size_t)pix * K + sub) * EF);
-#pragma unroll
-            for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
-            p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
+            for (int c = 0; c < C; ++c) g[c] = live ? o[c] : 0.f;
         }
     }
 
+    int pid = 0;
+    float desc[CPAD];
+#pragma unroll
+    for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
+    float a = 0.f;
+    int slot = 0;
+    if (has)
+    {
+        pid               = p.lists[(size_t)pix * K + sub];
+        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
+        const float4 r0   = rec[0];
+#pragma unroll
+        for (int q = 0; q < CPAD / 4; ++q)
+        {
+            const float4 t  = rec[1 + q];
+            desc[4 * q]     = t.x;
+            desc[4 * q + 1] = t.y;
+            desc[4 * q + 2] = t.z;
+            desc[4 * q + 3] = t.w;
+        }
+        const float mfac = 1.f / float(1 << layer);
+        const float ux = r0.x * mfac, uy = r0.y * mfac;
+        float w = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
+        if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
+        a = w * r0.w;
+        a *= layer_factor_encoded(r0.z, layer, p.num_layers);
+        // which of the point's four footprint pixels this one is
+        const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
+        slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
+    }
+
+    // exclusive transmittance, same chain as the forward
+    const float T = ROW == 8 ? half_exclusive_product(1.f - a, mmax) : row_exclusive_product(1.f - a, mmax);
+    // transmittance after the m retained entries decides whether the background is reached
+    // (RenderBackward.cu:205-210,302-308)
+    float T_after = T * (1.f - a);
+    T_after       = __shfl(T_after, max(m - 1, 0), ROW);
+    if (m == 0) T_after = 1.f;
+    const bool bg_reached = live && (T_after >= 0.001f);
+
+    float s = 0.f, sbg = 0.f;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        s += desc[c] * g[c];
+        sbg += p.background[c] * g[c];
+    }
+    const float ta = T * a;
+    const float q  = has ? ta * s : 0.f;
+    float later    = ROW == 8 ? half_exclusive_suffix_sum(q) : row_exclusive_suffix_sum(q);  // entries i > j
+    if (bg_reached) later += T_after * sbg;
+    const float dem        = 1.f / (1.f - a + 1e-9f);
+    const float grad_alpha = T * s - later * dem;
+
+    if (bg_reached && sub == 0)
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c) acc_bg[c] += (double)(T_after * g[c]);
+    }
+    if (has)
+    {
+        // {dL/dalpha, T*alpha*g[0..C)} padded to a multiple of 4 floats: one aligned gather for pass 2
+        float e[EF];
+        e[0] = grad_alpha;
+#pragma unroll
+        for (int c = 0; c < C; ++c) e[1 + c] = ta * g[c];
+#pragma unroll
+        for (int c = 1 + C; c < EF; ++c) e[c] = 0.f;
+        float4* dst = reinterpret_cast<float4*>(p.entry_grad + ((size_t)pix * K + sub) * EF);
+#pragma unroll
+        for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
+        p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
+    }
 }
 
 template <int C>

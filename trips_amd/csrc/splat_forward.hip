@@ -750,15 +750,15 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     }
     else
     {
-    const u64* src = p.keys;
-    if (start < 0)
-    {
-        // a long list: the reduction pass left the 16 smallest keys of each of its segments
-        src      = p.cand;
-        start    = (-1 - start) * 16ll;
-        readable = ((len + kLongSegment - 1) / kLongSegment) * 16;
-    }
-    best = row_top16(src, start, readable);
+        const u64* src = p.keys;
+        if (start < 0)
+        {
+            // a long list: the reduction pass left the 16 smallest keys of each of its segments
+            src      = p.cand;
+            start    = (-1 - start) * 16ll;
+            readable = ((len + kLongSegment - 1) / kLongSegment) * 16;
+        }
+        best = row_top16(src, start, readable);
     }
 
     // ---- blend (RenderForward.cu:820-1048) ----
