@@ -848,8 +848,16 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
             p.retained[pix] = live ? ret : 0;
             p.lengths[pix]  = live ? len : 0;
         }
-        if (sub < K) p.lists[(size_t)pix * K + sub] = has ? pid : -1;
-        if (ROW == 8 && sub + 8 < K) p.lists[(size_t)pix * K + sub + 8] = -1;
+        const int mine = has ? pid : -1;
+        if (ROW == 8)
+        {
+            // one 8-byte store per lane covers the pixel's whole row (K <= 16 ids): lanes 0..3 carry the ids of lane
+            // pairs, the others the -1 padding
+            const int lo = __shfl(mine, (2 * sub) & 7, 8), hi = __shfl(mine, (2 * sub + 1) & 7, 8);
+            if (2 * sub < K) *reinterpret_cast<int2*>(p.lists + (size_t)pix * K + 2 * sub) = sub < 4 ? make_int2(lo, hi) : make_int2(-1, -1);
+        }
+        else if (sub < K)
+            p.lists[(size_t)pix * K + sub] = mine;
     }
 }
 
