@@ -316,6 +316,11 @@ def main():
                      "wall_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4)},
         "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
+        # the same with the HBM traffic rocprofv3 measured (committed summary under profiles/) instead of the
+        # algorithmic bytes: what the memory system actually moved per second
+        "hbm_frac_fwd_bwd_measured_traffic": round(
+            sum(measured_traffic_bytes(k) for k in PMC_KIB_DEFAULT_WORKLOAD if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
+            HBM_PEAK_GBS, 4) if (fwd_bwd_ms > 0 and args.points == DEFAULT_POINTS and args.point_order == "random") else None,
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": measured_traffic_bytes(dom) if args.points == DEFAULT_POINTS and args.point_order == "random" else None,
