@@ -104,8 +104,8 @@ constexpr int kPointRecordFloats = 8;
 constexpr int kTileShift  = 5;
 constexpr int kTile       = 1 << kTileShift;
 constexpr int kTilePixels = kTile * kTile;
-constexpr int kBinThreads = 512;    // workgroup size of the two binning kernels
-constexpr int kBinGroups  = 512;    // workgroups (= contiguous chunks of points) of the two binning kernels
+constexpr int kBinThreads = 1024;    // workgroup size of the two binning kernels
+constexpr int kBinGroups  = 256;    // workgroups (= contiguous chunks of points) of the two binning kernels
 constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
 // bin entries of a tile above which the tile is split into slices of that many entries, one workgroup each
 constexpr int kSliceEntries = 8192;
