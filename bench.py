@@ -29,15 +29,15 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (134008, 477943),
-    "bin_scatter": (50060, 203347),
-    "tile_count": (51864, 34387),
-    "tile_scatter": (87152, 451113),
-    "sort_blend": (374727, 254802),
+    "project_bin": (135302, 473876),
+    "bin_scatter": (48408, 203077),
+    "tile_count": (51870, 34387),
+    "tile_scatter": (87370, 451924),
+    "sort_blend": (374811, 254810),
     "fill_rank": (12, 187500),
-    "backward_pixels": (504725, 652902),
-    "backward_points": (1223729, 198835),
-    "adam_fused": (582969, 792823),
+    "backward_pixels": (504625, 652939),
+    "backward_points": (1223715, 198835),
+    "adam_fused": (582963, 792823),
 }
 
 
