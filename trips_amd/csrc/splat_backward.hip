@@ -10,8 +10,8 @@
 //   1. pixels: a 16-lane row (an 8-lane half row for short lists) owns a pixel, each lane one retained entry. Alpha and transmittance are recomputed
 //      from the per-point record exactly as the forward computed them; the "all later entries" sum of
 //      RenderBackward.cu:284-301 is a suffix sum across the row. Per entry it writes {dL/dalpha, T*alpha*dL/dimage}
-//      into the pixel's row of a [P,K] table and one byte, the entry's rank, into the point's 32-slot table
-//      (slot = layer * 4 + footprint corner).
+//      into the pixel's row of a [P,K] table. The forward's blend kernel has left one byte per retained entry, its
+//      rank in the pixel's list, in the point's 32-slot table (slot = layer * 4 + footprint corner).
 //   2. points: one thread per point walks its slots, gathers those records (one aligned load each), sums the image-space gradient of all its entries and runs the projection chain ONCE
 //      (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then adds its gradients
 //      with plain read-modify-writes. Pose / intrinsics partials stay in double registers over a grid-stride
@@ -60,7 +60,7 @@ __device__ __forceinline__ double wave_sum(double v)
 
 
 // ---------------------------------------------------------------------------------------------------------
-// Pass 1: per pixel row. Writes entry_grad[pix*K + j] = {dL/dalpha_j, T_j alpha_j g[0..C)} and rank[pid*32 + slot] = j.
+// Pass 1: per pixel row. Writes entry_grad[pix*K + j] = {dL/dalpha_j, T_j alpha_j g[0..C)}.
 // 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
 // than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
 template <int C, int ROW>
@@ -110,7 +110,6 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
 #pragma unroll
     for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
     float a = 0.f;
-    int slot = 0;
     if (has)
     {
         pid               = p.lists[(size_t)pix * K + sub];
@@ -131,9 +130,6 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
         if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
         a = w * r0.w;
         a *= layer_factor_encoded(r0.z, layer, p.num_layers);
-        // which of the point's four footprint pixels this one is
-        const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
-        slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
     }
 
     // exclusive transmittance, same chain as the forward
@@ -176,7 +172,6 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
         float4* dst = reinterpret_cast<float4*>(p.entry_grad + ((size_t)pix * K + sub) * EF);
 #pragma unroll
         for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
-        p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
     }
 }
 
@@ -443,16 +438,6 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
     if (N <= 0) 
     {
         // no points: only the background receives gradient
-    }
-    {
-        ProfScope ps(prof, "fill_rank", stream);
-        const long long words = (long long)N * 8;  // 32 bytes per point
-        if (words > 0)
-        {
-            int blocks = (int)min((words + 255) / 256, 8192ll);
-            hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks), dim3(256), 0, stream,
-                               reinterpret_cast<unsigned*>(p.rank), 0xFFFFFFFFu, words);
-        }
     }
     {
         ProfScope ps(prof, "backward_pixels", stream);

@@ -50,9 +50,9 @@ __device__ __forceinline__ Camera load_camera(const double* pose, const float* i
     return c;
 }
 
-__global__ __launch_bounds__(256) void fill_zero_kernel(uint4* __restrict__ p, long long n)
+__global__ __launch_bounds__(256) void fill_words_kernel(uint4* __restrict__ p, unsigned v, long long n)
 {
-    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = make_uint4(v, v, v, v);
 }
 
 __global__ void clear_header_kernel(ViewHeader* h)
@@ -769,6 +769,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     const int pid  = (int)(unsigned)(best & 0xffffffffull);
 
     float a = 0.f;
+    int slot = 0;  // which of the point's (layer, footprint corner) pixels this one is
     float desc[CPAD];
 #pragma unroll
     for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
@@ -791,6 +792,8 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
         if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
         a = w * r0.w;
         a *= layer_factor_encoded(r0.z, layer, p.num_layers);
+        const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
+        slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
     }
 
     // exclusive transmittance: lane j latches prod_{k<j} (1 - a_k), built left to right
@@ -848,6 +851,8 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
             p.retained[pix] = live ? ret : 0;
             p.lengths[pix]  = live ? len : 0;
         }
+        // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
+        if (has && sub < ret) p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
         const int mine = has ? pid : -1;
         if (ROW == 8)
         {
@@ -948,8 +953,8 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         hipLaunchKernelGGL(slice_plan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_start, p.capacity, NB, p.slice_start, p.bin_total, p.long_count);
         // counts and run are neighbours in the workspace: one fill clears both
         const long long words = 2ll * NB * kTilePixels;
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)std::min<long long>((words / 4 + 255) / 256, 4096)), dim3(256), 0, stream,
-                           reinterpret_cast<uint4*>(p.counts), words / 4);
+        hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((words / 4 + 255) / 256, 4096)), dim3(256), 0, stream,
+                           reinterpret_cast<uint4*>(p.counts), 0u, words / 4);
         hipLaunchKernelGGL((tile_lists_kernel<false>), dim3(NB + max_slices), dim3(256), 0, stream, p);
     }
     {
@@ -965,6 +970,15 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         ProfScope ps(prof, "long_lists", stream);
         const int blocks = std::min((p.max_long_items + 15) / 16, 2048);
         hipLaunchKernelGGL(long_list_reduce_kernel, dim3(blocks), dim3(256), 0, stream, p);
+    }
+    if (train && p.num_points > 0)
+    {
+        // the rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
+        // pixel's list): cleared here, filled by sort_blend
+        ProfScope ps(prof, "fill_rank", stream);
+        const long long quads = (long long)p.num_points * 2;  // 32 bytes per point
+        hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((quads + 255) / 256, 8192)), dim3(256), 0, stream,
+                           reinterpret_cast<uint4*>(p.rank), 0xFFFFFFFFu, quads);
     }
     {
         ProfScope ps(prof, "sort_blend", stream);

@@ -179,13 +179,13 @@ struct SavedLayout
     size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded)
     size_t retained;  // int32 [Pi]
     size_t lengths;   // int32 [Pi]
+    size_t rank;      // uint8 [N, 32] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none
     size_t bytes_per_view;
 };
 
 struct BackwardWorkspaceLayout
 {
     size_t entry_grad;  // float [P, K, EF]
-    size_t rank;        // uint8 [N, 32]
     size_t bytes;
 };
 
@@ -259,6 +259,7 @@ struct ForwardParams
     int32_t* lists;
     int32_t* retained;
     int32_t* lengths;
+    unsigned char* rank;  // training only
     ViewHeader* header;  // counters of this view
     ViewHeader* status;  // overflow flag of the whole forward call (start of the workspace)
     float* image[TRIPS_MAX_LAYERS];
@@ -283,7 +284,7 @@ struct BackwardParams
     const ViewHeader* header;
     const float* grad_image[TRIPS_MAX_LAYERS];
     float* entry_grad;    // [P, K, EF] {dL/dalpha, T alpha dL/dimage[0..C)}, EF = (1+C) rounded up to 4 (workspace)
-    unsigned char* rank;  // [N, 32] rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
+    const unsigned char* rank;  // [N, 32] (saved state) rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
     float* d_texture;
     float* d_confidence;
     float* d_background;

@@ -200,6 +200,8 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(P * sizeof(int32_t));
     s.lengths = o;
     o += align256(P * sizeof(int32_t));
+    s.rank = o;
+    o += align256(N * 32);
     s.bytes_per_view = o;
     return s;
 }
@@ -257,12 +259,10 @@ namespace
 BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     BackwardWorkspaceLayout w;
-    const size_t N = (size_t)d.num_points, P = (size_t)g.bin_off[d.num_layers] * kTilePixels, K = (size_t)d.list_depth;
+    const size_t P = (size_t)g.bin_off[d.num_layers] * kTilePixels, K = (size_t)d.list_depth;
     size_t o       = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
     w.entry_grad   = o;
     o += align256(P * K * (size_t)((1 + d.num_channels + 3) & ~3) * sizeof(float));
-    w.rank = o;
-    o += align256(N * 32);
     w.bytes = o;
     return w;
 }
@@ -418,6 +418,7 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
             p.lists      = reinterpret_cast<int32_t*>(sv + sl.lists);
             p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
             p.lengths    = reinterpret_cast<int32_t*>(sv + sl.lengths);
+            p.rank       = reinterpret_cast<unsigned char*>(sv + sl.rank);
         }
         else
         {
@@ -486,7 +487,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.retained     = reinterpret_cast<const int32_t*>(sv + sl.retained);
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
         p.entry_grad   = reinterpret_cast<float*>(ws + bl.entry_grad);
-        p.rank         = reinterpret_cast<unsigned char*>(ws + bl.rank);
+        p.rank         = reinterpret_cast<const unsigned char*>(sv + sl.rank);
         for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
         p.d_texture    = grads->d_texture;
         p.d_confidence = grads->d_confidence;
