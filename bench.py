@@ -29,15 +29,15 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (135302, 473876),
-    "bin_scatter": (48408, 203077),
-    "tile_count": (51870, 34387),
-    "tile_scatter": (87370, 451924),
-    "sort_blend": (374811, 254810),
-    "fill_rank": (12, 187500),
-    "backward_pixels": (504625, 652939),
-    "backward_points": (1223715, 198835),
-    "adam_fused": (582963, 792823),
+    "project_bin": (135407, 473823),
+    "bin_scatter": (48405, 202963),
+    "tile_count": (51871, 34387),
+    "tile_scatter": (87155, 451010),
+    "fill_rank": (15, 187500),
+    "sort_blend": (394389, 417377),
+    "backward_pixels": (471406, 417113),
+    "backward_points": (1223690, 198835),
+    "adam_fused": (582968, 792823),
 }
 
 
