@@ -922,6 +922,16 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
 
     if (first_view) hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.status);
     hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header);
+    if (train && p.num_points > 0)
+    {
+        // the rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
+        // pixel's list): filled by sort_blend; cleared first thing, not in front of sort_blend, where the fill would
+        // push the keys that the list kernels have just written out of the last-level cache
+        ProfScope ps(prof, "fill_rank", stream);
+        const long long quads = (long long)p.num_points * 2;  // 32 bytes per point
+        hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((quads + 255) / 256, 8192)), dim3(256), 0, stream,
+                           reinterpret_cast<uint4*>(p.rank), 0xFFFFFFFFu, quads);
+    }
     const int G          = p.bin_groups;
     const size_t lds_hist = (size_t)NB * sizeof(int);
     {
@@ -970,15 +980,6 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         ProfScope ps(prof, "long_lists", stream);
         const int blocks = std::min((p.max_long_items + 15) / 16, 2048);
         hipLaunchKernelGGL(long_list_reduce_kernel, dim3(blocks), dim3(256), 0, stream, p);
-    }
-    if (train && p.num_points > 0)
-    {
-        // the rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
-        // pixel's list): cleared here, filled by sort_blend
-        ProfScope ps(prof, "fill_rank", stream);
-        const long long quads = (long long)p.num_points * 2;  // 32 bytes per point
-        hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((quads + 255) / 256, 8192)), dim3(256), 0, stream,
-                           reinterpret_cast<uint4*>(p.rank), 0xFFFFFFFFu, quads);
     }
     {
         ProfScope ps(prof, "sort_blend", stream);
