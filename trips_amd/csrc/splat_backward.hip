@@ -64,20 +64,21 @@ __device__ __forceinline__ double wave_sum(double v)
 // 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
 // than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
 template <int C, int ROW>
-__device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, long long pix_first, int m_in, double (&acc_bg)[C])
+__device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, const TileCtx& tc, const float* gi, int pix_first,
+                                                    int m_in, double (&acc_bg)[C])
 {
     constexpr int CPAD = (C + 3) & ~3;
+    constexpr int RF   = 4 + CPAD;          // floats per blend record
     constexpr int EF   = (1 + C + 3) & ~3;  // floats per entry of entry_grad
     const int lane     = threadIdx.x & 63;
     const int sub      = lane & (ROW - 1);
     const int grp      = lane / ROW;
-    const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
-    const int K        = p.list_depth;
-    const long long pix_ll = pix_first + grp;
-    const int pix          = pix_ll < P ? (int)pix_ll : 0;
-    int layer, gx, gy;
-    const bool live = pix_decode(p.geom, pix, layer, gx, gy) && pix_ll < P;
-    const int lw = p.geom.w[layer], lh = p.geom.h[layer];
+    const int kshift   = p.list_depth == 16 ? 4 : 3;
+    // the group's pixels lie side by side in one row of the tile
+    const int pix   = pix_first + grp;
+    const int layer = tc.layer, lw = tc.w, lh = tc.h;
+    const int gx = tc.x0 + (pix & (kTile - 1)), gy = tc.y0 + ((pix >> kTileShift) & (kTile - 1));
+    const bool live = gx < lw && gy < lh;  // false for the padding of partial tiles
 
     const int m    = live ? m_in : 0;
     const bool has = sub < m;
@@ -89,19 +90,21 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
 
     float g[C];
     {
-        const float* gi = p.grad_image[layer];
+        // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
         if (p.layout == TRIPS_LAYOUT_CHW)
         {
             const size_t plane = (size_t)lw * lh;
-            const float* o     = gi + ((size_t)p.view_index * C) * plane + (size_t)gy * lw + gx;
+            const float* o     = gi + ((size_t)p.view_index * C) * plane;
+            const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
 #pragma unroll
-            for (int c = 0; c < C; ++c) g[c] = live ? o[c * plane] : 0.f;
+            for (int c = 0; c < C; ++c) g[c] = live ? (o + c * plane)[at] : 0.f;
         }
         else
         {
-            const float* o = gi + (((size_t)p.view_index * lh + gy) * lw + gx) * C;
+            const float* o    = gi + ((size_t)p.view_index * lh * lw) * C;
+            const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
 #pragma unroll
-            for (int c = 0; c < C; ++c) g[c] = live ? o[c] : 0.f;
+            for (int c = 0; c < C; ++c) g[c] = live ? o[at + c] : 0.f;
         }
     }
 
@@ -112,8 +115,8 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
     float a = 0.f;
     if (has)
     {
-        pid               = p.lists[(size_t)pix * K + sub];
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
+        pid               = p.lists[((size_t)(unsigned)pix << kshift) + sub];
+        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
         const float4 r0   = rec[0];
 #pragma unroll
         for (int q = 0; q < CPAD / 4; ++q)
@@ -124,7 +127,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
             desc[4 * q + 2] = t.z;
             desc[4 * q + 3] = t.w;
         }
-        const float mfac = 1.f / float(1 << layer);
+        const float mfac = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
         const float ux = r0.x * mfac, uy = r0.y * mfac;
         float w = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
         if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
@@ -169,7 +172,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
         for (int c = 0; c < C; ++c) e[1 + c] = ta * g[c];
 #pragma unroll
         for (int c = 1 + C; c < EF; ++c) e[c] = 0.f;
-        float4* dst = reinterpret_cast<float4*>(p.entry_grad + ((size_t)pix * K + sub) * EF);
+        float4* dst = reinterpret_cast<float4*>(p.entry_grad + (((size_t)(unsigned)pix << kshift) + sub) * EF);
 #pragma unroll
         for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
     }
@@ -178,8 +181,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, lon
 template <int C>
 __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardParams p)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int P    = p.geom.bin_off[p.num_layers] * kTilePixels;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     double acc_bg[C];
 #pragma unroll
     for (int i = 0; i < C; ++i) acc_bg[i] = 0.0;
@@ -192,27 +194,30 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
     const long long num_tiles   = p.geom.bin_off[p.num_layers];
     const long long tile_stride = (long long)(gridDim.x / (kPerTile * kNumXcd)) * kNumXcd;
 
-    for (long long lb = xcd_tile_block(blockIdx.x, kPerTile); lb < num_tiles * kPerTile; lb += tile_stride * kPerTile)
+    for (long long lbl = xcd_tile_block(blockIdx.x, kPerTile); lbl < num_tiles * kPerTile; lbl += tile_stride * kPerTile)
     {
+        const int lb = (int)lbl;  // quarter tile number; all its pixels exist (tiles are padded to 1024 pixels)
+        // the quarter's pixels share a tile: its layer and position are found once, on the scalar unit
+        const TileCtx tc      = tile_ctx(p.geom, lb / kPerTile);
+        const float* const gi = p.grad_image[tc.layer];
         // lane -> pixel (lane % 8) of this wavefront's group number lane / 8
-        const long long my_pix = lb * kQuarter + ((lane >> 3) * 4 + wave) * 8 + (lane & 7);
-        int m_all              = my_pix < P ? p.retained[my_pix] : 0;  // 0 for the padding of partial tiles
-        int m_grp              = m_all;
-        m_grp                  = max(m_grp, __shfl_xor(m_grp, 1));
-        m_grp                  = max(m_grp, __shfl_xor(m_grp, 2));
-        m_grp                  = max(m_grp, __shfl_xor(m_grp, 4));
+        const int my_pix = lb * kQuarter + ((lane >> 3) * 4 + wave) * 8 + (lane & 7);
+        int m_all        = p.retained[my_pix];  // 0 for the padding of partial tiles
+        int m_grp        = m_all;
+        m_grp            = max(m_grp, __shfl_xor(m_grp, 1));
+        m_grp            = max(m_grp, __shfl_xor(m_grp, 2));
+        m_grp            = max(m_grp, __shfl_xor(m_grp, 4));
 #pragma unroll 1
         for (int it = 0; it < 8; ++it)
         {
-            const long long pix_first = lb * kQuarter + (it * 4 + wave) * 8;
-            if (pix_first >= P) break;
-            const int m8 = __builtin_amdgcn_readfirstlane(__shfl(m_grp, it * 8));
+            const int pix_first = lb * kQuarter + (it * 4 + wave) * 8;
+            const int m8        = __builtin_amdgcn_readfirstlane(__shfl(m_grp, it * 8));
             if (m8 <= 8)
-                backward_pixel_rows<C, 8>(p, pix_first, __shfl(m_all, it * 8 + (lane >> 3)), acc_bg);
+                backward_pixel_rows<C, 8>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 3)), acc_bg);
             else
             {
-                backward_pixel_rows<C, 16>(p, pix_first, __shfl(m_all, it * 8 + (lane >> 4)), acc_bg);
-                backward_pixel_rows<C, 16>(p, pix_first + 4, __shfl(m_all, it * 8 + 4 + (lane >> 4)), acc_bg);
+                backward_pixel_rows<C, 16>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 4)), acc_bg);
+                backward_pixel_rows<C, 16>(p, tc, gi, pix_first + 4, __shfl(m_all, it * 8 + 4 + (lane >> 4)), acc_bg);
             }
         }
     }
@@ -239,9 +244,10 @@ template <int C>
 __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardParams p)
 {
     constexpr int EF   = (1 + C + 3) & ~3;
+    constexpr int RF   = 4 + ((C + 3) & ~3);  // floats per blend record
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
     const int lane     = threadIdx.x & 63;
-    const int K        = p.list_depth;
+    const int kshift   = p.list_depth == 16 ? 4 : 3;
     const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     float R[9];
     rotation_matrix(cam.V, R);
@@ -262,7 +268,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         if (!(tail.y > 0.f)) continue;
         const int tex       = __float_as_int(tail.x);
         const int max_layer = __float_as_int(tail.z);
-        const float4 r0     = *reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);  // ip.x ip.y size field conf
+        const float4 r0     = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);  // ip.x ip.y size field conf
         const float4 rv     = prec[0];  // view xyz, softplus'(raw size)
         const uint4* rk     = reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 32);
         const uint4 rk0 = rk[0], rk1 = rk[1];
@@ -293,8 +299,8 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             {
                 const unsigned j = (word >> (8 * corner)) & 0xFFu;
                 const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                const int pix = pix_index(p.geom, layer, gx, gy);
-                const float4* src = reinterpret_cast<const float4*>(p.entry_grad + ((size_t)pix * K + (j & 15u)) * EF);
+                const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
+                const float4* src  = reinterpret_cast<const float4*>(p.entry_grad + (size_t)((pix << kshift) + (j & 15u)) * EF);
 #pragma unroll
                 for (int q = 0; q < EF / 4; ++q) e[corner][q] = (j != 0xFFu) ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
             }

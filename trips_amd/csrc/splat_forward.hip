@@ -719,20 +719,22 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
 // list of the group is longer than 8 (two thirds of the pixels of a typical view have at most 4 entries: half the
 // lanes of a 16-lane row would idle through every instruction).
 template <int C, bool TRAIN, int ROW>
-__device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long long pix_first, bool group_in_range, int len_in,
-                                                int start_in)
+__device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const TileCtx& tc, float* img, int pix_first,
+                                                bool group_in_range, int len_in, int start_in)
 {
     constexpr int CPAD = (C + 3) & ~3;
+    constexpr int RF   = 4 + CPAD;  // floats per blend record
     const int lane     = threadIdx.x & 63;
     const int sub      = lane & (ROW - 1);
     const int grp      = lane / ROW;
-    const int P        = p.geom.bin_off[p.num_layers] * kTilePixels;  // tile-major numbering incl. padding
     const int K        = p.list_depth;
-    const long long pix_ll = pix_first + grp;
-    const bool in_range    = pix_ll < P && group_in_range;
-    const int pix          = in_range ? (int)pix_ll : 0;
-    int layer, gx, gy;
-    const bool live = pix_decode(p.geom, pix, layer, gx, gy) && in_range;  // false for the padding of partial tiles
+    const int kshift   = K == 16 ? 4 : 3;
+    // the group's pixels lie side by side in one row of the tile
+    const int pix   = group_in_range ? pix_first + grp : 0;
+    const int layer = tc.layer, lw = tc.w, lh = tc.h;
+    const int gx = tc.x0 + (pix & (kTile - 1)), gy = tc.y0 + ((pix >> kTileShift) & (kTile - 1));
+    const bool in_range = group_in_range;
+    const bool live     = in_range && gx < lw && gy < lh;  // false for the padding of partial tiles
 
     // length and first key of this lane's list: the caller has read them for the whole group
     const int len   = live ? len_in : 0;
@@ -762,8 +764,6 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     }
 
     // ---- blend (RenderForward.cu:820-1048) ----
-    const int lw = p.geom.w[layer], lh = p.geom.h[layer];
-
     const int n    = min(min(len, readable), K);
     const bool has = live && sub < n;
     const int pid  = (int)(unsigned)(best & 0xffffffffull);
@@ -775,7 +775,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
     for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
     if (has)
     {
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)pid * p.rec_floats);
+        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
         const float4 r0   = rec[0];
 #pragma unroll
         for (int q = 0; q < CPAD / 4; ++q)
@@ -786,7 +786,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
             desc[4 * q + 2] = t.z;
             desc[4 * q + 3] = t.w;
         }
-        const float m  = 1.f / float(1 << layer);
+        const float m  = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
         const float ux = r0.x * m, uy = r0.y * m;
         float w        = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
         if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
@@ -828,19 +828,21 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
 #pragma unroll
             for (int c = 0; c < C; ++c) col[c] += p.background[c] * (bgw * 1.f);
         }
-        float* img = p.image[layer];
+        // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
         if (p.layout == TRIPS_LAYOUT_CHW)
         {
             const size_t plane = (size_t)lw * lh;
-            float* o           = img + ((size_t)p.view_index * C) * plane + (size_t)gy * lw + gx;
+            float* o           = img + ((size_t)p.view_index * C) * plane;
+            const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
 #pragma unroll
-            for (int c = 0; c < C; ++c) o[c * plane] = col[c];
+            for (int c = 0; c < C; ++c) (o + c * plane)[at] = col[c];
         }
         else
         {
-            float* o = img + (((size_t)p.view_index * lh + gy) * lw + gx) * C;
+            float* o          = img + ((size_t)p.view_index * lh * lw) * C;
+            const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
 #pragma unroll
-            for (int c = 0; c < C; ++c) o[c] = col[c];
+            for (int c = 0; c < C; ++c) o[at + c] = col[c];
         }
     }
     // saved state, also for padding pixels (empty) so that every row of the tables is defined
@@ -852,17 +854,17 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, long lon
             p.lengths[pix]  = live ? len : 0;
         }
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
-        if (has && sub < ret) p.rank[(size_t)pid * 32 + slot] = (unsigned char)sub;
+        if (has && sub < ret) p.rank[((size_t)(unsigned)pid << 5) + slot] = (unsigned char)sub;
         const int mine = has ? pid : -1;
         if (ROW == 8)
         {
             // one 8-byte store per lane covers the pixel's whole row (K <= 16 ids): lanes 0..3 carry the ids of lane
             // pairs, the others the -1 padding
             const int lo = __shfl(mine, (2 * sub) & 7, 8), hi = __shfl(mine, (2 * sub + 1) & 7, 8);
-            if (2 * sub < K) *reinterpret_cast<int2*>(p.lists + (size_t)pix * K + 2 * sub) = sub < 4 ? make_int2(lo, hi) : make_int2(-1, -1);
+            if (2 * sub < K) *reinterpret_cast<int2*>(p.lists + (((size_t)(unsigned)pix << kshift) + 2 * sub)) = sub < 4 ? make_int2(lo, hi) : make_int2(-1, -1);
         }
         else if (sub < K)
-            p.lists[(size_t)pix * K + sub] = mine;
+            p.lists[((size_t)(unsigned)pix << kshift) + sub] = mine;
     }
 }
 
@@ -872,16 +874,20 @@ template <int C, bool TRAIN>
 __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
 {
     const int lane = threadIdx.x & 63;
-    const int P    = p.geom.bin_off[p.num_layers] * kTilePixels;
-    const long long nblocks     = ((long long)P + 31) / 32;  // 32 pixels per workgroup, 32 workgroups per tile
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int NB   = p.geom.bin_off[p.num_layers];
+    const long long nblocks     = (long long)NB * (kTilePixels / 32);  // 32 pixels per workgroup, 32 workgroups per tile
     const long long lblock      = xcd_tile_block(blockIdx.x, kTilePixels / 32);
-    const long long pix_first   = (lblock * 4 + (threadIdx.x >> 6)) * 8;
     const bool group_in_range   = lblock < nblocks;
+    const int pix_first         = group_in_range ? ((int)lblock * 4 + wave) * 8 : 0;
+    // the eight pixels share a tile: its layer and position are found once per wavefront, on the scalar unit
+    const TileCtx tc = tile_ctx(p.geom, pix_first >> (2 * kTileShift));
+    float* const img = p.image[tc.layer];
     // longest list of the eight pixels (lists that ran past the key storage count with what was written)
     int len8 = 0, my_len = 0, my_start = 0;  // lanes 0..7: one pixel of the group each
-    if (lane < 8 && group_in_range && pix_first + lane < P)
+    if (lane < 8 && group_in_range)
     {
-        const int pix = (int)(pix_first + lane);
+        const int pix = pix_first + lane;
         my_len        = p.counts[pix];  // 0 for the padding of partial tiles
         my_start      = p.cursor[pix];
         len8          = my_len;
@@ -893,11 +899,11 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     len8 = __builtin_amdgcn_readfirstlane(len8);
     // the rows take their pixel's length and list start from these lanes: no second memory round trip
     if (len8 <= 8)
-        sort_blend_rows<C, TRAIN, 8>(p, pix_first, group_in_range, __shfl(my_len, lane >> 3), __shfl(my_start, lane >> 3));
+        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 3), __shfl(my_start, lane >> 3));
     else
     {
-        sort_blend_rows<C, TRAIN, 16>(p, pix_first, group_in_range, __shfl(my_len, lane >> 4), __shfl(my_start, lane >> 4));
-        sort_blend_rows<C, TRAIN, 16>(p, pix_first + 4, group_in_range, __shfl(my_len, 4 + (lane >> 4)), __shfl(my_start, 4 + (lane >> 4)));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 4), __shfl(my_start, lane >> 4));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, __shfl(my_len, 4 + (lane >> 4)), __shfl(my_start, 4 + (lane >> 4)));
     }
 }
 

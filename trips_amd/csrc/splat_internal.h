@@ -124,6 +124,8 @@ struct PyramidGeom
     int32_t tiles_x[TRIPS_MAX_LAYERS];
     int32_t tiles_y[TRIPS_MAX_LAYERS];
     int32_t bin_off[TRIPS_MAX_LAYERS + 1];  // first bin of each layer; bin_off[L] = number of bins
+    // ceil(2^30 / tiles_x): (4 t * magic) >> 32 == t / tiles_x for t and tiles_x below 2^14 (kMaxBins is)
+    uint32_t tiles_x_magic[TRIPS_MAX_LAYERS];
 };
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Kernels that walk pixels remap their
@@ -143,6 +145,52 @@ __host__ __device__ inline int pix_index(const PyramidGeom& g, int layer, int x,
 {
     const int bin = g.bin_off[layer] + (y >> kTileShift) * g.tiles_x[layer] + (x >> kTileShift);
     return (bin << (2 * kTileShift)) | ((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1));
+}
+
+// The same on the device: tile counts and pixel coordinates are far below 2^24, so the full-rate 24-bit multiply is
+// exact.
+__device__ inline int pix_index_mul24(const PyramidGeom& g, int layer, int x, int y)
+{
+    const int bin = g.bin_off[layer] + (int)__umul24((unsigned)(y >> kTileShift), (unsigned)g.tiles_x[layer]) + (x >> kTileShift);
+    return (bin << (2 * kTileShift)) | ((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1));
+}
+
+// What the pixels of one 32 x 32 tile share: its layer, that layer's size and the tile's first pixel.
+struct TileCtx
+{
+    int layer, w, h, x0, y0;
+};
+
+// `bin` must be the same for the whole wavefront and come out of a scalar register (readfirstlane): the layer search
+// and the division by the layer's tile columns (a multiply by tiles_x_magic) then run on the scalar unit, once per
+// wavefront, instead of per lane with an integer division.
+__device__ __forceinline__ TileCtx tile_ctx(const PyramidGeom& g, int bin)
+{
+    int layer = 0, first = 0, tsx = g.tiles_x[0], w = g.w[0], h = g.h[0];
+    unsigned magic = g.tiles_x_magic[0];
+#pragma unroll
+    for (int l = 1; l < TRIPS_MAX_LAYERS; ++l)
+    {
+        if (l < g.num_layers && bin >= g.bin_off[l])
+        {
+            layer = l;
+            first = g.bin_off[l];
+            tsx   = g.tiles_x[l];
+            magic = g.tiles_x_magic[l];
+            w     = g.w[l];
+            h     = g.h[l];
+        }
+    }
+    const unsigned t  = (unsigned)(bin - first);
+    const unsigned ty = __umulhi(4u * t, magic);
+    const unsigned tx = t - ty * (unsigned)tsx;
+    TileCtx c;
+    c.layer = layer;
+    c.w     = w;
+    c.h     = h;
+    c.x0    = (int)(tx << kTileShift);
+    c.y0    = (int)(ty << kTileShift);
+    return c;
 }
 
 // internal pixel number -> (layer, x, y); false for the padding of partial tiles

@@ -51,50 +51,36 @@ __device__ __forceinline__ void log2_floor_ceil(float s, int& lo, int& hi)
     hi = lo + (man != 0 ? 1 : 0);
 }
 
-// compute_point_size_fac; grad may be nullptr
-__device__ __forceinline__ float layer_factor(float s, int layer, int max_layers, float* grad)
+// compute_point_size_fac (PointBlending.h:81-149) for s > 1 and more than one layer, the branch that interpolates
+// between two layers; written with selects only. (The other branch, 0.75 exp(s - 1) + 0.25 for a point that lands
+// in layer 0 only, is evaluated once per point by encode_size_field below.)
+// Between two layers the reference divides by 2^higher - 2^lower, which is 2^lower whenever the two differ (then
+// neither is clamped): multiplying by 2^-lower instead gives the same bits, the scaling being exact.
+__device__ __forceinline__ float layer_factor_interpolated(float s, int layer, int max_layers, float* grad)
 {
-    int layer_lower = 0, layer_higher = 0;
-    if (s > 1.f)
+    int lo, hi;
+    log2_floor_ceil(s, lo, hi);  // lo >= 0 as s > 1
+    const int layer_lower = min(lo, max_layers - 1), layer_higher = min(hi, max_layers - 1);
+    const float l_l = __uint_as_float((uint32_t)(127 + layer_lower) << 23);  // 2^lower
+    const float inv = __uint_as_float((uint32_t)(127 - layer_lower) << 23);  // 2^-lower
+    float f         = (s - l_l) * inv;
+    float J         = inv;
+    if (layer == layer_lower)
     {
-        int lo, hi;
-        log2_floor_ceil(s, lo, hi);
-        layer_lower  = min(max(0, lo), max_layers - 1);
-        layer_higher = min(max(0, hi), max_layers - 1);
+        f = 1.f - f;
+        J = -J;
+    }
+    if (layer_lower == layer_higher)
+    {
+        f = 1.f;
+        J = 1.f;
     }
     if (layer < layer_lower)
     {
-        if (grad) *grad = 0.f;
-        return 1.f;
+        f = 1.f;
+        J = 0.f;
     }
-    float f = 1.f;
-    if (layer_higher == 0)
-    {
-        f = 0.75f * exp_rn(s - 1.f) + 0.25f;
-        if (grad) *grad = 0.27591f * s;
-    }
-    else if (layer_lower == layer_higher)
-    {
-        if (grad) *grad = 1.f;
-    }
-    else
-    {
-        float l_l = float(1 << layer_lower);
-        float l_h = float(1 << layer_higher);
-        f         = (s - l_l) / (l_h - l_l);
-        if (layer == layer_lower) f = 1.f - f;
-        if (grad)
-        {
-            float J = 1.f / (l_h - l_l);
-            if (layer == layer_lower) J = -J;
-            *grad = J;
-        }
-        if (layer_lower == max_layers - 1)
-        {
-            f = 1.f;
-            if (grad) *grad = 1.f;
-        }
-    }
+    if (grad) *grad = J;
     return f;
 }
 
@@ -108,11 +94,11 @@ __device__ __forceinline__ float encode_size_field(float size_px, int max_layers
     return small_branch ? -(0.75f * exp_rn(size_px - 1.f) + 0.25f) : size_px;
 }
 
-// layer factor from the encoded size field; identical in value to layer_factor(size_px, ...)
+// layer factor from the encoded size field
 __device__ __forceinline__ float layer_factor_encoded(float field, int layer, int max_layers)
 {
     if (field < 0.f) return -field;
-    return layer_factor(field, layer, max_layers, nullptr);
+    return layer_factor_interpolated(field, layer, max_layers, nullptr);
 }
 
 // same with the reference's gradient; true_size is the un-encoded projected size
@@ -124,7 +110,7 @@ __device__ __forceinline__ float layer_factor_encoded_grad(float field, float tr
         *grad = 0.27591f * true_size;
         return -field;
     }
-    return layer_factor(field, layer, max_layers, grad);
+    return layer_factor_interpolated(field, layer, max_layers, grad);
 }
 
 struct Pose

@@ -136,6 +136,7 @@ void make_geom(const TripsSplatDesc& d, PyramidGeom& g)
             g.tiles_x[l]     = (cw + kTile - 1) / kTile;
             g.tiles_y[l]     = (ch + kTile - 1) / kTile;
             g.bin_off[l + 1] = g.bin_off[l] + g.tiles_x[l] * g.tiles_y[l];
+            g.tiles_x_magic[l] = g.tiles_x[l] > 0 ? ((1u << 30) + (uint32_t)g.tiles_x[l] - 1u) / (uint32_t)g.tiles_x[l] : 0u;
             if (!d.floor_layer_sizes)
             {
                 // PointRenderer.cu:385-389
@@ -156,6 +157,7 @@ void make_geom(const TripsSplatDesc& d, PyramidGeom& g)
             g.tiles_x[l]     = 0;
             g.tiles_y[l]     = 0;
             g.bin_off[l + 1] = g.bin_off[l];
+            g.tiles_x_magic[l] = 0;
         }
     }
 }
