@@ -121,11 +121,14 @@ def main():
             p.grad = grads[k]
         opt = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
 
+        small = [grads[k] for k in ("d_background", "d_pose", "d_intrinsics")]
+
         def step():
-            for g in grads.values():
+            # the per-point gradients are written by the backward, every element; only the small ones are added to
+            for g in small:
                 g.zero_()
             ctx.forward(desc, tin, images, saved, workspace)
-            ctx.backward(desc, tin, saved, grad_images, grads, workspace)
+            ctx.backward(desc, tin, saved, grad_images, grads, workspace, overwrite_point_grads=True)
             opt.step()
 
         for _ in range(args.warmup):
@@ -187,6 +190,7 @@ def main():
     sc, desc, t, tin, workspace, saved, images = (r[k] for k in ("sc", "desc", "t", "tin", "workspace", "saved", "images"))
     gen, grad_images, grads, opt, counters = (r[k] for k in ("gen", "grad_images", "grads", "opt", "counters"))
     nz, total_el, prof, ms_per_step = r["nz"], r["total_el"], r["prof"], r["ms_per_step"]
+    small = [grads[k] for k in ("d_background", "d_pose", "d_intrinsics")]  # the gradients that are added to
     N, C = desc.num_points, desc.num_channels
 
     alg = algorithmic_bytes(counters, N, C, adam_nonzero=nz, adam_zero=total_el - nz)
@@ -246,7 +250,7 @@ def main():
         zero_tail = [torch.zeros_like(im) for im in images[np_.num_layers:]]
 
         def train_step():
-            for g in grads.values():
+            for g in small:
                 g.zero_()
             net_opt.zero_grad(set_to_none=True)
             ctx.forward(desc, tin, images, saved, workspace)
@@ -254,7 +258,7 @@ def main():
             loss = (net.forward(ins) - target).abs().mean()
             loss.backward()
             gi = [t.grad for t in ins[:np_.num_layers]] + zero_tail
-            ctx.backward(desc, tin, saved, gi, grads, workspace)
+            ctx.backward(desc, tin, saved, gi, grads, workspace, overwrite_point_grads=True)
             opt.step()
             net_opt.step()
             return loss

@@ -113,16 +113,21 @@ typedef struct TripsSplatOut {
 } TripsSplatOut;
 
 /* Gradient outputs; the kernels ADD into these, the caller zeroes them first
- * (PointRendererCache::Build(info,false), PointRenderer.cu:226-272). NULL = not requested, where allowed. */
+ * (PointRendererCache::Build(info,false), PointRenderer.cu:226-272). NULL = not requested, where allowed.
+ * With overwrite_point_grads != 0 the four per-point outputs (d_texture, d_confidence, d_position, d_point_size) are
+ * WRITTEN instead: every element receives its value, zero where no gradient arrives (.w of d_position too), so the
+ * caller may pass uninitialised memory and skips four fills and the kernel the reads of a read-modify-write;
+ * d_background, d_pose and d_intrinsics are added to in either mode. */
 typedef struct TripsSplatGrads {
     float* d_texture;     /* [C,T]   required */
     float* d_confidence;  /* [T]     required */
     float* d_background;  /* [C]     required */
-    float* d_position;    /* [N,4]   or NULL (xyz written, .w untouched) */
+    float* d_position;    /* [N,4]   or NULL (xyz; .w untouched when adding) */
     float* d_point_size;  /* [N]     or NULL; NULL also drops the layer factor from d_confidence and
                                       d_position exactly as RenderBackward.cu:366-372 does */
     double* d_pose;       /* [F,6]   or NULL; translation first, rotation last */
     float* d_intrinsics;  /* [Cam,13] or NULL */
+    int32_t overwrite_point_grads; /* 0 = add into everything (the reference's contract); 1 = see above */
 } TripsSplatGrads;
 
 typedef struct TripsCtx TripsCtx;

@@ -38,17 +38,20 @@ class GpuRun:
         torch.cuda.synchronize()
         return [x.cpu().numpy() for x in out]
 
-    def backward(self, grad_images, want_position=True, want_point_size=True, want_pose=True, want_intrinsics=True):
+    def backward(self, grad_images, want_position=True, want_point_size=True, want_pose=True, want_intrinsics=True,
+                 overwrite=False):
+        """overwrite: the per-point outputs start as NaN and the call runs with overwrite_point_grads."""
         d, dev = self.desc, self.ctx.device
         z = lambda shape, dt=torch.float32: torch.zeros(shape, dtype=dt, device=dev)
-        grads = dict(d_texture=z((d.num_channels, d.num_texels)), d_confidence=z(d.num_texels),
+        big = (lambda shape: torch.full(shape, float("nan"), dtype=torch.float32, device=dev)) if overwrite else z
+        grads = dict(d_texture=big((d.num_channels, d.num_texels)), d_confidence=big((d.num_texels,)),
                      d_background=z(d.num_channels),
-                     d_position=z((d.num_points, 4)) if want_position else None,
-                     d_point_size=z(d.num_points) if want_point_size else None,
+                     d_position=big((d.num_points, 4)) if want_position else None,
+                     d_point_size=big((d.num_points,)) if want_point_size else None,
                      d_pose=z((d.num_images, 6), torch.float64) if want_pose else None,
                      d_intrinsics=z((d.num_cameras, 13)) if want_intrinsics else None)
         gi = [torch.as_tensor(np.ascontiguousarray(g), dtype=torch.float32).to(dev) for g in grad_images]
-        self.ctx.backward(d, self.tin, self.saved, gi, grads, self.workspace)
+        self.ctx.backward(d, self.tin, self.saved, gi, grads, self.workspace, overwrite_point_grads=overwrite)
         torch.cuda.synchronize()
         return {k: (None if v is None else v.cpu().numpy()) for k, v in grads.items()}
 

@@ -161,6 +161,43 @@ def test_backward_views_crop_distortion_optional_outputs(oracle):
     _check_backward(oracle, sc, d, want_position=False, want_pose=False, want_intrinsics=False)
 
 
+@pytest.mark.parametrize("case", ["two_views", "shared_columns", "spare_columns", "bad_index", "no_size_no_position"])
+def test_backward_overwrite_mode_equals_adding_into_zeros(case):
+    """overwrite_point_grads: the per-point outputs start as NaN and must come out bit-equal to what adding into
+    zeroed outputs gives (second view added on top of the first; descriptor columns shared between points, columns
+    no point uses and skipped points all end up defined)."""
+    from tests.gpu_util import GpuRun
+    views = 2 if case == "two_views" else 1
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=41, views=views, radius=(0.004, 0.4))
+    if case == "shared_columns":
+        sc.index = (np.arange(3000) // 2).astype(np.int32)  # two points per column, the upper half unused
+    if case == "spare_columns":
+        extra = 100
+        sc.texture = np.concatenate([sc.texture, np.ones((sc.texture.shape[0], extra), np.float32)], axis=1)
+        sc.confidence = np.concatenate([sc.confidence, np.full(extra, 0.5, np.float32)])
+    if case == "bad_index":
+        sc.index = sc.index.copy()
+        sc.index[::5] = sc.texture.shape[1] + 7
+    d = abi.desc_for_scene(sc)
+    want = dict(want_point_size=False, want_position=False) if case == "no_size_no_position" else {}
+    rng = np.random.default_rng(8)
+    run = GpuRun(sc, d)
+    images = run.forward()
+    grads = [rng.normal(0, 1, im.shape).astype(np.float32) for im in images]
+    added = run.backward(grads, **want)
+    written = run.backward(grads, overwrite=True, **want)
+    for k, v in added.items():
+        if v is None:
+            assert written[k] is None
+            continue
+        assert np.isfinite(written[k]).all(), k
+        if k in ("d_background", "d_pose", "d_intrinsics"):
+            np.testing.assert_allclose(written[k], v, rtol=1e-4, atol=1e-6)  # float atomics across workgroups
+        else:
+            assert np.array_equal(written[k], v), k
+    assert np.abs(added["d_texture"]).max() > 0
+
+
 def test_displacement_forward_backward(oracle):
     """Per-view displacements of the point positions (dynamic_refinement_t, PointRenderer.cu:703-713)."""
     sc = scenes.tiny(n=4000, w=70, h=50, f=60.0, num_layers=4, list_depth=16, seed=77, views=3, radius=(0.004, 0.4))

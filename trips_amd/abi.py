@@ -95,6 +95,7 @@ class TripsSplatGrads(C.Structure):
         ("d_point_size", C.c_void_p),
         ("d_pose", C.c_void_p),
         ("d_intrinsics", C.c_void_p),
+        ("overwrite_point_grads", C.c_int32),
     ]
 
 

@@ -255,6 +255,10 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     const bool want_intr = p.d_intrinsics != nullptr;
     const bool want_size = p.d_point_size != nullptr;
     const bool identity  = p.header->not_identity == 0;  // index[pid] == pid for every point
+    const bool overwrite = p.overwrite != 0;             // outputs are written, not added to
+    // In that mode every point stores all its outputs (zeros where it has no gradient), all lanes at one place, so that
+    // whole lines are written. (Descriptor columns other than the points' own, and all of them when the index is not
+    // the identity, were cleared by zero_texel_grads_kernel.)
 
     // a thread sees a handful of points: its own sums stay in single precision, everything across threads is double
     float acc[NACC];
@@ -265,13 +269,20 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     {
         const float4* prec = reinterpret_cast<const float4*>(p.prec + (size_t)pid * kPointRecordFloats);
         const float4 tail  = prec[1];  // {texture index, depth, layers written, size_px}
-        if (!(tail.y > 0.f)) continue;
+        const bool live = tail.y > 0.f;
+        if (!live && !overwrite) continue;
         const int tex       = __float_as_int(tail.x);
-        const int max_layer = __float_as_int(tail.z);
-        const float4 r0     = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);  // ip.x ip.y size field conf
-        const float4 rv     = prec[0];  // view xyz, softplus'(raw size)
-        const uint4* rk     = reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 32);
-        const uint4 rk0 = rk[0], rk1 = rk[1];
+        const int max_layer = live ? __float_as_int(tail.z) : 0;
+        float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), rv = r0;  // ip.x ip.y size field conf; view xyz, softplus'(raw size)
+        uint4 rk0 = make_uint4(~0u, ~0u, ~0u, ~0u), rk1 = rk0;
+        if (live)
+        {
+            r0              = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
+            rv              = prec[0];
+            const uint4* rk = reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 32);
+            rk0             = rk[0];
+            rk1             = rk[1];
+        }
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;
         float tex_grad[C];
@@ -349,44 +360,59 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         do_layer(5, rk1.y);
         do_layer(6, rk1.z);
         do_layer(7, rk1.w);
-        if (!any) continue;
+        if (!any && !overwrite) continue;
 
-        float g_point[3], g_pose[6], g_k[5], g_dis[8];
-        project_backward(cam, R, rv.x, rv.y, rv.z, d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
+        float g_point[3] = {0.f, 0.f, 0.f}, g_pose[6], g_k[5], g_dis[8];
+        if (any)
+        {
+            project_backward(cam, R, rv.x, rv.y, rv.z, d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
+            if (want_pose)
+            {
+#pragma unroll
+                for (int k = 0; k < 6; ++k) acc[k] += g_pose[k];
+            }
+            if (want_intr)
+            {
+#pragma unroll
+                for (int k = 0; k < 5; ++k) acc[6 + k] += g_k[k];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) acc[11 + k] += g_dis[k];
+            }
+        }
 
-        if (identity)
+        if (identity && overwrite)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c) p.d_texture[(size_t)c * p.num_texels + tex] = tex_grad[c];
+            p.d_confidence[tex] = conf_grad;
+        }
+        else if (identity)
         {
 #pragma unroll
             for (int c = 0; c < C; ++c) p.d_texture[(size_t)c * p.num_texels + tex] += tex_grad[c];
             p.d_confidence[tex] += conf_grad;
         }
-        else
+        else if (any)
         {
 #pragma unroll
             for (int c = 0; c < C; ++c) unsafeAtomicAdd(p.d_texture + (size_t)c * p.num_texels + tex, tex_grad[c]);
             unsafeAtomicAdd(p.d_confidence + tex, conf_grad);
         }
-        if (want_size) p.d_point_size[pid] += size_grad;
+        if (want_size)
+        {
+            if (overwrite)
+                p.d_point_size[pid] = size_grad;
+            else
+                p.d_point_size[pid] += size_grad;
+        }
         if (p.d_position)
         {
             float4* dp = reinterpret_cast<float4*>(p.d_position) + pid;
-            float4 v   = *dp;
+            float4 v   = overwrite ? make_float4(0.f, 0.f, 0.f, 0.f) : *dp;
             v.x += g_point[0];
             v.y += g_point[1];
             v.z += g_point[2];
             *dp = v;
-        }
-        if (want_pose)
-        {
-#pragma unroll
-            for (int k = 0; k < 6; ++k) acc[k] += g_pose[k];
-        }
-        if (want_intr)
-        {
-#pragma unroll
-            for (int k = 0; k < 5; ++k) acc[6 + k] += g_k[k];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) acc[11 + k] += g_dis[k];
         }
     }
 
@@ -419,11 +445,23 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     }
 }
 
-__global__ __launch_bounds__(256) void fill_u32_kernel(unsigned* __restrict__ p, unsigned v, long long n)
+// Overwrite mode, before the point pass of the first view: the descriptor and confidence gradients of the columns
+// that the point pass does not write itself. With the identity index (the forward noted it in the header) those are
+// the columns past the last point; otherwise all of them, the point pass then adds with atomics.
+__global__ __launch_bounds__(256) void zero_texel_grads_kernel(const ViewHeader* __restrict__ header, float* __restrict__ d_texture,
+                                                               float* __restrict__ d_confidence, int channels, int num_texels,
+                                                               int num_points)
 {
-    long long i      = (long long)blockIdx.x * 256 + threadIdx.x;
-    long long stride = (long long)gridDim.x * 256;
-    for (; i < n; i += stride) p[i] = v;
+    const int first = header->not_identity == 0 ? min(num_points, num_texels) : 0;
+    const int n     = num_texels - first;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < (long long)n * (channels + 1); i += (long long)gridDim.x * 256)
+    {
+        const int c = (int)(i / n), t = first + (int)(i - (long long)c * n);
+        if (c < channels)
+            d_texture[(size_t)c * num_texels + t] = 0.f;
+        else
+            d_confidence[t] = 0.f;
+    }
 }
 
 #define TRIPS_BW_DISPATCH(KERNEL, BLOCKS)                                                                      \
@@ -453,6 +491,9 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
         blocks                = ((blocks + 4 * kNumXcd - 1) / (4 * kNumXcd)) * (4 * kNumXcd);  // whole groups of 8 tiles x 4
         TRIPS_BW_DISPATCH(backward_pixels_kernel, blocks);
     }
+    if (p.overwrite)
+        hipLaunchKernelGGL(zero_texel_grads_kernel, dim3(1024), dim3(256), 0, stream, p.header, p.d_texture, p.d_confidence, channels,
+                           p.num_texels, N);
     if (N > 0)
     {
         ProfScope ps(prof, "backward_points", stream);

@@ -102,8 +102,9 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         {
             // a column outside the descriptor table: leave the point out (reported by the status query) rather
             // than read past the tables
-            bad_index = true;
-            skip      = true;
+            bad_index    = true;
+            not_identity = true;  // the backward then never uses the point's own number as a column
+            skip         = true;
         }
         if (p.viewer_only && !skip)
         {

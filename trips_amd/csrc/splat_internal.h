@@ -340,6 +340,7 @@ struct BackwardParams
     float* d_point_size;
     double* d_pose;       // row of this view's image or nullptr
     float* d_intrinsics;  // row of this view's camera or nullptr
+    int32_t overwrite;    // the per-point outputs are written, not added to (first view of a call in that mode)
 };
 
 }  // namespace trips

@@ -498,6 +498,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.d_point_size = grads->d_point_size;
         p.d_pose       = grads->d_pose ? grads->d_pose + 6 * (size_t)d.views[b].image_index : nullptr;
         p.d_intrinsics = grads->d_intrinsics ? grads->d_intrinsics + 13 * (size_t)d.views[b].camera_index : nullptr;
+        p.overwrite    = (grads->overwrite_point_grads != 0 && b == 0) ? 1 : 0;  // later views add to the first one's
         hipError_t e   = launch_backward_view(p, d.num_channels, stream, ctx->prof.enabled ? &ctx->prof : nullptr);
         if (e != hipSuccess) return hip_fail(e, "backward launch");
     }
