@@ -29,15 +29,15 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (135407, 473823),
-    "bin_scatter": (48405, 202963),
+    "project_bin": (135365, 473833),
+    "bin_scatter": (48402, 203115),
     "tile_count": (51871, 34387),
-    "tile_scatter": (87155, 451010),
+    "tile_scatter": (87336, 451243),
     "fill_rank": (15, 187500),
-    "sort_blend": (394389, 417377),
-    "backward_pixels": (471406, 417113),
-    "backward_points": (1223690, 198835),
-    "adam_fused": (582968, 792823),
+    "sort_blend": (397626, 424924),
+    "backward_pixels": (490246, 417187),
+    "backward_points": (1107439, 234887),
+    "adam_fused": (582979, 792823),
 }
 
 
