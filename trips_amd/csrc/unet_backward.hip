@@ -29,7 +29,7 @@ typedef half8 half8_unaligned __attribute__((aligned(2)));
 // d(elu(f) * sigmoid(m)) for an incoming gradient da
 __device__ __forceinline__ void gate_backward(float da, float f, float m, float& df, float& dm)
 {
-    const float s  = 1.f / (1.f + __expf(-m));
+    const float s  = __builtin_amdgcn_rcpf(1.f + __expf(-m));  // 1 ulp; the gradients are rounded to fp16 next
     const float ex = __expf(f);
     const float e  = f > 0.f ? f : ex - 1.f;
     const float de = f > 0.f ? 1.f : ex;

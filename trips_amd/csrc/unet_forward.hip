@@ -198,7 +198,8 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
                     s_pre[tp * PS + NPAD / 2 + ch] = _Float16(g);
                 }
                 const float e = f > 0.f ? f : (__expf(f) - 1.f);
-                const float s = 1.f / (1.f + __expf(-g));
+                // v_rcp_f32 is good to 1 ulp of fp32 and the product is rounded to fp16 next: no IEEE division needed
+                const float s = __builtin_amdgcn_rcpf(1.f + __expf(-g));
                 s_act[tp * AS + ch] = ch < p.cout ? _Float16(e * s) : _Float16(0.f);
             }
         }
