@@ -98,6 +98,28 @@ def test_forward_edge_cases(oracle):
     np.testing.assert_array_equal(lists[8 * 16 + 8], np.arange(16))
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_shapes_forward_backward(oracle, seed):
+    """Image sizes that are not multiples of the 32-pixel tiles (down to a few pixels, where the coarse layers are one
+    pixel wide), every layer count, both list depths, both layouts and layer-size rules, several views."""
+    rng = np.random.default_rng(1000 + seed)
+    w, h = int(rng.integers(3, 150)), int(rng.integers(3, 110))
+    L = int(rng.integers(1, 9))
+    K = int(rng.choice([8, 16]))
+    C = int(rng.choice([3, 4, 4, 6, 8, 16]))
+    views = int(rng.integers(1, 4))
+    floor = bool(rng.integers(0, 2))
+    if floor:
+        L = min(L, int(np.floor(np.log2(min(w, h)))) + 1)  # no empty layers
+    sc = scenes.tiny(n=int(rng.integers(200, 3000)), w=w, h=h, f=float(0.9 * max(w, h)), num_layers=L, list_depth=K,
+                     seed=300 + seed, views=views, channels=C, radius=(0.004, 0.5))
+    sc.confidence = (sc.confidence ** 0.3).astype(np.float32)
+    layout = int(rng.choice([abi.TRIPS_LAYOUT_CHW, abi.TRIPS_LAYOUT_HWC]))
+    d = abi.desc_for_scene(sc, layout=layout, floor_layer_sizes=floor, background_mode=int(rng.integers(0, 2)))
+    _check_forward(oracle, sc, d)
+    _check_backward(oracle, sc, d, seed=seed)
+
+
 def test_transmittance_cutoff_matches(oracle):
     n = 12
     sc = scenes.tiny(n=n, w=16, h=16, f=30.0, num_layers=1, list_depth=16, seed=3, background=0.5)
