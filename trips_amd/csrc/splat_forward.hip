@@ -410,15 +410,6 @@ __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restr
 // totals): exclusive scan of the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 |
 // point id) into their lists. A slice adds its counts to the tile's with atomics; when it places its keys it first
 // counts its own entries per pixel again and claims that many slots of each pixel's list with one atomic.
-__device__ __forceinline__ void tile_of_bin(const PyramidGeom& g, int bin, int& layer, int& tx, int& ty)
-{
-    layer = 0;
-    while (layer + 1 < g.num_layers && bin >= g.bin_off[layer + 1]) ++layer;
-    const int t = bin - g.bin_off[layer];
-    ty          = t / g.tiles_x[layer];
-    tx          = t - ty * g.tiles_x[layer];
-}
-
 // Calls f(local pixel index) for each of the entry's 2 x 2 pixels that lie in tile (tx, ty).
 template <typename F>
 __device__ __forceinline__ void for_corners_in_tile(const uint4& e, int tx, int ty, F&& f)
@@ -452,7 +443,9 @@ template <bool SCATTER>
 __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
 {
     __shared__ int s_cnt[kTilePixels];
+    // per-pixel entries of a slice (placement pass only; one word in the counting pass, whose code below never runs)
     __shared__ int s_mine[SCATTER ? kTilePixels : 1];
+    auto mine = [&](int i) -> int& { return s_mine[SCATTER ? i : 0]; };
     __shared__ int s_wave[4];
     const int NB = p.geom.bin_off[p.num_layers];
     int bin      = blockIdx.x;
@@ -474,8 +467,8 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
         bin   = lo;
         slice = e - p.slice_start[bin];
     }
-    int layer, tx, ty;
-    tile_of_bin(p.geom, bin, layer, tx, ty);
+    const TileCtx tc = tile_ctx(p.geom, bin);
+    const int tx = tc.x0 >> kTileShift, ty = tc.y0 >> kTileShift;
     long long first = p.bin_start[bin];
     long long last  = p.bin_start[bin + 1];
     if (last > p.capacity) last = p.capacity;  // entries beyond the capacity were dropped by the scatter
@@ -538,7 +531,7 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     }
     if (lane == 63) s_wave[wave] = inc;
     if (slice >= 0)
-        for (int i = threadIdx.x; i < kTilePixels; i += 256) s_mine[SCATTER ? i : 0] = 0;
+        for (int i = threadIdx.x; i < kTilePixels; i += 256) mine(i) = 0;
     __syncthreads();
     int prefix = inc - sum;
     for (int w = 0; w < wave; ++w) prefix += s_wave[w];
@@ -574,11 +567,11 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     {
         // this slice's share of every pixel's list: count, then claim the slots with one atomic per pixel
         int32_t* run = p.run + (size_t)bin * kTilePixels;
-        for_entries(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&s_mine[SCATTER ? i : 0], 1); }); });
+        for_entries(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&mine(i), 1); }); });
         __syncthreads();
         for (int i = threadIdx.x; i < kTilePixels; i += 256)
         {
-            const int c = s_mine[SCATTER ? i : 0];
+            const int c = mine(i);
             if (c) s_cnt[i] += atomicAdd(&run[i], c);  // cleared before the counting kernel
         }
         __syncthreads();

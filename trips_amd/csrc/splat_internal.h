@@ -193,19 +193,6 @@ __device__ __forceinline__ TileCtx tile_ctx(const PyramidGeom& g, int bin)
     return c;
 }
 
-// internal pixel number -> (layer, x, y); false for the padding of partial tiles
-__host__ __device__ inline bool pix_decode(const PyramidGeom& g, int ipix, int& layer, int& x, int& y)
-{
-    const int bin = ipix >> (2 * kTileShift), loc = ipix & (kTilePixels - 1);
-    layer         = 0;
-    while (layer + 1 < g.num_layers && bin >= g.bin_off[layer + 1]) ++layer;
-    const int t  = bin - g.bin_off[layer];
-    const int ty = t / g.tiles_x[layer], tx = t - ty * g.tiles_x[layer];
-    x            = (tx << kTileShift) + (loc & (kTile - 1));
-    y            = (ty << kTileShift) + (loc >> kTileShift);
-    return x < g.w[layer] && y < g.h[layer];
-}
-
 // Header at the start of each view's saved state (and of the workspace status block).
 struct ViewHeader
 {
