@@ -65,7 +65,7 @@ __device__ __forceinline__ double wave_sum(double v)
 // than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
 template <int C, int ROW>
 __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, const TileCtx& tc, const float* gi, int pix_first,
-                                                    int m_in, double (&acc_bg)[C])
+                                                    int m_in, float (&acc_bg)[C])
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int RF   = 4 + CPAD;          // floats per blend record
@@ -161,7 +161,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
     if (bg_reached && sub == 0)
     {
 #pragma unroll
-        for (int c = 0; c < C; ++c) acc_bg[c] += (double)(T_after * g[c]);
+        for (int c = 0; c < C; ++c) acc_bg[c] += T_after * g[c];
     }
     if (has)
     {
@@ -178,13 +178,16 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
     }
 }
 
+// (up to 4 channels the kernel needs 65 registers without the hint and fits the 64 of 8 wavefronts per SIMD with it,
+// no spills; with more channels the hint would cost spills)
 template <int C>
-__global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardParams p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 8 : 1))) void backward_pixels_kernel(const BackwardParams p)
 {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    double acc_bg[C];
+    // a lane sees a few dozen pixels: its own sums stay in single precision, everything across lanes is double
+    float acc_bg[C];
 #pragma unroll
-    for (int i = 0; i < C; ++i) acc_bg[i] = 0.0;
+    for (int i = 0; i < C; ++i) acc_bg[i] = 0.f;
 
     // A workgroup walks quarters of tiles (256 pixels = 32 groups of eight), 4 workgroups per tile, all on one XCD.
     // A wavefront takes every fourth group; it reads the retained counts of all its 64 pixels with one load, so the
@@ -226,7 +229,7 @@ __global__ __launch_bounds__(256) void backward_pixels_kernel(const BackwardPara
 #pragma unroll
     for (int i = 0; i < C; ++i)
     {
-        double v = wave_sum(acc_bg[i]);
+        double v = wave_sum((double)acc_bg[i]);
         if (lane == 0) s_acc[threadIdx.x >> 6][i] = v;
     }
     __syncthreads();
