@@ -714,7 +714,7 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
 // lanes of a 16-lane row would idle through every instruction).
 template <int C, bool TRAIN, int ROW>
 __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const TileCtx& tc, float* img, int pix_first,
-                                                bool group_in_range, int len_in, int start_in)
+                                                bool group_in_range, int len_in, int start_in, int readable_in)
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int RF   = 4 + CPAD;  // floats per blend record
@@ -730,18 +730,17 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     const bool in_range = group_in_range;
     const bool live     = in_range && gx < lw && gy < lh;  // false for the padding of partial tiles
 
-    // length and first key of this lane's list: the caller has read them for the whole group
-    const int len   = live ? len_in : 0;
-    long long start = live ? start_in : 0;
-    // entries beyond the capacity were never written
-    int readable = len;
-    if (start + len > p.capacity) readable = (int)max(0ll, p.capacity - start);
+    // length, first key and number of keys actually written (the key storage may have ended inside the list) of this
+    // lane's list: the caller has them for the whole group
+    const int len = live ? len_in : 0;
+    int start     = live ? start_in : 0;
+    int readable  = live ? readable_in : 0;
 
     const u64 kInf = ~0ull;
     u64 best       = kInf;
     if (ROW == 8)
     {
-        if (sub < readable) best = p.keys[start + sub];
+        if (sub < readable) best = p.keys[(unsigned)(start + sub)];
         best = half_sort8(best);
     }
     else
@@ -751,7 +750,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
         {
             // a long list: the reduction pass left the 16 smallest keys of each of its segments
             src      = p.cand;
-            start    = (-1 - start) * 16ll;
+            start    = (-1 - start) * 16;
             readable = ((len + kLongSegment - 1) / kLongSegment) * 16;
         }
         best = row_top16(src, start, readable);
@@ -878,26 +877,30 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     const TileCtx tc = tile_ctx(p.geom, pix_first >> (2 * kTileShift));
     float* const img = p.image[tc.layer];
     // longest list of the eight pixels (lists that ran past the key storage count with what was written)
-    int len8 = 0, my_len = 0, my_start = 0;  // lanes 0..7: one pixel of the group each
+    int my_len = 0, my_start = 0, my_read = 0;  // lanes 0..7: one pixel of the group each
     if (lane < 8 && group_in_range)
     {
         const int pix = pix_first + lane;
         my_len        = p.counts[pix];  // 0 for the padding of partial tiles
-        my_start      = p.cursor[pix];
-        len8          = my_len;
-        if (my_start >= 0 && (long long)my_start + len8 > p.capacity) len8 = (int)max(0ll, p.capacity - my_start);
+        my_start      = p.cursor[pix];  // negative: a long list, reduced to candidates by long_list_reduce_kernel
+        my_read       = my_len;
+        if (my_start >= 0 && (long long)my_start + my_len > p.capacity) my_read = (int)max(0ll, p.capacity - my_start);
     }
+    int len8 = my_read;
     len8 = max(len8, __shfl_xor(len8, 1));
     len8 = max(len8, __shfl_xor(len8, 2));
     len8 = max(len8, __shfl_xor(len8, 4));
     len8 = __builtin_amdgcn_readfirstlane(len8);
     // the rows take their pixel's length and list start from these lanes: no second memory round trip
     if (len8 <= 8)
-        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 3), __shfl(my_start, lane >> 3));
+        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 3), __shfl(my_start, lane >> 3),
+                                     __shfl(my_read, lane >> 3));
     else
     {
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 4), __shfl(my_start, lane >> 4));
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, __shfl(my_len, 4 + (lane >> 4)), __shfl(my_start, 4 + (lane >> 4)));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 4), __shfl(my_start, lane >> 4),
+                                      __shfl(my_read, lane >> 4));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, __shfl(my_len, 4 + (lane >> 4)),
+                                      __shfl(my_start, 4 + (lane >> 4)), __shfl(my_read, 4 + (lane >> 4)));
     }
 }
 
