@@ -35,7 +35,7 @@ PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
     "tile_scatter": (87336, 451243),
     "fill_rank": (15, 187500),
     "sort_blend": (397626, 424924),
-    "backward_pixels": (490246, 417187),
+    "backward_pixels": (528446, 417602),
     "backward_points": (1107439, 234887),
     "adam_fused": (582979, 792823),
 }
