@@ -424,29 +424,32 @@ __device__ __forceinline__ void for_corners_in_tile(const uint4& e, int tx, int 
 }
 
 // Walks entries [0, n) with the workgroup, four loads of a thread in flight together.
-template <typename F>
+template <int THREADS, typename F>
 __device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, int n, F&& f)
 {
-    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * 256)
+    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * THREADS)
     {
         uint4 e[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if (i0 + 256 * j < n) e[j] = entries[i0 + 256 * j];
+            if (i0 + THREADS * j < n) e[j] = entries[i0 + THREADS * j];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            if (i0 + 256 * j < n) f(e[j]);
+            if (i0 + THREADS * j < n) f(e[j]);
     }
 }
 
-template <bool SCATTER>
-__global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
+// (THREADS: 256 for the counting pass, whose idle workgroups for unused slices are cheaper that way; 1024 for the
+// placement pass, where two workgroups per CU with their 64 KB of LDS then make 32 wavefronts instead of 8)
+constexpr int kScatterThreads = 1024;
+template <bool SCATTER, int THREADS>
+__global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams p)
 {
     __shared__ int s_cnt[kTilePixels];
     // per-pixel entries of a slice (placement pass only; one word in the counting pass, whose code below never runs)
     __shared__ int s_mine[SCATTER ? kTilePixels : 1];
     auto mine = [&](int i) -> int& { return s_mine[SCATTER ? i : 0]; };
-    __shared__ int s_wave[4];
+    __shared__ int s_wave[THREADS / 64];
     const int NB = p.geom.bin_off[p.num_layers];
     int bin      = blockIdx.x;
     int slice    = -1;  // -1: the tile's own workgroup
@@ -485,12 +488,12 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     if (!SCATTER)
     {
         if (split && slice < 0) return;  // the slices do the counting
-        for (int i = threadIdx.x; i < kTilePixels; i += 256) s_cnt[i] = 0;
+        for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
-        for_entries(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&s_cnt[i], 1); }); });
+        for_entries<THREADS>(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&s_cnt[i], 1); }); });
         __syncthreads();
         int sum = 0;
-        for (int i = threadIdx.x; i < kTilePixels; i += 256)
+        for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
             const int c = s_cnt[i];
             if (slice < 0)
@@ -504,7 +507,8 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
         __syncthreads();
         if (threadIdx.x == 0)
         {
-            const int total = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+            int total = 0;
+            for (int w = 0; w < THREADS / 64; ++w) total += s_wave[w];
             if (slice < 0)
                 p.bin_total[bin] = total;
             else
@@ -513,11 +517,12 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
         return;
     }
 
-    // exclusive scan of the tile's 1024 lengths: 4 consecutive pixels per thread
-    const int base4 = threadIdx.x * 4;
-    int v[4], sum = 0;
+    // exclusive scan of the tile's 1024 lengths: PER consecutive pixels per thread
+    constexpr int PER = kTilePixels / THREADS;
+    const int base4   = threadIdx.x * PER;
+    int v[PER], sum = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < PER; ++i)
     {
         v[i] = counts[base4 + i];
         sum += v[i];
@@ -531,14 +536,14 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     }
     if (lane == 63) s_wave[wave] = inc;
     if (slice >= 0)
-        for (int i = threadIdx.x; i < kTilePixels; i += 256) mine(i) = 0;
+        for (int i = threadIdx.x; i < kTilePixels; i += THREADS) mine(i) = 0;
     __syncthreads();
     int prefix = inc - sum;
     for (int w = 0; w < wave; ++w) prefix += s_wave[w];
     const int key_start = p.bin_key_start[bin];
     int32_t* cursor     = p.cursor + (size_t)bin * kTilePixels;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < PER; ++i)
     {
         s_cnt[base4 + i] = key_start + prefix;  // running slot of the pixel
         if (slice < 0)
@@ -567,15 +572,15 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     {
         // this slice's share of every pixel's list: count, then claim the slots with one atomic per pixel
         int32_t* run = p.run + (size_t)bin * kTilePixels;
-        for_entries(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&mine(i), 1); }); });
+        for_entries<THREADS>(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&mine(i), 1); }); });
         __syncthreads();
-        for (int i = threadIdx.x; i < kTilePixels; i += 256)
+        for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
             const int c = mine(i);
             if (c) s_cnt[i] += atomicAdd(&run[i], c);  // cleared before the counting kernel
         }
         __syncthreads();
-        for_entries(entries, n,
+        for_entries<THREADS>(entries, n,
                     [&](const uint4& e)
                     {
                         const u64 key = ((u64)e.x << 32) | (u64)e.y;
@@ -597,7 +602,7 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     extern __shared__ u64 s_keys[];
     const int tile_total = p.bin_key_start[bin + 1] - key_start;
     const bool staged    = tile_total <= kStageKeys && (long long)key_start + tile_total <= p.capacity;
-    for_entries(entries, n,
+    for_entries<THREADS>(entries, n,
                 [&](const uint4& e)
                 {
                     const u64 key = ((u64)e.x << 32) | (u64)e.y;
@@ -617,7 +622,7 @@ __global__ __launch_bounds__(256) void tile_lists_kernel(const ForwardParams p)
     {
         __syncthreads();
         u64* dst = p.keys + key_start;
-        for (int i = threadIdx.x; i < tile_total; i += 256) dst[i] = s_keys[i];
+        for (int i = threadIdx.x; i < tile_total; i += THREADS) dst[i] = s_keys[i];
     }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
 }
@@ -968,7 +973,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         const long long words = 2ll * NB * kTilePixels;
         hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((words / 4 + 255) / 256, 4096)), dim3(256), 0, stream,
                            reinterpret_cast<uint4*>(p.counts), 0u, words / 4);
-        hipLaunchKernelGGL((tile_lists_kernel<false>), dim3(NB + max_slices), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((tile_lists_kernel<false, 256>), dim3(NB + max_slices), dim3(256), 0, stream, p);
     }
     {
         ProfScope ps(prof, "tile_scan", stream);
@@ -977,7 +982,12 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     }
     {
         ProfScope ps(prof, "tile_scatter", stream);
-        hipLaunchKernelGGL((tile_lists_kernel<true>), dim3(NB + max_slices), dim3(256), kStageKeys * sizeof(u64), stream, p);
+        // (64 KB of LDS with the static tables: above the default limit of a launch)
+        const hipError_t lds = hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_lists_kernel<true, kScatterThreads>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kStageKeys * sizeof(u64)));
+        if (lds != hipSuccess) return lds;
+        hipLaunchKernelGGL((tile_lists_kernel<true, kScatterThreads>), dim3(NB + max_slices), dim3(kScatterThreads), kStageKeys * sizeof(u64), stream,
+                           p);
     }
     {
         ProfScope ps(prof, "long_lists", stream);
