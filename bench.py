@@ -32,7 +32,7 @@ PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
     "project_bin": (135365, 473833),
     "bin_scatter": (48402, 203115),
     "tile_count": (51871, 34387),
-    "tile_scatter": (87336, 451243),
+    "tile_scatter": (83572, 464873),
     "fill_rank": (15, 187500),
     "sort_blend": (397626, 424924),
     "backward_pixels": (528446, 417602),
