@@ -120,6 +120,16 @@ def test_random_shapes_forward_backward(oracle, seed):
     _check_backward(oracle, sc, d, seed=seed)
 
 
+@pytest.mark.parametrize("w,h,L,n", [(4000, 40, 8, 20000), (37, 3000, 6, 20000), (1, 1, 1, 10), (2, 2, 2, 50), (33, 33, 6, 500)])
+def test_extreme_image_shapes(oracle, w, h, L, n):
+    """Very wide and very tall images (many tile columns / rows, coarse layers one pixel high) and images smaller than
+    one tile."""
+    sc = scenes.tiny(n=n, w=w, h=h, f=float(0.8 * max(w, h)), num_layers=L, list_depth=16, seed=w + h, radius=(0.002, 0.3))
+    d = abi.desc_for_scene(sc)
+    _check_forward(oracle, sc, d)
+    _check_backward(oracle, sc, d, seed=1)
+
+
 def test_transmittance_cutoff_matches(oracle):
     n = 12
     sc = scenes.tiny(n=n, w=16, h=16, f=30.0, num_layers=1, list_depth=16, seed=3, background=0.5)
