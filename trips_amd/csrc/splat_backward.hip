@@ -11,7 +11,8 @@
 //      from the per-point record exactly as the forward computed them; the "all later entries" sum of
 //      RenderBackward.cu:284-301 is a suffix sum across the row. Per entry it writes {dL/dalpha, T*alpha*dL/dimage}
 //      into the pixel's row of a [P,K] table. The forward's blend kernel has left one byte per retained entry, its
-//      rank in the pixel's list, in the point's 32-slot table (slot = layer * 4 + footprint corner).
+//      rank in the pixel's list, in the point's 32-slot table (slot = layer * 4 + footprint corner; two planes of 16
+//      slots per point, layers 0..3 and 4..7).
 //   2. points: one thread per point walks its slots, gathers those records (one aligned load each), sums the image-space gradient of all its entries and runs the projection chain ONCE
 //      (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then adds its gradients
 //      with plain read-modify-writes. Pose / intrinsics partials stay in double registers over a grid-stride
@@ -282,9 +283,9 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         {
             r0              = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
             rv              = prec[0];
-            const uint4* rk = reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 32);
-            rk0             = rk[0];
-            rk1             = rk[1];
+            rk0 = *reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 16);
+            // layers 4..7: a row of the second plane, defined only for the points that were written to those layers
+            if (max_layer > 4) rk1 = *reinterpret_cast<const uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)pid * 16);
         }
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;

@@ -180,6 +180,9 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 {
                     precv[0] = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
                     precv[1] = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
+                    // the few points that reach layer 4 and beyond clear their own row of the upper rank plane
+                    if (layer > 4)
+                        *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)pid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
                 }
             }
         }
@@ -852,7 +855,9 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
             p.lengths[pix]  = live ? len : 0;
         }
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
-        if (has && sub < ret) p.rank[((size_t)(unsigned)pid << 5) + slot] = (unsigned char)sub;
+        // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
+        if (has && sub < ret)
+            p.rank[(layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)(unsigned)pid << 4) + slot] = (unsigned char)sub;
         const int mine = has ? pid : -1;
         if (ROW == 8)
         {
@@ -932,11 +937,13 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header);
     if (train && p.num_points > 0)
     {
-        // the rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
-        // pixel's list): filled by sort_blend; cleared first thing, not in front of sort_blend, where the fill would
-        // push the keys that the list kernels have just written out of the last-level cache
+        // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
+        // pixel's list), filled by sort_blend: a plane of 16 bytes per point for layers 0..3 and a second one for
+        // layers 4..7. Only the first is cleared here (first thing, not in front of sort_blend, where the fill would
+        // push the keys that the list kernels have just written out of the last-level cache); the rows of the second
+        // are cleared by the projection kernel for the few points that reach those layers, and nobody else reads them.
         ProfScope ps(prof, "fill_rank", stream);
-        const long long quads = (long long)p.num_points * 2;  // 32 bytes per point
+        const long long quads = (long long)p.num_points;  // 16 bytes per point
         hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((quads + 255) / 256, 8192)), dim3(256), 0, stream,
                            reinterpret_cast<uint4*>(p.rank), 0xFFFFFFFFu, quads);
     }

@@ -214,7 +214,8 @@ struct SavedLayout
     size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded)
     size_t retained;  // int32 [Pi]
     size_t lengths;   // int32 [Pi]
-    size_t rank;      // uint8 [N, 32] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none
+    size_t rank;      // uint8 [2][N, 16] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none:
+                      // plane 0 layers 0..3, plane 1 layers 4..7 (rows defined only for points written to those layers)
     size_t bytes_per_view;
 };
 
@@ -319,7 +320,7 @@ struct BackwardParams
     const ViewHeader* header;
     const float* grad_image[TRIPS_MAX_LAYERS];
     float* entry_grad;    // [P, K, EF] {dL/dalpha, T alpha dL/dimage[0..C)}, EF = (1+C) rounded up to 4 (workspace)
-    const unsigned char* rank;  // [N, 32] (saved state) rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
+    const unsigned char* rank;  // [2][N, 16] (saved state) rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
     float* d_texture;
     float* d_confidence;
     float* d_background;
