@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void export_points_kernel(const float* __restr
     const int pid = blockIdx.x * 256 + threadIdx.x;
     if (pid >= n) return;
     const float* r  = rec + (size_t)pid * rec_floats;
-    const float4 tl = *reinterpret_cast<const float4*>(prec + (size_t)pid * kPointRecordFloats + 4);  // {tex, depth, max_layer, size_px}
+    const float4 tl = reinterpret_cast<const float4*>(prec)[pid];  // {softplus'(raw size), depth, max_layer, size_px}
     const bool ok   = tl.y > 0.f;
     if (ip)
     {

@@ -271,18 +271,28 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 
     for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
     {
-        const float4* prec = reinterpret_cast<const float4*>(p.prec + (size_t)pid * kPointRecordFloats);
-        const float4 tail  = prec[1];  // {texture index, depth, layers written, size_px}
-        const bool live = tail.y > 0.f;
+        const float4 tail = reinterpret_cast<const float4*>(p.prec)[pid];  // {softplus'(raw size), depth, layers written, size_px}
+        const bool live   = tail.y > 0.f;
         if (!live && !overwrite) continue;
-        const int tex       = __float_as_int(tail.x);
+        const int tex       = identity ? pid : p.index[pid];  // (a column outside the table: the point was culled)
         const int max_layer = live ? __float_as_int(tail.z) : 0;
         float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), rv = r0;  // ip.x ip.y size field conf; view xyz, softplus'(raw size)
         uint4 rk0 = make_uint4(~0u, ~0u, ~0u, ~0u), rk1 = rk0;
         if (live)
         {
             r0              = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
-            rv              = prec[0];
+            // the point in view space, exactly as the projection kernel computed it
+            float4 pos = p.position[pid];
+            if (p.displacement)
+            {
+                const float* dsp = p.displacement + (size_t)pid * 3;
+                pos.x += dsp[0];
+                pos.y += dsp[1];
+                pos.z += dsp[2];
+            }
+            float view[3];
+            transform_point(cam.V, pos.x, pos.y, pos.z, view);
+            rv = make_float4(view[0], view[1], view[2], tail.x);
             rk0 = *reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 16);
             // layers 4..7: a row of the second plane, defined only for the points that were written to those layers
             if (max_layer > 4) rk1 = *reinterpret_cast<const uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)pid * 16);

@@ -92,11 +92,10 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         bool skip   = false;
         const int tex = p.index[pid];
         constexpr int NREC = 1 + CPAD / 4;  // float4 per blend record
-        float4 recv[NREC], precv[2];
+        float4 recv[NREC];
 #pragma unroll
         for (int q = 0; q < NREC; ++q) recv[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-        precv[0] = make_float4(0.f, 0.f, 0.f, 0.f);
-        precv[1] = make_float4(__int_as_float(tex), -1.f, __int_as_float(0), 0.f);
+        float4 precv = make_float4(0.f, -1.f, __int_as_float(0), 0.f);
         not_identity |= (tex != pid);
         if ((unsigned)tex >= (unsigned)p.num_texels)
         {
@@ -178,24 +177,21 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 for (int q = 0; q < CPAD / 4; ++q) recv[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
                 if (TRAIN)
                 {
-                    precv[0] = make_float4(pr.vx, pr.vy, pr.vz, softplus_backward(p.point_size[pid]));
-                    precv[1] = make_float4(__int_as_float(tex), z, __int_as_float(layer), size_px);
+                    precv = make_float4(softplus_backward(p.point_size[pid]), z, __int_as_float(layer), size_px);
                     // the few points that reach layer 4 and beyond clear their own row of the upper rank plane
                     if (layer > 4)
                         *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)pid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
                 }
             }
         }
-        // The records of culled points are written too (zeros; tail {texture index, depth = -1, layers = 0}): whole
-        // lines leave the chip faster than lines with holes
+        // The records of culled points are written too (zeros; depth = -1, layers = 0): whole lines leave the chip
+        // faster than lines with holes
         float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)pid * p.rec_floats);
 #pragma unroll
         for (int q = 0; q < NREC; ++q) rec[q] = recv[q];
         if (TRAIN)
         {
-            float4* prec = reinterpret_cast<float4*>(p.prec + (size_t)pid * kPointRecordFloats);
-            prec[0]      = precv[0];
-            prec[1]      = precv[1];
+            reinterpret_cast<float4*>(p.prec)[pid] = precv;
         }
         p.ptk[pid] = ptk;
     }

@@ -92,10 +92,11 @@ namespace trips
 //              C = 4 (the reference reads a 5-float record, the confidence and C descriptor planes,
 //              src/lib/rendering/RenderForward.cu:875-899,952). Kept apart from the rest because a scattered gather
 //              costs the bytes of the whole aligned block it touches.
-//   prec[pid]  8 floats {view.x, view.y, view.z, softplus'(raw size), texture index, depth (-1 = culled), layers
-//              written, size_px}: read in point order by the point pass of the backward (training only).
+//   prec[pid]  4 floats {softplus'(raw size), depth (-1 = culled), layers written, size_px}: read in point order by
+//              the point pass of the backward (training only), which transforms the point into view space again
+//              rather than have the projection pass write those 12 bytes per point as well.
 __host__ __device__ inline int record_floats(int channels) { return 4 + ((channels + 3) & ~3); }
-constexpr int kPointRecordFloats = 8;
+constexpr int kPointRecordFloats = 4;
 
 // Pixels are binned into 32 x 32 tiles per layer. Internally a pixel is numbered tile-major:
 // (bin << 10) | (y & 31) << 5 | (x & 31), bin = bin_off[layer] + tile_y * tiles_x[layer] + tile_x, so that a
@@ -307,6 +308,9 @@ struct BackwardParams
     const double* pose;
     const float* intrinsics;
     const float* point_size;
+    const float4* position;     // as the forward saw them
+    const float* displacement;  // this view's [N,3] or nullptr
+    const int32_t* index;
     PyramidGeom geom;
     TripsView view;
     int32_t num_points, num_texels, num_layers, list_depth;

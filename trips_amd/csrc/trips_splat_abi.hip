@@ -447,6 +447,8 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
     if (!in || !saved || !grad_image || !grads) return fail(TRIPS_ERR_INVALID_ARG, "in / saved / grad_image / grads is NULL");
     if (!in->background || !in->poses_se3 || !in->intrinsics)
         return fail(TRIPS_ERR_INVALID_ARG, "background / poses_se3 / intrinsics is NULL");
+    if (d.num_points > 0 && (!in->position || !in->index))
+        return fail(TRIPS_ERR_INVALID_ARG, "position / index is NULL (the backward reads them again, unchanged since the forward)");
     if (!grads->d_texture || !grads->d_confidence || !grads->d_background)
         return fail(TRIPS_ERR_INVALID_ARG, "d_texture / d_confidence / d_background is required");
     for (int l = 0; l < d.num_layers; ++l)
@@ -472,6 +474,9 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.pose         = in->poses_se3 + 8 * (size_t)d.views[b].image_index;
         p.intrinsics   = in->intrinsics + 13 * (size_t)d.views[b].camera_index;
         p.point_size   = in->point_size;
+        p.position     = reinterpret_cast<const float4*>(in->position);
+        p.displacement = in->displacement ? in->displacement + (size_t)b * d.num_points * 3 : nullptr;
+        p.index        = in->index;
         p.geom         = g;
         p.view         = d.views[b];
         p.num_points   = d.num_points;
