@@ -29,14 +29,14 @@ DEFAULT_POINTS = 6_000_000
 # of the committed summary of those two runs and apply to the default --points only.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (137159, 476669),
+    "project_bin": (135221, 382703),
     "bin_scatter": (48402, 203115),
     "tile_count": (51871, 34387),
-    "tile_scatter": (83662, 466521),
+    "tile_scatter": (83710, 463290),
     "fill_rank": (13, 93750),
-    "sort_blend": (396898, 425090),
-    "backward_pixels": (528506, 417577),
-    "backward_points": (1065698, 234887),
+    "sort_blend": (396803, 424852),
+    "backward_pixels": (528132, 417618),
+    "backward_points": (1065514, 234887),
     "adam_fused": (582979, 792823),
 }
 

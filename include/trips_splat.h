@@ -148,6 +148,8 @@ int trips_splat_saved_size(const TripsSplatDesc* desc, size_t* bytes);
 int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* `in` must hold what the forward saw: besides background, poses and intrinsics the backward reads position, index,
+ * point_size and displacement again (the reference's backward likewise reads the points again, RenderBackward.cu:410,424). */
 int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const void* saved,
                          const float* const grad_image[TRIPS_MAX_LAYERS], const TripsSplatGrads* grads,
                          void* workspace, size_t workspace_bytes, void* stream);
