@@ -55,15 +55,20 @@ __global__ __launch_bounds__(256) void fill_words_kernel(uint4* __restrict__ p, 
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = make_uint4(v, v, v, v);
 }
 
-__global__ void clear_header_kernel(ViewHeader* h)
+// one launch for the counters of the view and, on the first view of a call, the status block of the whole call
+__global__ void clear_header_kernel(ViewHeader* h, ViewHeader* status)
 {
-    if (threadIdx.x == 0)
+    if (threadIdx.x < 2)
     {
-        h->n_valid   = 0;
-        h->n_entries = 0;
-        h->overflow  = 0;
-        h->retained = h->not_identity = h->bad_index = 0;
-        h->reserved[0] = h->reserved[1] = 0;
+        ViewHeader* t = threadIdx.x == 0 ? h : status;
+        if (t)
+        {
+            t->n_valid   = 0;
+            t->n_entries = 0;
+            t->overflow  = 0;
+            t->retained = t->not_identity = t->bad_index = 0;
+            t->reserved[0] = t->reserved[1] = 0;
+        }
     }
 }
 
@@ -929,8 +934,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
 {
     const int NB = p.geom.bin_off[p.num_layers];
 
-    if (first_view) hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.status);
-    hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header);
+    hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header, first_view ? p.status : (ViewHeader*)nullptr);
     if (train && p.num_points > 0)
     {
         // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
