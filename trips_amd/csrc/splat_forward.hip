@@ -365,10 +365,19 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
 // clusters) would keep a single workgroup busy for milliseconds; it is cut into slices of kSliceEntries entries,
 // each a workgroup of its own. slice_start[t] = number of slices of split tiles before tile t (ONE workgroup).
 // Also clears the per-tile key totals, which the slices of a split tile accumulate with atomics.
+// The workgroups after the first clear `clear_n` 16-byte words at `clear` (the per-pixel counters of the list kernels),
+// which saves a launch of its own.
 __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restrict__ bin_start, long long capacity, int NB,
                                                           int32_t* __restrict__ slice_start, int32_t* __restrict__ bin_total,
-                                                          int32_t* __restrict__ long_count)
+                                                          int32_t* __restrict__ long_count, uint4* __restrict__ clear,
+                                                          long long clear_n)
 {
+    if (blockIdx.x > 0)
+    {
+        for (long long i = (long long)(blockIdx.x - 1) * 1024 + threadIdx.x; i < clear_n; i += (long long)(gridDim.x - 1) * 1024)
+            clear[i] = make_uint4(0u, 0u, 0u, 0u);
+        return;
+    }
     if (threadIdx.x == 0) *long_count = 0;
     __shared__ int s_wave[16];
     __shared__ int s_carry;
@@ -408,12 +417,6 @@ __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restr
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// One workgroup per tile (blocks [0, NB)) plus one per slice of a split tile (blocks from NB on; those past the
-// number of slices the plan found return at once). Pass `SCATTER == false`: count the list length of the tile's
-// 1024 pixels in LDS and write them (plus the tile total). Pass `SCATTER == true` (after the scan of the tile
-// totals): exclusive scan of the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 |
-// point id) into their lists. A slice adds its counts to the tile's with atomics; when it places its keys it first
-// counts its own entries per pixel again and claims that many slots of each pixel's list with one atomic.
 // Calls f(local pixel index) for each of the entry's 2 x 2 pixels that lie in tile (tx, ty).
 template <typename F>
 __device__ __forceinline__ void for_corners_in_tile(const uint4& e, int tx, int ty, F&& f)
@@ -443,6 +446,12 @@ __device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, i
     }
 }
 
+// One workgroup per tile (blocks [0, NB)) plus one per slice of a split tile (blocks from NB on; those past the
+// number of slices the plan found return at once). Pass `SCATTER == false`: count the list length of the tile's
+// 1024 pixels in LDS and write them (plus the tile total). Pass `SCATTER == true` (after the scan of the tile
+// totals): exclusive scan of the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 |
+// point id) into their lists. A slice adds its counts to the tile's with atomics; when it places its keys it first
+// counts its own entries per pixel again and claims that many slots of each pixel's list with one atomic.
 // (THREADS: 256 for the counting pass, whose idle workgroups for unused slices are cheaper that way; 1024 for the
 // placement pass, where two workgroups per CU with their 64 KB of LDS then make 32 wavefronts instead of 8)
 constexpr int kScatterThreads = 1024;
@@ -975,11 +984,10 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     const int max_slices = (int)std::min<long long>(2 * (p.capacity / kSliceEntries) + 1, 1 << 20);
     {
         ProfScope ps(prof, "tile_count", stream);
-        hipLaunchKernelGGL(slice_plan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_start, p.capacity, NB, p.slice_start, p.bin_total, p.long_count);
-        // counts and run are neighbours in the workspace: one fill clears both
-        const long long words = 2ll * NB * kTilePixels;
-        hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((words / 4 + 255) / 256, 4096)), dim3(256), 0, stream,
-                           reinterpret_cast<uint4*>(p.counts), 0u, words / 4);
+        // counts and run are neighbours in the workspace: cleared together, by the workgroups behind the planning one
+        const long long quads = 2ll * NB * kTilePixels / 4;
+        hipLaunchKernelGGL(slice_plan_kernel, dim3(1 + (unsigned)std::min<long long>((quads + 1023) / 1024, 1024)), dim3(1024), 0, stream,
+                           p.bin_start, p.capacity, NB, p.slice_start, p.bin_total, p.long_count, reinterpret_cast<uint4*>(p.counts), quads);
         hipLaunchKernelGGL((tile_lists_kernel<false, 256>), dim3(NB + max_slices), dim3(256), 0, stream, p);
     }
     {
