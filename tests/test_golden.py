@@ -39,7 +39,7 @@ def test_oracle_reproduces_golden(oracle):
 @pytest.mark.gpu
 def test_hip_path_matches_golden():
     import torch
-    from tests.gpu_util import GpuRun, rel_err
+    from tests.gpu_util import GpuRun, assert_grads_close
     from trips_amd.renderer import get_context
     z = np.load(PATH)
     sc = _scene(z)
@@ -59,8 +59,7 @@ def test_hip_path_matches_golden():
                 np.testing.assert_array_equal(ip, z["ip"][b])
                 np.testing.assert_array_equal(max_layer, z["max_layer"][b])
             g = run.backward([z[f"grad_image_{l}"] for l in range(3)])
-            for k, v in g.items():
-                assert rel_err(v, z[k]) < 1e-4, k
+            assert_grads_close(g, {k: z[k] for k in g})
             # one Adam step on the positions with the golden gradient
             ctx = get_context(0)
             n = sc.position.size

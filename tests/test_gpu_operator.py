@@ -18,7 +18,7 @@ def _info(sc, ns, train=True, **params):
 
 
 def test_blend_point_cloud_forward_backward_matches_oracle(oracle):
-    from tests.gpu_util import rel_err
+    from tests.gpu_util import assert_grad_close
     from trips_amd.renderer import BlendPointCloud, NeuralScene
     sc = scenes.tiny(n=5000, w=80, h=60, f=70.0, num_layers=4, list_depth=16, seed=41, views=2, radius=(0.004, 0.4))
     ns = NeuralScene.from_arrays(sc, requires_grad=True)
@@ -34,13 +34,13 @@ def test_blend_point_cloud_forward_backward_matches_oracle(oracle):
     loss = sum((o * torch.as_tensor(g).cuda()).sum() for o, g in zip(outs, grads))
     loss.backward()
     g_ref = oracle.backward(sc, d, ref, grads)
-    pairs = [(ns.texture.texture.grad, g_ref["d_texture"]), (ns.texture.background_color.grad, g_ref["d_background"]),
-             (ns.point_cloud_cuda.t_position.grad, g_ref["d_position"]),
-             (ns.poses.tangent_poses.grad, g_ref["d_pose"]), (ns.intrinsics.intrinsics.grad, g_ref["d_intrinsics"]),
-             (ns.texture.confidence_value_of_point.grad.reshape(-1), g_ref["d_confidence"]),
-             (ns.point_cloud_cuda.t_point_size.grad.reshape(-1), g_ref["d_point_size"])]
-    for got, want in pairs:
-        assert rel_err(got.cpu().numpy(), want) < 1e-4
+    pairs = [("d_texture", ns.texture.texture.grad), ("d_background", ns.texture.background_color.grad),
+             ("d_position", ns.point_cloud_cuda.t_position.grad), ("d_pose", ns.poses.tangent_poses.grad),
+             ("d_intrinsics", ns.intrinsics.intrinsics.grad),
+             ("d_confidence", ns.texture.confidence_value_of_point.grad.reshape(-1)),
+             ("d_point_size", ns.point_cloud_cuda.t_point_size.grad.reshape(-1))]
+    for key, got in pairs:
+        assert_grad_close(key, got.cpu().numpy(), g_ref[key])
     assert ns.texture.confidence_value_of_point.grad.shape == (1, 5000)
     assert ns.point_cloud_cuda.t_point_size.grad.shape == (5000, 1)
     assert ns.poses.tangent_poses.grad.dtype == torch.float64
@@ -61,7 +61,7 @@ def test_eval_mode_returns_permuted_views_and_no_graph(oracle):
 
 
 def test_only_requested_gradients_are_produced(oracle):
-    from tests.gpu_util import rel_err
+    from tests.gpu_util import assert_grad_close
     from trips_amd.renderer import BlendPointCloud, NeuralScene
     sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=43)
     ns = NeuralScene.from_arrays(sc)
@@ -76,8 +76,8 @@ def test_only_requested_gradients_are_produced(oracle):
     ones = [np.ones(o.shape, np.float32) for o in outs]
     g_ref = oracle.backward(sc, d, ref, ones, want_position=False, want_point_size=False, want_pose=False,
                             want_intrinsics=False)
-    assert rel_err(ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
-    assert rel_err(ns.texture.confidence_value_of_point.grad.cpu().numpy().reshape(-1), g_ref["d_confidence"]) < 1e-4
+    assert_grad_close("d_texture", ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"])
+    assert_grad_close("d_confidence", ns.texture.confidence_value_of_point.grad.cpu().numpy().reshape(-1), g_ref["d_confidence"])
 
 
 def test_dropout_is_drawn_per_forward_in_train_mode():
@@ -124,15 +124,15 @@ def test_unused_layers_and_extra_outputs(oracle):
     ref = oracle.forward(sc, d)
     grads = [g0.cpu().numpy(), g1.cpu().numpy()] + [np.zeros_like(ref["images"][l]) for l in (2, 3)]
     g_ref = oracle.backward(sc, d, ref, grads)
-    from tests.gpu_util import rel_err
-    assert rel_err(ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
-    assert rel_err(ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"]) < 1e-4
+    from tests.gpu_util import assert_grad_close
+    assert_grad_close("d_texture", ns.texture.texture.grad.cpu().numpy(), g_ref["d_texture"])
+    assert_grad_close("d_position", ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"])
 
 
 def test_dynamic_refinement_displaces_points_per_view(oracle):
     """A [B,N,3] dynamic_refinement_t moves the points of view b; the [1] dummy does nothing; no gradient comes back
     for it (the reference never allocates one, PointRenderer.cu:243-252)."""
-    from tests.gpu_util import rel_err
+    from tests.gpu_util import assert_grad_close
     from trips_amd.renderer import BlendPointCloud, NeuralScene
     sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=43, views=2)
     sc.displacement = np.random.default_rng(6).normal(0, 0.05, (2, 3000, 3)).astype(np.float32)
@@ -147,8 +147,8 @@ def test_dynamic_refinement_displaces_points_per_view(oracle):
     grads = [rng.normal(0, 1, o.shape).astype(np.float32) for o in outs]
     sum((o * torch.as_tensor(g).cuda()).sum() for o, g in zip(outs, grads)).backward()
     g_ref = oracle.backward(sc, d, ref, grads)
-    assert rel_err(ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"]) < 1e-4
-    assert rel_err(ns.poses.tangent_poses.grad.cpu().numpy(), g_ref["d_pose"]) < 1e-4
+    assert_grad_close("d_position", ns.point_cloud_cuda.t_position.grad.cpu().numpy(), g_ref["d_position"])
+    assert_grad_close("d_pose", ns.poses.tangent_poses.grad.cpu().numpy(), g_ref["d_pose"])
     assert ns.dynamic_refinement_t.grad is None
     ns.dynamic_refinement_t = torch.zeros((2, 5, 3), device="cuda")
     with pytest.raises(ValueError):
@@ -216,3 +216,24 @@ def test_step_replays_from_a_hip_graph(oracle):
         assert torch.allclose(graphed["grads"]["d_pose"], eager["grads"]["d_pose"], rtol=1e-9, atol=1e-12)
         (eager["images"][0].sum() + graphed["images"][0].sum()).item()  # eager work and a synchronisation in between
         step(eager)
+
+
+def test_normalize_grads_changes_nothing_on_this_path():
+    """RenderParams.normalize_grads divides the point gradients by per-point counts (PointRenderer.cu:1193-1230,
+    1348-1411), but the backward of this path never increments those counts (RenderBackward.cu has no count
+    atomics), so `c > 0` at PointRenderer.cu:1202,1223 is never true and the flag leaves the gradients as they are."""
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=45)
+    rng = np.random.default_rng(2)
+    grads = None
+    results = []
+    for flag in (False, True):
+        ns = NeuralScene.from_arrays(sc, requires_grad=True)
+        outs = BlendPointCloud(_info(sc, ns, normalize_grads=flag))
+        if grads is None:
+            grads = [torch.as_tensor(rng.normal(0, 1, o.shape).astype(np.float32)).cuda() for o in outs]
+        sum((o * g).sum() for o, g in zip(outs, grads)).backward()
+        results.append([t.grad.clone() for t in (ns.texture.texture, ns.texture.confidence_value_of_point,
+                                                  ns.point_cloud_cuda.t_position, ns.point_cloud_cuda.t_point_size)])
+    for a, b in zip(*results):
+        assert float(a.abs().max()) > 0 and torch.equal(a, b)

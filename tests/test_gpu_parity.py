@@ -1,7 +1,9 @@
 """Parity of the HIP path (called through the C ABI) with the CPU oracle on the same seeded inputs.
 
-Bars: per-point records and per-pixel index lists bit-exact; forward images within 1e-5 relative;
-gradients within 1e-4 of the largest gradient magnitude (float atomics sum in a different order)."""
+Bars: per-point records and per-pixel index lists bit-exact; forward images within 1e-5 relative; per-point
+gradients within 1e-4 relative per element (plus a floor of 3e-7 of the tensor's largest magnitude for elements that
+are differences of larger terms); the block sums (pose, intrinsics, background) within 1e-4 of their largest
+magnitude (tests/gpu_util.py)."""
 import numpy as np
 import pytest
 
@@ -10,7 +12,6 @@ from trips_amd import abi, scenes
 pytestmark = pytest.mark.gpu
 
 IMG_RTOL = 1e-5
-GRAD_RTOL = 1e-4
 
 
 def _check_forward(oracle, sc, desc, dropout=None, views=None):
@@ -142,7 +143,7 @@ def test_transmittance_cutoff_matches(oracle):
 
 
 def _check_backward(oracle, sc, desc, seed=0, **want):
-    from tests.gpu_util import GpuRun, rel_err
+    from tests.gpu_util import GpuRun, assert_grads_close
     ref = oracle.forward(sc, desc)
     rng = np.random.default_rng(seed)
     shape = (lambda w, h: (desc.num_views, desc.num_channels, h, w)) if desc.layout == abi.TRIPS_LAYOUT_CHW else \
@@ -152,14 +153,8 @@ def _check_backward(oracle, sc, desc, seed=0, **want):
     run = GpuRun(sc, desc)
     run.forward()
     g = run.backward(grads, **want)
-    errs = {}
-    for k, v in g_ref.items():
-        if v is None:
-            assert g[k] is None
-            continue
-        errs[k] = rel_err(g[k], v)
-        assert errs[k] < GRAD_RTOL, f"{k}: {errs[k]:.3e}"
-    return errs, g, g_ref
+    assert_grads_close(g, g_ref)
+    return None, g, g_ref
 
 
 @pytest.mark.parametrize("L,K,bg", [(1, 16, 1), (3, 8, 0), (4, 16, 1), (8, 16, 0)])
@@ -322,9 +317,11 @@ def test_config4_contention_full(oracle):
 
 def test_point_order_does_not_matter_at_full_size():
     """Size-independent property at the benchmark's size: shuffling the point order permutes the per-point
-    gradients and leaves the images unchanged (depth ties aside, which break by point id)."""
+    gradients and leaves the images unchanged, except where two entries of a pixel list have the same depth: the
+    tie breaks by point id, so a shuffle may swap them. The run counts those pixels itself (adjacent equal depths
+    among the sorted entries of a list) and allows only that many pixels, and that many times K points, to differ."""
     import dataclasses
-    from tests.gpu_util import GpuRun
+    from tests.gpu_util import GRAD_FLOOR, GRAD_RTOL, GpuRun, rel_err
     sc = scenes.config3()
     rng = np.random.Generator(np.random.Philox(99))
     perm = rng.permutation(sc.num_points)
@@ -338,27 +335,35 @@ def test_point_order_does_not_matter_at_full_size():
     ia = a.forward()
     ga = a.backward(gi)
     ca = a.ctx.counters(d, a.saved, 0)
+    lists, retained, _ = a.lists(0)
+    _, depth, _, _ = a.points(0)
     del a
+    # pixels with a depth tie among their sorted entries, and the points on such pixels
+    K = lists.shape[1]
+    dl = np.where(lists >= 0, depth[np.clip(lists, 0, None)], np.inf)
+    tied = ((dl[:, 1:] == dl[:, :-1]) & np.isfinite(dl[:, 1:])).any(axis=1)
+    n_tied = int(tied.sum())
+    assert n_tied < 1000  # config 3 has 173 of them among 2.76 M pixels
     b = GpuRun(sc2, d)
     ib = b.forward()
     gb = b.backward(gi)
     cb = b.ctx.counters(d, b.saved, 0)
     assert ca == cb
+    differing_pixels = 0
     for x, y in zip(ia, ib):
-        # pixels whose two front-most entries tie in depth may order differently
-        assert (np.abs(x - y) > 1e-5 * (1 + np.abs(y))).mean() < 1e-4
+        differing_pixels += int((np.abs(x - y) > 1e-5 * np.abs(y) + 1e-6).any(axis=1).sum())
+    assert differing_pixels <= n_tied, (differing_pixels, n_tied)
 
-    def off(got, want):
-        # fraction of elements further apart than the gradient bar; a depth tie reorders two entries of a pixel
-        # and moves the gradients of those two points
+    def differing_points(got, want, axis):
         got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
-        return float((np.abs(got - want) > GRAD_RTOL * np.abs(want).max()).mean())
+        bad = np.abs(got - want) > GRAD_RTOL * np.abs(want) + GRAD_FLOOR * np.abs(want).max()
+        return int(bad.any(axis=axis).sum()) if bad.ndim > 1 else int(bad.sum())
 
-    assert off(gb["d_position"], ga["d_position"][perm]) < 1e-4
-    assert off(gb["d_point_size"], ga["d_point_size"][perm]) < 1e-4
-    assert off(gb["d_confidence"], ga["d_confidence"][perm]) < 1e-4
-    assert off(gb["d_texture"], ga["d_texture"][:, perm]) < 1e-4
-    from tests.gpu_util import rel_err
+    allowed = n_tied * K  # every entry of a tied pixel's list may see another transmittance
+    assert differing_points(gb["d_position"], ga["d_position"][perm], 1) <= allowed
+    assert differing_points(gb["d_point_size"], ga["d_point_size"][perm], None) <= allowed
+    assert differing_points(gb["d_confidence"], ga["d_confidence"][perm], None) <= allowed
+    assert differing_points(gb["d_texture"], ga["d_texture"][:, perm], 0) <= allowed
     assert rel_err(gb["d_pose"], ga["d_pose"]) < 1e-3
     assert rel_err(gb["d_background"], ga["d_background"]) < 1e-3
 

@@ -38,7 +38,7 @@ def _session(sc, requires_grad=True):
 
 @pytest.mark.gpu
 def test_cpp_blend_point_cloud_forward_backward(oracle):
-    from tests.gpu_util import rel_err
+    from tests.gpu_util import assert_grad_close
     sc = scenes.tiny(n=5000, w=80, h=60, f=70.0, num_layers=4, list_depth=16, seed=51, views=2, radius=(0.004, 0.4))
     s, t = _session(sc)
     views = [[v["w"], v["h"], v["image_index"], v["camera_index"]] for v in sc.views]
@@ -52,12 +52,12 @@ def test_cpp_blend_point_cloud_forward_backward(oracle):
     grads = [rng.normal(0, 1, o.shape).astype(np.float32) for o in outs]
     sum((o * torch.as_tensor(g).cuda()).sum() for o, g in zip(outs, grads)).backward()
     g_ref = oracle.backward(sc, d, ref, grads)
-    pairs = [(t["texture"].grad, g_ref["d_texture"]), (t["background"].grad, g_ref["d_background"]),
-             (t["position"].grad, g_ref["d_position"]), (t["tangent_poses"].grad, g_ref["d_pose"]),
-             (t["intrinsics"].grad, g_ref["d_intrinsics"]), (t["confidence"].grad.reshape(-1), g_ref["d_confidence"]),
-             (t["point_size"].grad.reshape(-1), g_ref["d_point_size"])]
-    for got, want in pairs:
-        assert rel_err(got.cpu().numpy(), want) < 1e-4
+    pairs = [("d_texture", t["texture"].grad), ("d_background", t["background"].grad),
+             ("d_position", t["position"].grad), ("d_pose", t["tangent_poses"].grad),
+             ("d_intrinsics", t["intrinsics"].grad), ("d_confidence", t["confidence"].grad.reshape(-1)),
+             ("d_point_size", t["point_size"].grad.reshape(-1))]
+    for key, got in pairs:
+        assert_grad_close(key, got.cpu().numpy(), g_ref[key])
 
 
 @pytest.mark.gpu
@@ -148,7 +148,7 @@ def test_cpp_unet_forward_backward_matches_python_mirror():
 
 @pytest.mark.gpu
 def test_cpp_unused_layers_and_extra_outputs(oracle):
-    from tests.gpu_util import rel_err
+    from tests.gpu_util import assert_grad_close
     sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=4, list_depth=16, seed=9)
     s, t = _session(sc)
     views = [[v["w"], v["h"], v["image_index"], v["camera_index"]] for v in sc.views]
@@ -160,8 +160,8 @@ def test_cpp_unused_layers_and_extra_outputs(oracle):
     d = abi.desc_for_scene(sc)
     ref = oracle.forward(sc, d)
     g_ref = oracle.backward(sc, d, ref, [g0] + [np.zeros_like(ref["images"][l]) for l in (1, 2, 3)])
-    assert rel_err(t["texture"].grad.cpu().numpy(), g_ref["d_texture"]) < 1e-4
-    assert rel_err(t["position"].grad.cpu().numpy(), g_ref["d_position"]) < 1e-4
+    assert_grad_close("d_texture", t["texture"].grad.cpu().numpy(), g_ref["d_texture"])
+    assert_grad_close("d_position", t["position"].grad.cpu().numpy(), g_ref["d_position"])
 
 
 @pytest.mark.gpu
