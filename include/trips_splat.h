@@ -154,6 +154,21 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
                          const float* const grad_image[TRIPS_MAX_LAYERS], const TripsSplatGrads* grads,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* The forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc) and have no workspace to hand over. It has no counterpart in the reference, whose
+ * forward allocates through libtorch's caching allocator (PointRenderer.cu:276-528). Same arguments, results and
+ * errors as trips_splat_forward, except that the workspace is a static array inside the library:
+ * TRIPS_STATIC_WORKSPACE_BYTES per GPU, present from library load until the process ends. A scene whose
+ * trips_splat_workspace_size exceeds that is rejected with TRIPS_ERR_WORKSPACE_SMALL (nothing is launched);
+ * desc->max_list_entries lowers the need. The call allocates nothing on the host or the device and creates no
+ * events (the per-kernel timer of trips_profile_enable does not cover it). All calls on one GPU share the one array:
+ * calls that overlap on the same GPU (two streams, two threads, two contexts) race; calls on one stream are ordered
+ * and each call clears the counters it relies on. trips_splat_check(ctx, NULL, stream) reports on the last such call.
+ * The caller still passes the images and, with desc->train, the saved state. */
+#define TRIPS_STATIC_WORKSPACE_BYTES (64u << 20)
+int trips_splat_forward_static(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
+                               void* stream);
+
 /* Synchronises `stream` and reports what the last forward that used `workspace` found on the device: a list
  * overflow (TRIPS_ERR_LIST_OVERFLOW, only possible when desc->max_list_entries was set below the worst case) or
  * values of `index` outside [0, num_texels) (TRIPS_ERR_INVALID_ARG; such points are left out of the image, the

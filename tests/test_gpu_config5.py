@@ -163,7 +163,7 @@ def test_config5_full_size_steps():
         rgb = net.forward(list(outs))
         loss = (rgb - target).abs().mean()
         loss.backward()
-        return rgb.detach(), float(loss)
+        return rgb.detach(), float(loss.detach())
 
     rgb_a, loss_a = step()
     grads_a = {k: q.grad.clone() for k, q in pp.items()}

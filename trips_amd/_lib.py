@@ -13,7 +13,8 @@ LIB_PATH = os.path.join(HERE, "libtrips_splat.so")
 # every symbol include/trips_splat.h declares
 SYMBOLS = [
     "trips_version", "trips_last_error_string", "trips_ctx_create", "trips_ctx_destroy", "trips_splat_layer_sizes",
-    "trips_splat_workspace_size", "trips_splat_saved_size", "trips_splat_forward", "trips_splat_backward",
+    "trips_splat_workspace_size", "trips_splat_saved_size", "trips_splat_forward", "trips_splat_forward_static",
+    "trips_splat_backward",
     "trips_splat_check", "trips_splat_counters", "trips_splat_export_lists", "trips_splat_export_points",
     "trips_adam_step_fused", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
 ]
@@ -50,6 +51,8 @@ def load():
     lib.trips_splat_saved_size.argtypes = [C.POINTER(abi.TripsSplatDesc), C.POINTER(C.c_size_t)]
     lib.trips_splat_forward.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), C.POINTER(abi.TripsSplatIn),
                                         C.POINTER(abi.TripsSplatOut), vp, C.c_size_t, vp]
+    lib.trips_splat_forward_static.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), C.POINTER(abi.TripsSplatIn),
+                                               C.POINTER(abi.TripsSplatOut), vp]
     lib.trips_splat_backward.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), C.POINTER(abi.TripsSplatIn), vp,
                                          C.POINTER(vp), C.POINTER(abi.TripsSplatGrads), vp, C.c_size_t, vp]
     lib.trips_splat_check.argtypes = [vp, vp, vp]

@@ -10,7 +10,7 @@ LIB = os.path.join(HERE, "libtrips_splat.so")
 SOURCES = ["trips_splat_abi.hip", "splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "unet_forward.hip",
            "unet_backward.hip"]
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # packed FP32 instructions are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
@@ -24,11 +24,34 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose=False):
-    cmd = [hipcc()] + FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
+HEADERS = ["splat_internal.h", "trips_math.h", "row16.h", "unet_common.h", os.path.join("..", "..", "include", "trips_splat.h"),
+           os.path.join("..", "..", "include", "trips_unet.h")]
+
+
+def build(verbose=False, incremental=False):
+    """One hipcc process per translation unit, side by side, then one link. `incremental` skips units whose object
+    is newer than the unit and every header (a convenience while editing; the default compiles everything)."""
+    objdir = os.path.join(CSRC, "_obj")
+    os.makedirs(objdir, exist_ok=True)
+    newest_header = max(os.path.getmtime(os.path.join(CSRC, h)) for h in HEADERS)
+    procs, objs = [], []
+    for src in SOURCES:
+        path = os.path.join(CSRC, src)
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(path), newest_header):
+            continue
+        cmd = [hipcc()] + FLAGS + ["-c", path, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((cmd, subprocess.Popen(cmd)))
+    for cmd, pr in procs:
+        if pr.wait() != 0:
+            raise subprocess.CalledProcessError(pr.returncode, cmd)
+    link = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]
     if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+        print(" ".join(link), flush=True)
+    subprocess.check_call(link)
     return LIB
 
 
@@ -71,7 +94,7 @@ def build_torch_shim(verbose=False):
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, incremental="--incremental" in sys.argv)
     print(LIB)
     if "--shim" in sys.argv:
         print(build_torch_shim(verbose=True))

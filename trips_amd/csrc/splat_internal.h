@@ -82,6 +82,9 @@ struct TripsCtx
 {
     int device;
     trips::Profiler prof;
+    // this device's copy of the library's static scratch array (trips_splat_forward_static), resolved when the
+    // context is created
+    void* static_scratch = nullptr;
 };
 
 namespace trips

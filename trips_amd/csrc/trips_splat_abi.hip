@@ -30,6 +30,12 @@ using namespace trips;
 namespace
 {
 thread_local char g_error[512] = "";
+
+// Workspace of trips_splat_forward_static, the entry point for callers that cannot allocate: one array per GPU the
+// library runs on, held until the process ends. Host code must not use this name as an address (it is a host-side
+// stand-in); every use goes through the pointer hipGetSymbolAddress returns for the current device, kept in the
+// context.
+static __device__ __align__(256) unsigned char scratch[TRIPS_STATIC_WORKSPACE_BYTES];
 }
 
 namespace trips
@@ -282,9 +288,20 @@ int trips_ctx_create(TripsCtx** out_ctx, int device)
     hipError_t e = hipGetDeviceCount(&count);
     if (e != hipSuccess) return hip_fail(e, "hipGetDeviceCount");
     if (device < 0 || device >= count) return fail(TRIPS_ERR_INVALID_ARG, "device %d of %d", device, count);
-    TripsCtx* c = new TripsCtx;
-    c->device   = device;
-    *out_ctx    = c;
+    // address of this device's copy of the static scratch array, with that device current
+    int previous = 0;
+    e            = hipGetDevice(&previous);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
+    void* ptr = nullptr;
+    e         = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    (void)hipSetDevice(previous);
+    if (e != hipSuccess || !ptr) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    TripsCtx* c       = new TripsCtx;
+    c->device         = device;
+    c->static_scratch = ptr;
+    *out_ctx          = c;
     return TRIPS_OK;
 }
 
@@ -332,8 +349,12 @@ int trips_splat_saved_size(const TripsSplatDesc* desc, size_t* bytes)
     return TRIPS_OK;
 }
 
-int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
-                        void* workspace, size_t workspace_bytes, void* stream_)
+}  // extern "C"
+
+namespace
+{
+int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
+                 void* workspace, size_t workspace_bytes, void* stream_, bool use_profiler)
 {
     if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
     if (int e = check_desc(desc)) return e;
@@ -430,10 +451,35 @@ int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSp
         }
         p.status = reinterpret_cast<ViewHeader*>(ws);
         for (int l = 0; l < d.num_layers; ++l) p.image[l] = out->image[l];
-        hipError_t e = launch_forward_view(p, d.num_channels, train, b == 0, stream, ctx->prof.enabled ? &ctx->prof : nullptr);
+        hipError_t e = launch_forward_view(p, d.num_channels, train, b == 0, stream,
+                                           (use_profiler && ctx->prof.enabled) ? &ctx->prof : nullptr);
         if (e != hipSuccess) return hip_fail(e, "forward launch");
     }
     return TRIPS_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int trips_splat_forward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
+                        void* workspace, size_t workspace_bytes, void* stream)
+{
+    return forward_impl(ctx, desc, in, out, workspace, workspace_bytes, stream, true);
+}
+
+int trips_splat_forward_static(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
+                               void* stream)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    size_t need = 0;
+    if (int e = trips_splat_workspace_size(desc, &need)) return e;
+    if (need > (size_t)TRIPS_STATIC_WORKSPACE_BYTES)
+        return fail(TRIPS_ERR_WORKSPACE_SMALL,
+                    "this scene needs %zu bytes of workspace, the static one holds %zu: use trips_splat_forward with a "
+                    "caller-owned workspace, or lower max_list_entries",
+                    need, (size_t)TRIPS_STATIC_WORKSPACE_BYTES);
+    // no event creation either: the per-kernel timer is left out of this entry point
+    return forward_impl(ctx, desc, in, out, ctx->static_scratch, (size_t)TRIPS_STATIC_WORKSPACE_BYTES, stream, false);
 }
 
 int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const void* saved,
@@ -512,8 +558,9 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
 
 int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
 {
-    const void* header_owner = workspace;
-    if (!ctx || !header_owner) return fail(TRIPS_ERR_INVALID_ARG, "ctx / workspace is NULL");
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    const void* header_owner = workspace ? workspace : ctx->static_scratch;  // NULL: the last trips_splat_forward_static
+    if (!header_owner) return fail(TRIPS_ERR_INVALID_ARG, "workspace is NULL");
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     ViewHeader h;
     hipError_t e = hipMemcpyAsync(&h, header_owner, sizeof(h), hipMemcpyDeviceToHost, stream);

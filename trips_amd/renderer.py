@@ -98,6 +98,17 @@ class SplatContext:
         _lib.check(self.lib.trips_splat_forward(self.ctx, C.byref(desc), C.byref(tin), C.byref(out), _ptr(workspace),
                                                 workspace.numel(), _stream_ptr(self.device)))
 
+    def forward_static(self, desc, tin, images, saved):
+        """The forward on the library's own static workspace (abi.TRIPS_STATIC_WORKSPACE_BYTES per GPU): allocates
+        nothing; raises TripsError(TRIPS_ERR_WORKSPACE_SMALL) for scenes that need more. Calls on one GPU must not
+        overlap."""
+        out = abi.TripsSplatOut()
+        for l, im in enumerate(images):
+            out.image[l] = im.data_ptr()
+        out.saved = _ptr(saved)
+        _lib.check(self.lib.trips_splat_forward_static(self.ctx, C.byref(desc), C.byref(tin), C.byref(out),
+                                                       _stream_ptr(self.device)))
+
     def backward(self, desc, tin, saved, grad_images, grads, workspace=None, overwrite_point_grads=False):
         """Adds into `grads` (zeroed by the caller); with overwrite_point_grads the four per-point outputs
         (d_texture, d_confidence, d_position, d_point_size) are written instead and may be uninitialised."""
@@ -115,6 +126,7 @@ class SplatContext:
                                                  _stream_ptr(self.device)))
 
     def check(self, workspace):
+        """workspace None: the library's static workspace (after forward_static)."""
         _lib.check(self.lib.trips_splat_check(self.ctx, _ptr(workspace), _stream_ptr(self.device)))
 
     def counters(self, desc, saved, view=0):
