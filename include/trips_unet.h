@@ -36,7 +36,7 @@ extern "C" {
 typedef struct TripsUnetDesc {
     int32_t abi_version;          /* TRIPS_ABI_VERSION */
     int32_t num_levels;           /* L, 1..8: in[0..L-1] are consumed (MultiScaleUnet2dParams::num_layers) */
-    int32_t num_input_channels;   /* C, 1..8 (4 in every shipped config) */
+    int32_t num_input_channels;   /* C, 1..4 (4 in every shipped config) */
     int32_t num_output_channels;  /* 1..4 (3) */
     int32_t batch;                /* images per call */
     int32_t filters[TRIPS_UNET_MAX_LEVELS];  /* F[0..L-1] (filters_network); conv outputs must be >= 1 and <= 64 */

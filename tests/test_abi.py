@@ -183,7 +183,10 @@ def test_too_many_points_for_32_bit_offsets():
     d.num_layers = 8
     b = C.c_size_t(0)
     assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_UNSUPPORTED
+    # a granted capacity does not shorten the 32-bit prefix sums over the entries that could exist: still refused
     d.max_list_entries = 1_000_000_000
+    assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_UNSUPPORTED
+    d.num_points = 60_000_000  # 4*N*L = 1.92e9 fits
     assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == 0
 
 

@@ -237,3 +237,16 @@ def test_normalize_grads_changes_nothing_on_this_path():
                                                   ns.point_cloud_cuda.t_position, ns.point_cloud_cuda.t_point_size)])
     for a, b in zip(*results):
         assert float(a.abs().max()) > 0 and torch.equal(a, b)
+
+
+def test_backward_refuses_inputs_modified_in_place_after_the_forward():
+    """The backward reads position, size, index, poses and intrinsics again; an optimiser step between forward and
+    backward would silently give the gradients of another scene."""
+    from trips_amd.renderer import BlendPointCloud, NeuralScene
+    sc = scenes.tiny(n=2000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=46)
+    ns = NeuralScene.from_arrays(sc, requires_grad=True)
+    outs = BlendPointCloud(_info(sc, ns))
+    with torch.no_grad():
+        ns.point_cloud_cuda.t_position.add_(0.0)
+    with pytest.raises(RuntimeError, match="modified in place"):
+        sum(o.sum() for o in outs).backward()

@@ -176,3 +176,15 @@ def test_cpp_dynamic_refinement(oracle):
     ref = oracle.forward(sc, abi.desc_for_scene(sc))
     for a, b in zip(outs, ref["images"]):
         np.testing.assert_allclose(a.cpu().numpy(), b, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_cpp_backward_refuses_inputs_modified_in_place_after_the_forward():
+    sc = scenes.tiny(n=2000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=46)
+    s, t = _session(sc)
+    views = [[v["w"], v["h"], v["image_index"], v["camera_index"]] for v in sc.views]
+    outs = s.blend_point_cloud(views, sc.num_layers, True, 0.0, 0, 16)
+    with torch.no_grad():
+        t["position"].add_(0.0)
+    with pytest.raises(RuntimeError, match="modified in place"):
+        sum(o.sum() for o in outs).backward()

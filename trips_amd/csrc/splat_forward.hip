@@ -344,7 +344,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
             auto put = [&](int* c)
             {
                 const int slot = atomicAdd(c, 1);
-                if ((long long)slot < p.capacity)
+                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
                     p.bin_entries[slot] = e;
                 else
                     dropped += 1;
@@ -601,7 +601,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
                                             [&](int i)
                                             {
                                                 const int slot = atomicAdd(&s_cnt[i], 1);
-                                                if ((long long)slot < p.capacity)
+                                                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
                                                     p.keys[slot] = key;
                                                 else
                                                     dropped += 1;
@@ -625,7 +625,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
                                             const int slot = atomicAdd(&s_cnt[i], 1);
                                             if (staged)
                                                 s_keys[slot - key_start] = key;
-                                            else if ((long long)slot < p.capacity)
+                                            else if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
                                                 p.keys[slot] = key;
                                             else
                                                 dropped += 1;

@@ -6,29 +6,44 @@
 #include <torch/library.h>
 
 #include <cfloat>
+#include <map>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 
 namespace
 {
-struct Ctx
+// one context per device for the whole process
+struct ContextTable
 {
-    TripsCtx* ctx = nullptr;
-    int device    = -1;
+    std::mutex lock;
+    std::map<int, TripsCtx*> by_device;
+    ~ContextTable()
+    {
+        for (auto& kv : by_device) trips_ctx_destroy(kv.second);
+    }
 };
+ContextTable g_contexts;
+}  // namespace
 
+TripsCtx* trips_shim_context(int device)
+{
+    std::lock_guard<std::mutex> guard(g_contexts.lock);
+    auto it = g_contexts.by_device.find(device);
+    if (it != g_contexts.by_device.end()) return it->second;
+    TripsCtx* c = nullptr;
+    int rc      = trips_ctx_create(&c, device);
+    TORCH_CHECK(rc == TRIPS_OK, "trips_ctx_create: ", trips_last_error_string());
+    g_contexts.by_device[device] = c;
+    return c;
+}
+
+namespace
+{
 TripsCtx* context_for(const torch::Tensor& t)
 {
-    static thread_local Ctx cached;
     TORCH_CHECK(t.is_cuda(), "trips: tensors must live on the GPU (there is no CPU implementation of the splat path)");
-    const int dev = t.get_device();
-    if (cached.ctx && cached.device == dev) return cached.ctx;
-    TripsCtx* c = nullptr;
-    int rc      = trips_ctx_create(&c, dev);
-    TORCH_CHECK(rc == TRIPS_OK, "trips_ctx_create: ", trips_last_error_string());
-    cached.ctx    = c;
-    cached.device = dev;
-    return c;
+    return trips_shim_context(t.get_device());
 }
 
 void* current_stream(const torch::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
@@ -93,6 +108,24 @@ struct SavedForBackward : public torch::CustomClassHolder
     torch::Tensor saved_state;
     torch::Tensor position, point_size, index, texture, confidence, background, poses_se3, intrinsics, dropout;
     torch::Tensor displacement;  // [B,N,3] when the scene optimises per-view displacements
+    // The backward reads position, point_size, index, poses, intrinsics and displacement again through these
+    // tensors (the saved state holds per-point records, not copies of the inputs). Their version counters at the
+    // time of the forward: an in-place change in between (an optimiser step or ApplyTangent under gradient
+    // accumulation) would silently give gradients of another scene, so the backward refuses it.
+    std::vector<std::pair<const char*, uint32_t>> versions;
+    std::vector<torch::Tensor> versioned;
+    void remember(const char* name, const torch::Tensor& t)
+    {
+        if (!t.defined()) return;
+        versions.emplace_back(name, t._version());
+        versioned.push_back(t);
+    }
+    void check_unchanged() const
+    {
+        for (size_t i = 0; i < versioned.size(); ++i)
+            TORCH_CHECK(versioned[i]._version() == versions[i].second, "PointRender::backward: ", versions[i].first,
+                        " was modified in place after the forward that this backward belongs to");
+    }
 };
 
 TripsSplatIn make_in(const SavedForBackward& s)
@@ -198,6 +231,12 @@ variable_list PointRender::forward(AutogradContext* ctx, Variable texture, Varia
     check(trips_splat_forward(tc, &d, &in, &out, info->cache->workspace.data_ptr(), (size_t)info->cache->workspace.numel(),
                               current_stream(texture)),
           "trips_splat_forward");
+    s->remember("t_position", s->position);
+    s->remember("t_point_size", s->point_size);
+    s->remember("t_index", s->index);
+    s->remember("poses_se3", s->poses_se3);
+    s->remember("intrinsics", s->intrinsics);
+    s->remember("dynamic_refinement_t", s->displacement);
     ctx->saved_data["trips_saved"] = IValue(s);
     if (!info->train)
         for (auto& im : images) im = im.permute({0, 3, 1, 2});  // PointRenderer.cu:747-749
@@ -218,6 +257,7 @@ variable_list PointRender::backward(AutogradContext* ctx, variable_list grad_out
     NeuralRenderInfo* info = info_v.toCustomClass<NeuralRenderInfo>().get();
     auto s                 = ctx->saved_data["trips_saved"].toCustomClass<SavedForBackward>();
     TORCH_CHECK(s->saved_state.defined(), "PointRender::backward needs a forward with info->train == true");
+    s->check_unchanged();
     const TripsSplatDesc& d = s->desc;
     TripsCtx* tc            = context_for(s->texture);
     const auto dev          = s->texture.device();

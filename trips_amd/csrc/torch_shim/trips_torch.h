@@ -176,3 +176,8 @@ class MyAdam : public Optimizer
     void appendToInternalState(int param_group_index, int new_size);
 };
 }  // namespace torch::optim
+
+// The library context of a device, shared by every thread of the process (forward runs on the caller's thread, backward
+// on the autograd engine's): created on first use, destroyed when the shim is unloaded. trips_profile_enable on it
+// therefore covers forward and backward kernels alike.
+TripsCtx* trips_shim_context(int device);

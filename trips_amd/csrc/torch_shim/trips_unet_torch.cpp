@@ -9,20 +9,8 @@ namespace
 {
 TripsCtx* unet_context(const torch::Tensor& t)
 {
-    struct Ctx
-    {
-        TripsCtx* ctx = nullptr;
-        int device    = -1;
-    };
-    static thread_local Ctx cached;
     TORCH_CHECK(t.is_cuda(), "trips: the net needs GPU tensors (there is no CPU implementation)");
-    const int dev = t.get_device();
-    if (cached.ctx && cached.device == dev) return cached.ctx;
-    TripsCtx* c = nullptr;
-    TORCH_CHECK(trips_ctx_create(&c, dev) == TRIPS_OK, "trips_ctx_create: ", trips_last_error_string());
-    cached.ctx    = c;
-    cached.device = dev;
-    return c;
+    return trips_shim_context(t.get_device());
 }
 
 void* stream_of(const torch::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.get_device()).stream(); }

@@ -98,9 +98,10 @@ int check_desc(const TripsSplatDesc* d)
         if (v.camera_index < 0 || v.camera_index >= d->num_cameras)
             return fail(TRIPS_ERR_INVALID_ARG, "view %d: camera_index %d out of range", b, v.camera_index);
     }
-    // list entries are addressed with 32-bit offsets
-    if (4ll * d->num_points * d->num_layers > 0x7fffffffll && d->max_list_entries == 0)
-        return fail(TRIPS_ERR_UNSUPPORTED, "4*N*L exceeds 2^31-1; set max_list_entries");
+    // List entries and their prefix sums are 32-bit: no scan may exceed the worst case of 4 N L entries, whatever the
+    // capacity the caller grants (a smaller max_list_entries only drops entries, it does not shorten the scans).
+    if (4ll * d->num_points * d->num_layers > 0x7fffffffll)
+        return fail(TRIPS_ERR_UNSUPPORTED, "4*N*L = %lld list entries exceed 2^31-1", 4ll * d->num_points * d->num_layers);
     if (d->max_list_entries > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "max_list_entries exceeds 2^31-1");
     {
         // one LDS counter per 32 x 32 tile of the pyramid in the binning kernels

@@ -324,6 +324,9 @@ class PointRender(torch.autograd.Function):
         ctx.render_info = info
         ctx.desc = desc
         ctx.tensors = tensors
+        # the backward reads these again through their pointers: remember their version counters
+        ctx.versions = {k: tensors[k]._version for k in ("position", "point_size", "index", "poses_se3", "intrinsics",
+                                                          "displacement") if tensors[k] is not None}
         ctx.saved_state = saved
         ctx.shapes = dict(points=points.shape, layer=layer_value_of_point.shape, confidence=confidence.shape,
                           pose=pose_tangents.shape)
@@ -342,6 +345,10 @@ class PointRender(torch.autograd.Function):
         info, desc, t = ctx.render_info, ctx.desc, ctx.tensors
         if ctx.saved_state is None:
             raise RuntimeError("backward needs a forward with info.train = True")
+        for k, v in ctx.versions.items():
+            if t[k]._version != v:
+                raise RuntimeError(f"PointRender.backward: {k} was modified in place after the forward that this "
+                                   "backward belongs to (the backward reads it again)")
         sctx = get_context(t["texture"].device)
         need = ctx.needs_input_grad
         dev = t["texture"].device
