@@ -248,15 +248,18 @@ hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream
 }
 
 // ---- exports from the saved state ----
+// (the records are kept per valid point, at its compact number)
 __global__ __launch_bounds__(256) void export_points_kernel(const float* __restrict__ rec, int rec_floats,
-                                                            const float* __restrict__ prec, int n, float* ip,
-                                                            float* depth, float* size_px, int32_t* max_layer)
+                                                            const float* __restrict__ prec, const int32_t* __restrict__ cid_of,
+                                                            int n, float* ip, float* depth, float* size_px, int32_t* max_layer)
 {
     const int pid = blockIdx.x * 256 + threadIdx.x;
     if (pid >= n) return;
-    const float* r  = rec + (size_t)pid * rec_floats;
-    const float4 tl = reinterpret_cast<const float4*>(prec)[pid];  // {softplus'(raw size), depth, max_layer, size_px}
-    const bool ok   = tl.y > 0.f;
+    const int cid   = cid_of[pid];
+    const bool ok   = cid >= 0;
+    const float* r  = rec + (size_t)(ok ? cid : 0) * rec_floats;
+    // {softplus'(raw size), depth, max_layer, size_px}
+    const float4 tl = ok ? reinterpret_cast<const float4*>(prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
     if (ip)
     {
         ip[2 * (size_t)pid]     = ok ? r[0] : 0.f;
@@ -267,11 +270,11 @@ __global__ __launch_bounds__(256) void export_points_kernel(const float* __restr
     if (max_layer) max_layer[pid] = ok ? __float_as_int(tl.z) : 0;
 }
 
-hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, int n, float* ip, float* depth,
-                                float* size_px, int32_t* max_layer, hipStream_t stream)
+hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, const int32_t* cid_of, int n, float* ip,
+                                float* depth, float* size_px, int32_t* max_layer, hipStream_t stream)
 {
     if (n <= 0) return hipSuccess;
-    hipLaunchKernelGGL(export_points_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, rec, rec_floats, prec, n, ip,
+    hipLaunchKernelGGL(export_points_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, rec, rec_floats, prec, cid_of, n, ip,
                        depth, size_px, max_layer);
     return hipGetLastError();
 }
@@ -279,7 +282,8 @@ hipError_t launch_export_points(const float* rec, int rec_floats, const float* p
 // saved tables are tile-major (padded); the exports are row-major, layer by layer
 __global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, int K, const int32_t* __restrict__ lists,
                                                            const int32_t* __restrict__ retained,
-                                                           const int32_t* __restrict__ lengths, int32_t* out_lists,
+                                                           const int32_t* __restrict__ lengths,
+                                                           const int32_t* __restrict__ pid_of, int32_t* out_lists,
                                                            int32_t* out_retained, int32_t* out_lengths)
 {
     const int P = g.off[g.num_layers];
@@ -293,17 +297,21 @@ __global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, 
     if (out_retained) out_retained[r] = retained[ip];
     if (out_lengths) out_lengths[r] = lengths[ip];
     if (out_lists)
-        for (int k = 0; k < K; ++k) out_lists[(size_t)r * K + k] = lists[(size_t)ip * K + k];
+        for (int k = 0; k < K; ++k)
+        {
+            const int cid                = lists[(size_t)ip * K + k];  // compact number of the point, -1 = none
+            out_lists[(size_t)r * K + k] = cid >= 0 ? pid_of[cid] : -1;
+        }
 }
 
 hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
-                               const int32_t* lengths, int32_t* out_lists, int32_t* out_retained, int32_t* out_lengths,
-                               hipStream_t stream)
+                               const int32_t* lengths, const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
+                               int32_t* out_lengths, hipStream_t stream)
 {
     const int P = g.off[g.num_layers];
     if (P <= 0) return hipSuccess;
     hipLaunchKernelGGL(export_lists_kernel, dim3((P + 255) / 256), dim3(256), 0, stream, g, K, lists, retained, lengths,
-                       out_lists, out_retained, out_lengths);
+                       pid_of, out_lists, out_retained, out_lengths);
     return hipGetLastError();
 }
 

@@ -109,15 +109,15 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
         }
     }
 
-    int pid = 0;
+    int cid = 0;  // compact number of the entry's point
     float desc[CPAD];
 #pragma unroll
     for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
     float a = 0.f;
     if (has)
     {
-        pid               = p.lists[((size_t)(unsigned)pix << kshift) + sub];
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
+        cid               = p.lists[((size_t)(unsigned)pix << kshift) + sub];
+        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
         const float4 r0   = rec[0];
 #pragma unroll
         for (int q = 0; q < CPAD / 4; ++q)
@@ -271,16 +271,20 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 
     for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
     {
-        const float4 tail = reinterpret_cast<const float4*>(p.prec)[pid];  // {softplus'(raw size), depth, layers written, size_px}
-        const bool live   = tail.y > 0.f;
+        // the records of a valid point sit at its compact number (valid points numbered in point order: lanes that are
+        // neighbours here are neighbours there)
+        const int cid   = p.cid_of[pid];
+        const bool live = cid >= 0;
         if (!live && !overwrite) continue;
+        // {softplus'(raw size), depth, layers written, size_px}
+        const float4 tail = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
         const int tex       = identity ? pid : p.index[pid];  // (a column outside the table: the point was culled)
         const int max_layer = live ? __float_as_int(tail.z) : 0;
         float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), rv = r0;  // ip.x ip.y size field conf; view xyz, softplus'(raw size)
         uint4 rk0 = make_uint4(~0u, ~0u, ~0u, ~0u), rk1 = rk0;
         if (live)
         {
-            r0              = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
+            r0              = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
             // the point in view space, exactly as the projection kernel computed it
             float4 pos = p.position[pid];
             if (p.displacement)
@@ -293,9 +297,9 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             float view[3];
             transform_point(cam.V, pos.x, pos.y, pos.z, view);
             rv = make_float4(view[0], view[1], view[2], tail.x);
-            rk0 = *reinterpret_cast<const uint4*>(p.rank + (size_t)pid * 16);
+            rk0 = *reinterpret_cast<const uint4*>(p.rank + (size_t)cid * 16);
             // layers 4..7: a row of the second plane, defined only for the points that were written to those layers
-            if (max_layer > 4) rk1 = *reinterpret_cast<const uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)pid * 16);
+            if (max_layer > 4) rk1 = *reinterpret_cast<const uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16);
         }
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;

@@ -50,11 +50,6 @@ __device__ __forceinline__ Camera load_camera(const double* pose, const float* i
     return c;
 }
 
-__global__ __launch_bounds__(256) void fill_words_kernel(uint4* __restrict__ p, unsigned v, long long n)
-{
-    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) p[i] = make_uint4(v, v, v, v);
-}
-
 // one launch for the counters of the view and, on the first view of a call, the status block of the whole call
 __global__ void clear_header_kernel(ViewHeader* h, ViewHeader* status)
 {
@@ -73,153 +68,220 @@ __global__ void clear_header_kernel(ViewHeader* h, ViewHeader* status)
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Projection, validity, layer selection, tile binning. One point per thread, grid-stride.
+// Projection, validity and layer selection of one point (CountAndCollectTiled, RenderForward.cu:168-366, without its
+// counter updates). Both front-end passes call it and must see the same answer: it reads the inputs only.
+struct PointProjection
+{
+    bool valid;
+    int tex;        // descriptor column
+    int layers;     // layers the point is written to (0 if culled)
+    float ipx, ipy, z, size_px;
+};
+
+template <bool TRAIN>
+__device__ __forceinline__ PointProjection project_point(const ForwardParams& p, const Camera& cam, int pid, bool& not_identity,
+                                                         bool& bad_index)
+{
+    PointProjection o;
+    o.valid  = false;
+    o.layers = 0;
+    o.ipx = o.ipy = 0.f;
+    o.z       = -1.f;
+    o.size_px = 0.f;
+    const int L = p.num_layers;
+    bool skip   = false;
+    o.tex       = p.index[pid];
+    not_identity |= (o.tex != pid);
+    if ((unsigned)o.tex >= (unsigned)p.num_texels)
+    {
+        // a column outside the descriptor table: leave the point out (reported by the status query) rather
+        // than read past the tables
+        bad_index    = true;
+        not_identity = true;  // the backward then never uses the point's own number as a column
+        skip         = true;
+    }
+    if (p.viewer_only && !skip)
+    {
+        if (p.confidence[o.tex] < p.stability_cutoff_value) skip = true;
+    }
+    if (TRAIN && p.dropout)
+    {
+        if (p.dropout[pid] == 1.f) skip = true;
+    }
+    if (skip) return o;
+    float4 pos = p.position[pid];
+    if (p.displacement)
+    {
+        const float* dsp = p.displacement + (size_t)pid * 3;
+        pos.x += dsp[0];
+        pos.y += dsp[1];
+        pos.z += dsp[2];
+    }
+    const float size    = softplus(p.point_size[pid]);
+    const Projected pr  = project(cam, pos.x, pos.y, pos.z);
+    const float z       = pr.z;
+    float radius_px     = pr.scale * pos.w / z;
+    const float size_px = pr.scale * size / z;
+
+    auto valid = [&](float x, float y, int layer, float radius) -> bool
+    {
+        if (z <= 0.f) return false;
+        if (!(x >= 0.f) || x >= float(p.geom.w[layer] - 1) || !(y >= 0.f) || y >= float(p.geom.h[layer] - 1)) return false;
+        if (p.drop_out_points_by_radius && float(trunc_sat(radius)) < p.drop_out_radius_threshold) return false;
+        return true;
+    };
+    if (!valid(pr.ipx, pr.ipy, 0, radius_px)) return o;
+    int layer_higher = 0;
+    if (size_px > 1.f)
+    {
+        int lo, hi;
+        log2_floor_ceil(size_px, lo, hi);
+        layer_higher = min(hi, L - 1);
+    }
+    int layer = 0;
+    float lx = pr.ipx, ly = pr.ipy;
+    for (; layer < layer_higher + 1; ++layer, lx *= 0.5f, ly *= 0.5f, radius_px *= 0.5f)
+    {
+        const int px = (int)floorf(lx), py = (int)floorf(ly);
+        if (!valid(float(px), float(py), layer, radius_px)) break;
+    }
+    o.valid   = true;
+    o.layers  = layer;
+    o.ipx     = pr.ipx;
+    o.ipy     = pr.ipy;
+    o.z       = z;
+    o.size_px = size_px;
+    return o;
+}
+
+// Calls f(layer, px, py, first tile counter, tiles per row, crosses x, crosses y) for the layers a point is written
+// to. The 2 x 2 footprint (px..px+1, py..py+1) touches 1, 2 or 4 tiles; px+1 and py+1 are inside the image because
+// px < w-1 and py < h-1.
+template <typename F>
+__device__ __forceinline__ void for_point_tiles(const PyramidGeom& g, const PointProjection& o, int* tile_table, F&& f)
+{
+    float lx = o.ipx, ly = o.ipy;
+    for (int layer = 0; layer < o.layers; ++layer, lx *= 0.5f, ly *= 0.5f)
+    {
+        const int px = (int)floorf(lx), py = (int)floorf(ly);
+        const int tsx = g.tiles_x[layer];
+        int* bc       = tile_table + g.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
+        const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
+        f(layer, px, py, bc, tsx, cx, cy);
+    }
+}
+
+// A workgroup of the two binning kernels owns one contiguous chunk of points and walks it 1024 points at a time. The
+// valid points of the chunk are numbered in point order from the chunk's first point number on ("compact numbers":
+// cid = chunk begin + rank among the chunk's valid points; per step a ballot per wavefront and one exchange of the 16
+// wavefront counts through LDS). The numbers grow with the point id, so a sort key built from them orders like one
+// built from point ids; the records written at them are dense from the start of every chunk (whole lines, nothing
+// for culled points).
+__device__ __forceinline__ void chunk_point_range(const ForwardParams& p, int& begin, int& end)
+{
+    begin = min(p.num_points, (int)blockIdx.x * p.points_per_block);
+    end   = min(p.num_points, begin + p.points_per_block);
+}
+
+// Projection, validity, layer selection; the records of the valid points at their compact numbers; LDS histogram of
+// the tiles that the 2 x 2 footprints of this workgroup's points touch.
 template <int C, bool TRAIN>
 __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardParams p)
 {
-    constexpr int CPAD = (C + 3) & ~3;
+    constexpr int CPAD  = (C + 3) & ~3;
+    constexpr int NREC  = 1 + CPAD / 4;  // float4 per blend record
+    constexpr int WAVES = kBinThreads / 64;
     extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
-    const Camera cam   = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
-    const int L        = p.num_layers;
-    const int NB       = p.geom.bin_off[L];
-    unsigned my_valid  = 0;
-    bool not_identity  = false;  // some point's descriptor column differs from its own index
-    bool bad_index     = false;
+    __shared__ int s_valid[2][WAVES];  // valid points of every wavefront in this step (two steps in flight)
+    const Camera cam  = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
+    const int L       = p.num_layers;
+    const int NB      = p.geom.bin_off[L];
+    bool not_identity = false;  // some point's descriptor column differs from its own index
+    bool bad_index    = false;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) s_hist[i] = 0;
     __syncthreads();
 
-    // a workgroup owns one contiguous chunk of points; bin_scatter_kernel walks the same chunks
-    const int chunk_begin = min(p.num_points, (int)blockIdx.x * p.points_per_block);
-    const int chunk_end   = min(p.num_points, chunk_begin + p.points_per_block);
-    for (int pid = chunk_begin + threadIdx.x; pid < chunk_end; pid += kBinThreads)
+    int begin, end;
+    chunk_point_range(p, begin, end);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int next       = begin;  // workgroup-uniform: compact number of the chunk's next valid point
+    int step       = 0;
+    for (int base = begin; base < end; base += kBinThreads, step ^= 1)
     {
-        float4 ptk  = make_float4(0.f, 0.f, -1.f, 0.f);
-        bool skip   = false;
-        const int tex = p.index[pid];
-        constexpr int NREC = 1 + CPAD / 4;  // float4 per blend record
+        const int pid = base + threadIdx.x;
+        PointProjection o;
+        o.valid = false;
+        if (pid < end) o = project_point<TRAIN>(p, cam, pid, not_identity, bad_index);
+        const unsigned long long vm = __ballot(o.valid);
+        if (lane == 0) s_valid[step][wave] = (int)__popcll(vm);
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w)
+        {
+            const int c = s_valid[step][w];
+            before += w < wave ? c : 0;
+            total += c;
+        }
+        const int cid = next + before + (int)__popcll(vm & ((1ull << lane) - 1ull));
+        next += total;
+        if (pid >= end) continue;
+        if (TRAIN) p.cid_of[pid] = o.valid ? cid : -1;
+        if (!o.valid) continue;
+
+        // record for the blend (and the pixel pass of the backward)
         float4 recv[NREC];
+        recv[0] = make_float4(o.ipx, o.ipy, encode_size_field(o.size_px, L), p.confidence[o.tex]);
+        float d[CPAD];
 #pragma unroll
-        for (int q = 0; q < NREC; ++q) recv[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-        float4 precv = make_float4(0.f, -1.f, __int_as_float(0), 0.f);
-        not_identity |= (tex != pid);
-        if ((unsigned)tex >= (unsigned)p.num_texels)
-        {
-            // a column outside the descriptor table: leave the point out (reported by the status query) rather
-            // than read past the tables
-            bad_index    = true;
-            not_identity = true;  // the backward then never uses the point's own number as a column
-            skip         = true;
-        }
-        if (p.viewer_only && !skip)
-        {
-            if (p.confidence[tex] < p.stability_cutoff_value) skip = true;
-        }
-        if (TRAIN && p.dropout)
-        {
-            if (p.dropout[pid] == 1.f) skip = true;
-        }
-        if (!skip)
-        {
-            float4 pos = p.position[pid];
-            if (p.displacement)
-            {
-                const float* dsp = p.displacement + (size_t)pid * 3;
-                pos.x += dsp[0];
-                pos.y += dsp[1];
-                pos.z += dsp[2];
-            }
-            const float size = softplus(p.point_size[pid]);
-            const Projected pr = project(cam, pos.x, pos.y, pos.z);
-            const float z      = pr.z;
-            float radius_px    = pr.scale * pos.w / z;
-            const float size_px = pr.scale * size / z;
-            float ipx = pr.ipx, ipy = pr.ipy;
-
-            auto valid = [&](float x, float y, int layer, float radius) -> bool
-            {
-                if (z <= 0.f) return false;
-                if (!(x >= 0.f) || x >= float(p.geom.w[layer] - 1) || !(y >= 0.f) || y >= float(p.geom.h[layer] - 1))
-                    return false;
-                if (p.drop_out_points_by_radius && float(trunc_sat(radius)) < p.drop_out_radius_threshold)
-                    return false;
-                return true;
-            };
-
-            if (valid(ipx, ipy, 0, radius_px))
-            {
-                my_valid += 1;
-                int layer_higher = 0;
-                if (size_px > 1.f)
-                {
-                    int lo, hi;
-                    log2_floor_ceil(size_px, lo, hi);
-                    layer_higher = min(hi, L - 1);
-                }
-                int layer = 0;
-                float lx = ipx, ly = ipy;
-                for (; layer < layer_higher + 1; ++layer, lx *= 0.5f, ly *= 0.5f, radius_px *= 0.5f)
-                {
-                    const int px = (int)floorf(lx), py = (int)floorf(ly);
-                    if (!valid(float(px), float(py), layer, radius_px)) break;
-                    // the 2 x 2 footprint (px..px+1, py..py+1) touches 1, 2 or 4 tiles; px+1 and py+1 are inside
-                    // the image because px < w-1 and py < h-1
-                    const int tsx = p.geom.tiles_x[layer];
-                    int* bc       = s_hist + p.geom.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
-                    const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
-                    atomicAdd(bc, 1);
-                    if (cx) atomicAdd(bc + 1, 1);
-                    if (cy) atomicAdd(bc + tsx, 1);
-                    if (cx && cy) atomicAdd(bc + tsx + 1, 1);
-                }
-                ptk = make_float4(ipx, ipy, z, __int_as_float(layer));
-
-                // record for blend (+ backward)
-                recv[0] = make_float4(ipx, ipy, encode_size_field(size_px, L), p.confidence[tex]);
-                float d[CPAD];
+        for (int c = 0; c < CPAD; ++c) d[c] = c < C ? p.texture[(size_t)c * p.num_texels + o.tex] : 0.f;
 #pragma unroll
-                for (int c = 0; c < CPAD; ++c) d[c] = c < C ? p.texture[(size_t)c * p.num_texels + tex] : 0.f;
-#pragma unroll
-                for (int q = 0; q < CPAD / 4; ++q) recv[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
-                if (TRAIN)
-                {
-                    precv = make_float4(softplus_backward(p.point_size[pid]), z, __int_as_float(layer), size_px);
-                    // the few points that reach layer 4 and beyond clear their own row of the upper rank plane
-                    if (layer > 4)
-                        *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)pid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
-                }
-            }
-        }
-        // The records of culled points are written too (zeros; depth = -1, layers = 0): whole lines leave the chip
-        // faster than lines with holes
-        float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)pid * p.rec_floats);
+        for (int q = 0; q < CPAD / 4; ++q) recv[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
+        float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)cid * p.rec_floats);
 #pragma unroll
         for (int q = 0; q < NREC; ++q) rec[q] = recv[q];
+        // point record: depth and layers for the scatter pass; softplus' and the size for the backward
+        reinterpret_cast<float4*>(p.prec)[cid] =
+            make_float4(TRAIN ? softplus_backward(p.point_size[pid]) : 0.f, o.z, __int_as_float(o.layers), o.size_px);
         if (TRAIN)
         {
-            reinterpret_cast<float4*>(p.prec)[pid] = precv;
+            p.pid_of[cid] = pid;
+            // the few points that reach layer 4 and beyond clear their own row of the upper rank plane
+            if (o.layers > 4)
+                *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
         }
-        p.ptk[pid] = ptk;
+        for_point_tiles(p.geom, o, s_hist,
+                        [&](int, int, int, int* bc, int tsx, bool cx, bool cy)
+                        {
+                            atomicAdd(bc, 1);
+                            if (cx) atomicAdd(bc + 1, 1);
+                            if (cy) atomicAdd(bc + tsx, 1);
+                            if (cx && cy) atomicAdd(bc + tsx + 1, 1);
+                        });
+    }
+    if (threadIdx.x == 0)
+    {
+        p.chunk_valid[blockIdx.x] = next - begin;
+        if (next > begin) atomicAdd(&p.header->n_valid, (u64)(next - begin));
     }
 
     // this workgroup's row of the histogram matrix [workgroup][bin]
     __syncthreads();
     int32_t* row = p.bin_hist + (size_t)blockIdx.x * NB;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) row[i] = s_hist[i];
+    if (__ballot(not_identity) != 0 && lane == 0) atomicOr(&p.header->not_identity, 1ull);
+    if (__ballot(bad_index) != 0 && lane == 0) atomicOr(&p.status->bad_index, 1ull);
+}
 
-    // one counter update per block
-    __shared__ unsigned s_valid[kBinThreads / 64];
-    unsigned v = my_valid;
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    if ((threadIdx.x & 63) == 0) s_valid[threadIdx.x >> 6] = v;
-    __syncthreads();
-    if (threadIdx.x == 0)
-    {
-        unsigned t = 0;
-        for (int i = 0; i < kBinThreads / 64; ++i) t += s_valid[i];
-        if (t) atomicAdd(&p.header->n_valid, (u64)t);
-    }
-    if (__ballot(not_identity) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.header->not_identity, 1ull);
-    if (__ballot(bad_index) != 0 && (threadIdx.x & 63) == 0) atomicOr(&p.status->bad_index, 1ull);
+// Training: the rows of the first rank plane := 0xFF for the compact numbers in use (a run from the start of every
+// chunk).
+__global__ __launch_bounds__(kBinThreads) void fill_rank_kernel(const ForwardParams p)
+{
+    int begin, end;
+    chunk_point_range(p, begin, end);
+    const int n = p.chunk_valid[blockIdx.x];
+    uint4* rows = reinterpret_cast<uint4*>(p.rank);
+    for (int i = (int)threadIdx.x; i < n; i += kBinThreads) rows[begin + i] = make_uint4(~0u, ~0u, ~0u, ~0u);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -314,9 +376,9 @@ __global__ __launch_bounds__(256) void bin_column_scan_kernel(int32_t* __restric
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// One bin entry {depth bits, point id, px | py << 16} per (point, layer, touched tile). A workgroup walks the same
-// chunk of points as in project_bin_kernel; its slots inside every bin are contiguous and start at
-// bin_start[bin] + hist[workgroup][bin].
+// One bin entry {depth bits, compact point number, px | py << 16} per (point, layer, touched tile). A workgroup walks
+// the records that its chunk of the points left at the compact numbers; its slots inside every bin are contiguous
+// and start at bin_start[bin] + hist[workgroup][bin].
 __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardParams p)
 {
     extern __shared__ int s_cur[];
@@ -324,38 +386,35 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
     const int32_t* row = p.bin_hist + (size_t)blockIdx.x * NB;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) s_cur[i] = p.bin_start[i] + row[i];
     __syncthreads();
-    const int chunk_begin = min(p.num_points, (int)blockIdx.x * p.points_per_block);
-    const int chunk_end   = min(p.num_points, chunk_begin + p.points_per_block);
-    unsigned dropped      = 0;
-    for (int pid = chunk_begin + threadIdx.x; pid < chunk_end; pid += kBinThreads)
+    int begin, end;
+    chunk_point_range(p, begin, end);
+    const int n      = p.chunk_valid[blockIdx.x];
+    unsigned dropped = 0;
+    for (int cid = begin + (int)threadIdx.x; cid < begin + n; cid += kBinThreads)
     {
-        const float4 k = p.ptk[pid];
-        const float z  = k.z;
-        if (!(z > 0.f)) continue;
-        const int max_layer = __float_as_int(k.w);
-        float lx = k.x, ly = k.y;
-        for (int layer = 0; layer < max_layer; ++layer)
-        {
-            const int px = (int)floorf(lx), py = (int)floorf(ly);
-            const int tsx = p.geom.tiles_x[layer];
-            int* bc       = s_cur + p.geom.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
-            const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
-            const uint4 e = make_uint4(__float_as_uint(z), (unsigned)pid, (unsigned)px | ((unsigned)py << 16), 0u);
-            auto put = [&](int* c)
-            {
-                const int slot = atomicAdd(c, 1);
-                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
-                    p.bin_entries[slot] = e;
-                else
-                    dropped += 1;
-            };
-            put(bc);
-            if (cx) put(bc + 1);
-            if (cy) put(bc + tsx);
-            if (cx && cy) put(bc + tsx + 1);
-            lx *= 0.5f;
-            ly *= 0.5f;
-        }
+        const float4 tail = reinterpret_cast<const float4*>(p.prec)[cid];  // {softplus', depth, layers, size_px}
+        const float2 ip   = *reinterpret_cast<const float2*>(p.rec + (size_t)cid * p.rec_floats);
+        PointProjection o;
+        o.ipx    = ip.x;
+        o.ipy    = ip.y;
+        o.layers = __float_as_int(tail.z);
+        for_point_tiles(p.geom, o, s_cur,
+                        [&](int, int px, int py, int* bc, int tsx, bool cx, bool cy)
+                        {
+                            const uint4 e = make_uint4(__float_as_uint(tail.y), (unsigned)cid, (unsigned)px | ((unsigned)py << 16), 0u);
+                            auto put      = [&](int* c)
+                            {
+                                const int slot = atomicAdd(c, 1);
+                                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
+                                    p.bin_entries[slot] = e;
+                                else
+                                    dropped += 1;
+                            };
+                            put(bc);
+                            if (cx) put(bc + 1);
+                            if (cy) put(bc + tsx);
+                            if (cx && cy) put(bc + tsx + 1);
+                        });
     }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
 }
@@ -777,7 +836,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     // ---- blend (RenderForward.cu:820-1048) ----
     const int n    = min(min(len, readable), K);
     const bool has = live && sub < n;
-    const int pid  = (int)(unsigned)(best & 0xffffffffull);
+    const int cid  = (int)(unsigned)(best & 0xffffffffull);  // compact number of the entry's point
 
     float a = 0.f;
     int slot = 0;  // which of the point's (layer, footprint corner) pixels this one is
@@ -786,7 +845,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
     if (has)
     {
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)pid * RF);
+        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
         const float4 r0   = rec[0];
 #pragma unroll
         for (int q = 0; q < CPAD / 4; ++q)
@@ -867,8 +926,8 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
         // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
         if (has && sub < ret)
-            p.rank[(layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)(unsigned)pid << 4) + slot] = (unsigned char)sub;
-        const int mine = has ? pid : -1;
+            p.rank[(layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)(unsigned)cid << 4) + slot] = (unsigned char)sub;
+        const int mine = has ? cid : -1;
         if (ROW == 8)
         {
             // one 8-byte store per lane covers the pixel's whole row (K <= 16 ids): lanes 0..3 carry the ids of lane
@@ -944,19 +1003,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     const int NB = p.geom.bin_off[p.num_layers];
 
     hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header, first_view ? p.status : (ViewHeader*)nullptr);
-    if (train && p.num_points > 0)
-    {
-        // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
-        // pixel's list), filled by sort_blend: a plane of 16 bytes per point for layers 0..3 and a second one for
-        // layers 4..7. Only the first is cleared here (first thing, not in front of sort_blend, where the fill would
-        // push the keys that the list kernels have just written out of the last-level cache); the rows of the second
-        // are cleared by the projection kernel for the few points that reach those layers, and nobody else reads them.
-        ProfScope ps(prof, "fill_rank", stream);
-        const long long quads = (long long)p.num_points;  // 16 bytes per point
-        hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)std::min<long long>((quads + 255) / 256, 8192)), dim3(256), 0, stream,
-                           reinterpret_cast<uint4*>(p.rank), 0xFFFFFFFFu, quads);
-    }
-    const int G          = p.bin_groups;
+    const int G           = p.bin_groups;
     const size_t lds_hist = (size_t)NB * sizeof(int);
     {
         ProfScope ps(prof, "project_bin", stream);
@@ -974,6 +1021,16 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + kScanCols - 1) / kScanCols), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
         hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_count, p.bin_start,
                            (int32_t*)nullptr, NB, (unsigned long long*)nullptr);
+    }
+    if (train && p.num_points > 0)
+    {
+        // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
+        // pixel's list), filled by sort_blend: a plane of 16 bytes per compact number for layers 0..3 and a second one
+        // for layers 4..7. Only the first is cleared here (early, not in front of sort_blend, where the fill would push
+        // the keys that the list kernels have just written out of the last-level cache); the rows of the second are
+        // cleared by the projection kernel for the few points that reach those layers, and nobody else reads them.
+        ProfScope ps(prof, "fill_rank", stream);
+        hipLaunchKernelGGL(fill_rank_kernel, dim3(G), dim3(kBinThreads), 0, stream, p);
     }
     {
         ProfScope ps(prof, "bin_scatter", stream);

@@ -89,15 +89,18 @@ struct TripsCtx
 
 namespace trips
 {
-// Per-point records written by the projection pass.
-//   rec[pid]   4 + Cpad floats {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)}:
+// Per-point records written by the projection kernel, for the VALID points of a view only, at the point's compact
+// number cid (see wave_point_range: dense runs in point order; cid_of / pid_of translate). The 64-bit sort key of a
+// list entry is depth bits << 32 | cid: cid grows with the point id, so the order is that of depth bits << 32 |
+// point id.
+//   rec[cid]   4 + Cpad floats {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)}:
 //              everything the blend and the pixel pass of the backward need in one aligned gather of 32 bytes at
 //              C = 4 (the reference reads a 5-float record, the confidence and C descriptor planes,
 //              src/lib/rendering/RenderForward.cu:875-899,952). Kept apart from the rest because a scattered gather
 //              costs the bytes of the whole aligned block it touches.
-//   prec[pid]  4 floats {softplus'(raw size), depth (-1 = culled), layers written, size_px}: read in point order by
-//              the point pass of the backward (training only), which transforms the point into view space again
-//              rather than have the projection pass write those 12 bytes per point as well.
+//   prec[cid]  4 floats {softplus'(raw size), depth, layers written, size_px}: read by the kernel that makes the bin
+//              entries and, in point order, by the point pass of the backward, which transforms the point into view
+//              space again rather than have the projection kernel write those 12 bytes per point as well.
 __host__ __device__ inline int record_floats(int channels) { return 4 + ((channels + 3) & ~3); }
 constexpr int kPointRecordFloats = 4;
 
@@ -220,6 +223,8 @@ struct SavedLayout
     size_t lengths;   // int32 [Pi]
     size_t rank;      // uint8 [2][N, 16] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none:
                       // plane 0 layers 0..3, plane 1 layers 4..7 (rows defined only for points written to those layers)
+    size_t cid_of;    // int32 [N] compact number of every point (-1 = culled)
+    size_t pid_of;    // int32 [N] point of every compact number (the first n_valid are defined)
     size_t bytes_per_view;
 };
 
@@ -231,7 +236,8 @@ struct BackwardWorkspaceLayout
 
 struct WorkspaceLayout
 {
-    size_t ptk;          // float4 [N]   {ip.x, ip.y, depth (-1 culled), max_layer bits}
+    size_t chunk_valid;   // int32 [G]  valid points of every chunk of the binning kernels
+    size_t prec;         // float4 [N]         point records, when there is no saved state to hold them
     size_t counts;       // int32 [Pi]   list length per pixel
     size_t cursor;       // int32 [Pi]   first key of each pixel's list
     size_t run;          // int32 [Pi]   keys of a pixel already claimed by slices of a split tile (zeroed per view)
@@ -275,7 +281,9 @@ struct ForwardParams
     int32_t drop_out_points_by_radius, viewer_only;
     float drop_out_radius_threshold, dist_cutoff, stability_cutoff_value;
     // buffers
-    float4* ptk;
+    int32_t* chunk_valid;
+    int32_t* cid_of;  // training only: compact number of every point, -1 = culled
+    int32_t* pid_of;  // training only: point of every compact number
     int32_t* counts;
     int32_t* cursor;
     int32_t* bin_count;
@@ -294,7 +302,7 @@ struct ForwardParams
     unsigned long long* keys;
     long long capacity;
     float* rec;
-    float* prec;  // training only
+    float* prec;
     int32_t rec_floats;
     int32_t* lists;
     int32_t* retained;
@@ -324,6 +332,7 @@ struct BackwardParams
     int32_t rec_floats;
     const int32_t* lists;
     const int32_t* retained;
+    const int32_t* cid_of;
     const ViewHeader* header;
     const float* grad_image[TRIPS_MAX_LAYERS];
     float* entry_grad;    // [P, K, EF] {dL/dalpha, T alpha dL/dimage[0..C)}, EF = (1+C) rounded up to 4 (workspace)

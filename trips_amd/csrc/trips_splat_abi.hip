@@ -17,12 +17,12 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof);
 hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_t stream, Profiler* prof);
 hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t stream);
-hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, int n, float* ip, float* depth,
-                                float* size_px, int32_t* max_layer, hipStream_t stream);
+hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, const int32_t* cid_of, int n, float* ip,
+                                float* depth, float* size_px, int32_t* max_layer, hipStream_t stream);
 hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream);
 hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
-                               const int32_t* lengths, int32_t* out_lists, int32_t* out_retained, int32_t* out_lengths,
-                               hipStream_t stream);
+                               const int32_t* lengths, const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
+                               int32_t* out_lengths, hipStream_t stream);
 }  // namespace trips
 
 using namespace trips;
@@ -211,6 +211,10 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(P * sizeof(int32_t));
     s.rank = o;
     o += align256(N * 32);
+    s.cid_of = o;
+    o += align256(N * sizeof(int32_t));
+    s.pid_of = o;
+    o += align256(N * sizeof(int32_t));
     s.bytes_per_view = o;
     return s;
 }
@@ -226,8 +230,10 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(sizeof(ViewHeader));
     o += align256(sizeof(ViewHeader));
     o += align256(N * (size_t)record_floats(d.num_channels) * sizeof(float));
-    w.ptk = o;
-    o += align256(N * sizeof(float4));
+    w.chunk_valid = o;
+    o += align256((size_t)kBinGroups * (kBinThreads / 64) * sizeof(int32_t));
+    w.prec = o;
+    o += align256(N * kPointRecordFloats * sizeof(float));
     w.counts = o;
     o += align256(P * sizeof(int32_t));
     w.run = o;  // directly behind counts: one fill clears both
@@ -413,7 +419,7 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
         p.drop_out_radius_threshold = d.drop_out_radius_threshold;
         p.dist_cutoff               = d.dist_cutoff;
         p.stability_cutoff_value    = d.stability_cutoff_value;
-        p.ptk        = reinterpret_cast<float4*>(ws + wl.ptk);
+        p.chunk_valid = reinterpret_cast<int32_t*>(ws + wl.chunk_valid);
         p.counts     = reinterpret_cast<int32_t*>(ws + wl.counts);
         p.cursor     = reinterpret_cast<int32_t*>(ws + wl.cursor);
         p.bin_count  = reinterpret_cast<int32_t*>(ws + wl.bin_count);
@@ -443,11 +449,14 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
             p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
             p.lengths    = reinterpret_cast<int32_t*>(sv + sl.lengths);
             p.rank       = reinterpret_cast<unsigned char*>(sv + sl.rank);
+            p.cid_of     = reinterpret_cast<int32_t*>(sv + sl.cid_of);
+            p.pid_of     = reinterpret_cast<int32_t*>(sv + sl.pid_of);
         }
         else
         {
             p.header     = reinterpret_cast<ViewHeader*>(ws + align256(sizeof(ViewHeader)));
             p.rec        = reinterpret_cast<float*>(ws + 2 * align256(sizeof(ViewHeader)));
+            p.prec       = reinterpret_cast<float*>(ws + wl.prec);
             p.rec_floats = record_floats(d.num_channels);
         }
         p.status = reinterpret_cast<ViewHeader*>(ws);
@@ -539,6 +548,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.rec_floats   = record_floats(d.num_channels);
         p.lists        = reinterpret_cast<const int32_t*>(sv + sl.lists);
         p.retained     = reinterpret_cast<const int32_t*>(sv + sl.retained);
+        p.cid_of       = reinterpret_cast<const int32_t*>(sv + sl.cid_of);
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
         p.entry_grad   = reinterpret_cast<float*>(ws + bl.entry_grad);
         p.rank         = reinterpret_cast<const unsigned char*>(sv + sl.rank);
@@ -616,7 +626,8 @@ int trips_splat_export_lists(TripsCtx* ctx, const TripsSplatDesc* desc, const vo
     const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
     hipError_t e = launch_export_lists(g, desc->list_depth, reinterpret_cast<const int32_t*>(sv + sl.lists),
                                        reinterpret_cast<const int32_t*>(sv + sl.retained),
-                                       reinterpret_cast<const int32_t*>(sv + sl.lengths), device_lists, device_retained,
+                                       reinterpret_cast<const int32_t*>(sv + sl.lengths),
+                                       reinterpret_cast<const int32_t*>(sv + sl.pid_of), device_lists, device_retained,
                                        device_lengths, stream);
     if (e != hipSuccess) return hip_fail(e, "export copy");
     return TRIPS_OK;
@@ -635,7 +646,7 @@ int trips_splat_export_points(TripsCtx* ctx, const TripsSplatDesc* desc, const v
     const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
     hipError_t e = launch_export_points(reinterpret_cast<const float*>(sv + sl.rec), record_floats(desc->num_channels),
                                         reinterpret_cast<const float*>(sv + sl.prec),
-                                        desc->num_points, device_ip, device_depth, device_size_px, device_max_layer,
+                                        reinterpret_cast<const int32_t*>(sv + sl.cid_of), desc->num_points, device_ip, device_depth, device_size_px, device_max_layer,
                                         reinterpret_cast<hipStream_t>(stream_));
     if (e != hipSuccess) return hip_fail(e, "export points");
     return TRIPS_OK;
