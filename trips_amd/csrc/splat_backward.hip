@@ -61,7 +61,7 @@ __device__ __forceinline__ double wave_sum(double v)
 
 
 // ---------------------------------------------------------------------------------------------------------
-// Pass 1: per pixel row. Writes entry_grad[pix*K + j] = {dL/dalpha_j, T_j alpha_j g[0..C)}.
+// Pass 1: per pixel row. Writes the pixel's 128-byte row {g[0..Cpad), {dL/dalpha_j, T_j alpha_j} for j < kRowEntries}.
 // 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
 // than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
 template <int C, int ROW>
@@ -70,7 +70,6 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int RF   = 4 + CPAD;          // floats per blend record
-    constexpr int EF   = (1 + C + 3) & ~3;  // floats per entry of entry_grad
     const int lane     = threadIdx.x & 63;
     const int sub      = lane & (ROW - 1);
     const int grp      = lane / ROW;
@@ -164,18 +163,25 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
 #pragma unroll
         for (int c = 0; c < C; ++c) acc_bg[c] += T_after * g[c];
     }
+    // For pass 2, one 128-byte row per pixel: the pixel's image gradient (a point finds all channels and its entry in
+    // one line) followed by {dL/dalpha, T alpha} of the first kRowEntries retained entries; the few entries beyond that
+    // go to a table of their own.
+    constexpr int KIN = entry_row_entries(CPAD);
+    float* row        = p.entry_grad + ((size_t)(unsigned)pix << 5);
     if (has)
     {
-        // {dL/dalpha, T*alpha*g[0..C)} padded to a multiple of 4 floats: one aligned gather for pass 2
-        float e[EF];
-        e[0] = grad_alpha;
+        if (sub < KIN)
+            reinterpret_cast<float2*>(row + CPAD)[sub] = make_float2(grad_alpha, ta);
+        else
+            reinterpret_cast<float2*>(p.entry_over)[(size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)] = make_float2(grad_alpha, ta);
+    }
+    if (sub == 0 && m > 0)
+    {
+        float gp[CPAD];
 #pragma unroll
-        for (int c = 0; c < C; ++c) e[1 + c] = ta * g[c];
+        for (int c = 0; c < CPAD; ++c) gp[c] = c < C ? g[c] : 0.f;
 #pragma unroll
-        for (int c = 1 + C; c < EF; ++c) e[c] = 0.f;
-        float4* dst = reinterpret_cast<float4*>(p.entry_grad + (((size_t)(unsigned)pix << kshift) + sub) * EF);
-#pragma unroll
-        for (int q = 0; q < EF / 4; ++q) dst[q] = make_float4(e[4 * q], e[4 * q + 1], e[4 * q + 2], e[4 * q + 3]);
+        for (int q = 0; q < CPAD / 4; ++q) reinterpret_cast<float4*>(row)[q] = make_float4(gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]);
     }
 }
 
@@ -247,12 +253,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 8 
 template <int C>
 __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardParams p)
 {
-    constexpr int EF   = (1 + C + 3) & ~3;
-    constexpr int RF   = 4 + ((C + 3) & ~3);  // floats per blend record
+    constexpr int CPAD = (C + 3) & ~3;
+    constexpr int KIN  = entry_row_entries(CPAD);
+    constexpr int RF   = 4 + CPAD;  // floats per blend record
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
     const int lane     = threadIdx.x & 63;
-    const int kshift   = p.list_depth == 16 ? 4 : 3;
-    const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
+        const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     float R[9];
     rotation_matrix(cam.V, R);
     const bool want_pose = p.d_pose != nullptr;
@@ -322,16 +328,23 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             const float sx = ux - fx, sy = uy - fy;
             float lfac = 1.f, J_lf = 0.f;
             if (want_size) lfac = layer_factor_encoded_grad(r0.z, tail.w, layer, p.num_layers, &J_lf);
-            float4 e[4][EF / 4];
+            float2 e[4];
+            float4 gq[4][CPAD / 4];
 #pragma unroll
             for (int corner = 0; corner < 4; ++corner)
             {
                 const unsigned j = (word >> (8 * corner)) & 0xFFu;
                 const int gx = px + (corner & 1), gy = py + (corner >> 1);
                 const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
-                const float4* src  = reinterpret_cast<const float4*>(p.entry_grad + (size_t)((pix << kshift) + (j & 15u)) * EF);
+                const bool on      = j != 0xFFu;
+                const float* row   = p.entry_grad + ((size_t)pix << 5);  // the pixel's 128-byte row
+                const unsigned jj  = j & 15u;
+                const float2* src2 = jj < (unsigned)KIN ? reinterpret_cast<const float2*>(row + CPAD) + jj
+                                                        : reinterpret_cast<const float2*>(p.entry_over) + ((size_t)pix * (16 - KIN) + (jj - KIN));
+                e[corner]          = on ? *src2 : make_float2(0.f, 0.f);
+                const float4* src  = reinterpret_cast<const float4*>(row);
 #pragma unroll
-                for (int q = 0; q < EF / 4; ++q) e[corner][q] = (j != 0xFFu) ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+                for (int q = 0; q < CPAD / 4; ++q) gq[corner][q] = on ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
             }
 #pragma unroll
             for (int corner = 0; corner < 4; ++corner)
@@ -339,18 +352,19 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
                 const unsigned j = (word >> (8 * corner)) & 0xFFu;
                 if (j == 0xFFu) continue;
                 const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                float ev[EF];
+                float gv[CPAD];
 #pragma unroll
-                for (int q = 0; q < EF / 4; ++q)
+                for (int q = 0; q < CPAD / 4; ++q)
                 {
-                    ev[4 * q]     = e[corner][q].x;
-                    ev[4 * q + 1] = e[corner][q].y;
-                    ev[4 * q + 2] = e[corner][q].z;
-                    ev[4 * q + 3] = e[corner][q].w;
+                    gv[4 * q]     = gq[corner][q].x;
+                    gv[4 * q + 1] = gq[corner][q].y;
+                    gv[4 * q + 2] = gq[corner][q].z;
+                    gv[4 * q + 3] = gq[corner][q].w;
                 }
-                const float grad_alpha = ev[0];
+                const float grad_alpha = e[corner].x;
+                const float ta         = e[corner].y;
 #pragma unroll
-                for (int c = 0; c < C; ++c) tex_grad[c] += ev[1 + c];
+                for (int c = 0; c < C; ++c) tex_grad[c] += ta * gv[c];
                 // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
                 // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
                 const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);

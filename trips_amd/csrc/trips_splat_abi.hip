@@ -274,10 +274,12 @@ namespace
 BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     BackwardWorkspaceLayout w;
-    const size_t P = (size_t)g.bin_off[d.num_layers] * kTilePixels, K = (size_t)d.list_depth;
+    const size_t P = (size_t)g.bin_off[d.num_layers] * kTilePixels;
     size_t o       = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
     w.entry_grad   = o;
-    o += align256(P * K * (size_t)((1 + d.num_channels + 3) & ~3) * sizeof(float));
+    o += align256(P * 128);
+    w.entry_over = o;
+    o += align256(P * (size_t)(16 - entry_row_entries((d.num_channels + 3) & ~3)) * 2 * sizeof(float));
     w.bytes = o;
     return w;
 }
@@ -551,6 +553,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.cid_of       = reinterpret_cast<const int32_t*>(sv + sl.cid_of);
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
         p.entry_grad   = reinterpret_cast<float*>(ws + bl.entry_grad);
+        p.entry_over   = reinterpret_cast<float*>(ws + bl.entry_over);
         p.rank         = reinterpret_cast<const unsigned char*>(sv + sl.rank);
         for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
         p.d_texture    = grads->d_texture;
