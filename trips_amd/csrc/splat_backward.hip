@@ -37,7 +37,12 @@ __device__ __forceinline__ Camera load_camera_bw(const double* pose, const float
     c.cx = intr[2];
     c.cy = intr[3];
     c.s  = intr[4];
-    for (int i = 0; i < 8; ++i) c.dist[i] = intr[5 + i];
+    c.no_distortion = true;
+    for (int i = 0; i < 8; ++i)
+    {
+        c.dist[i] = intr[5 + i];
+        c.no_distortion = c.no_distortion && c.dist[i] == 0.f;
+    }
     c.cfx         = v.crop_transform[0];
     c.cfy         = v.crop_transform[1];
     c.ccx         = v.crop_transform[2];

@@ -34,7 +34,12 @@ __device__ __forceinline__ Camera load_camera(const double* pose, const float* i
     c.cx = intr[2];
     c.cy = intr[3];
     c.s  = intr[4];
-    for (int i = 0; i < 8; ++i) c.dist[i] = intr[5 + i];
+    c.no_distortion = true;
+    for (int i = 0; i < 8; ++i)
+    {
+        c.dist[i] = intr[5 + i];
+        c.no_distortion = c.no_distortion && c.dist[i] == 0.f;
+    }
     c.cfx         = v.crop_transform[0];
     c.cfy         = v.crop_transform[1];
     c.ccx         = v.crop_transform[2];
@@ -68,8 +73,8 @@ __global__ void clear_header_kernel(ViewHeader* h, ViewHeader* status)
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Projection, validity and layer selection of one point (CountAndCollectTiled, RenderForward.cu:168-366, without its
-// counter updates). Both front-end passes call it and must see the same answer: it reads the inputs only.
+// Projection, validity and layer selection of one point (CountAndCollectTiled, RenderForward.cu:168-366; its per-pixel
+// counter updates become per-tile ones).
 struct PointProjection
 {
     bool valid;
@@ -78,9 +83,11 @@ struct PointProjection
     float ipx, ipy, z, size_px;
 };
 
+// `s_hist`: LDS counters, one per tile; the 2 x 2 footprint (px..px+1, py..py+1) of every layer the point is written to
+// adds one to the 1, 2 or 4 tiles it touches (px+1 and py+1 are inside the image because px < w-1 and py < h-1).
 template <bool TRAIN>
-__device__ __forceinline__ PointProjection project_point(const ForwardParams& p, const Camera& cam, int pid, bool& not_identity,
-                                                         bool& bad_index)
+__device__ __forceinline__ PointProjection project_point(const ForwardParams& p, const Camera& cam, int pid, int* s_hist,
+                                                         bool& not_identity, bool& bad_index)
 {
     PointProjection o;
     o.valid  = false;
@@ -144,6 +151,13 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
     {
         const int px = (int)floorf(lx), py = (int)floorf(ly);
         if (!valid(float(px), float(py), layer, radius_px)) break;
+        const int tsx = p.geom.tiles_x[layer];
+        int* bc       = s_hist + p.geom.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
+        const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
+        atomicAdd(bc, 1);
+        if (cx) atomicAdd(bc + 1, 1);
+        if (cy) atomicAdd(bc + tsx, 1);
+        if (cx && cy) atomicAdd(bc + tsx + 1, 1);
     }
     o.valid   = true;
     o.layers  = layer;
@@ -211,7 +225,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         const int pid = base + threadIdx.x;
         PointProjection o;
         o.valid = false;
-        if (pid < end) o = project_point<TRAIN>(p, cam, pid, not_identity, bad_index);
+        if (pid < end) o = project_point<TRAIN>(p, cam, pid, s_hist, not_identity, bad_index);
         const unsigned long long vm = __ballot(o.valid);
         if (lane == 0) s_valid[step][wave] = (int)__popcll(vm);
         __syncthreads();
@@ -246,18 +260,14 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         if (TRAIN)
         {
             p.pid_of[cid] = pid;
-            // the few points that reach layer 4 and beyond clear their own row of the upper rank plane
+            // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
+            // pixel's list; filled by sort_blend): a plane of 16 bytes per compact number for layers 0..3 and a second
+            // one for layers 4..7. Every valid point clears its row of the first, the few points that reach layer 4 and
+            // beyond their row of the second as well.
+            *reinterpret_cast<uint4*>(p.rank + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
             if (o.layers > 4)
                 *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
         }
-        for_point_tiles(p.geom, o, s_hist,
-                        [&](int, int, int, int* bc, int tsx, bool cx, bool cy)
-                        {
-                            atomicAdd(bc, 1);
-                            if (cx) atomicAdd(bc + 1, 1);
-                            if (cy) atomicAdd(bc + tsx, 1);
-                            if (cx && cy) atomicAdd(bc + tsx + 1, 1);
-                        });
     }
     if (threadIdx.x == 0)
     {
@@ -271,17 +281,6 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     for (int i = threadIdx.x; i < NB; i += kBinThreads) row[i] = s_hist[i];
     if (__ballot(not_identity) != 0 && lane == 0) atomicOr(&p.header->not_identity, 1ull);
     if (__ballot(bad_index) != 0 && lane == 0) atomicOr(&p.status->bad_index, 1ull);
-}
-
-// Training: the rows of the first rank plane := 0xFF for the compact numbers in use (a run from the start of every
-// chunk).
-__global__ __launch_bounds__(kBinThreads) void fill_rank_kernel(const ForwardParams p)
-{
-    int begin, end;
-    chunk_point_range(p, begin, end);
-    const int n = p.chunk_valid[blockIdx.x];
-    uint4* rows = reinterpret_cast<uint4*>(p.rank);
-    for (int i = (int)threadIdx.x; i < n; i += kBinThreads) rows[begin + i] = make_uint4(~0u, ~0u, ~0u, ~0u);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -390,31 +389,49 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
     chunk_point_range(p, begin, end);
     const int n      = p.chunk_valid[blockIdx.x];
     unsigned dropped = 0;
-    for (int cid = begin + (int)threadIdx.x; cid < begin + n; cid += kBinThreads)
+    constexpr int U  = 2;  // records of a thread in flight together
+    for (int cid0 = begin + (int)threadIdx.x; cid0 < begin + n; cid0 += U * kBinThreads)
     {
-        const float4 tail = reinterpret_cast<const float4*>(p.prec)[cid];  // {softplus', depth, layers, size_px}
-        const float2 ip   = *reinterpret_cast<const float2*>(p.rec + (size_t)cid * p.rec_floats);
-        PointProjection o;
-        o.ipx    = ip.x;
-        o.ipy    = ip.y;
-        o.layers = __float_as_int(tail.z);
-        for_point_tiles(p.geom, o, s_cur,
-                        [&](int, int px, int py, int* bc, int tsx, bool cx, bool cy)
-                        {
-                            const uint4 e = make_uint4(__float_as_uint(tail.y), (unsigned)cid, (unsigned)px | ((unsigned)py << 16), 0u);
-                            auto put      = [&](int* c)
+        float4 tail[U];  // {softplus', depth, layers, size_px}
+        float2 ip[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+        {
+            const int cid = cid0 + u * kBinThreads;
+            if (cid < begin + n)
+            {
+                tail[u] = reinterpret_cast<const float4*>(p.prec)[cid];
+                ip[u]   = *reinterpret_cast<const float2*>(p.rec + (size_t)cid * p.rec_floats);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+        {
+            const int cid = cid0 + u * kBinThreads;
+            if (cid >= begin + n) break;
+            PointProjection o;
+            o.ipx    = ip[u].x;
+            o.ipy    = ip[u].y;
+            o.layers = __float_as_int(tail[u].z);
+            const unsigned zbits = __float_as_uint(tail[u].y);
+            for_point_tiles(p.geom, o, s_cur,
+                            [&](int, int px, int py, int* bc, int tsx, bool cx, bool cy)
                             {
-                                const int slot = atomicAdd(c, 1);
-                                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
-                                    p.bin_entries[slot] = e;
-                                else
-                                    dropped += 1;
-                            };
-                            put(bc);
-                            if (cx) put(bc + 1);
-                            if (cy) put(bc + tsx);
-                            if (cx && cy) put(bc + tsx + 1);
-                        });
+                                const uint4 e = make_uint4(zbits, (unsigned)cid, (unsigned)px | ((unsigned)py << 16), 0u);
+                                auto put      = [&](int* c)
+                                {
+                                    const int slot = atomicAdd(c, 1);
+                                    if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
+                                        p.bin_entries[slot] = e;
+                                    else
+                                        dropped += 1;
+                                };
+                                put(bc);
+                                if (cx) put(bc + 1);
+                                if (cy) put(bc + tsx);
+                                if (cx && cy) put(bc + tsx + 1);
+                            });
+        }
     }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
 }
@@ -1021,16 +1038,6 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + kScanCols - 1) / kScanCols), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
         hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_count, p.bin_start,
                            (int32_t*)nullptr, NB, (unsigned long long*)nullptr);
-    }
-    if (train && p.num_points > 0)
-    {
-        // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
-        // pixel's list), filled by sort_blend: a plane of 16 bytes per compact number for layers 0..3 and a second one
-        // for layers 4..7. Only the first is cleared here (early, not in front of sort_blend, where the fill would push
-        // the keys that the list kernels have just written out of the last-level cache); the rows of the second are
-        // cleared by the projection kernel for the few points that reach those layers, and nobody else reads them.
-        ProfScope ps(prof, "fill_rank", stream);
-        hipLaunchKernelGGL(fill_rank_kernel, dim3(G), dim3(kBinThreads), 0, stream, p);
     }
     {
         ProfScope ps(prof, "bin_scatter", stream);

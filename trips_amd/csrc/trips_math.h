@@ -230,6 +230,7 @@ struct Camera
     Pose V;
     float fx, fy, cx, cy, s;
     float dist[8];
+    bool no_distortion;            // all of dist[] are zero (wave-uniform: the forward then skips the rational model)
     float cfx, cfy, ccx, ccy, cs;  // crop transform
     float r00, r01, r10, r11;      // crop rotation
     float centre_x, centre_y;      // float(w/2), float(h/2), integer division
@@ -250,7 +251,16 @@ __device__ __forceinline__ Projected project(const Camera& cam, float px, float 
     float iz = 1.f / view[2];
     float nx = view[0] * iz, ny = view[1] * iz;
     float dx, dy;
-    distort(nx, ny, cam.dist, cam.dist_cutoff, dx, dy, nullptr, nullptr);
+    if (cam.no_distortion)
+    {
+        // all eight coefficients are zero: the model is x * (1 / 1) + 0 in float arithmetic, which is x + 0 (the
+        // addition turns a negative zero into a positive one, as the full expression does); the cut-off stays
+        dx = nx + 0.f;
+        dy = ny + 0.f;
+        if (nx * nx + ny * ny > cam.dist_cutoff * cam.dist_cutoff) dx = dy = 100000.f;
+    }
+    else
+        distort(nx, ny, cam.dist, cam.dist_cutoff, dx, dy, nullptr, nullptr);
     if (dx == 100000.f) z = 0.f;
     float ix = cam.fx * dx + cam.s * dy + cam.cx;
     float iy = cam.fy * dy + cam.cy;
