@@ -26,31 +26,39 @@ DEFAULT_POINTS = 6_000_000
 # (KiB per dispatch, one counter per run, same bench.py command with --steps 2 --warmup 1 --cpu-steps 0
 # --calibration-copy). A plain 256 MiB device copy reads FETCH_SIZE = 131084 and WRITE_SIZE = 262144 for
 # 262144 KiB each way, hence the scale factors. bench.py cannot run the profiler on itself; these are the figures
-# of the committed summary of those two runs and apply to the default --points only.
+# of the committed summary of those two runs and apply to the default --points only. They belong to the kernel
+# sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
+# profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
+PMC_SOURCES_SHA256 = "unprofiled"
 PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (135221, 382703),
-    "bin_scatter": (48402, 203115),
-    "tile_count": (51871, 34387),
-    "tile_scatter": (83710, 463290),
-    "fill_rank": (13, 93750),
-    "sort_blend": (396803, 424852),
-    "backward_pixels": (528132, 417618),
-    "backward_points": (1065514, 234887),
-    "adam_fused": (582979, 792823),
 }
+SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
+                        "splat_internal.h", "trips_math.h", "row16.h")
 
 
-def measured_traffic_bytes(kernel):
-    if kernel not in PMC_KIB_DEFAULT_WORKLOAD:
+def kernel_sources_sha256():
+    """Digest of the sources of the splat and Adam kernels, as shipped next to this file."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in SPLAT_KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "trips_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic_bytes(kernel, usable=True):
+    if not usable or kernel not in PMC_KIB_DEFAULT_WORKLOAD:
         return None
     f, w = PMC_KIB_DEFAULT_WORKLOAD[kernel]
     return int((f * PMC_FETCH_SCALE + w * PMC_WRITE_SCALE) * 1024)
 
 
-def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0):
+def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam_step_bytes=4):
     """Algorithmic HBM bytes per launch of each kernel, from the run's own counters
-    (N points, E list entries, R retained entries, P pyramid pixels)."""
+    (N points, E list entries, R retained entries, P pyramid pixels). Adam: an updated element reads w, g, m, v and its
+    step counter and writes w, m, v and the counter (28 + 2 x counter bytes: 44 with the reference's int64 counters,
+    36 with int32 ones); an element with zero gradient is counted with 8 bytes in both."""
     N, E, R, P, C = n_points, c["E"], c["R"], c["P"], channels
     return {
         "project_bin": 24 * N,                                    # position 16 + size 4 + index 4
@@ -58,7 +66,7 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0):
         "sort_blend": 8 * E + (20 + 4 + 4 * C + 28) * R + 4 * C * P,  # keys read, record+conf+descriptor, saved, image
         "backward_pixels": 4 * C * P + (28 + 4 * C + 4 + 20) * R,  # dL/dimage, saved entry, descriptor+conf+record
         "backward_points": (4 * C + 4 + 12 + 4) * R,              # one write per accumulated gradient float
-        "adam_fused": 44 * adam_nonzero + 8 * adam_zero,
+        "adam_fused": (28 + 2 * adam_step_bytes) * adam_nonzero + 8 * adam_zero,
     }
 
 
@@ -168,7 +176,23 @@ def main():
             torch.cuda.synchronize()
             graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
             del graph
-        return dict(graph_ms=graph_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
+        # Adam on its own, with the step counters the product uses (int32) and with the reference's int64 state tensor
+        adam_ms = {}
+        for name, dt in (("int32_counters", torch.int32), ("int64_counters", torch.int64)):
+            o2 = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, param_steps_dtype=dt)
+            for _ in range(2):
+                o2.step()
+            torch.cuda.synchronize()
+            ctx.profile_enable(True)
+            ctx.profile_read()
+            for _ in range(args.steps):
+                o2.step()
+            torch.cuda.synchronize()
+            ms, launches = ctx.profile_read()["adam_fused"]  # HIP events around the launch, as for the step's kernels
+            ctx.profile_enable(False)
+            adam_ms[name] = ms / max(launches, 1)
+            del o2
+        return dict(graph_ms=graph_ms, adam_ms=adam_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
                     grad_images=grad_images, grads=grads, opt=opt, counters=counters, nz=nz, total_el=total_el,
                     prof=prof, ms_per_step=ms_per_step)
 
@@ -193,7 +217,11 @@ def main():
     small = [grads[k] for k in ("d_background", "d_pose", "d_intrinsics")]  # the gradients that are added to
     N, C = desc.num_points, desc.num_channels
 
-    alg = algorithmic_bytes(counters, N, C, adam_nonzero=nz, adam_zero=total_el - nz)
+    # the timed step runs the product's optimiser state: int32 step counters, 36 bytes per updated element
+    alg = algorithmic_bytes(counters, N, C, adam_nonzero=nz, adam_zero=total_el - nz, adam_step_bytes=4)
+    alg_adam_i64 = algorithmic_bytes(counters, N, C, adam_nonzero=nz, adam_zero=total_el - nz, adam_step_bytes=8)["adam_fused"]
+    pmc_usable = (args.points == DEFAULT_POINTS and args.point_order == "random" and
+                  kernel_sources_sha256() == PMC_SOURCES_SHA256)
     kernels = {}
     for name, (ms, launches) in prof.items():
         avg = ms / max(launches, 1)
@@ -201,6 +229,12 @@ def main():
         if name in alg and avg > 0:
             entry["alg_bytes"] = int(alg[name])
             entry["alg_GBs"] = round(alg[name] / (avg * 1e-3) / 1e9, 1)
+            entry["roofline_frac"] = round(alg[name] / (avg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        traffic = measured_traffic_bytes(name, pmc_usable)
+        if traffic is not None:
+            entry["traffic_bytes"] = traffic
+            if name in alg:
+                entry["traffic_over_alg"] = round(traffic / alg[name], 2)
         kernels[name] = entry
     dom = max((k for k in kernels if k in alg), key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches_per_step"])
     achieved = kernels[dom]["alg_GBs"]
@@ -320,15 +354,27 @@ def main():
                      "wall_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4)},
         "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
-        # the same with the HBM traffic rocprofv3 measured (committed summary under profiles/) instead of the
-        # algorithmic bytes: what the memory system actually moved per second
-        "hbm_frac_fwd_bwd_measured_traffic": round(
+        # How busy the memory system was, NOT the target metric: the HBM traffic rocprofv3 measured (committed summary
+        # under profiles/; wasted re-reads included) per second of forward + backward kernels over the peak. null when
+        # the kernel sources have changed since that profile.
+        "hbm_busy_frac": round(
             sum(measured_traffic_bytes(k) for k in PMC_KIB_DEFAULT_WORKLOAD if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
-            HBM_PEAK_GBS, 4) if (fwd_bwd_ms > 0 and args.points == DEFAULT_POINTS and args.point_order == "random") else None,
+            HBM_PEAK_GBS, 4) if (fwd_bwd_ms > 0 and pmc_usable) else None,
+        "traffic_profile": {"sources_sha256": PMC_SOURCES_SHA256, "matches_these_sources": pmc_usable},
         "roofline": {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic_bytes(dom) if args.points == DEFAULT_POINTS and args.point_order == "random" else None,
+                     "traffic": measured_traffic_bytes(dom, pmc_usable),
                      "algorithmic_bytes": int(alg[dom]), "avg_ms": kernels[dom]["avg_ms"]},
+        # the kernel whose measured traffic is furthest above its algorithmic bytes
+        "worst_traffic_ratio": (lambda c: {"kernel": c[0], "traffic_over_alg": c[1]} if c else None)(
+            max(((k, v["traffic_over_alg"]) for k, v in kernels.items() if "traffic_over_alg" in v),
+                key=lambda kv: kv[1], default=None)),
+        "adam": {"timed_step_state": "int32 step counters (36 B per updated element)",
+                 "kernel_ms_int32_counters": round(r["adam_ms"]["int32_counters"], 4),
+                 "kernel_ms_int64_counters": round(r["adam_ms"]["int64_counters"], 4),
+                 "alg_bytes_int32": int(alg["adam_fused"]), "alg_bytes_int64": int(alg_adam_i64),
+                 "alg_GBs_int32": round(alg["adam_fused"] / (r["adam_ms"]["int32_counters"] * 1e-3) / 1e9, 1),
+                 "alg_GBs_int64": round(alg_adam_i64 / (r["adam_ms"]["int64_counters"] * 1e-3) / 1e9, 1)},
         "kernels": kernels,
         "other_point_order": other_order,
         "unet": unet,

@@ -15,7 +15,11 @@ from .renderer import get_context
 
 class MyAdam(torch.optim.Optimizer):
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, relative_weight_decay=0.0,
-                 absolute_weight_decay=0.0, weight_clipping_magnitude=0.0, adabound=False):
+                 absolute_weight_decay=0.0, weight_clipping_magnitude=0.0, adabound=False,
+                 param_steps_dtype=torch.int32):
+        if param_steps_dtype not in (torch.int32, torch.int64):
+            raise ValueError("param_steps_dtype must be torch.int32 or torch.int64 (the reference's state tensor)")
+        self.param_steps_dtype = param_steps_dtype
         if lr < 0:
             raise ValueError(f"Invalid learning rate: {lr}")
         if eps < 0:
@@ -36,7 +40,7 @@ class MyAdam(torch.optim.Optimizer):
     def _state_for(self, p):
         st = self.state[p]
         if len(st) == 0:
-            st["param_steps"] = torch.zeros(p.shape, dtype=torch.int32, device=p.device)
+            st["param_steps"] = torch.zeros(p.shape, dtype=self.param_steps_dtype, device=p.device)
             st["first_moments"] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
             st["second_moments"] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
             st["current_step"] = 0
