@@ -129,35 +129,35 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
             const int g = item % GROUPS, pp = item / GROUPS;
             const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
-            float v[8];
+            // The interpolation runs in packed fp16: the weights are products of 0, 1/4, 3/4 and 1 (exact in fp16), the
+            // operands are fp16 already and the result is stored as fp16; three fused multiply-adds per pair of channels
+            // instead of eight conversions and four fp32 operations per channel.
+            half8 h;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = 0.f;
+            for (int i = 0; i < 8; ++i) h[i] = _Float16(0.f);
             if (y >= 0 && y < p.H && x >= 0 && x < p.W)
             {
                 int ya, yb, xa, xb;
                 float ly, lx;
                 up2_source(y, p.Hb, ya, yb, ly);
                 up2_source(x, p.Wb, xa, xb, lx);
-                const float w00 = (1.f - ly) * (1.f - lx), w01 = (1.f - ly) * lx, w10 = ly * (1.f - lx), w11 = ly * lx;
+                const _Float16 w00 = _Float16((1.f - ly) * (1.f - lx)), w01 = _Float16((1.f - ly) * lx);
+                const _Float16 w10 = _Float16(ly * (1.f - lx)), w11 = _Float16(ly * lx);
                 const half8 a = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
                 const half8 b = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
                 const half8 c = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
                 const half8 d = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = w00 * float(a[i]) + w01 * float(b[i]) + w10 * float(c[i]) + w11 * float(d[i]);
+                const half8 W00 = {w00, w00, w00, w00, w00, w00, w00, w00}, W01 = {w01, w01, w01, w01, w01, w01, w01, w01};
+                const half8 W10 = {w10, w10, w10, w10, w10, w10, w10, w10}, W11 = {w11, w11, w11, w11, w11, w11, w11, w11};
+                h = __builtin_elementwise_fma(d, W11, __builtin_elementwise_fma(c, W10, __builtin_elementwise_fma(b, W01, a * W00)));
             }
             _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
             if (g == 0)
             {
-                for (int i = C; i < 8; ++i) dst[i] = _Float16(v[i]);  // [0, C) holds this level's image
+                for (int i = C; i < 8; ++i) dst[i] = h[i];  // [0, C) holds this level's image
             }
             else
-            {
-                half8 h;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) h[i] = _Float16(v[i]);
                 *reinterpret_cast<half8*>(dst) = h;
-            }
         }
     }
 
