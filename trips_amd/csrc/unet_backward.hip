@@ -293,8 +293,9 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     extern __shared__ _Float16 smem[];
     _Float16* s_patch = smem;
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
-    ConvTapRing<KC, NN> ring;
-    conv_taps_prefetch(ring, p.wt);  // in flight while the patch is loaded
+    ConvTapStage<KC, NN> taps;
+    conv_tap_fetch(taps, p.wt, 0);  // in flight while the patch is loaded
+    _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;  // two tap buffers of the weights
     // the patch of pre-activation gradients, four 16-byte loads of a thread in flight together
     constexpr int kItems = kConvPatchH * kConvPatchW * GROUPS;
     for (int item0 = threadIdx.x; item0 < kItems; item0 += 4 * 256)
@@ -319,9 +320,10 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
             if (item < kItems) *reinterpret_cast<half8*>(s_patch + (size_t)(item / GROUPS) * ROW + 8 * (item % GROUPS)) = v[j];
         }
     }
+    conv_tap_stage(taps, s_taps);
     __syncthreads();
     floatx4 acc[4][NB];
-    conv_taps_mfma<KC, NN>(s_patch, p.wt, ring, acc);
+    conv_taps_mfma<KC, NN>(s_patch, s_taps, p.wt, taps, acc);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
     // ---- epilogue: the tile staged in LDS (the patch is no longer needed) and written channels innermost with
@@ -898,7 +900,8 @@ namespace
 template <int KC, int NN>
 hipError_t launch_bwd_data(const BwdDataParams& p, hipStream_t stream)
 {
-    const size_t lds_in  = (size_t)kConvPatchH * kConvPatchW * (KC + kLdsChanPad) * sizeof(_Float16);  // up to 92 KB
+    // the patch and two tap buffers of the weights: up to 92 + 35 KB
+    const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW + 2 * NN) * (KC + kLdsChanPad) * sizeof(_Float16);
     const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NN + kLdsChanPad) * sizeof(_Float16) + 4 * sizeof(float));
     const size_t lds     = std::max(lds_in, lds_out);
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN>),

@@ -34,51 +34,66 @@ __device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i
 }
 
 
-// The 9-tap implicit-GEMM core shared by the forward convolution and the data gradient: A operands are 16-byte
-// LDS reads from a (8+2) x (32+2) pixel patch with KIN channels innermost (row stride KIN + 8 halves), B operands
-// (packed weights [tap][NOUT][KIN], L2-resident) are loaded from memory directly into a ring of registers, DEPTH taps
-// ahead of their use: the first DEPTH taps are requested by conv_taps_prefetch, which a kernel calls before it
-// assembles its patch, so their latency (a tap's fragments are one dependent L2 round trip) hides behind that work;
-// the tap loop has no barrier. A wavefront owns two rows of the 8 x 32 output tile = four 16-pixel row blocks;
-// acc[m][n] is the 16 x 16 block of pixels m, outputs 16n .. 16n+15.
+// The 9-tap implicit-GEMM core shared by the forward convolution and the data gradient. A operands are 16-byte LDS
+// reads from a (8+2) x (32+2) pixel patch with KIN channels innermost (row stride KIN + 8 halves). B operands (packed
+// weights [tap][NOUT][KIN]) reach the matrix cores through LDS as well: with every wavefront loading its own
+// fragments from memory, each of a tile's four wavefronts pulled the level's whole weight set (18 - 147 KB) out of
+// the L2 again, 0.6 GB per launch at the two finest levels, and that traffic, not the MFMAs, set the length of the
+// tap loop. Now the workgroup copies one tap's weights at a time into LDS (the next tap's words travel in registers
+// while the current tap is multiplied, then go to the other of two buffers; one barrier per tap) and every wavefront
+// reads its fragments from there: a quarter of the L2 traffic, the same bank-conflict-free row layout as the patch.
+// A wavefront owns two rows of the 8 x 32 output tile = four 16-pixel row blocks; acc[m][n] is the 16 x 16 block of
+// pixels m, outputs 16n .. 16n+15.
 template <int KIN, int NOUT>
-struct ConvTapRing
+struct ConvTapStage
 {
-    static constexpr int NB = NOUT / 16;
-    static constexpr int KB = KIN / 32;
-    // three taps ahead while that costs at most 128 registers, else one (registers decide how many workgroups share a CU)
-    static constexpr int DEPTH = KB * NB <= 8 ? 3 : 1;
-    half8 b[DEPTH + 1][KB][NB];
+    static constexpr int NB    = NOUT / 16;
+    static constexpr int KB    = KIN / 32;
+    static constexpr int ROW   = KIN + kLdsChanPad;   // halves per output row of a tap in LDS
+    static constexpr int ITEMS = NOUT * KIN / 8;      // 16-byte words per tap
+    static constexpr int PER   = (ITEMS + 255) / 256;  // per thread
+    static constexpr int BUF   = NOUT * ROW;           // halves per tap buffer; the kernel provides two
+    half8 r[PER];
 };
 
+// this thread's share of tap `tap` from memory into registers
 template <int KIN, int NOUT>
-__device__ __forceinline__ void conv_taps_load(ConvTapRing<KIN, NOUT>& ring, const _Float16* __restrict__ wpack, int tap)
+__device__ __forceinline__ void conv_tap_fetch(ConvTapStage<KIN, NOUT>& st, const _Float16* __restrict__ wpack, int tap)
 {
-    using R = ConvTapRing<KIN, NOUT>;
-    const int lane = threadIdx.x & 63;
-    const _Float16* wt = wpack + (size_t)tap * NOUT * KIN + (size_t)(lane & 15) * KIN + (lane >> 4) * 8;
+    using S = ConvTapStage<KIN, NOUT>;
+    const half8* src = reinterpret_cast<const half8*>(wpack + (size_t)tap * NOUT * KIN);
 #pragma unroll
-    for (int kb = 0; kb < R::KB; ++kb)
-#pragma unroll
-        for (int n = 0; n < R::NB; ++n)
-            ring.b[tap % (R::DEPTH + 1)][kb][n] = *reinterpret_cast<const half8*>(wt + (size_t)(n * 16) * KIN + kb * 32);
+    for (int j = 0; j < S::PER; ++j)
+    {
+        const int item = threadIdx.x + 256 * j;
+        if (S::ITEMS % 256 == 0 || item < S::ITEMS) st.r[j] = src[item];
+    }
 }
 
+// ... and from the registers into a tap buffer
 template <int KIN, int NOUT>
-__device__ __forceinline__ void conv_taps_prefetch(ConvTapRing<KIN, NOUT>& ring, const _Float16* __restrict__ wpack)
+__device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT>& st, _Float16* s_tap)
 {
+    using S = ConvTapStage<KIN, NOUT>;
 #pragma unroll
-    for (int tap = 0; tap < ConvTapRing<KIN, NOUT>::DEPTH; ++tap) conv_taps_load(ring, wpack, tap);
+    for (int j = 0; j < S::PER; ++j)
+    {
+        const int item = threadIdx.x + 256 * j;
+        if (S::ITEMS % 256 == 0 || item < S::ITEMS)
+            *reinterpret_cast<half8*>(s_tap + (item / (KIN / 8)) * S::ROW + (item % (KIN / 8)) * 8) = st.r[j];
+    }
 }
 
+// Precondition: tap 0 sits in s_taps[0 .. BUF) (conv_tap_fetch + conv_tap_stage) and a barrier has passed since.
+// Every thread of the workgroup must call this (it contains barriers).
 template <int KIN, int NOUT>
-__device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, const _Float16* __restrict__ wpack,
-                                               ConvTapRing<KIN, NOUT>& ring, floatx4 (&acc)[4][NOUT / 16])
+__device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16* s_taps, const _Float16* __restrict__ wpack,
+                                               ConvTapStage<KIN, NOUT>& st, floatx4 (&acc)[4][NOUT / 16])
 {
-    using R = ConvTapRing<KIN, NOUT>;
+    using S = ConvTapStage<KIN, NOUT>;
     constexpr int ROW = KIN + kLdsChanPad;
-    constexpr int NB  = R::NB;
-    constexpr int KB  = R::KB;
+    constexpr int NB  = S::NB;
+    constexpr int KB  = S::KB;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 #pragma unroll
@@ -89,20 +104,25 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, const _F
     for (int tap = 0; tap < 9; ++tap)
     {
         const int dy = tap / 3, dx = tap - dy * 3;  // patch coordinates already include the halo
-        if (tap + R::DEPTH < 9) conv_taps_load(ring, wpack, tap + R::DEPTH);
+        if (tap + 1 < 9) conv_tap_fetch(st, wpack, tap + 1);
+        const _Float16* sb = s_taps + (tap & 1) * S::BUF;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
         {
+            half8 bfrag[NB];
+#pragma unroll
+            for (int n = 0; n < NB; ++n) bfrag[n] = *reinterpret_cast<const half8*>(sb + (n * 16 + lrow) * S::ROW + kb * 32 + lk);
 #pragma unroll
             for (int m = 0; m < 4; ++m)
             {
                 const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
                 const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
 #pragma unroll
-                for (int n = 0; n < NB; ++n)
-                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ring.b[tap % (R::DEPTH + 1)][kb][n], acc[m][n], 0, 0, 0);
+                for (int n = 0; n < NB; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[n], acc[m][n], 0, 0, 0);
             }
         }
+        if (tap + 1 < 9) conv_tap_stage(st, s_taps + ((tap + 1) & 1) * S::BUF);
+        __syncthreads();  // the next tap is in place; nobody reads this tap's buffer any more
     }
 }
 

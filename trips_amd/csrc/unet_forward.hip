@@ -58,8 +58,8 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
     const bool has_below = p.Hb > 0;
-    ConvTapRing<CIN, NPAD> ring;
-    conv_taps_prefetch(ring, p.wpack);  // in flight while the patch is assembled
+    ConvTapStage<CIN, NPAD> taps;
+    conv_tap_fetch(taps, p.wpack, 0);  // in flight while the patch is assembled
     // weights and biases of the 1x1 output convolution, rounded to fp16 like every other operand
     __shared__ float s_fw[4 * (4 + 64) + 4];
     if (p.final_out)
@@ -161,9 +161,13 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         }
     }
 
-    __syncthreads();  // patch complete
+    __syncthreads();  // patch complete; the patch of the level below is no longer needed
+    // two tap buffers for the weights, in place of the patch of the level below
+    _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;
+    conv_tap_stage(taps, s_taps);
+    __syncthreads();
     floatx4 acc[4][NB];
-    conv_taps_mfma<CIN, NPAD>(s_patch, p.wpack, ring, acc);
+    conv_taps_mfma<CIN, NPAD>(s_patch, s_taps, p.wpack, taps, acc);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
 
@@ -267,7 +271,8 @@ template <int CIN, int NPAD>
 hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
 {
     constexpr int ROW  = CIN + kLdsChanPad;
-    const size_t lds_in  = (size_t)((kConvPatchH * kConvPatchW + kBelowH * kBelowW) * ROW) * sizeof(_Float16);  // 36 or 65 KB
+    // the patch, then the patch of the level below or (later) two tap buffers of the weights, whichever is larger
+    const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW * ROW + std::max(kBelowH * kBelowW * ROW, 2 * NPAD * ROW)) * sizeof(_Float16);
     const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NPAD / 2 + kLdsChanPad) + (p.pre ? NPAD + kLdsChanPad : 0)) * sizeof(_Float16);
     const size_t lds     = std::max(lds_in, lds_out);  // up to 104 KB when the largest block saves its pre-activations
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD>),
