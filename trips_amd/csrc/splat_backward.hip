@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     constexpr int RF   = 4 + CPAD;  // floats per blend record
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
     const int lane     = threadIdx.x & 63;
-        const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
+    const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     float R[9];
     rotation_matrix(cam.V, R);
     const bool want_pose = p.d_pose != nullptr;
