@@ -83,8 +83,8 @@ struct PointProjection
     float ipx, ipy, z, size_px;
 };
 
-// `s_hist`: LDS counters, one per tile; the 2 x 2 footprint (px..px+1, py..py+1) of every layer the point is written to
-// adds one to the 1, 2 or 4 tiles it touches (px+1 and py+1 are inside the image because px < w-1 and py < h-1).
+// `s_hist`: LDS counters, one per tile; every layer the point is written to adds one to the tile of the footprint's
+// first pixel (px, py). (The footprint (px..px+1, py..py+1) lies inside the image because px < w-1 and py < h-1.)
 template <bool TRAIN>
 __device__ __forceinline__ PointProjection project_point(const ForwardParams& p, const Camera& cam, int pid, int* s_hist,
                                                          bool& not_identity, bool& bad_index)
@@ -151,13 +151,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
     {
         const int px = (int)floorf(lx), py = (int)floorf(ly);
         if (!valid(float(px), float(py), layer, radius_px)) break;
-        const int tsx = p.geom.tiles_x[layer];
-        int* bc       = s_hist + p.geom.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
-        const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
-        atomicAdd(bc, 1);
-        if (cx) atomicAdd(bc + 1, 1);
-        if (cy) atomicAdd(bc + tsx, 1);
-        if (cx && cy) atomicAdd(bc + tsx + 1, 1);
+        atomicAdd(s_hist + p.geom.bin_off[layer] + (py >> kTileShift) * p.geom.tiles_x[layer] + (px >> kTileShift), 1);
     }
     o.valid   = true;
     o.layers  = layer;
@@ -168,9 +162,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
     return o;
 }
 
-// Calls f(layer, px, py, first tile counter, tiles per row, crosses x, crosses y) for the layers a point is written
-// to. The 2 x 2 footprint (px..px+1, py..py+1) touches 1, 2 or 4 tiles; px+1 and py+1 are inside the image because
-// px < w-1 and py < h-1.
+// Calls f(px, py, counter of the tile of (px, py)) for the layers a point is written to.
 template <typename F>
 __device__ __forceinline__ void for_point_tiles(const PyramidGeom& g, const PointProjection& o, int* tile_table, F&& f)
 {
@@ -178,10 +170,7 @@ __device__ __forceinline__ void for_point_tiles(const PyramidGeom& g, const Poin
     for (int layer = 0; layer < o.layers; ++layer, lx *= 0.5f, ly *= 0.5f)
     {
         const int px = (int)floorf(lx), py = (int)floorf(ly);
-        const int tsx = g.tiles_x[layer];
-        int* bc       = tile_table + g.bin_off[layer] + (py >> kTileShift) * tsx + (px >> kTileShift);
-        const bool cx = (px & (kTile - 1)) == kTile - 1, cy = (py & (kTile - 1)) == kTile - 1;
-        f(layer, px, py, bc, tsx, cx, cy);
+        f(px, py, tile_table + g.bin_off[layer] + (py >> kTileShift) * g.tiles_x[layer] + (px >> kTileShift));
     }
 }
 
@@ -375,7 +364,7 @@ __global__ __launch_bounds__(256) void bin_column_scan_kernel(int32_t* __restric
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// One bin entry {depth bits, compact point number, px | py << 16} per (point, layer, touched tile). A workgroup walks
+// One bin entry {depth bits, compact point number, px | py << 16} per (point, layer), in the tile of (px, py). A workgroup walks
 // the records that its chunk of the points left at the compact numbers; its slots inside every bin are contiguous
 // and start at bin_start[bin] + hist[workgroup][bin].
 __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardParams p)
@@ -415,21 +404,13 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
             o.layers = __float_as_int(tail[u].z);
             const unsigned zbits = __float_as_uint(tail[u].y);
             for_point_tiles(p.geom, o, s_cur,
-                            [&](int, int px, int py, int* bc, int tsx, bool cx, bool cy)
+                            [&](int px, int py, int* bc)
                             {
-                                const uint4 e = make_uint4(zbits, (unsigned)cid, (unsigned)px | ((unsigned)py << 16), 0u);
-                                auto put      = [&](int* c)
-                                {
-                                    const int slot = atomicAdd(c, 1);
-                                    if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
-                                        p.bin_entries[slot] = e;
-                                    else
-                                        dropped += 1;
-                                };
-                                put(bc);
-                                if (cx) put(bc + 1);
-                                if (cy) put(bc + tsx);
-                                if (cx && cy) put(bc + tsx + 1);
+                                const int slot = atomicAdd(bc, 1);
+                                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
+                                    p.bin_entries[slot] = make_uint4(zbits, (unsigned)cid, (unsigned)px | ((unsigned)py << 16), 0u);
+                                else
+                                    dropped += 1;
                             });
         }
     }
@@ -444,7 +425,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
 // The workgroups after the first clear `clear_n` 16-byte words at `clear` (the per-pixel counters of the list kernels),
 // which saves a launch of its own.
 __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restrict__ bin_start, long long capacity, int NB,
-                                                          int32_t* __restrict__ slice_start, int32_t* __restrict__ bin_total,
+                                                          int32_t* __restrict__ slice_start,
                                                           int32_t* __restrict__ long_count, uint4* __restrict__ clear,
                                                           long long clear_n)
 {
@@ -471,7 +452,6 @@ __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restr
             if (last > capacity) last = capacity;
             const long long n = last > first ? last - first : 0;
             v                 = n > kSliceEntries ? (int)((n + kSliceEntries - 1) / kSliceEntries) : 0;
-            bin_total[idx]    = 0;
         }
         int inc = v;
         for (int o = 1; o < 64; o <<= 1)
@@ -493,17 +473,10 @@ __global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restr
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Calls f(local pixel index) for each of the entry's 2 x 2 pixels that lie in tile (tx, ty).
-template <typename F>
-__device__ __forceinline__ void for_corners_in_tile(const uint4& e, int tx, int ty, F&& f)
+// Index, inside its tile, of the cell (px, py) that an entry's footprint starts at.
+__device__ __forceinline__ int entry_cell(const uint4& e)
 {
-    const int px = (int)(e.z & 0xffffu), py = (int)(e.z >> 16);
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-    {
-        const int x = px + (c & 1), y = py + (c >> 1);
-        if ((x >> kTileShift) == tx && (y >> kTileShift) == ty) f(((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1)));
-    }
+    return (int)(((e.z >> 16) & (kTile - 1)) << kTileShift) | (int)(e.z & (kTile - 1));
 }
 
 // Walks entries [0, n) with the workgroup, four loads of a thread in flight together.
@@ -522,12 +495,15 @@ __device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, i
     }
 }
 
+// The keys of a tile are filed by cell: the cell (px, py) holds the points whose 2 x 2 footprint starts at that pixel,
+// so that a (point, layer) pair is written once and the four pixels it covers gather it from the cell. There is one key
+// per bin entry: the keys of a tile start where its bin entries do.
 // One workgroup per tile (blocks [0, NB)) plus one per slice of a split tile (blocks from NB on; those past the
-// number of slices the plan found return at once). Pass `SCATTER == false`: count the list length of the tile's
-// 1024 pixels in LDS and write them (plus the tile total). Pass `SCATTER == true` (after the scan of the tile
-// totals): exclusive scan of the 1024 lengths, per-pixel list starts, and the 64-bit keys (depth bits << 32 |
-// point id) into their lists. A slice adds its counts to the tile's with atomics; when it places its keys it first
-// counts its own entries per pixel again and claims that many slots of each pixel's list with one atomic.
+// number of slices the plan found return at once). Pass `SCATTER == false`: count the entries of the tile's 1024
+// cells in LDS and write the counts. Pass `SCATTER == true`: exclusive scan of the 1024 counts, per-cell list starts,
+// and the 64-bit keys (depth bits << 32 | compact point number) into their lists. A slice adds its counts to the
+// tile's with atomics; when it places its keys it first counts its own entries per cell again and claims that many
+// slots of each cell's list with one atomic.
 // (THREADS: 256 for the counting pass, whose idle workgroups for unused slices are cheaper that way; 1024 for the
 // placement pass, where two workgroups per CU with their 64 KB of LDS then make 32 wavefronts instead of 8)
 constexpr int kScatterThreads = 1024;
@@ -535,7 +511,7 @@ template <bool SCATTER, int THREADS>
 __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams p)
 {
     __shared__ int s_cnt[kTilePixels];
-    // per-pixel entries of a slice (placement pass only; one word in the counting pass, whose code below never runs)
+    // per-cell entries of a slice (placement pass only; one word in the counting pass, whose code below never runs)
     __shared__ int s_mine[SCATTER ? kTilePixels : 1];
     auto mine = [&](int i) -> int& { return s_mine[SCATTER ? i : 0]; };
     __shared__ int s_wave[THREADS / 64];
@@ -559,8 +535,6 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         bin   = lo;
         slice = e - p.slice_start[bin];
     }
-    const TileCtx tc = tile_ctx(p.geom, bin);
-    const int tx = tc.x0 >> kTileShift, ty = tc.y0 >> kTileShift;
     long long first = p.bin_start[bin];
     long long last  = p.bin_start[bin + 1];
     if (last > p.capacity) last = p.capacity;  // entries beyond the capacity were dropped by the scatter
@@ -579,9 +553,8 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         if (split && slice < 0) return;  // the slices do the counting
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
-        for_entries<THREADS>(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&s_cnt[i], 1); }); });
+        for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&s_cnt[entry_cell(e)], 1); });
         __syncthreads();
-        int sum = 0;
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
             const int c = s_cnt[i];
@@ -589,19 +562,6 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
                 counts[i] = c;
             else if (c)
                 atomicAdd(&counts[i], c);  // cleared before this kernel
-            sum += c;
-        }
-        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-        if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = sum;
-        __syncthreads();
-        if (threadIdx.x == 0)
-        {
-            int total = 0;
-            for (int w = 0; w < THREADS / 64; ++w) total += s_wave[w];
-            if (slice < 0)
-                p.bin_total[bin] = total;
-            else
-                atomicAdd(&p.bin_total[bin], total);
         }
         return;
     }
@@ -629,18 +589,18 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     __syncthreads();
     int prefix = inc - sum;
     for (int w = 0; w < wave; ++w) prefix += s_wave[w];
-    const int key_start = p.bin_key_start[bin];
+    const int key_start = p.bin_start[bin];  // one key per bin entry: the tile's keys start where its entries do
     int32_t* cursor     = p.cursor + (size_t)bin * kTilePixels;
 #pragma unroll
     for (int i = 0; i < PER; ++i)
     {
-        s_cnt[base4 + i] = key_start + prefix;  // running slot of the pixel
+        s_cnt[base4 + i] = key_start + prefix;  // running slot of the cell
         if (slice < 0)
         {
             int where = key_start + prefix;
             if (v[i] > kLongList && (long long)key_start + prefix + v[i] <= p.capacity)
             {
-                // a long list: hand its segments to the reduction pass and point the pixel at their results
+                // a long list: hand its segments to the reduction pass and point the cell at their results
                 const int nseg = (v[i] + kLongSegment - 1) / kLongSegment;
                 const int base = atomicAdd(p.long_count, nseg);
                 if (base + nseg <= p.max_long_items)
@@ -659,9 +619,9 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     unsigned dropped = 0;
     if (slice >= 0)
     {
-        // this slice's share of every pixel's list: count, then claim the slots with one atomic per pixel
+        // this slice's share of every cell's list: count, then claim the slots with one atomic per cell
         int32_t* run = p.run + (size_t)bin * kTilePixels;
-        for_entries<THREADS>(entries, n, [&](const uint4& e) { for_corners_in_tile(e, tx, ty, [&](int i) { atomicAdd(&mine(i), 1); }); });
+        for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&mine(entry_cell(e)), 1); });
         __syncthreads();
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
@@ -672,16 +632,12 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         for_entries<THREADS>(entries, n,
                     [&](const uint4& e)
                     {
-                        const u64 key = ((u64)e.x << 32) | (u64)e.y;
-                        for_corners_in_tile(e, tx, ty,
-                                            [&](int i)
-                                            {
-                                                const int slot = atomicAdd(&s_cnt[i], 1);
-                                                if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
-                                                    p.keys[slot] = key;
-                                                else
-                                                    dropped += 1;
-                                            });
+                        const u64 key  = ((u64)e.x << 32) | (u64)e.y;
+                        const int slot = atomicAdd(&s_cnt[entry_cell(e)], 1);
+                        if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
+                            p.keys[slot] = key;
+                        else
+                            dropped += 1;
                     });
         if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
         return;
@@ -689,23 +645,19 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     // Keys of a tile whose lists fit into LDS are staged there and copied out with full-line stores; the keys of
     // bigger tiles go to their lists directly (8-byte stores scattered over the tile's region).
     extern __shared__ u64 s_keys[];
-    const int tile_total = p.bin_key_start[bin + 1] - key_start;
+    const int tile_total = p.bin_start[bin + 1] - key_start;
     const bool staged    = tile_total <= kStageKeys && (long long)key_start + tile_total <= p.capacity;
     for_entries<THREADS>(entries, n,
                 [&](const uint4& e)
                 {
-                    const u64 key = ((u64)e.x << 32) | (u64)e.y;
-                    for_corners_in_tile(e, tx, ty,
-                                        [&](int i)
-                                        {
-                                            const int slot = atomicAdd(&s_cnt[i], 1);
-                                            if (staged)
-                                                s_keys[slot - key_start] = key;
-                                            else if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
-                                                p.keys[slot] = key;
-                                            else
-                                                dropped += 1;
-                                        });
+                    const u64 key  = ((u64)e.x << 32) | (u64)e.y;
+                    const int slot = atomicAdd(&s_cnt[entry_cell(e)], 1);
+                    if (staged)
+                        s_keys[slot - key_start] = key;
+                    else if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
+                        p.keys[slot] = key;
+                    else
+                        dropped += 1;
                 });
     if (staged)
     {
@@ -725,9 +677,10 @@ __device__ __forceinline__ u64 shfl16(u64 v, int src)
     return ((u64)hi << 32) | lo;
 }
 
-// The 16 smallest of keys[start, start + readable) for each of the wavefront's four 16-lane rows, ascending over
-// the row's lanes (all-ones where the list is shorter).
-__device__ __forceinline__ u64 row_top16(const u64* __restrict__ keys, long long start, int readable)
+// The 16 smallest of key_at(0 .. readable - 1) for each of the wavefront's four 16-lane rows, ascending over the row's
+// lanes (all-ones where the row has fewer keys).
+template <typename KeyAt>
+__device__ __forceinline__ u64 row_top16(KeyAt&& key_at, int readable)
 {
     const int lane = threadIdx.x & 63;
     const int sub = lane & 15, grp = lane >> 4;
@@ -740,45 +693,49 @@ __device__ __forceinline__ u64 row_top16(const u64* __restrict__ keys, long long
     maxlen             = __builtin_amdgcn_readfirstlane(maxlen);
     {
         u64 k = kInf;
-        if (sub < readable) k = keys[start + sub];
+        if (sub < readable) k = key_at(sub);
         best = row_sort16(k);
     }
     // A chunk of 16 further keys is sorted and merged only if one of them beats the current 16th; most chunks of a
     // long list are passed over, so the loop runs at the latency of its loads: four chunks are requested together
     // and the next four are in flight while these are looked at.
-    auto load4 = [&](int base, u64 (&kk)[4])
+    struct Four
     {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
+        u64 k0, k1, k2, k3;
+    };
+    auto load4 = [&](int base)
+    {
+        Four f;
+        const int i = base + sub;
+        f.k0        = i < readable ? key_at(i) : kInf;
+        f.k1        = i + 16 < readable ? key_at(i + 16) : kInf;
+        f.k2        = i + 32 < readable ? key_at(i + 32) : kInf;
+        f.k3        = i + 48 < readable ? key_at(i + 48) : kInf;
+        return f;
+    };
+    auto consider = [&](u64 k)
+    {
+        const u64 worst = shfl16(best, 15);
+        const bool need = k < worst;
+        if (__ballot(need) & grp_mask)
         {
-            const int i = base + 16 * j + sub;
-            kk[j]       = i < readable ? keys[start + i] : kInf;
+            k           = row_sort16(k);
+            const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
+            best        = best < r ? best : r;
+            best        = row_merge16(best);
         }
     };
     if (maxlen > 16)
     {
-        u64 cur[4], nxt[4];
-        load4(16, cur);
+        Four cur = load4(16), nxt = cur;
         for (int base = 16; base < maxlen; base += 64)
         {
-            if (base + 64 < maxlen) load4(base + 64, nxt);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-            {
-                if (base + 16 * j >= maxlen) break;
-                u64 k           = cur[j];
-                const u64 worst = shfl16(best, 15);
-                const bool need = k < worst;
-                if (__ballot(need) & grp_mask)
-                {
-                    k           = row_sort16(k);
-                    const u64 r = row_xor_u64<15>(k);  // reversed: lane i sees the (15-i)-th smallest new key
-                    best        = best < r ? best : r;
-                    best        = row_merge16(best);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
+            if (base + 64 < maxlen) nxt = load4(base + 64);
+            consider(cur.k0);
+            if (base + 16 < maxlen) consider(cur.k1);
+            if (base + 32 < maxlen) consider(cur.k2);
+            if (base + 48 < maxlen) consider(cur.k3);
+            cur = nxt;
         }
     }
     return best;
@@ -797,18 +754,29 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
         int2 seg       = make_int2(0, 0);
         if (item < n) seg = p.long_items[item];
         if (seg.x < 0 || seg.y < 0 || seg.y > kLongSegment || (long long)seg.x + seg.y > p.capacity) seg = make_int2(0, 0);
-        const u64 best = row_top16(p.keys, seg.x, seg.y);
+        const u64* src = p.keys + seg.x;
+        const u64 best = row_top16([&](int i) { return src[i]; }, seg.y);
         if (item < n) p.cand[(size_t)item * 16 + (lane & 15)] = best;
     }
 }
 
-// Top-16 of each pixel list by key, then the alpha blend, for 64 / ROW consecutive pixels starting at `pix_first`:
+// A pixel's list is the union of the lists of the four cells whose 2 x 2 footprints cover it: (x-1, y-1), (x, y-1),
+// (x-1, y), (x, y) (CountAndCollectTiled adds every point to the four pixels of its footprint,
+// RenderForward.cu:300-366; here a point is filed once, under its footprint's first pixel, and the pixels gather).
+// Top-16 of each pixel's union by key, then the alpha blend, for 64 / ROW consecutive pixels starting at `pix_first`:
 // ROW = 16 lanes per pixel (one DPP row; lists of any length stream through in chunks of 16), or ROW = 8 when no
-// list of the group is longer than 8 (two thirds of the pixels of a typical view have at most 4 entries: half the
+// pixel of the group has more than 8 entries (two thirds of the pixels of a typical view have at most 4: half the
 // lanes of a 16-lane row would idle through every instruction).
+// First key (negative: a long list, reduced to candidates) and number of readable keys of the four cells of a pixel.
+struct PixelCells
+{
+    int s0, s1, s2, s3;
+    int r0, r1, r2, r3;
+};
+
 template <int C, bool TRAIN, int ROW>
 __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const TileCtx& tc, float* img, int pix_first,
-                                                bool group_in_range, int len_in, int start_in, int readable_in)
+                                                bool group_in_range, const PixelCells cells)
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int RF   = 4 + CPAD;  // floats per blend record
@@ -824,34 +792,40 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     const bool in_range = group_in_range;
     const bool live     = in_range && gx < lw && gy < lh;  // false for the padding of partial tiles
 
-    // length, first key and number of keys actually written (the key storage may have ended inside the list) of this
-    // lane's list: the caller has them for the whole group
-    const int len = live ? len_in : 0;
-    int start     = live ? start_in : 0;
-    int readable  = live ? readable_in : 0;
+    // position i of the concatenation of the four cell lists lies in cell (i >= o1) + (i >= o2) + (i >= o3)
+    const int o1 = cells.r0, o2 = o1 + cells.r1, o3 = o2 + cells.r2;
+    const int total = live ? o3 + cells.r3 : 0;
 
     const u64 kInf = ~0ull;
     u64 best       = kInf;
     if (ROW == 8)
     {
-        if (sub < readable) best = p.keys[(unsigned)(start + sub)];
+        // at most 8 keys: none of the cells has a long list
+        // (sums of steps rather than a chain of selects: the compiler turns the chain into a table in memory)
+        const int b0 = cells.s0, b1 = cells.s1 - o1, b2 = cells.s2 - o2, b3 = cells.s3 - o3;
+        const int base = b0 + (sub >= o1 ? b1 - b0 : 0) + (sub >= o2 ? b2 - b1 : 0) + (sub >= o3 ? b3 - b2 : 0);
+        if (sub < total) best = p.keys[(unsigned)(base + sub)];
         best = half_sort8(best);
     }
     else
     {
-        const u64* src = p.keys;
-        if (start < 0)
-        {
-            // a long list: the reduction pass left the 16 smallest keys of each of its segments
-            src      = p.cand;
-            start    = (-1 - start) * 16;
-            readable = ((len + kLongSegment - 1) / kLongSegment) * 16;
-        }
-        best = row_top16(src, start, readable);
+        // the candidates that the reduction pass left for long lists are addressed relative to the keys as well
+        const long long cand_off = ((long long)(intptr_t)p.cand - (long long)(intptr_t)p.keys) / (long long)sizeof(u64);
+        auto first_key = [&](int s) -> long long { return s >= 0 ? (long long)s : cand_off + (long long)(-1 - s) * 16; };
+        const long long b0 = first_key(cells.s0), b1 = first_key(cells.s1) - o1, b2 = first_key(cells.s2) - o2,
+                        b3 = first_key(cells.s3) - o3;
+        const long long d1 = b1 - b0, d2 = b2 - b1, d3 = b3 - b2;
+        best = row_top16(
+            [&](int i)
+            {
+                const long long b = b0 + (i >= o1 ? d1 : 0ll) + (i >= o2 ? d2 : 0ll) + (i >= o3 ? d3 : 0ll);
+                return p.keys[b + i];
+            },
+            total);
     }
 
     // ---- blend (RenderForward.cu:820-1048) ----
-    const int n    = min(min(len, readable), K);
+    const int n    = min(total, K);
     const bool has = live && sub < n;
     const int cid  = (int)(unsigned)(best & 0xffffffffull);  // compact number of the entry's point
 
@@ -935,11 +909,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     // saved state, also for padding pixels (empty) so that every row of the tables is defined
     if (TRAIN && in_range)
     {
-        if (sub == 0)
-        {
-            p.retained[pix] = live ? ret : 0;
-            p.lengths[pix]  = live ? len : 0;
-        }
+        if (sub == 0) p.retained[pix] = live ? ret : 0;
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
         // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
         if (has && sub < ret)
@@ -957,7 +927,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     }
 }
 
-// One wavefront = eight consecutive pixels: all at once in 8-lane rows when none of their lists is longer than 8,
+// One wavefront = eight consecutive pixels: all at once in 8-lane rows when none of them has more than 8 entries,
 // else four and four in 16-lane rows.
 template <int C, bool TRAIN>
 __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
@@ -972,31 +942,54 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     // the eight pixels share a tile: its layer and position are found once per wavefront, on the scalar unit
     const TileCtx tc = tile_ctx(p.geom, pix_first >> (2 * kTileShift));
     float* const img = p.image[tc.layer];
-    // longest list of the eight pixels (lists that ran past the key storage count with what was written)
-    int my_len = 0, my_start = 0, my_read = 0;  // lanes 0..7: one pixel of the group each
-    if (lane < 8 && group_in_range)
+    // The eight pixels (gx0 .. gx0 + 7, gy) gather from the cells (gx0 - 1 .. gx0 + 7) x (gy - 1, gy): lanes 0..8 read
+    // length and first key of the upper row of cells, lanes 9..17 those of the lower row; pixel g takes the cells of
+    // lanes g, g + 1, g + 9, g + 10. Cells outside the layer, and the last row and column (no footprint starts there),
+    // are empty.
+    int c_len = 0, c_start = 0, c_read = 0;
+    if (lane < 18 && group_in_range)
     {
-        const int pix = pix_first + lane;
-        my_len        = p.counts[pix];  // 0 for the padding of partial tiles
-        my_start      = p.cursor[pix];  // negative: a long list, reduced to candidates by long_list_reduce_kernel
-        my_read       = my_len;
-        if (my_start >= 0 && (long long)my_start + my_len > p.capacity) my_read = (int)max(0ll, p.capacity - my_start);
+        const int lower = lane >= 9 ? 1 : 0;
+        const int cx    = tc.x0 + (pix_first & (kTile - 1)) - 1 + (lane - 9 * lower);
+        const int cy    = tc.y0 + ((pix_first >> kTileShift) & (kTile - 1)) - 1 + lower;
+        if (cx >= 0 && cy >= 0 && cx < tc.w - 1 && cy < tc.h - 1)
+        {
+            const int bin  = tc.bin + ((cx - tc.x0) >> kTileShift) + ((cy - tc.y0) >> kTileShift) * tc.tiles_x;  // shifts round down
+            const int cell = (bin << (2 * kTileShift)) | ((cy & (kTile - 1)) << kTileShift) | (cx & (kTile - 1));
+            c_len          = p.counts[cell];
+            c_start        = p.cursor[cell];  // negative: a long list, reduced to candidates by long_list_reduce_kernel
+            // keys actually there: the key storage may have ended inside the list
+            if (c_start < 0)
+                c_read = ((c_len + kLongSegment - 1) / kLongSegment) * 16;
+            else
+                c_read = (int)max(0ll, min((long long)c_len, p.capacity - c_start));
+        }
     }
-    int len8 = my_read;
-    len8 = max(len8, __shfl_xor(len8, 1));
-    len8 = max(len8, __shfl_xor(len8, 2));
-    len8 = max(len8, __shfl_xor(len8, 4));
-    len8 = __builtin_amdgcn_readfirstlane(len8);
-    // the rows take their pixel's length and list start from these lanes: no second memory round trip
-    if (len8 <= 8)
-        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 3), __shfl(my_start, lane >> 3),
-                                     __shfl(my_read, lane >> 3));
+    int tot8 = c_read + __shfl_down(c_read, 1) + __shfl_down(c_read, 9) + __shfl_down(c_read, 10);
+    if (TRAIN)
+    {
+        const int len = c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 9) + __shfl_down(c_len, 10);
+        if (lane < 8 && group_in_range) p.lengths[pix_first + lane] = len;  // 0 for the padding of partial tiles
+    }
+    if (lane >= 8) tot8 = 0;
+    tot8 = max(tot8, __shfl_xor(tot8, 1));
+    tot8 = max(tot8, __shfl_xor(tot8, 2));
+    tot8 = max(tot8, __shfl_xor(tot8, 4));
+    tot8 = __builtin_amdgcn_readfirstlane(tot8);
+    // the rows take their cells' list starts and lengths from these lanes: no second memory round trip
+    auto cells_of = [&](int g)
+    {
+        PixelCells c;
+        c.s0 = __shfl(c_start, g), c.s1 = __shfl(c_start, g + 1), c.s2 = __shfl(c_start, g + 9), c.s3 = __shfl(c_start, g + 10);
+        c.r0 = __shfl(c_read, g), c.r1 = __shfl(c_read, g + 1), c.r2 = __shfl(c_read, g + 9), c.r3 = __shfl(c_read, g + 10);
+        return c;
+    };
+    if (tot8 <= 8)
+        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, cells_of(lane >> 3));
     else
     {
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, __shfl(my_len, lane >> 4), __shfl(my_start, lane >> 4),
-                                      __shfl(my_read, lane >> 4));
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, __shfl(my_len, 4 + (lane >> 4)),
-                                      __shfl(my_start, 4 + (lane >> 4)), __shfl(my_read, 4 + (lane >> 4)));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, cells_of(lane >> 4));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, cells_of(4 + (lane >> 4)));
     }
 }
 
@@ -1037,7 +1030,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         ProfScope ps(prof, "bin_scan", stream);
         hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + kScanCols - 1) / kScanCols), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
         hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_count, p.bin_start,
-                           (int32_t*)nullptr, NB, (unsigned long long*)nullptr);
+                           (int32_t*)nullptr, NB, &p.header->n_entries);
     }
     {
         ProfScope ps(prof, "bin_scatter", stream);
@@ -1051,13 +1044,8 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         // counts and run are neighbours in the workspace: cleared together, by the workgroups behind the planning one
         const long long quads = 2ll * NB * kTilePixels / 4;
         hipLaunchKernelGGL(slice_plan_kernel, dim3(1 + (unsigned)std::min<long long>((quads + 1023) / 1024, 1024)), dim3(1024), 0, stream,
-                           p.bin_start, p.capacity, NB, p.slice_start, p.bin_total, p.long_count, reinterpret_cast<uint4*>(p.counts), quads);
+                           p.bin_start, p.capacity, NB, p.slice_start, p.long_count, reinterpret_cast<uint4*>(p.counts), quads);
         hipLaunchKernelGGL((tile_lists_kernel<false, 256>), dim3(NB + max_slices), dim3(256), 0, stream, p);
-    }
-    {
-        ProfScope ps(prof, "tile_scan", stream);
-        hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_total, p.bin_key_start,
-                           (int32_t*)nullptr, NB, &p.header->n_entries);
     }
     {
         ProfScope ps(prof, "tile_scatter", stream);

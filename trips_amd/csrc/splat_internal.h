@@ -166,6 +166,7 @@ __device__ inline int pix_index_mul24(const PyramidGeom& g, int layer, int x, in
 struct TileCtx
 {
     int layer, w, h, x0, y0;
+    int bin, tiles_x;  // the tile's number and the tile columns of its layer
 };
 
 // `bin` must be the same for the whole wavefront and come out of a scalar register (readfirstlane): the layer search
@@ -197,6 +198,8 @@ __device__ __forceinline__ TileCtx tile_ctx(const PyramidGeom& g, int bin)
     c.h     = h;
     c.x0    = (int)(tx << kTileShift);
     c.y0    = (int)(ty << kTileShift);
+    c.bin     = bin;
+    c.tiles_x = tsx;
     return c;
 }
 
@@ -204,7 +207,7 @@ __device__ __forceinline__ TileCtx tile_ctx(const PyramidGeom& g, int bin)
 struct ViewHeader
 {
     unsigned long long n_valid;     // points that passed the validity test
-    unsigned long long n_entries;   // E: total list entries (from the scan)
+    unsigned long long n_entries;   // (point, layer) pairs filed (from the scan); each is in four pixel lists: E = 4 x
     unsigned long long overflow;    // entries dropped because the list storage was too small
     unsigned long long retained;    // R: sum of the retained entries (filled by the counters query)
     unsigned long long not_identity;  // some point's descriptor column differs from its own index
@@ -243,9 +246,9 @@ struct WorkspaceLayout
 {
     size_t chunk_valid;   // int32 [G]  valid points of every chunk of the binning kernels
     size_t prec;         // float4 [N]         point records, when there is no saved state to hold them
-    size_t counts;       // int32 [Pi]   list length per pixel
-    size_t cursor;       // int32 [Pi]   first key of each pixel's list
-    size_t run;          // int32 [Pi]   keys of a pixel already claimed by slices of a split tile (zeroed per view)
+    size_t counts;       // int32 [Pi]   list length per cell (the points whose 2 x 2 footprint starts at that pixel)
+    size_t cursor;       // int32 [Pi]   first key of each cell's list (-1 - first candidate row for a long list)
+    size_t run;          // int32 [Pi]   keys of a cell already claimed by slices of a split tile (zeroed per view)
     size_t slice_start;  // int32 [NB+1] exclusive scan of the slices of split tiles (0 for a tile that is not split)
     size_t long_count;   // int32 [1]    segments of long lists handed out so far
     size_t long_items;   // int2  [max_long_items] {first key, number of keys} of each segment of a long list
@@ -254,11 +257,9 @@ struct WorkspaceLayout
     size_t bin_count;    // int32 [NB]   bin entries per tile
     size_t bin_start;    // int32 [NB+1] exclusive scan of bin_count
     size_t bin_hist;     // int32 [G, NB] bin entries per (workgroup, tile), then its column-wise exclusive prefix
-    size_t bin_total;    // int32 [NB]   list entries per tile
-    size_t bin_key_start;  // int32 [NB+1] exclusive scan of bin_total
-    size_t bin_entries;  // uint4 [capacity] {depth bits, point id, px | py << 16, -}
-    size_t keys;         // uint64 [capacity]
-    size_t capacity;     // entries
+    size_t bin_entries;  // uint4 [capacity] {depth bits, compact point number, px | py << 16, -}, one per (point, layer), by tile
+    size_t keys;         // uint64 [capacity] depth bits << 32 | compact point number, by cell
+    size_t capacity;     // (point, layer) pairs
     size_t bytes;
 };
 
@@ -295,8 +296,6 @@ struct ForwardParams
     int32_t* bin_start;
     int32_t* bin_hist;
     int32_t bin_groups, points_per_block;
-    int32_t* bin_total;
-    int32_t* bin_key_start;
     int32_t* run;
     int32_t* slice_start;
     int32_t* long_count;

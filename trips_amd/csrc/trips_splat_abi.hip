@@ -223,7 +223,8 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     WorkspaceLayout w;
     const size_t N = (size_t)d.num_points, NB = (size_t)g.bin_off[d.num_layers], P = NB * kTilePixels;
-    w.capacity     = d.max_list_entries > 0 ? (size_t)d.max_list_entries : 4 * N * (size_t)d.num_layers;
+    // a (point, layer) pair is filed once and appears in the lists of the four pixels of its footprint
+    w.capacity     = d.max_list_entries > 0 ? ((size_t)d.max_list_entries + 3) / 4 : N * (size_t)d.num_layers;
     size_t o       = 0;
     // status header (overflow flag of the whole call), then for eval mode, which has no saved state to live
     // in, the per-view counters and the per-point records
@@ -256,10 +257,6 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256((NB + 1) * sizeof(int32_t));
     w.bin_hist = o;
     o += align256((size_t)kBinGroups * NB * sizeof(int32_t));
-    w.bin_total = o;
-    o += align256(NB * sizeof(int32_t));
-    w.bin_key_start = o;
-    o += align256((NB + 1) * sizeof(int32_t));
     w.bin_entries = o;
     o += align256(w.capacity * sizeof(uint4));
     w.keys = o;
@@ -429,8 +426,6 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
         p.bin_hist   = reinterpret_cast<int32_t*>(ws + wl.bin_hist);
         p.bin_groups = kBinGroups;
         p.points_per_block = (d.num_points + kBinGroups - 1) / kBinGroups;
-        p.bin_total  = reinterpret_cast<int32_t*>(ws + wl.bin_total);
-        p.bin_key_start = reinterpret_cast<int32_t*>(ws + wl.bin_key_start);
         p.run         = reinterpret_cast<int32_t*>(ws + wl.run);
         p.slice_start = reinterpret_cast<int32_t*>(ws + wl.slice_start);
         p.long_count  = reinterpret_cast<int32_t*>(ws + wl.long_count);
@@ -582,7 +577,7 @@ int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
     e = hipStreamSynchronize(stream);
     if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
     if (h.bad_index) return fail(TRIPS_ERR_INVALID_ARG, "index holds values outside [0, num_texels): those points were left out");
-    if (h.overflow) return fail(TRIPS_ERR_LIST_OVERFLOW, "%llu list entries dropped: max_list_entries too small", h.overflow);
+    if (h.overflow) return fail(TRIPS_ERR_LIST_OVERFLOW, "%llu list entries dropped: max_list_entries too small", 4 * h.overflow);
     return TRIPS_OK;
 }
 
@@ -609,7 +604,7 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
     e = hipStreamSynchronize(stream);
     if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
     counters[0] = (int64_t)h.n_valid;
-    counters[1] = (int64_t)h.n_entries;
+    counters[1] = (int64_t)(4 * h.n_entries);  // the header counts (point, layer) pairs, each in four pixel lists
     counters[2] = (int64_t)h.retained;
     counters[3] = (int64_t)P;
     return TRIPS_OK;
