@@ -500,8 +500,8 @@ __device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, i
 // per bin entry: the keys of a tile start where its bin entries do.
 // One workgroup per tile (blocks [0, NB)) plus one per slice of a split tile (blocks from NB on; those past the
 // number of slices the plan found return at once). Pass `SCATTER == false`: count the entries of the tile's 1024
-// cells in LDS and write the counts. Pass `SCATTER == true`: exclusive scan of the 1024 counts, per-cell list starts,
-// and the 64-bit keys (depth bits << 32 | compact point number) into their lists. A slice adds its counts to the
+// cells in LDS and write the counts (split tiles only). Pass `SCATTER == true`: the counts of a tile that is not
+// split, then the exclusive scan of the 1024 counts, per-cell list starts, and the 64-bit keys (depth bits << 32 | compact point number) into their lists. A slice adds its counts to the
 // tile's with atomics; when it places its keys it first counts its own entries per cell again and claims that many
 // slots of each cell's list with one atomic.
 // (THREADS: 256 for the counting pass, whose idle workgroups for unused slices are cheaper that way; 1024 for the
@@ -550,7 +550,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
 
     if (!SCATTER)
     {
-        if (split && slice < 0) return;  // the slices do the counting
+        if (slice < 0) return;  // the slices count for a split tile; any other tile is counted where its keys are placed
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
         for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&s_cnt[entry_cell(e)], 1); });
@@ -558,10 +558,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
             const int c = s_cnt[i];
-            if (slice < 0)
-                counts[i] = c;
-            else if (c)
-                atomicAdd(&counts[i], c);  // cleared before this kernel
+            if (c) atomicAdd(&counts[i], c);  // cleared before this kernel
         }
         return;
     }
@@ -570,10 +567,21 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     constexpr int PER = kTilePixels / THREADS;
     const int base4   = threadIdx.x * PER;
     int v[PER], sum = 0;
+    if (!split)
+    {
+        // count here (the entries come from the L2 when they are read again for the placement)
+        for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
+        __syncthreads();
+        for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&s_cnt[entry_cell(e)], 1); });
+        __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < PER; ++i)
     {
-        v[i] = counts[base4 + i];
+        if (split)
+            v[i] = counts[base4 + i];
+        else
+            counts[base4 + i] = v[i] = s_cnt[base4 + i];  // (the slots that this thread overwrites with the list starts below)
         sum += v[i];
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
