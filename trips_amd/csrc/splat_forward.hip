@@ -174,9 +174,9 @@ __device__ __forceinline__ void for_point_tiles(const PyramidGeom& g, const Poin
     }
 }
 
-// A workgroup of the two binning kernels owns one contiguous chunk of points and walks it 1024 points at a time. The
-// valid points of the chunk are numbered in point order from the chunk's first point number on ("compact numbers":
-// cid = chunk begin + rank among the chunk's valid points; per step a ballot per wavefront and one exchange of the 16
+// A workgroup of the two binning kernels owns one contiguous chunk of points and walks it one point per thread at a
+// time. The valid points of the chunk are numbered in point order from the chunk's first point number on ("compact numbers":
+// cid = chunk begin + rank among the chunk's valid points; per step a ballot per wavefront and one exchange of the
 // wavefront counts through LDS). The numbers grow with the point id, so a sort key built from them orders like one
 // built from point ids; the records written at them are dense from the start of every chunk (whole lines, nothing
 // for culled points).
@@ -187,9 +187,9 @@ __device__ __forceinline__ void chunk_point_range(const ForwardParams& p, int& b
 }
 
 // Projection, validity, layer selection; the records of the valid points at their compact numbers; LDS histogram of
-// the tiles that the 2 x 2 footprints of this workgroup's points touch.
+// the tiles that this workgroup's points fall into.
 template <int C, bool TRAIN>
-__global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardParams p)
+__global__ __launch_bounds__(kBinThreads, 6) void project_bin_kernel(const ForwardParams p)
 {
     constexpr int CPAD  = (C + 3) & ~3;
     constexpr int NREC  = 1 + CPAD / 4;  // float4 per blend record
