@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 8 
 // ---------------------------------------------------------------------------------------------------------
 // Pass 2: per point.
 template <int C>
-__global__ __launch_bounds__(256) void backward_points_kernel(const BackwardParams p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 : 1))) void backward_points_kernel(const BackwardParams p)
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int KIN  = entry_row_entries(CPAD);

@@ -189,7 +189,7 @@ __device__ __forceinline__ void chunk_point_range(const ForwardParams& p, int& b
 // Projection, validity, layer selection; the records of the valid points at their compact numbers; LDS histogram of
 // the tiles that this workgroup's points fall into.
 template <int C, bool TRAIN>
-__global__ __launch_bounds__(kBinThreads, 6) void project_bin_kernel(const ForwardParams p)
+__global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardParams p)
 {
     constexpr int CPAD  = (C + 3) & ~3;
     constexpr int NREC  = 1 + CPAD / 4;  // float4 per blend record

@@ -111,10 +111,10 @@ constexpr int kPointRecordFloats = 4;
 constexpr int kTileShift  = 5;
 constexpr int kTile       = 1 << kTileShift;
 constexpr int kTilePixels = kTile * kTile;
-// The two binning kernels run at the latency of their loads and LDS atomics: three workgroups of 512 threads per CU
-// (24 wavefronts, the projection kernel held to 80 registers) are faster than one of 1024 (16 wavefronts).
-constexpr int kBinThreads = 512;    // workgroup size of the two binning kernels
-constexpr int kBinGroups  = 768;    // workgroups (= contiguous chunks of points) of the two binning kernels
+// (One workgroup of 1024 threads per CU: three of 512, with the projection kernel held to 80 registers, measured 1 %
+// slower over the step: the histogram matrix grows with the number of workgroups.)
+constexpr int kBinThreads = 1024;   // workgroup size of the two binning kernels
+constexpr int kBinGroups  = 256;    // workgroups (= contiguous chunks of points) of the two binning kernels
 constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
 // bin entries of a tile above which the tile is split into slices of that many entries, one workgroup each
 constexpr int kSliceEntries = 8192;
