@@ -66,7 +66,7 @@ __device__ __forceinline__ double wave_sum(double v)
 
 
 // ---------------------------------------------------------------------------------------------------------
-// Pass 1: per pixel row. Writes the pixel's 128-byte row {g[0..Cpad), {dL/dalpha_j, T_j alpha_j} for j < kRowEntries}.
+// Pass 1: per pixel row. Writes the pixel's exchange row {g[0..Cpad), {dL/dalpha_j, T_j alpha_j} for j < entry_row_entries}.
 // 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
 // than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
 template <int C, int ROW>
@@ -168,11 +168,11 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
 #pragma unroll
         for (int c = 0; c < C; ++c) acc_bg[c] += T_after * g[c];
     }
-    // For pass 2, one 128-byte row per pixel: the pixel's image gradient (a point finds all channels and its entry in
-    // one line) followed by {dL/dalpha, T alpha} of the first kRowEntries retained entries; the few entries beyond that
-    // go to a table of their own.
+    // For pass 2, one row of 64 bytes (128 above 8 channels) per pixel: the pixel's image gradient (a point finds all
+    // channels and its entry in one line) followed by {dL/dalpha, T alpha} of the first entry_row_entries retained
+    // entries; the entries beyond that go to a table of their own.
     constexpr int KIN = entry_row_entries(CPAD);
-    float* row        = p.entry_grad + ((size_t)(unsigned)pix << 5);
+    float* row        = p.entry_grad + (size_t)(unsigned)pix * entry_row_floats(CPAD);
     if (has)
     {
         if (sub < KIN)
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
                 const int gx = px + (corner & 1), gy = py + (corner >> 1);
                 const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
                 const bool on      = j != 0xFFu;
-                const float* row   = p.entry_grad + ((size_t)pix << 5);  // the pixel's 128-byte row
+                const float* row   = p.entry_grad + (size_t)pix * entry_row_floats(CPAD);  // the pixel's row
                 const unsigned jj  = j & 15u;
                 const float2* src2 = jj < (unsigned)KIN ? reinterpret_cast<const float2*>(row + CPAD) + jj
                                                         : reinterpret_cast<const float2*>(p.entry_over) + ((size_t)pix * (16 - KIN) + (jj - KIN));

@@ -274,7 +274,7 @@ BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const
     const size_t P = (size_t)g.bin_off[d.num_layers] * kTilePixels;
     size_t o       = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
     w.entry_grad   = o;
-    o += align256(P * 128);
+    o += align256(P * (size_t)entry_row_floats((d.num_channels + 3) & ~3) * sizeof(float));
     w.entry_over = o;
     o += align256(P * (size_t)(16 - entry_row_entries((d.num_channels + 3) & ~3)) * 2 * sizeof(float));
     w.bytes = o;
