@@ -83,11 +83,28 @@ struct PointProjection
     float ipx, ipy, z, size_px;
 };
 
+// What the projection reads of a point in point order (fetched one step ahead of its use).
+struct PointInputs
+{
+    int tex;  // descriptor column
+    float4 pos;
+    float raw_size;
+};
+
+__device__ __forceinline__ PointInputs load_point(const ForwardParams& p, int pid)
+{
+    PointInputs in;
+    in.tex      = p.index[pid];
+    in.pos      = p.position[pid];
+    in.raw_size = p.point_size[pid];
+    return in;
+}
+
 // `s_hist`: LDS counters, one per tile; every layer the point is written to adds one to the tile of the footprint's
 // first pixel (px, py). (The footprint (px..px+1, py..py+1) lies inside the image because px < w-1 and py < h-1.)
 template <bool TRAIN>
-__device__ __forceinline__ PointProjection project_point(const ForwardParams& p, const Camera& cam, int pid, int* s_hist,
-                                                         bool& not_identity, bool& bad_index)
+__device__ __forceinline__ PointProjection project_point(const ForwardParams& p, const Camera& cam, int pid, const PointInputs& in,
+                                                         int* s_hist, bool& not_identity, bool& bad_index)
 {
     PointProjection o;
     o.valid  = false;
@@ -97,7 +114,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
     o.size_px = 0.f;
     const int L = p.num_layers;
     bool skip   = false;
-    o.tex       = p.index[pid];
+    o.tex       = in.tex;
     not_identity |= (o.tex != pid);
     if ((unsigned)o.tex >= (unsigned)p.num_texels)
     {
@@ -116,7 +133,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
         if (p.dropout[pid] == 1.f) skip = true;
     }
     if (skip) return o;
-    float4 pos = p.position[pid];
+    float4 pos = in.pos;
     if (p.displacement)
     {
         const float* dsp = p.displacement + (size_t)pid * 3;
@@ -124,7 +141,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
         pos.y += dsp[1];
         pos.z += dsp[2];
     }
-    const float size    = softplus(p.point_size[pid]);
+    const float size    = softplus(in.raw_size);
     const Projected pr  = project(cam, pos.x, pos.y, pos.z);
     const float z       = pr.z;
     float radius_px     = pr.scale * pos.w / z;
@@ -209,12 +226,30 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int next       = begin;  // workgroup-uniform: compact number of the chunk's next valid point
     int step       = 0;
+    // the loads of the next step's points are in flight while this step's are projected
+    PointInputs nxt;
+    nxt.tex = 0, nxt.pos = make_float4(0.f, 0.f, 0.f, 0.f), nxt.raw_size = 0.f;
+    if (begin + (int)threadIdx.x < end) nxt = load_point(p, begin + (int)threadIdx.x);
     for (int base = begin; base < end; base += kBinThreads, step ^= 1)
     {
-        const int pid = base + threadIdx.x;
+        const int pid        = base + threadIdx.x;
+        const PointInputs in = nxt;
+        if (pid + kBinThreads < end) nxt = load_point(p, pid + kBinThreads);
+        // the descriptor of the point is requested before it is known whether the point is visible: the loads then run
+        // beside the projection instead of after it
+        float conf = 0.f;
+        float d[CPAD];
+#pragma unroll
+        for (int c = 0; c < CPAD; ++c) d[c] = 0.f;
+        if (pid < end && (unsigned)in.tex < (unsigned)p.num_texels)
+        {
+            conf = p.confidence[in.tex];
+#pragma unroll
+            for (int c = 0; c < C; ++c) d[c] = p.texture[(size_t)c * p.num_texels + in.tex];
+        }
         PointProjection o;
         o.valid = false;
-        if (pid < end) o = project_point<TRAIN>(p, cam, pid, s_hist, not_identity, bad_index);
+        if (pid < end) o = project_point<TRAIN>(p, cam, pid, in, s_hist, not_identity, bad_index);
         const unsigned long long vm = __ballot(o.valid);
         if (lane == 0) s_valid[step][wave] = (int)__popcll(vm);
         __syncthreads();
@@ -234,10 +269,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
 
         // record for the blend (and the pixel pass of the backward)
         float4 recv[NREC];
-        recv[0] = make_float4(o.ipx, o.ipy, encode_size_field(o.size_px, L), p.confidence[o.tex]);
-        float d[CPAD];
-#pragma unroll
-        for (int c = 0; c < CPAD; ++c) d[c] = c < C ? p.texture[(size_t)c * p.num_texels + o.tex] : 0.f;
+        recv[0] = make_float4(o.ipx, o.ipy, encode_size_field(o.size_px, L), conf);
 #pragma unroll
         for (int q = 0; q < CPAD / 4; ++q) recv[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
         float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)cid * p.rec_floats);
@@ -245,7 +277,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         for (int q = 0; q < NREC; ++q) rec[q] = recv[q];
         // point record: depth and layers for the scatter pass; softplus' and the size for the backward
         reinterpret_cast<float4*>(p.prec)[cid] =
-            make_float4(TRAIN ? softplus_backward(p.point_size[pid]) : 0.f, o.z, __int_as_float(o.layers), o.size_px);
+            make_float4(TRAIN ? softplus_backward(in.raw_size) : 0.f, o.z, __int_as_float(o.layers), o.size_px);
         if (TRAIN)
         {
             p.pid_of[cid] = pid;
