@@ -30,16 +30,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "af9e7cecab99fa6802495a589a383268a0aa691ae978db7f98e4e4ad999bfb44"
-PMC_KIB_DEFAULT_WORKLOAD = {  # kernel: (FETCH_SIZE, WRITE_SIZE)
-    "project_bin": (129624, 271874),
-    "bin_scatter": (88421, 195765),
-    "tile_count": (51862, 12445),
-    "tile_scatter": (83819, 464240),
-    "sort_blend": (395422, 425570),
-    "backward_pixels": (505826, 163895),
-    "backward_points": (1040711, 234887),
-    "adam_fused": (582966, 792823),
+PMC_SOURCES_SHA256 = "65468a1844737f5fddf9488656588c43326a26457a5987d81cf449e8b8262a8b"
+PMC_KIB_DEFAULT_WORKLOAD = {
+    "project_bin": (129129, 271476),
+    "bin_scatter": (87944, 186054),
+    "tile_count": (26200, 2296),
+    "tile_scatter": (70420, 115408),
+    "sort_blend": (334593, 417430),
+    "backward_pixels": (498577, 165610),
+    "backward_points": (1045046, 234887),
+    "adam_fused": (582964, 792823),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
