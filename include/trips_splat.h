@@ -86,7 +86,8 @@ typedef struct TripsSplatDesc {
     float dist_cutoff;
     int32_t viewer_only; /* 1: cull points whose confidence < stability_cutoff_value (RenderForward.cu:122-130,226-230) */
     float stability_cutoff_value;
-    /* capacity, in entries, of the per-pixel list storage of ONE view; 0 = worst case 4*N*L */
+    /* capacity, in list entries (a point covers four pixels per layer it is written to), of the list storage of ONE
+     * view; 0 = worst case 4*N*L. The storage itself keeps one key per four entries. */
     int64_t max_list_entries;
     TripsView views[TRIPS_MAX_VIEWS];
 } TripsSplatDesc;
