@@ -275,6 +275,30 @@ def test_tight_cluster_long_lists_and_split_tiles(oracle):
         small.ctx.check(small.workspace)
 
 
+def test_footprints_on_tile_and_image_borders_with_equal_depths(oracle):
+    """A dense grid of points in a plane that faces the camera: footprints start at every pixel, also at the last
+    column and row of a 32-pixel tile (their other pixels belong to the neighbouring tiles) and at the last pixels of
+    every layer (a footprint that would leave the image is culled), and all depths are equal, so the order of every
+    list is decided by the point ids alone, whichever of a pixel's four cells an entry was filed under."""
+    w, h, gx, gy = 100, 70, 230, 170
+    sc = scenes.tiny(n=gx * gy, w=w, h=h, f=90.0, num_layers=4, list_depth=16, seed=17, radius=(0.004, 0.12))
+    xr, yr = 1.15 * 3.0 * (w / 2) / 90.0, 1.15 * 3.0 * (h / 2) / 90.0  # a little more than the view covers at depth 3
+    X, Y = np.meshgrid(np.linspace(-xr, xr, gx), np.linspace(-yr, yr, gy))
+    order = np.random.default_rng(5).permutation(gx * gy)  # ids unrelated to the screen position
+    sc.position[:, 0] = X.reshape(-1)[order]
+    sc.position[:, 1] = Y.reshape(-1)[order]
+    sc.position[:, 2] = 0.0
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    depth = ref["depth"][0]
+    assert len(np.unique(depth[depth > 0])) == 1  # every visible point at the same depth
+    ip = ref["ip"][0][depth > 0]
+    px = np.floor(ip[:, 0]).astype(int)
+    assert {31, 32, 63, 64, w - 2} <= set(px.tolist()) and px.max() == w - 2
+    assert ref["lengths"][0].max() > 16
+    _check_backward(oracle, sc, d, seed=4)
+
+
 def test_config1_forward_full(oracle):
     sc = scenes.config1()
     _check_forward(oracle, sc, abi.desc_for_scene(sc, train=True))
