@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     floatx4 acc[4][NB];
     conv_taps_mfma<CIN, NPAD>(s_patch, s_taps, p.wpack, taps, acc);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lrow = lane & 15;
+    const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
     // ---- epilogue: elu(feature) * sigmoid(mask) in fp16, staged in LDS (the patch is no longer needed) and
     // written channels innermost with full-line stores; the pre-activations too when the backward needs them ----
@@ -213,29 +213,63 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     if (p.pre) store_tile_nhwc(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
     if (p.final_out)
     {
-        // `final` of the net (Networks.h:1129-1131): one thread per pixel of the tile, weights rounded to fp16 like
-        // every other operand
-        const int y = y0 + threadIdx.x / kConvTileW, x = x0 + threadIdx.x % kConvTileW;
-        if (y < p.H && x < p.W)
+        // `final` of the net (Networks.h:1129-1131) on the matrix cores: per 16 pixels one MFMA per 32 input channels,
+        // A = the staged tile rows (block outputs, then the image in the row's padding columns), B = the 1x1 weights,
+        // rounded to fp16 like every other operand, outputs in the first columns.
+        constexpr int KF  = NPAD / 2 + kLdsChanPad;  // block outputs (padded) | image | zeros
+        constexpr int KFB = (KF + 31) / 32;
+        const int cin     = C + p.cout;
+        // the image joins the staged rows (columns NPAD/2 .. NPAD/2 + 7; nobody has read them yet)
         {
-            const int cin           = C + p.cout;
-            const _Float16* a       = s_act + (size_t)threadIdx.x * AS;
-            const size_t plane      = (size_t)p.H * p.W;
-            float o[4] = {0.f, 0.f, 0.f, 0.f};
-            for (int c = 0; c < C; ++c)
+            _Float16* row = s_act + (size_t)threadIdx.x * AS + NPAD / 2;
 #pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (k < p.final_cout) o[k] += s_fw[k * cin + c] * my_feat[c];
-            for (int c = 0; c < p.cout; ++c)
+            for (int c = 0; c < kLdsChanPad; ++c) row[c] = c < C ? _Float16(my_feat[c]) : _Float16(0.f);
+        }
+        half8 bfin[KFB];
+#pragma unroll
+        for (int kb = 0; kb < KFB; ++kb)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
             {
-                const float v = float(a[c]);
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (k < p.final_cout) o[k] += s_fw[k * cin + C + c] * v;
+                const int k = kb * 32 + lk + i;  // position in a staged row
+                float w     = 0.f;
+                if (lrow < p.final_cout)
+                {
+                    if (k < p.cout)
+                        w = s_fw[lrow * cin + C + k];
+                    else if (k >= NPAD / 2 && k < NPAD / 2 + C)
+                        w = s_fw[lrow * cin + (k - NPAD / 2)];
+                }
+                bfin[kb][i] = _Float16(w);  // exact: the table holds fp16 values
             }
+        __syncthreads();  // image columns in place
+        const size_t plane = (size_t)p.H * p.W;
+        const float fb     = lrow < p.final_cout ? s_fw[4 * (4 + 64) + lrow] : 0.f;
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (k < p.final_cout) p.final_out[k * plane + (size_t)y * p.W + x] = o[k] + s_fw[4 * (4 + 64) + k];
+        for (int m = 0; m < 4; ++m)
+        {
+            const int tp0 = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16;  // first pixel of this 16-pixel block
+            floatx4 o     = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb = 0; kb < KFB; ++kb)
+            {
+                half8 a;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a[i] = _Float16(0.f);
+                if (kb * 32 + lk < KF) a = *reinterpret_cast<const half8*>(s_act + (size_t)(tp0 + lrow) * AS + kb * 32 + lk);
+                o = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfin[kb], o, 0, 0, 0);
+            }
+            // lane: output channel lrow, pixels tp0 + (lane / 16) * 4 .. + 3
+            if (lrow < p.final_cout)
+            {
+                const int tp = tp0 + (lane >> 4) * 4;
+                const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
+                float* dst = p.final_out + lrow * plane + (size_t)y * p.W + x;
+                if (y < p.H)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (x + i < p.W) dst[i] = o[i] + fb;
+            }
         }
     }
 }
