@@ -9,6 +9,7 @@
 namespace trips
 {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kConvTileH   = 8;

@@ -87,7 +87,10 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
             if (in)
                 for (int c = 0; c < C; ++c) v[c] = p.feat[c * plane + (size_t)y * p.W + x];
             _Float16* row = s_patch + (size_t)item * ROW;
-            for (int c = 0; c < C; ++c) row[c] = _Float16(v[c]);
+            if (C == 4)  // one 8-byte LDS store instead of four 2-byte ones
+                *reinterpret_cast<half4*>(row) = half4{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3])};
+            else
+                for (int c = 0; c < C; ++c) row[c] = _Float16(v[c]);
             if (!has_below)
             {
                 // start block: the image is the whole input
@@ -108,7 +111,14 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
             _Float16* row = s_below + (size_t)bp * ROW;
             if (q == 0)
             {
-                for (int c = 0; c < C; ++c) row[C + c] = _Float16(p.feat_below[c * pb + (size_t)yy * p.Wb + xx]);
+                if (C == 4)
+                {
+                    const float* src = p.feat_below + (size_t)yy * p.Wb + xx;
+                    const float v0 = src[0], v1 = src[pb], v2 = src[2 * pb], v3 = src[3 * pb];
+                    *reinterpret_cast<half4*>(row + 4) = half4{_Float16(v0), _Float16(v1), _Float16(v2), _Float16(v3)};
+                }
+                else
+                    for (int c = 0; c < C; ++c) row[C + c] = _Float16(p.feat_below[c * pb + (size_t)yy * p.Wb + xx]);
                 for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);  // padding channels
             }
             else
@@ -154,7 +164,11 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
             _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
             if (g == 0)
             {
-                for (int i = C; i < 8; ++i) dst[i] = h[i];  // [0, C) holds this level's image
+                // [0, C) holds this level's image
+                if (C == 4)
+                    *reinterpret_cast<half4*>(dst + 4) = half4{h[4], h[5], h[6], h[7]};
+                else
+                    for (int i = C; i < 8; ++i) dst[i] = h[i];
             }
             else
                 *reinterpret_cast<half8*>(dst) = h;
