@@ -87,7 +87,10 @@ __device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT>& st
 
 // Precondition: tap 0 sits in s_taps[0 .. BUF) (conv_tap_fetch + conv_tap_stage) and a barrier has passed since.
 // Every thread of the workgroup must call this (it contains barriers).
-template <int KIN, int NOUT>
+// Result layout: lane l holds, of the 16 x 16 block acc[m][n], pixels (l / 16) * 4 .. + 3 of output 16n + l % 16; with
+// OUTPUTS_IN_ROWS (the operands of the MFMA exchanged) outputs 16n + (l / 16) * 4 .. + 3 of pixel l % 16, four
+// neighbouring channels of one pixel, which an epilogue can store as one 8-byte word.
+template <int KIN, int NOUT, bool OUTPUTS_IN_ROWS = false>
 __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16* s_taps, const _Float16* __restrict__ wpack,
                                                ConvTapStage<KIN, NOUT>& st, floatx4 (&acc)[4][NOUT / 16])
 {
@@ -119,7 +122,9 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
                 const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
                 const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
 #pragma unroll
-                for (int n = 0; n < NB; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[n], acc[m][n], 0, 0, 0);
+                for (int n = 0; n < NB; ++n)
+                    acc[m][n] = OUTPUTS_IN_ROWS ? __builtin_amdgcn_mfma_f32_16x16x32_f16(bfrag[n], a, acc[m][n], 0, 0, 0)
+                                                : __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[n], acc[m][n], 0, 0, 0);
             }
         }
         if (tap + 1 < 9) conv_tap_stage(st, s_taps + ((tap + 1) & 1) * S::BUF);

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     conv_tap_stage(taps, s_taps);
     __syncthreads();
     floatx4 acc[4][NB];
-    conv_taps_mfma<CIN, NPAD>(s_patch, s_taps, p.wpack, taps, acc);
+    conv_taps_mfma<CIN, NPAD, true>(s_patch, s_taps, p.wpack, taps, acc);  // a lane: four channels of one pixel
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
@@ -200,26 +200,30 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 #pragma unroll
     for (int m = 0; m < 4; ++m)
     {
+        const int tp = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + lrow;  // this lane's pixel of the block
 #pragma unroll
         for (int j = 0; j < HB; ++j)
         {
-            const int ch = 16 * j + lrow;
-            const float bf = p.bias[ch], bm = p.bias[NPAD / 2 + ch];
+            const int ch0   = 16 * j + (lane >> 4) * 4;  // this lane's four channels
+            const float4 bf = *reinterpret_cast<const float4*>(p.bias + ch0), bm = *reinterpret_cast<const float4*>(p.bias + NPAD / 2 + ch0);
+            const float f[4] = {acc[m][j][0] + bf.x, acc[m][j][1] + bf.y, acc[m][j][2] + bf.z, acc[m][j][3] + bf.w};
+            // (both 0 for padding channels)
+            const float g[4] = {acc[m][HB + j][0] + bm.x, acc[m][HB + j][1] + bm.y, acc[m][HB + j][2] + bm.z, acc[m][HB + j][3] + bm.w};
+            if (p.pre)
+            {
+                *reinterpret_cast<half4*>(s_pre + tp * PS + ch0)            = half4{_Float16(f[0]), _Float16(f[1]), _Float16(f[2]), _Float16(f[3])};
+                *reinterpret_cast<half4*>(s_pre + tp * PS + NPAD / 2 + ch0) = half4{_Float16(g[0]), _Float16(g[1]), _Float16(g[2]), _Float16(g[3])};
+            }
+            half4 out;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
-                const int tp  = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + (lane >> 4) * 4 + i;
-                const float f = acc[m][j][i] + bf, g = acc[m][HB + j][i] + bm;  // both 0 for padding channels
-                if (p.pre)
-                {
-                    s_pre[tp * PS + ch]            = _Float16(f);
-                    s_pre[tp * PS + NPAD / 2 + ch] = _Float16(g);
-                }
-                const float e = f > 0.f ? f : (__expf(f) - 1.f);
+                const float e = f[i] > 0.f ? f[i] : (__expf(f[i]) - 1.f);
                 // v_rcp_f32 is good to 1 ulp of fp32 and the product is rounded to fp16 next: no IEEE division needed
-                const float s = __builtin_amdgcn_rcpf(1.f + __expf(-g));
-                s_act[tp * AS + ch] = ch < p.cout ? _Float16(e * s) : _Float16(0.f);
+                const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-g[i]));
+                out[i]         = ch0 + i < p.cout ? _Float16(e * sg) : _Float16(0.f);
             }
+            *reinterpret_cast<half4*>(s_act + tp * AS + ch0) = out;
         }
     }
     __syncthreads();
