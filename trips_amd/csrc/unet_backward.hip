@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     conv_tap_stage(taps, s_taps);
     __syncthreads();
     floatx4 acc[4][NB];
-    conv_taps_mfma<KC, NN>(s_patch, s_taps, p.wt, taps, acc);
+    conv_taps_mfma<KC, NN, true>(s_patch, s_taps, p.wt, taps, acc);  // a lane: four channels of one pixel
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
     // ---- epilogue: the tile staged in LDS (the patch is no longer needed) and written channels innermost with
@@ -335,17 +335,17 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
 #pragma unroll
     for (int m = 0; m < 4; ++m)
     {
+        const int tp = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + lrow;  // this lane's pixel of the block
 #pragma unroll
         for (int n = 0; n < NB; ++n)
         {
-            const int c = 16 * n + lrow;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
+            const int c0 = 16 * n + (lane >> 4) * 4;  // this lane's four channels
+            *reinterpret_cast<half4*>(s_out + tp * OS + c0) =
+                half4{_Float16(acc[m][n][0]), _Float16(acc[m][n][1]), _Float16(acc[m][n][2]), _Float16(acc[m][n][3])};
+            if (n == 0 && c0 == 0)
             {
-                const int tp  = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + (lane >> 4) * 4 + i;
-                const float v = acc[m][n][i];
-                s_out[tp * OS + c] = _Float16(v);
-                if (n == 0 && c < 4) s_img[c * (kConvTileH * kConvTileW) + tp] = v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s_img[i * (kConvTileH * kConvTileW) + tp] = acc[m][0][i];
             }
         }
     }
