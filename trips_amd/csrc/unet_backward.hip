@@ -9,9 +9,11 @@
 //   up2_adjoint_gate_kernel   adjoint of the bilinear 2x upsampling (a gather over <= 4 x 4 finer pixels), then
 //                             dL/d in[i+1] and the gate of the coarser block
 //   conv_bwd_weight_kernel    weight gradients: GEMM with the pixels as the reduction dimension. Both operands are
-//                             needed pixel-contiguous, so the tiles are written to LDS transposed ([channel][pixel]);
-//                             persistent workgroups keep their partial sums in registers over many tiles
-//                             and sum the pre-activation gradients of their tiles for the bias gradients
+//                             needed pixel-contiguous; the tiles stay pixel-major in LDS, as they are assembled, and
+//                             the operands are fetched with the transposing LDS read (ds_read_b64_tr_b16);
+//                             persistent workgroups keep their partial sums in registers over many tiles; the
+//                             bias gradients (sums of the pre-activation gradients) are one more MFMA per tile row
+//                             against a matrix of ones
 //   bias_grad_kernel          bias gradients alone, when no weight gradient is asked for
 //   reduce_weight_grad_kernel
 //
@@ -24,7 +26,6 @@
 
 namespace trips
 {
-typedef half8 half8_unaligned __attribute__((aligned(2)));
 
 // d(elu(f) * sigmoid(m)) for an incoming gradient da
 __device__ __forceinline__ void gate_backward(float da, float f, float m, float& df, float& dm)
@@ -537,19 +538,73 @@ struct BwdWeightParams
     float* bias_part;      // [gridDim.x][NPAD] or nullptr
 };
 
-constexpr int kXtRow   = 40;                          // halves per patch row in the transposed input tile
-constexpr int kXtChan  = kConvPatchH * kXtRow + 8;    // halves per channel (padding spreads the 16 channels of a read over the banks)
-constexpr int kDtChan  = kConvTileH * kConvTileW + 8;  // halves per pre-activation channel in the transposed gradient tile
+// Pixel-major tiles and the transposing LDS read. Both operands of the weight-gradient GEMM are needed with eight
+// consecutive pixels per lane, while the tiles are assembled (and arrive from memory) with the channels of a pixel side
+// by side. ds_read_b64_tr_b16 closes the gap: the 16 lanes of a group read a 4 x 16 block of halves row by row (lane
+// i: row i / 4, columns 4 (i % 4) .. + 3) and each receives one column (lane n: rows 0 .. 3 of column n). Two such
+// reads give a lane the eight pixels of its channel; the tiles stay as the forward kernel builds them, written with
+// 16-byte stores (written transposed, 2 bytes at a time, the staging took most of the kernel's time).
+typedef short short4v __attribute__((ext_vector_type(4)));
+// rows `pix` .. `pix + 7` of column `col0 + lane % 16` of a tile [pixel][stride halves]; `col0` a multiple of 16
+__device__ __forceinline__ half8 lds_read_pixels_of_channel(const _Float16* tile, int stride, int pix, int col0)
+{
+    const int i = threadIdx.x & 15;
+    const _Float16* src = tile + (size_t)(pix + (i >> 2)) * stride + col0 + (i & 3) * 4;
+    using lds_ptr = __attribute__((address_space(3))) short4v*;
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 4 * stride));
+    union
+    {
+        short s[8];
+        half8 h;
+    } u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        u.s[k]     = lo[k];
+        u.s[4 + k] = hi[k];
+    }
+    return u.h;
+}
+
+// The same for the three horizontal taps at once: pixels `pix + dx` .. `pix + dx + 7`, dx = 0, 1, 2, of column
+// `col0 + lane % 16`, from three reads of four pixels (ten of the twelve are used; the last two may lie past the
+// tile, inside the workgroup's LDS) instead of six: the window of dx = 2 is a whole register further, the window of
+// dx = 1 is stitched together with four funnel shifts.
+__device__ __forceinline__ void lds_read_pixel_windows(const _Float16* tile, int stride, int pix, int col0, half8 (&w)[3])
+{
+    const int i = threadIdx.x & 15;
+    const _Float16* src = tile + (size_t)(pix + (i >> 2)) * stride + col0 + (i & 3) * 4;
+    using lds_ptr = __attribute__((address_space(3))) short4v*;
+    union
+    {
+        short4v v[3];
+        unsigned d[6];
+    } in;
+    in.v[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+    in.v[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 4 * stride));
+    in.v[2] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 8 * stride));
+    union
+    {
+        unsigned d[4];
+        half8 h;
+    } out;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out.d[k] = in.d[k];
+    w[0] = out.h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out.d[k] = __builtin_amdgcn_alignbit(in.d[k + 1], in.d[k], 16);
+    w[1] = out.h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out.d[k] = in.d[k + 1];
+    w[2] = out.h;
+}
 
 template <int CIN, int NPAD, bool BIAS>
 __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightParams p)
 {
-    // bias sums: thread t adds up segment t / NPAD (kBiasSegLen pixels) of row t % NPAD of the gradient tile
-    constexpr int kBiasSegs   = 256 / NPAD;
-    constexpr int kBiasSegLen = kConvTileH * kConvTileW / kBiasSegs;
-    const int bias_n = threadIdx.x % NPAD, bias_seg = threadIdx.x / NPAD;
-    float bias_acc = 0.f;
-    constexpr int ROW    = CIN + kLdsChanPad;
+    constexpr int ROW    = CIN + kLdsChanPad;   // halves per pixel of the input patch
+    constexpr int DS     = NPAD + kLdsChanPad;  // halves per pixel of the gradient tile
     constexpr int GROUPS = CIN / 8;
     constexpr int NB     = NPAD / 16;
     constexpr int CB     = CIN / 16;
@@ -562,13 +617,13 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     constexpr int MYNB   = NB / NBW;
     static_assert(CB % CBW == 0 && NB % NBW == 0, "block split");
     extern __shared__ _Float16 smem[];
-    _Float16* s_below = smem;                                  // [kBelowH * kBelowW][ROW]
-    _Float16* s_xt    = s_below + kBelowH * kBelowW * ROW;     // [CIN][kXtChan]
-    _Float16* s_dt    = s_xt + CIN * kXtChan;                  // [NPAD][kDtChan]
+    _Float16* s_patch = smem;                                           // [kConvPatchH * kConvPatchW][ROW]
+    _Float16* s_below = s_patch + kConvPatchH * kConvPatchW * ROW;      // [kBelowH * kBelowW][ROW]
+    _Float16* s_d     = s_below + kBelowH * kBelowW * ROW;              // [kConvTileH * kConvTileW][DS]
     const bool has_below = p.Hb > 0;
     const int C          = p.c_feat;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lrow = lane & 15, lk = (lane >> 4) * 8;
+    const int lk = (lane >> 4) * 8;
 
     const int cb0 = (wave % CBW) * MYCB, nb0 = (wave / CBW) * MYNB;
     floatx4 acc[9][MYNB][MYCB];
@@ -578,13 +633,19 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         for (int n = 0; n < MYNB; ++n)
 #pragma unroll
             for (int c = 0; c < MYCB; ++c) acc[t][n][c] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    // channels that no stage writes stay zero for every tile
-    for (int i = threadIdx.x; i < CIN * kXtChan; i += 256) s_xt[i] = _Float16(0.f);
+    // Bias gradients = sums of the pre-activation gradients over the pixels: one more MFMA per tile row and block with
+    // a matrix of ones as the other operand (every column of the result is the row sum), by the wavefronts that own
+    // the first input blocks.
+    floatx4 bias_acc[MYNB];
+#pragma unroll
+    for (int n = 0; n < MYNB; ++n) bias_acc[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    half8 ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ones[i] = _Float16(1.f);
 
     // ---- stage 1 in two halves: every global load of a tile is issued into registers (a thread's loads are all in
-    // flight together), and written to LDS (transposed) one tile later, so that the loads of tile t + 1 travel while
-    // tile t is upsampled and multiplied ----
+    // flight together), and written to LDS one tile later, so that the loads of tile t + 1 travel while tile t is
+    // upsampled and multiplied ----
     constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + 255) / 256;
     constexpr int kMaxPerPix  = 1 + (CIN - 8) / 8;  // image below + groups of 8 block outputs (C = 4)
     constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + 255) / 256;
@@ -642,12 +703,42 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         for (int k = 0; k < kDpreItems; ++k)
         {
             const int item = threadIdx.x + 256 * k;
-            const int tp = item % (kConvTileH * kConvTileW), g = item / (kConvTileH * kConvTileW);
+            const int g = item % kDpreItems, tp = item / kDpreItems;
             const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
 #pragma unroll
             for (int i = 0; i < 8; ++i) r.dpre[k][i] = _Float16(0.f);
             if (y < p.H && x < p.W) r.dpre[k] = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * NPAD + 8 * g);
         }
+    };
+    // this level's image into channels [0, C) of a patch pixel (the channels [C, 8) follow from the upsampling, or are
+    // zero for the start block, whose other channels are cleared once, below)
+    auto put_image = [&](int item, const float (&v)[4])
+    {
+        _Float16* row = s_patch + (size_t)item * ROW;
+        if (has_below && C == 4)
+            *reinterpret_cast<half4*>(row) = half4{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3])};
+        else if (has_below)
+        {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)  // a run-time bound would put the register array into scratch memory
+                if (c < C) row[c] = _Float16(v[c]);
+        }
+        else
+            *reinterpret_cast<half8*>(row) = half8{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3]),
+                                                   _Float16(0.f), _Float16(0.f), _Float16(0.f), _Float16(0.f)};
+    };
+    auto put_below_image = [&](int bp, const float (&v)[4])
+    {
+        _Float16* row = s_below + (size_t)bp * ROW;
+        if (C == 4)
+            *reinterpret_cast<half4*>(row + 4) = half4{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3])};
+        else
+        {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (c < C) row[C + c] = _Float16(v[c]);
+        }
+        for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
     };
     auto commit_loads = [&](const TileLoads& r)
     {
@@ -655,13 +746,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         for (int k = 0; k < kFeatItems; ++k)
         {
             const int item = threadIdx.x + 256 * k;
-            if (item < kConvPatchH * kConvPatchW)
-            {
-                const int py = item / kConvPatchW, px = item - py * kConvPatchW;
-#pragma unroll
-                for (int c = 0; c < 4; ++c)  // a run-time bound would put the register array into scratch memory
-                    if (c < C) s_xt[c * kXtChan + py * kXtRow + px] = _Float16(r.feat[k][c]);
-            }
+            if (item < kConvPatchH * kConvPatchW) put_image(item, r.feat[k]);
         }
         if (has_below)
         {
@@ -672,17 +757,14 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
                 if (item < kBelowH * kBelowW * per_pixel)
                 {
                     const int q = item % per_pixel, bp = item / per_pixel;
-                    _Float16* row = s_below + (size_t)bp * ROW;
                     if (q == 0)
                     {
-                        const unsigned f[4] = {r.below[k].x, r.below[k].y, r.below[k].z, r.below[k].w};
-#pragma unroll
-                        for (int c = 0; c < 4; ++c)
-                            if (c < C) row[C + c] = _Float16(__uint_as_float(f[c]));
-                        for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
+                        const float f[4] = {__uint_as_float(r.below[k].x), __uint_as_float(r.below[k].y), __uint_as_float(r.below[k].z),
+                                            __uint_as_float(r.below[k].w)};
+                        put_below_image(bp, f);
                     }
                     else
-                        *reinterpret_cast<uint4*>(row + 2 * C + 8 * (q - 1)) = r.below[k];
+                        *reinterpret_cast<uint4*>(s_below + (size_t)bp * ROW + 2 * C + 8 * (q - 1)) = r.below[k];
                 }
             }
         }
@@ -690,9 +772,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         for (int k = 0; k < kDpreItems; ++k)
         {
             const int item = threadIdx.x + 256 * k;
-            const int tp = item % (kConvTileH * kConvTileW), g = item / (kConvTileH * kConvTileW);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s_dt[(8 * g + i) * kDtChan + tp] = r.dpre[k][i];
+            *reinterpret_cast<half8*>(s_d + (size_t)(item / kDpreItems) * DS + 8 * (item % kDpreItems)) = r.dpre[k];
         }
     };
 
@@ -706,45 +786,55 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
                 const int py = item / kConvPatchW, px = item - py * kConvPatchW;
                 const int y = y0 + py - 1, x = x0 + px - 1;
                 const bool in = y >= 0 && y < p.H && x >= 0 && x < p.W;
-                for (int c = 0; c < C; ++c)
-                    s_xt[c * kXtChan + py * kXtRow + px] = in ? _Float16(p.feat[c * plane + (size_t)y * p.W + x]) : _Float16(0.f);
+                float v[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) v[c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+                put_image(item, v);
             }
         }
         if (has_below)
         {
-            const size_t pb      = (size_t)p.Hb * p.Wb;
-            const int act_groups = p.cb_store / 8;
-            const int per_pixel  = 1 + act_groups;
+            const size_t pb = (size_t)p.Hb * p.Wb;
             for (int item = threadIdx.x; item < kBelowH * kBelowW * per_pixel; item += 256)
             {
                 const int q = item % per_pixel, bp = item / per_pixel;
                 const int r = bp / kBelowW, c0 = bp - r * kBelowW;
                 const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
-                _Float16* row = s_below + (size_t)bp * ROW;
                 if (q == 0)
                 {
-                    for (int c = 0; c < C; ++c) row[C + c] = _Float16(p.feat_below[c * pb + (size_t)yy * p.Wb + xx]);
-                    for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
+                    float v[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) v[c] = c < C ? p.feat_below[c * pb + (size_t)yy * p.Wb + xx] : 0.f;
+                    put_below_image(bp, v);
                 }
                 else
                 {
-                    *reinterpret_cast<half8*>(row + 2 * C + 8 * (q - 1)) =
+                    *reinterpret_cast<half8*>(s_below + (size_t)bp * ROW + 2 * C + 8 * (q - 1)) =
                         *reinterpret_cast<const half8*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
                 }
             }
         }
-        for (int item = threadIdx.x; item < kConvTileH * kConvTileW * (NPAD / 8); item += 256)
+        for (int item = threadIdx.x; item < kConvTileH * kConvTileW * kDpreItems; item += 256)
         {
-            const int tp = item % (kConvTileH * kConvTileW), g = item / (kConvTileH * kConvTileW);
+            const int g = item % kDpreItems, tp = item / kDpreItems;
             const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
             half8 v;
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = _Float16(0.f);
             if (y < p.H && x < p.W) v = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * NPAD + 8 * g);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s_dt[(8 * g + i) * kDtChan + tp] = v[i];
+            *reinterpret_cast<half8*>(s_d + (size_t)tp * DS + 8 * g) = v;
         }
     };
+
+    // start block: the channels beyond the first eight of a patch pixel are never written and stay zero
+    if (!has_below)
+        for (int i = threadIdx.x; i < kConvPatchH * kConvPatchW * (GROUPS - 1); i += 256)
+        {
+            half8 z;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) z[k] = _Float16(0.f);
+            *reinterpret_cast<half8*>(s_patch + (size_t)(i / (GROUPS - 1)) * ROW + 8 * (1 + i % (GROUPS - 1))) = z;
+        }
 
     // with 64 input channels and more than 64 pre-activations the accumulators leave no registers for a tile in flight
     constexpr bool kPrefetch = !(CIN == 64 && NPAD > 64);
@@ -764,48 +854,46 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         if (has_below)
         {
             __syncthreads();
-            // ---- stage 2: bilinear 2x upsampling from the below patch, written transposed ----
+            // ---- stage 2: bilinear 2x upsampling from the below patch into channels [C, CIN) of the patch, in packed
+            // fp16 exactly as the forward kernel does it (the weights are products of 0, 1/4, 3/4 and 1) ----
             for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
             {
-                const int pp = item % (kConvPatchH * kConvPatchW), g = item / (kConvPatchH * kConvPatchW);
+                const int g = item % GROUPS, pp = item / GROUPS;
                 const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
                 const int y = y0 + py - 1, x = x0 + px - 1;
-                float v[8];
+                half8 h;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[i] = 0.f;
+                for (int i = 0; i < 8; ++i) h[i] = _Float16(0.f);
                 if (y >= 0 && y < p.H && x >= 0 && x < p.W)
                 {
                     int ya, yb, xa, xb;
                     float ly, lx;
                     up2_source(y, p.Hb, ya, yb, ly);
                     up2_source(x, p.Wb, xa, xb, lx);
-                    const float w00 = (1.f - ly) * (1.f - lx), w01 = (1.f - ly) * lx, w10 = ly * (1.f - lx), w11 = ly * lx;
+                    const _Float16 w00 = _Float16((1.f - ly) * (1.f - lx)), w01 = _Float16((1.f - ly) * lx);
+                    const _Float16 w10 = _Float16(ly * (1.f - lx)), w11 = _Float16(ly * lx);
                     const half8 a = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
                     const half8 b = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
                     const half8 c = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
                     const half8 d = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) v[i] = w00 * float(a[i]) + w01 * float(b[i]) + w10 * float(c[i]) + w11 * float(d[i]);
+                    const half8 W00 = {w00, w00, w00, w00, w00, w00, w00, w00}, W01 = {w01, w01, w01, w01, w01, w01, w01, w01};
+                    const half8 W10 = {w10, w10, w10, w10, w10, w10, w10, w10}, W11 = {w11, w11, w11, w11, w11, w11, w11, w11};
+                    h = __builtin_elementwise_fma(d, W11, __builtin_elementwise_fma(c, W10, __builtin_elementwise_fma(b, W01, a * W00)));
                 }
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    if (8 * g + i >= C) s_xt[(8 * g + i) * kXtChan + py * kXtRow + px] = _Float16(v[i]);
+                _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
+                if (g == 0)
+                {
+                    // [0, C) holds this level's image
+                    if (C == 4)
+                        *reinterpret_cast<half4*>(dst + 4) = half4{h[4], h[5], h[6], h[7]};
+                    else
+                        for (int i = C; i < 8; ++i) dst[i] = h[i];
+                }
+                else
+                    *reinterpret_cast<half8*>(dst) = h;
             }
         }
         __syncthreads();
-        if (BIAS && (int)threadIdx.x < kBiasSegs * NPAD)
-        {
-            const _Float16* src = s_dt + bias_n * kDtChan + bias_seg * kBiasSegLen;
-            float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-            for (int q = 0; q < kBiasSegLen / 8; ++q)
-            {
-                const half8 v = *reinterpret_cast<const half8*>(src + 8 * q);
-                s0 += (float(v[0]) + float(v[1])) + (float(v[2]) + float(v[3]));
-                s1 += (float(v[4]) + float(v[5])) + (float(v[6]) + float(v[7]));
-            }
-            bias_acc += s0 + s1;
-        }
         // ---- dW[tap][n][c] += sum over the tile's pixels of dpre[pixel][n] * x[pixel + tap][c] ----
 #pragma unroll
         for (int r = 0; r < kConvTileH; ++r)
@@ -813,33 +901,39 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
             half8 a[MYNB];
 #pragma unroll
             for (int n = 0; n < MYNB; ++n)
-                a[n] = *reinterpret_cast<const half8*>(s_dt + ((nb0 + n) * 16 + lrow) * kDtChan + r * kConvTileW + lk);
-#pragma unroll
-            for (int tap = 0; tap < 9; ++tap)
             {
-                const int dy = tap / 3, dx = tap - dy * 3;
+                a[n] = lds_read_pixels_of_channel(s_d, DS, r * kConvTileW + lk, (nb0 + n) * 16);
+                if (BIAS && cb0 == 0) bias_acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[n], ones, bias_acc[n], 0, 0, 0);
+            }
+#pragma unroll
+            for (int dy = 0; dy < 3; ++dy)
+            {
 #pragma unroll
                 for (int c = 0; c < MYCB; ++c)
                 {
-                    const half8 b = *reinterpret_cast<const half8_unaligned*>(s_xt + ((cb0 + c) * 16 + lrow) * kXtChan + (r + dy) * kXtRow + lk + dx);
+                    half8 b[3];
+                    lds_read_pixel_windows(s_patch, ROW, (r + dy) * kConvPatchW + lk, (cb0 + c) * 16, b);
 #pragma unroll
-                    for (int n = 0; n < MYNB; ++n) acc[tap][n][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[n], b, acc[tap][n][c], 0, 0, 0);
+                    for (int dx = 0; dx < 3; ++dx)
+#pragma unroll
+                        for (int n = 0; n < MYNB; ++n)
+                            acc[3 * dy + dx][n][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[n], b[dx], acc[3 * dy + dx][n][c], 0, 0, 0);
                 }
             }
         }
     }
 
-    if (BIAS)
+    if (BIAS && cb0 == 0 && (lane & 15) == 0)
     {
-        __syncthreads();  // all tiles consumed: the tile memory is free
-        float* s_bias = reinterpret_cast<float*>(smem);
-        if ((int)threadIdx.x < NPAD) s_bias[threadIdx.x] = 0.f;
-        __syncthreads();
-        if ((int)threadIdx.x < kBiasSegs * NPAD) atomicAdd(&s_bias[bias_n], bias_acc);
-        __syncthreads();
-        if ((int)threadIdx.x < NPAD) p.bias_part[(size_t)blockIdx.x * NPAD + threadIdx.x] = s_bias[threadIdx.x];
+        // column 0 of the row sums: this lane holds rows (lane / 16) * 4 .. + 3 of every block
+        float* dst = p.bias_part + (size_t)blockIdx.x * NPAD;
+#pragma unroll
+        for (int n = 0; n < MYNB; ++n)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[(nb0 + n) * 16 + (lane >> 4) * 4 + i] = bias_acc[n][i];
     }
     float* part = p.part + (size_t)blockIdx.x * 9 * NPAD * CIN;
+    const int lrow = lane & 15;
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)
 #pragma unroll
@@ -925,7 +1019,8 @@ hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipS
 template <int CIN, int NPAD, bool BIAS>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
-    const size_t lds = ((size_t)kBelowH * kBelowW * (CIN + kLdsChanPad) + (size_t)CIN * kXtChan + (size_t)NPAD * kDtChan) *
+    const size_t lds = ((size_t)(kConvPatchH * kConvPatchW + kBelowH * kBelowW) * (CIN + kLdsChanPad) +
+                        (size_t)kConvTileH * kConvTileW * (NPAD + kLdsChanPad)) *
                        sizeof(_Float16);  // up to 133 KB
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD, BIAS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
