@@ -257,7 +257,10 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
         lv.din_off = bw;
         bw += align256(pixels * lv.cin_pad * sizeof(_Float16));
         const int tiles = ((lv.W + kConvTileW - 1) / kConvTileW) * ((lv.H + kConvTileH - 1) / kConvTileH);
-        lv.groups       = tiles < 1024 ? tiles : 1024;
+        // persistent workgroups of the weight-gradient kernel: as many as are resident at once (two per CU for the
+        // smallest shape, else one); every further one would only add a set of partial sums to write and reduce
+        const int resident = (lv.cin_pad * lv.npad <= 1024 ? 2 : 1) * 256;
+        lv.groups          = tiles < resident ? tiles : resident;
         lv.part_off     = bw;
         bw += align256((size_t)d.batch * lv.groups * 9 * lv.npad * lv.cin_pad * sizeof(float));
         lv.sliced_off = bw;
