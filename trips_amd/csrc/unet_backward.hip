@@ -917,7 +917,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
                     for (int dx = 0; dx < 3; ++dx)
 #pragma unroll
                         for (int n = 0; n < MYNB; ++n)
-                            acc[3 * dy + dx][n][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[n], b[dx], acc[3 * dy + dx][n][c], 0, 0, 0);
+                            acc[3 * dy + dx][n][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[dx], a[n], acc[3 * dy + dx][n][c], 0, 0, 0);
                 }
             }
         }
@@ -934,15 +934,15 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     }
     float* part = p.part + (size_t)blockIdx.x * 9 * NPAD * CIN;
     const int lrow = lane & 15;
+    // (the input channels are the rows of the MFMA result: a lane holds four neighbouring ones of output lrow)
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)
 #pragma unroll
         for (int n = 0; n < MYNB; ++n)
 #pragma unroll
             for (int c = 0; c < MYCB; ++c)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    part[((size_t)tap * NPAD + (nb0 + n) * 16 + (lane >> 4) * 4 + i) * CIN + (cb0 + c) * 16 + lrow] = acc[tap][n][c][i];
+                *reinterpret_cast<float4*>(part + ((size_t)tap * NPAD + (nb0 + n) * 16 + lrow) * CIN + (cb0 + c) * 16 + (lane >> 4) * 4) =
+                    make_float4(acc[tap][n][c][0], acc[tap][n][c][1], acc[tap][n][c][2], acc[tap][n][c][3]);
 }
 
 // Sum of the partial weight gradients of all workgroups (and images), in two steps so that many loads are in
