@@ -40,10 +40,24 @@ __device__ __forceinline__ void gate_backward(float da, float f, float m, float&
 
 // wt[tap'][c][n] = W[n][c][8 - tap']: the data gradient is a correlation of the pre-activation gradient with the
 // spatially flipped kernel, input and output channels exchanged
-__global__ __launch_bounds__(256) void pack_conv_weights_T_kernel(const float* __restrict__ wf, const float* __restrict__ wm,
-                                                                  int cout, int cin_real, int cin_pad, int npad,
-                                                                  _Float16* __restrict__ wt)
+// (all levels in one launch, the level is blockIdx.y: a launch per level costs more than the work itself)
+struct PackTLevel
 {
+    const float *wf, *wm;
+    int cout, cin_real, cin_pad, npad;
+    _Float16* wt;
+};
+struct PackTTable
+{
+    PackTLevel lv[TRIPS_UNET_MAX_LEVELS];
+};
+__global__ __launch_bounds__(256) void pack_conv_weights_T_kernel(const PackTTable t)
+{
+    const PackTLevel& l = t.lv[blockIdx.y];
+    const float* __restrict__ wf = l.wf;
+    const float* __restrict__ wm = l.wm;
+    const int cout = l.cout, cin_real = l.cin_real, cin_pad = l.cin_pad, npad = l.npad;
+    _Float16* __restrict__ wt = l.wt;
     const int total = 9 * cin_pad * npad;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256)
     {
@@ -260,18 +274,6 @@ __global__ __launch_bounds__(256) void final_reduce_kernel(const float* __restri
     if (!(t < cout * cin ? d_weight : d_bias)) return;  // the caller asked for one of the two only
     const float s = block_column_sum(part, rows, 4 * maxc + 4, col);
     if (threadIdx.x == 0) *dst = s;
-}
-
-// feature and mask bias gradients of a block from the weight-gradient kernel's per-workgroup sums [rows][npad]
-__global__ __launch_bounds__(256) void bias_reduce_kernel(const float* __restrict__ part, int rows, int npad, int cout, float scale_inv,
-                                                          float* __restrict__ d_bias_f, float* __restrict__ d_bias_m)
-{
-    const int n = blockIdx.x, half = npad / 2;
-    const int o = n < half ? n : n - half;
-    float* dst  = n < half ? d_bias_f : d_bias_m;
-    if (o >= cout || !dst) return;
-    const float s = block_column_sum(part, rows, npad, n);
-    if (threadIdx.x == 0) dst[o] = s * scale_inv;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -948,10 +950,29 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 // Sum of the partial weight gradients of all workgroups (and images), in two steps so that many loads are in
 // flight and every load is a full line: slice y of kReduceSlices sums its share of the partials element by element
 // (consecutive threads = consecutive elements), then the slices are summed into the reference's [Cout][Cin][3][3].
+// All levels in one launch each (the level is blockIdx.z): a launch per level and step costs more than the sums.
 constexpr int kReduceSlices = 16;
-__global__ __launch_bounds__(256) void reduce_weight_grad_slices_kernel(const float* __restrict__ part, int groups, int total,
-                                                                        float* __restrict__ sliced)
+struct ReduceLevel
 {
+    const float* part;  // [groups][total]
+    float* sliced;      // [kReduceSlices][total]
+    int groups, total;
+    int cout, cin_real, cin_pad, npad;
+    float *d_wf, *d_wm;
+    const float* bias_part;  // [groups][npad] or nullptr
+    float *d_bf, *d_bm;
+};
+struct ReduceTable
+{
+    ReduceLevel lv[TRIPS_UNET_MAX_LEVELS];
+    float scale_inv;
+};
+__global__ __launch_bounds__(256) void reduce_weight_grad_slices_kernel(const ReduceTable t)
+{
+    const ReduceLevel& l = t.lv[blockIdx.z];
+    const float* __restrict__ part = l.part;
+    float* __restrict__ sliced     = l.sliced;
+    const int groups = l.groups, total = l.total;
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const int per = (groups + kReduceSlices - 1) / kReduceSlices;
@@ -969,11 +990,29 @@ __global__ __launch_bounds__(256) void reduce_weight_grad_slices_kernel(const fl
     sliced[(size_t)blockIdx.y * total + i] = (s0 + s1) + (s2 + s3);
 }
 
-__global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const float* __restrict__ sliced, int cout, int cin_real,
-                                                                 int cin_pad, int npad, float scale_inv,
-                                                                 float* __restrict__ d_wf, float* __restrict__ d_wm)
+// ... and, in the workgroups behind those of the weights, the bias gradients from the per-workgroup sums
+__global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const ReduceTable t)
 {
+    const ReduceLevel& l = t.lv[blockIdx.z];
+    const float* __restrict__ sliced = l.sliced;
+    const int cout = l.cout, cin_real = l.cin_real, cin_pad = l.cin_pad, npad = l.npad;
+    const float scale_inv = t.scale_inv;
+    float* __restrict__ d_wf = l.d_wf;
+    float* __restrict__ d_wm = l.d_wm;
     const int total = 9 * npad * cin_pad;
+    const int wblocks = (total + 255) / 256;
+    if ((int)blockIdx.x >= wblocks)
+    {
+        // one workgroup per pre-activation channel
+        const int n = blockIdx.x - wblocks, half = npad / 2;
+        if (n >= npad || !l.bias_part) return;
+        const int o = n < half ? n : n - half;
+        float* dst  = n < half ? l.d_bf : l.d_bm;
+        if (o >= cout || !dst) return;
+        const float s = block_column_sum(l.bias_part, l.groups, npad, n);
+        if (threadIdx.x == 0) dst[o] = s * scale_inv;
+        return;
+    }
     const int i     = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const int c = i % cin_pad, n = (i / cin_pad) % npad, tap = i / (cin_pad * npad);
@@ -1114,13 +1153,19 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
 
     {
         ProfScope ps(prof, "unet_bwd_prepare", stream);
+        PackTTable pt;
+        int most = 0;
         for (int i = 0; i < L; ++i)
         {
             const LevelPlan& lv = np.lv[i];
-            const int total     = 9 * lv.npad * lv.cin_pad;
-            hipLaunchKernelGGL(pack_conv_weights_T_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
-                               weights->feature_weight[i], weights->mask_weight[i], lv.cout, lv.cin_real, lv.cin_pad, lv.npad,
-                               reinterpret_cast<_Float16*>(ws + lv.wt_off));
+            pt.lv[i] = PackTLevel{weights->feature_weight[i], weights->mask_weight[i], lv.cout, lv.cin_real, lv.cin_pad, lv.npad,
+                                  reinterpret_cast<_Float16*>(ws + lv.wt_off)};
+            most     = std::max(most, 9 * lv.npad * lv.cin_pad);
+        }
+        hipLaunchKernelGGL(pack_conv_weights_T_kernel, dim3((most + 255) / 256, L), dim3(256), 0, stream, pt);
+        for (int i = 0; i < L; ++i)
+        {
+            const LevelPlan& lv = np.lv[i];
             if (!grads->feature_weight[i] && !grads->mask_weight[i])  // bias_grad_kernel accumulates; otherwise they are written
             {
                 fill(grads->feature_bias[i], lv.cout);
@@ -1218,19 +1263,6 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
                     if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "weight gradient launch (level %d): %s", i, hipGetErrorString(e));
                 }
             }
-            if (grads->feature_weight[i] || grads->mask_weight[i])
-            {
-                const int total = 9 * lv.npad * lv.cin_pad;
-                float* sliced   = reinterpret_cast<float*>(ws + lv.sliced_off);
-                hipLaunchKernelGGL(reduce_weight_grad_slices_kernel, dim3((total + 255) / 256, kReduceSlices), dim3(256), 0, stream,
-                                   reinterpret_cast<const float*>(ws + lv.part_off), d.batch * lv.groups, total, sliced);
-                hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, sliced, lv.cout,
-                                   lv.cin_real, lv.cin_pad, lv.npad, scale_inv, grads->feature_weight[i], grads->mask_weight[i]);
-                if (grads->feature_bias[i] || grads->mask_bias[i])
-                    hipLaunchKernelGGL(bias_reduce_kernel, dim3(lv.npad), dim3(256), 0, stream,
-                                       reinterpret_cast<const float*>(ws + lv.bias_part_off), d.batch * lv.groups, lv.npad, lv.cout,
-                                       scale_inv, grads->feature_bias[i], grads->mask_bias[i]);
-            }
         }
         {
             ProfScope ps(prof, kDataNames[i], stream);
@@ -1267,6 +1299,37 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
         }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "backward launch (level %d): %s", i, hipGetErrorString(e));
+    }
+    // the partial weight and bias gradients of all levels are summed at the end, one launch per step of the sum
+    {
+        ProfScope ps(prof, "unet_bwd_reduce", stream);
+        ReduceTable rt;
+        rt.scale_inv = scale_inv;
+        int n = 0, most = 0, most_npad = 0;
+        for (int i = 0; i < L; ++i)
+        {
+            const LevelPlan& lv = np.lv[i];
+            if (!grads->feature_weight[i] && !grads->mask_weight[i]) continue;
+            ReduceLevel& r = rt.lv[n++];
+            r.part      = reinterpret_cast<const float*>(ws + lv.part_off);
+            r.sliced    = reinterpret_cast<float*>(ws + lv.sliced_off);
+            r.groups    = d.batch * lv.groups;
+            r.total     = 9 * lv.npad * lv.cin_pad;
+            r.cout = lv.cout, r.cin_real = lv.cin_real, r.cin_pad = lv.cin_pad, r.npad = lv.npad;
+            r.d_wf = grads->feature_weight[i], r.d_wm = grads->mask_weight[i];
+            const bool bias = grads->feature_bias[i] || grads->mask_bias[i];
+            r.bias_part = bias ? reinterpret_cast<const float*>(ws + lv.bias_part_off) : nullptr;
+            r.d_bf = grads->feature_bias[i], r.d_bm = grads->mask_bias[i];
+            most      = std::max(most, r.total);
+            most_npad = std::max(most_npad, lv.npad);
+        }
+        if (n > 0)
+        {
+            hipLaunchKernelGGL(reduce_weight_grad_slices_kernel, dim3((most + 255) / 256, kReduceSlices, n), dim3(256), 0, stream, rt);
+            hipLaunchKernelGGL(reduce_weight_grad_kernel, dim3((most + 255) / 256 + most_npad, 1, n), dim3(256), 0, stream, rt);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return set_error(TRIPS_ERR_HIP, "gradient sums launch: %s", hipGetErrorString(e));
+        }
     }
     return TRIPS_OK;
 }

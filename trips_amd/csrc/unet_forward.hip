@@ -292,12 +292,29 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     }
 }
 
-// wpack[tap][n][c]: n < NPAD/2 feature output n, else mask output n - NPAD/2; zero outside the real ranges
-__global__ __launch_bounds__(256) void pack_conv_weights_kernel(const float* __restrict__ wf, const float* __restrict__ bf,
-                                                                const float* __restrict__ wm, const float* __restrict__ bm,
-                                                                int cout, int cin_real, int cin_pad, int npad,
-                                                                _Float16* __restrict__ wpack, float* __restrict__ bias)
+// wpack[tap][n][c]: n < NPAD/2 feature output n, else mask output n - NPAD/2; zero outside the real ranges.
+// All levels in one launch, the level is blockIdx.y (a launch per level costs more than the work itself).
+struct PackLevel
 {
+    const float *wf, *bf, *wm, *bm;
+    int cout, cin_real, cin_pad, npad;
+    _Float16* wpack;
+    float* bias;
+};
+struct PackTable
+{
+    PackLevel lv[TRIPS_UNET_MAX_LEVELS];
+};
+__global__ __launch_bounds__(256) void pack_conv_weights_kernel(const PackTable t)
+{
+    const PackLevel& l = t.lv[blockIdx.y];
+    const float* __restrict__ wf = l.wf;
+    const float* __restrict__ bf = l.bf;
+    const float* __restrict__ wm = l.wm;
+    const float* __restrict__ bm = l.bm;
+    const int cout = l.cout, cin_real = l.cin_real, cin_pad = l.cin_pad, npad = l.npad;
+    _Float16* __restrict__ wpack = l.wpack;
+    float* __restrict__ bias     = l.bias;
     const int total = 9 * npad * cin_pad;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256)
     {
@@ -424,15 +441,17 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
 
     {
         ProfScope ps(prof, "unet_pack_weights", stream);
+        PackTable pt;
+        int most = 0;
         for (int i = 0; i < L; ++i)
         {
             const LevelPlan& lv = np.lv[i];
-            const int total     = 9 * lv.npad * lv.cin_pad;
-            hipLaunchKernelGGL(pack_conv_weights_kernel, dim3((total + 255) / 256), dim3(256), 0, stream,
-                               weights->feature_weight[i], weights->feature_bias[i], weights->mask_weight[i],
-                               weights->mask_bias[i], lv.cout, lv.cin_real, lv.cin_pad, lv.npad,
-                               reinterpret_cast<_Float16*>(ws + lv.wpack_off), reinterpret_cast<float*>(ws + lv.bias_off));
+            pt.lv[i] = PackLevel{weights->feature_weight[i], weights->feature_bias[i], weights->mask_weight[i], weights->mask_bias[i],
+                                 lv.cout, lv.cin_real, lv.cin_pad, lv.npad, reinterpret_cast<_Float16*>(ws + lv.wpack_off),
+                                 reinterpret_cast<float*>(ws + lv.bias_off)};
+            most     = std::max(most, 9 * lv.npad * lv.cin_pad);
         }
+        hipLaunchKernelGGL(pack_conv_weights_kernel, dim3((most + 255) / 256, L), dim3(256), 0, stream, pt);
     }
     static const char* const kLevelNames[TRIPS_UNET_MAX_LEVELS] = {"unet_conv_l0", "unet_conv_l1", "unet_conv_l2", "unet_conv_l3",
                                                                    "unet_conv_l4", "unet_conv_l5", "unet_conv_l6", "unet_conv_l7"};
