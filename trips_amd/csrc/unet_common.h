@@ -18,7 +18,7 @@ constexpr int kConvPatchH  = kConvTileH + 2;
 constexpr int kConvPatchW  = kConvTileW + 2;
 constexpr int kBelowH      = kConvTileH / 2 + 2;  // rows / columns of the level below that an upsampled patch touches
 constexpr int kBelowW      = kConvTileW / 2 + 2;
-constexpr int kFinalPixelsPerBlock = 2048;  // pixels a workgroup of the 1x1 convolution's backward takes at a time
+constexpr int kFinalPixelsPerBlock = 512;   // pixels a workgroup of the 1x1 convolution's backward takes at a time
 constexpr int kFinalPartFloats     = 4 * (4 + 64) + 4;  // its partial sums: [4 outputs][4 image + <= 64 block channels], 4 biases
 constexpr int kLdsChanPad  = 8;  // halves added to every LDS row so that 16 lanes reading 16 bytes hit 64 distinct banks
 
@@ -270,7 +270,9 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
     }
     {
         const size_t chunks = ((size_t)np.lv[0].H * np.lv[0].W + kFinalPixelsPerBlock - 1) / kFinalPixelsPerBlock;
-        np.final_groups     = chunks < 1024 ? (int)chunks : 1024;
+        // as many workgroups as are resident at once (three per CU at the kernel's 160 registers) walk the chunks: a
+        // second, partly filled round of one-chunk workgroups cost a third of the kernel's time
+        np.final_groups     = chunks < 768 ? (int)chunks : 768;
         np.final_part_off   = bw;
         bw += align256((size_t)d.batch * np.final_groups * kFinalPartFloats * sizeof(float));
     }
