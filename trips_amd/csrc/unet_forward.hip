@@ -38,7 +38,7 @@ struct ConvParams
     const _Float16* act_below;  // [Hb][Wb][cb_store]
     const _Float16* wpack;    // [9][NPAD][CIN]
     const float* bias;        // [NPAD]: feature biases, then mask biases, each padded to NPAD / 2
-    _Float16* out;            // [H][W][cout_store]
+    _Float16* out;            // [H][W][cout_store], or nullptr when only the fused 1x1 consumes the block's output
     _Float16* pre;            // [H][W][NPAD] pre-activations (feature | mask) for the backward, or nullptr
     // the finest block also applies the net's 1x1 output convolution to x_0 = cat(image, block output)
     const float* final_w;     // [final_cout][C + cout] or nullptr
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         }
     }
     __syncthreads();
-    store_tile_nhwc(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
+    if (p.out) store_tile_nhwc(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
     if (p.pre) store_tile_nhwc(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
     if (p.final_out)
     {
@@ -471,7 +471,8 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
             p.feat       = inputs[i] + (size_t)b * C * lv.H * lv.W;
             p.wpack      = reinterpret_cast<const _Float16*>(ws + lv.wpack_off);
             p.bias       = reinterpret_cast<const float*>(ws + lv.bias_off);
-            p.out        = act_ptr(i, b);
+            // (without a saved state nobody reads the finest block's output again: its 1x1 runs in the same kernel)
+            p.out        = (i == 0 && !sv) ? nullptr : act_ptr(i, b);
             p.pre        = sv ? reinterpret_cast<_Float16*>(sv + lv.saved_pre_off) + (size_t)b * lv.H * lv.W * lv.npad : nullptr;
             if (i < L - 1)
             {
