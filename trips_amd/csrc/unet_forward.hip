@@ -76,21 +76,71 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     _Float16* s_below    = s_patch + kConvPatchH * kConvPatchW * ROW;  // [kBelowH * kBelowW][ROW]
     const int by0 = y0 / 2 - 1, bx0 = x0 / 2 - 1;
     const int C   = p.c_feat;
+    // (first every load into registers, then the conversions and LDS stores: written as loops that load and store
+    // item by item, a thread's five round trips to memory ran one after the other and stage 1 was 39 % of a
+    // workgroup's life)
+    constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + 255) / 256;
+    constexpr int kMaxPerPix  = 1 + CIN / 8;  // image below + groups of 8 block outputs
+    constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + 255) / 256;
+    float feat_v[kFeatItems][4];
+    uint4 below_v[kBelowItems];
+    const int act_groups = has_below ? p.cb_store / 8 : 0;
+    const int per_pixel  = 1 + act_groups;  // item 0 of a pixel: the image below; others: 8 activations each
     {
         const size_t plane = (size_t)p.H * p.W;
-        for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW; item += 256)
+#pragma unroll
+        for (int k = 0; k < kFeatItems; ++k)
         {
+            const int item = threadIdx.x + 256 * k;
             const int py = item / kConvPatchW, px = item - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
-            const bool in = y >= 0 && y < p.H && x >= 0 && x < p.W;
-            float v[4] = {0.f, 0.f, 0.f, 0.f};
-            if (in)
-                for (int c = 0; c < C; ++c) v[c] = p.feat[c * plane + (size_t)y * p.W + x];
+            const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) feat_v[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+        }
+    }
+    if (has_below)
+    {
+        const size_t pb = (size_t)p.Hb * p.Wb;
+#pragma unroll
+        for (int k = 0; k < kBelowItems; ++k)
+        {
+            const int item = threadIdx.x + 256 * k;
+            below_v[k]     = make_uint4(0u, 0u, 0u, 0u);
+            if (item < kBelowH * kBelowW * per_pixel)
+            {
+                const int q = item % per_pixel, bp = item / per_pixel;
+                const int r = bp / kBelowW, c0 = bp - r * kBelowW;
+                const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
+                if (q == 0)
+                {
+                    const float* src = p.feat_below + (size_t)yy * p.Wb + xx;
+                    float f[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) f[c] = c < C ? src[c * pb] : 0.f;
+                    below_v[k] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+                }
+                else
+                    below_v[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kFeatItems; ++k)
+    {
+        const int item = threadIdx.x + 256 * k;
+        if (item < kConvPatchH * kConvPatchW)
+        {
             _Float16* row = s_patch + (size_t)item * ROW;
             if (C == 4)  // one 8-byte LDS store instead of four 2-byte ones
-                *reinterpret_cast<half4*>(row) = half4{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3])};
+                *reinterpret_cast<half4*>(row) =
+                    half4{_Float16(feat_v[k][0]), _Float16(feat_v[k][1]), _Float16(feat_v[k][2]), _Float16(feat_v[k][3])};
             else
-                for (int c = 0; c < C; ++c) row[c] = _Float16(v[c]);
+            {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)  // (a run-time bound would put the register array into scratch memory)
+                    if (c < C) row[c] = _Float16(feat_v[k][c]);
+            }
             if (!has_below)
             {
                 // start block: the image is the whole input
@@ -100,36 +150,40 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     }
     if (has_below)
     {
-        const size_t pb = (size_t)p.Hb * p.Wb;
-        const int act_groups = p.cb_store / 8;
-        const int per_pixel  = 1 + act_groups;  // item 0 of a pixel: the image below; others: 8 activations each
-        for (int item = threadIdx.x; item < kBelowH * kBelowW * per_pixel; item += 256)
+#pragma unroll
+        for (int k = 0; k < kBelowItems; ++k)
         {
-            const int q = item % per_pixel, bp = item / per_pixel;
-            const int r = bp / kBelowW, c0 = bp - r * kBelowW;
-            const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
-            _Float16* row = s_below + (size_t)bp * ROW;
-            if (q == 0)
+            const int item = threadIdx.x + 256 * k;
+            if (item < kBelowH * kBelowW * per_pixel)
             {
-                if (C == 4)
+                const int q = item % per_pixel, bp = item / per_pixel;
+                _Float16* row = s_below + (size_t)bp * ROW;
+                if (q == 0)
                 {
-                    const float* src = p.feat_below + (size_t)yy * p.Wb + xx;
-                    const float v0 = src[0], v1 = src[pb], v2 = src[2 * pb], v3 = src[3 * pb];
-                    *reinterpret_cast<half4*>(row + 4) = half4{_Float16(v0), _Float16(v1), _Float16(v2), _Float16(v3)};
+                    const float f[4] = {__uint_as_float(below_v[k].x), __uint_as_float(below_v[k].y), __uint_as_float(below_v[k].z),
+                                        __uint_as_float(below_v[k].w)};
+                    if (C == 4)
+                        *reinterpret_cast<half4*>(row + 4) = half4{_Float16(f[0]), _Float16(f[1]), _Float16(f[2]), _Float16(f[3])};
+                    else
+                    {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            if (c < C) row[C + c] = _Float16(f[c]);
+                    }
+                    for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);  // padding channels
                 }
                 else
-                    for (int c = 0; c < C; ++c) row[C + c] = _Float16(p.feat_below[c * pb + (size_t)yy * p.Wb + xx]);
-                for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);  // padding channels
-            }
-            else
-            {
-                const half8 a = *reinterpret_cast<const half8*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
-                const int pos = 2 * C + 8 * (q - 1);
-                if (C == 4)
-                    *reinterpret_cast<half8*>(row + pos) = a;
-                else
-                    for (int i = 0; i < 8; ++i)
-                        if (pos + i < CIN) row[pos + i] = a[i];
+                {
+                    const int pos = 2 * C + 8 * (q - 1);
+                    if (C == 4)
+                        *reinterpret_cast<uint4*>(row + pos) = below_v[k];
+                    else
+                    {
+                        const half8 a = __builtin_bit_cast(half8, below_v[k]);
+                        for (int i = 0; i < 8; ++i)
+                            if (pos + i < CIN) row[pos + i] = a[i];
+                    }
+                }
             }
         }
         __syncthreads();
