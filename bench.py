@@ -30,16 +30,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "65468a1844737f5fddf9488656588c43326a26457a5987d81cf449e8b8262a8b"
+PMC_SOURCES_SHA256 = "5e5e906da63461331ec4e034c6bceacffd70f74c28801fc5e50d47596e5b1350"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129129, 271476),
-    "bin_scatter": (87944, 186054),
+    "project_bin": (129133, 271433),
+    "bin_scatter": (87912, 186198),
     "tile_count": (26200, 2296),
-    "tile_scatter": (70420, 115408),
-    "sort_blend": (334593, 417430),
-    "backward_pixels": (498577, 165610),
-    "backward_points": (1045046, 234887),
-    "adam_fused": (582964, 792823),
+    "tile_scatter": (70861, 114521),
+    "sort_blend": (333873, 417473),
+    "backward_pixels": (498794, 165612),
+    "backward_points": (1045013, 234887),
+    "adam_fused": (582965, 792823),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")

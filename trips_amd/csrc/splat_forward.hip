@@ -9,12 +9,14 @@
 //
 // Differences in shape, not in result. The reference increments one global counter per (point, layer, corner),
 // scans layer by layer with two blocking read-backs each, and takes one more global atomic per entry to place
-// its key. Scattered global atomics run at about 2.7e10 per second on this GPU, so here a point is first binned
-// into 32 x 32 pixel tiles (one global atomic per (point, layer), a second one for the few footprints that cross
-// a tile border); a workgroup per tile then counts, scans and places the keys of its 1024 pixels with LDS
-// atomics. A wavefront of the sort holds four pixel lists of 16 lanes (one DPP row each) instead of two per
-// 32-lane warp; the per-point record gathered by the blend carries position, size, confidence and descriptor
-// together; what is kept for the backward is the sorted id list per pixel (64 B) instead of 16 x 7 floats.
+// its key. Scattered global atomics run at about 2.7e10 per second on this GPU, so here a (point, layer) pair is
+// first binned, once, into the 32 x 32 pixel tile of its footprint's first pixel (workgroup-private LDS histograms
+// and a column scan: no global atomics); a workgroup per tile then counts, scans and places the keys of its 1024
+// cells with LDS atomics, one key per pair, and the blend gathers a pixel's list from the four cells whose
+// footprints cover it. A wavefront of the sort holds four pixel lists of 16 lanes (one DPP row each, or eight of 8
+// lanes) instead of two per 32-lane warp; the per-point record gathered by the blend carries position, size,
+// confidence and descriptor together; what is kept for the backward is the sorted id list per pixel (64 B) instead
+// of 16 x 7 floats.
 #include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"

@@ -90,7 +90,7 @@ struct TripsCtx
 namespace trips
 {
 // Per-point records written by the projection kernel, for the VALID points of a view only, at the point's compact
-// number cid (see wave_point_range: dense runs in point order; cid_of / pid_of translate). The 64-bit sort key of a
+// number cid (see chunk_point_range: dense runs in point order; cid_of / pid_of translate). The 64-bit sort key of a
 // list entry is depth bits << 32 | cid: cid grows with the point id, so the order is that of depth bits << 32 |
 // point id.
 //   rec[cid]   4 + Cpad floats {ip.x, ip.y, size field (see encode_size_field), confidence, descriptor[0..C)}:
