@@ -602,19 +602,20 @@ __device__ __forceinline__ void lds_read_pixel_windows(const _Float16* tile, int
     w[2] = out.h;
 }
 
-template <int CIN, int NPAD, bool BIAS>
-__global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightParams p)
+// THREADS: 256, or 512 for the largest shape, whose 9 x NPAD x CIN sums are 288 registers per lane of four wavefronts.
+template <int CIN, int NPAD, bool BIAS, int THREADS>
+__global__ __launch_bounds__(THREADS) void conv_bwd_weight_kernel(const BwdWeightParams p)
 {
     constexpr int ROW    = CIN + kLdsChanPad;   // halves per pixel of the input patch
     constexpr int DS     = NPAD + kLdsChanPad;  // halves per pixel of the gradient tile
     constexpr int GROUPS = CIN / 8;
     constexpr int NB     = NPAD / 16;
     constexpr int CB     = CIN / 16;
-    // The 4 wavefronts split the NPAD x CIN result: CBW ways over the 16-channel input blocks, NBW ways over the
+    // The wavefronts split the NPAD x CIN result: CBW ways over the 16-channel input blocks, NBW ways over the
     // 16-channel pre-activation blocks; each keeps all 9 taps of its blocks. Per tile row a wavefront reads its A
     // fragments (pre-activation gradients, the same for every tap) once and one B fragment per tap and input block.
     constexpr int CBW    = CB < 4 ? CB : 4;
-    constexpr int NBW    = 4 / CBW;
+    constexpr int NBW    = (THREADS / 64) / CBW;
     constexpr int MYCB   = CB / CBW;
     constexpr int MYNB   = NB / NBW;
     static_assert(CB % CBW == 0 && NB % NBW == 0, "block split");
@@ -648,10 +649,11 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     // ---- stage 1 in two halves: every global load of a tile is issued into registers (a thread's loads are all in
     // flight together), and written to LDS one tile later, so that the loads of tile t + 1 travel while tile t is
     // upsampled and multiplied ----
-    constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + 255) / 256;
+    constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + THREADS - 1) / THREADS;
     constexpr int kMaxPerPix  = 1 + (CIN - 8) / 8;  // image below + groups of 8 block outputs (C = 4)
-    constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + 255) / 256;
-    constexpr int kDpreItems  = NPAD / 8;
+    constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + THREADS - 1) / THREADS;
+    constexpr int kDpreGroups = NPAD / 8;  // 16-byte groups of a pixel's gradient row
+    constexpr int kDpreItems  = (kConvTileH * kConvTileW * kDpreGroups + THREADS - 1) / THREADS;
     struct TileLoads
     {
         float feat[kFeatItems][4];
@@ -669,7 +671,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
         for (int k = 0; k < kFeatItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
+            const int item = threadIdx.x + THREADS * k;
             const int py = item / kConvPatchW, px = item - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
             const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
@@ -682,7 +684,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
             for (int k = 0; k < kBelowItems; ++k)
             {
-                const int item = threadIdx.x + 256 * k;
+                const int item = threadIdx.x + THREADS * k;
                 r.below[k]     = make_uint4(0u, 0u, 0u, 0u);
                 if (item < kBelowH * kBelowW * per_pixel)
                 {
@@ -704,12 +706,13 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
         for (int k = 0; k < kDpreItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
-            const int g = item % kDpreItems, tp = item / kDpreItems;
+            const int item = threadIdx.x + THREADS * k;
+            const int g = item % kDpreGroups, tp = item / kDpreGroups;
             const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
 #pragma unroll
             for (int i = 0; i < 8; ++i) r.dpre[k][i] = _Float16(0.f);
-            if (y < p.H && x < p.W) r.dpre[k] = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * NPAD + 8 * g);
+            if (tp < kConvTileH * kConvTileW && y < p.H && x < p.W)
+                r.dpre[k] = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * NPAD + 8 * g);
         }
     };
     // this level's image into channels [0, C) of a patch pixel (the channels [C, 8) follow from the upsampling, or are
@@ -747,7 +750,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
         for (int k = 0; k < kFeatItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
+            const int item = threadIdx.x + THREADS * k;
             if (item < kConvPatchH * kConvPatchW) put_image(item, r.feat[k]);
         }
         if (has_below)
@@ -755,7 +758,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
             for (int k = 0; k < kBelowItems; ++k)
             {
-                const int item = threadIdx.x + 256 * k;
+                const int item = threadIdx.x + THREADS * k;
                 if (item < kBelowH * kBelowW * per_pixel)
                 {
                     const int q = item % per_pixel, bp = item / per_pixel;
@@ -773,8 +776,9 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 #pragma unroll
         for (int k = 0; k < kDpreItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
-            *reinterpret_cast<half8*>(s_d + (size_t)(item / kDpreItems) * DS + 8 * (item % kDpreItems)) = r.dpre[k];
+            const int item = threadIdx.x + THREADS * k;
+            if (item < kConvTileH * kConvTileW * kDpreGroups)
+                *reinterpret_cast<half8*>(s_d + (size_t)(item / kDpreGroups) * DS + 8 * (item % kDpreGroups)) = r.dpre[k];
         }
     };
 
@@ -783,7 +787,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
     {
         {
             const size_t plane = (size_t)p.H * p.W;
-            for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW; item += 256)
+            for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW; item += THREADS)
             {
                 const int py = item / kConvPatchW, px = item - py * kConvPatchW;
                 const int y = y0 + py - 1, x = x0 + px - 1;
@@ -797,7 +801,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
         if (has_below)
         {
             const size_t pb = (size_t)p.Hb * p.Wb;
-            for (int item = threadIdx.x; item < kBelowH * kBelowW * per_pixel; item += 256)
+            for (int item = threadIdx.x; item < kBelowH * kBelowW * per_pixel; item += THREADS)
             {
                 const int q = item % per_pixel, bp = item / per_pixel;
                 const int r = bp / kBelowW, c0 = bp - r * kBelowW;
@@ -816,9 +820,9 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
                 }
             }
         }
-        for (int item = threadIdx.x; item < kConvTileH * kConvTileW * kDpreItems; item += 256)
+        for (int item = threadIdx.x; item < kConvTileH * kConvTileW * kDpreGroups; item += THREADS)
         {
-            const int g = item % kDpreItems, tp = item / kDpreItems;
+            const int g = item % kDpreGroups, tp = item / kDpreGroups;
             const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
             half8 v;
 #pragma unroll
@@ -830,7 +834,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
 
     // start block: the channels beyond the first eight of a patch pixel are never written and stay zero
     if (!has_below)
-        for (int i = threadIdx.x; i < kConvPatchH * kConvPatchW * (GROUPS - 1); i += 256)
+        for (int i = threadIdx.x; i < kConvPatchH * kConvPatchW * (GROUPS - 1); i += THREADS)
         {
             half8 z;
 #pragma unroll
@@ -858,7 +862,7 @@ __global__ __launch_bounds__(256) void conv_bwd_weight_kernel(const BwdWeightPar
             __syncthreads();
             // ---- stage 2: bilinear 2x upsampling from the below patch into channels [C, CIN) of the patch, in packed
             // fp16 exactly as the forward kernel does it (the weights are products of 0, 1/4, 3/4 and 1) ----
-            for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
+            for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += THREADS)
             {
                 const int g = item % GROUPS, pp = item / GROUPS;
                 const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
@@ -1058,13 +1062,14 @@ hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipS
 template <int CIN, int NPAD, bool BIAS>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
+    constexpr int THREADS = (CIN == 64 && NPAD == 128) ? 512 : 256;
     const size_t lds = ((size_t)(kConvPatchH * kConvPatchW + kBelowH * kBelowW) * (CIN + kLdsChanPad) +
                         (size_t)kConvTileH * kConvTileW * (NPAD + kLdsChanPad)) *
                        sizeof(_Float16);  // up to 133 KB
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD, BIAS>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD, BIAS, THREADS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD, BIAS>), dim3(groups), dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD, BIAS, THREADS>), dim3(groups), dim3(THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
