@@ -1062,7 +1062,7 @@ hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipS
 template <int CIN, int NPAD, bool BIAS>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
-    constexpr int THREADS = (CIN == 64 && NPAD == 128) ? 512 : 256;
+    constexpr int THREADS = (CIN == 64 && NPAD >= 64) ? 512 : 256;
     const size_t lds = ((size_t)(kConvPatchH * kConvPatchW + kBelowH * kBelowW) * (CIN + kLdsChanPad) +
                         (size_t)kConvTileH * kConvTileW * (NPAD + kLdsChanPad)) *
                        sizeof(_Float16);  // up to 133 KB
