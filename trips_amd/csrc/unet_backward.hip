@@ -604,7 +604,7 @@ __device__ __forceinline__ void lds_read_pixel_windows(const _Float16* tile, int
 
 // THREADS: 256, or 512 for the largest shape, whose 9 x NPAD x CIN sums are 288 registers per lane of four wavefronts.
 template <int CIN, int NPAD, bool BIAS, int THREADS>
-__global__ __launch_bounds__(THREADS) void conv_bwd_weight_kernel(const BwdWeightParams p)
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 32 && NPAD == 32 ? 4 : 1))) void conv_bwd_weight_kernel(const BwdWeightParams p)
 {
     constexpr int ROW    = CIN + kLdsChanPad;   // halves per pixel of the input patch
     constexpr int DS     = NPAD + kLdsChanPad;  // halves per pixel of the gradient tile
@@ -615,10 +615,16 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_weight_kernel(const BwdWeigh
     // 16-channel pre-activation blocks; each keeps all 9 taps of its blocks. Per tile row a wavefront reads its A
     // fragments (pre-activation gradients, the same for every tap) once and one B fragment per tap and input block.
     constexpr int CBW    = CB < 4 ? CB : 4;
-    constexpr int NBW    = (THREADS / 64) / CBW;
+    // (More wavefronts than 16 x 16 blocks to deal out: the wavefronts also split the rows of a tile, RW ways, and every
+    // row share writes a set of partial sums of its own.)
+    constexpr int WAVES  = THREADS / 64;
+    constexpr int NBW    = wgrad_nbw(CIN, NPAD);
+    constexpr int RW     = wgrad_row_split(CIN, NPAD);
+    static_assert(THREADS == wgrad_threads(CIN, NPAD) && CBW == wgrad_cbw(CIN), "work split");
     constexpr int MYCB   = CB / CBW;
     constexpr int MYNB   = NB / NBW;
-    static_assert(CB % CBW == 0 && NB % NBW == 0, "block split");
+    constexpr int MYROWS = kConvTileH / RW;
+    static_assert(CB % CBW == 0 && NB % NBW == 0 && CBW * NBW * RW == WAVES && kConvTileH % RW == 0, "block split");
     extern __shared__ _Float16 smem[];
     _Float16* s_patch = smem;                                           // [kConvPatchH * kConvPatchW][ROW]
     _Float16* s_below = s_patch + kConvPatchH * kConvPatchW * ROW;      // [kBelowH * kBelowW][ROW]
@@ -628,7 +634,10 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_weight_kernel(const BwdWeigh
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lk = (lane >> 4) * 8;
 
-    const int cb0 = (wave % CBW) * MYCB, nb0 = (wave / CBW) * MYNB;
+    const int cb0 = (wave % CBW) * MYCB, nb0 = (RW == 1 ? wave / CBW : (wave / CBW) % NBW) * MYNB;
+    const int share = RW == 1 ? 0 : wave / (CBW * NBW);
+    const int row0  = share * MYROWS;           // this wavefront's rows of a tile
+    const int set   = blockIdx.x * RW + share;  // ... and its set of partial sums
     floatx4 acc[9][MYNB][MYCB];
 #pragma unroll
     for (int t = 0; t < 9; ++t)
@@ -902,7 +911,7 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_weight_kernel(const BwdWeigh
         __syncthreads();
         // ---- dW[tap][n][c] += sum over the tile's pixels of dpre[pixel][n] * x[pixel + tap][c] ----
 #pragma unroll
-        for (int r = 0; r < kConvTileH; ++r)
+        for (int r = row0; r < row0 + MYROWS; ++r)
         {
             half8 a[MYNB];
 #pragma unroll
@@ -932,13 +941,13 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_weight_kernel(const BwdWeigh
     if (BIAS && cb0 == 0 && (lane & 15) == 0)
     {
         // column 0 of the row sums: this lane holds rows (lane / 16) * 4 .. + 3 of every block
-        float* dst = p.bias_part + (size_t)blockIdx.x * NPAD;
+        float* dst = p.bias_part + (size_t)set * NPAD;
 #pragma unroll
         for (int n = 0; n < MYNB; ++n)
 #pragma unroll
             for (int i = 0; i < 4; ++i) dst[(nb0 + n) * 16 + (lane >> 4) * 4 + i] = bias_acc[n][i];
     }
-    float* part = p.part + (size_t)blockIdx.x * 9 * NPAD * CIN;
+    float* part = p.part + (size_t)set * 9 * NPAD * CIN;
     const int lrow = lane & 15;
     // (the input channels are the rows of the MFMA result: a lane holds four neighbouring ones of output lrow)
 #pragma unroll
@@ -1062,7 +1071,9 @@ hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipS
 template <int CIN, int NPAD, bool BIAS>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
-    constexpr int THREADS = (CIN == 64 && NPAD >= 64) ? 512 : 256;
+    // `groups` counts sets of partial sums: two per workgroup where the wavefronts also split the rows
+    constexpr int THREADS = wgrad_threads(CIN, NPAD);
+    groups /= wgrad_row_split(CIN, NPAD);
     const size_t lds = ((size_t)(kConvPatchH * kConvPatchW + kBelowH * kBelowW) * (CIN + kLdsChanPad) +
                         (size_t)kConvTileH * kConvTileW * (NPAD + kLdsChanPad)) *
                        sizeof(_Float16);  // up to 133 KB
