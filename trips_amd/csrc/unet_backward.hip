@@ -615,8 +615,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
     // 16-channel pre-activation blocks; each keeps all 9 taps of its blocks. Per tile row a wavefront reads its A
     // fragments (pre-activation gradients, the same for every tap) once and one B fragment per tap and input block.
     constexpr int CBW    = CB < 4 ? CB : 4;
-    // (More wavefronts than 16 x 16 blocks to deal out: the wavefronts also split the rows of a tile, RW ways, and every
-    // row share writes a set of partial sums of its own.)
+    // (More wavefronts than 16 x 16 blocks to deal out: the wavefronts also split the rows of a tile, RW ways; the
+    // shares are added up through LDS at the end.)
     constexpr int WAVES  = THREADS / 64;
     constexpr int NBW    = wgrad_nbw(CIN, NPAD);
     constexpr int RW     = wgrad_row_split(CIN, NPAD);
@@ -637,7 +637,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
     const int cb0 = (wave % CBW) * MYCB, nb0 = (RW == 1 ? wave / CBW : (wave / CBW) % NBW) * MYNB;
     const int share = RW == 1 ? 0 : wave / (CBW * NBW);
     const int row0  = share * MYROWS;           // this wavefront's rows of a tile
-    const int set   = blockIdx.x * RW + share;  // ... and its set of partial sums
+    const int set   = blockIdx.x;               // the workgroup's set of partial sums
     floatx4 acc[9][MYNB][MYCB];
 #pragma unroll
     for (int t = 0; t < 9; ++t)
@@ -938,6 +938,37 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
         }
     }
 
+    if (RW > 1)
+    {
+        // the row shares of a workgroup add their sums up through LDS (the tiles are consumed), so that the workgroup
+        // writes one set: share s > 0 leaves its registers there, share 0 adds them
+        static_assert(RW <= 2, "row shares");
+        __syncthreads();
+        floatx4* s_sum = reinterpret_cast<floatx4*>(smem);  // [wavefront of the share][tap and bias][block][lane]
+        constexpr int PER_WAVE = (9 * MYNB * MYCB + MYNB) * 64;
+        floatx4* mine = s_sum + (size_t)(wave % (CBW * NBW)) * PER_WAVE + lane;
+        if (share > 0)
+        {
+#pragma unroll
+            for (int t = 0; t < 9; ++t)
+#pragma unroll
+                for (int n = 0; n < MYNB; ++n)
+#pragma unroll
+                    for (int c = 0; c < MYCB; ++c) mine[((t * MYNB + n) * MYCB + c) * 64] = acc[t][n][c];
+#pragma unroll
+            for (int n = 0; n < MYNB; ++n) mine[(9 * MYNB * MYCB + n) * 64] = bias_acc[n];
+        }
+        __syncthreads();
+        if (share > 0) return;
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+#pragma unroll
+            for (int n = 0; n < MYNB; ++n)
+#pragma unroll
+                for (int c = 0; c < MYCB; ++c) acc[t][n][c] += mine[((t * MYNB + n) * MYCB + c) * 64];
+#pragma unroll
+        for (int n = 0; n < MYNB; ++n) bias_acc[n] += mine[(9 * MYNB * MYCB + n) * 64];
+    }
     if (BIAS && cb0 == 0 && (lane & 15) == 0)
     {
         // column 0 of the row sums: this lane holds rows (lane / 16) * 4 .. + 3 of every block
@@ -1071,9 +1102,7 @@ hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipS
 template <int CIN, int NPAD, bool BIAS>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
-    // `groups` counts sets of partial sums: two per workgroup where the wavefronts also split the rows
     constexpr int THREADS = wgrad_threads(CIN, NPAD);
-    groups /= wgrad_row_split(CIN, NPAD);
     const size_t lds = ((size_t)(kConvPatchH * kConvPatchW + kBelowH * kBelowW) * (CIN + kLdsChanPad) +
                         (size_t)kConvTileH * kConvTileW * (NPAD + kLdsChanPad)) *
                        sizeof(_Float16);  // up to 133 KB

@@ -150,8 +150,7 @@ __device__ __forceinline__ void store_tile_nhwc(const _Float16* s_tile, int lds_
 
 // Work split of the weight-gradient kernel for a (padded input channels, padded pre-activations) shape: threads per
 // workgroup; how many ways the wavefronts split the 16-channel input blocks, the 16-channel pre-activation blocks and,
-// where there are more wavefronts than blocks, the rows of a tile (every row share keeps a set of partial sums of its
-// own).
+// where there are more wavefronts than blocks, the rows of a tile.
 constexpr int wgrad_threads(int cin, int npad) { return (cin == 32 && npad == 96) ? 256 : 512; }
 constexpr int wgrad_cbw(int cin) { return cin / 16 < 4 ? cin / 16 : 4; }
 constexpr int wgrad_nbw(int cin, int npad)
@@ -175,7 +174,7 @@ struct LevelPlan
     size_t part_off;    // partial weight gradients [groups][9][npad][cin_pad] fp32
     size_t sliced_off;  // partial sums of the partials [16][9][npad][cin_pad] fp32
     size_t bias_part_off;  // per-workgroup sums of the pre-activation gradients [batch * groups][npad] fp32
-    int groups;         // sets of partial sums of the weight-gradient kernel (per image): its persistent workgroups x their row shares
+    int groups;         // persistent workgroups of the weight-gradient kernel (per image)
 };
 
 struct NetPlan
@@ -272,8 +271,7 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
         // persistent workgroups of the weight-gradient kernel: as many as are resident at once (two per CU for the
         // smallest shape, else one); every further one would only add a set of partial sums to write and reduce
         const int resident = (lv.cin_pad * lv.npad <= 1024 ? 2 : 1) * 256;
-        // (counted in sets of partial sums: the workgroups times the row shares of each)
-        lv.groups          = (tiles < resident ? tiles : resident) * wgrad_row_split(lv.cin_pad, lv.npad);
+        lv.groups          = tiles < resident ? tiles : resident;
         lv.part_off     = bw;
         bw += align256((size_t)d.batch * lv.groups * 9 * lv.npad * lv.cin_pad * sizeof(float));
         lv.sliced_off = bw;
