@@ -45,42 +45,45 @@ __device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i
 // reads its fragments from there: a quarter of the L2 traffic, the same bank-conflict-free row layout as the patch.
 // A wavefront owns two rows of the 8 x 32 output tile = four 16-pixel row blocks; acc[m][n] is the 16 x 16 block of
 // pixels m, outputs 16n .. 16n+15.
-template <int KIN, int NOUT>
+// THREADS = threads of the workgroup: 256 (a wavefront owns two rows of the tile = four 16-pixel row blocks) or 512 (one
+// row = two row blocks).
+template <int KIN, int NOUT, int THREADS = 256>
 struct ConvTapStage
 {
     static constexpr int NB    = NOUT / 16;
     static constexpr int KB    = KIN / 32;
     static constexpr int ROW   = KIN + kLdsChanPad;   // halves per output row of a tap in LDS
     static constexpr int ITEMS = NOUT * KIN / 8;      // 16-byte words per tap
-    static constexpr int PER   = (ITEMS + 255) / 256;  // per thread
+    static constexpr int PER   = (ITEMS + THREADS - 1) / THREADS;  // per thread
+    static constexpr int MB    = 16 / (THREADS / 64);  // 16-pixel row blocks of a wavefront
     static constexpr int BUF   = NOUT * ROW;           // halves per tap buffer; the kernel provides two
     half8 r[PER];
 };
 
 // this thread's share of tap `tap` from memory into registers
-template <int KIN, int NOUT>
-__device__ __forceinline__ void conv_tap_fetch(ConvTapStage<KIN, NOUT>& st, const _Float16* __restrict__ wpack, int tap)
+template <int KIN, int NOUT, int THREADS>
+__device__ __forceinline__ void conv_tap_fetch(ConvTapStage<KIN, NOUT, THREADS>& st, const _Float16* __restrict__ wpack, int tap)
 {
-    using S = ConvTapStage<KIN, NOUT>;
+    using S = ConvTapStage<KIN, NOUT, THREADS>;
     const half8* src = reinterpret_cast<const half8*>(wpack + (size_t)tap * NOUT * KIN);
 #pragma unroll
     for (int j = 0; j < S::PER; ++j)
     {
-        const int item = threadIdx.x + 256 * j;
-        if (S::ITEMS % 256 == 0 || item < S::ITEMS) st.r[j] = src[item];
+        const int item = threadIdx.x + THREADS * j;
+        if (S::ITEMS % THREADS == 0 || item < S::ITEMS) st.r[j] = src[item];
     }
 }
 
 // ... and from the registers into a tap buffer
-template <int KIN, int NOUT>
-__device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT>& st, _Float16* s_tap)
+template <int KIN, int NOUT, int THREADS>
+__device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT, THREADS>& st, _Float16* s_tap)
 {
-    using S = ConvTapStage<KIN, NOUT>;
+    using S = ConvTapStage<KIN, NOUT, THREADS>;
 #pragma unroll
     for (int j = 0; j < S::PER; ++j)
     {
-        const int item = threadIdx.x + 256 * j;
-        if (S::ITEMS % 256 == 0 || item < S::ITEMS)
+        const int item = threadIdx.x + THREADS * j;
+        if (S::ITEMS % THREADS == 0 || item < S::ITEMS)
             *reinterpret_cast<half8*>(s_tap + (item / (KIN / 8)) * S::ROW + (item % (KIN / 8)) * 8) = st.r[j];
     }
 }
@@ -90,18 +93,20 @@ __device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT>& st
 // Result layout: lane l holds, of the 16 x 16 block acc[m][n], pixels (l / 16) * 4 .. + 3 of output 16n + l % 16; with
 // OUTPUTS_IN_ROWS (the operands of the MFMA exchanged) outputs 16n + (l / 16) * 4 .. + 3 of pixel l % 16, four
 // neighbouring channels of one pixel, which an epilogue can store as one 8-byte word.
-template <int KIN, int NOUT, bool OUTPUTS_IN_ROWS = false>
+template <int KIN, int NOUT, bool OUTPUTS_IN_ROWS = false, int THREADS = 256>
 __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16* s_taps, const _Float16* __restrict__ wpack,
-                                               ConvTapStage<KIN, NOUT>& st, floatx4 (&acc)[4][NOUT / 16])
+                                               ConvTapStage<KIN, NOUT, THREADS>& st,
+                                               floatx4 (&acc)[ConvTapStage<KIN, NOUT, THREADS>::MB][NOUT / 16])
 {
-    using S = ConvTapStage<KIN, NOUT>;
+    using S = ConvTapStage<KIN, NOUT, THREADS>;
+    constexpr int MB = S::MB;
     constexpr int ROW = KIN + kLdsChanPad;
     constexpr int NB  = S::NB;
     constexpr int KB  = S::KB;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 #pragma unroll
-    for (int m = 0; m < 4; ++m)
+    for (int m = 0; m < MB; ++m)
 #pragma unroll
         for (int n = 0; n < NB; ++n) acc[m][n] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -117,9 +122,9 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
 #pragma unroll
             for (int n = 0; n < NB; ++n) bfrag[n] = *reinterpret_cast<const half8*>(sb + (n * 16 + lrow) * S::ROW + kb * 32 + lk);
 #pragma unroll
-            for (int m = 0; m < 4; ++m)
+            for (int m = 0; m < MB; ++m)
             {
-                const int r = 2 * wave + (m >> 1), cb = (m & 1) * 16;
+                const int r = MB == 4 ? 2 * wave + (m >> 1) : wave, cb = (m & 1) * 16;
                 const half8 a = *reinterpret_cast<const half8*>(s_patch + ((r + dy) * kConvPatchW + cb + lrow + dx) * ROW + kb * 32 + lk);
 #pragma unroll
                 for (int n = 0; n < NB; ++n)
@@ -135,10 +140,11 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
 // Copies `groups` x 8 halves per pixel of an 8 x 32 tile staged in LDS ([256][lds_stride]) to a channels-innermost
 // image ([H][W][dst_stride]) with 16-byte stores: consecutive lanes write consecutive 16 bytes, so a tile row leaves
 // as whole lines (2-byte stores straight from the MFMA result layout cost twice the memory requests).
+template <int THREADS = 256>
 __device__ __forceinline__ void store_tile_nhwc(const _Float16* s_tile, int lds_stride, int groups, _Float16* dst,
                                                 int dst_stride, int x0, int y0, int W, int H)
 {
-    for (int item = threadIdx.x; item < kConvTileH * kConvTileW * groups; item += 256)
+    for (int item = threadIdx.x; item < kConvTileH * kConvTileW * groups; item += THREADS)
     {
         const int g = item % groups, tp = item / groups;
         const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;

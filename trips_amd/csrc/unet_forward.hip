@@ -47,9 +47,10 @@ struct ConvParams
     int final_cout;
 };
 
-template <int CIN, int NPAD>
-__global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
+template <int CIN, int NPAD, int THREADS>
+__global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams p)
 {
+    constexpr int MB = 16 / (THREADS / 64);  // 16-pixel row blocks of a wavefront: two rows of the tile, or one
     constexpr int ROW  = CIN + kLdsChanPad;  // halves per patch pixel in LDS
     constexpr int NB   = NPAD / 16;          // 16-column blocks; the first half are feature outputs
     constexpr int HB   = NB / 2;
@@ -58,14 +59,14 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
     const bool has_below = p.Hb > 0;
-    ConvTapStage<CIN, NPAD> taps;
+    ConvTapStage<CIN, NPAD, THREADS> taps;
     conv_tap_fetch(taps, p.wpack, 0);  // in flight while the patch is assembled
     // weights and biases of the 1x1 output convolution, rounded to fp16 like every other operand
     __shared__ float s_fw[4 * (4 + 64) + 4];
     if (p.final_out)
     {
         const int cin = p.c_feat + p.cout;
-        for (int i = threadIdx.x; i < p.final_cout * cin; i += 256) s_fw[i] = float(_Float16(p.final_w[i]));
+        for (int i = threadIdx.x; i < p.final_cout * cin; i += THREADS) s_fw[i] = float(_Float16(p.final_w[i]));
         if ((int)threadIdx.x < p.final_cout) s_fw[4 * (4 + 64) + threadIdx.x] = p.final_b[threadIdx.x];
     }
 
@@ -79,9 +80,9 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     // (first every load into registers, then the conversions and LDS stores: written as loops that load and store
     // item by item, a thread's five round trips to memory ran one after the other and stage 1 was 39 % of a
     // workgroup's life)
-    constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + 255) / 256;
+    constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + THREADS - 1) / THREADS;
     constexpr int kMaxPerPix  = 1 + CIN / 8;  // image below + groups of 8 block outputs
-    constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + 255) / 256;
+    constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + THREADS - 1) / THREADS;
     float feat_v[kFeatItems][4];
     uint4 below_v[kBelowItems];
     const int act_groups = has_below ? p.cb_store / 8 : 0;
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 #pragma unroll
         for (int k = 0; k < kFeatItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
+            const int item = threadIdx.x + THREADS * k;
             const int py = item / kConvPatchW, px = item - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
             const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 #pragma unroll
         for (int k = 0; k < kBelowItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
+            const int item = threadIdx.x + THREADS * k;
             below_v[k]     = make_uint4(0u, 0u, 0u, 0u);
             if (item < kBelowH * kBelowW * per_pixel)
             {
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 #pragma unroll
     for (int k = 0; k < kFeatItems; ++k)
     {
-        const int item = threadIdx.x + 256 * k;
+        const int item = threadIdx.x + THREADS * k;
         if (item < kConvPatchH * kConvPatchW)
         {
             _Float16* row = s_patch + (size_t)item * ROW;
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
 #pragma unroll
         for (int k = 0; k < kBelowItems; ++k)
         {
-            const int item = threadIdx.x + 256 * k;
+            const int item = threadIdx.x + THREADS * k;
             if (item < kBelowH * kBelowW * per_pixel)
             {
                 const int q = item % per_pixel, bp = item / per_pixel;
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         }
         __syncthreads();
         // ---- stage 2: bilinear 2x upsampling from the below patch into channels [C, CIN) of the patch ----
-        for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += 256)
+        for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += THREADS)
         {
             const int g = item % GROUPS, pp = item / GROUPS;
             const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
@@ -234,8 +235,8 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;
     conv_tap_stage(taps, s_taps);
     __syncthreads();
-    floatx4 acc[4][NB];
-    conv_taps_mfma<CIN, NPAD, true>(s_patch, s_taps, p.wpack, taps, acc);  // a lane: four channels of one pixel
+    floatx4 acc[MB][NB];
+    conv_taps_mfma<CIN, NPAD, true, THREADS>(s_patch, s_taps, p.wpack, taps, acc);  // a lane: four channels of one pixel
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
@@ -245,16 +246,17 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
     _Float16* s_act = smem;                                      // [256][AS]
     _Float16* s_pre = smem + kConvTileH * kConvTileW * AS;       // [256][PS]
     float my_feat[4] = {0.f, 0.f, 0.f, 0.f};  // this thread's pixel of the image, as the convolution saw it (fp16)
-    if (p.final_out)
+    const bool owns_pixel = THREADS == kConvTileH * kConvTileW || (int)threadIdx.x < kConvTileH * kConvTileW;  // one thread per pixel
+    if (p.final_out && owns_pixel)
     {
         const _Float16* row = s_patch + (size_t)((threadIdx.x / kConvTileW + 1) * kConvPatchW + threadIdx.x % kConvTileW + 1) * ROW;
         for (int c = 0; c < C; ++c) my_feat[c] = float(row[c]);
     }
     __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
-    for (int m = 0; m < 4; ++m)
+    for (int m = 0; m < MB; ++m)
     {
-        const int tp = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + lrow;  // this lane's pixel of the block
+        const int tp = (MB == 4 ? 2 * wave + (m >> 1) : wave) * kConvTileW + (m & 1) * 16 + lrow;  // this lane's pixel of the block
 #pragma unroll
         for (int j = 0; j < HB; ++j)
         {
@@ -281,8 +283,8 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         }
     }
     __syncthreads();
-    if (p.out) store_tile_nhwc(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
-    if (p.pre) store_tile_nhwc(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
+    if (p.out) store_tile_nhwc<THREADS>(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
+    if (p.pre) store_tile_nhwc<THREADS>(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
     if (p.final_out)
     {
         // `final` of the net (Networks.h:1129-1131) on the matrix cores: per 16 pixels one MFMA per 32 input channels,
@@ -292,6 +294,7 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         constexpr int KFB = (KF + 31) / 32;
         const int cin     = C + p.cout;
         // the image joins the staged rows (columns NPAD/2 .. NPAD/2 + 7; nobody has read them yet)
+        if (owns_pixel)
         {
             _Float16* row = s_act + (size_t)threadIdx.x * AS + NPAD / 2;
 #pragma unroll
@@ -318,9 +321,9 @@ __global__ __launch_bounds__(256) void gated_conv3x3_kernel(const ConvParams p)
         const size_t plane = (size_t)p.H * p.W;
         const float fb     = lrow < p.final_cout ? s_fw[4 * (4 + 64) + lrow] : 0.f;
 #pragma unroll
-        for (int m = 0; m < 4; ++m)
+        for (int m = 0; m < MB; ++m)
         {
-            const int tp0 = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16;  // first pixel of this 16-pixel block
+            const int tp0 = (MB == 4 ? 2 * wave + (m >> 1) : wave) * kConvTileW + (m & 1) * 16;  // first pixel of this 16-pixel block
             floatx4 o     = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb = 0; kb < KFB; ++kb)
@@ -398,11 +401,14 @@ hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
     const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW * ROW + std::max(kBelowH * kBelowW * ROW, 2 * NPAD * ROW)) * sizeof(_Float16);
     const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NPAD / 2 + kLdsChanPad) + (p.pre ? NPAD + kLdsChanPad : 0)) * sizeof(_Float16);
     const size_t lds     = std::max(lds_in, lds_out);  // up to 104 KB when the largest block saves its pre-activations
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD>),
+    // eight wavefronts per tile (one row each): the phases around the tap loop run at the latency of their loads and LDS
+    // round trips, and twice the wavefronts per tile hide twice as much of it
+    constexpr int THREADS = 512;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD, THREADS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     dim3 grid((p.W + kConvTileW - 1) / kConvTileW, (p.H + kConvTileH - 1) / kConvTileH);
-    hipLaunchKernelGGL((gated_conv3x3_kernel<CIN, NPAD>), grid, dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((gated_conv3x3_kernel<CIN, NPAD, THREADS>), grid, dim3(THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
