@@ -287,27 +287,28 @@ struct BwdDataParams
     _Float16* d_in;        // [H][W][NN] or nullptr (start block: nothing below)
 };
 
-template <int KC, int NN>
-__global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams p)
+template <int KC, int NN, int THREADS>
+__global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataParams p)
 {
+    constexpr int MB = 16 / (THREADS / 64);  // 16-pixel row blocks of a wavefront: two rows of the tile, or one
     constexpr int ROW    = KC + kLdsChanPad;
     constexpr int GROUPS = KC / 8;
     constexpr int NB     = NN / 16;
     extern __shared__ _Float16 smem[];
     _Float16* s_patch = smem;
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
-    ConvTapStage<KC, NN> taps;
+    ConvTapStage<KC, NN, THREADS> taps;
     conv_tap_fetch(taps, p.wt, 0);  // in flight while the patch is loaded
     _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;  // two tap buffers of the weights
     // the patch of pre-activation gradients, four 16-byte loads of a thread in flight together
     constexpr int kItems = kConvPatchH * kConvPatchW * GROUPS;
-    for (int item0 = threadIdx.x; item0 < kItems; item0 += 4 * 256)
+    for (int item0 = threadIdx.x; item0 < kItems; item0 += 4 * THREADS)
     {
         half8 v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
         {
-            const int item = item0 + 256 * j;
+            const int item = item0 + THREADS * j;
             const int g = item % GROUPS, pp = item / GROUPS;
             const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
@@ -319,14 +320,14 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
 #pragma unroll
         for (int j = 0; j < 4; ++j)
         {
-            const int item = item0 + 256 * j;
+            const int item = item0 + THREADS * j;
             if (item < kItems) *reinterpret_cast<half8*>(s_patch + (size_t)(item / GROUPS) * ROW + 8 * (item % GROUPS)) = v[j];
         }
     }
     conv_tap_stage(taps, s_taps);
     __syncthreads();
-    floatx4 acc[4][NB];
-    conv_taps_mfma<KC, NN, true>(s_patch, s_taps, p.wt, taps, acc);  // a lane: four channels of one pixel
+    floatx4 acc[MB][NB];
+    conv_taps_mfma<KC, NN, true, THREADS>(s_patch, s_taps, p.wt, taps, acc);  // a lane: four channels of one pixel
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15;
     // ---- epilogue: the tile staged in LDS (the patch is no longer needed) and written channels innermost with
@@ -336,9 +337,9 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
     float* s_img       = reinterpret_cast<float*>(smem + kConvTileH * kConvTileW * OS);          // [4][256]
     __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
-    for (int m = 0; m < 4; ++m)
+    for (int m = 0; m < MB; ++m)
     {
-        const int tp = (2 * wave + (m >> 1)) * kConvTileW + (m & 1) * 16 + lrow;  // this lane's pixel of the block
+        const int tp = (MB == 4 ? 2 * wave + (m >> 1) : wave) * kConvTileW + (m & 1) * 16 + lrow;  // this lane's pixel of the block
 #pragma unroll
         for (int n = 0; n < NB; ++n)
         {
@@ -353,11 +354,11 @@ __global__ __launch_bounds__(256) void conv_bwd_data_kernel(const BwdDataParams 
         }
     }
     __syncthreads();
-    if (p.d_in) store_tile_nhwc(s_out, OS, NN / 8, p.d_in, NN, x0, y0, p.W, p.H);
+    if (p.d_in) store_tile_nhwc<THREADS>(s_out, OS, NN / 8, p.d_in, NN, x0, y0, p.W, p.H);
     {
         const size_t plane = (size_t)p.H * p.W;
         const int y = y0 + threadIdx.x / kConvTileW, x = x0 + threadIdx.x % kConvTileW;
-        if (y < p.H && x < p.W)
+        if ((int)threadIdx.x < kConvTileH * kConvTileW && y < p.H && x < p.W)
         {
             float old[4];
             for (int c = 0; c < p.c_feat; ++c) old[c] = p.d_feat[c * plane + (size_t)y * p.W + x];
@@ -1081,11 +1082,12 @@ hipError_t launch_bwd_data(const BwdDataParams& p, hipStream_t stream)
     const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW + 2 * NN) * (KC + kLdsChanPad) * sizeof(_Float16);
     const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NN + kLdsChanPad) * sizeof(_Float16) + 4 * sizeof(float));
     const size_t lds     = std::max(lds_in, lds_out);
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN>),
+    constexpr int THREADS = 512;  // eight wavefronts per tile, as in the forward convolution
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN, THREADS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     dim3 grid((p.W + kConvTileW - 1) / kConvTileW, (p.H + kConvTileH - 1) / kConvTileH);
-    hipLaunchKernelGGL((conv_bwd_data_kernel<KC, NN>), grid, dim3(256), lds, stream, p);
+    hipLaunchKernelGGL((conv_bwd_data_kernel<KC, NN, THREADS>), grid, dim3(THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
