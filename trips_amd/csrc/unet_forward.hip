@@ -341,9 +341,16 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
                 const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
                 float* dst = p.final_out + lrow * plane + (size_t)y * p.W + x;
                 if (y < p.H)
+                {
+                    if (x + 3 < p.W && (reinterpret_cast<uintptr_t>(dst) & 15) == 0)
+                        *reinterpret_cast<float4*>(dst) = make_float4(o[0] + fb, o[1] + fb, o[2] + fb, o[3] + fb);
+                    else
+                    {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        if (x + i < p.W) dst[i] = o[i] + fb;
+                        for (int i = 0; i < 4; ++i)
+                            if (x + i < p.W) dst[i] = o[i] + fb;
+                    }
+                }
             }
         }
     }
