@@ -50,6 +50,8 @@ def _compare(net, inputs, tol_rounded=2e-3, tol_fp32=2e-2):
     ([32, 32, 32, 32, 32], 5, 100, 60),  # the shipped configuration's filters; odd sizes -> centre crop
     ([16, 24], 2, 37, 29),               # partial tiles everywhere
     ([20], 1, 40, 24),                   # start block only
+    ([32, 64, 64], 3, 70, 50),           # 64 input channels at the finest level, whose kernel also holds the 1x1
+    ([16, 48, 32], 3, 70, 50),           # 40 outputs on 32 inputs: the one shape whose weight gradient runs four wavefronts
 ])
 def test_unet_forward_matches_torch(filters, levels, w, h):
     net = _net(filters, levels, seed=levels)
@@ -96,6 +98,8 @@ GRAD_TOL = 2e-2
     ([16, 32, 64, 64], 4, 96, 72, 1),      # the benchmark's channel plan
     ([32, 32, 32, 32, 32], 5, 100, 60, 2),  # shipped filters, odd sizes, two images
     ([16, 24], 2, 37, 29, 1),               # partial tiles
+    ([32, 64, 64], 3, 70, 50, 1),           # 64 input channels at the finest level
+    ([16, 48, 32], 3, 70, 50, 2),           # 40 outputs on 32 inputs (the weight gradient's four-wavefront shape)
 ])
 def test_unet_backward_matches_torch_autograd(filters, levels, w, h, batch):
     import copy
