@@ -139,14 +139,11 @@ def main():
             p.grad = grads[k]
         opt = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
 
-        small = [grads[k] for k in ("d_background", "d_pose", "d_intrinsics")]
-
         def step():
-            # the per-point gradients are written by the backward, every element; only the small ones are added to
-            for g in small:
-                g.zero_()
+            # the per-point gradients are written by the backward, every element; the block sums (background, pose,
+            # intrinsics) are cleared by the backward itself before it adds to them
             ctx.forward(desc, tin, images, saved, workspace)
-            ctx.backward(desc, tin, saved, grad_images, grads, workspace, overwrite_point_grads=True)
+            ctx.backward(desc, tin, saved, grad_images, grads, workspace, overwrite_point_grads=True, clear_block_sums=True)
             opt.step()
 
         for _ in range(args.warmup):

@@ -118,7 +118,9 @@ typedef struct TripsSplatOut {
  * With overwrite_point_grads != 0 the four per-point outputs (d_texture, d_confidence, d_position, d_point_size) are
  * WRITTEN instead: every element receives its value, zero where no gradient arrives (.w of d_position too), so the
  * caller may pass uninitialised memory and skips four fills and the kernel the reads of a read-modify-write;
- * d_background, d_pose and d_intrinsics are added to in either mode. */
+ * d_background, d_pose and d_intrinsics are added to in either mode; with clear_block_sums != 0 the call clears them
+ * itself first (all of d_background, every row of d_pose [num_images, 6] and of d_intrinsics [num_cameras, 13]), which
+ * spares the caller three fill launches per step. */
 typedef struct TripsSplatGrads {
     float* d_texture;     /* [C,T]   required */
     float* d_confidence;  /* [T]     required */
@@ -129,6 +131,7 @@ typedef struct TripsSplatGrads {
     double* d_pose;       /* [F,6]   or NULL; translation first, rotation last */
     float* d_intrinsics;  /* [Cam,13] or NULL */
     int32_t overwrite_point_grads; /* 0 = add into everything (the reference's contract); 1 = see above */
+    int32_t clear_block_sums;      /* 1 = d_background, d_pose, d_intrinsics are cleared by the call before it adds */
 } TripsSplatGrads;
 
 typedef struct TripsCtx TripsCtx;

@@ -39,19 +39,22 @@ class GpuRun:
         return [x.cpu().numpy() for x in out]
 
     def backward(self, grad_images, want_position=True, want_point_size=True, want_pose=True, want_intrinsics=True,
-                 overwrite=False):
-        """overwrite: the per-point outputs start as NaN and the call runs with overwrite_point_grads."""
+                 overwrite=False, clear=False):
+        """overwrite: the per-point outputs start as NaN and the call runs with overwrite_point_grads;
+        clear: the block sums start as NaN and the call runs with clear_block_sums."""
         d, dev = self.desc, self.ctx.device
         z = lambda shape, dt=torch.float32: torch.zeros(shape, dtype=dt, device=dev)
         big = (lambda shape: torch.full(shape, float("nan"), dtype=torch.float32, device=dev)) if overwrite else z
+        zs = (lambda shape, dt=torch.float32: torch.full(shape, float("nan"), dtype=dt, device=dev)) if clear else z
         grads = dict(d_texture=big((d.num_channels, d.num_texels)), d_confidence=big((d.num_texels,)),
-                     d_background=z(d.num_channels),
+                     d_background=zs((d.num_channels,)),
                      d_position=big((d.num_points, 4)) if want_position else None,
                      d_point_size=big((d.num_points,)) if want_point_size else None,
-                     d_pose=z((d.num_images, 6), torch.float64) if want_pose else None,
-                     d_intrinsics=z((d.num_cameras, 13)) if want_intrinsics else None)
+                     d_pose=zs((d.num_images, 6), torch.float64) if want_pose else None,
+                     d_intrinsics=zs((d.num_cameras, 13)) if want_intrinsics else None)
         gi = [torch.as_tensor(np.ascontiguousarray(g), dtype=torch.float32).to(dev) for g in grad_images]
-        self.ctx.backward(d, self.tin, self.saved, gi, grads, self.workspace, overwrite_point_grads=overwrite)
+        self.ctx.backward(d, self.tin, self.saved, gi, grads, self.workspace, overwrite_point_grads=overwrite,
+                          clear_block_sums=clear)
         torch.cuda.synchronize()
         return {k: (None if v is None else v.cpu().numpy()) for k, v in grads.items()}
 

@@ -225,6 +225,33 @@ def test_backward_overwrite_mode_equals_adding_into_zeros(case):
     assert np.abs(added["d_texture"]).max() > 0
 
 
+@pytest.mark.parametrize("views", [1, 2])
+@pytest.mark.parametrize("overwrite", [False, True])
+def test_backward_clearing_the_block_sums_equals_adding_into_zeros(views, overwrite):
+    """clear_block_sums: d_background, every row of d_pose and every row of d_intrinsics start as NaN and must come out
+    as what adding into zeroed buffers gives: cleared once, before the first view of the batch, and added to by every
+    view after it; rows of images and cameras no view of the batch touches come out as zero."""
+    from tests.gpu_util import GpuRun
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=16, seed=43, views=views, radius=(0.004, 0.4))
+    sc.poses_se3 = np.concatenate([sc.poses_se3, sc.poses_se3[:1]])  # one image and one camera no view refers to
+    sc.intrinsics = np.concatenate([sc.intrinsics, sc.intrinsics[:1]])
+    d = abi.desc_for_scene(sc)
+    rng = np.random.default_rng(9)
+    run = GpuRun(sc, d)
+    images = run.forward()
+    grads = [rng.normal(0, 1, im.shape).astype(np.float32) for im in images]
+    added = run.backward(grads, overwrite=overwrite)
+    cleared = run.backward(grads, overwrite=overwrite, clear=True)
+    for k, v in added.items():
+        assert np.isfinite(cleared[k]).all(), k
+        if k in ("d_background", "d_pose", "d_intrinsics"):
+            np.testing.assert_allclose(cleared[k], v, rtol=1e-4, atol=1e-6)  # float atomics across workgroups
+        else:
+            assert np.array_equal(cleared[k], v), k
+    assert np.abs(added["d_pose"]).max() > 0 and np.abs(added["d_background"]).max() > 0
+    assert not cleared["d_pose"][-1].any() and not cleared["d_intrinsics"][-1].any()
+
+
 def test_displacement_forward_backward(oracle):
     """Per-view displacements of the point positions (dynamic_refinement_t, PointRenderer.cu:703-713)."""
     sc = scenes.tiny(n=4000, w=70, h=50, f=60.0, num_layers=4, list_depth=16, seed=77, views=3, radius=(0.004, 0.4))

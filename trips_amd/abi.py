@@ -97,6 +97,7 @@ class TripsSplatGrads(C.Structure):
         ("d_pose", C.c_void_p),
         ("d_intrinsics", C.c_void_p),
         ("overwrite_point_grads", C.c_int32),
+        ("clear_block_sums", C.c_int32),
     ]
 
 

@@ -482,13 +482,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
     }
 }
 
-// Overwrite mode, before the point pass of the first view: the descriptor and confidence gradients of the columns
-// that the point pass does not write itself. With the identity index (the forward noted it in the header) those are
-// the columns past the last point; otherwise all of them, the point pass then adds with atomics.
+// Before the two passes of the first view. Overwrite mode (`texels`): the descriptor and confidence gradients of the
+// columns that the point pass does not write itself. With the identity index (the forward noted it in the header)
+// those are the columns past the last point; otherwise all of them, the point pass then adds with atomics.
+// `clear_sums`: the block sums that both passes add to (background, every pose row, every intrinsics row).
 __global__ __launch_bounds__(256) void zero_texel_grads_kernel(const ViewHeader* __restrict__ header, float* __restrict__ d_texture,
                                                                float* __restrict__ d_confidence, int channels, int num_texels,
-                                                               int num_points)
+                                                               int num_points, int texels, int clear_sums,
+                                                               float* __restrict__ d_background, double* __restrict__ d_pose,
+                                                               int num_images, float* __restrict__ d_intrinsics, int num_cameras)
 {
+    if (clear_sums && blockIdx.x == 0)
+    {
+        if (d_background)
+            for (int i = threadIdx.x; i < channels; i += 256) d_background[i] = 0.f;
+        if (d_pose)
+            for (int i = threadIdx.x; i < num_images * 6; i += 256) d_pose[i] = 0.0;
+        if (d_intrinsics)
+            for (int i = threadIdx.x; i < num_cameras * 13; i += 256) d_intrinsics[i] = 0.f;
+    }
+    if (!texels) return;
     const int first = header->not_identity == 0 ? min(num_points, num_texels) : 0;
     const int n     = num_texels - first;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < (long long)n * (channels + 1); i += (long long)gridDim.x * 256)
@@ -516,10 +529,11 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
 {
     const int P           = p.geom.bin_off[p.num_layers] * kTilePixels;
     const int N           = p.num_points;
-    if (N <= 0) 
-    {
-        // no points: only the background receives gradient
-    }
+    // (no points: only the background receives gradient)
+    if (p.overwrite || p.clear_block_sums)
+        hipLaunchKernelGGL(zero_texel_grads_kernel, dim3(p.overwrite ? 1024 : 1), dim3(256), 0, stream, p.header, p.d_texture,
+                           p.d_confidence, channels, p.num_texels, N, p.overwrite, p.clear_block_sums, p.d_background, p.d_pose_all,
+                           p.num_images, p.d_intrinsics_all, p.num_cameras);
     {
         ProfScope ps(prof, "backward_pixels", stream);
         const long long waves = ((long long)P + 3) / 4;
@@ -528,9 +542,6 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
         blocks                = ((blocks + 4 * kNumXcd - 1) / (4 * kNumXcd)) * (4 * kNumXcd);  // whole groups of 8 tiles x 4
         TRIPS_BW_DISPATCH(backward_pixels_kernel, blocks);
     }
-    if (p.overwrite)
-        hipLaunchKernelGGL(zero_texel_grads_kernel, dim3(1024), dim3(256), 0, stream, p.header, p.d_texture, p.d_confidence, channels,
-                           p.num_texels, N);
     if (N > 0)
     {
         ProfScope ps(prof, "backward_points", stream);

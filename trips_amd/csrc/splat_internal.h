@@ -356,6 +356,11 @@ struct BackwardParams
     double* d_pose;       // row of this view's image or nullptr
     float* d_intrinsics;  // row of this view's camera or nullptr
     int32_t overwrite;    // the per-point outputs are written, not added to (first view of a call in that mode)
+    // first view of a call that clears the block sums itself: all of d_background, d_pose and d_intrinsics
+    int32_t clear_block_sums;
+    double* d_pose_all;       // [num_images][6] or nullptr
+    float* d_intrinsics_all;  // [num_cameras][13] or nullptr
+    int32_t num_images, num_cameras;
 };
 
 }  // namespace trips

@@ -267,13 +267,13 @@ variable_list PointRender::backward(AutogradContext* ctx, variable_list grad_out
     // the small ones are added to and start at zero.
     torch::Tensor g_texture    = torch::empty_like(s->texture);
     torch::Tensor g_confidence = torch::empty_like(s->confidence);
-    torch::Tensor g_background = torch::zeros_like(s->background);
+    torch::Tensor g_background = torch::empty_like(s->background);  // the block sums are cleared by the backward itself
     torch::Tensor g_points, g_layer, g_pose, g_intrinsics;
     if (ctx->needs_input_grad(2)) g_points = torch::empty_like(s->position);
     if (ctx->needs_input_grad(7)) g_layer = torch::empty_like(s->point_size);
     if (ctx->needs_input_grad(3))
-        g_pose = torch::zeros({d.num_images, 6}, torch::TensorOptions().dtype(torch::kFloat64).device(dev));
-    if (ctx->needs_input_grad(4)) g_intrinsics = torch::zeros_like(s->intrinsics);
+        g_pose = torch::empty({d.num_images, 6}, torch::TensorOptions().dtype(torch::kFloat64).device(dev));
+    if (ctx->needs_input_grad(4)) g_intrinsics = torch::empty_like(s->intrinsics);
 
     std::vector<torch::Tensor> gi;
     const float* gptr[TRIPS_MAX_LAYERS] = {};
@@ -302,6 +302,7 @@ variable_list PointRender::backward(AutogradContext* ctx, variable_list grad_out
     g.d_pose        = g_pose.defined() ? g_pose.data_ptr<double>() : nullptr;
     g.d_intrinsics  = g_intrinsics.defined() ? g_intrinsics.data_ptr<float>() : nullptr;
     g.overwrite_point_grads = 1;
+    g.clear_block_sums      = 1;
     TripsSplatIn in = make_in(*s);
     check(trips_splat_backward(tc, &d, &in, s->saved_state.data_ptr(), gptr, &g, info->cache->workspace.data_ptr(),
                                (size_t)info->cache->workspace.numel(), current_stream(s->texture)),

@@ -559,6 +559,11 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.d_pose       = grads->d_pose ? grads->d_pose + 6 * (size_t)d.views[b].image_index : nullptr;
         p.d_intrinsics = grads->d_intrinsics ? grads->d_intrinsics + 13 * (size_t)d.views[b].camera_index : nullptr;
         p.overwrite    = (grads->overwrite_point_grads != 0 && b == 0) ? 1 : 0;  // later views add to the first one's
+        p.clear_block_sums = (grads->clear_block_sums != 0 && b == 0) ? 1 : 0;
+        p.d_pose_all       = grads->d_pose;
+        p.d_intrinsics_all = grads->d_intrinsics;
+        p.num_images       = d.num_images;
+        p.num_cameras      = d.num_cameras;
         hipError_t e   = launch_backward_view(p, d.num_channels, stream, ctx->prof.enabled ? &ctx->prof : nullptr);
         if (e != hipSuccess) return hip_fail(e, "backward launch");
     }

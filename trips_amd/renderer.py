@@ -109,9 +109,11 @@ class SplatContext:
         _lib.check(self.lib.trips_splat_forward_static(self.ctx, C.byref(desc), C.byref(tin), C.byref(out),
                                                        _stream_ptr(self.device)))
 
-    def backward(self, desc, tin, saved, grad_images, grads, workspace=None, overwrite_point_grads=False):
+    def backward(self, desc, tin, saved, grad_images, grads, workspace=None, overwrite_point_grads=False,
+                 clear_block_sums=False):
         """Adds into `grads` (zeroed by the caller); with overwrite_point_grads the four per-point outputs
-        (d_texture, d_confidence, d_position, d_point_size) are written instead and may be uninitialised."""
+        (d_texture, d_confidence, d_position, d_point_size) are written instead and may be uninitialised; with
+        clear_block_sums the call clears d_background, d_pose and d_intrinsics itself before it adds to them."""
         arr = (C.c_void_p * abi.TRIPS_MAX_LAYERS)()
         for l, g in enumerate(grad_images):
             arr[l] = g.data_ptr()
@@ -120,6 +122,7 @@ class SplatContext:
                   "d_intrinsics"):
             setattr(tg, k, _ptr(grads.get(k)))
         tg.overwrite_point_grads = int(bool(overwrite_point_grads))
+        tg.clear_block_sums = int(bool(clear_block_sums))
         _lib.check(self.lib.trips_splat_backward(self.ctx, C.byref(desc), C.byref(tin), _ptr(saved), arr,
                                                  C.byref(tg), _ptr(workspace),
                                                  0 if workspace is None else workspace.numel(),
@@ -356,18 +359,18 @@ class PointRender(torch.autograd.Function):
         grads = dict(
             d_texture=torch.empty_like(t["texture"]),
             d_confidence=torch.empty(desc.num_texels, dtype=torch.float32, device=dev),
-            d_background=torch.zeros_like(t["background"]),
+            d_background=torch.empty_like(t["background"]),
             d_position=torch.empty_like(t["position"]) if need[2] else None,
             d_point_size=torch.empty(desc.num_points, dtype=torch.float32, device=dev) if need[7] else None,
-            d_pose=torch.zeros((desc.num_images, 6), dtype=torch.float64, device=dev) if need[3] else None,
-            d_intrinsics=torch.zeros_like(t["intrinsics"]) if need[4] else None,
+            d_pose=torch.empty((desc.num_images, 6), dtype=torch.float64, device=dev) if need[3] else None,
+            d_intrinsics=torch.empty_like(t["intrinsics"]) if need[4] else None,
         )
         # a layer nobody consumed (a net with fewer levels than the pyramid) arrives without a gradient
         gi = [g.contiguous() if g is not None else torch.zeros(shape, dtype=torch.float32, device=dev)
               for g, shape in zip(grad_output[:desc.num_layers], ctx.image_shapes)]
         tin = SplatContext.make_in(**t)
         sctx.backward(desc, tin, ctx.saved_state, gi, grads, info.cache.workspace if info.cache else None,
-                      overwrite_point_grads=True)
+                      overwrite_point_grads=True, clear_block_sums=True)
         d_layer = grads["d_point_size"].reshape(ctx.shapes["layer"]) if need[7] else None
         d_conf = grads["d_confidence"].reshape(ctx.shapes["confidence"])
         # order of PointRenderer.cu:1423-1426, then None for `info`
