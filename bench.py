@@ -30,16 +30,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "5e5e906da63461331ec4e034c6bceacffd70f74c28801fc5e50d47596e5b1350"
+PMC_SOURCES_SHA256 = "4bd354a2622d8f041997405108031029e95e6d2cc8c0c29819e312e3f69fc324"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129133, 271433),
-    "bin_scatter": (87912, 186198),
+    "project_bin": (129132, 271473),
+    "bin_scatter": (87922, 186160),
     "tile_count": (26200, 2296),
-    "tile_scatter": (70861, 114521),
-    "sort_blend": (333873, 417473),
-    "backward_pixels": (498794, 165612),
-    "backward_points": (1045013, 234887),
-    "adam_fused": (582965, 792823),
+    "tile_scatter": (70639, 113744),
+    "sort_blend": (333824, 417709),
+    "backward_pixels": (498848, 165601),
+    "backward_points": (1045060, 234887),
+    "adam_fused": (582966, 792823),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
@@ -221,7 +221,6 @@ def main():
     sc, desc, t, tin, workspace, saved, images = (r[k] for k in ("sc", "desc", "t", "tin", "workspace", "saved", "images"))
     gen, grad_images, grads, opt, counters = (r[k] for k in ("gen", "grad_images", "grads", "opt", "counters"))
     nz, total_el, prof, ms_per_step = r["nz"], r["total_el"], r["prof"], r["ms_per_step"]
-    small = [grads[k] for k in ("d_background", "d_pose", "d_intrinsics")]  # the gradients that are added to
     N, C = desc.num_points, desc.num_channels
 
     # the timed step runs the product's optimiser state: int32 step counters, 36 bytes per updated element
@@ -291,15 +290,13 @@ def main():
         zero_tail = [torch.zeros_like(im) for im in images[np_.num_layers:]]
 
         def train_step():
-            for g in small:
-                g.zero_()
             net_opt.zero_grad(set_to_none=True)
             ctx.forward(desc, tin, images, saved, workspace)
             ins = [im.detach().requires_grad_(True) for im in images]
             loss = (net.forward(ins) - target).abs().mean()
             loss.backward()
             gi = [t.grad for t in ins[:np_.num_layers]] + zero_tail
-            ctx.backward(desc, tin, saved, gi, grads, workspace, overwrite_point_grads=True)
+            ctx.backward(desc, tin, saved, gi, grads, workspace, overwrite_point_grads=True, clear_block_sums=True)
             opt.step()
             net_opt.step()
             return loss
