@@ -313,12 +313,35 @@ def main():
         c1 = time.perf_counter()
         tprof = ctx.profile_read()
         ctx.profile_enable(False)
+        # the same training step captured once into a HIP graph and replayed (autograd included: every tensor it
+        # creates comes out of the graph's own memory pool, so the replays run on the addresses of the capture)
+        train_graph_ms = None
+        if not args.no_graph:
+            try:
+                side = torch.cuda.Stream()
+                with torch.cuda.stream(side):
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        train_step()
+                torch.cuda.synchronize()
+                for _ in range(2):
+                    graph.replay()
+                torch.cuda.synchronize()
+                g0 = time.perf_counter()
+                for _ in range(args.steps):
+                    graph.replay()
+                torch.cuda.synchronize()
+                train_graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
+                del graph
+            except Exception as e:  # the eager figure above stands on its own
+                print(f"bench.py: graph capture of the config-5 step failed: {e}", file=sys.stderr)
         net_bwd_ms = sum(ms for k, (ms, _) in tprof.items() if k.startswith("unet_bwd")) / args.steps
         net_fwd_ms = sum(ms for k, (ms, _) in tprof.items() if k.startswith("unet_") and not k.startswith("unet_bwd")) / args.steps
         unet["train_step"] = {
             "workload": "config5: splat forward + net forward + L1 loss + net backward + splat backward + fused Adam "
                         "(point parameters and net weights), 6M points, 1920x1080",
             "ms_per_step_wall": round((c1 - c0) * 1e3 / args.steps, 4),
+            "ms_per_step_hip_graph": None if train_graph_ms is None else round(train_graph_ms, 4),
             "ms_all_kernels": round(sum(ms for ms, _ in tprof.values()) / args.steps, 4),
             "ms_net_forward": round(net_fwd_ms, 4), "ms_net_backward": round(net_bwd_ms, 4),
             "net_backward_tflops": round(2 * flops / (net_bwd_ms * 1e-3) / 1e12, 1) if net_bwd_ms > 0 else None,

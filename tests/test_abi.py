@@ -54,7 +54,7 @@ def test_unet_ctypes_mirrors_and_host_checks(tmp_path):
     d = abi.make_unet_desc([16, 32, 64, 64], abi.layer_sizes(1920, 1080, 4))
     b, f = C.c_size_t(0), C.c_double(0)
     assert lib.trips_unet_workspace_size(C.byref(d), C.byref(b)) == 0
-    assert b.value >= 1920 * 1080 * 16 * 2  # fp16 activations of the finest level
+    assert b.value >= 960 * 540 * 32 * 2  # fp16 block outputs of the second level (the finest one's stay in its kernel)
     assert lib.trips_unet_flops(C.byref(d), C.byref(f)) == 0
     # two 3x3 convolutions per level, 2 flops per multiply-accumulate, plus the 1x1
     want = sum(2 * 2 * 9 * cin * cout * w * h for (cin, cout, (w, h)) in

@@ -28,7 +28,8 @@ namespace trips
 {
 
 // d(elu(f) * sigmoid(m)) for an incoming gradient da
-__device__ __forceinline__ void gate_backward(float da, float f, float m, float& df, float& dm)
+// (`act`: the gated value itself, elu(f) * sigmoid(m), with the forward's formula)
+__device__ __forceinline__ void gate_backward(float da, float f, float m, float& df, float& dm, float& act)
 {
     const float s  = __builtin_amdgcn_rcpf(1.f + __expf(-m));  // 1 ulp; the gradients are rounded to fp16 next
     const float ex = __expf(f);
@@ -36,6 +37,12 @@ __device__ __forceinline__ void gate_backward(float da, float f, float m, float&
     const float de = f > 0.f ? 1.f : ex;
     df             = da * s * de;
     dm             = da * e * s * (1.f - s);
+    act            = e * s;
+}
+__device__ __forceinline__ void gate_backward(float da, float f, float m, float& df, float& dm)
+{
+    float act;
+    gate_backward(da, f, m, df, dm, act);
 }
 
 // wt[tap'][c][n] = W[n][c][8 - tap']: the data gradient is a correlation of the pre-activation gradient with the
@@ -80,7 +87,6 @@ struct FinalBwdParams
     int H, W, c_feat, cact, cact_store, cout, npad;
     float scale;
     const float* feat;        // [C][H][W]
-    const _Float16* act;      // [H][W][cact_store]
     const _Float16* pre;      // [H][W][npad]
     const float* weight;      // [cout][c_feat + cact]
     const float* d_out;       // [cout][H][W]
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
     struct Loaded
     {
         float g[4], x;
-        half8 v, mine;
+        half8 mine;
     };
     auto load = [&](size_t pix, bool valid)
     {
@@ -153,8 +159,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
         for (int k = 0; k < 4; ++k) l.g[k] = (valid && k < p.cout) ? p.d_out[k * plane + pix] : 0.f;
         l.x = (WGRAD && valid && has_img) ? p.feat[g * plane + pix] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) l.v[i] = l.mine[i] = _Float16(0.f);
-        if (WGRAD && valid && has_act) l.v = *reinterpret_cast<const half8*>(p.act + pix * CS + ch0);
+        for (int i = 0; i < 8; ++i) l.mine[i] = _Float16(0.f);
         if (valid && in_row) l.mine = *reinterpret_cast<const half8*>(p.pre + pix * p.npad + 8 * g);
         return l;
     };
@@ -178,15 +183,17 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
             const half8 other = __builtin_bit_cast(half8, oth);
             const half8 f8 = is_f ? cur.mine : other, m8 = is_f ? other : cur.mine;
             half8 out;
+            float v[8];  // the block's output as the forward's 1x1 convolution read it (fp16), on the feature lanes
 #pragma unroll
             for (int i = 0; i < 8; ++i)
             {
                 float da = 0.f;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) da += wj[k][i] * cur.g[k];
-                float df, dm;
-                gate_backward(da * p.scale, float(f8[i]), float(m8[i]), df, dm);
+                float df, dm, a;
+                gate_backward(da * p.scale, float(f8[i]), float(m8[i]), df, dm, a);
                 out[i] = _Float16(is_f ? df : dm);
+                v[i]   = (valid && has_act && ch0 + i < p.cact) ? float(_Float16(a)) : 0.f;
             }
             if (valid && in_row) *reinterpret_cast<half8*>(p.dpre + pix * p.npad + 8 * g) = out;
             if (valid && has_img)
@@ -205,7 +212,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
                     accb[k] += cur.g[k];
                     acc_img[k] += cur.g[k] * xr;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc[k][i] += cur.g[k] * float(cur.v[i]);
+                    for (int i = 0; i < 8; ++i) acc[k][i] += cur.g[k] * v[i];
                 }
             }
         }
@@ -1231,7 +1238,6 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             p.H = lv.H, p.W = lv.W, p.c_feat = C, p.cact = lv.cout, p.cact_store = lv.cout_store, p.cout = K, p.npad = lv.npad;
             p.scale    = grad_scale;
             p.feat     = inputs[0] + (size_t)b * C * plane;
-            p.act      = act_ptr(0, b);
             p.pre      = pre_ptr(0, b);
             p.weight   = weights->final_weight;
             p.d_out    = d_output + (size_t)b * K * plane;

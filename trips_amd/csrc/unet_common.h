@@ -254,8 +254,10 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
     }
     for (int i = 0; i < L; ++i)
     {
+        // (the finest block's output never leaves its kernel: the 1x1 convolution that reads it runs there, and the
+        // backward recomputes it from the saved pre-activations)
         np.lv[i].act_off = o;
-        o += align256((size_t)d.batch * np.lv[i].H * np.lv[i].W * np.lv[i].cout_store * sizeof(_Float16));
+        if (i > 0) o += align256((size_t)d.batch * np.lv[i].H * np.lv[i].W * np.lv[i].cout_store * sizeof(_Float16));
     }
     np.bytes = o;
     size_t sv = 0, bw = 0;
@@ -264,7 +266,7 @@ inline NetPlan make_plan(const TripsUnetDesc& d)
         LevelPlan& lv       = np.lv[i];
         const size_t pixels = (size_t)d.batch * lv.H * lv.W;
         lv.saved_act_off    = sv;
-        sv += align256(pixels * lv.cout_store * sizeof(_Float16));
+        if (i > 0) sv += align256(pixels * lv.cout_store * sizeof(_Float16));
         lv.saved_pre_off = sv;
         sv += align256(pixels * lv.npad * sizeof(_Float16));
         lv.wt_off = bw;

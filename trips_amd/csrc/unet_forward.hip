@@ -538,8 +538,9 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
             p.feat       = inputs[i] + (size_t)b * C * lv.H * lv.W;
             p.wpack      = reinterpret_cast<const _Float16*>(ws + lv.wpack_off);
             p.bias       = reinterpret_cast<const float*>(ws + lv.bias_off);
-            // (without a saved state nobody reads the finest block's output again: its 1x1 runs in the same kernel)
-            p.out        = (i == 0 && !sv) ? nullptr : act_ptr(i, b);
+            // (nobody reads the finest block's output again: its 1x1 runs in the same kernel, and the backward takes
+            // it from the pre-activations)
+            p.out        = i == 0 ? nullptr : act_ptr(i, b);
             p.pre        = sv ? reinterpret_cast<_Float16*>(sv + lv.saved_pre_off) + (size_t)b * lv.H * lv.W * lv.npad : nullptr;
             if (i < L - 1)
             {
