@@ -58,6 +58,9 @@ __device__ __forceinline__ Camera load_camera_bw(const double* pose, const float
     return c;
 }
 
+typedef float vf2 __attribute__((ext_vector_type(2)));
+typedef float vf4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ double wave_sum(double v)
 {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -120,7 +123,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
     float a = 0.f;
     if (has)
     {
-        cid               = p.lists[((size_t)(unsigned)pix << kshift) + sub];
+        cid               = __builtin_nontemporal_load(p.lists + (((size_t)(unsigned)pix << kshift) + sub));
         const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
         const float4 r0   = rec[0];
 #pragma unroll
@@ -176,9 +179,9 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
     if (has)
     {
         if (sub < KIN)
-            reinterpret_cast<float2*>(row + CPAD)[sub] = make_float2(grad_alpha, ta);
+            __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row + CPAD) + sub);
         else
-            reinterpret_cast<float2*>(p.entry_over)[(size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)] = make_float2(grad_alpha, ta);
+            __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(p.entry_over) + ((size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)));
     }
     if (sub == 0 && m > 0)
     {
@@ -186,7 +189,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
 #pragma unroll
         for (int c = 0; c < CPAD; ++c) gp[c] = c < C ? g[c] : 0.f;
 #pragma unroll
-        for (int q = 0; q < CPAD / 4; ++q) reinterpret_cast<float4*>(row)[q] = make_float4(gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]);
+        for (int q = 0; q < CPAD / 4; ++q) __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row) + q);
     }
 }
 

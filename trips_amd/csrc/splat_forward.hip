@@ -25,6 +25,7 @@
 
 namespace trips
 {
+typedef unsigned vu4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ Camera load_camera(const double* pose, const float* intr, const TripsView& v,
                                               float dist_cutoff)
@@ -282,12 +283,12 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
             make_float4(TRAIN ? softplus_backward(in.raw_size) : 0.f, o.z, __int_as_float(o.layers), o.size_px);
         if (TRAIN)
         {
-            p.pid_of[cid] = pid;
+            __builtin_nontemporal_store(pid, p.pid_of + cid);
             // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
             // pixel's list; filled by sort_blend): a plane of 16 bytes per compact number for layers 0..3 and a second
             // one for layers 4..7. Every valid point clears its row of the first, the few points that reach layer 4 and
             // beyond their row of the second as well.
-            *reinterpret_cast<uint4*>(p.rank + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
+            __builtin_nontemporal_store(vu4{~0u, ~0u, ~0u, ~0u}, reinterpret_cast<vu4*>(p.rank + (size_t)cid * 16));
             if (o.layers > 4)
                 *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
         }
@@ -938,20 +939,20 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
             float* o           = img + ((size_t)p.view_index * C) * plane;
             const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
 #pragma unroll
-            for (int c = 0; c < C; ++c) (o + c * plane)[at] = col[c];
+            for (int c = 0; c < C; ++c) __builtin_nontemporal_store(col[c], (o + c * plane) + at);
         }
         else
         {
             float* o          = img + ((size_t)p.view_index * lh * lw) * C;
             const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
 #pragma unroll
-            for (int c = 0; c < C; ++c) o[at + c] = col[c];
+            for (int c = 0; c < C; ++c) __builtin_nontemporal_store(col[c], o + at + c);
         }
     }
     // saved state, also for padding pixels (empty) so that every row of the tables is defined
     if (TRAIN && in_range)
     {
-        if (sub == 0) p.retained[pix] = live ? ret : 0;
+        if (sub == 0) __builtin_nontemporal_store(live ? ret : 0, p.retained + pix);
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
         // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
         if (has && sub < ret)
@@ -962,10 +963,10 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
             // one 8-byte store per lane covers the pixel's whole row (K <= 16 ids): lanes 0..3 carry the ids of lane
             // pairs, the others the -1 padding
             const int lo = __shfl(mine, (2 * sub) & 7, 8), hi = __shfl(mine, (2 * sub + 1) & 7, 8);
-            if (2 * sub < K) *reinterpret_cast<int2*>(p.lists + (((size_t)(unsigned)pix << kshift) + 2 * sub)) = sub < 4 ? make_int2(lo, hi) : make_int2(-1, -1);
+            if (2 * sub < K) __builtin_nontemporal_store(sub < 4 ? (long long)(unsigned)lo | ((long long)hi << 32) : -1ll, reinterpret_cast<long long*>(p.lists + (((size_t)(unsigned)pix << kshift) + 2 * sub)));
         }
         else if (sub < K)
-            p.lists[((size_t)(unsigned)pix << kshift) + sub] = mine;
+            __builtin_nontemporal_store(mine, p.lists + (((size_t)(unsigned)pix << kshift) + sub));
     }
 }
 
@@ -1011,7 +1012,7 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     if (TRAIN)
     {
         const int len = c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 9) + __shfl_down(c_len, 10);
-        if (lane < 8 && group_in_range) p.lengths[pix_first + lane] = len;  // 0 for the padding of partial tiles
+        if (lane < 8 && group_in_range) __builtin_nontemporal_store(len, p.lengths + (pix_first + lane));  // 0 for the padding of partial tiles
     }
     if (lane >= 8) tot8 = 0;
     tot8 = max(tot8, __shfl_xor(tot8, 1));
