@@ -30,16 +30,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "4bd354a2622d8f041997405108031029e95e6d2cc8c0c29819e312e3f69fc324"
+PMC_SOURCES_SHA256 = "40cd30c5a2db732ba4214e7b23681251f23216372c31704e8a301d94b1645a62"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129132, 271473),
-    "bin_scatter": (87922, 186160),
+    "project_bin": (129125, 298338),
+    "bin_scatter": (89120, 186823),
     "tile_count": (26200, 2296),
-    "tile_scatter": (70639, 113744),
-    "sort_blend": (333824, 417709),
-    "backward_pixels": (498848, 165601),
-    "backward_points": (1045060, 234887),
-    "adam_fused": (582966, 792823),
+    "tile_scatter": (69588, 114815),
+    "sort_blend": (330637, 454557),
+    "backward_pixels": (464967, 188210),
+    "backward_points": (1045087, 234887),
+    "adam_fused": (582965, 792823),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")

@@ -26,6 +26,7 @@
 namespace trips
 {
 typedef unsigned vu4 __attribute__((ext_vector_type(4)));
+typedef float vf4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ Camera load_camera(const double* pose, const float* intr, const TripsView& v,
                                               float dist_cutoff)
@@ -277,10 +278,10 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         for (int q = 0; q < CPAD / 4; ++q) recv[1 + q] = make_float4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3]);
         float4* rec = reinterpret_cast<float4*>(p.rec + (size_t)cid * p.rec_floats);
 #pragma unroll
-        for (int q = 0; q < NREC; ++q) rec[q] = recv[q];
+        for (int q = 0; q < NREC; ++q) __builtin_nontemporal_store(vf4{recv[q].x, recv[q].y, recv[q].z, recv[q].w}, reinterpret_cast<vf4*>(rec) + q);
         // point record: depth and layers for the scatter pass; softplus' and the size for the backward
-        reinterpret_cast<float4*>(p.prec)[cid] =
-            make_float4(TRAIN ? softplus_backward(in.raw_size) : 0.f, o.z, __int_as_float(o.layers), o.size_px);
+        __builtin_nontemporal_store(vf4{TRAIN ? softplus_backward(in.raw_size) : 0.f, o.z, __int_as_float(o.layers), o.size_px},
+                                    reinterpret_cast<vf4*>(p.prec) + cid);
         if (TRAIN)
         {
             __builtin_nontemporal_store(pid, p.pid_of + cid);
@@ -424,7 +425,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
             const int cid = cid0 + u * kBinThreads;
             if (cid < begin + n)
             {
-                tail[u] = reinterpret_cast<const float4*>(p.prec)[cid];
+                const vf4 t = __builtin_nontemporal_load(reinterpret_cast<const vf4*>(p.prec) + cid);
+                tail[u]     = make_float4(t.x, t.y, t.z, t.w);
                 ip[u]   = *reinterpret_cast<const float2*>(p.rec + (size_t)cid * p.rec_floats);
             }
         }
@@ -706,7 +708,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     {
         __syncthreads();
         u64* dst = p.keys + key_start;
-        for (int i = threadIdx.x; i < tile_total; i += THREADS) dst[i] = s_keys[i];
+        for (int i = threadIdx.x; i < tile_total; i += THREADS) __builtin_nontemporal_store(s_keys[i], dst + i);
     }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
 }

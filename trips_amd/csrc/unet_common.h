@@ -139,8 +139,9 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
 
 // Copies `groups` x 8 halves per pixel of an 8 x 32 tile staged in LDS ([256][lds_stride]) to a channels-innermost
 // image ([H][W][dst_stride]) with 16-byte stores: consecutive lanes write consecutive 16 bytes, so a tile row leaves
-// as whole lines (2-byte stores straight from the MFMA result layout cost twice the memory requests).
-template <int THREADS = 256>
+// as whole lines (2-byte stores straight from the MFMA result layout cost twice the memory requests). STREAM: with
+// the non-temporal hint, for data that nothing reads again soon.
+template <int THREADS = 256, bool STREAM = false>
 __device__ __forceinline__ void store_tile_nhwc(const _Float16* s_tile, int lds_stride, int groups, _Float16* dst,
                                                 int dst_stride, int x0, int y0, int W, int H)
 {
@@ -149,8 +150,14 @@ __device__ __forceinline__ void store_tile_nhwc(const _Float16* s_tile, int lds_
         const int g = item % groups, tp = item / groups;
         const int y = y0 + tp / kConvTileW, x = x0 + tp % kConvTileW;
         if (y < H && x < W)
-            *reinterpret_cast<half8*>(dst + ((size_t)y * W + x) * dst_stride + 8 * g) =
-                *reinterpret_cast<const half8*>(s_tile + (size_t)tp * lds_stride + 8 * g);
+        {
+            const half8 v = *reinterpret_cast<const half8*>(s_tile + (size_t)tp * lds_stride + 8 * g);
+            half8* to     = reinterpret_cast<half8*>(dst + ((size_t)y * W + x) * dst_stride + 8 * g);
+            if (STREAM)
+                __builtin_nontemporal_store(v, to);
+            else
+                *to = v;
+        }
     }
 }
 

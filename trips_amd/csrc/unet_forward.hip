@@ -284,7 +284,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     }
     __syncthreads();
     if (p.out) store_tile_nhwc<THREADS>(s_act, AS, p.cout_store / 8, p.out, p.cout_store, x0, y0, p.W, p.H);
-    if (p.pre) store_tile_nhwc<THREADS>(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
+    if (p.pre) store_tile_nhwc<THREADS, true>(s_pre, PS, NPAD / 8, p.pre, NPAD, x0, y0, p.W, p.H);
     if (p.final_out)
     {
         // `final` of the net (Networks.h:1129-1131) on the matrix cores: per 16 pixels one MFMA per 32 input channels,
