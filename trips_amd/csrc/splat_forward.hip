@@ -59,23 +59,6 @@ __device__ __forceinline__ Camera load_camera(const double* pose, const float* i
     return c;
 }
 
-// one launch for the counters of the view and, on the first view of a call, the status block of the whole call
-__global__ void clear_header_kernel(ViewHeader* h, ViewHeader* status)
-{
-    if (threadIdx.x < 2)
-    {
-        ViewHeader* t = threadIdx.x == 0 ? h : status;
-        if (t)
-        {
-            t->n_valid   = 0;
-            t->n_entries = 0;
-            t->overflow  = 0;
-            t->retained = t->not_identity = t->bad_index = 0;
-            t->reserved[0] = t->reserved[1] = 0;
-        }
-    }
-}
-
 // ---------------------------------------------------------------------------------------------------------
 // Projection, validity and layer selection of one point (CountAndCollectTiled, RenderForward.cu:168-366; its per-pixel
 // counter updates become per-tile ones).
@@ -217,12 +200,14 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     constexpr int WAVES = kBinThreads / 64;
     extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
     __shared__ int s_valid[2][WAVES];  // valid points of every wavefront in this step (two steps in flight)
+    __shared__ int s_flags;            // bit 0: not_identity, bit 1: bad_index, of any point of the chunk
     const Camera cam  = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L       = p.num_layers;
     const int NB      = p.geom.bin_off[L];
     bool not_identity = false;  // some point's descriptor column differs from its own index
     bool bad_index    = false;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) s_hist[i] = 0;
+    if (threadIdx.x == 0) s_flags = 0;
     __syncthreads();
 
     int begin, end;
@@ -294,61 +279,132 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
         }
     }
-    if (threadIdx.x == 0)
     {
-        p.chunk_valid[blockIdx.x] = next - begin;
-        if (next > begin) atomicAdd(&p.header->n_valid, (u64)(next - begin));
+        const int flags = (__ballot(not_identity) != 0 ? 1 : 0) | (__ballot(bad_index) != 0 ? 2 : 0);
+        if (flags && lane == 0) atomicOr(&s_flags, flags);
     }
 
-    // this workgroup's row of the histogram matrix [workgroup][bin]
+    // this workgroup's row of the histogram matrix [workgroup][bin]; its valid points and flags for the scan kernel,
+    // which adds the chunks up (no counter of the view is touched here: nothing has to be cleared before this kernel)
     __syncthreads();
     int32_t* row = p.bin_hist + (size_t)blockIdx.x * NB;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) row[i] = s_hist[i];
-    if (__ballot(not_identity) != 0 && lane == 0) atomicOr(&p.header->not_identity, 1ull);
-    if (__ballot(bad_index) != 0 && lane == 0) atomicOr(&p.status->bad_index, 1ull);
+    if (threadIdx.x == 0)
+    {
+        p.chunk_valid[blockIdx.x]                = next - begin;
+        p.chunk_valid[p.bin_groups + blockIdx.x] = s_flags;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Exclusive scan of a short int array by ONE workgroup: out[i] = sum_{k<i} in[i], out[n] = total; optionally a
-// copy of the scan (the running slots of the scatter) and the total as a counter in the header.
-__global__ __launch_bounds__(1024) void small_scan_kernel(const int32_t* __restrict__ in, int32_t* __restrict__ out,
-                                                          int32_t* __restrict__ out_copy, int n,
-                                                          unsigned long long* total_out)
+// Everything between the projection and the scatter that ONE workgroup can do, in one launch:
+//   * the view's counters, written (not added to, so that nothing has to clear them first): valid points and flags
+//     summed over the chunks of the projection, entries from the scan; on the first view of a call the status block
+//     of the whole call as well;
+//   * exclusive scan of the tile totals: bin_start[i] = sum_{k<i} bin_count[k], bin_start[NB] = total;
+//   * slices of split tiles: a tile with more than kSliceEntries bin entries (hundreds of points per pixel, e.g.
+//     tight clusters) would keep a single workgroup busy for milliseconds; it is cut into slices of kSliceEntries
+//     entries, each a workgroup of its own. slice_start[t] = number of slices of split tiles before tile t.
+// The workgroups after the first clear `clear_n` 16-byte words at `clear` (the per-cell counters of the list
+// kernels), which saves a launch of its own.
+__global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restrict__ bin_count, int32_t* __restrict__ bin_start,
+                                                         int32_t* __restrict__ slice_start, int NB, long long capacity,
+                                                         const int32_t* __restrict__ chunk_valid, int G, ViewHeader* header,
+                                                         ViewHeader* status, int first_view, int32_t* __restrict__ long_count,
+                                                         uint4* __restrict__ clear, long long clear_n)
 {
-    __shared__ int s_wave[16];
-    __shared__ int s_carry;
-    if (threadIdx.x == 0) s_carry = 0;
+    if (blockIdx.x > 0)
+    {
+        for (long long i = (long long)(blockIdx.x - 1) * 1024 + threadIdx.x; i < clear_n; i += (long long)(gridDim.x - 1) * 1024)
+            clear[i] = make_uint4(0u, 0u, 0u, 0u);
+        return;
+    }
+    __shared__ int s_wave[2][16];
+    __shared__ int s_carry[2];
+    __shared__ unsigned long long s_valid_total;
+    __shared__ int s_flags;
+    if (threadIdx.x == 0)
+    {
+        s_carry[0] = s_carry[1] = 0;
+        s_valid_total           = 0;
+        s_flags                 = 0;
+        *long_count             = 0;
+    }
     __syncthreads();
+    for (int g = threadIdx.x; g < G; g += 1024)
+    {
+        const int v = chunk_valid[g], f = chunk_valid[G + g];
+        if (v) atomicAdd(&s_valid_total, (unsigned long long)v);
+        if (f) atomicOr(&s_flags, f);
+    }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int base = 0; base < n; base += 1024)
+    for (int base = 0; base < NB; base += 1024)
     {
         const int idx = base + threadIdx.x;
-        const int v   = idx < n ? in[idx] : 0;
+        const int v   = idx < NB ? bin_count[idx] : 0;
         int inc       = v;
         for (int o = 1; o < 64; o <<= 1)
         {
             int t = __shfl_up(inc, o);
             if (lane >= o) inc += t;
         }
-        if (lane == 63) s_wave[wave] = inc;
+        if (lane == 63) s_wave[0][wave] = inc;
         __syncthreads();
         int wave_prefix = 0;
-        for (int w = 0; w < wave; ++w) wave_prefix += s_wave[w];
-        const int carry = s_carry;
-        if (idx < n)
+        for (int w = 0; w < wave; ++w) wave_prefix += s_wave[0][w];
+        const int carry = s_carry[0];
+        const int ex    = carry + wave_prefix + inc - v;  // first slot of the tile
+        if (idx < NB) bin_start[idx] = ex;
+        // slices of the tile's entries that fit the capacity
+        int sl = 0;
+        if (idx < NB)
         {
-            const int ex = carry + wave_prefix + inc - v;
-            out[idx]     = ex;
-            if (out_copy) out_copy[idx] = ex;
+            const long long first = ex;
+            long long last        = (long long)ex + v;
+            if (last > capacity) last = capacity;
+            const long long n = last > first ? last - first : 0;
+            sl                = n > kSliceEntries ? (int)((n + kSliceEntries - 1) / kSliceEntries) : 0;
         }
+        int inc2 = sl;
+        for (int o = 1; o < 64; o <<= 1)
+        {
+            int t = __shfl_up(inc2, o);
+            if (lane >= o) inc2 += t;
+        }
+        if (lane == 63) s_wave[1][wave] = inc2;
         __syncthreads();
-        if (threadIdx.x == 1023) s_carry = carry + wave_prefix + inc;
+        int wave_prefix2 = 0;
+        for (int w = 0; w < wave; ++w) wave_prefix2 += s_wave[1][w];
+        const int carry2 = s_carry[1];
+        if (idx < NB) slice_start[idx] = carry2 + wave_prefix2 + inc2 - sl;
+        __syncthreads();
+        if (threadIdx.x == 1023)
+        {
+            s_carry[0] = carry + wave_prefix + inc;
+            s_carry[1] = carry2 + wave_prefix2 + inc2;
+        }
         __syncthreads();
     }
     if (threadIdx.x == 0)
     {
-        out[n] = s_carry;
-        if (total_out) *total_out = (u64)(unsigned)s_carry;
+        bin_start[NB]   = s_carry[0];
+        slice_start[NB] = s_carry[1];
+        const unsigned long long bad = (unsigned long long)((s_flags >> 1) & 1);
+        header->n_valid      = s_valid_total;
+        header->n_entries    = (unsigned long long)(unsigned)s_carry[0];
+        header->overflow     = 0;
+        header->retained     = 0;
+        header->not_identity = (unsigned long long)(s_flags & 1);
+        header->bad_index    = 0;
+        header->reserved[0] = header->reserved[1] = 0;
+        if (first_view)
+        {
+            status->n_valid = status->n_entries = status->overflow = status->retained = status->not_identity = 0;
+            status->bad_index                                                       = bad;
+            status->reserved[0] = status->reserved[1] = 0;
+        }
+        else if (bad)
+            status->bad_index = 1;  // (the views of a call run one after the other on the stream)
     }
 }
 
@@ -452,61 +508,6 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
         }
     }
     if (dropped) atomicAdd(&p.status->overflow, (u64)dropped);
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// Slices of split tiles: a tile with more than kSliceEntries bin entries (hundreds of points per pixel, e.g. tight
-// clusters) would keep a single workgroup busy for milliseconds; it is cut into slices of kSliceEntries entries,
-// each a workgroup of its own. slice_start[t] = number of slices of split tiles before tile t (ONE workgroup).
-// Also clears the per-tile key totals, which the slices of a split tile accumulate with atomics.
-// The workgroups after the first clear `clear_n` 16-byte words at `clear` (the per-pixel counters of the list kernels),
-// which saves a launch of its own.
-__global__ __launch_bounds__(1024) void slice_plan_kernel(const int32_t* __restrict__ bin_start, long long capacity, int NB,
-                                                          int32_t* __restrict__ slice_start,
-                                                          int32_t* __restrict__ long_count, uint4* __restrict__ clear,
-                                                          long long clear_n)
-{
-    if (blockIdx.x > 0)
-    {
-        for (long long i = (long long)(blockIdx.x - 1) * 1024 + threadIdx.x; i < clear_n; i += (long long)(gridDim.x - 1) * 1024)
-            clear[i] = make_uint4(0u, 0u, 0u, 0u);
-        return;
-    }
-    if (threadIdx.x == 0) *long_count = 0;
-    __shared__ int s_wave[16];
-    __shared__ int s_carry;
-    if (threadIdx.x == 0) s_carry = 0;
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int base = 0; base < NB; base += 1024)
-    {
-        const int idx = base + threadIdx.x;
-        int v         = 0;
-        if (idx < NB)
-        {
-            const long long first = bin_start[idx];
-            long long last        = bin_start[idx + 1];
-            if (last > capacity) last = capacity;
-            const long long n = last > first ? last - first : 0;
-            v                 = n > kSliceEntries ? (int)((n + kSliceEntries - 1) / kSliceEntries) : 0;
-        }
-        int inc = v;
-        for (int o = 1; o < 64; o <<= 1)
-        {
-            int t = __shfl_up(inc, o);
-            if (lane >= o) inc += t;
-        }
-        if (lane == 63) s_wave[wave] = inc;
-        __syncthreads();
-        int wave_prefix = 0;
-        for (int w = 0; w < wave; ++w) wave_prefix += s_wave[w];
-        const int carry = s_carry;
-        if (idx < NB) slice_start[idx] = carry + wave_prefix + inc - v;
-        __syncthreads();
-        if (threadIdx.x == 1023) s_carry = carry + wave_prefix + inc;
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) slice_start[NB] = s_carry;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -1057,7 +1058,6 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
 {
     const int NB = p.geom.bin_off[p.num_layers];
 
-    hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(64), 0, stream, p.header, first_view ? p.status : (ViewHeader*)nullptr);
     const int G           = p.bin_groups;
     const size_t lds_hist = (size_t)NB * sizeof(int);
     {
@@ -1074,8 +1074,11 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     {
         ProfScope ps(prof, "bin_scan", stream);
         hipLaunchKernelGGL(bin_column_scan_kernel, dim3((NB + kScanCols - 1) / kScanCols), dim3(256), 0, stream, p.bin_hist, p.bin_count, NB, G);
-        hipLaunchKernelGGL(small_scan_kernel, dim3(1), dim3(1024), 0, stream, p.bin_count, p.bin_start,
-                           (int32_t*)nullptr, NB, &p.header->n_entries);
+        // counts and run are neighbours in the workspace: cleared together, by the workgroups behind the scanning one
+        const long long quads = 2ll * NB * kTilePixels / 4;
+        hipLaunchKernelGGL(scan_plan_kernel, dim3(1 + (unsigned)std::min<long long>((quads + 1023) / 1024, 1024)), dim3(1024), 0, stream,
+                           p.bin_count, p.bin_start, p.slice_start, NB, p.capacity, p.chunk_valid, G, p.header, p.status, first_view ? 1 : 0,
+                           p.long_count, reinterpret_cast<uint4*>(p.counts), quads);
     }
     {
         ProfScope ps(prof, "bin_scatter", stream);
@@ -1086,10 +1089,6 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     const int max_slices = (int)std::min<long long>(2 * (p.capacity / kSliceEntries) + 1, 1 << 20);
     {
         ProfScope ps(prof, "tile_count", stream);
-        // counts and run are neighbours in the workspace: cleared together, by the workgroups behind the planning one
-        const long long quads = 2ll * NB * kTilePixels / 4;
-        hipLaunchKernelGGL(slice_plan_kernel, dim3(1 + (unsigned)std::min<long long>((quads + 1023) / 1024, 1024)), dim3(1024), 0, stream,
-                           p.bin_start, p.capacity, NB, p.slice_start, p.long_count, reinterpret_cast<uint4*>(p.counts), quads);
         hipLaunchKernelGGL((tile_lists_kernel<false, 256>), dim3(NB + max_slices), dim3(256), 0, stream, p);
     }
     {

@@ -249,7 +249,7 @@ struct BackwardWorkspaceLayout
 
 struct WorkspaceLayout
 {
-    size_t chunk_valid;   // int32 [G]  valid points of every chunk of the binning kernels
+    size_t chunk_valid;   // int32 [2 G]  valid points of every chunk of the binning kernels, then the chunks' flags
     size_t prec;         // float4 [N]         point records, when there is no saved state to hold them
     size_t counts;       // int32 [Pi]   list length per cell (the points whose 2 x 2 footprint starts at that pixel)
     size_t cursor;       // int32 [Pi]   first key of each cell's list (-1 - first candidate row for a long list)
