@@ -195,6 +195,18 @@ def main():
             torch.cuda.synchronize()
             graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
             del graph
+        # the forward as a viewer runs it: eval mode, nothing kept for a backward
+        desc_eval = abi.desc_for_scene(sc, train=False)
+        ws_eval = ctx.alloc_bytes(ctx.workspace_size(desc_eval))
+        for _ in range(3):
+            ctx.forward(desc_eval, tin, images, None, ws_eval)
+        torch.cuda.synchronize()
+        v0 = time.perf_counter()
+        for _ in range(args.steps):
+            ctx.forward(desc_eval, tin, images, None, ws_eval)
+        torch.cuda.synchronize()
+        eval_ms = (time.perf_counter() - v0) * 1e3 / args.steps
+        del ws_eval
         # Adam on its own, with the step counters the product uses (int32) and with the reference's int64 state tensor
         adam_ms = {}
         for name, dt in (() if args.no_adam_variants else (("int32_counters", torch.int32), ("int64_counters", torch.int64))):
@@ -211,7 +223,7 @@ def main():
             ctx.profile_enable(False)
             adam_ms[name] = ms / max(launches, 1)
             del o2
-        return dict(graph_ms=graph_ms, events_ms=ms_per_step_events, adam_ms=adam_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
+        return dict(graph_ms=graph_ms, events_ms=ms_per_step_events, eval_ms=eval_ms, adam_ms=adam_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
                     grad_images=grad_images, grads=grads, opt=opt, counters=counters, nz=nz, total_el=total_el,
                     prof=prof, ms_per_step=ms_per_step)
 
@@ -223,6 +235,7 @@ def main():
         other_order = {"point_order": "morton_blocks (Morton curve, blocks of 256 shuffled: SceneData.cpp:115-116)",
                        "ms_per_step": round(r["ms_per_step"], 4),
                        "ms_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4),
+                       "forward_eval_mode_ms": round(r["eval_ms"], 4),
                        "fwd_bwd_kernels_ms": round(sum(v for k, v in ms_k.items() if k != "adam_fused"), 4),
                        "points_per_s": round(r["desc"].num_points / (r["ms_per_step"] * 1e-3), 1),
                        "kernels_ms": {k: round(v, 4) for k, v in ms_k.items()}}
@@ -394,7 +407,8 @@ def main():
                    "list_depth": desc.list_depth, "counters": counters},
         "frame_ms": {"fwd_bwd_kernels": round(fwd_bwd_ms, 4), "all_kernels": round(kernel_ms, 4),
                      "wall_per_step": round(ms_per_step, 4), "wall_per_step_with_kernel_events": round(r["events_ms"], 4),
-                     "wall_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4)},
+                     "wall_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4),
+                     "forward_eval_mode": round(r["eval_ms"], 4)},
         "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
         # How busy the memory system was, NOT the target metric: the HBM traffic rocprofv3 measured (committed summary
