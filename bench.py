@@ -408,7 +408,9 @@ def main():
         "frame_ms": {"fwd_bwd_kernels": round(fwd_bwd_ms, 4), "all_kernels": round(kernel_ms, 4),
                      "wall_per_step": round(ms_per_step, 4), "wall_per_step_with_kernel_events": round(r["events_ms"], 4),
                      "wall_per_step_hip_graph": None if r["graph_ms"] is None else round(r["graph_ms"], 4),
-                     "forward_eval_mode": round(r["eval_ms"], 4)},
+                     "forward_eval_mode": round(r["eval_ms"], 4),
+                     "kernel_times_from": "a second pass of the same steps with HIP events around every kernel; the timed "
+                                          "region that value comes from carries no events"},
         "hbm_frac_fwd_bwd": round(sum(alg[k] for k in alg if k != "adam_fused") / (fwd_bwd_ms * 1e-3) / 1e9 /
                                   HBM_PEAK_GBS, 4) if fwd_bwd_ms > 0 else None,
         # How busy the memory system was, NOT the target metric: the HBM traffic rocprofv3 measured (committed summary
