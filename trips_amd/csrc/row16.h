@@ -137,6 +137,24 @@ __device__ __forceinline__ u64 half_sort8(u64 v)
     return v;
 }
 
+// ---- and into four lists of 4 lanes (the DPP quads) ----
+// ascending sort of the 4 keys of each quad
+__device__ __forceinline__ u64 quad_sort4(u64 v)
+{
+    v = bitonic_step<2, 1>(v);
+    v = bitonic_step_half_ascending<2>(v);
+    v = bitonic_step_half_ascending<1>(v);
+    return v;
+}
+
+// sum over each quad, valid in its lane 0; the first two steps of row_sum_to_lane0
+__device__ __forceinline__ float quad_sum_to_lane0(float v)
+{
+    v = v + dpp_f<kDppXor1>(v);
+    v = v + dpp_f<kDppXor2>(v);
+    return v;
+}
+
 // sum over each half row, valid in its lane 0; same pairing as row_sum_to_lane0 without the last step
 __device__ __forceinline__ float half_sum_to_lane0(float v)
 {
@@ -195,6 +213,22 @@ __device__ __forceinline__ float half_exclusive_product(float f, int steps)
     {
         pre = row_shr1(pre * f, 1.f);
         pre = __builtin_amdgcn_inverse_ballot_w64(kFirst) ? 1.f : pre;  // position 8 must not see position 7
+        T   = __builtin_amdgcn_inverse_ballot_w64(latch) ? pre : T;
+        latch <<= 1;
+    }
+    return T;
+}
+
+// the same per quad (steps 1..4)
+__device__ __forceinline__ float quad_exclusive_product(float f, int steps)
+{
+    float pre = 1.f, T = 1.f;
+    u64 latch = rows4(0x2222u);
+    constexpr u64 kFirst = rows4(0x1111u);
+    for (int s = 1; s < steps; ++s)
+    {
+        pre = row_shr1(pre * f, 1.f);
+        pre = __builtin_amdgcn_inverse_ballot_w64(kFirst) ? 1.f : pre;  // a quad's first position must not see the quad before
         T   = __builtin_amdgcn_inverse_ballot_w64(latch) ? pre : T;
         latch <<= 1;
     }

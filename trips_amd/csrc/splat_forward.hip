@@ -27,6 +27,7 @@ namespace trips
 {
 typedef unsigned vu4 __attribute__((ext_vector_type(4)));
 typedef float vf4 __attribute__((ext_vector_type(4)));
+typedef int vi4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ Camera load_camera(const double* pose, const float* intr, const TripsView& v,
                                               float dist_cutoff)
@@ -844,14 +845,14 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
 
     const u64 kInf = ~0ull;
     u64 best       = kInf;
-    if (ROW == 8)
+    if (ROW <= 8)
     {
-        // at most 8 keys: none of the cells has a long list
+        // at most ROW keys: none of the cells has a long list
         // (sums of steps rather than a chain of selects: the compiler turns the chain into a table in memory)
         const int b0 = cells.s0, b1 = cells.s1 - o1, b2 = cells.s2 - o2, b3 = cells.s3 - o3;
         const int base = b0 + (sub >= o1 ? b1 - b0 : 0) + (sub >= o2 ? b2 - b1 : 0) + (sub >= o3 ? b3 - b2 : 0);
         if (sub < total) best = p.keys[(unsigned)(base + sub)];
-        best = half_sort8(best);
+        best = ROW == 8 ? half_sort8(best) : quad_sort4(best);
     }
     else
     {
@@ -906,11 +907,14 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     // exclusive transmittance: lane j latches prod_{k<j} (1 - a_k), built left to right
     // only the first n positions of a row matter; n <= K
     int nmax = n;
-    if (ROW == 8) nmax = max(nmax, __shfl_xor(nmax, 8));
+    if (ROW == 4) nmax = max(nmax, __shfl_xor(nmax, 4));
+    if (ROW <= 8) nmax = max(nmax, __shfl_xor(nmax, 8));
     nmax     = max(nmax, __shfl_xor(nmax, 16));
     nmax     = max(nmax, __shfl_xor(nmax, 32));
     nmax     = __builtin_amdgcn_readfirstlane(nmax);
-    const float T     = ROW == 8 ? half_exclusive_product(1.f - a, nmax) : row_exclusive_product(1.f - a, nmax);
+    const float T     = ROW == 4   ? quad_exclusive_product(1.f - a, nmax)
+                        : ROW == 8 ? half_exclusive_product(1.f - a, nmax)
+                                   : row_exclusive_product(1.f - a, nmax);
     const float Tc    = (T >= kAlphaDestCutoff) ? T : 0.f;
     const bool kept   = has && Tc >= kAlphaDestCutoff;
     const unsigned kb = (unsigned)((__ballot(kept) >> (grp * ROW)) & ((1u << ROW) - 1u));
@@ -921,7 +925,7 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
 #pragma unroll
     for (int c = 0; c < C; ++c) col[c] = wgt * desc[c];
 #pragma unroll
-    for (int c = 0; c < C; ++c) col[c] = ROW == 8 ? half_sum_to_lane0(col[c]) : row_sum_to_lane0(col[c]);
+    for (int c = 0; c < C; ++c) col[c] = ROW == 4 ? quad_sum_to_lane0(col[c]) : ROW == 8 ? half_sum_to_lane0(col[c]) : row_sum_to_lane0(col[c]);
 
     // background weight (RenderForward.cu:1002-1022); empty list -> 1
     float bgw_lane = (p.background_mode == TRIPS_BG_REFERENCE) ? Tc : T * (1.f - a);
@@ -961,7 +965,15 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
         if (has && sub < ret)
             p.rank[(layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)(unsigned)cid << 4) + slot] = (unsigned char)sub;
         const int mine = has ? cid : -1;
-        if (ROW == 8)
+        if (ROW == 4)
+        {
+            // one 16-byte store per lane: lane 0 of the quad carries the four ids, the others the -1 padding
+            const int i0 = __shfl(mine, 0, 4), i1 = __shfl(mine, 1, 4), i2 = __shfl(mine, 2, 4), i3 = __shfl(mine, 3, 4);
+            if (4 * sub < K)
+                __builtin_nontemporal_store(sub == 0 ? vi4{i0, i1, i2, i3} : vi4{-1, -1, -1, -1},
+                                            reinterpret_cast<vi4*>(p.lists + (((size_t)(unsigned)pix << kshift) + 4 * sub)));
+        }
+        else if (ROW == 8)
         {
             // one 8-byte store per lane covers the pixel's whole row (K <= 16 ids): lanes 0..3 carry the ids of lane
             // pairs, the others the -1 padding
@@ -974,7 +986,8 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
 }
 
 // One wavefront = eight consecutive pixels: all at once in 8-lane rows when none of them has more than 8 entries,
-// else four and four in 16-lane rows.
+// else four and four in 16-lane rows; sixteen pixels in 4-lane rows when none of the sixteen of a pair of wavefronts
+// has more than 4.
 template <int C, bool TRAIN>
 __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
 {
@@ -988,16 +1001,19 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     // the eight pixels share a tile: its layer and position are found once per wavefront, on the scalar unit
     const TileCtx tc = tile_ctx(p.geom, pix_first >> (2 * kTileShift));
     float* const img = p.image[tc.layer];
-    // The eight pixels (gx0 .. gx0 + 7, gy) gather from the cells (gx0 - 1 .. gx0 + 7) x (gy - 1, gy): lanes 0..8 read
-    // length and first key of the upper row of cells, lanes 9..17 those of the lower row; pixel g takes the cells of
-    // lanes g, g + 1, g + 9, g + 10. Cells outside the layer, and the last row and column (no footprint starts there),
-    // are empty.
+    // Two wavefronts share a run of 16 pixels (gx0 .. gx0 + 15, gy), which gather from the cells (gx0 - 1 .. gx0 + 15)
+    // x (gy - 1, gy): lanes 0..16 read length and first key of the upper row of cells, lanes 17..33 those of the lower
+    // row; pixel j of the run takes the cells of lanes j, j + 1, j + 17, j + 18. Cells outside the layer, and the last
+    // row and column (no footprint starts there), are empty. Both wavefronts read all 34 cells: when none of the 16
+    // pixels has more than 4 entries the first one takes all of them in rows of 4 lanes and the second one ends.
+    const int half       = wave & 1;
+    const int pair_first = pix_first - 8 * half;
     int c_len = 0, c_start = 0, c_read = 0;
-    if (lane < 18 && group_in_range)
+    if (lane < 34 && group_in_range)
     {
-        const int lower = lane >= 9 ? 1 : 0;
-        const int cx    = tc.x0 + (pix_first & (kTile - 1)) - 1 + (lane - 9 * lower);
-        const int cy    = tc.y0 + ((pix_first >> kTileShift) & (kTile - 1)) - 1 + lower;
+        const int lower = lane >= 17 ? 1 : 0;
+        const int cx    = tc.x0 + (pair_first & (kTile - 1)) - 1 + (lane - 17 * lower);
+        const int cy    = tc.y0 + ((pair_first >> kTileShift) & (kTile - 1)) - 1 + lower;
         if (cx >= 0 && cy >= 0 && cx < tc.w - 1 && cy < tc.h - 1)
         {
             const int bin  = tc.bin + ((cx - tc.x0) >> kTileShift) + ((cy - tc.y0) >> kTileShift) * tc.tiles_x;  // shifts round down
@@ -1011,31 +1027,38 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
                 c_read = (int)max(0ll, min((long long)c_len, p.capacity - c_start));
         }
     }
-    int tot8 = c_read + __shfl_down(c_read, 1) + __shfl_down(c_read, 9) + __shfl_down(c_read, 10);
+    // lane j < 16: readable keys of pixel j of the run
+    int tot = c_read + __shfl_down(c_read, 1) + __shfl_down(c_read, 17) + __shfl_down(c_read, 18);
     if (TRAIN)
     {
-        const int len = c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 9) + __shfl_down(c_len, 10);
-        if (lane < 8 && group_in_range) __builtin_nontemporal_store(len, p.lengths + (pix_first + lane));  // 0 for the padding of partial tiles
+        const int len = c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 17) + __shfl_down(c_len, 18);
+        // (this wavefront's eight pixels; 0 for the padding of partial tiles)
+        if ((lane >> 3) == half && group_in_range) __builtin_nontemporal_store(len, p.lengths + (pair_first + lane));
     }
-    if (lane >= 8) tot8 = 0;
-    tot8 = max(tot8, __shfl_xor(tot8, 1));
-    tot8 = max(tot8, __shfl_xor(tot8, 2));
-    tot8 = max(tot8, __shfl_xor(tot8, 4));
-    tot8 = __builtin_amdgcn_readfirstlane(tot8);
+    if (lane >= 16) tot = 0;
+    tot = max(tot, __shfl_xor(tot, 1));
+    tot = max(tot, __shfl_xor(tot, 2));
+    tot = max(tot, __shfl_xor(tot, 4));
+    const int tot8  = __builtin_amdgcn_readlane(tot, 8 * half);  // longest list of this wavefront's eight pixels
+    const int tot16 = max(__builtin_amdgcn_readlane(tot, 0), __builtin_amdgcn_readlane(tot, 8));
     // the rows take their cells' list starts and lengths from these lanes: no second memory round trip
-    auto cells_of = [&](int g)
+    auto cells_of = [&](int j)  // pixel j of the run
     {
         PixelCells c;
-        c.s0 = __shfl(c_start, g), c.s1 = __shfl(c_start, g + 1), c.s2 = __shfl(c_start, g + 9), c.s3 = __shfl(c_start, g + 10);
-        c.r0 = __shfl(c_read, g), c.r1 = __shfl(c_read, g + 1), c.r2 = __shfl(c_read, g + 9), c.r3 = __shfl(c_read, g + 10);
+        c.s0 = __shfl(c_start, j), c.s1 = __shfl(c_start, j + 1), c.s2 = __shfl(c_start, j + 17), c.s3 = __shfl(c_start, j + 18);
+        c.r0 = __shfl(c_read, j), c.r1 = __shfl(c_read, j + 1), c.r2 = __shfl(c_read, j + 17), c.r3 = __shfl(c_read, j + 18);
         return c;
     };
-    if (tot8 <= 8)
-        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, cells_of(lane >> 3));
+    if (tot16 <= 4)
+    {
+        if (half == 0) sort_blend_rows<C, TRAIN, 4>(p, tc, img, pair_first, group_in_range, cells_of(lane >> 2));
+    }
+    else if (tot8 <= 8)
+        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, cells_of(8 * half + (lane >> 3)));
     else
     {
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, cells_of(lane >> 4));
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, cells_of(4 + (lane >> 4)));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, cells_of(8 * half + (lane >> 4)));
+        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, cells_of(8 * half + 4 + (lane >> 4)));
     }
 }
 
