@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "5672dbb295ba1bacd5a84b9c094c2775f73000a4d1ebd603828e1f477a1ac5a1"
+PMC_SOURCES_SHA256 = "bd3136c45796b5399622e75a1a417ed7b8e478853fe7a27705e6e1b8b02b0f36"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129124, 302918),
-    "bin_scatter": (89130, 186670),
+    "project_bin": (129124, 303576),
+    "bin_scatter": (89132, 186677),
     "tile_count": (26193, 2296),
-    "tile_scatter": (69629, 112655),
-    "sort_blend": (331116, 455080),
-    "backward_pixels": (464996, 188162),
-    "backward_points": (1045030, 234887),
-    "adam_fused": (582966, 792823),
+    "tile_scatter": (69984, 113643),
+    "sort_blend": (331013, 450528),
+    "backward_pixels": (465130, 188215),
+    "backward_points": (1045019, 234887),
+    "adam_fused": (582967, 792823),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
