@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "bd3136c45796b5399622e75a1a417ed7b8e478853fe7a27705e6e1b8b02b0f36"
+PMC_SOURCES_SHA256 = "afb232e8d9c53d70647a4a87ebb7b04c8608e4971c1de9628147017441633189"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129124, 303576),
-    "bin_scatter": (89132, 186677),
+    "project_bin": (129125, 302584),
+    "bin_scatter": (89126, 186603),
     "tile_count": (26193, 2296),
-    "tile_scatter": (69984, 113643),
-    "sort_blend": (331013, 450528),
-    "backward_pixels": (465130, 188215),
-    "backward_points": (1045019, 234887),
-    "adam_fused": (582967, 792823),
+    "tile_scatter": (69846, 112963),
+    "sort_blend": (332969, 450626),
+    "backward_pixels": (465012, 188307),
+    "backward_points": (1045207, 234887),
+    "adam_fused": (383882, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
@@ -106,7 +106,7 @@ def main():
     import numpy as np
     import torch
     from trips_amd import abi, scenes
-    from trips_amd.adam import MyAdam
+    from trips_amd.adam import MyAdam, MyAdamPoints
     from trips_amd.renderer import SplatContext, get_context
 
     if not torch.cuda.is_available():
@@ -138,7 +138,9 @@ def main():
         gkeys = ("d_position", "d_point_size", "d_texture", "d_confidence")
         for p, k in zip(params, gkeys):
             p.grad = grads[k]
-        opt = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+        # the optimiser of the point parameters, its state packed per point (int32 step counters): a point that the view
+        # culls costs it the read of its zero gradients and nothing else
+        opt = MyAdamPoints(params, *params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
 
         def step():
             # the per-point gradients are written by the backward, every element; the block sums (background, pose,
@@ -429,7 +431,11 @@ def main():
             max(((k, v["traffic_over_alg"]) for k, v in kernels.items() if "traffic_over_alg" in v),
                 key=lambda kv: kv[1], default=None)),
         "adam": None if not r["adam_ms"] else {
-            "timed_step_state": "int32 step counters (36 B per updated element)",
+            "timed_step_state": "packed per point: {first moment, second moment, int32 step counter} of a point's 10 "
+                                "elements in one 128-byte row (36 B per updated element)",
+            "kernel_ms_packed_state_in_step": round(kernels["adam_fused"]["avg_ms"], 4),
+            "per_tensor_state": "the same step with the reference's state layout (one array per tensor), kernel alone, "
+                                "gradients of the last step",
             "kernel_ms_int32_counters": round(r["adam_ms"]["int32_counters"], 4),
             "kernel_ms_int64_counters": round(r["adam_ms"]["int64_counters"], 4),
             "alg_bytes_int32": int(alg["adam_fused"]), "alg_bytes_int64": int(alg_adam_i64),

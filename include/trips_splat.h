@@ -221,6 +221,20 @@ typedef struct TripsAdamTensor {
 /* `tensors` is a HOST array of n_tensors descriptors; one launch covers all of them. */
 int trips_adam_step_fused(TripsCtx* ctx, const TripsAdamTensor* tensors, int n_tensors, void* stream);
 
+/* The same step (MyAdam.cu:41-88,164-345) for the four parameter tensors of a point cloud at once, optimiser state
+ * packed per point: tensors[0] = t_position [N,4], tensors[1] = t_point_size [N] (NeuralPointCloudCuda.cpp:103-108),
+ * tensors[2] = texture [C,N], tensors[3] = confidence [N] (NeuralTexture.cpp:53-55), all float32; their first_moment /
+ * second_moment / steps fields are ignored. `state`: N rows of `row_bytes` bytes (a multiple of 128), zero-filled by
+ * the caller before the first step; a row holds {first moment f32, second moment f32, step counter i32} for the
+ * point's 6 + C elements in the order position xyzw, size, descriptors 0..C-1, confidence. An element is updated
+ * exactly as by trips_adam_step_fused (bit-identical weights and moments); a point whose gradients are all zero is
+ * skipped without its row being read, which per-tensor state arrays cannot offer: there the state of such a point
+ * shares every line with its neighbours'. Point removal / addition (MyAdam.cu:346-415) = row selection / appended
+ * zero rows. */
+int trips_adam_points_state_size(int num_points, int num_channels, size_t* bytes, int* row_bytes);
+int trips_adam_step_points(TripsCtx* ctx, const TripsAdamTensor tensors[4], int num_points, int num_channels, void* state,
+                           void* stream);
+
 /* pose <- se3_exp(t with rotation part * 0.1) * pose; t <- 0   (PointRenderer.cu:1428-1447)
  * tangent [F,6] f64 device, poses_se3 [F,8] f64 device. */
 int trips_apply_tangent(TripsCtx* ctx, double* tangent, double* poses_se3, int n, void* stream);

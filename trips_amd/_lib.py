@@ -16,7 +16,7 @@ SYMBOLS = [
     "trips_splat_workspace_size", "trips_splat_saved_size", "trips_splat_forward", "trips_splat_forward_static",
     "trips_splat_backward",
     "trips_splat_check", "trips_splat_counters", "trips_splat_export_lists", "trips_splat_export_points",
-    "trips_adam_step_fused", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
+    "trips_adam_step_fused", "trips_adam_points_state_size", "trips_adam_step_points", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
 ]
 # every symbol include/trips_unet.h declares
 UNET_SYMBOLS = ["trips_unet_workspace_size", "trips_unet_saved_size", "trips_unet_backward_workspace_size",
@@ -60,6 +60,8 @@ def load():
     lib.trips_splat_export_lists.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), vp, i32, vp, vp, vp, vp]
     lib.trips_splat_export_points.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), vp, i32, vp, vp, vp, vp, vp]
     lib.trips_adam_step_fused.argtypes = [vp, C.POINTER(abi.TripsAdamTensor), i32, vp]
+    lib.trips_adam_points_state_size.argtypes = [i32, i32, C.POINTER(C.c_size_t), C.POINTER(i32)]
+    lib.trips_adam_step_points.argtypes = [vp, C.POINTER(abi.TripsAdamTensor), i32, i32, vp, vp]
     lib.trips_apply_tangent.argtypes = [vp, vp, vp, i32, vp]
     lib.trips_unet_workspace_size.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_size_t)]
     lib.trips_unet_flops.argtypes = [C.POINTER(abi.TripsUnetDesc), C.POINTER(C.c_double)]

@@ -28,8 +28,19 @@ struct AdamScalars
     float lr, beta1, beta2, eps, rel_wd, abs_wd, clip, lo, hi, loss_scale;
 };
 
+// learning rate with the bias correction of step `current_step` (MyAdam.cu:66-68)
+__device__ __forceinline__ float adam_corrected_lr(const AdamScalars& h, uint32_t current_step)
+{
+    float learning_rate = h.lr;
+    learning_rate *= sqrtf(1 - powf(h.beta2, (float)current_step)) / (1 - powf(h.beta1, (float)current_step));
+    return learning_rate;
+}
+
+// `lr_of_step`: the corrected learning rate of step `lr_step`, if the caller has it already (two powf, a square root
+// and a division that elements with equal counters share); lr_step = 0 for none.
 __device__ __forceinline__ bool adam_element(const AdamScalars& h, float gradient_raw, float weight_fp, float& m,
-                                             float& v, long long& step, float& new_weight)
+                                             float& v, long long& step, float& new_weight, uint32_t lr_step = 0,
+                                             float lr_of_step = 0.f)
 {
     float gradient = gradient_raw / h.loss_scale;
     if (gradient == 0.f) return false;  // parameter not seen in this step (MyAdam.cu:57-61)
@@ -40,8 +51,8 @@ __device__ __forceinline__ bool adam_element(const AdamScalars& h, float gradien
     v                         = second_moment;
     step                      = step + 1;
     const uint32_t current_step = (uint32_t)step;
-    float learning_rate         = h.lr;
-    learning_rate *= sqrtf(1 - powf(h.beta2, (float)current_step)) / (1 - powf(h.beta1, (float)current_step));
+    float learning_rate         = lr_of_step;
+    if (current_step != lr_step) learning_rate = adam_corrected_lr(h, current_step);
     const float effective_learning_rate =
         fminf(fmaxf(learning_rate / (sqrtf(second_moment) + h.eps), h.lo), h.hi);
     const float rel            = h.rel_wd * learning_rate;
@@ -171,6 +182,176 @@ hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_
         if (tab.n == 0 || block == 0) continue;
         if (block > 0x7fffffffll) return hipErrorInvalidValue;
         hipLaunchKernelGGL(adam_fused_kernel, dim3((unsigned)block), dim3(256), 0, stream, tab);
+    }
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// The four parameter tensors of a point cloud (position [N,4], size [N], descriptors [C,N], confidence [N]) stepped
+// together, with the optimiser state packed per point: one row of CHUNKS x 16 bytes holding {first moment, second
+// moment, step counter} of the point's 6 + C elements (position xyzw, size, descriptors, confidence). A point that
+// was not seen has zero gradients everywhere and is skipped as a whole (MyAdam.cu:57-61 per element): with per-tensor
+// state arrays its state shares every line with its neighbours' and travels anyway; packed, the row of a point that
+// is skipped is never touched. Same arithmetic per element as adam_fused_kernel.
+// One thread per point. The rows of a wavefront's live points pass through LDS so that the accesses to memory stay
+// whole lines: 64 / CHUNKS rows per load instruction, lane = (row, 16-byte chunk).
+struct AdamPointsParams
+{
+    float *w_pos, *w_size, *w_tex, *w_conf;
+    const float *g_pos, *g_size, *g_tex, *g_conf;
+    uint4* state;  // [N][CHUNKS]
+    long long tex_stride;  // elements between two descriptor rows
+    int num_points;
+    AdamScalars h[4];  // position, size, descriptors, confidence
+};
+
+template <int C, int CHUNKS>
+__global__ __launch_bounds__(256) void adam_points_kernel(const AdamPointsParams p)
+{
+    constexpr int E   = 6 + C;
+    constexpr int LS  = CHUNKS + 1;  // LDS row stride in 16-byte words: an odd multiple spreads the rows over the banks
+    constexpr int RPP = 64 / CHUNKS;  // rows per load instruction
+    static_assert(3 * E <= 4 * CHUNKS, "row too short");
+    __shared__ uint4 s_rows[4][64 * LS];
+    __shared__ unsigned char s_list[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long long first = (long long)blockIdx.x * 256 + wave * 64;  // first point of this wavefront
+    const long long point = first + lane;
+    const bool in         = point < p.num_points;
+    float g[E];
+    {
+        const float4 gp = in ? reinterpret_cast<const float4*>(p.g_pos)[point] : make_float4(0.f, 0.f, 0.f, 0.f);
+        g[0] = gp.x, g[1] = gp.y, g[2] = gp.z, g[3] = gp.w;
+        g[4] = in ? p.g_size[point] : 0.f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) g[5 + c] = in ? p.g_tex[c * p.tex_stride + point] : 0.f;
+        g[5 + C] = in ? p.g_conf[point] : 0.f;
+    }
+    bool live = false;
+#pragma unroll
+    for (int e = 0; e < E; ++e) live = live || g[e] != 0.f;
+    const unsigned long long mask = __ballot(live);
+    if (mask == 0) return;  // (no barrier below: a wavefront is on its own)
+    const int nlive = (int)__popcll(mask);
+    if (live) s_list[wave][__popcll(mask & ((1ull << lane) - 1ull))] = (unsigned char)lane;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // the weights of the live points: in flight beside the rows
+    float w[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) w[e] = 0.f;
+    if (live)
+    {
+        const float4 wp = reinterpret_cast<const float4*>(p.w_pos)[point];
+        w[0] = wp.x, w[1] = wp.y, w[2] = wp.z, w[3] = wp.w;
+        w[4] = p.w_size[point];
+#pragma unroll
+        for (int c = 0; c < C; ++c) w[5 + c] = p.w_tex[c * p.tex_stride + point];
+        w[5 + C] = p.w_conf[point];
+    }
+    const int my_r = lane / CHUNKS, my_c = lane - my_r * CHUNKS;
+    for (int base = 0; base < nlive; base += RPP)
+    {
+        const int r = base + my_r;
+        if (my_r < RPP && r < nlive)
+        {
+            const int src                      = s_list[wave][r];
+            s_rows[wave][src * LS + my_c] = p.state[(first + src) * CHUNKS + my_c];
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (live)
+    {
+        uint32_t row[4 * CHUNKS];
+#pragma unroll
+        for (int j = 0; j < CHUNKS; ++j)
+        {
+            const uint4 t = s_rows[wave][lane * LS + j];
+            row[4 * j] = t.x, row[4 * j + 1] = t.y, row[4 * j + 2] = t.z, row[4 * j + 3] = t.w;
+        }
+        // The elements of a tensor are mostly updated together, so their counters agree: the bias correction of the
+        // tensor's largest counter is computed once and taken by every element whose new counter equals it.
+        int top[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+        {
+            const int t = e < 4 ? 0 : e == 4 ? 1 : e < 5 + C ? 2 : 3;
+            top[t]      = max(top[t], (int)row[3 * e + 2]);
+        }
+        float top_lr[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) top_lr[t] = adam_corrected_lr(p.h[t], (uint32_t)(top[t] + 1));
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+        {
+            const int t = e < 4 ? 0 : e == 4 ? 1 : e < 5 + C ? 2 : 3;
+            float m = __uint_as_float(row[3 * e]), v = __uint_as_float(row[3 * e + 1]), nw;
+            long long s = (long long)(int)row[3 * e + 2];
+            if (adam_element(p.h[t], g[e], w[e], m, v, s, nw, (uint32_t)(top[t] + 1), top_lr[t]))
+            {
+                w[e]           = nw;
+                row[3 * e]     = __float_as_uint(m);
+                row[3 * e + 1] = __float_as_uint(v);
+                row[3 * e + 2] = (uint32_t)(int)s;
+            }
+        }
+        reinterpret_cast<float4*>(p.w_pos)[point] = make_float4(w[0], w[1], w[2], w[3]);
+        p.w_size[point]                          = w[4];
+#pragma unroll
+        for (int c = 0; c < C; ++c) p.w_tex[c * p.tex_stride + point] = w[5 + c];
+        p.w_conf[point] = w[5 + C];
+#pragma unroll
+        for (int j = 0; j < CHUNKS; ++j)
+            s_rows[wave][lane * LS + j] = make_uint4(row[4 * j], row[4 * j + 1], row[4 * j + 2], row[4 * j + 3]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int base = 0; base < nlive; base += RPP)
+    {
+        const int r = base + my_r;
+        if (my_r < RPP && r < nlive)
+        {
+            const int src                          = s_list[wave][r];
+            p.state[(first + src) * CHUNKS + my_c] = s_rows[wave][src * LS + my_c];
+        }
+    }
+}
+
+// 16-byte chunks of a packed state row: 12 bytes per element, rounded up to whole 128-byte lines
+int adam_points_row_chunks(int channels) { return ((6 + channels) * 12 + 127) / 128 * 8; }
+
+hipError_t launch_adam_points(const TripsAdamTensor tensors[4], int num_points, int channels, void* state, hipStream_t stream,
+                              Profiler* prof)
+{
+    ProfScope ps(prof, "adam_fused", stream);
+    if (num_points <= 0) return hipSuccess;
+    AdamPointsParams p;
+    p.w_pos = (float*)tensors[0].weights, p.w_size = (float*)tensors[1].weights, p.w_tex = (float*)tensors[2].weights,
+    p.w_conf = (float*)tensors[3].weights;
+    p.g_pos = (const float*)tensors[0].grads, p.g_size = (const float*)tensors[1].grads, p.g_tex = (const float*)tensors[2].grads,
+    p.g_conf = (const float*)tensors[3].grads;
+    p.state      = reinterpret_cast<uint4*>(state);
+    p.tex_stride = num_points;
+    p.num_points = num_points;
+    for (int i = 0; i < 4; ++i)
+    {
+        const TripsAdamTensor& T = tensors[i];
+        p.h[i] = AdamScalars{T.lr, T.beta1, T.beta2, T.eps, T.relative_weight_decay, T.absolute_weight_decay,
+                             T.weight_clipping_magnitude, T.lower_lr_bound, T.upper_lr_bound, T.loss_scale};
+    }
+    const unsigned blocks = (unsigned)((num_points + 255) / 256);
+    switch (channels)
+    {
+        case 3: hipLaunchKernelGGL((adam_points_kernel<3, 8>), dim3(blocks), dim3(256), 0, stream, p); break;
+        case 4: hipLaunchKernelGGL((adam_points_kernel<4, 8>), dim3(blocks), dim3(256), 0, stream, p); break;
+        case 6: hipLaunchKernelGGL((adam_points_kernel<6, 16>), dim3(blocks), dim3(256), 0, stream, p); break;
+        case 8: hipLaunchKernelGGL((adam_points_kernel<8, 16>), dim3(blocks), dim3(256), 0, stream, p); break;
+        case 16: hipLaunchKernelGGL((adam_points_kernel<16, 24>), dim3(blocks), dim3(256), 0, stream, p); break;
+        default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }

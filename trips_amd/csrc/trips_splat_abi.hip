@@ -16,6 +16,9 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
                                Profiler* prof);
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof);
 hipError_t launch_adam(const TripsAdamTensor* tensors, int n_tensors, hipStream_t stream, Profiler* prof);
+int adam_points_row_chunks(int channels);
+hipError_t launch_adam_points(const TripsAdamTensor tensors[4], int num_points, int channels, void* state, hipStream_t stream,
+                              Profiler* prof);
 hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t stream);
 hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, const int32_t* cid_of, int n, float* ip,
                                 float* depth, float* size_px, int32_t* max_layer, hipStream_t stream);
@@ -673,6 +676,43 @@ int trips_adam_step_fused(TripsCtx* ctx, const TripsAdamTensor* tensors, int n_t
             return fail(TRIPS_ERR_UNSUPPORTED, "tensor %d: steps_dtype %d", i, t.steps_dtype);
     }
     hipError_t e = launch_adam(tensors, n_tensors, reinterpret_cast<hipStream_t>(stream_), ctx->prof.enabled ? &ctx->prof : nullptr);
+    if (e != hipSuccess) return hip_fail(e, "adam launch");
+    return TRIPS_OK;
+}
+
+int trips_adam_points_state_size(int num_points, int num_channels, size_t* bytes, int* row_bytes)
+{
+    if (!bytes) return fail(TRIPS_ERR_INVALID_ARG, "bytes is NULL");
+    if (num_points < 0) return fail(TRIPS_ERR_INVALID_ARG, "num_points < 0");
+    if (!channels_ok(num_channels)) return fail(TRIPS_ERR_UNSUPPORTED, "num_channels %d not in {3,4,6,8,16}", num_channels);
+    const int row = adam_points_row_chunks(num_channels) * 16;
+    if (row_bytes) *row_bytes = row;
+    *bytes = (size_t)num_points * (size_t)row;
+    return TRIPS_OK;
+}
+
+int trips_adam_step_points(TripsCtx* ctx, const TripsAdamTensor tensors[4], int num_points, int num_channels, void* state,
+                           void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (!tensors) return fail(TRIPS_ERR_INVALID_ARG, "tensors is NULL");
+    if (num_points < 0) return fail(TRIPS_ERR_INVALID_ARG, "num_points < 0");
+    if (!channels_ok(num_channels)) return fail(TRIPS_ERR_UNSUPPORTED, "num_channels %d not in {3,4,6,8,16}", num_channels);
+    if (num_points == 0) return TRIPS_OK;
+    if (!state || (reinterpret_cast<uintptr_t>(state) & 127)) return fail(TRIPS_ERR_INVALID_ARG, "state must be a 128-byte aligned device pointer");
+    const long long want[4] = {4ll * num_points, num_points, (long long)num_channels * num_points, num_points};
+    for (int i = 0; i < 4; ++i)
+    {
+        const TripsAdamTensor& t = tensors[i];
+        if (t.n != want[i]) return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: %lld elements, %lld expected", i, (long long)t.n, want[i]);
+        if (!t.weights || !t.grads) return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: NULL pointer", i);
+        if (t.dtype != TRIPS_DTYPE_F32) return fail(TRIPS_ERR_UNSUPPORTED, "tensor %d: dtype %d (the point parameters are float32)", i, t.dtype);
+        if (!(t.loss_scale != 0.f)) return fail(TRIPS_ERR_INVALID_ARG, "tensor %d: loss_scale is 0", i);
+    }
+    if ((reinterpret_cast<uintptr_t>(tensors[0].weights) & 15) || (reinterpret_cast<uintptr_t>(tensors[0].grads) & 15))
+        return fail(TRIPS_ERR_INVALID_ARG, "position and its gradient must be 16-byte aligned");
+    hipError_t e = launch_adam_points(tensors, num_points, num_channels, state, reinterpret_cast<hipStream_t>(stream_),
+                                      ctx->prof.enabled ? &ctx->prof : nullptr);
     if (e != hipSuccess) return hip_fail(e, "adam launch");
     return TRIPS_OK;
 }

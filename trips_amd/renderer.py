@@ -178,6 +178,19 @@ class SplatContext:
         arr = (abi.TripsAdamTensor * n)(*tensor_descs)
         _lib.check(self.lib.trips_adam_step_fused(self.ctx, arr, n, _stream_ptr(self.device)))
 
+    def adam_points_state_size(self, num_points, num_channels):
+        """(bytes, bytes per row) of the packed optimiser state of a point cloud."""
+        b, row = C.c_size_t(0), C.c_int(0)
+        _lib.check(self.lib.trips_adam_points_state_size(int(num_points), int(num_channels), C.byref(b), C.byref(row)))
+        return b.value, row.value
+
+    def adam_step_points(self, tensor_descs, num_points, num_channels, state):
+        """tensor_descs: four abi.TripsAdamTensor (position, point size, descriptors, confidence); state: the packed
+        rows (a device tensor of adam_points_state_size bytes, zero before the first step)."""
+        arr = (abi.TripsAdamTensor * 4)(*tensor_descs)
+        _lib.check(self.lib.trips_adam_step_points(self.ctx, arr, int(num_points), int(num_channels), _ptr(state),
+                                                   _stream_ptr(self.device)))
+
     def apply_tangent(self, tangent, poses_se3):
         assert tangent.dtype == torch.float64 and poses_se3.dtype == torch.float64
         assert tangent.is_contiguous() and poses_se3.is_contiguous()
