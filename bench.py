@@ -31,15 +31,15 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "afb232e8d9c53d70647a4a87ebb7b04c8608e4971c1de9628147017441633189"
+PMC_SOURCES_SHA256 = "768e6add7425866a1537ecc6e63cdc3343effd7e31ba9ac494bb9864cac29157"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129125, 302584),
-    "bin_scatter": (89126, 186603),
+    "project_bin": (129126, 302826),
+    "bin_scatter": (89112, 186582),
     "tile_count": (26193, 2296),
-    "tile_scatter": (69846, 112963),
-    "sort_blend": (332969, 450626),
-    "backward_pixels": (465012, 188307),
-    "backward_points": (1045207, 234887),
+    "tile_scatter": (69686, 114744),
+    "sort_blend": (331033, 450783),
+    "backward_pixels": (464969, 188190),
+    "backward_points": (1045773, 234887),
     "adam_fused": (383882, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",

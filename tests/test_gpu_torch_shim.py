@@ -110,6 +110,42 @@ def test_cpp_myadam_and_apply_tangent(oracle):
 
 
 @pytest.mark.gpu
+def test_cpp_myadam_points_equals_per_tensor_myadam():
+    """torch::optim::MyAdamPoints (C++ shim, state packed per point) against the Python MyAdam with the reference's
+    per-tensor state: the same groups and options, points without gradient, a step in which the sizes have no
+    gradient, and the pose tangents as a parameter outside the packed four. Bit for bit."""
+    from trips_amd.adam import MyAdam
+    sc = scenes.tiny(n=3001, w=48, h=40, f=45.0, num_layers=2, list_depth=16, seed=57)
+    s, t = _session(sc)
+    names = ("position", "point_size", "texture", "confidence", "tangent_poses")
+    twin = {k: torch.nn.Parameter(t[k].detach().clone()) for k in names}
+    lr = 1e-2
+    plain = MyAdam([{"params": [twin["position"]]}, {"params": [twin["point_size"]]},
+                    {"params": [twin["texture"]], "lr": 2 * lr}, {"params": [twin["confidence"]]},
+                    {"params": [twin["tangent_poses"]]}], lr=lr)
+    s.make_adam_points([t["tangent_poses"]], lr)
+    rng = np.random.default_rng(4)
+    n = sc.num_points
+    for step in range(3):
+        dead = torch.as_tensor(rng.random(n) < 0.4).cuda()
+        for k in names:
+            g = torch.as_tensor(rng.normal(0, 1, tuple(t[k].shape))).to(t[k].dtype).cuda()
+            if k in ("position", "point_size"):
+                g[dead] = 0
+            elif k in ("texture", "confidence"):
+                g[:, dead] = 0
+            if k == "point_size" and step == 1:
+                g = None
+            t[k].grad = g
+            twin[k].grad = None if g is None else g.clone()
+        s.adam_step()
+        plain.step()
+    torch.cuda.synchronize()
+    for k in names:
+        assert torch.equal(t[k].detach(), twin[k].detach()), k
+
+
+@pytest.mark.gpu
 def test_cpp_unet_forward_backward_matches_python_mirror():
     """The C++ module (trips_unet_torch.cpp) and the Python mirror drive the same kernels: same weights -> same
     output and gradients; torch autograd through the C++ autograd node reaches inputs and parameters."""

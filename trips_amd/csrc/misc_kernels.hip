@@ -2,6 +2,7 @@
 //
 //   adam_fused_kernel    <- adam_step      src/lib/models/MyAdam.cu:41-88 (one launch for all tensors instead of
 //                                          one 128-thread launch per tensor, :226-288)
+//   adam_points_kernel   <- the same step for the four tensors of a point cloud, optimiser state packed per point
 //   apply_tangent_kernel <- ApplyTangent   src/lib/rendering/PointRenderer.cu:1428-1447
 #include <float.h>
 

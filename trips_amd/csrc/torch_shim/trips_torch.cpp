@@ -351,6 +351,61 @@ MyAdam::MyAdam(std::vector<OptimizerParamGroup> param_groups, MyAdamOptions defa
     TORCH_CHECK(defaults.absolute_weight_decay() >= 0, "Invalid absolute_weight_decay value: ", defaults.absolute_weight_decay());
 }
 
+bool MyAdam::describe(Tensor& p, OptimizerParamGroup& group, bool packed, TripsAdamTensor& t, std::vector<Tensor>& keep)
+{
+    auto grad = p.grad();
+    TORCH_CHECK(!grad.is_sparse(), "Adam does not support sparse gradients");
+    TORCH_CHECK(p.is_contiguous(), "MyAdam needs contiguous parameters");
+    TORCH_CHECK(p.scalar_type() == torch::kFloat || p.scalar_type() == torch::kDouble, "float32 / float64 only");
+    auto& options = static_cast<MyAdamOptions&>(group.options());
+    int64_t current_step = 0;
+    t                    = TripsAdamTensor{};
+    if (!packed)
+    {
+        auto it = state_.find(p.unsafeGetTensorImpl());
+        if (it == state_.end())
+        {
+            auto st = std::make_unique<MyAdamParamState>();
+            st->param_steps(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kInt32));
+            st->first_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
+            st->second_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
+            st->current_step(0);
+            state_[p.unsafeGetTensorImpl()] = std::move(st);
+        }
+        auto& st = static_cast<MyAdamParamState&>(*state_[p.unsafeGetTensorImpl()]);
+        st.current_step(st.current_step() + 1);
+        current_step    = st.current_step();
+        t.first_moment  = st.first_moments().data_ptr<float>();
+        t.second_moment = st.second_moments().data_ptr<float>();
+        t.steps         = st.param_steps().data_ptr();
+        t.steps_dtype   = st.param_steps().scalar_type() == torch::kInt32 ? TRIPS_STEPS_I32 : TRIPS_STEPS_I64;
+    }
+    const double beta1 = std::get<0>(options.betas()), beta2 = std::get<1>(options.betas());
+    Tensor g = grad.contiguous();
+    keep.push_back(g);
+    t.weights                   = p.data_ptr();
+    t.grads                     = g.data_ptr();
+    t.n                         = p.numel();
+    t.dtype                     = p.scalar_type() == torch::kDouble ? TRIPS_DTYPE_F64 : TRIPS_DTYPE_F32;
+    t.lr                        = (float)options.lr();
+    t.beta1                     = (float)beta1;
+    t.beta2                     = (float)beta2;
+    t.eps                       = (float)options.eps();
+    t.relative_weight_decay     = (float)options.relative_weight_decay();
+    t.absolute_weight_decay     = (float)options.absolute_weight_decay();
+    t.weight_clipping_magnitude = (float)options.weight_clipping_magnitude();
+    t.lower_lr_bound            = 0;
+    t.upper_lr_bound            = FLT_MAX;
+    t.loss_scale                = 1.f;
+    if (options.adabound() && !packed)
+    {
+        // AdaBound bounds, MyAdam.cu:213-221
+        t.lower_lr_bound = 0.1f - 0.1f / ((1 - (float)beta2) * (float)current_step + 1);
+        t.upper_lr_bound = 0.1f + 0.1f / ((1 - (float)beta2) * (float)current_step);
+    }
+    return true;
+}
+
 torch::Tensor MyAdam::step(LossClosure closure)
 {
     NoGradGuard no_grad;
@@ -368,52 +423,8 @@ torch::Tensor MyAdam::step(LossClosure closure)
         for (auto& p : group.params())
         {
             if (!p.grad().defined()) continue;
-            auto grad = p.grad();
-            TORCH_CHECK(!grad.is_sparse(), "Adam does not support sparse gradients");
-            TORCH_CHECK(p.is_contiguous(), "MyAdam needs contiguous parameters");
-            TORCH_CHECK(p.scalar_type() == torch::kFloat || p.scalar_type() == torch::kDouble, "float32 / float64 only");
-            auto& options = static_cast<MyAdamOptions&>(group.options());
-            auto it       = state_.find(p.unsafeGetTensorImpl());
-            if (it == state_.end())
-            {
-                auto st = std::make_unique<MyAdamParamState>();
-                st->param_steps(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kInt32));
-                st->first_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
-                st->second_moments(torch::zeros_like(p, MemoryFormat::Preserve).to(torch::kFloat32));
-                st->current_step(0);
-                state_[p.unsafeGetTensorImpl()] = std::move(st);
-            }
-            auto& st = static_cast<MyAdamParamState&>(*state_[p.unsafeGetTensorImpl()]);
-            st.current_step(st.current_step() + 1);
-            const double beta1 = std::get<0>(options.betas()), beta2 = std::get<1>(options.betas());
-            float lower = 0, upper = FLT_MAX;
-            if (options.adabound())
-            {
-                // AdaBound bounds, MyAdam.cu:213-221
-                lower = 0.1f - 0.1f / ((1 - (float)beta2) * (float)st.current_step() + 1);
-                upper = 0.1f + 0.1f / ((1 - (float)beta2) * (float)st.current_step());
-            }
-            Tensor g = grad.contiguous();
-            keep.push_back(g);
-            TripsAdamTensor t{};
-            t.weights                   = p.data_ptr();
-            t.grads                     = g.data_ptr();
-            t.first_moment              = st.first_moments().data_ptr<float>();
-            t.second_moment             = st.second_moments().data_ptr<float>();
-            t.steps                     = st.param_steps().data_ptr();
-            t.steps_dtype               = st.param_steps().scalar_type() == torch::kInt32 ? TRIPS_STEPS_I32 : TRIPS_STEPS_I64;
-            t.n                         = p.numel();
-            t.dtype                     = p.scalar_type() == torch::kDouble ? TRIPS_DTYPE_F64 : TRIPS_DTYPE_F32;
-            t.lr                        = (float)options.lr();
-            t.beta1                     = (float)beta1;
-            t.beta2                     = (float)beta2;
-            t.eps                       = (float)options.eps();
-            t.relative_weight_decay     = (float)options.relative_weight_decay();
-            t.absolute_weight_decay     = (float)options.absolute_weight_decay();
-            t.weight_clipping_magnitude = (float)options.weight_clipping_magnitude();
-            t.lower_lr_bound            = lower;
-            t.upper_lr_bound            = upper;
-            t.loss_scale                = 1.f;
+            TripsAdamTensor t;
+            describe(p, group, false, t, keep);
             descs.push_back(t);
             any = p;
         }
@@ -422,6 +433,121 @@ torch::Tensor MyAdam::step(LossClosure closure)
         check(trips_adam_step_fused(context_for(any), descs.data(), (int)descs.size(), current_stream(any)),
               "trips_adam_step_fused");
     return loss;
+}
+
+MyAdamPoints::MyAdamPoints(std::vector<OptimizerParamGroup> param_groups, Tensor position, Tensor point_size, Tensor texture,
+                           Tensor confidence, MyAdamOptions defaults)
+    : MyAdam(std::move(param_groups), defaults)
+{
+    packed_[0] = position, packed_[1] = point_size, packed_[2] = texture, packed_[3] = confidence;
+    for (auto& q : packed_)
+    {
+        TORCH_CHECK(q.defined() && q.scalar_type() == torch::kFloat && q.is_contiguous(),
+                    "MyAdamPoints: the point parameters must be contiguous float32 tensors");
+        bool found = false;
+        for (auto& group : param_groups_)
+            for (auto& p : group.params()) found = found || p.unsafeGetTensorImpl() == q.unsafeGetTensorImpl();
+        TORCH_CHECK(found, "MyAdamPoints: position, point_size, texture and confidence must be among the optimised parameters");
+    }
+}
+
+int MyAdamPoints::slot_of(const Tensor& p) const
+{
+    for (int i = 0; i < 4; ++i)
+        if (packed_[i].unsafeGetTensorImpl() == p.unsafeGetTensorImpl()) return i;
+    return -1;
+}
+
+torch::Tensor MyAdamPoints::step(LossClosure closure)
+{
+    NoGradGuard no_grad;
+    Tensor loss = {};
+    if (closure != nullptr)
+    {
+        at::AutoGradMode enable_grad(true);
+        loss = closure();
+    }
+    bool any_packed_grad = false;
+    for (auto& q : packed_) any_packed_grad = any_packed_grad || q.grad().defined();
+    std::vector<TripsAdamTensor> descs;
+    TripsAdamTensor packed_descs[4];
+    std::vector<Tensor> keep;
+    Tensor any;
+    for (auto& group : param_groups_)
+    {
+        for (auto& p : group.params())
+        {
+            const int slot = slot_of(p);
+            if (slot < 0)
+            {
+                if (!p.grad().defined()) continue;
+                TripsAdamTensor t;
+                describe(p, group, false, t, keep);
+                descs.push_back(t);
+                any = p;
+                continue;
+            }
+            if (!any_packed_grad) continue;
+            const bool has_grad = p.grad().defined();
+            if (!has_grad)
+            {
+                // a point parameter without a gradient in this step: zeros leave it and its state as they are
+                if (!zero_grads_[slot].defined() || zero_grads_[slot].sizes() != p.sizes()) zero_grads_[slot] = torch::zeros_like(p);
+                p.mutable_grad() = zero_grads_[slot];
+            }
+            describe(p, group, true, packed_descs[slot], keep);
+            if (!has_grad) p.mutable_grad() = Tensor();
+            if (has_grad) packed_steps_[slot] += 1;
+            auto& options = static_cast<MyAdamOptions&>(group.options());
+            if (options.adabound() && packed_steps_[slot] > 0)
+            {
+                const float beta2                 = (float)std::get<1>(options.betas());
+                packed_descs[slot].lower_lr_bound = 0.1f - 0.1f / ((1 - beta2) * (float)packed_steps_[slot] + 1);
+                packed_descs[slot].upper_lr_bound = 0.1f + 0.1f / ((1 - beta2) * (float)packed_steps_[slot]);
+            }
+        }
+    }
+    if (any_packed_grad)
+    {
+        const int64_t n = packed_[0].size(0), c = packed_[2].size(0);
+        TORCH_CHECK(packed_[0].dim() == 2 && packed_[0].size(1) == 4 && packed_[2].dim() == 2 && packed_[2].size(1) == n &&
+                        packed_[1].numel() == n && packed_[3].numel() == n,
+                    "MyAdamPoints: position [N,4], point_size [N], texture [C,N], confidence [N] expected");
+        size_t bytes = 0;
+        int row      = 0;
+        check(trips_adam_points_state_size((int)n, (int)c, &bytes, &row), "trips_adam_points_state_size");
+        if (!packed_state.defined())
+            packed_state = torch::zeros({n, row / 4}, torch::TensorOptions().dtype(torch::kInt32).device(packed_[0].device()));
+        TORCH_CHECK(packed_state.size(0) == n && packed_state.size(1) == row / 4,
+                    "MyAdamPoints: the number of points changed without shrinkInternalState / appendToInternalState");
+        check(trips_adam_step_points(context_for(packed_[0]), packed_descs, (int)n, (int)c, packed_state.data_ptr(),
+                                     current_stream(packed_[0])),
+              "trips_adam_step_points");
+    }
+    if (!descs.empty())
+        check(trips_adam_step_fused(context_for(any), descs.data(), (int)descs.size(), current_stream(any)),
+              "trips_adam_step_fused");
+    return loss;
+}
+
+void MyAdamPoints::shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep)
+{
+    TORCH_CHECK(param_group_index < (int)param_groups_.size());
+    for (auto& p : param_groups_[param_group_index].params())
+        if (slot_of(p) == 2 && packed_state.defined())
+            packed_state = packed_state.index_select(0, indices_to_keep.squeeze().to(packed_state.device())).contiguous();
+    MyAdam::shrinkInternalState(param_group_index, indices_to_keep);  // (the packed four have no per-tensor state)
+}
+
+void MyAdamPoints::appendToInternalState(int param_group_index, int new_size)
+{
+    TORCH_CHECK(param_group_index < (int)param_groups_.size());
+    for (auto& p : param_groups_[param_group_index].params())
+        if (slot_of(p) == 2 && packed_state.defined())
+            packed_state = torch::cat({packed_state, torch::zeros({new_size - packed_state.size(0), packed_state.size(1)},
+                                                                  packed_state.options())})
+                               .contiguous();
+    MyAdam::appendToInternalState(param_group_index, new_size);
 }
 
 // state follows the last dimension of the parameter (MyAdam.cu:346-415)

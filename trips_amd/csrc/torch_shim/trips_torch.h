@@ -172,8 +172,35 @@ class MyAdam : public Optimizer
     {
     }
     torch::Tensor step(LossClosure closure = nullptr) override;
-    void shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep);
-    void appendToInternalState(int param_group_index, int new_size);
+    virtual void shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep);
+    virtual void appendToInternalState(int param_group_index, int new_size);
+
+   protected:
+    // one parameter's step description for the library (creates its state on first use unless `packed`)
+    bool describe(Tensor& p, OptimizerParamGroup& group, bool packed, TripsAdamTensor& t, std::vector<Tensor>& keep);
+};
+
+// MyAdam whose state for the four parameter tensors of a point cloud (t_position [N,4], t_point_size [N,1],
+// texture [C,N], confidence_value_of_point [1,N]; NeuralPointCloudCuda.cpp:103-108, NeuralTexture.cpp:53-55) is one
+// row per point of {first moment, second moment, step counter} of the point's elements. The four must be among the
+// parameters of the groups (each group's options apply as usual); every other parameter is stepped as MyAdam steps
+// it. Same arithmetic per element, bit-identical results; a point whose gradients are all zero is skipped without its
+// state being read. Point removal / addition: the rows follow the group that holds `texture`.
+class MyAdamPoints : public MyAdam
+{
+   public:
+    MyAdamPoints(std::vector<OptimizerParamGroup> param_groups, Tensor position, Tensor point_size, Tensor texture,
+                 Tensor confidence, MyAdamOptions defaults = {});
+    torch::Tensor step(LossClosure closure = nullptr) override;
+    void shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep) override;
+    void appendToInternalState(int param_group_index, int new_size) override;
+    torch::Tensor packed_state;  // [N, row bytes / 4] int32, defined after the first step
+
+   private:
+    int slot_of(const Tensor& p) const;
+    Tensor packed_[4];
+    Tensor zero_grads_[4];
+    int64_t packed_steps_[4] = {0, 0, 0, 0};
 };
 }  // namespace torch::optim
 

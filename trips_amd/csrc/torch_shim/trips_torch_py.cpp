@@ -186,5 +186,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         .def("make_adam",
              [](Session& s, std::vector<torch::Tensor> params, double lr)
              { s.optimizer = std::make_unique<torch::optim::MyAdam>(params, torch::optim::MyAdamOptions(lr)); })
+        .def("make_adam_points",
+             [](Session& s, std::vector<torch::Tensor> others, double lr)
+             {
+                 // one group per point tensor (descriptors with twice the learning rate), one for the rest
+                 auto& pc = *s.scene.point_cloud_cuda;
+                 auto& tx = *s.scene.texture;
+                 std::vector<torch::optim::OptimizerParamGroup> groups;
+                 groups.emplace_back(std::vector<torch::Tensor>{pc.t_position});
+                 groups.emplace_back(std::vector<torch::Tensor>{pc.t_point_size});
+                 groups.emplace_back(std::vector<torch::Tensor>{tx.texture}, std::make_unique<torch::optim::MyAdamOptions>(2 * lr));
+                 groups.emplace_back(std::vector<torch::Tensor>{tx.confidence_value_of_point});
+                 if (!others.empty()) groups.emplace_back(others);
+                 s.optimizer = std::make_unique<torch::optim::MyAdamPoints>(groups, pc.t_position, pc.t_point_size, tx.texture,
+                                                                            tx.confidence_value_of_point,
+                                                                            torch::optim::MyAdamOptions(lr));
+             })
         .def("adam_step", [](Session& s) { s.optimizer->step(); });
 }
