@@ -175,6 +175,20 @@ def test_view_validation_and_null_arguments():
     assert lib.trips_profile_enable(None, 1) == abi.TRIPS_ERR_INVALID_ARG
 
 
+def test_packed_adam_state_size_host_only():
+    """Rows of the packed optimiser state: 12 bytes per element of a point (6 + C of them), whole 128-byte lines."""
+    lib = _lib.load()
+    for c, row in ((3, 128), (4, 128), (6, 256), (8, 256), (16, 384)):
+        b, r = C.c_size_t(0), C.c_int(0)
+        assert lib.trips_adam_points_state_size(1000, c, C.byref(b), C.byref(r)) == 0
+        assert r.value == row and b.value == 1000 * row and 12 * (6 + c) <= row
+    b = C.c_size_t(0)
+    assert lib.trips_adam_points_state_size(10, 5, C.byref(b), None) == abi.TRIPS_ERR_UNSUPPORTED
+    assert lib.trips_adam_points_state_size(-1, 4, C.byref(b), None) == abi.TRIPS_ERR_INVALID_ARG
+    assert lib.trips_adam_points_state_size(10, 4, None, None) == abi.TRIPS_ERR_INVALID_ARG
+    assert lib.trips_adam_step_points(None, None, 10, 4, None, None) == abi.TRIPS_ERR_INVALID_ARG
+
+
 def test_too_many_points_for_32_bit_offsets():
     lib = _lib.load()
     sc = scenes.tiny(n=10)
