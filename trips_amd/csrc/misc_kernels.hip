@@ -252,14 +252,27 @@ __global__ __launch_bounds__(256) void adam_points_kernel(const AdamPointsParams
         w[5 + C] = p.w_conf[point];
     }
     const int my_r = lane / CHUNKS, my_c = lane - my_r * CHUNKS;
-    for (int base = 0; base < nlive; base += RPP)
     {
-        const int r = base + my_r;
-        if (my_r < RPP && r < nlive)
+        // every load of the wavefront's rows is issued before the first one is waited for (as a loop that loads and
+        // stores pass by pass the round trips to memory ran one after the other)
+        constexpr int PASSES = (64 + RPP - 1) / RPP;
+        uint4 v[PASSES];
+        int src[PASSES];
+#pragma unroll
+        for (int it = 0; it < PASSES; ++it)
         {
-            const int src                      = s_list[wave][r];
-            s_rows[wave][src * LS + my_c] = p.state[(first + src) * CHUNKS + my_c];
+            const int r = it * RPP + my_r;
+            src[it]     = -1;
+            v[it]       = make_uint4(0u, 0u, 0u, 0u);
+            if (my_r < RPP && r < nlive)
+            {
+                src[it] = s_list[wave][r];
+                v[it]   = p.state[(first + src[it]) * CHUNKS + my_c];
+            }
         }
+#pragma unroll
+        for (int it = 0; it < PASSES; ++it)
+            if (src[it] >= 0) s_rows[wave][src[it] * LS + my_c] = v[it];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
