@@ -107,7 +107,7 @@ def _point_grads(n, c, rng, dead_frac):
     return g
 
 
-@pytest.mark.parametrize("n,c", [(1000, 4), (70001, 3), (5003, 6), (3000, 8), (2000, 16), (63, 4), (1, 4)])
+@pytest.mark.parametrize("n,c", [(1000, 4), (70001, 3), (5003, 6), (3000, 8), (2000, 16), (63, 4), (1, 4), (6_000_000, 4)])
 def test_packed_point_adam_equals_per_tensor_adam(oracle, n, c):
     """MyAdamPoints (state packed per point, trips_adam_step_points) against MyAdam (trips_adam_step_fused) with
     different options per tensor, points without gradient, single elements without gradient, a step in which one of
@@ -142,9 +142,10 @@ def test_packed_point_adam_equals_per_tensor_adam(oracle, n, c):
                 ps[1].grad = None  # the sizes are not optimised in this step
         plain.step()
         packed.step()
-        for i in (0, 2, 3):  # (the sizes, with their AdaBound bounds and the step they sit out, are pinned by `plain`)
-            ref[i]["g"] = g[i].reshape(-1)
-        oracle.adam_step([ref[0], ref[2], ref[3]])
+        if n <= 100_000:  # (the scalar oracle: small sizes only; the per-tensor kernel is pinned by it at any size)
+            for i in (0, 2, 3):  # (the sizes, with their AdaBound bounds and the step they sit out, are pinned by `plain`)
+                ref[i]["g"] = g[i].reshape(-1)
+            oracle.adam_step([ref[0], ref[2], ref[3]])
     torch.cuda.synchronize()
     for a, b in zip(pa + [ea], pb + [eb]):
         assert torch.equal(a.data, b.data)
@@ -153,8 +154,9 @@ def test_packed_point_adam_equals_per_tensor_adam(oracle, n, c):
         for k in ("first_moments", "second_moments"):
             assert torch.equal(sa[k], sb[k]), k
         assert torch.equal(sa["param_steps"].to(torch.int32), sb["param_steps"])
-    for i in (0, 2, 3):
-        np.testing.assert_allclose(pb[i].detach().cpu().numpy().reshape(-1), ref[i]["w"], rtol=2e-6, atol=1e-7)
+    if n <= 100_000:
+        for i in (0, 2, 3):
+            np.testing.assert_allclose(pb[i].detach().cpu().numpy().reshape(-1), ref[i]["w"], rtol=2e-6, atol=1e-7)
     if n < 4:
         return
     # point removal / addition: the rows follow the group of the descriptors; one more step must agree again
