@@ -489,12 +489,13 @@ __global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, 
     const int local = r - g.off[layer];
     const int x = local % g.w[layer], y = local / g.w[layer];
     const int ip = pix_index(g, layer, x, y);
-    if (out_retained) out_retained[r] = retained[ip];
+    const int word = retained[ip];  // retained entries | filled list positions << 8
+    if (out_retained) out_retained[r] = word & 0xFF;
     if (out_lengths) out_lengths[r] = lengths[ip];
     if (out_lists)
         for (int k = 0; k < K; ++k)
         {
-            const int cid                = lists[(size_t)ip * K + k];  // compact number of the point, -1 = none
+            const int cid                = k < (word >> 8) ? lists[(size_t)ip * K + k] : -1;  // compact number of the point
             out_lists[(size_t)r * K + k] = cid >= 0 ? pid_of[cid] : -1;
         }
 }
@@ -510,27 +511,28 @@ hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists
     return hipGetLastError();
 }
 
-__global__ __launch_bounds__(256) void sum_i32_kernel(const int32_t* __restrict__ v, long long n,
+__global__ __launch_bounds__(256) void sum_i32_kernel(const int32_t* __restrict__ v, long long n, unsigned mask,
                                                       unsigned long long* out)
 {
     __shared__ unsigned long long s[4];
     unsigned long long acc = 0;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
-        acc += (unsigned long long)(unsigned)v[i];
+        acc += (unsigned long long)((unsigned)v[i] & mask);
     for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
     if ((threadIdx.x & 63) == 0) s[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0) atomicAdd(out, s[0] + s[1] + s[2] + s[3]);
 }
 
-hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream)
+// *out = sum of (v[i] & mask)
+hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned mask, unsigned long long* out, hipStream_t stream)
 {
     hipError_t e = hipMemsetAsync(out, 0, sizeof(unsigned long long), stream);
     if (e != hipSuccess) return e;
     if (n <= 0) return hipSuccess;
     int blocks = (int)((n + 255) / 256);
     if (blocks > 1024) blocks = 1024;
-    hipLaunchKernelGGL(sum_i32_kernel, dim3(blocks), dim3(256), 0, stream, v, n, out);
+    hipLaunchKernelGGL(sum_i32_kernel, dim3(blocks), dim3(256), 0, stream, v, n, mask, out);
     return hipGetLastError();
 }
 

@@ -959,7 +959,9 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     // saved state, also for padding pixels (empty) so that every row of the tables is defined
     if (TRAIN && in_range)
     {
-        if (sub == 0) __builtin_nontemporal_store(live ? ret : 0, p.retained + pix);
+        // (bits 0..7: retained entries; bits 8..15: list positions that hold an id. Only those are stored below: the
+        // backward reads the retained ones, the export fills the rest of a row with -1 itself.)
+        if (sub == 0) __builtin_nontemporal_store(live ? (ret | (n << 8)) : 0, p.retained + pix);
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
         // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
         if (has && sub < ret)
@@ -967,20 +969,19 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
         const int mine = has ? cid : -1;
         if (ROW == 4)
         {
-            // one 16-byte store per lane: lane 0 of the quad carries the four ids, the others the -1 padding
+            // one 16-byte store: lane 0 of the quad carries the four ids
             const int i0 = __shfl(mine, 0, 4), i1 = __shfl(mine, 1, 4), i2 = __shfl(mine, 2, 4), i3 = __shfl(mine, 3, 4);
-            if (4 * sub < K)
+            if (4 * sub < n)
                 __builtin_nontemporal_store(sub == 0 ? vi4{i0, i1, i2, i3} : vi4{-1, -1, -1, -1},
                                             reinterpret_cast<vi4*>(p.lists + (((size_t)(unsigned)pix << kshift) + 4 * sub)));
         }
         else if (ROW == 8)
         {
-            // one 8-byte store per lane covers the pixel's whole row (K <= 16 ids): lanes 0..3 carry the ids of lane
-            // pairs, the others the -1 padding
+            // 8-byte stores: lanes 0..3 carry the ids of lane pairs
             const int lo = __shfl(mine, (2 * sub) & 7, 8), hi = __shfl(mine, (2 * sub + 1) & 7, 8);
-            if (2 * sub < K) __builtin_nontemporal_store(sub < 4 ? (long long)(unsigned)lo | ((long long)hi << 32) : -1ll, reinterpret_cast<long long*>(p.lists + (((size_t)(unsigned)pix << kshift) + 2 * sub)));
+            if (2 * sub < n) __builtin_nontemporal_store(sub < 4 ? (long long)(unsigned)lo | ((long long)hi << 32) : -1ll, reinterpret_cast<long long*>(p.lists + (((size_t)(unsigned)pix << kshift) + 2 * sub)));
         }
-        else if (sub < K)
+        else if (sub < n)
             __builtin_nontemporal_store(mine, p.lists + (((size_t)(unsigned)pix << kshift) + sub));
     }
 }

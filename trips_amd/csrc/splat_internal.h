@@ -223,8 +223,8 @@ struct SavedLayout
     size_t header;    // ViewHeader
     size_t rec;       // float [N * record_floats]
     size_t prec;      // float [N * kPointRecordFloats]
-    size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded)
-    size_t retained;  // int32 [Pi]
+    size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded); a row's positions past its ids are undefined
+    size_t retained;  // int32 [Pi]: retained entries in bits 0..7, list positions that hold an id (min(length, K)) in bits 8..15
     size_t lengths;   // int32 [Pi]
     size_t rank;      // uint8 [2][N, 16] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none:
                       // plane 0 layers 0..3, plane 1 layers 4..7 (rows defined only for points written to those layers)

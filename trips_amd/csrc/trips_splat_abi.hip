@@ -22,7 +22,7 @@ hipError_t launch_adam_points(const TripsAdamTensor tensors[4], int num_points, 
 hipError_t launch_apply_tangent(double* tangent, double* poses, int n, hipStream_t stream);
 hipError_t launch_export_points(const float* rec, int rec_floats, const float* prec, const int32_t* cid_of, int n, float* ip,
                                 float* depth, float* size_px, int32_t* max_layer, hipStream_t stream);
-hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned long long* out, hipStream_t stream);
+hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned mask, unsigned long long* out, hipStream_t stream);
 hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
                                const int32_t* lengths, const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
                                int32_t* out_lengths, hipStream_t stream);
@@ -604,7 +604,8 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
     ViewHeader* hd       = reinterpret_cast<ViewHeader*>(sv + sl.header);
     const long long P    = g.off[desc->num_layers];
     const long long Pi   = (long long)g.bin_off[desc->num_layers] * kTilePixels;  // padding rows hold 0
-    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, &hd->retained, stream);
+    // (the low byte of a pixel's word: its retained entries)
+    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, 0xFFu, &hd->retained, stream);
     if (e != hipSuccess) return hip_fail(e, "retained sum");
     ViewHeader h;
     e = hipMemcpyAsync(&h, hd, sizeof(h), hipMemcpyDeviceToHost, stream);
