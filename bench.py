@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "3f2f6b6d5fe5cc827b6ba979c196612011cc1e279cf555c86afa3c011270ac6a"
+PMC_SOURCES_SHA256 = "4f9ba9c4ae3dea4d9f34617e4eaf2dac734509eaef31cedb51e55074becaf9a7"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129125, 302740),
-    "bin_scatter": (89130, 186621),
+    "project_bin": (129124, 302639),
+    "bin_scatter": (89121, 186689),
     "tile_count": (26193, 2296),
-    "tile_scatter": (69825, 114407),
-    "sort_blend": (332380, 450678),
-    "backward_pixels": (464772, 188403),
-    "backward_points": (1044970, 234887),
-    "adam_fused": (383854, 498420),
+    "tile_scatter": (69901, 114599),
+    "sort_blend": (332527, 366274),
+    "backward_pixels": (465296, 188116),
+    "backward_points": (1045299, 234887),
+    "adam_fused": (383865, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
