@@ -73,8 +73,11 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam
         "project_bin": 24 * N,                                    # position 16 + size 4 + index 4
         "tile_scatter": 8 * E,                                    # one 64-bit key written per entry
         "sort_blend": 8 * E + (20 + 4 + 4 * C + 28) * R + 4 * C * P,  # keys read, record+conf+descriptor, saved, image
-        "backward_pixels": 4 * C * P + (28 + 4 * C + 4 + 20) * R,  # dL/dimage, saved entry, descriptor+conf+record
-        "backward_points": (4 * C + 4 + 12 + 4) * R,              # one write per accumulated gradient float
+        # the backward's bytes split as its two passes split the work: the compositing (pixel pass) reads dL/dimage, the
+        # saved entry, descriptor and confidence; the geometry (point pass) reads position + size again (20 B per entry)
+        # and makes the one write per accumulated gradient float
+        "backward_pixels": 4 * C * P + (28 + 4 * C + 4) * R,
+        "backward_points": (20 + 4 * C + 4 + 12 + 4) * R,
         "adam_fused": (28 + 2 * adam_step_bytes) * adam_nonzero + 8 * adam_zero,
     }
 
