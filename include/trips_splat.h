@@ -186,7 +186,8 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
 
 /* Debug / parity export: writes for view `view` the sorted, depth-limited per-pixel point-id lists as a dense
  * [P,K] int32 array (-1 padded; all min(len,K) sorted entries), the per-pixel number of retained entries [P]
- * (those the blend kept, transmittance >= 0.001) and the per-pixel list length [P] (before the top-K cut).
+ * (those the blend kept, transmittance >= 0.001) and the per-pixel list length [P] (before the top-K cut; a length
+ * above 4 194 303 is reported as that number).
  * Pixels are numbered layer by layer, row-major inside a layer. Any of the three may be NULL. */
 int trips_splat_export_lists(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view,
                              int32_t* device_lists, int32_t* device_retained, int32_t* device_lengths, void* stream);

@@ -106,7 +106,7 @@ def test_size_queries_and_layer_sizes_host_only():
     assert lib.trips_splat_workspace_size(C.byref(d), C.byref(ws)) == 0
     assert lib.trips_splat_saved_size(C.byref(d), C.byref(sv)) == 0
     _, _, P = abi.pyramid_pixels(d)
-    assert ws.value >= 100 * 8 * (8 + 16) + 2 * P * 4  # worst case: a key and a bin entry per (point, layer) + counters
+    assert ws.value >= 100 * 8 * (8 + 8) + 2 * P * 4  # worst case: a key and a bin entry per (point, layer) + counters
     assert sv.value >= P * d.list_depth * 4 + 100 * 64
     # a capped list storage shrinks the forward's share of the workspace (eval mode has no backward share)
     ws1, ws2 = C.c_size_t(0), C.c_size_t(0)
@@ -114,7 +114,7 @@ def test_size_queries_and_layer_sizes_host_only():
     assert lib.trips_splat_workspace_size(C.byref(abi.desc_for_scene(sc_big, train=False)), C.byref(ws1)) == 0
     assert lib.trips_splat_workspace_size(C.byref(abi.desc_for_scene(sc_big, train=False, max_list_entries=1000)),
                                           C.byref(ws2)) == 0
-    assert ws2.value < ws1.value and ws1.value >= 100_000 * 8 * (8 + 16)
+    assert ws2.value < ws1.value and ws1.value >= 100_000 * 8 * (8 + 8)
     # two views double the saved state
     sc2 = scenes.tiny(n=100, w=64, h=48, num_layers=3, views=2)
     sc1 = scenes.tiny(n=100, w=64, h=48, num_layers=3, views=1)

@@ -326,6 +326,23 @@ def test_footprints_on_tile_and_image_borders_with_equal_depths(oracle):
     _check_backward(oracle, sc, d, seed=4)
 
 
+def test_more_than_2_to_the_23_points(oracle):
+    """Clouds above 2^23 points take the 16-byte form of the tile entries (the 8-byte form has 23 bits for a point's
+    number). Most points lie behind the camera; the visible ones sit at both ends of the cloud, enough of them at the
+    end that their numbers pass 2^23."""
+    n = (1 << 23) + 6000
+    sc = scenes.tiny(n=n, w=96, h=64, f=80.0, num_layers=4, list_depth=16, seed=23, radius=(0.004, 0.2))
+    sc.position[:, 2] = -10.0  # behind the camera, which looks along +z from z = -3
+    rng = np.random.default_rng(8)
+    for sl in (slice(0, 3000), slice(n - 40000, n)):
+        sc.position[sl, 2] = rng.uniform(-1, 1, sc.position[sl].shape[0]).astype(np.float32)
+    d = abi.desc_for_scene(sc)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    lists = ref["lists"][0]
+    assert lists.max() >= 1 << 23 and 0 <= lists[lists >= 0].min() < 3000
+    _check_backward(oracle, sc, d, seed=5)
+
+
 def test_config1_forward_full(oracle):
     sc = scenes.config1()
     _check_forward(oracle, sc, abi.desc_for_scene(sc, train=True))

@@ -477,7 +477,6 @@ hipError_t launch_export_points(const float* rec, int rec_floats, const float* p
 // saved tables are tile-major (padded); the exports are row-major, layer by layer
 __global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, int K, const int32_t* __restrict__ lists,
                                                            const int32_t* __restrict__ retained,
-                                                           const int32_t* __restrict__ lengths,
                                                            const int32_t* __restrict__ pid_of, int32_t* out_lists,
                                                            int32_t* out_retained, int32_t* out_lengths)
 {
@@ -489,25 +488,26 @@ __global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, 
     const int local = r - g.off[layer];
     const int x = local % g.w[layer], y = local / g.w[layer];
     const int ip = pix_index(g, layer, x, y);
-    const int word = retained[ip];  // retained entries | filled list positions << 8
-    if (out_retained) out_retained[r] = word & 0xFF;
-    if (out_lengths) out_lengths[r] = lengths[ip];
+    const unsigned word = (unsigned)retained[ip];  // retained entries | filled list positions << 5 | list length << 10
+    const int filled    = (int)((word >> kRetainedBits) & kRetainedMask);
+    if (out_retained) out_retained[r] = (int)(word & kRetainedMask);
+    if (out_lengths) out_lengths[r] = (int)(word >> (2 * kRetainedBits));
     if (out_lists)
         for (int k = 0; k < K; ++k)
         {
-            const int cid                = k < (word >> 8) ? lists[(size_t)ip * K + k] : -1;  // compact number of the point
+            const int cid                = k < filled ? lists[(size_t)ip * K + k] : -1;  // compact number of the point
             out_lists[(size_t)r * K + k] = cid >= 0 ? pid_of[cid] : -1;
         }
 }
 
 hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
-                               const int32_t* lengths, const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
+                               const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
                                int32_t* out_lengths, hipStream_t stream)
 {
     const int P = g.off[g.num_layers];
     if (P <= 0) return hipSuccess;
-    hipLaunchKernelGGL(export_lists_kernel, dim3((P + 255) / 256), dim3(256), 0, stream, g, K, lists, retained, lengths,
-                       pid_of, out_lists, out_retained, out_lengths);
+    hipLaunchKernelGGL(export_lists_kernel, dim3((P + 255) / 256), dim3(256), 0, stream, g, K, lists, retained, pid_of,
+                       out_lists, out_retained, out_lengths);
     return hipGetLastError();
 }
 

@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 8 
         const float* const gi = p.grad_image[tc.layer];
         // lane -> pixel (lane % 8) of this wavefront's group number lane / 8
         const int my_pix = lb * kQuarter + ((lane >> 3) * 4 + wave) * 8 + (lane & 7);
-        int m_all        = p.retained[my_pix] & 0xFF;  // (bits 8..15: filled list positions) 0 for the padding of partial tiles
+        int m_all        = p.retained[my_pix] & kRetainedMask;  // (low bits of the word) 0 for the padding of partial tiles
         int m_grp        = m_all;
         m_grp            = max(m_grp, __shfl_xor(m_grp, 1));
         m_grp            = max(m_grp, __shfl_xor(m_grp, 2));

@@ -457,11 +457,48 @@ __global__ __launch_bounds__(256) void bin_column_scan_kernel(int32_t* __restric
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// One bin entry {depth bits, compact point number, px | py << 16} per (point, layer), in the tile of (px, py). A workgroup walks
+// A bin entry holds what the list kernels need of a (point, layer) pair: the depth bits, the compact point number and
+// the cell of its tile that the footprint starts at. Depths of valid points are positive (31 bits), a cell takes 10
+// bits, so clouds of up to 2^23 points have entries of 8 bytes; larger ones use 16.
+template <bool PACKED>
+struct BinEntry;
+template <>
+struct BinEntry<true>
+{
+    using T = u64;
+    static __device__ __forceinline__ T make(unsigned zbits, unsigned cid, int px, int py)
+    {
+        const unsigned cell = (unsigned)((py & (kTile - 1)) << kTileShift) | (unsigned)(px & (kTile - 1));
+        return ((u64)zbits << (kPackedIdBits + 2 * kTileShift)) | ((u64)cid << (2 * kTileShift)) | cell;
+    }
+    static __device__ __forceinline__ int cell(const T& e) { return (int)((unsigned)e & (kTilePixels - 1)); }
+    static __device__ __forceinline__ u64 key(const T& e)
+    {
+        return ((e >> (kPackedIdBits + 2 * kTileShift)) << 32) | ((e >> (2 * kTileShift)) & ((1u << kPackedIdBits) - 1));
+    }
+};
+template <>
+struct BinEntry<false>
+{
+    using T = uint4;
+    static __device__ __forceinline__ T make(unsigned zbits, unsigned cid, int px, int py)
+    {
+        const unsigned cell = (unsigned)((py & (kTile - 1)) << kTileShift) | (unsigned)(px & (kTile - 1));
+        return make_uint4(zbits, cid, cell, 0u);
+    }
+    static __device__ __forceinline__ int cell(const T& e) { return (int)e.z; }
+    static __device__ __forceinline__ u64 key(const T& e) { return ((u64)e.x << 32) | (u64)e.y; }
+};
+static_assert(kTilePixels == 1 << (2 * kTileShift), "a cell number takes 2 kTileShift bits");
+
+// One bin entry per (point, layer), in the tile of the footprint's first pixel. A workgroup walks
 // the records that its chunk of the points left at the compact numbers; its slots inside every bin are contiguous
 // and start at bin_start[bin] + hist[workgroup][bin].
+template <bool PACKED>
 __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardParams p)
 {
+    using E = BinEntry<PACKED>;
+    typename E::T* __restrict__ entries = reinterpret_cast<typename E::T*>(p.bin_entries);
     extern __shared__ int s_cur[];
     const int NB       = p.geom.bin_off[p.num_layers];
     const int32_t* row = p.bin_hist + (size_t)blockIdx.x * NB;
@@ -502,7 +539,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
                             {
                                 const int slot = atomicAdd(bc, 1);
                                 if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
-                                    p.bin_entries[slot] = make_uint4(zbits, (unsigned)cid, (unsigned)px | ((unsigned)py << 16), 0u);
+                                    entries[slot] = E::make(zbits, (unsigned)cid, px, py);
                                 else
                                     dropped += 1;
                             });
@@ -512,19 +549,13 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Index, inside its tile, of the cell (px, py) that an entry's footprint starts at.
-__device__ __forceinline__ int entry_cell(const uint4& e)
-{
-    return (int)(((e.z >> 16) & (kTile - 1)) << kTileShift) | (int)(e.z & (kTile - 1));
-}
-
 // Walks entries [0, n) with the workgroup, four loads of a thread in flight together.
-template <int THREADS, typename F>
-__device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, int n, F&& f)
+template <int THREADS, typename T, typename F>
+__device__ __forceinline__ void for_entries(const T* __restrict__ entries, int n, F&& f)
 {
     for (int i0 = threadIdx.x; i0 < n; i0 += 4 * THREADS)
     {
-        uint4 e[4];
+        T e[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             if (i0 + THREADS * j < n) e[j] = entries[i0 + THREADS * j];
@@ -546,9 +577,11 @@ __device__ __forceinline__ void for_entries(const uint4* __restrict__ entries, i
 // (THREADS: 256 for the counting pass, whose idle workgroups for unused slices are cheaper that way; 1024 for the
 // placement pass, where two workgroups per CU with their 64 KB of LDS then make 32 wavefronts instead of 8)
 constexpr int kScatterThreads = 1024;
-template <bool SCATTER, int THREADS>
+template <bool SCATTER, int THREADS, bool PACKED>
 __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams p)
 {
+    using E  = BinEntry<PACKED>;
+    using ET = typename E::T;
     __shared__ int s_cnt[kTilePixels];
     // per-cell entries of a slice (placement pass only; one word in the counting pass, whose code below never runs)
     __shared__ int s_mine[SCATTER ? kTilePixels : 1];
@@ -584,7 +617,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         last = min(last, first + kSliceEntries);
     }
     const int n          = first < last ? (int)(last - first) : 0;
-    const uint4* entries = p.bin_entries + first;
+    const ET* entries    = reinterpret_cast<const ET*>(p.bin_entries) + first;
     int32_t* counts      = p.counts + (size_t)bin * kTilePixels;
 
     if (!SCATTER)
@@ -592,7 +625,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         if (slice < 0) return;  // the slices count for a split tile; any other tile is counted where its keys are placed
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
-        for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&s_cnt[entry_cell(e)], 1); });
+        for_entries<THREADS>(entries, n, [&](const ET& e) { atomicAdd(&s_cnt[E::cell(e)], 1); });
         __syncthreads();
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
@@ -611,7 +644,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         // count here (the entries come from the L2 when they are read again for the placement)
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
-        for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&s_cnt[entry_cell(e)], 1); });
+        for_entries<THREADS>(entries, n, [&](const ET& e) { atomicAdd(&s_cnt[E::cell(e)], 1); });
         __syncthreads();
     }
 #pragma unroll
@@ -668,7 +701,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     {
         // this slice's share of every cell's list: count, then claim the slots with one atomic per cell
         int32_t* run = p.run + (size_t)bin * kTilePixels;
-        for_entries<THREADS>(entries, n, [&](const uint4& e) { atomicAdd(&mine(entry_cell(e)), 1); });
+        for_entries<THREADS>(entries, n, [&](const ET& e) { atomicAdd(&mine(E::cell(e)), 1); });
         __syncthreads();
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
@@ -677,10 +710,10 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         }
         __syncthreads();
         for_entries<THREADS>(entries, n,
-                    [&](const uint4& e)
+                    [&](const ET& e)
                     {
-                        const u64 key  = ((u64)e.x << 32) | (u64)e.y;
-                        const int slot = atomicAdd(&s_cnt[entry_cell(e)], 1);
+                        const u64 key  = E::key(e);
+                        const int slot = atomicAdd(&s_cnt[E::cell(e)], 1);
                         if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
                             p.keys[slot] = key;
                         else
@@ -695,10 +728,10 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     const int tile_total = p.bin_start[bin + 1] - key_start;
     const bool staged    = tile_total <= kStageKeys && (long long)key_start + tile_total <= p.capacity;
     for_entries<THREADS>(entries, n,
-                [&](const uint4& e)
+                [&](const ET& e)
                 {
-                    const u64 key  = ((u64)e.x << 32) | (u64)e.y;
-                    const int slot = atomicAdd(&s_cnt[entry_cell(e)], 1);
+                    const u64 key  = E::key(e);
+                    const int slot = atomicAdd(&s_cnt[E::cell(e)], 1);
                     if (staged)
                         s_keys[slot - key_start] = key;
                     else if ((unsigned long long)(unsigned)slot < (unsigned long long)p.capacity)
@@ -819,6 +852,7 @@ struct PixelCells
 {
     int s0, s1, s2, s3;
     int r0, r1, r2, r3;
+    int length;  // entries of the four lists (more than the readable keys when a list is long or was cut by the capacity)
 };
 
 template <int C, bool TRAIN, int ROW>
@@ -959,9 +993,14 @@ __device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const Ti
     // saved state, also for padding pixels (empty) so that every row of the tables is defined
     if (TRAIN && in_range)
     {
-        // (bits 0..7: retained entries; bits 8..15: list positions that hold an id. Only those are stored below: the
-        // backward reads the retained ones, the export fills the rest of a row with -1 itself.)
-        if (sub == 0) __builtin_nontemporal_store(live ? (ret | (n << 8)) : 0, p.retained + pix);
+        // (bits 0..4: retained entries; bits 5..9: list positions that hold an id. Only those are stored below: the
+        // backward reads the retained ones, the export fills the rest of a row with -1 itself. Bits 10..31: length of
+        // the pixel's list before the cut to K, for the export; saturates.)
+        if (sub == 0)
+            __builtin_nontemporal_store(live ? (int)((unsigned)ret | ((unsigned)n << kRetainedBits) |
+                                                     ((unsigned)min(cells.length, kMaxExportedLength) << (2 * kRetainedBits)))
+                                             : 0,
+                                        p.retained + pix);
         // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
         // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
         if (has && sub < ret)
@@ -1030,12 +1069,8 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
     }
     // lane j < 16: readable keys of pixel j of the run
     int tot = c_read + __shfl_down(c_read, 1) + __shfl_down(c_read, 17) + __shfl_down(c_read, 18);
-    if (TRAIN)
-    {
-        const int len = c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 17) + __shfl_down(c_len, 18);
-        // (this wavefront's eight pixels; 0 for the padding of partial tiles)
-        if ((lane >> 3) == half && group_in_range) __builtin_nontemporal_store(len, p.lengths + (pair_first + lane));
-    }
+    // lane j < 16: entries of pixel j's lists (0 for the padding of partial tiles)
+    const int len = TRAIN ? c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 17) + __shfl_down(c_len, 18) : 0;
     if (lane >= 16) tot = 0;
     tot = max(tot, __shfl_xor(tot, 1));
     tot = max(tot, __shfl_xor(tot, 2));
@@ -1048,6 +1083,7 @@ __global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
         PixelCells c;
         c.s0 = __shfl(c_start, j), c.s1 = __shfl(c_start, j + 1), c.s2 = __shfl(c_start, j + 17), c.s3 = __shfl(c_start, j + 18);
         c.r0 = __shfl(c_read, j), c.r1 = __shfl(c_read, j + 1), c.r2 = __shfl(c_read, j + 17), c.r3 = __shfl(c_read, j + 18);
+        c.length = TRAIN ? __shfl(len, j) : 0;
         return c;
     };
     if (tot16 <= 4)
@@ -1084,6 +1120,8 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
 
     const int G           = p.bin_groups;
     const size_t lds_hist = (size_t)NB * sizeof(int);
+    // compact point numbers are below num_points: entries of 8 bytes when they fit kPackedIdBits bits
+    const bool packed = p.num_points <= (1 << kPackedIdBits);
     {
         ProfScope ps(prof, "project_bin", stream);
         if (train)
@@ -1106,23 +1144,34 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     }
     {
         ProfScope ps(prof, "bin_scatter", stream);
-        hipLaunchKernelGGL(bin_scatter_kernel, dim3(G), dim3(kBinThreads), lds_hist, stream, p);
+        if (packed)
+            hipLaunchKernelGGL(bin_scatter_kernel<true>, dim3(G), dim3(kBinThreads), lds_hist, stream, p);
+        else
+            hipLaunchKernelGGL(bin_scatter_kernel<false>, dim3(G), dim3(kBinThreads), lds_hist, stream, p);
     }
     // workgroups for the slices of split tiles: at most capacity / kSliceEntries full slices plus one partial slice
     // per split tile
     const int max_slices = (int)std::min<long long>(2 * (p.capacity / kSliceEntries) + 1, 1 << 20);
     {
         ProfScope ps(prof, "tile_count", stream);
-        hipLaunchKernelGGL((tile_lists_kernel<false, 256>), dim3(NB + max_slices), dim3(256), 0, stream, p);
+        if (packed)
+            hipLaunchKernelGGL((tile_lists_kernel<false, 256, true>), dim3(NB + max_slices), dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((tile_lists_kernel<false, 256, false>), dim3(NB + max_slices), dim3(256), 0, stream, p);
     }
     {
         ProfScope ps(prof, "tile_scatter", stream);
         // (64 KB of LDS with the static tables: above the default limit of a launch)
-        const hipError_t lds = hipFuncSetAttribute(reinterpret_cast<const void*>(&tile_lists_kernel<true, kScatterThreads>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kStageKeys * sizeof(u64)));
+        const void* fn = packed ? reinterpret_cast<const void*>(&tile_lists_kernel<true, kScatterThreads, true>)
+                                : reinterpret_cast<const void*>(&tile_lists_kernel<true, kScatterThreads, false>);
+        const hipError_t lds = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kStageKeys * sizeof(u64)));
         if (lds != hipSuccess) return lds;
-        hipLaunchKernelGGL((tile_lists_kernel<true, kScatterThreads>), dim3(NB + max_slices), dim3(kScatterThreads), kStageKeys * sizeof(u64), stream,
-                           p);
+        if (packed)
+            hipLaunchKernelGGL((tile_lists_kernel<true, kScatterThreads, true>), dim3(NB + max_slices), dim3(kScatterThreads),
+                               kStageKeys * sizeof(u64), stream, p);
+        else
+            hipLaunchKernelGGL((tile_lists_kernel<true, kScatterThreads, false>), dim3(NB + max_slices), dim3(kScatterThreads),
+                               kStageKeys * sizeof(u64), stream, p);
     }
     {
         ProfScope ps(prof, "long_lists", stream);

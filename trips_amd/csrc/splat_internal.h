@@ -113,6 +113,10 @@ constexpr int kTile       = 1 << kTileShift;
 constexpr int kTilePixels = kTile * kTile;
 // (One workgroup of 1024 threads per CU: three of 512, with the projection kernel held to 80 registers, measured 1 %
 // slower over the step: the histogram matrix grows with the number of workgroups.)
+constexpr int kPackedIdBits = 23;  // clouds of up to 2^23 points have bin entries of 8 bytes (31 depth bits, id, 10 cell bits)
+// a pixel's word of the saved state: retained entries | list positions that hold an id << 5 | list length << 10
+constexpr int kRetainedBits = 5, kRetainedMask = (1 << kRetainedBits) - 1;
+constexpr int kMaxExportedLength = (1 << (32 - 2 * kRetainedBits)) - 1;  // longer lists are exported as this length
 constexpr int kBinThreads = 1024;   // workgroup size of the two binning kernels
 constexpr int kBinGroups  = 256;    // workgroups (= contiguous chunks of points) of the two binning kernels
 constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning kernels (60 KB)
@@ -224,8 +228,7 @@ struct SavedLayout
     size_t rec;       // float [N * record_floats]
     size_t prec;      // float [N * kPointRecordFloats]
     size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded); a row's positions past its ids are undefined
-    size_t retained;  // int32 [Pi]: retained entries in bits 0..7, list positions that hold an id (min(length, K)) in bits 8..15
-    size_t lengths;   // int32 [Pi]
+    size_t retained;  // int32 [Pi]: retained entries in bits 0..4, list positions that hold an id (min(length, K)) in bits 5..9, list length from bit 10
     size_t rank;      // uint8 [2][N, 16] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none:
                       // plane 0 layers 0..3, plane 1 layers 4..7 (rows defined only for points written to those layers)
     size_t cid_of;    // int32 [N] compact number of every point (-1 = culled)
@@ -262,7 +265,7 @@ struct WorkspaceLayout
     size_t bin_count;    // int32 [NB]   bin entries per tile
     size_t bin_start;    // int32 [NB+1] exclusive scan of bin_count
     size_t bin_hist;     // int32 [G, NB] bin entries per (workgroup, tile), then its column-wise exclusive prefix
-    size_t bin_entries;  // uint4 [capacity] {depth bits, compact point number, px | py << 16, -}, one per (point, layer), by tile
+    size_t bin_entries;  // [capacity] {depth bits, compact point number, cell}, one per (point, layer), by tile: 8 bytes each for up to 2^23 points, else 16
     size_t keys;         // uint64 [capacity] depth bits << 32 | compact point number, by cell
     size_t capacity;     // (point, layer) pairs
     size_t bytes;
@@ -307,7 +310,7 @@ struct ForwardParams
     int2* long_items;
     unsigned long long* cand;
     int32_t max_long_items;
-    uint4* bin_entries;
+    void* bin_entries;
     unsigned long long* keys;
     long long capacity;
     float* rec;
@@ -315,7 +318,6 @@ struct ForwardParams
     int32_t rec_floats;
     int32_t* lists;
     int32_t* retained;
-    int32_t* lengths;
     unsigned char* rank;  // training only
     ViewHeader* header;  // counters of this view
     ViewHeader* status;  // overflow flag of the whole forward call (start of the workspace)

@@ -24,7 +24,7 @@ hipError_t launch_export_points(const float* rec, int rec_floats, const float* p
                                 float* depth, float* size_px, int32_t* max_layer, hipStream_t stream);
 hipError_t launch_sum_i32(const int32_t* v, long long n, unsigned mask, unsigned long long* out, hipStream_t stream);
 hipError_t launch_export_lists(const PyramidGeom& g, int K, const int32_t* lists, const int32_t* retained,
-                               const int32_t* lengths, const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
+                               const int32_t* pid_of, int32_t* out_lists, int32_t* out_retained,
                                int32_t* out_lengths, hipStream_t stream);
 }  // namespace trips
 
@@ -210,8 +210,6 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(P * K * sizeof(int32_t));
     s.retained = o;
     o += align256(P * sizeof(int32_t));
-    s.lengths = o;
-    o += align256(P * sizeof(int32_t));
     s.rank = o;
     o += align256(N * 32);
     s.cid_of = o;
@@ -261,7 +259,7 @@ WorkspaceLayout workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     w.bin_hist = o;
     o += align256((size_t)kBinGroups * NB * sizeof(int32_t));
     w.bin_entries = o;
-    o += align256(w.capacity * sizeof(uint4));
+    o += align256(w.capacity * (N <= ((size_t)1 << kPackedIdBits) ? sizeof(unsigned long long) : sizeof(uint4)));
     w.keys = o;
     o += align256(w.capacity * sizeof(unsigned long long));
     w.bytes = o;
@@ -435,7 +433,7 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
         p.long_items  = reinterpret_cast<int2*>(ws + wl.long_items);
         p.cand        = reinterpret_cast<unsigned long long*>(ws + wl.cand);
         p.max_long_items = (int32_t)wl.max_long_items;
-        p.bin_entries   = reinterpret_cast<uint4*>(ws + wl.bin_entries);
+        p.bin_entries   = ws + wl.bin_entries;
         p.keys       = reinterpret_cast<unsigned long long*>(ws + wl.keys);
         p.capacity   = (long long)wl.capacity;
         if (train)
@@ -447,7 +445,6 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
             p.rec_floats = record_floats(d.num_channels);
             p.lists      = reinterpret_cast<int32_t*>(sv + sl.lists);
             p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
-            p.lengths    = reinterpret_cast<int32_t*>(sv + sl.lengths);
             p.rank       = reinterpret_cast<unsigned char*>(sv + sl.rank);
             p.cid_of     = reinterpret_cast<int32_t*>(sv + sl.cid_of);
             p.pid_of     = reinterpret_cast<int32_t*>(sv + sl.pid_of);
@@ -604,8 +601,8 @@ int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* 
     ViewHeader* hd       = reinterpret_cast<ViewHeader*>(sv + sl.header);
     const long long P    = g.off[desc->num_layers];
     const long long Pi   = (long long)g.bin_off[desc->num_layers] * kTilePixels;  // padding rows hold 0
-    // (the low byte of a pixel's word: its retained entries)
-    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, 0xFFu, &hd->retained, stream);
+    // (the low bits of a pixel's word: its retained entries)
+    hipError_t e = launch_sum_i32(reinterpret_cast<const int32_t*>(sv + sl.retained), Pi, (unsigned)kRetainedMask, &hd->retained, stream);
     if (e != hipSuccess) return hip_fail(e, "retained sum");
     ViewHeader h;
     e = hipMemcpyAsync(&h, hd, sizeof(h), hipMemcpyDeviceToHost, stream);
@@ -633,7 +630,6 @@ int trips_splat_export_lists(TripsCtx* ctx, const TripsSplatDesc* desc, const vo
     const char* sv       = reinterpret_cast<const char*>(saved) + sl.bytes_per_view * (size_t)view;
     hipError_t e = launch_export_lists(g, desc->list_depth, reinterpret_cast<const int32_t*>(sv + sl.lists),
                                        reinterpret_cast<const int32_t*>(sv + sl.retained),
-                                       reinterpret_cast<const int32_t*>(sv + sl.lengths),
                                        reinterpret_cast<const int32_t*>(sv + sl.pid_of), device_lists, device_retained,
                                        device_lengths, stream);
     if (e != hipSuccess) return hip_fail(e, "export copy");
