@@ -69,6 +69,7 @@ struct PointProjection
     int tex;        // descriptor column
     int layers;     // layers the point is written to (0 if culled)
     float ipx, ipy, z, size_px;
+    float d_softplus;  // softplus'(raw size), training mode
 };
 
 // What the projection reads of a point in point order (fetched one step ahead of its use).
@@ -100,6 +101,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
     o.ipx = o.ipy = 0.f;
     o.z       = -1.f;
     o.size_px = 0.f;
+    o.d_softplus = 0.f;
     const int L = p.num_layers;
     bool skip   = false;
     o.tex       = in.tex;
@@ -129,7 +131,8 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
         pos.y += dsp[1];
         pos.z += dsp[2];
     }
-    const float size    = softplus(in.raw_size);
+    float d_softplus    = 0.f;
+    const float size    = TRAIN ? softplus_and_derivative(in.raw_size, &d_softplus) : softplus(in.raw_size);
     const Projected pr  = project(cam, pos.x, pos.y, pos.z);
     const float z       = pr.z;
     float radius_px     = pr.scale * pos.w / z;
@@ -164,6 +167,7 @@ __device__ __forceinline__ PointProjection project_point(const ForwardParams& p,
     o.ipy     = pr.ipy;
     o.z       = z;
     o.size_px = size_px;
+    o.d_softplus = d_softplus;
     return o;
 }
 
@@ -266,7 +270,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
 #pragma unroll
         for (int q = 0; q < NREC; ++q) __builtin_nontemporal_store(vf4{recv[q].x, recv[q].y, recv[q].z, recv[q].w}, reinterpret_cast<vf4*>(rec) + q);
         // point record: depth and layers for the scatter pass; softplus' and the size for the backward
-        __builtin_nontemporal_store(vf4{TRAIN ? softplus_backward(in.raw_size) : 0.f, o.z, __int_as_float(o.layers), o.size_px},
+        __builtin_nontemporal_store(vf4{TRAIN ? o.d_softplus : 0.f, o.z, __int_as_float(o.layers), o.size_px},
                                     reinterpret_cast<vf4*>(p.prec) + cid);
         if (TRAIN)
         {

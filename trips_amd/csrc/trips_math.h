@@ -35,6 +35,19 @@ __device__ __forceinline__ float softplus_backward(float y)
     return z / (z + 1.f);
 }
 
+// both at once, with the one exponential that they share (same bits as the two functions above)
+__device__ __forceinline__ float softplus_and_derivative(float x, float* derivative)
+{
+    if (x > 20.f)
+    {
+        *derivative = 1.f;
+        return x;
+    }
+    const float z = exp_rn(x);
+    *derivative   = z / (z + 1.f);
+    return log_rn(1.f + z);
+}
+
 // floor(log2 s), ceil(log2 s) for finite s > 0 from the bit pattern (exact; the reference rounds log2f first)
 __device__ __forceinline__ void log2_floor_ceil(float s, int& lo, int& hi)
 {
