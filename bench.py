@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "4f9ba9c4ae3dea4d9f34617e4eaf2dac734509eaef31cedb51e55074becaf9a7"
+PMC_SOURCES_SHA256 = "e2fa78f619d5204072c0a9d0873ae4dcfdd92584e1ec321e68804d7f0fe3913c"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129124, 302639),
-    "bin_scatter": (89121, 186689),
-    "tile_count": (26193, 2296),
-    "tile_scatter": (69901, 114599),
-    "sort_blend": (332527, 366274),
-    "backward_pixels": (465296, 188116),
-    "backward_points": (1045299, 234887),
-    "adam_fused": (383865, 498420),
+    "project_bin": (129123, 299639),
+    "bin_scatter": (88884, 152706),
+    "tile_count": (13139, 2296),
+    "tile_scatter": (32620, 110293),
+    "sort_blend": (332127, 350809),
+    "backward_pixels": (465002, 187842),
+    "backward_points": (1045008, 234887),
+    "adam_fused": (383885, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
