@@ -42,6 +42,11 @@ typedef struct TripsUnetDesc {
     int32_t filters[TRIPS_UNET_MAX_LEVELS];  /* F[0..L-1] (filters_network); conv outputs must be >= 1 and <= 64 */
     int32_t level_w[TRIPS_UNET_MAX_LEVELS];  /* size of in[i]; level i+1 must be ceil or floor of half of level i */
     int32_t level_h[TRIPS_UNET_MAX_LEVELS];
+    int32_t weights_packed;       /* trips_unet_forward only. Nonzero: `workspace` still holds the fp16 weights that an
+                                     earlier forward with the same desc and the same weight values packed there, and
+                                     nothing has written to it since except such forwards (a viewer's frames: the weights
+                                     change when a checkpoint is loaded, not per frame); the call skips the packing.
+                                     0: the weights are packed by this call (training: they change every step). */
 } TripsUnetDesc;
 
 /* Weights in the reference's tensor layouts (torch::nn::Conv2d): weight [Cout, Cin, 3, 3] and bias [Cout], fp32,

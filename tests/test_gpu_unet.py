@@ -68,6 +68,49 @@ def test_unet_forward_three_input_channels():
     _compare(net, inputs)
 
 
+def test_unet_packed_weights_are_reused_on_request():
+    """A viewer's frames: with reuse_packed_weights the fp16 weights are packed by the first no-grad forward only
+    (TripsUnetDesc.weights_packed); the later frames give the same bits, and a changed weight takes effect after
+    invalidate_packed_weights()."""
+    from trips_amd.renderer import get_context
+    net = _net([16, 32, 64, 64], 4, seed=3).cuda()
+    inputs = [t.cuda() for t in _pyramid(96, 72, 4, 4, batch=1, seed=4)]
+    ctx = get_context(0)
+    with torch.no_grad():
+        ctx.profile_enable(True)
+        ctx.profile_read()
+        first = net.forward(inputs).clone()  # packs
+        names_first = set(ctx.profile_read())
+        net.reuse_packed_weights = True
+        a = net.forward(inputs).clone()      # reuses what the call before left in the workspace
+        names_a = set(ctx.profile_read())
+        b = net.forward(inputs).clone()
+        names_b = set(ctx.profile_read())
+        assert "unet_pack_weights" in names_first and "unet_conv_l0" in names_b
+        assert "unet_pack_weights" not in names_a and "unet_pack_weights" not in names_b
+        assert torch.equal(first, a) and torch.equal(a, b)
+        other = [t * 0.5 for t in inputs]
+        assert torch.equal(net.forward(other), _fresh_forward(net, other))  # other inputs, same weights: still reused
+        net.final_conv.bias.add_(1.0)
+        net.block(1).feature_conv.weight.mul_(2.0)
+        net.invalidate_packed_weights()
+        c = net.forward(inputs).clone()
+        names_c = set(ctx.profile_read())
+        ctx.profile_enable(False)
+        assert "unet_pack_weights" in names_c
+        assert not torch.equal(c, a) and torch.equal(c, _fresh_forward(net, inputs))
+
+
+def _fresh_forward(net, inputs):
+    """The same forward with the packing done by the call itself."""
+    keep, net.reuse_packed_weights = net.reuse_packed_weights, False
+    try:
+        return net.forward(inputs).clone()
+    finally:
+        net.reuse_packed_weights = keep
+        net.invalidate_packed_weights()
+
+
 def test_unet_extra_input_layers_are_ignored():
     # the splat renders 8 layers, the net may consume fewer (num_input_layers > num_layers)
     from trips_amd.unet import MultiScaleUnet2dDecOnlySmallFixed, MultiScaleUnet2dParams

@@ -135,6 +135,7 @@ class TripsUnetDesc(C.Structure):
         ("filters", C.c_int32 * TRIPS_UNET_MAX_LEVELS),
         ("level_w", C.c_int32 * TRIPS_UNET_MAX_LEVELS),
         ("level_h", C.c_int32 * TRIPS_UNET_MAX_LEVELS),
+        ("weights_packed", C.c_int32),
     ]
 
 

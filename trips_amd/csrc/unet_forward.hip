@@ -506,6 +506,7 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
         return reinterpret_cast<_Float16*>(base) + (size_t)b * l.H * l.W * l.cout_store;
     };
 
+    if (!d.weights_packed)
     {
         ProfScope ps(prof, "unet_pack_weights", stream);
         PackTable pt;

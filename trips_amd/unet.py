@@ -110,6 +110,14 @@ class MultiScaleUnet2dDecOnlySmallFixed(torch.nn.Module):
             self.add_module(f"up{i + 1}", UpsampleDecOnlySmallBlockFixed(F[i + 1], out))
         self.final = torch.nn.Sequential(torch.nn.Conv2d(F[0], p.num_output_channels, 1), torch.nn.Identity())
         self._buffers_dev = {}
+        # A viewer sets this: the weights then count as unchanged from one no-grad forward to the next (they are packed
+        # to fp16 once, not per frame). Whoever changes them in place afterwards (load_state_dict, an optimiser step)
+        # calls invalidate_packed_weights().
+        self.reuse_packed_weights = False
+        self._packed_key = None
+
+    def invalidate_packed_weights(self):
+        self._packed_key = None
 
     def block(self, i):
         """Gated block of pyramid level i (the start block's for the coarsest level)."""
@@ -183,6 +191,12 @@ class MultiScaleUnet2dDecOnlySmallFixed(torch.nn.Module):
         w = self._weights_struct(params)
         nbytes = self._size("trips_unet_workspace_size", ins)
         ws = self._alloc("forward", nbytes, dev)
+        # the packed weights in the workspace stay valid while the weights do (reuse_packed_weights), for the same
+        # buffer and level sizes
+        key = (ws.data_ptr(), bytes(d), tuple(q.data_ptr() for q in params))
+        if self.reuse_packed_weights and saved is None and self._packed_key == key:
+            d.weights_packed = 1
+        self._packed_key = key if saved is None else None
         out = torch.empty((d.batch, d.num_output_channels, d.level_h[0], d.level_w[0]), dtype=torch.float32, device=dev)
         _lib.check(ctx.lib.trips_unet_forward(ctx.ctx, C.byref(d), C.byref(w), self._input_ptrs(ins), _ptr(out),
                                               _ptr(saved), _ptr(ws), nbytes, _stream_ptr(dev)))
