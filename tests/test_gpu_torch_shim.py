@@ -180,6 +180,19 @@ def test_cpp_unet_forward_backward_matches_python_mirror():
         assert cpp_params[n].grad is not None, n
         # bias and 1x1 gradients are summed with float atomics: same values up to summation order
         assert torch.allclose(cpp_params[n].grad, q.grad, rtol=1e-4, atol=1e-7 * float(q.grad.abs().max())), n
+    # without gradients nothing is kept for a backward; a viewer's frames reuse the packed weights on request
+    plain = [t.cuda() for t in ins]
+    frame = cpp.forward_no_grad(plain)
+    assert torch.equal(frame, out_cpp.detach())
+    cpp.set_reuse_packed_weights(True)
+    assert torch.equal(cpp.forward_no_grad(plain), frame) and torch.equal(cpp.forward_no_grad(plain), frame)
+    name = next(n for n, _ in py.named_parameters() if n.endswith("feature_transform.0.weight"))
+    with torch.no_grad():
+        cpp_params[name].mul_(1.5)
+        dict(py.named_parameters())[name].mul_(1.5)
+        cpp.invalidate_packed_weights()
+        changed = cpp.forward_no_grad(plain)
+        assert not torch.equal(changed, frame) and torch.equal(changed, py.forward(plain))
 
 
 @pytest.mark.gpu

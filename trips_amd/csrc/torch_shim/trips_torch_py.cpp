@@ -107,6 +107,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         .def("named_parameters", &UnetSession::named_parameters)
         .def("cuda", [](UnetSession& s) { s.net->to(torch::kCUDA); })
         .def("forward", [](UnetSession& s, std::vector<torch::Tensor> inputs) { return s.net->forward(inputs); })
+        .def("forward_no_grad",
+             [](UnetSession& s, std::vector<torch::Tensor> inputs)
+             {
+                 torch::NoGradGuard guard;
+                 return s.net->forward(inputs);
+             })
+        .def("set_reuse_packed_weights", [](UnetSession& s, bool on) { s.net->reuse_packed_weights = on; })
+        .def("invalidate_packed_weights", [](UnetSession& s) { s.net->invalidate_packed_weights(); })
         .def("save", [](UnetSession& s, const std::string& file) { torch::save(s.net, file); })
         .def("load", [](UnetSession& s, const std::string& file) { torch::load(s.net, file); });
 

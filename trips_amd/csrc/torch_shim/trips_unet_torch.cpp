@@ -213,6 +213,42 @@ at::Tensor MultiScaleUnet2dDecOnlySmallFixedImpl::forward(std::vector<torch::Ten
                     "trips: inputs[", i, "] must be float32 [B, ", params.num_input_channels, ", H, W]");
         tensors.push_back(inputs[i]);
     }
-    for (auto& p : ordered_parameters()) tensors.push_back(p);
+    bool needs_grad = false;
+    for (auto& p : ordered_parameters())
+    {
+        tensors.push_back(p);
+        needs_grad |= p.requires_grad();
+    }
+    for (int i = 0; i < L; ++i) needs_grad |= inputs[i].requires_grad();
+    if (!torch::GradMode::is_enabled() || !needs_grad)
+        return forward_without_grad(std::vector<torch::Tensor>(tensors.begin(), tensors.begin() + L),
+                                    std::vector<torch::Tensor>(tensors.begin() + L, tensors.end()));
+    packed_key.clear();  // (the training forward packs into the same workspace, and the weights are about to change)
     return UnetFunction::apply(reinterpret_cast<int64_t>(this), at::TensorList(tensors))[0];
+}
+
+// Nothing is kept for a backward: the block outputs live in the workspace.
+at::Tensor MultiScaleUnet2dDecOnlySmallFixedImpl::forward_without_grad(std::vector<torch::Tensor> ins, std::vector<torch::Tensor> prm)
+{
+    const int L = params.num_layers;
+    for (auto& t : ins) t = t.detach().contiguous();
+    for (auto& t : prm) t = t.detach().to(ins[0].device(), torch::kFloat32).contiguous();
+    TripsUnetDesc d          = desc(ins);
+    const TripsUnetWeights w = weights_struct(L, prm);
+    size_t ws = 0;
+    check(trips_unet_workspace_size(&d, &ws), "trips_unet_workspace_size");
+    if (!forward_workspace.defined() || (size_t)forward_workspace.numel() < ws || forward_workspace.device() != ins[0].device())
+        forward_workspace = bytes_on(ins[0], ws);
+    std::vector<uint64_t> key{(uint64_t)reinterpret_cast<uintptr_t>(forward_workspace.data_ptr()), (uint64_t)d.batch};
+    for (int i = 0; i < L; ++i) key.push_back(((uint64_t)d.level_w[i] << 32) | (uint64_t)d.level_h[i]);
+    for (auto& t : prm) key.push_back((uint64_t)reinterpret_cast<uintptr_t>(t.data_ptr()));
+    if (reuse_packed_weights && key == packed_key) d.weights_packed = 1;
+    packed_key = key;
+    torch::Tensor out = torch::empty({d.batch, d.num_output_channels, d.level_h[0], d.level_w[0]}, ins[0].options());
+    const float* in_ptrs[TRIPS_UNET_MAX_LEVELS] = {};
+    for (int i = 0; i < L; ++i) in_ptrs[i] = ins[i].data_ptr<float>();
+    check(trips_unet_forward(unet_context(ins[0]), &d, &w, in_ptrs, out.data_ptr<float>(), /*saved*/ nullptr,
+                             forward_workspace.data_ptr(), (size_t)forward_workspace.numel(), stream_of(ins[0])),
+          "trips_unet_forward");
+    return out;
 }

@@ -79,5 +79,15 @@ class MultiScaleUnet2dDecOnlySmallFixedImpl : public torch::nn::Module
     SmallDecStartBlock start = nullptr;
     UpsampleDecOnlySmallBlockFixed up[TRIPS_UNET_MAX_LEVELS - 1] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     torch::Tensor forward_workspace, backward_workspace;
+
+    // A viewer sets this: the weights then count as unchanged from one forward without gradients to the next (they
+    // are packed to fp16 once, not per frame). Whoever changes them in place afterwards (load, an optimiser step)
+    // calls invalidate_packed_weights().
+    bool reuse_packed_weights = false;
+    void invalidate_packed_weights() { packed_key.clear(); }
+
+   private:
+    at::Tensor forward_without_grad(std::vector<torch::Tensor> ins, std::vector<torch::Tensor> prm);
+    std::vector<uint64_t> packed_key;  // workspace, level sizes and weight pointers of the last packing
 };
 TORCH_MODULE(MultiScaleUnet2dDecOnlySmallFixed);
