@@ -121,6 +121,21 @@ def test_random_shapes_forward_backward(oracle, seed):
     _check_backward(oracle, sc, d, seed=seed)
 
 
+@pytest.mark.parametrize("channels,K,layout,views", [(3, 16, abi.TRIPS_LAYOUT_HWC, 1), (6, 8, abi.TRIPS_LAYOUT_CHW, 2),
+                                                     (8, 16, abi.TRIPS_LAYOUT_CHW, 1), (16, 8, abi.TRIPS_LAYOUT_HWC, 2),
+                                                     (16, 16, abi.TRIPS_LAYOUT_CHW, 1)])
+def test_medium_views_other_channel_counts(oracle, channels, K, layout, views):
+    """300 000 points on 640 x 480 and 8 layers (hundreds of tiles, every chunk of the binning populated, lists up to a
+    few hundred entries) for the kernel variants that the full-size configurations, all 4-channel, do not reach."""
+    sc = scenes.tiny(n=300_000, w=640, h=480, f=520.0, num_layers=8, list_depth=K, seed=40 + channels + K, views=views,
+                     channels=channels, radius=(0.0005, 0.05))
+    sc.confidence = (sc.confidence ** 0.3).astype(np.float32)
+    d = abi.desc_for_scene(sc, layout=layout, background_mode=views % 2)
+    run, ref, _ = _check_forward(oracle, sc, d)
+    assert ref["lengths"].max() > 64 and ref["counters"][0][0] > 100_000
+    _check_backward(oracle, sc, d, seed=channels)
+
+
 @pytest.mark.parametrize("w,h,L,n", [(4000, 40, 8, 20000), (37, 3000, 6, 20000), (1, 1, 1, 10), (2, 2, 2, 50), (33, 33, 6, 500)])
 def test_extreme_image_shapes(oracle, w, h, L, n):
     """Very wide and very tall images (many tile columns / rows, coarse layers one pixel high) and images smaller than
