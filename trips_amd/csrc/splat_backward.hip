@@ -257,7 +257,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 8 
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Pass 2: per point.
+// Pass 2: per point. A wavefront takes 64 consecutive points. The work of a point is one item per layer in which some
+// pixel retained it (the rank bytes say which); points differ in the layers they reach, so the items of the 64 points
+// are dealt out to the lanes through LDS, one item per lane and round (usually one round): every lane then issues the
+// gathers of its item at once, instead of all lanes walking the layers of the deepest point one memory round trip
+// after the other. An item's sums return through LDS and each point adds its items up in layer order.
+// The kernel is a chain of dependent memory round trips per step; it is kept short: the compact number of a step's
+// point is requested one step ahead, and what does not change from step to step (camera, rotation matrix) waits in LDS
+// rather than in registers, which the items need.
+constexpr int kItemFloats(int cpad) { return 4 + cpad; }  // {confidence, ip.x, ip.y, size} sums, then the descriptor's
+
+struct PointPassCamera
+{
+    Camera cam;
+    float R[9];
+};
+
 template <int C>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 : 1))) void backward_points_kernel(const BackwardParams p)
 {
@@ -265,10 +280,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
     constexpr int KIN  = entry_row_entries(CPAD);
     constexpr int RF   = 4 + CPAD;  // floats per blend record
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
+    constexpr int NIT  = kItemFloats(CPAD);
     const int lane     = threadIdx.x & 63;
-    const Camera cam   = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
-    float R[9];
-    rotation_matrix(cam.V, R);
+    const int wave     = threadIdx.x >> 6;
     const bool want_pose = p.d_pose != nullptr;
     const bool want_intr = p.d_intrinsics != nullptr;
     const bool want_size = p.d_point_size != nullptr;
@@ -278,27 +292,49 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
     // whole lines are written. (Descriptor columns other than the points' own, and all of them when the index is not
     // the identity, were cleared by zero_texel_grads_kernel.)
 
+    __shared__ PointPassCamera s_cam;
+    // what an item needs of its point {ip.x, ip.y, size field, confidence, size_px, softplus' * d size_px / d size},
+    // then the point in view space, kept here for the point's own lane
+    __shared__ float s_point[4][64][9];
+    __shared__ uint2 s_item[4][64 * 8];                 // {lane of the point | layer << 8, the layer's four rank bytes}
+    __shared__ __align__(16) float s_sums[4][64][NIT];  // sums of the items of one round
+    if (threadIdx.x == 0)
+    {
+        s_cam.cam = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
+        rotation_matrix(s_cam.cam.V, s_cam.R);
+    }
+    __syncthreads();
+
     // a thread sees a handful of points: its own sums stay in single precision, everything across threads is double
     float acc[NACC];
 #pragma unroll
     for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
 
-    for (int pid = blockIdx.x * 256 + threadIdx.x; pid < p.num_points; pid += gridDim.x * 256)
+    const int stride = (int)gridDim.x * 256;
+    int cid_next     = -1;
     {
+        const int pid0 = (int)blockIdx.x * 256 + (int)threadIdx.x;
+        if (pid0 < p.num_points) cid_next = p.cid_of[pid0];
+    }
+    for (int base = blockIdx.x * 256; base < p.num_points; base += stride)
+    {
+        asm volatile("" ::: "memory");  // what waits in LDS is read where it is used, in every step
+        const int pid = base + (int)threadIdx.x;
         // the records of a valid point sit at its compact number (valid points numbered in point order: lanes that are
         // neighbours here are neighbours there)
-        const int cid   = p.cid_of[pid];
+        const int cid   = cid_next;
         const bool live = cid >= 0;
-        if (!live && !overwrite) continue;
+        {
+            const long long pid2 = (long long)pid + stride;
+            cid_next             = pid2 < p.num_points ? p.cid_of[pid2] : -1;  // in flight during this step
+        }
         // {softplus'(raw size), depth, layers written, size_px}
         const float4 tail = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
-        const int tex       = identity ? pid : p.index[pid];  // (a column outside the table: the point was culled)
         const int max_layer = live ? __float_as_int(tail.z) : 0;
-        float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), rv = r0;  // ip.x ip.y size field conf; view xyz, softplus'(raw size)
         uint4 rk0 = make_uint4(~0u, ~0u, ~0u, ~0u), rk1 = rk0;
         if (live)
         {
-            r0              = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
+            const float4 r0 = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);  // ip.x ip.y size field conf
             // the point in view space, exactly as the projection kernel computed it
             float4 pos = p.position[pid];
             if (p.displacement)
@@ -308,104 +344,165 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
                 pos.y += dsp[1];
                 pos.z += dsp[2];
             }
-            float view[3];
-            transform_point(cam.V, pos.x, pos.y, pos.z, view);
-            rv = make_float4(view[0], view[1], view[2], tail.x);
             rk0 = *reinterpret_cast<const uint4*>(p.rank + (size_t)cid * 16);
             // layers 4..7: a row of the second plane, defined only for the points that were written to those layers
             if (max_layer > 4) rk1 = *reinterpret_cast<const uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16);
+            float view[3];
+            transform_point(s_cam.cam.V, pos.x, pos.y, pos.z, view);
+            const float J_softmax_proj = s_cam.cam.fx * s_cam.cam.cfx / fmaxf(view[2], 0.f);
+            float* sp = s_point[wave][lane];
+            sp[0] = r0.x, sp[1] = r0.y, sp[2] = r0.z, sp[3] = r0.w, sp[4] = tail.w, sp[5] = tail.x * J_softmax_proj;
+            sp[6] = view[0], sp[7] = view[1], sp[8] = view[2];
         }
+
+        // ---- the point's items: the layers it was written to in which some corner pixel retained it ----
+        const unsigned words[8] = {rk0.x, rk0.y, rk0.z, rk0.w, rk1.x, rk1.y, rk1.z, rk1.w};
+        unsigned layer_mask = 0;
+#pragma unroll
+        for (int l = 0; l < 8; ++l)
+            if (l < max_layer && words[l] != 0xFFFFFFFFu) layer_mask |= 1u << l;
+        const int my_items = __popc(layer_mask);
+        int first_item     = my_items;  // inclusive prefix over the wavefront, then made exclusive
+        for (int o = 1; o < 64; o <<= 1)
+        {
+            const int t = __shfl_up(first_item, o);
+            if (lane >= o) first_item += t;
+        }
+        const int num_items = __builtin_amdgcn_readlane(first_item, 63);  // <= 64 * 8
+        first_item -= my_items;
+        {
+            int k = first_item;
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+                if (layer_mask & (1u << l)) s_item[wave][k++] = make_uint2((unsigned)lane | ((unsigned)l << 8), words[l]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;
         float tex_grad[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) tex_grad[c] = 0.f;
-        const float conf = r0.w;
-        bool any         = false;
-        const float J_softmax_proj = cam.fx * cam.cfx / fmaxf(rv.z, 0.f);
+        const bool any = my_items > 0;
 
-        // one layer: the four gathers are issued together, then consumed in corner order
-        auto do_layer = [&](const int layer, const unsigned word)
+        for (int round = 0; round < num_items; round += 64)
         {
-            if (layer >= max_layer || word == 0xFFFFFFFFu) return;
-            any              = true;
-            const float mfac = 1.f / float(1 << layer);
-            const float ux = r0.x * mfac, uy = r0.y * mfac;
-            const float fx = floorf(ux), fy = floorf(uy);
-            const int px = (int)fx, py = (int)fy;
-            const float sx = ux - fx, sy = uy - fy;
-            float lfac = 1.f, J_lf = 0.f;
-            if (want_size) lfac = layer_factor_encoded_grad(r0.z, tail.w, layer, p.num_layers, &J_lf);
-            float2 e[4];
-            float4 gq[4][CPAD / 4];
-#pragma unroll
-            for (int corner = 0; corner < 4; ++corner)
+            if (round + lane < num_items)
             {
-                const unsigned j = (word >> (8 * corner)) & 0xFFu;
-                const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
-                const bool on      = j != 0xFFu;
-                const float* row   = p.entry_grad + (size_t)pix * entry_row_floats(CPAD);  // the pixel's row
-                const unsigned jj  = j & 15u;
-                const float2* src2 = jj < (unsigned)KIN ? reinterpret_cast<const float2*>(row + CPAD) + jj
-                                                        : reinterpret_cast<const float2*>(p.entry_over) + ((size_t)pix * (16 - KIN) + (jj - KIN));
-                e[corner]          = on ? *src2 : make_float2(0.f, 0.f);
-                const float4* src  = reinterpret_cast<const float4*>(row);
+                // one layer of one point: the four gathers are issued together, then consumed in corner order
+                const uint2 item    = s_item[wave][round + lane];
+                const int layer     = (int)(item.x >> 8);
+                const unsigned word = item.y;
+                const float* sp     = s_point[wave][item.x & 63u];
+                const float ipx = sp[0], ipy = sp[1], size_field = sp[2], conf = sp[3], size_px = sp[4], size_chain = sp[5];
+                const float mfac = 1.f / float(1 << layer);
+                const float ux = ipx * mfac, uy = ipy * mfac;
+                const float fx = floorf(ux), fy = floorf(uy);
+                const int px = (int)fx, py = (int)fy;
+                const float sx = ux - fx, sy = uy - fy;
+                float lfac = 1.f, J_lf = 0.f;
+                if (want_size) lfac = layer_factor_encoded_grad(size_field, size_px, layer, p.num_layers, &J_lf);
+                float2 e[4];
+                float4 gq[4][CPAD / 4];
 #pragma unroll
-                for (int q = 0; q < CPAD / 4; ++q) gq[corner][q] = on ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+                for (int corner = 0; corner < 4; ++corner)
+                {
+                    const unsigned j = (word >> (8 * corner)) & 0xFFu;
+                    const int gx = px + (corner & 1), gy = py + (corner >> 1);
+                    const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
+                    const bool on      = j != 0xFFu;
+                    const float* row   = p.entry_grad + (size_t)pix * entry_row_floats(CPAD);  // the pixel's row
+                    const unsigned jj  = j & 15u;
+                    const float2* src2 = jj < (unsigned)KIN ? reinterpret_cast<const float2*>(row + CPAD) + jj
+                                                            : reinterpret_cast<const float2*>(p.entry_over) + ((size_t)pix * (16 - KIN) + (jj - KIN));
+                    e[corner]          = on ? *src2 : make_float2(0.f, 0.f);
+                    const float4* src  = reinterpret_cast<const float4*>(row);
+#pragma unroll
+                    for (int q = 0; q < CPAD / 4; ++q) gq[corner][q] = on ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+                float i_conf = 0.f, i_d0 = 0.f, i_d1 = 0.f, i_size = 0.f;
+                float i_tex[CPAD];
+#pragma unroll
+                for (int c = 0; c < CPAD; ++c) i_tex[c] = 0.f;
+#pragma unroll
+                for (int corner = 0; corner < 4; ++corner)
+                {
+                    const unsigned j = (word >> (8 * corner)) & 0xFFu;
+                    if (j == 0xFFu) continue;
+                    const int gx = px + (corner & 1), gy = py + (corner >> 1);
+                    float gv[CPAD];
+#pragma unroll
+                    for (int q = 0; q < CPAD / 4; ++q)
+                    {
+                        gv[4 * q]     = gq[corner][q].x;
+                        gv[4 * q + 1] = gq[corner][q].y;
+                        gv[4 * q + 2] = gq[corner][q].z;
+                        gv[4 * q + 3] = gq[corner][q].w;
+                    }
+                    const float grad_alpha = e[corner].x;
+                    const float ta         = e[corner].y;
+#pragma unroll
+                    for (int c = 0; c < C; ++c) i_tex[c] += ta * gv[c];
+                    // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
+                    // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
+                    const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
+                    const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
+                    float blend    = wx * wy;
+                    const float J0 = x_hi ? wy : -wy;
+                    const float J1 = y_hi ? wx : -wx;
+                    if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
+                    i_conf += blend * lfac * grad_alpha;
+                    const float gbs = conf * lfac * grad_alpha;
+                    i_d0 += J0 * gbs;
+                    i_d1 += J1 * gbs;
+                    if (want_size)
+                    {
+                        const float grad_layer_ps = size_chain * J_lf * grad_alpha;
+                        i_size += blend * conf * grad_layer_ps;
+                    }
+                }
+                float4* out = reinterpret_cast<float4*>(s_sums[wave][lane]);
+                out[0]      = make_float4(i_conf, i_d0, i_d1, i_size);
+#pragma unroll
+                for (int q = 0; q < CPAD / 4; ++q) out[1 + q] = make_float4(i_tex[4 * q], i_tex[4 * q + 1], i_tex[4 * q + 2], i_tex[4 * q + 3]);
             }
-#pragma unroll
-            for (int corner = 0; corner < 4; ++corner)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // the point's items of this round, in layer order
+            const int j_end = min(first_item + my_items, round + 64);
+            for (int j = max(first_item, round); j < j_end; ++j)
             {
-                const unsigned j = (word >> (8 * corner)) & 0xFFu;
-                if (j == 0xFFu) continue;
-                const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                float gv[CPAD];
+                const float4* in = reinterpret_cast<const float4*>(s_sums[wave][j - round]);
+                const float4 a   = in[0];
+                conf_grad += a.x;
+                d0 += a.y;
+                d1 += a.z;
+                size_grad += a.w;
 #pragma unroll
                 for (int q = 0; q < CPAD / 4; ++q)
                 {
-                    gv[4 * q]     = gq[corner][q].x;
-                    gv[4 * q + 1] = gq[corner][q].y;
-                    gv[4 * q + 2] = gq[corner][q].z;
-                    gv[4 * q + 3] = gq[corner][q].w;
-                }
-                const float grad_alpha = e[corner].x;
-                const float ta         = e[corner].y;
-#pragma unroll
-                for (int c = 0; c < C; ++c) tex_grad[c] += ta * gv[c];
-                // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
-                // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
-                const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
-                const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
-                float blend    = wx * wy;
-                const float J0 = x_hi ? wy : -wy;
-                const float J1 = y_hi ? wx : -wx;
-                if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
-                conf_grad += blend * lfac * grad_alpha;
-                const float gbs = conf * lfac * grad_alpha;
-                d0 += J0 * gbs;
-                d1 += J1 * gbs;
-                if (want_size)
-                {
-                    const float grad_layer_ps = rv.w * J_softmax_proj * J_lf * grad_alpha;
-                    size_grad += blend * conf * grad_layer_ps;
+                    const float4 t = in[1 + q];
+                    if (4 * q < C) tex_grad[4 * q] += t.x;
+                    if (4 * q + 1 < C) tex_grad[4 * q + 1] += t.y;
+                    if (4 * q + 2 < C) tex_grad[4 * q + 2] += t.z;
+                    if (4 * q + 3 < C) tex_grad[4 * q + 3] += t.w;
                 }
             }
-        };
-        do_layer(0, rk0.x);
-        do_layer(1, rk0.y);
-        do_layer(2, rk0.z);
-        do_layer(3, rk0.w);
-        do_layer(4, rk1.x);
-        do_layer(5, rk1.y);
-        do_layer(6, rk1.z);
-        do_layer(7, rk1.w);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        if (pid >= p.num_points || (!live && !overwrite)) continue;
+        const int tex = identity ? pid : p.index[pid];  // (a column outside the table: the point was culled)
         if (!any && !overwrite) continue;
 
         float g_point[3] = {0.f, 0.f, 0.f}, g_pose[6], g_k[5], g_dis[8];
         if (any)
         {
-            project_backward(cam, R, rv.x, rv.y, rv.z, d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
+            const float* sp = s_point[wave][lane];
+            project_backward(s_cam.cam, s_cam.R, sp[6], sp[7], sp[8], d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
             if (want_pose)
             {
 #pragma unroll
