@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "e2fa78f619d5204072c0a9d0873ae4dcfdd92584e1ec321e68804d7f0fe3913c"
+PMC_SOURCES_SHA256 = "b87d4f1121f549844f6f51a88e75379fdbeb64171927590ee355b28565b3a082"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129123, 299639),
-    "bin_scatter": (88884, 152706),
+    "project_bin": (129122, 299923),
+    "bin_scatter": (88873, 152862),
     "tile_count": (13139, 2296),
-    "tile_scatter": (32620, 110293),
-    "sort_blend": (332127, 350809),
-    "backward_pixels": (465002, 187842),
-    "backward_points": (1045008, 234887),
-    "adam_fused": (383885, 498420),
+    "tile_scatter": (32705, 110869),
+    "sort_blend": (330764, 350719),
+    "backward_pixels": (465026, 187848),
+    "backward_points": (1045854, 234887),
+    "adam_fused": (383860, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
