@@ -183,6 +183,19 @@ def test_backward_small(oracle, L, K, bg):
     assert np.abs(g["d_pose"]).max() > 0 and np.abs(g["d_intrinsics"]).max() > 0
 
 
+@pytest.mark.parametrize("channels", [4, 16])
+def test_backward_points_written_to_many_layers(oracle, channels):
+    """Every point is large enough for four to eight layers: a wavefront of the point pass then has several hundred
+    (point, layer) items for its 64 points, which it works off in several rounds."""
+    sc = scenes.tiny(n=3000, w=128, h=96, f=110.0, num_layers=8, list_depth=16, seed=77, channels=channels,
+                     radius=(0.08, 1.2))
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    layers = ref["max_layer"][0][ref["depth"][0] > 0]
+    assert np.median(layers) >= 4 and layers.max() >= 7
+    _check_backward(oracle, sc, d, seed=9)
+
+
 @pytest.mark.parametrize("channels,K", [(3, 16), (8, 8), (16, 16)])
 def test_backward_other_channel_counts(oracle, channels, K):
     sc = scenes.tiny(n=2500, w=56, h=40, f=50.0, num_layers=3, list_depth=K, seed=60 + channels, channels=channels,
