@@ -170,6 +170,13 @@ __device__ __forceinline__ float row_shr1(float v, float fill)
     return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), kDppShr1, 0xf, 0xf, false));
 }
 
+// lane i reads lane i-S of the row; the first S lanes of the row read `fill`
+template <int S>
+__device__ __forceinline__ float row_shr(float v, float fill)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x110 + S, 0xf, 0xf, false));
+}
+
 // lane i reads lane i+S of the row; lanes past the end read 0
 template <int S>
 __device__ __forceinline__ float row_shl0(float v)

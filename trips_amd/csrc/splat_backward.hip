@@ -174,29 +174,53 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
     // For pass 2, one row of 64 bytes (128 above 8 channels) per pixel: the pixel's image gradient (a point finds all
     // channels and its entry in one line) followed by {dL/dalpha, T alpha} of the first entry_row_entries retained
     // entries; the entries beyond that go to a table of their own.
-    constexpr int KIN = entry_row_entries(CPAD);
-    float* row        = p.entry_grad + (size_t)(unsigned)pix * entry_row_floats(CPAD);
-    if (has)
+    // Rows of 64 bytes are written a second time, one row further on (see BackwardParams).
+    constexpr int KIN       = entry_row_entries(CPAD);
+    constexpr bool kShifted = entry_row_floats(CPAD) == 16;
+    float* row              = p.entry_grad + (size_t)(unsigned)pix * entry_row_floats(CPAD);
+    float* row2             = kShifted ? p.entry_grad_shifted + (size_t)(unsigned)pix * 16 : nullptr;
+    if (has && sub >= KIN)
+        __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(p.entry_over) + ((size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)));
+    if (CPAD == 4)
     {
-        if (sub < KIN)
-            __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row + CPAD) + sub);
-        else
-            __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(p.entry_over) + ((size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)));
+        // the whole row with one store instruction, 8 bytes per lane: lanes 0 and 1 the image gradient, lanes 2..7 the
+        // entries of lanes 0..5 (64 contiguous bytes per pixel instead of a 16-byte and six 8-byte pieces)
+        const float ga_before = row_shr<2>(grad_alpha, 0.f), ta_before = row_shr<2>(ta, 0.f);
+        const float g2 = C > 2 ? g[C > 2 ? 2 : 0] : 0.f, g3 = C > 3 ? g[C > 3 ? 3 : 0] : 0.f;
+        const vf2 v      = sub == 0 ? vf2{g[0], g[1]} : sub == 1 ? vf2{g2, g3} : vf2{ga_before, ta_before};
+        const bool store = sub < 2 ? m > 0 : (sub < 8 && sub - 2 < m);
+        if (store)
+        {
+            __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row) + sub);
+            __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row2) + sub);
+        }
     }
-    if (sub == 0 && m > 0)
+    else
     {
-        float gp[CPAD];
+        if (has && sub < KIN)
+        {
+            __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row + CPAD) + sub);
+            if (kShifted) __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row2 + CPAD) + sub);
+        }
+        if (sub == 0 && m > 0)
+        {
+            float gp[CPAD];
 #pragma unroll
-        for (int c = 0; c < CPAD; ++c) gp[c] = c < C ? g[c] : 0.f;
+            for (int c = 0; c < CPAD; ++c) gp[c] = c < C ? g[c] : 0.f;
 #pragma unroll
-        for (int q = 0; q < CPAD / 4; ++q) __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row) + q);
+            for (int q = 0; q < CPAD / 4; ++q)
+            {
+                __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row) + q);
+                if (kShifted)
+                    __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row2) + q);
+            }
+        }
     }
 }
 
-// (up to 4 channels the kernel needs 65 registers without the hint and fits the 64 of 8 wavefronts per SIMD with it,
-// no spills; with more channels the hint would cost spills)
+// (up to 4 channels the kernel needs 77 registers: seven wavefronts per SIMD; held to the 64 of eight it spills)
 template <int C>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 8 : 1))) void backward_pixels_kernel(const BackwardParams p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 7 : 1))) void backward_pixels_kernel(const BackwardParams p)
 {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // a lane sees a few dozen pixels: its own sums stay in single precision, everything across lanes is double
@@ -405,6 +429,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
                 if (want_size) lfac = layer_factor_encoded_grad(size_field, size_px, layer, p.num_layers, &J_lf);
                 float2 e[4];
                 float4 gq[4][CPAD / 4];
+                // 64-byte rows: a footprint that starts at an odd pixel reads the copy in which its two pixels of a
+                // row share a line (not across the border of a tile, where they are not neighbours in memory)
+                const float* rows = (entry_row_floats(CPAD) == 16 && (px & 1) && (px & (kTile - 1)) != kTile - 1)
+                                        ? p.entry_grad_shifted
+                                        : p.entry_grad;
 #pragma unroll
                 for (int corner = 0; corner < 4; ++corner)
                 {
@@ -412,7 +441,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
                     const int gx = px + (corner & 1), gy = py + (corner >> 1);
                     const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
                     const bool on      = j != 0xFFu;
-                    const float* row   = p.entry_grad + (size_t)pix * entry_row_floats(CPAD);  // the pixel's row
+                    const float* row   = rows + (size_t)pix * entry_row_floats(CPAD);  // the pixel's row
                     const unsigned jj  = j & 15u;
                     const float2* src2 = jj < (unsigned)KIN ? reinterpret_cast<const float2*>(row + CPAD) + jj
                                                             : reinterpret_cast<const float2*>(p.entry_over) + ((size_t)pix * (16 - KIN) + (jj - KIN));

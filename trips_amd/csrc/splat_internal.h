@@ -246,6 +246,7 @@ __host__ __device__ constexpr int entry_row_entries(int cpad) { return (entry_ro
 struct BackwardWorkspaceLayout
 {
     size_t entry_grad;  // float [Pi, entry_row_floats]
+    size_t entry_grad_shifted;  // 64-byte rows only: float [1 + Pi + 1, 16], a second copy one row further on (0: none)
     size_t entry_over;  // float2 [Pi, 16 - entry_row_entries]
     size_t bytes;
 };
@@ -349,6 +350,11 @@ struct BackwardParams
     float* entry_grad;    // [Pi, entry_row_floats] a row per pixel: dL/dimage[0..Cpad), then float2 {dL/dalpha, T alpha} of
                           // the first entry_row_entries retained entries (workspace)
     float* entry_over;    // [Pi, 16 - entry_row_entries] float2: the retained entries beyond those (workspace)
+    // Rows of 64 bytes: two pixels share a 128-byte line, the pairs (0,1), (2,3), ... of a tile row. A footprint that
+    // starts at an odd pixel would find its two pixels of a row in two lines; the rows are therefore written a second
+    // time, one row further on, where the pairs are (1,2), (3,4), ...: row of pixel pix at entry_grad_shifted + 16 pix
+    // (the pointer already includes the shift; null when a row is a line of its own).
+    float* entry_grad_shifted;
     const unsigned char* rank;  // [2][N, 16] (saved state) rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
     float* d_texture;
     float* d_confidence;

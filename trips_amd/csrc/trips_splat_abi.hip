@@ -278,6 +278,12 @@ BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const
     o += align256(P * (size_t)entry_row_floats((d.num_channels + 3) & ~3) * sizeof(float));
     w.entry_over = o;
     o += align256(P * (size_t)(16 - entry_row_entries((d.num_channels + 3) & ~3)) * 2 * sizeof(float));
+    w.entry_grad_shifted = 0;
+    if (entry_row_floats((d.num_channels + 3) & ~3) == 16)
+    {
+        w.entry_grad_shifted = o;
+        o += align256((P + 2) * 16 * sizeof(float));
+    }
     w.bytes = o;
     return w;
 }
@@ -549,6 +555,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
         p.entry_grad   = reinterpret_cast<float*>(ws + bl.entry_grad);
         p.entry_over   = reinterpret_cast<float*>(ws + bl.entry_over);
+        p.entry_grad_shifted = bl.entry_grad_shifted ? reinterpret_cast<float*>(ws + bl.entry_grad_shifted) + 16 : nullptr;
         p.rank         = reinterpret_cast<const unsigned char*>(sv + sl.rank);
         for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
         p.d_texture    = grads->d_texture;
