@@ -136,6 +136,25 @@ def test_medium_views_other_channel_counts(oracle, channels, K, layout, views):
     _check_backward(oracle, sc, d, seed=channels)
 
 
+@pytest.mark.parametrize("order", ["random", "by_screen_tile"])
+def test_medium_view_memory_order_of_the_points(oracle, order):
+    """The backward lays its exchange rows out differently for clouds whose memory order is coherent on the screen
+    (neighbouring points in the same tile) and for randomly ordered ones: the same view with the points in both orders."""
+    sc = scenes.tiny(n=200_000, w=640, h=480, f=520.0, num_layers=6, list_depth=16, seed=61, radius=(0.0005, 0.05))
+    if order == "by_screen_tile":
+        d0 = abi.desc_for_scene(sc)
+        ip = oracle.forward(sc, d0)["ip"][0]
+        key = (np.floor(ip[:, 1] / 32).astype(np.int64) * 64 + np.floor(ip[:, 0] / 32).astype(np.int64))
+        perm = np.argsort(key, kind="stable")
+        sc.position = np.ascontiguousarray(sc.position[perm])
+        sc.point_size = np.ascontiguousarray(sc.point_size[perm])
+        sc.texture = np.ascontiguousarray(sc.texture[:, perm])
+        sc.confidence = np.ascontiguousarray(sc.confidence[perm])
+    d = abi.desc_for_scene(sc)
+    _check_forward(oracle, sc, d)
+    _check_backward(oracle, sc, d, seed=3)
+
+
 @pytest.mark.parametrize("w,h,L,n", [(4000, 40, 8, 20000), (37, 3000, 6, 20000), (1, 1, 1, 10), (2, 2, 2, 50), (33, 33, 6, 500)])
 def test_extreme_image_shapes(oracle, w, h, L, n):
     """Very wide and very tall images (many tile columns / rows, coarse layers one pixel high) and images smaller than

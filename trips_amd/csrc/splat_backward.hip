@@ -72,7 +72,7 @@ __device__ __forceinline__ double wave_sum(double v)
 // Pass 1: per pixel row. Writes the pixel's exchange row {g[0..Cpad), {dL/dalpha_j, T_j alpha_j} for j < entry_row_entries}.
 // 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
 // than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
-template <int C, int ROW>
+template <int C, int ROW, bool SECOND>
 __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, const TileCtx& tc, const float* gi, int pix_first,
                                                     int m_in, float (&acc_bg)[C])
 {
@@ -178,6 +178,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
     constexpr int KIN       = entry_row_entries(CPAD);
     constexpr bool kShifted = entry_row_floats(CPAD) == 16;
     float* row              = p.entry_grad + (size_t)(unsigned)pix * entry_row_floats(CPAD);
+    constexpr bool second   = kShifted && SECOND;
     float* row2             = kShifted ? p.entry_grad_shifted + (size_t)(unsigned)pix * 16 : nullptr;
     if (has && sub >= KIN)
         __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(p.entry_over) + ((size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)));
@@ -192,7 +193,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
         if (store)
         {
             __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row) + sub);
-            __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row2) + sub);
+            if (second) __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row2) + sub);
         }
     }
     else
@@ -200,7 +201,7 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
         if (has && sub < KIN)
         {
             __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row + CPAD) + sub);
-            if (kShifted) __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row2 + CPAD) + sub);
+            if (second) __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row2 + CPAD) + sub);
         }
         if (sub == 0 && m > 0)
         {
@@ -211,16 +212,16 @@ __device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, con
             for (int q = 0; q < CPAD / 4; ++q)
             {
                 __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row) + q);
-                if (kShifted)
+                if (second)
                     __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row2) + q);
             }
         }
     }
 }
 
-// (up to 4 channels the kernel needs 77 registers: seven wavefronts per SIMD; held to the 64 of eight it spills)
-template <int C>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 7 : 1))) void backward_pixels_kernel(const BackwardParams p)
+// SECOND: the exchange rows are written twice (see BackwardParams::entry_grad_shifted).
+template <int C, bool SECOND>
+__device__ __forceinline__ void backward_pixels_body(const BackwardParams& p)
 {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // a lane sees a few dozen pixels: its own sums stay in single precision, everything across lanes is double
@@ -255,11 +256,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 7 
             const int pix_first = lb * kQuarter + (it * 4 + wave) * 8;
             const int m8        = __builtin_amdgcn_readfirstlane(__shfl(m_grp, it * 8));
             if (m8 <= 8)
-                backward_pixel_rows<C, 8>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 3)), acc_bg);
+                backward_pixel_rows<C, 8, SECOND>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 3)), acc_bg);
             else
             {
-                backward_pixel_rows<C, 16>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 4)), acc_bg);
-                backward_pixel_rows<C, 16>(p, tc, gi, pix_first + 4, __shfl(m_all, it * 8 + 4 + (lane >> 4)), acc_bg);
+                backward_pixel_rows<C, 16, SECOND>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 4)), acc_bg);
+                backward_pixel_rows<C, 16, SECOND>(p, tc, gi, pix_first + 4, __shfl(m_all, it * 8 + 4 + (lane >> 4)), acc_bg);
             }
         }
     }
@@ -278,6 +279,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 7 
         double v    = s_acc[0][i] + s_acc[1][i] + s_acc[2][i] + s_acc[3][i];
         if (v != 0.0) unsafeAtomicAdd(p.d_background + i, (float)v);
     }
+}
+
+// (up to 4 channels the kernel needs 77 registers: seven wavefronts per SIMD; held to the 64 of eight it spills)
+// The two forms of the body are separate code: a flag tested at every store costs registers that the kernel lacks.
+template <int C>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 7 : 1))) void backward_pixels_kernel(const BackwardParams p)
+{
+    if (entry_row_floats((C + 3) & ~3) == 16 && use_shifted_rows(*p.header))
+        backward_pixels_body<C, true>(p);
+    else
+        backward_pixels_body<C, false>(p);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -312,6 +324,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
     const bool want_size = p.d_point_size != nullptr;
     const bool identity  = p.header->not_identity == 0;  // index[pid] == pid for every point
     const bool overwrite = p.overwrite != 0;             // outputs are written, not added to
+    const bool shifted_rows = entry_row_floats(CPAD) == 16 && use_shifted_rows(*p.header);
     // In that mode every point stores all its outputs (zeros where it has no gradient), all lanes at one place, so that
     // whole lines are written. (Descriptor columns other than the points' own, and all of them when the index is not
     // the identity, were cleared by zero_texel_grads_kernel.)
@@ -431,7 +444,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
                 float4 gq[4][CPAD / 4];
                 // 64-byte rows: a footprint that starts at an odd pixel reads the copy in which its two pixels of a
                 // row share a line (not across the border of a tile, where they are not neighbours in memory)
-                const float* rows = (entry_row_floats(CPAD) == 16 && (px & 1) && (px & (kTile - 1)) != kTile - 1)
+                const float* rows = (shifted_rows && (px & 1) && (px & (kTile - 1)) != kTile - 1)
                                         ? p.entry_grad_shifted
                                         : p.entry_grad;
 #pragma unroll

@@ -206,14 +206,16 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
     __shared__ int s_valid[2][WAVES];  // valid points of every wavefront in this step (two steps in flight)
     __shared__ int s_flags;            // bit 0: not_identity, bit 1: bad_index, of any point of the chunk
+    __shared__ int s_same_tile;        // valid points in the finest-layer tile of the point before them
     const Camera cam  = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L       = p.num_layers;
     const int NB      = p.geom.bin_off[L];
     bool not_identity = false;  // some point's descriptor column differs from its own index
     bool bad_index    = false;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) s_hist[i] = 0;
-    if (threadIdx.x == 0) s_flags = 0;
+    if (threadIdx.x == 0) s_flags = 0, s_same_tile = 0;
     __syncthreads();
+    int same_tile = 0;  // (wavefront-uniform)
 
     int begin, end;
     chunk_point_range(p, begin, end);
@@ -246,6 +248,12 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         if (pid < end) o = project_point<TRAIN>(p, cam, pid, in, s_hist, not_identity, bad_index);
         const unsigned long long vm = __ballot(o.valid);
         if (lane == 0) s_valid[step][wave] = (int)__popcll(vm);
+        {
+            // how coherent the cloud's memory order is on the screen (lane 0 of a wavefront has no neighbour here)
+            const int tile      = o.valid ? (((int)o.ipy >> kTileShift) << 16) | ((int)o.ipx >> kTileShift) : -1;
+            const int tile_prev = __shfl_up(tile, 1);
+            same_tile += (int)__popcll(__ballot(o.valid && lane > 0 && tile == tile_prev));
+        }
         __syncthreads();
         int before = 0, total = 0;
 #pragma unroll
@@ -287,6 +295,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     {
         const int flags = (__ballot(not_identity) != 0 ? 1 : 0) | (__ballot(bad_index) != 0 ? 2 : 0);
         if (flags && lane == 0) atomicOr(&s_flags, flags);
+        if (same_tile && lane == 0) atomicAdd(&s_same_tile, same_tile);
     }
 
     // this workgroup's row of the histogram matrix [workgroup][bin]; its valid points and flags for the scan kernel,
@@ -298,6 +307,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     {
         p.chunk_valid[blockIdx.x]                = next - begin;
         p.chunk_valid[p.bin_groups + blockIdx.x] = s_flags;
+        p.chunk_valid[2 * p.bin_groups + blockIdx.x] = s_same_tile;
     }
 }
 
@@ -326,20 +336,21 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
     }
     __shared__ int s_wave[2][16];
     __shared__ int s_carry[2];
-    __shared__ unsigned long long s_valid_total;
+    __shared__ unsigned long long s_valid_total, s_same_total;
     __shared__ int s_flags;
     if (threadIdx.x == 0)
     {
         s_carry[0] = s_carry[1] = 0;
-        s_valid_total           = 0;
+        s_valid_total = s_same_total = 0;
         s_flags                 = 0;
         *long_count             = 0;
     }
     __syncthreads();
     for (int g = threadIdx.x; g < G; g += 1024)
     {
-        const int v = chunk_valid[g], f = chunk_valid[G + g];
+        const int v = chunk_valid[g], f = chunk_valid[G + g], st = chunk_valid[2 * G + g];
         if (v) atomicAdd(&s_valid_total, (unsigned long long)v);
+        if (st) atomicAdd(&s_same_total, (unsigned long long)st);
         if (f) atomicOr(&s_flags, f);
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -401,12 +412,13 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
         header->retained     = 0;
         header->not_identity = (unsigned long long)(s_flags & 1);
         header->bad_index    = 0;
-        header->reserved[0] = header->reserved[1] = 0;
+        header->same_tile_as_previous = s_same_total;
+        header->reserved              = 0;
         if (first_view)
         {
             status->n_valid = status->n_entries = status->overflow = status->retained = status->not_identity = 0;
             status->bad_index                                                       = bad;
-            status->reserved[0] = status->reserved[1] = 0;
+            status->same_tile_as_previous = status->reserved = 0;
         }
         else if (bad)
             status->bad_index = 1;  // (the views of a call run one after the other on the stream)

@@ -218,8 +218,16 @@ struct ViewHeader
     unsigned long long retained;    // R: sum of the retained entries (filled by the counters query)
     unsigned long long not_identity;  // some point's descriptor column differs from its own index
     unsigned long long bad_index;   // some point's descriptor column lies outside [0, num_texels): the point was skipped
-    unsigned long long reserved[2];
+    // valid points whose finest-layer tile is also that of the point before them in memory: near n_valid for a cloud
+    // stored along a space-filling curve, near zero for one in random order (the backward chooses its exchange layout
+    // by it)
+    unsigned long long same_tile_as_previous;
+    unsigned long long reserved;
 };
+
+// The backward keeps a second, shifted copy of its exchange rows (BackwardParams::entry_grad_shifted) when fewer than a
+// quarter of the valid points lie in the finest-layer tile of the point before them in memory.
+__host__ __device__ inline bool use_shifted_rows(const ViewHeader& h) { return 4 * h.same_tile_as_previous < h.n_valid; }
 
 // Layout of one view's saved state (all offsets in bytes, 256-aligned)
 struct SavedLayout
@@ -253,7 +261,7 @@ struct BackwardWorkspaceLayout
 
 struct WorkspaceLayout
 {
-    size_t chunk_valid;   // int32 [2 G]  valid points of every chunk of the binning kernels, then the chunks' flags
+    size_t chunk_valid;   // int32 [3 G]  valid points of every chunk of the binning kernels, the chunks' flags, their same-tile counts
     size_t prec;         // float4 [N]         point records, when there is no saved state to hold them
     size_t counts;       // int32 [Pi]   list length per cell (the points whose 2 x 2 footprint starts at that pixel)
     size_t cursor;       // int32 [Pi]   first key of each cell's list (-1 - first candidate row for a long list)
@@ -353,7 +361,9 @@ struct BackwardParams
     // Rows of 64 bytes: two pixels share a 128-byte line, the pairs (0,1), (2,3), ... of a tile row. A footprint that
     // starts at an odd pixel would find its two pixels of a row in two lines; the rows are therefore written a second
     // time, one row further on, where the pairs are (1,2), (3,4), ...: row of pixel pix at entry_grad_shifted + 16 pix
-    // (the pointer already includes the shift; null when a row is a line of its own).
+    // (the pointer already includes the shift; null when a row is a line of its own). Written and read only for clouds
+    // whose memory order is not coherent on the screen (use_shifted_rows): in a coherent one the lines are shared
+    // by neighbouring lanes anyway, and the second copy costs the pixel pass more than it saves the point pass.
     float* entry_grad_shifted;
     const unsigned char* rank;  // [2][N, 16] (saved state) rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
     float* d_texture;
