@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "f60d65ea99038be665cda69597fcd3e4b92efa1712a35012c69f0688fb8e4587"
+PMC_SOURCES_SHA256 = "fe09383b6ccf15aea54b3b474b4f64f2c8cad5bb14ebf416b16dfa9c5a0b7e24"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129124, 299844),
-    "bin_scatter": (88890, 152732),
-    "tile_count": (13139, 2296),
-    "tile_scatter": (32532, 110347),
-    "sort_blend": (331282, 350879),
-    "backward_pixels": (450282, 288117),
-    "backward_points": (866920, 234887),
-    "adam_fused": (383883, 498420),
+    "project_bin": (129126, 293064),
+    "bin_scatter": (88895, 152859),
+    "tile_count": (13142, 2296),
+    "tile_scatter": (32679, 110240),
+    "sort_blend": (330873, 351175),
+    "backward_pixels": (453194, 296274),
+    "backward_points": (866953, 234887),
+    "adam_fused": (383881, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")

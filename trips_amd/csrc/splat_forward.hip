@@ -346,14 +346,30 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
         *long_count             = 0;
     }
     __syncthreads();
-    for (int g = threadIdx.x; g < G; g += 1024)
-    {
-        const int v = chunk_valid[g], f = chunk_valid[G + g], st = chunk_valid[2 * G + g];
-        if (v) atomicAdd(&s_valid_total, (unsigned long long)v);
-        if (st) atomicAdd(&s_same_total, (unsigned long long)st);
-        if (f) atomicOr(&s_flags, f);
-    }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    {
+        // sums over the chunks: per wavefront first, then one LDS atomic per wavefront and sum
+        unsigned long long v = 0, st = 0;
+        int f = 0;
+        for (int g = threadIdx.x; g < G; g += 1024)
+        {
+            v += (unsigned long long)(unsigned)chunk_valid[g];
+            f |= chunk_valid[G + g];
+            st += (unsigned long long)(unsigned)chunk_valid[2 * G + g];
+        }
+        for (int o = 32; o > 0; o >>= 1)
+        {
+            v += __shfl_xor(v, o);
+            st += __shfl_xor(st, o);
+            f |= __shfl_xor(f, o);
+        }
+        if (lane == 0)
+        {
+            if (v) atomicAdd(&s_valid_total, v);
+            if (st) atomicAdd(&s_same_total, st);
+            if (f) atomicOr(&s_flags, f);
+        }
+    }
     for (int base = 0; base < NB; base += 1024)
     {
         const int idx = base + threadIdx.x;
