@@ -31,16 +31,16 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "fe09383b6ccf15aea54b3b474b4f64f2c8cad5bb14ebf416b16dfa9c5a0b7e24"
+PMC_SOURCES_SHA256 = "5b71e9a27a10fa76f013affe06541409e80f7e317b3c265497fefd3d6d0a417f"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129126, 293064),
-    "bin_scatter": (88895, 152859),
+    "project_bin": (129125, 292728),
+    "bin_scatter": (88876, 152867),
     "tile_count": (13142, 2296),
-    "tile_scatter": (32679, 110240),
-    "sort_blend": (330873, 351175),
-    "backward_pixels": (453194, 296274),
-    "backward_points": (866953, 234887),
-    "adam_fused": (383881, 498420),
+    "tile_scatter": (32640, 110285),
+    "sort_blend": (333383, 350795),
+    "backward_pixels": (453556, 296281),
+    "backward_points": (866929, 234887),
+    "adam_fused": (383862, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
