@@ -5,7 +5,8 @@
 //   bin_scan / bin_scatter / tile_count / tile_scatter
 //                        <- per-pixel counting (:355-361), cub ExclusiveSum section (:1155-1232) and
 //                           SplattingPass (:368-436)
-//   sort_blend_kernel    <- FastSortFusedNew    src/lib/rendering/RenderForward.cu:474-1059
+//   cell_sort_kernel / blend_kernel
+//                        <- FastSortFusedNew    src/lib/rendering/RenderForward.cu:474-1059
 //
 // Differences in shape, not in result. The reference increments one global counter per (point, layer, corner),
 // scans layer by layer with two blocking read-backs each, and takes one more global atomic per entry to place
@@ -13,13 +14,15 @@
 // first binned, once, into the 32 x 32 pixel tile of its footprint's first pixel (workgroup-private LDS histograms
 // and a column scan: no global atomics); a workgroup per tile then counts, scans and places the keys of its 1024
 // cells with LDS atomics, one key per pair, and the blend gathers a pixel's list from the four cells whose
-// footprints cover it. A wavefront of the sort holds four pixel lists of 16 lanes (one DPP row each, or eight of 8
-// lanes) instead of two per 32-lane warp; the per-point record gathered by the blend carries position, size,
+// footprints cover it. The sort is done per cell (each serves four pixels); a pixel is one lane of a wavefront that
+// owns 8 x 8 of them, merges its four cell lists and blends front to back, instead of two lists per 32-lane warp; the per-point record gathered by the blend carries position, size,
 // confidence and descriptor together; what is kept for the backward is the sorted id list per pixel (64 B) instead
 // of 16 x 7 floats.
 #include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"
+
+#include <type_traits>
 
 #pragma clang fp contract(off)
 
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         {
             __builtin_nontemporal_store(pid, p.pid_of + cid);
             // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
-            // pixel's list; filled by sort_blend): a plane of 16 bytes per compact number for layers 0..3 and a second
+            // pixel's list; filled by the blend kernels): a plane of 16 bytes per compact number for layers 0..3 and a second
             // one for layers 4..7. Every valid point clears its row of the first, the few points that reach layer 4 and
             // beyond their row of the second as well.
             __builtin_nontemporal_store(vu4{~0u, ~0u, ~0u, ~0u}, reinterpret_cast<vu4*>(p.rank + (size_t)cid * 16));
@@ -781,6 +784,179 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// A pixel's list is the union of the lists of the four cells whose 2 x 2 footprints cover it: (x-1, y-1), (x, y-1),
+// (x-1, y), (x, y) (CountAndCollectTiled adds every point to the four pixels of its footprint,
+// RenderForward.cu:300-366; here a point is filed once, under its footprint's first pixel, and the pixels gather).
+// The K nearest entries of a pixel are among the K nearest of each of its cells, and a cell serves four pixels, so the
+// sort (FastSortFusedNew, RenderForward.cu:474-1059) is split:
+//   cell_sort_kernel   every cell's list sorted in place, ascending, and cut to its 16 smallest keys: a list of up to
+//                      8 keys by one lane (a sorting network over registers), a longer one by a 16-lane DPP row that
+//                      streams it in chunks of 16.
+//   blend_kernel       a wavefront owns an 8 x 8 block of pixels, one pixel per lane: a pixel with up to 8 entries
+//                      sorts them with a network, any other merges the (sorted, cut) lists of its four cells; then the
+//                      alpha blend front to back (RenderForward.cu:820-1048).
+// A pixel's colour is summed in the order of a balanced binary tree over the list positions.
+constexpr int kCellKeep    = 16;  // keys of a cell that can reach a pixel's list (the largest list depth)
+constexpr int kLaneSortMax = 8;   // longest list that a lane sorts with a network
+constexpr int kStagedKeys  = 8;   // keys per cell that blend_kernel stages in LDS for the merging lanes
+
+// {first key (negative: a long list, whose candidates are in `cand`), readable keys, entries} of a cell
+__device__ __forceinline__ int4 cell_info(const ForwardParams& p, int cell)
+{
+    const int len   = p.counts[cell];
+    const int start = p.cursor[cell];  // negative: a long list, reduced to candidates by long_list_reduce_kernel
+    // keys actually there: the key storage may have ended inside the list
+    const int rd = start < 0 ? ((len + kLongSegment - 1) / kLongSegment) * 16 : (int)max(0ll, min((long long)len, p.capacity - start));
+    return make_int4(start, rd, len, 0);
+}
+
+// the keys of a cell: in the key array, or the candidate rows that the reduction pass left for a long list
+__device__ __forceinline__ u64* cell_keys(const ForwardParams& p, int start)
+{
+    return start >= 0 ? p.keys + (unsigned)start : p.cand + (size_t)(unsigned)(-1 - start) * 16;
+}
+
+// the same for the cell (cx, cy) of the layer of `tc`, its readable keys cut to the kCellKeep that cell_sort_kernel
+// left in order (empty outside the layer and in its last row and column, where no footprint starts)
+__device__ __forceinline__ int4 load_cell(const ForwardParams& p, const TileCtx& tc, int cx, int cy)
+{
+    int4 r = make_int4(0, 0, 0, 0);
+    if (cx >= 0 && cy >= 0 && cx < tc.w - 1 && cy < tc.h - 1)
+    {
+        const int bin = tc.bin + ((cx - tc.x0) >> kTileShift) + ((cy - tc.y0) >> kTileShift) * tc.tiles_x;  // shifts round down
+        r   = cell_info(p, (bin << (2 * kTileShift)) | ((cy & (kTile - 1)) << kTileShift) | (cx & (kTile - 1)));
+        r.y = min(r.y, kCellKeep);
+    }
+    return r;
+}
+
+// alpha of a list entry at pixel (gx, gy) of `layer` and the entry's (layer, footprint corner) slot of its point
+__device__ __forceinline__ float entry_alpha(const float4& r0, int layer, int num_layers, int gx, int gy, int& slot)
+{
+    const float m  = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
+    const float ux = r0.x * m, uy = r0.y * m;
+    float w        = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
+    if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
+    float a = w * r0.w;
+    a *= layer_factor_encoded(r0.z, layer, num_layers);
+    const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
+    slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
+    return a;
+}
+
+template <int C>
+__device__ __forceinline__ void store_pixel(const ForwardParams& p, float* img, int lw, int lh, int gx, int gy, const float (&col)[C])
+{
+    // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
+    if (p.layout == TRIPS_LAYOUT_CHW)
+    {
+        const size_t plane = (size_t)lw * lh;
+        float* o           = img + ((size_t)p.view_index * C) * plane;
+        const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
+#pragma unroll
+        for (int c = 0; c < C; ++c) __builtin_nontemporal_store(col[c], (o + c * plane) + at);
+    }
+    else
+    {
+        float* o          = img + ((size_t)p.view_index * lh * lw) * C;
+        const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
+#pragma unroll
+        for (int c = 0; c < C; ++c) __builtin_nontemporal_store(col[c], o + at + c);
+    }
+}
+
+// ---- one list per lane: sorting networks over registers (Batcher's odd-even merge sort; keys are distinct or the
+// all-ones filler) ----
+__device__ __forceinline__ void sort_pair(u64& a, u64& b)
+{
+    const bool sw = b < a;
+    const u64 lo = sw ? b : a, hi = sw ? a : b;
+    a = lo;
+    b = hi;
+}
+__device__ __forceinline__ void lane_sort4(u64 (&k)[kLaneSortMax])
+{
+    sort_pair(k[0], k[1]), sort_pair(k[2], k[3]);
+    sort_pair(k[0], k[2]), sort_pair(k[1], k[3]);
+    sort_pair(k[1], k[2]);
+}
+__device__ __forceinline__ void lane_sort8(u64 (&k)[kLaneSortMax])
+{
+    sort_pair(k[0], k[1]), sort_pair(k[2], k[3]), sort_pair(k[4], k[5]), sort_pair(k[6], k[7]);
+    sort_pair(k[0], k[2]), sort_pair(k[1], k[3]), sort_pair(k[4], k[6]), sort_pair(k[5], k[7]);
+    sort_pair(k[1], k[2]), sort_pair(k[5], k[6]);
+    sort_pair(k[0], k[4]), sort_pair(k[1], k[5]), sort_pair(k[2], k[6]), sort_pair(k[3], k[7]);
+    sort_pair(k[2], k[4]), sort_pair(k[3], k[5]);
+    sort_pair(k[1], k[2]), sort_pair(k[3], k[4]), sort_pair(k[5], k[6]);
+}
+// ascending sort of the first nmax (wave-uniform) of the lane's keys
+__device__ __forceinline__ void lane_sort(u64 (&k)[kLaneSortMax], int nmax)
+{
+    if (nmax > 4)
+        lane_sort8(k);
+    else if (nmax > 2)
+        lane_sort4(k);
+    else if (nmax > 1)
+        sort_pair(k[0], k[1]);
+}
+// largest value of v (0 .. LIMIT) over the wavefront's lanes, as a scalar
+template <int LIMIT>
+__device__ __forceinline__ int wave_max_small(int v)
+{
+    int m = 0;
+#pragma unroll
+    for (int t = 1; t <= LIMIT; ++t)
+        if (__ballot(v >= t)) m = t;
+    return m;
+}
+
+// Sum of a sequence in the order of a balanced binary tree over the positions, (0 + 1) + (2 + 3), ...: push<J>(v) for
+// J = 0, 1, ..., then total(). A skipped tail counts as zeros.
+template <int C, int LEVELS>
+struct TreeSum
+{
+    float acc[LEVELS][C];
+    __device__ __forceinline__ TreeSum()
+    {
+#pragma unroll
+        for (int l = 0; l < LEVELS; ++l)
+#pragma unroll
+            for (int c = 0; c < C; ++c) acc[l][c] = 0.f;
+    }
+    template <int J>
+    __device__ __forceinline__ void push(const float (&v)[C])
+    {
+        float t[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) t[c] = v[c];
+#pragma unroll
+        for (int l = 0; l < LEVELS; ++l)
+        {
+            if ((J >> l) & 1)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c) t[c] = acc[l][c] + t[c], acc[l][c] = 0.f;
+            }
+            else
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c) acc[l][c] = t[c];
+                break;
+            }
+        }
+    }
+    __device__ __forceinline__ void total(float (&out)[C])
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c) out[c] = acc[0][c];
+#pragma unroll
+        for (int l = 1; l < LEVELS; ++l)
+#pragma unroll
+            for (int c = 0; c < C; ++c) out[c] = acc[l][c] + out[c];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------------
 __device__ __forceinline__ u64 shfl16(u64 v, int src)
 {
     unsigned lo = (unsigned)v, hi = (unsigned)(v >> 32);
@@ -872,265 +1048,313 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
     }
 }
 
-// A pixel's list is the union of the lists of the four cells whose 2 x 2 footprints cover it: (x-1, y-1), (x, y-1),
-// (x-1, y), (x, y) (CountAndCollectTiled adds every point to the four pixels of its footprint,
-// RenderForward.cu:300-366; here a point is filed once, under its footprint's first pixel, and the pixels gather).
-// Top-16 of each pixel's union by key, then the alpha blend, for 64 / ROW consecutive pixels starting at `pix_first`:
-// ROW = 16 lanes per pixel (one DPP row; lists of any length stream through in chunks of 16), or ROW = 8 when no
-// pixel of the group has more than 8 entries (two thirds of the pixels of a typical view have at most 4: half the
-// lanes of a 16-lane row would idle through every instruction).
-// First key (negative: a long list, reduced to candidates) and number of readable keys of the four cells of a pixel.
-struct PixelCells
+// Every cell's list in ascending order, in place; of a list longer than kCellKeep its kCellKeep smallest keys, at its
+// start. A wavefront takes 64 consecutive cells (their lists follow each other in the key array), a workgroup a
+// quarter of a tile; the four workgroups of a tile run on the XCD that blends the tile.
+__global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
 {
-    int s0, s1, s2, s3;
-    int r0, r1, r2, r3;
-    int length;  // entries of the four lists (more than the readable keys when a list is long or was cut by the capacity)
-};
+    const int lane = threadIdx.x & 63;
+    const int NB   = p.geom.bin_off[p.num_layers];
+    const long long lblock = xcd_tile_block(blockIdx.x, 4);
+    if (lblock >= (long long)NB * 4) return;
+    const int cell  = ((int)lblock * 4 + (int)(threadIdx.x >> 6)) * 64 + lane;
+    const int4 info = cell_info(p, cell);
+    const int rd    = info.y;
+    u64* const base = cell_keys(p, info.x);
+    // ---- up to kLaneSortMax keys: one cell per lane ----
+    {
+        const int mine = rd <= kLaneSortMax ? rd : 0;
+        const int nmax = wave_max_small<kLaneSortMax>(mine);
+        if (nmax > 1)
+        {
+            u64 k[kLaneSortMax];
+#pragma unroll
+            for (int i = 0; i < kLaneSortMax; ++i)
+            {
+                k[i] = ~0ull;
+                if (i < nmax && i < mine) k[i] = base[i];
+            }
+            lane_sort(k, nmax);
+            if (mine > 1)
+            {
+#pragma unroll
+                for (int i = 0; i < kLaneSortMax; ++i)
+                    if (i < nmax && i < mine) base[i] = k[i];
+            }
+        }
+    }
+    // ---- longer lists: one cell per 16-lane row, four at a time ----
+    u64 todo = __ballot(rd > kLaneSortMax);
+    const int sub = lane & 15, grp = lane >> 4;
+    while (todo)
+    {
+        int src = -1;  // the lane whose cell this row takes
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+        {
+            if (todo)
+            {
+                const int l = (int)__builtin_ctzll(todo);
+                todo &= todo - 1;
+                if (grp == r) src = l;
+            }
+        }
+        const int from      = max(src, 0);
+        const int row_rd    = __shfl(rd, from);  // (by every lane: a source lane may sit in a row that has no cell)
+        const unsigned b_lo = (unsigned)__shfl((int)(unsigned)(uintptr_t)base, from);
+        const unsigned b_hi = (unsigned)__shfl((int)(unsigned)((uintptr_t)base >> 32), from);
+        u64* const row_base = reinterpret_cast<u64*>(((uintptr_t)b_hi << 32) | (uintptr_t)b_lo);
+        const int readable  = src >= 0 ? row_rd : 0;
+        const u64 best      = row_top16([&](int i) { return row_base[i]; }, readable);
+        if (sub < min(readable, kCellKeep)) row_base[sub] = best;
+    }
+}
 
-template <int C, bool TRAIN, int ROW>
-__device__ __forceinline__ void sort_blend_rows(const ForwardParams& p, const TileCtx& tc, float* img, int pix_first,
-                                                bool group_in_range, const PixelCells cells)
+// One pixel per lane, 8 x 8 pixels per wavefront, a quarter of a tile per workgroup (the four of a tile on one XCD).
+template <int C, bool TRAIN>
+__global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
 {
     constexpr int CPAD = (C + 3) & ~3;
     constexpr int RF   = 4 + CPAD;  // floats per blend record
-    const int lane     = threadIdx.x & 63;
-    const int sub      = lane & (ROW - 1);
-    const int grp      = lane / ROW;
-    const int K        = p.list_depth;
-    const int kshift   = K == 16 ? 4 : 3;
-    // the group's pixels lie side by side in one row of the tile
-    const int pix   = group_in_range ? pix_first + grp : 0;
-    const int layer = tc.layer, lw = tc.w, lh = tc.h;
-    const int gx = tc.x0 + (pix & (kTile - 1)), gy = tc.y0 + ((pix >> kTileShift) & (kTile - 1));
-    const bool in_range = group_in_range;
-    const bool live     = in_range && gx < lw && gy < lh;  // false for the padding of partial tiles
-
-    // position i of the concatenation of the four cell lists lies in cell (i >= o1) + (i >= o2) + (i >= o3)
-    const int o1 = cells.r0, o2 = o1 + cells.r1, o3 = o2 + cells.r2;
-    const int total = live ? o3 + cells.r3 : 0;
-
-    const u64 kInf = ~0ull;
-    u64 best       = kInf;
-    if (ROW <= 8)
+    constexpr int NQ   = CPAD / 4;
+    constexpr int BATCH = CPAD <= 8 ? 8 : 4;  // list positions whose records are requested together
+    __shared__ int4 s_cells[4][81];
+    __shared__ u64 s_keys[4][81 * kStagedKeys];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int NB   = p.geom.bin_off[p.num_layers];
+    const long long lblock = xcd_tile_block(blockIdx.x, 4);
+    if (lblock >= (long long)NB * 4) return;
+    const int bin = (int)(lblock >> 2), quarter = (int)(lblock & 3);
+    const TileCtx tc = tile_ctx(p.geom, bin);
+    const int bx = ((quarter & 1) << 4) + ((wave & 1) << 3), by = ((quarter >> 1) << 4) + ((wave >> 1) << 3);
+    const int lx = lane & 7, ly = lane >> 3;
+    const int pix = (bin << (2 * kTileShift)) | ((by + ly) << kTileShift) | (bx + lx);
+    const int gx = tc.x0 + bx + lx, gy = tc.y0 + by + ly;
+    const bool live = gx < tc.w && gy < tc.h;  // false for the padding of partial tiles
+    if (tc.x0 + bx >= tc.w || tc.y0 + by >= tc.h)
     {
-        // at most ROW keys: none of the cells has a long list
-        // (sums of steps rather than a chain of selects: the compiler turns the chain into a table in memory)
-        const int b0 = cells.s0, b1 = cells.s1 - o1, b2 = cells.s2 - o2, b3 = cells.s3 - o3;
-        const int base = b0 + (sub >= o1 ? b1 - b0 : 0) + (sub >= o2 ? b2 - b1 : 0) + (sub >= o3 ? b3 - b2 : 0);
-        if (sub < total) best = p.keys[(unsigned)(base + sub)];
-        best = ROW == 8 ? half_sort8(best) : quad_sort4(best);
-    }
-    else
-    {
-        // the candidates that the reduction pass left for long lists are addressed relative to the keys as well
-        const long long cand_off = ((long long)(intptr_t)p.cand - (long long)(intptr_t)p.keys) / (long long)sizeof(u64);
-        auto first_key = [&](int s) -> long long { return s >= 0 ? (long long)s : cand_off + (long long)(-1 - s) * 16; };
-        const long long b0 = first_key(cells.s0), b1 = first_key(cells.s1) - o1, b2 = first_key(cells.s2) - o2,
-                        b3 = first_key(cells.s3) - o3;
-        const long long d1 = b1 - b0, d2 = b2 - b1, d3 = b3 - b2;
-        best = row_top16(
-            [&](int i)
-            {
-                const long long b = b0 + (i >= o1 ? d1 : 0ll) + (i >= o2 ? d2 : 0ll) + (i >= o3 ? d3 : 0ll);
-                return p.keys[b + i];
-            },
-            total);
+        // a block of padding: its rows of the saved tables are defined as empty
+        if (TRAIN) __builtin_nontemporal_store(0, p.retained + pix);
+        return;
     }
 
-    // ---- blend (RenderForward.cu:820-1048) ----
-    const int n    = min(total, K);
-    const bool has = live && sub < n;
-    const int cid  = (int)(unsigned)(best & 0xffffffffull);  // compact number of the entry's point
-
-    float a = 0.f;
-    int slot = 0;  // which of the point's (layer, footprint corner) pixels this one is
-    float desc[CPAD];
-#pragma unroll
-    for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
-    if (has)
+    // The block gathers from the 9 x 9 cells (gx0 - 1 .. gx0 + 7) x (gy0 - 1 .. gy0 + 7): one cell per lane, then
+    // the 17 that are left; a pixel takes its four from LDS.
     {
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
-        const float4 r0   = rec[0];
+        const int i1 = lane, i2 = 64 + lane;
+        s_cells[wave][i1] = load_cell(p, tc, tc.x0 + bx - 1 + i1 % 9, tc.y0 + by - 1 + i1 / 9);
+        if (i2 < 81) s_cells[wave][i2] = load_cell(p, tc, tc.x0 + bx - 1 + i2 % 9, tc.y0 + by - 1 + i2 / 9);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int ci0 = ly * 9 + lx;  // the pixel's cells: ci0, ci0 + 1, ci0 + 9, ci0 + 10
+    const int4 c0 = s_cells[wave][ci0], c1 = s_cells[wave][ci0 + 1], c2 = s_cells[wave][ci0 + 9], c3 = s_cells[wave][ci0 + 10];
+    const int total  = live ? c0.y + c1.y + c2.y + c3.y : 0;  // keys to choose from (each cell's cut to kCellKeep)
+    const int length = c0.z + c1.z + c2.z + c3.z;             // entries (0 for padding: its cells are empty)
+    const int n      = min(total, p.list_depth);              // list positions that hold an entry
+    const bool merges = total > kLaneSortMax;
+
+    unsigned id[16];  // compact numbers of the pixel's entries, nearest first
 #pragma unroll
-        for (int q = 0; q < CPAD / 4; ++q)
+    for (int j = 0; j < 16; ++j) id[j] = ~0u;
+
+    // ---- up to kLaneSortMax keys: load them all, sort with a network ----
+    {
+        const int mine = merges ? 0 : total;
+        const int nmax = wave_max_small<kLaneSortMax>(mine);
+        if (nmax > 0)
         {
-            const float4 t  = rec[1 + q];
-            desc[4 * q]     = t.x;
-            desc[4 * q + 1] = t.y;
-            desc[4 * q + 2] = t.z;
-            desc[4 * q + 3] = t.w;
+            // position i of the concatenation of the four cell lists lies in cell (i >= o1) + (i >= o2) + (i >= o3)
+            // (sums of steps rather than a chain of selects: the compiler turns the chain into a table in memory);
+            // none of these cells has a long list
+            u64 k[kLaneSortMax];
+            const int o1 = c0.y, o2 = o1 + c1.y, o3 = o2 + c2.y;
+            const int b0 = c0.x, b1 = c1.x - o1, b2 = c2.x - o2, b3 = c3.x - o3;
+#pragma unroll
+            for (int i = 0; i < kLaneSortMax; ++i)
+            {
+                k[i] = ~0ull;
+                if (i < nmax)
+                {
+                    const int base = b0 + (i >= o1 ? b1 - b0 : 0) + (i >= o2 ? b2 - b1 : 0) + (i >= o3 ? b3 - b2 : 0);
+                    if (i < mine) k[i] = p.keys[(unsigned)(base + i)];
+                }
+            }
+            lane_sort(k, nmax);
+#pragma unroll
+            for (int i = 0; i < kLaneSortMax; ++i)
+                if (i < mine) id[i] = (unsigned)k[i];
         }
-        const float m  = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
-        const float ux = r0.x * m, uy = r0.y * m;
-        float w        = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
-        if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
-        a = w * r0.w;
-        a *= layer_factor_encoded(r0.z, layer, p.num_layers);
-        const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
-        slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
+    }
+    // ---- more: merge the four sorted cell lists. The first kStagedKeys keys of the block's cells wait in LDS; a
+    // lane that needs more of one cell reads them from memory. ----
+    const u64 merging = __ballot(merges);
+    if (merging)
+    {
+        // slot s = cell (s / kStagedKeys), key (s % kStagedKeys): kStagedKeys lanes read consecutive keys of a cell
+        static_assert(kStagedKeys == 8, "the slot arithmetic below");
+#pragma unroll 1
+        for (int s0 = 0; s0 < 81 * kStagedKeys; s0 += 64)
+        {
+            const int s = s0 + lane;
+            if (s < 81 * kStagedKeys)
+            {
+                const int4 c = s_cells[wave][s >> 3];
+                if ((s & 7) < c.y) s_keys[wave][s] = cell_keys(p, c.x)[s & 7];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (merges)
+        {
+            const u64 kInf = ~0ull;
+            // key q of one of the pixel's cells (all-ones past its end)
+            auto key_of = [&](int ci, const int4& c, int q) -> u64
+            {
+                u64 v = kInf;
+                if (q < c.y) v = q < kStagedKeys ? s_keys[wave][ci * kStagedKeys + q] : cell_keys(p, c.x)[q];
+                return v;
+            };
+            u64 h0 = key_of(ci0, c0, 0), h1 = key_of(ci0 + 1, c1, 0), h2 = key_of(ci0 + 9, c2, 0), h3 = key_of(ci0 + 10, c3, 0);
+            int q0 = 0, q1 = 0, q2 = 0, q3 = 0;  // heads of the four lists
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+            {
+                if (j < n)
+                {
+                    const bool b01 = h1 < h0, b23 = h3 < h2;
+                    const u64 m01 = b01 ? h1 : h0, m23 = b23 ? h3 : h2;
+                    const bool hi = m23 < m01;
+                    id[j]         = (unsigned)(hi ? m23 : m01);
+                    const int w   = hi ? (b23 ? 3 : 2) : (b01 ? 1 : 0);  // the list that gave the key
+                    q0 += w == 0, q1 += w == 1, q2 += w == 2, q3 += w == 3;
+                    if (j + 1 < n)
+                    {
+                        const int ci   = ci0 + (w & 1) + 9 * (w >> 1);
+                        const int4 c   = w == 0 ? c0 : w == 1 ? c1 : w == 2 ? c2 : c3;
+                        const int q    = w == 0 ? q0 : w == 1 ? q1 : w == 2 ? q2 : q3;
+                        const u64 next = key_of(ci, c, q);
+                        h0 = w == 0 ? next : h0, h1 = w == 1 ? next : h1, h2 = w == 2 ? next : h2, h3 = w == 3 ? next : h3;
+                    }
+                }
+            }
+        }
     }
 
-    // exclusive transmittance: lane j latches prod_{k<j} (1 - a_k), built left to right
-    // only the first n positions of a row matter; n <= K
-    int nmax = n;
-    if (ROW == 4) nmax = max(nmax, __shfl_xor(nmax, 4));
-    if (ROW <= 8) nmax = max(nmax, __shfl_xor(nmax, 8));
-    nmax     = max(nmax, __shfl_xor(nmax, 16));
-    nmax     = max(nmax, __shfl_xor(nmax, 32));
-    nmax     = __builtin_amdgcn_readfirstlane(nmax);
-    const float T     = ROW == 4   ? quad_exclusive_product(1.f - a, nmax)
-                        : ROW == 8 ? half_exclusive_product(1.f - a, nmax)
-                                   : row_exclusive_product(1.f - a, nmax);
-    const float Tc    = (T >= kAlphaDestCutoff) ? T : 0.f;
-    const bool kept   = has && Tc >= kAlphaDestCutoff;
-    const unsigned kb = (unsigned)((__ballot(kept) >> (grp * ROW)) & ((1u << ROW) - 1u));
-    const int ret     = __ffs(~kb) - 1;  // length of the leading run of kept entries (kb has at most ROW bits)
+    // ---- blend (RenderForward.cu:820-1048), front to back ----
+    const int nmax = wave_max_small<16>(n);  // longest list of the block
+    TreeSum<C, 5> sum;  // (five levels: up to 16 positions)
+    float T       = 1.f;
+    float bgw     = 1.f;  // empty list -> 1
+    int ret       = 0;    // length of the leading run of kept entries
+    bool run_open = true;
+    float4 r0[BATCH], rd[BATCH][NQ];
+    // one list position, its number a compile-time constant (the arrays indexed by it stay in registers)
+    auto position = [&](auto jc)
+    {
+        constexpr int j = decltype(jc)::value;
+        constexpr int b = j % BATCH;
+        const bool has  = j < n;
+        int slot        = 0;
+        float a         = 0.f;
+        if (has) a = entry_alpha(r0[b], tc.layer, p.num_layers, gx, gy, slot);
+        const float Tc  = (T >= kAlphaDestCutoff) ? T : 0.f;
+        const bool kept = has && Tc >= kAlphaDestCutoff;
+        run_open        = run_open && kept;
+        if (run_open) ret = j + 1;
+        const float wgt = has ? Tc * a : 0.f;
+        float pr[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            const float4 t = rd[b][c / 4];
+            const float d  = (c & 3) == 0 ? t.x : (c & 3) == 1 ? t.y : (c & 3) == 2 ? t.z : t.w;
+            pr[c]          = has ? wgt * d : 0.f;
+        }
+        sum.template push<j>(pr);
+        // background weight (RenderForward.cu:1002-1022): taken at the last list position
+        if (j == n - 1) bgw = (p.background_mode == TRIPS_BG_REFERENCE) ? Tc : T * (1.f - a);
+        // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
+        // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
+#ifndef EXP_NORANK
+        if (TRAIN && run_open)
+            p.rank[(tc.layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)id[j] << 4) + slot] = (unsigned char)j;
+#endif
+        T = T * (1.f - a);
+    };
+    // the records of BATCH positions are requested together, then the positions are walked
+    auto batch = [&](auto first)
+    {
+        constexpr int j0 = decltype(first)::value;
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b)
+        {
+            r0[b] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) rd[b][q] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (j0 + b < nmax && j0 + b < n)
+            {
+                const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)id[j0 + b] * RF);
+                r0[b]             = rec[0];
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) rd[b][q] = rec[1 + q];
+            }
+        }
+        if (j0 + 0 < nmax) position(std::integral_constant<int, j0 + 0>{});
+        if (j0 + 1 < nmax) position(std::integral_constant<int, j0 + 1>{});
+        if (j0 + 2 < nmax) position(std::integral_constant<int, j0 + 2>{});
+        if (j0 + 3 < nmax) position(std::integral_constant<int, j0 + 3>{});
+        if constexpr (BATCH > 4)
+        {
+            if (j0 + 4 < nmax) position(std::integral_constant<int, j0 + 4>{});
+            if (j0 + 5 < nmax) position(std::integral_constant<int, j0 + 5>{});
+            if (j0 + 6 < nmax) position(std::integral_constant<int, j0 + 6>{});
+            if (j0 + 7 < nmax) position(std::integral_constant<int, j0 + 7>{});
+        }
+    };
+    if (nmax > 0) batch(std::integral_constant<int, 0>{});
+    if constexpr (BATCH == 4)
+    {
+        if (nmax > 4) batch(std::integral_constant<int, 4>{});
+        if (nmax > 8) batch(std::integral_constant<int, 8>{});
+        if (nmax > 12) batch(std::integral_constant<int, 12>{});
+    }
+    else if (nmax > 8)
+        batch(std::integral_constant<int, 8>{});
 
     float col[C];
-    const float wgt = has ? Tc * a : 0.f;
-#pragma unroll
-    for (int c = 0; c < C; ++c) col[c] = wgt * desc[c];
-#pragma unroll
-    for (int c = 0; c < C; ++c) col[c] = ROW == 4 ? quad_sum_to_lane0(col[c]) : ROW == 8 ? half_sum_to_lane0(col[c]) : row_sum_to_lane0(col[c]);
-
-    // background weight (RenderForward.cu:1002-1022); empty list -> 1
-    float bgw_lane = (p.background_mode == TRIPS_BG_REFERENCE) ? Tc : T * (1.f - a);
-    float bgw      = __shfl(bgw_lane, max(n - 1, 0), ROW);
-    if (n == 0) bgw = 1.f;
-
-    if (live && sub == 0)
+    sum.total(col);
+    if (live)
     {
         if (bgw >= kAlphaDestCutoff)
         {
 #pragma unroll
             for (int c = 0; c < C; ++c) col[c] += p.background[c] * (bgw * 1.f);
         }
-        // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
-        if (p.layout == TRIPS_LAYOUT_CHW)
-        {
-            const size_t plane = (size_t)lw * lh;
-            float* o           = img + ((size_t)p.view_index * C) * plane;
-            const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
-#pragma unroll
-            for (int c = 0; c < C; ++c) __builtin_nontemporal_store(col[c], (o + c * plane) + at);
-        }
-        else
-        {
-            float* o          = img + ((size_t)p.view_index * lh * lw) * C;
-            const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
-#pragma unroll
-            for (int c = 0; c < C; ++c) __builtin_nontemporal_store(col[c], o + at + c);
-        }
+        store_pixel<C>(p, p.image[tc.layer], tc.w, tc.h, gx, gy, col);
     }
     // saved state, also for padding pixels (empty) so that every row of the tables is defined
-    if (TRAIN && in_range)
+    if (TRAIN)
     {
         // (bits 0..4: retained entries; bits 5..9: list positions that hold an id. Only those are stored below: the
         // backward reads the retained ones, the export fills the rest of a row with -1 itself. Bits 10..31: length of
         // the pixel's list before the cut to K, for the export; saturates.)
-        if (sub == 0)
-            __builtin_nontemporal_store(live ? (int)((unsigned)ret | ((unsigned)n << kRetainedBits) |
-                                                     ((unsigned)min(cells.length, kMaxExportedLength) << (2 * kRetainedBits)))
-                                             : 0,
-                                        p.retained + pix);
-        // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
-        // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
-        if (has && sub < ret)
-            p.rank[(layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)(unsigned)cid << 4) + slot] = (unsigned char)sub;
-        const int mine = has ? cid : -1;
-        if (ROW == 4)
-        {
-            // one 16-byte store: lane 0 of the quad carries the four ids
-            const int i0 = __shfl(mine, 0, 4), i1 = __shfl(mine, 1, 4), i2 = __shfl(mine, 2, 4), i3 = __shfl(mine, 3, 4);
-            if (4 * sub < n)
-                __builtin_nontemporal_store(sub == 0 ? vi4{i0, i1, i2, i3} : vi4{-1, -1, -1, -1},
-                                            reinterpret_cast<vi4*>(p.lists + (((size_t)(unsigned)pix << kshift) + 4 * sub)));
-        }
-        else if (ROW == 8)
-        {
-            // 8-byte stores: lanes 0..3 carry the ids of lane pairs
-            const int lo = __shfl(mine, (2 * sub) & 7, 8), hi = __shfl(mine, (2 * sub + 1) & 7, 8);
-            if (2 * sub < n) __builtin_nontemporal_store(sub < 4 ? (long long)(unsigned)lo | ((long long)hi << 32) : -1ll, reinterpret_cast<long long*>(p.lists + (((size_t)(unsigned)pix << kshift) + 2 * sub)));
-        }
-        else if (sub < n)
-            __builtin_nontemporal_store(mine, p.lists + (((size_t)(unsigned)pix << kshift) + sub));
+        __builtin_nontemporal_store(live ? (int)((unsigned)ret | ((unsigned)n << kRetainedBits) |
+                                                 ((unsigned)min(length, kMaxExportedLength) << (2 * kRetainedBits)))
+                                         : 0,
+                                    p.retained + pix);
+        const int kshift = p.list_depth == 16 ? 4 : 3;
+        vi4* row         = reinterpret_cast<vi4*>(p.lists + ((size_t)(unsigned)pix << kshift));
+#ifndef EXP_NOLISTS
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (4 * q < n) __builtin_nontemporal_store(vi4{(int)id[4 * q], (int)id[4 * q + 1], (int)id[4 * q + 2], (int)id[4 * q + 3]}, row + q);
+#endif
     }
 }
-
-// One wavefront = eight consecutive pixels: all at once in 8-lane rows when none of them has more than 8 entries,
-// else four and four in 16-lane rows; sixteen pixels in 4-lane rows when none of the sixteen of a pair of wavefronts
-// has more than 4.
-template <int C, bool TRAIN>
-__global__ __launch_bounds__(256) void sort_blend_kernel(const ForwardParams p)
-{
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int NB   = p.geom.bin_off[p.num_layers];
-    const long long nblocks     = (long long)NB * (kTilePixels / 32);  // 32 pixels per workgroup, 32 workgroups per tile
-    const long long lblock      = xcd_tile_block(blockIdx.x, kTilePixels / 32);
-    const bool group_in_range   = lblock < nblocks;
-    const int pix_first         = group_in_range ? ((int)lblock * 4 + wave) * 8 : 0;
-    // the eight pixels share a tile: its layer and position are found once per wavefront, on the scalar unit
-    const TileCtx tc = tile_ctx(p.geom, pix_first >> (2 * kTileShift));
-    float* const img = p.image[tc.layer];
-    // Two wavefronts share a run of 16 pixels (gx0 .. gx0 + 15, gy), which gather from the cells (gx0 - 1 .. gx0 + 15)
-    // x (gy - 1, gy): lanes 0..16 read length and first key of the upper row of cells, lanes 17..33 those of the lower
-    // row; pixel j of the run takes the cells of lanes j, j + 1, j + 17, j + 18. Cells outside the layer, and the last
-    // row and column (no footprint starts there), are empty. Both wavefronts read all 34 cells: when none of the 16
-    // pixels has more than 4 entries the first one takes all of them in rows of 4 lanes and the second one ends.
-    const int half       = wave & 1;
-    const int pair_first = pix_first - 8 * half;
-    int c_len = 0, c_start = 0, c_read = 0;
-    if (lane < 34 && group_in_range)
-    {
-        const int lower = lane >= 17 ? 1 : 0;
-        const int cx    = tc.x0 + (pair_first & (kTile - 1)) - 1 + (lane - 17 * lower);
-        const int cy    = tc.y0 + ((pair_first >> kTileShift) & (kTile - 1)) - 1 + lower;
-        if (cx >= 0 && cy >= 0 && cx < tc.w - 1 && cy < tc.h - 1)
-        {
-            const int bin  = tc.bin + ((cx - tc.x0) >> kTileShift) + ((cy - tc.y0) >> kTileShift) * tc.tiles_x;  // shifts round down
-            const int cell = (bin << (2 * kTileShift)) | ((cy & (kTile - 1)) << kTileShift) | (cx & (kTile - 1));
-            c_len          = p.counts[cell];
-            c_start        = p.cursor[cell];  // negative: a long list, reduced to candidates by long_list_reduce_kernel
-            // keys actually there: the key storage may have ended inside the list
-            if (c_start < 0)
-                c_read = ((c_len + kLongSegment - 1) / kLongSegment) * 16;
-            else
-                c_read = (int)max(0ll, min((long long)c_len, p.capacity - c_start));
-        }
-    }
-    // lane j < 16: readable keys of pixel j of the run
-    int tot = c_read + __shfl_down(c_read, 1) + __shfl_down(c_read, 17) + __shfl_down(c_read, 18);
-    // lane j < 16: entries of pixel j's lists (0 for the padding of partial tiles)
-    const int len = TRAIN ? c_len + __shfl_down(c_len, 1) + __shfl_down(c_len, 17) + __shfl_down(c_len, 18) : 0;
-    if (lane >= 16) tot = 0;
-    tot = max(tot, __shfl_xor(tot, 1));
-    tot = max(tot, __shfl_xor(tot, 2));
-    tot = max(tot, __shfl_xor(tot, 4));
-    const int tot8  = __builtin_amdgcn_readlane(tot, 8 * half);  // longest list of this wavefront's eight pixels
-    const int tot16 = max(__builtin_amdgcn_readlane(tot, 0), __builtin_amdgcn_readlane(tot, 8));
-    // the rows take their cells' list starts and lengths from these lanes: no second memory round trip
-    auto cells_of = [&](int j)  // pixel j of the run
-    {
-        PixelCells c;
-        c.s0 = __shfl(c_start, j), c.s1 = __shfl(c_start, j + 1), c.s2 = __shfl(c_start, j + 17), c.s3 = __shfl(c_start, j + 18);
-        c.r0 = __shfl(c_read, j), c.r1 = __shfl(c_read, j + 1), c.r2 = __shfl(c_read, j + 17), c.r3 = __shfl(c_read, j + 18);
-        c.length = TRAIN ? __shfl(len, j) : 0;
-        return c;
-    };
-    if (tot16 <= 4)
-    {
-        if (half == 0) sort_blend_rows<C, TRAIN, 4>(p, tc, img, pair_first, group_in_range, cells_of(lane >> 2));
-    }
-    else if (tot8 <= 8)
-        sort_blend_rows<C, TRAIN, 8>(p, tc, img, pix_first, group_in_range, cells_of(8 * half + (lane >> 3)));
-    else
-    {
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first, group_in_range, cells_of(8 * half + (lane >> 4)));
-        sort_blend_rows<C, TRAIN, 16>(p, tc, img, pix_first + 4, group_in_range, cells_of(8 * half + 4 + (lane >> 4)));
-    }
-}
-
 
 // ---------------------------------------------------------------------------------------------------------
 // host-side launchers
@@ -1210,17 +1434,21 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         const int blocks = std::min((p.max_long_items + 15) / 16, 2048);
         hipLaunchKernelGGL(long_list_reduce_kernel, dim3(blocks), dim3(256), 0, stream, p);
     }
+    const long long tiles8 = (((long long)NB + kNumXcd - 1) / kNumXcd) * kNumXcd;  // tiles rounded up to 8
+    const int quarter_tiles = (int)(tiles8 * 4);                                   // a quarter tile per workgroup
     {
-        ProfScope ps(prof, "sort_blend", stream);
-        const long long tiles8 = (((long long)NB + kNumXcd - 1) / kNumXcd) * kNumXcd;  // tiles rounded up to 8
-        int blocks             = (int)(tiles8 * (kTilePixels / 32));
+        ProfScope ps(prof, "cell_sort", stream);
+        hipLaunchKernelGGL(cell_sort_kernel, dim3(quarter_tiles), dim3(256), 0, stream, p);
+    }
+    {
+        ProfScope ps(prof, "blend", stream);
         if (train)
         {
-            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((sort_blend_kernel<CC, true>), dim3(blocks), dim3(256), 0, stream, p));
+            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((blend_kernel<CC, true>), dim3(quarter_tiles), dim3(256), 0, stream, p));
         }
         else
         {
-            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((sort_blend_kernel<CC, false>), dim3(blocks), dim3(256), 0, stream, p));
+            TRIPS_DISPATCH_C(channels, hipLaunchKernelGGL((blend_kernel<CC, false>), dim3(quarter_tiles), dim3(256), 0, stream, p));
         }
     }
     return hipGetLastError();
