@@ -1,27 +1,33 @@
 // Backward kernels of the splat path for gfx950 (wave64).
 //
-//   backward_pixels_kernel + backward_points_kernel <- BlendBackwardsBilinearTiled
-//                                                      src/lib/rendering/RenderBackward.cu:90-618
+//   backward_tiles_kernel + backward_points_kernel <- BlendBackwardsBilinearTiled
+//                                                     src/lib/rendering/RenderBackward.cu:90-618
 //
 // The reference walks one pixel list per thread and scatters every entry's gradient with float atomics
-// (3 position + 1 size + 1 confidence + C descriptor atomics per retained entry). Scattered atomics run at
-// about 2e10 per second on this GPU while scattered loads run at 5e10 and cost the same for 4 or 64 bytes,
-// so the work is split in two passes without atomics on the per-point arrays:
-//   1. pixels: a 16-lane row (an 8-lane half row for short lists) owns a pixel, each lane one retained entry. Alpha and transmittance are recomputed
-//      from the per-point record exactly as the forward computed them; the "all later entries" sum of
-//      RenderBackward.cu:284-301 is a suffix sum across the row. Per entry it writes {dL/dalpha, T*alpha*dL/dimage}
-//      into the pixel's row of a [P,K] table. The forward's blend kernel has left one byte per retained entry, its
-//      rank in the pixel's list, in the point's 32-slot table (slot = layer * 4 + footprint corner; two planes of 16
-//      slots per point, layers 0..3 and 4..7).
-//   2. points: one thread per point walks its slots, gathers those records (one aligned load each), sums the image-space gradient of all its entries and runs the projection chain ONCE
-//      (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then adds its gradients
-//      with plain read-modify-writes. Pose / intrinsics partials stay in double registers over a grid-stride
-//      loop before one block-level reduction and one atomic per value and block (the reference keeps them in
-//      shared double arrays, :160-187,546-617).
-// Gradients are therefore summed in a fixed order and are bit-reproducible from run to run.
+// (3 position + 1 size + 1 confidence + C descriptor atomics per retained entry). Scattered atomics run at about
+// 2e10 per second on this GPU, and what bounds the kernels of this path is the number of scattered memory requests,
+// whatever their size. So the four pixels of a point's footprint meet in LDS, not in memory:
+//   1. tiles: a workgroup owns 16 x 16 cells of a tile (a cell = the footprints that start at that pixel) and walks
+//      the 17 x 17 pixels they cover, one pixel per lane (its right column and bottom row are walked again by the
+//      neighbours). A lane recomputes alpha and transmittance of its pixel's retained entries from the per-point
+//      record exactly as the forward computed them, forms dL/dalpha (the "all later entries" sum of
+//      RenderBackward.cu:284-301 is a running sum from the back of the list) and leaves {dL/dalpha, T alpha} of every
+//      entry in LDS, together with the entry's rank under the (cell, place in the cell's list) that the forward noted
+//      for it. Then a lane per cell collects, for each of the cell's points, the four corner pixels' entries and
+//      writes ONE row per (point, layer) pair: sum over the corners of T alpha dL/dimage and the four dL/dalpha.
+//   2. points: one thread per point reads the rows of its pairs (consecutive in memory, numbered in point order),
+//      evaluates the bilinear weights' Jacobian and the layer factor per corner (PointBlending.h:216-264,
+//      RenderBackward.cu:366-438), sums the image-space gradient of all its entries and runs the projection chain
+//      ONCE (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then stores or adds its
+//      gradients. Pose / intrinsics partials stay in registers over a grid-stride loop before one block-level
+//      reduction and one atomic per value and block (the reference keeps them in shared double arrays,
+//      :160-187,546-617).
+// Gradients are summed in a fixed order and are bit-reproducible from run to run.
 #include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"
+
+#include <type_traits>
 
 #pragma clang fp contract(off)
 
@@ -58,8 +64,9 @@ __device__ __forceinline__ Camera load_camera_bw(const double* pose, const float
     return c;
 }
 
-typedef float vf2 __attribute__((ext_vector_type(2)));
 typedef float vf4 __attribute__((ext_vector_type(4)));
+typedef int vi4 __attribute__((ext_vector_type(4)));
+typedef unsigned vu4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ double wave_sum(double v)
 {
@@ -67,205 +74,261 @@ __device__ __forceinline__ double wave_sum(double v)
     return v;
 }
 
-
-// ---------------------------------------------------------------------------------------------------------
-// Pass 1: per pixel row. Writes the pixel's exchange row {g[0..Cpad), {dL/dalpha_j, T_j alpha_j} for j < entry_row_entries}.
-// 64 / ROW consecutive pixels starting at pix_first: ROW = 16 lanes per pixel, or 8 when none of them retained more
-// than 8 entries. m_in = retained entries of this lane's pixel (the caller has them already).
-template <int C, int ROW, bool SECOND>
-__device__ __forceinline__ void backward_pixel_rows(const BackwardParams& p, const TileCtx& tc, const float* gi, int pix_first,
-                                                    int m_in, float (&acc_bg)[C])
+// largest value of v (0 .. LIMIT) over the wavefront's lanes, as a scalar
+template <int LIMIT>
+__device__ __forceinline__ int wave_max_small(int v)
 {
-    constexpr int CPAD = (C + 3) & ~3;
-    constexpr int RF   = 4 + CPAD;          // floats per blend record
-    const int lane     = threadIdx.x & 63;
-    const int sub      = lane & (ROW - 1);
-    const int grp      = lane / ROW;
-    const int kshift   = p.list_depth == 16 ? 4 : 3;
-    // the group's pixels lie side by side in one row of the tile
-    const int pix   = pix_first + grp;
-    const int layer = tc.layer, lw = tc.w, lh = tc.h;
-    const int gx = tc.x0 + (pix & (kTile - 1)), gy = tc.y0 + ((pix >> kTileShift) & (kTile - 1));
-    const bool live = gx < lw && gy < lh;  // false for the padding of partial tiles
-
-    const int m    = live ? m_in : 0;
-    const bool has = sub < m;
-    int mmax       = m;
-    if (ROW == 8) mmax = max(mmax, __shfl_xor(mmax, 8));
-    mmax           = max(mmax, __shfl_xor(mmax, 16));
-    mmax           = max(mmax, __shfl_xor(mmax, 32));
-    mmax           = __builtin_amdgcn_readfirstlane(mmax);
-
-    float g[C];
-    {
-        // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
-        if (p.layout == TRIPS_LAYOUT_CHW)
-        {
-            const size_t plane = (size_t)lw * lh;
-            const float* o     = gi + ((size_t)p.view_index * C) * plane;
-            const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
+    int m = 0;
 #pragma unroll
-            for (int c = 0; c < C; ++c) g[c] = live ? (o + c * plane)[at] : 0.f;
-        }
-        else
-        {
-            const float* o    = gi + ((size_t)p.view_index * lh * lw) * C;
-            const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
-#pragma unroll
-            for (int c = 0; c < C; ++c) g[c] = live ? o[at + c] : 0.f;
-        }
-    }
-
-    int cid = 0;  // compact number of the entry's point
-    float desc[CPAD];
-#pragma unroll
-    for (int c = 0; c < CPAD; ++c) desc[c] = 0.f;
-    float a = 0.f;
-    if (has)
-    {
-        cid               = __builtin_nontemporal_load(p.lists + (((size_t)(unsigned)pix << kshift) + sub));
-        const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
-        const float4 r0   = rec[0];
-#pragma unroll
-        for (int q = 0; q < CPAD / 4; ++q)
-        {
-            const float4 t  = rec[1 + q];
-            desc[4 * q]     = t.x;
-            desc[4 * q + 1] = t.y;
-            desc[4 * q + 2] = t.z;
-            desc[4 * q + 3] = t.w;
-        }
-        const float mfac = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
-        const float ux = r0.x * mfac, uy = r0.y * mfac;
-        float w = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
-        if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
-        a = w * r0.w;
-        a *= layer_factor_encoded(r0.z, layer, p.num_layers);
-    }
-
-    // exclusive transmittance, same chain as the forward
-    const float T = ROW == 8 ? half_exclusive_product(1.f - a, mmax) : row_exclusive_product(1.f - a, mmax);
-    // transmittance after the m retained entries decides whether the background is reached
-    // (RenderBackward.cu:205-210,302-308)
-    float T_after = T * (1.f - a);
-    T_after       = __shfl(T_after, max(m - 1, 0), ROW);
-    if (m == 0) T_after = 1.f;
-    const bool bg_reached = live && (T_after >= 0.001f);
-
-    float s = 0.f, sbg = 0.f;
-#pragma unroll
-    for (int c = 0; c < C; ++c)
-    {
-        s += desc[c] * g[c];
-        sbg += p.background[c] * g[c];
-    }
-    const float ta = T * a;
-    const float q  = has ? ta * s : 0.f;
-    float later    = ROW == 8 ? half_exclusive_suffix_sum(q) : row_exclusive_suffix_sum(q);  // entries i > j
-    if (bg_reached) later += T_after * sbg;
-    const float dem        = 1.f / (1.f - a + 1e-9f);
-    const float grad_alpha = T * s - later * dem;
-
-    if (bg_reached && sub == 0)
-    {
-#pragma unroll
-        for (int c = 0; c < C; ++c) acc_bg[c] += T_after * g[c];
-    }
-    // For pass 2, one row of 64 bytes (128 above 8 channels) per pixel: the pixel's image gradient (a point finds all
-    // channels and its entry in one line) followed by {dL/dalpha, T alpha} of the first entry_row_entries retained
-    // entries; the entries beyond that go to a table of their own.
-    // Rows of 64 bytes are written a second time, one row further on (see BackwardParams).
-    constexpr int KIN       = entry_row_entries(CPAD);
-    constexpr bool kShifted = entry_row_floats(CPAD) == 16;
-    float* row              = p.entry_grad + (size_t)(unsigned)pix * entry_row_floats(CPAD);
-    constexpr bool second   = kShifted && SECOND;
-    float* row2             = kShifted ? p.entry_grad_shifted + (size_t)(unsigned)pix * 16 : nullptr;
-    if (has && sub >= KIN)
-        __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(p.entry_over) + ((size_t)(unsigned)pix * (16 - KIN) + (sub - KIN)));
-    if (CPAD == 4)
-    {
-        // the whole row with one store instruction, 8 bytes per lane: lanes 0 and 1 the image gradient, lanes 2..7 the
-        // entries of lanes 0..5 (64 contiguous bytes per pixel instead of a 16-byte and six 8-byte pieces)
-        const float ga_before = row_shr<2>(grad_alpha, 0.f), ta_before = row_shr<2>(ta, 0.f);
-        const float g2 = C > 2 ? g[C > 2 ? 2 : 0] : 0.f, g3 = C > 3 ? g[C > 3 ? 3 : 0] : 0.f;
-        const vf2 v      = sub == 0 ? vf2{g[0], g[1]} : sub == 1 ? vf2{g2, g3} : vf2{ga_before, ta_before};
-        const bool store = sub < 2 ? m > 0 : (sub < 8 && sub - 2 < m);
-        if (store)
-        {
-            __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row) + sub);
-            if (second) __builtin_nontemporal_store(v, reinterpret_cast<vf2*>(row2) + sub);
-        }
-    }
-    else
-    {
-        if (has && sub < KIN)
-        {
-            __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row + CPAD) + sub);
-            if (second) __builtin_nontemporal_store(vf2{grad_alpha, ta}, reinterpret_cast<vf2*>(row2 + CPAD) + sub);
-        }
-        if (sub == 0 && m > 0)
-        {
-            float gp[CPAD];
-#pragma unroll
-            for (int c = 0; c < CPAD; ++c) gp[c] = c < C ? g[c] : 0.f;
-#pragma unroll
-            for (int q = 0; q < CPAD / 4; ++q)
-            {
-                __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row) + q);
-                if (second)
-                    __builtin_nontemporal_store(vf4{gp[4 * q], gp[4 * q + 1], gp[4 * q + 2], gp[4 * q + 3]}, reinterpret_cast<vf4*>(row2) + q);
-            }
-        }
-    }
+    for (int t = 1; t <= LIMIT; ++t)
+        if (__ballot(v >= t)) m = t;
+    return m;
 }
 
-// SECOND: the exchange rows are written twice (see BackwardParams::entry_grad_shifted).
-template <int C, bool SECOND>
-__device__ __forceinline__ void backward_pixels_body(const BackwardParams& p)
+// ---------------------------------------------------------------------------------------------------------
+// Pass 1: per block of 16 x 16 cells.
+constexpr int kBlockCells  = 16;                       // cells per side of a workgroup's block
+constexpr int kBlockSide   = kBlockCells + 1;          // pixels per side that those cells' footprints cover
+constexpr int kBlockPixels = kBlockSide * kBlockSide;  // 289
+constexpr int kListMax     = 16;                       // entries of a pixel's list (the larger list depth)
+
+// LDS of a block: {dL/dalpha, T alpha} per (pixel, list position); dL/dimage per pixel; per (cell, place in the cell's
+// sorted list) the list positions of that point's entry in its four corner pixels (0xFF: none) and its compact number
+__host__ __device__ constexpr size_t tiles_lds_bytes(int cpad)
 {
+    return (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * cpad * 4 + (size_t)kBlockCells * kBlockCells * kCellKeep * 8;
+}
+
+template <int C>
+__global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParams p)
+{
+    constexpr int CPAD  = (C + 3) & ~3;
+    constexpr int RF    = 4 + CPAD;  // floats per blend record
+    constexpr int NQ    = CPAD / 4;
+    constexpr int PRF   = pair_row_floats(CPAD);
+    constexpr int BATCH = 4;  // list positions whose records are requested together
+    extern __shared__ __align__(16) unsigned char s_mem[];
+    float2* const s_ex     = reinterpret_cast<float2*>(s_mem);
+    float* const s_g       = reinterpret_cast<float*>(s_mem + (size_t)kBlockPixels * kListMax * 8);
+    unsigned* const s_rank = reinterpret_cast<unsigned*>(s_mem + (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * CPAD * 4);
+    unsigned* const s_cid  = s_rank + kBlockCells * kBlockCells * kCellKeep;
+    __shared__ double s_acc[4][C];
+
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // a lane sees a few dozen pixels: its own sums stay in single precision, everything across lanes is double
-    float acc_bg[C];
+    const int NB   = p.geom.bin_off[p.num_layers];
+    // a quarter of a tile per workgroup, the four of a tile on one XCD
+    const long long lblock = xcd_tile_block(blockIdx.x, 4);
+    if (lblock >= (long long)NB * 4) return;
+    const int bin = (int)(lblock >> 2), quarter = (int)(lblock & 3);
+    const TileCtx tc = tile_ctx(p.geom, bin);
+    const int bx = (quarter & 1) * kBlockCells, by = (quarter >> 1) * kBlockCells;
+    if (tc.x0 + bx >= tc.w || tc.y0 + by >= tc.h) return;  // a block of padding
+    const float* const gi = p.grad_image[tc.layer];
+    const int kshift      = p.list_depth == 16 ? 4 : 3;
+
+    // no entry yet under any (cell, place)
+    for (int i = threadIdx.x; i < kBlockCells * kBlockCells * kCellKeep / 4; i += 256)
+        reinterpret_cast<uint4*>(s_rank)[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+    __syncthreads();
+
+    float acc_bg[C];  // a lane sees a few pixels: its own sums stay in single precision, everything across lanes is double
 #pragma unroll
-    for (int i = 0; i < C; ++i) acc_bg[i] = 0.f;
+    for (int c = 0; c < C; ++c) acc_bg[c] = 0.f;
 
-    // A workgroup walks quarters of tiles (256 pixels = 32 groups of eight), 4 workgroups per tile, all on one XCD.
-    // A wavefront takes every fourth group; it reads the retained counts of all its 64 pixels with one load, so the
-    // choice of the row width and the rows' own lengths cost no further memory round trip.
-    constexpr int kPerTile      = 4;
-    constexpr int kQuarter      = kTilePixels / kPerTile;
-    const long long num_tiles   = p.geom.bin_off[p.num_layers];
-    const long long tile_stride = (long long)(gridDim.x / (kPerTile * kNumXcd)) * kNumXcd;
-
-    for (long long lbl = xcd_tile_block(blockIdx.x, kPerTile); lbl < num_tiles * kPerTile; lbl += tile_stride * kPerTile)
+    // ---- the block's pixels, one per lane: 256, then the 33 that are left (the first wavefront) ----
+    for (int round = 0; round < 2; ++round)
     {
-        const int lb = (int)lbl;  // quarter tile number; all its pixels exist (tiles are padded to 1024 pixels)
-        // the quarter's pixels share a tile: its layer and position are found once, on the scalar unit
-        const TileCtx tc      = tile_ctx(p.geom, lb / kPerTile);
-        const float* const gi = p.grad_image[tc.layer];
-        // lane -> pixel (lane % 8) of this wavefront's group number lane / 8
-        const int my_pix = lb * kQuarter + ((lane >> 3) * 4 + wave) * 8 + (lane & 7);
-        int m_all        = p.retained[my_pix] & kRetainedMask;  // (low bits of the word) 0 for the padding of partial tiles
-        int m_grp        = m_all;
-        m_grp            = max(m_grp, __shfl_xor(m_grp, 1));
-        m_grp            = max(m_grp, __shfl_xor(m_grp, 2));
-        m_grp            = max(m_grp, __shfl_xor(m_grp, 4));
-#pragma unroll 1
-        for (int it = 0; it < 8; ++it)
+        if (round == 1 && wave > 0) break;
+        const int t       = round * 256 + (int)threadIdx.x;
+        const bool active = t < kBlockPixels;
+        const int py = t / kBlockSide, px = t - py * kBlockSide;
+        const int gx = tc.x0 + bx + px, gy = tc.y0 + by + py;
+        const bool inside = active && gx < tc.w && gy < tc.h;
+        const bool owned  = inside && px < kBlockCells && py < kBlockCells;  // (the rest belongs to a neighbour's block)
+        const unsigned pix = inside ? (unsigned)pix_index_mul24(p.geom, tc.layer, gx, gy) : 0u;
+        const int m        = inside ? (p.retained[pix] & kRetainedMask) : 0;
+        const int mmax     = wave_max_small<kListMax>(m);
+
+        float g[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) g[c] = 0.f;
+        if (inside)
         {
-            const int pix_first = lb * kQuarter + (it * 4 + wave) * 8;
-            const int m8        = __builtin_amdgcn_readfirstlane(__shfl(m_grp, it * 8));
-            if (m8 <= 8)
-                backward_pixel_rows<C, 8, SECOND>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 3)), acc_bg);
+            // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
+            if (p.layout == TRIPS_LAYOUT_CHW)
+            {
+                const size_t plane = (size_t)tc.w * tc.h;
+                const float* o     = gi + ((size_t)p.view_index * C) * plane;
+                const unsigned at  = __umul24((unsigned)gy, (unsigned)tc.w) + (unsigned)gx;
+#pragma unroll
+                for (int c = 0; c < C; ++c) g[c] = (o + c * plane)[at];
+            }
             else
             {
-                backward_pixel_rows<C, 16, SECOND>(p, tc, gi, pix_first, __shfl(m_all, it * 8 + (lane >> 4)), acc_bg);
-                backward_pixel_rows<C, 16, SECOND>(p, tc, gi, pix_first + 4, __shfl(m_all, it * 8 + 4 + (lane >> 4)), acc_bg);
+                const float* o    = gi + ((size_t)p.view_index * tc.h * tc.w) * C;
+                const unsigned at = (__umul24((unsigned)gy, (unsigned)tc.w) + (unsigned)gx) * C;
+#pragma unroll
+                for (int c = 0; c < C; ++c) g[c] = o[at + c];
+            }
+        }
+        if (active)
+        {
+#pragma unroll
+            for (int c = 0; c < CPAD; ++c) s_g[t * CPAD + c] = c < C ? g[c] : 0.f;
+        }
+        float sbg = 0.f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) sbg += p.background[c] * g[c];
+
+        // the pixel's list: compact numbers and where each entry came from
+        int id[kListMax];
+        unsigned tagw[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            vi4 v = {0, 0, 0, 0};
+            if (4 * q < mmax && 4 * q < m) v = __builtin_nontemporal_load(reinterpret_cast<const vi4*>(p.lists + ((size_t)pix << kshift)) + q);
+            id[4 * q] = v.x, id[4 * q + 1] = v.y, id[4 * q + 2] = v.z, id[4 * q + 3] = v.w;
+        }
+        if (m > 0)
+        {
+            const vu4 v = __builtin_nontemporal_load(reinterpret_cast<const vu4*>(p.tags) + pix);
+            tagw[0] = v.x, tagw[1] = v.y, tagw[2] = v.z, tagw[3] = v.w;
+        }
+
+        // front to back: alpha, transmittance (the forward's chain), descriptor . dL/dimage
+        float A[kListMax], Tr[kListMax], S[kListMax];
+#pragma unroll
+        for (int j = 0; j < kListMax; ++j) A[j] = 0.f, Tr[j] = 0.f, S[j] = 0.f;
+        float T = 1.f;
+        float4 r0[BATCH], rd[BATCH][NQ];
+        auto position = [&](auto jc)
+        {
+            constexpr int j = decltype(jc)::value;
+            constexpr int b = j % BATCH;
+            const bool has  = j < m;
+            float a         = 0.f;
+            if (has) a = entry_alpha(r0[b], tc.layer, p.num_layers, gx, gy);
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                const float4 t4 = rd[b][c / 4];
+                const float d   = (c & 3) == 0 ? t4.x : (c & 3) == 1 ? t4.y : (c & 3) == 2 ? t4.z : t4.w;
+                s += d * g[c];
+            }
+            A[j]  = a;
+            Tr[j] = T;
+            S[j]  = has ? s : 0.f;
+            T     = T * (1.f - a);
+        };
+        auto batch = [&](auto first)
+        {
+            constexpr int j0 = decltype(first)::value;
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b)
+            {
+                r0[b] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) rd[b][q] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (j0 + b < mmax && j0 + b < m)
+                {
+                    const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)id[j0 + b] * RF);
+                    r0[b]             = rec[0];
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) rd[b][q] = rec[1 + q];
+                }
+            }
+            if (j0 + 0 < mmax) position(std::integral_constant<int, j0 + 0>{});
+            if (j0 + 1 < mmax) position(std::integral_constant<int, j0 + 1>{});
+            if (j0 + 2 < mmax) position(std::integral_constant<int, j0 + 2>{});
+            if (j0 + 3 < mmax) position(std::integral_constant<int, j0 + 3>{});
+        };
+        if (mmax > 0) batch(std::integral_constant<int, 0>{});
+        if (mmax > 4) batch(std::integral_constant<int, 4>{});
+        if (mmax > 8) batch(std::integral_constant<int, 8>{});
+        if (mmax > 12) batch(std::integral_constant<int, 12>{});
+
+        // transmittance after the m retained entries decides whether the background is reached
+        // (RenderBackward.cu:205-210,302-308); T is that product (1 for an empty list)
+        const float T_after   = T;
+        const bool bg_reached = inside && (T_after >= 0.001f);
+        if (bg_reached && owned)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c) acc_bg[c] += T_after * g[c];
+        }
+        const float bg_term = bg_reached ? T_after * sbg : 0.f;
+
+        // back to front: dL/dalpha_j = T_j s_j - (sum_{i>j} T_i alpha_i s_i + background term) / (1 - alpha_j + 1e-9)
+        // (RenderBackward.cu:262-302); the entry goes to LDS under its pixel and under its (cell, place)
+        float later = 0.f;  // sum over the entries behind this one
+#pragma unroll
+        for (int j = kListMax - 1; j >= 0; --j)
+        {
+            if (j < mmax)
+            {
+                const float ta = Tr[j] * A[j];
+                if (j < m)
+                {
+                    const float dem        = 1.f / (1.f - A[j] + 1e-9f);
+                    const float grad_alpha = Tr[j] * S[j] - (later + bg_term) * dem;
+                    s_ex[t * kListMax + j] = make_float2(grad_alpha, ta);
+                    const unsigned tag     = (tagw[j / 4] >> (8 * (j & 3))) & 0xFFu;
+                    const int w = (int)(tag >> 4) & 3, place = (int)(tag & 15u);
+                    // the cell the entry came from: (x-1, y-1), (x, y-1), (x-1, y), (x, y) for w = 0..3; this pixel is corner
+                    // 3 - w of that footprint
+                    const int cxl = px - 1 + (w & 1), cyl = py - 1 + (w >> 1);
+                    if ((unsigned)cxl < (unsigned)kBlockCells && (unsigned)cyl < (unsigned)kBlockCells)
+                    {
+                        const int slot = (cyl * kBlockCells + cxl) * kCellKeep + place;
+                        reinterpret_cast<unsigned char*>(s_rank)[slot * 4 + (3 - w)] = (unsigned char)j;
+                        s_cid[slot] = (unsigned)id[j];  // (the four corners write the same number)
+                    }
+                }
+                later += ta * S[j];
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- the block's cells, one per lane: a row per (point, layer) pair that some pixel retained ----
+    {
+        const int cell = threadIdx.x;  // (cyl * 16 + cxl)
+        const int cyl = cell >> 4, cxl = cell & 15;
+#pragma unroll 1
+        for (int place = 0; place < kCellKeep; ++place)
+        {
+            const unsigned word = s_rank[cell * kCellKeep + place];
+            if (!__ballot(word != ~0u)) continue;
+            if (word == ~0u) continue;
+            const unsigned cid = s_cid[cell * kCellKeep + place];
+            const long long pair = (long long)p.pair_first[cid] + tc.layer;
+            float tex[CPAD], ga[4];
+#pragma unroll
+            for (int c = 0; c < CPAD; ++c) tex[c] = 0.f;
+#pragma unroll
+            for (int corner = 0; corner < 4; ++corner)
+            {
+                const unsigned r = (word >> (8 * corner)) & 0xFFu;
+                ga[corner]       = 0.f;
+                if (r == 0xFFu) continue;
+                const int tp   = (cyl + (corner >> 1)) * kBlockSide + cxl + (corner & 1);
+                const float2 e = s_ex[tp * kListMax + (int)r];
+                ga[corner]     = e.x;
+#pragma unroll
+                for (int c = 0; c < C; ++c) tex[c] += e.y * s_g[tp * CPAD + c];
+            }
+            if (pair < p.pair_capacity)
+            {
+                vf4* row = reinterpret_cast<vf4*>(p.pair_sums + (size_t)pair * PRF);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) row[q] = vf4{tex[4 * q], tex[4 * q + 1], tex[4 * q + 2], tex[4 * q + 3]};
+                row[NQ] = vf4{ga[0], ga[1], ga[2], ga[3]};
             }
         }
     }
 
-    __shared__ double s_acc[4][C];
 #pragma unroll
     for (int i = 0; i < C; ++i)
     {
@@ -281,28 +344,10 @@ __device__ __forceinline__ void backward_pixels_body(const BackwardParams& p)
     }
 }
 
-// (up to 4 channels the kernel needs 77 registers: seven wavefronts per SIMD; held to the 64 of eight it spills)
-// The two forms of the body are separate code: a flag tested at every store costs registers that the kernel lacks.
-template <int C>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 7 : 1))) void backward_pixels_kernel(const BackwardParams p)
-{
-    if (entry_row_floats((C + 3) & ~3) == 16 && use_shifted_rows(*p.header))
-        backward_pixels_body<C, true>(p);
-    else
-        backward_pixels_body<C, false>(p);
-}
-
 // ---------------------------------------------------------------------------------------------------------
-// Pass 2: per point. A wavefront takes 64 consecutive points. The work of a point is one item per layer in which some
-// pixel retained it (the rank bytes say which); points differ in the layers they reach, so the items of the 64 points
-// are dealt out to the lanes through LDS, one item per lane and round (usually one round): every lane then issues the
-// gathers of its item at once, instead of all lanes walking the layers of the deepest point one memory round trip
-// after the other. An item's sums return through LDS and each point adds its items up in layer order.
-// The kernel is a chain of dependent memory round trips per step; it is kept short: the compact number of a step's
-// point is requested one step ahead, and what does not change from step to step (camera, rotation matrix) waits in LDS
-// rather than in registers, which the items need.
-constexpr int kItemFloats(int cpad) { return 4 + cpad; }  // {confidence, ip.x, ip.y, size} sums, then the descriptor's
-
+// Pass 2: per point. The rows of a point's pairs follow each other (layer by layer), and those of consecutive valid
+// points as well: the loads below are dense. What does not change from point to point (camera, rotation matrix) waits
+// in LDS rather than in registers.
 struct PointPassCamera
 {
     Camera cam;
@@ -310,31 +355,24 @@ struct PointPassCamera
 };
 
 template <int C>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 : 1))) void backward_points_kernel(const BackwardParams p)
+__global__ __launch_bounds__(256) void backward_points_kernel(const BackwardParams p)
 {
     constexpr int CPAD = (C + 3) & ~3;
-    constexpr int KIN  = entry_row_entries(CPAD);
     constexpr int RF   = 4 + CPAD;  // floats per blend record
+    constexpr int NQ   = CPAD / 4;
+    constexpr int PRF  = pair_row_floats(CPAD);
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
-    constexpr int NIT  = kItemFloats(CPAD);
     const int lane     = threadIdx.x & 63;
-    const int wave     = threadIdx.x >> 6;
     const bool want_pose = p.d_pose != nullptr;
     const bool want_intr = p.d_intrinsics != nullptr;
     const bool want_size = p.d_point_size != nullptr;
     const bool identity  = p.header->not_identity == 0;  // index[pid] == pid for every point
     const bool overwrite = p.overwrite != 0;             // outputs are written, not added to
-    const bool shifted_rows = entry_row_floats(CPAD) == 16 && use_shifted_rows(*p.header);
     // In that mode every point stores all its outputs (zeros where it has no gradient), all lanes at one place, so that
     // whole lines are written. (Descriptor columns other than the points' own, and all of them when the index is not
-    // the identity, were cleared by zero_texel_grads_kernel.)
+    // the identity, were cleared by the prologue kernel.)
 
     __shared__ PointPassCamera s_cam;
-    // what an item needs of its point {ip.x, ip.y, size field, confidence, size_px, softplus' * d size_px / d size},
-    // then the point in view space, kept here for the point's own lane
-    __shared__ float s_point[4][64][9];
-    __shared__ uint2 s_item[4][64 * 8];                 // {lane of the point | layer << 8, the layer's four rank bytes}
-    __shared__ __align__(16) float s_sums[4][64][NIT];  // sums of the items of one round
     if (threadIdx.x == 0)
     {
         s_cam.cam = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
@@ -366,12 +404,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
             cid_next             = pid2 < p.num_points ? p.cid_of[pid2] : -1;  // in flight during this step
         }
         // {softplus'(raw size), depth, layers written, size_px}
-        const float4 tail = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
+        const float4 tail   = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
         const int max_layer = live ? __float_as_int(tail.z) : 0;
-        uint4 rk0 = make_uint4(~0u, ~0u, ~0u, ~0u), rk1 = rk0;
+        float4 r0           = make_float4(0.f, 0.f, 0.f, 0.f);  // ip.x ip.y size field conf
+        float view[3]       = {0.f, 0.f, 1.f};
+        long long first     = 0;
         if (live)
         {
-            const float4 r0 = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);  // ip.x ip.y size field conf
+            r0    = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
+            first = p.pair_first[cid];
             // the point in view space, exactly as the projection kernel computed it
             float4 pos = p.position[pid];
             if (p.displacement)
@@ -381,160 +422,80 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
                 pos.y += dsp[1];
                 pos.z += dsp[2];
             }
-            rk0 = *reinterpret_cast<const uint4*>(p.rank + (size_t)cid * 16);
-            // layers 4..7: a row of the second plane, defined only for the points that were written to those layers
-            if (max_layer > 4) rk1 = *reinterpret_cast<const uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16);
-            float view[3];
             transform_point(s_cam.cam.V, pos.x, pos.y, pos.z, view);
-            const float J_softmax_proj = s_cam.cam.fx * s_cam.cam.cfx / fmaxf(view[2], 0.f);
-            float* sp = s_point[wave][lane];
-            sp[0] = r0.x, sp[1] = r0.y, sp[2] = r0.z, sp[3] = r0.w, sp[4] = tail.w, sp[5] = tail.x * J_softmax_proj;
-            sp[6] = view[0], sp[7] = view[1], sp[8] = view[2];
         }
-
-        // ---- the point's items: the layers it was written to in which some corner pixel retained it ----
-        const unsigned words[8] = {rk0.x, rk0.y, rk0.z, rk0.w, rk1.x, rk1.y, rk1.z, rk1.w};
-        unsigned layer_mask = 0;
-#pragma unroll
-        for (int l = 0; l < 8; ++l)
-            if (l < max_layer && words[l] != 0xFFFFFFFFu) layer_mask |= 1u << l;
-        const int my_items = __popc(layer_mask);
-        int first_item     = my_items;  // inclusive prefix over the wavefront, then made exclusive
-        for (int o = 1; o < 64; o <<= 1)
-        {
-            const int t = __shfl_up(first_item, o);
-            if (lane >= o) first_item += t;
-        }
-        const int num_items = __builtin_amdgcn_readlane(first_item, 63);  // <= 64 * 8
-        first_item -= my_items;
-        {
-            int k = first_item;
-#pragma unroll
-            for (int l = 0; l < 8; ++l)
-                if (layer_mask & (1u << l)) s_item[wave][k++] = make_uint2((unsigned)lane | ((unsigned)l << 8), words[l]);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const float ipx = r0.x, ipy = r0.y, size_field = r0.z, conf = r0.w, size_px = tail.w;
+        const float size_chain = tail.x * (s_cam.cam.fx * s_cam.cam.cfx / fmaxf(view[2], 0.f));  // softplus' * d size_px / d size
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;
         float tex_grad[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) tex_grad[c] = 0.f;
-        const bool any = my_items > 0;
+        bool any = false;
 
-        for (int round = 0; round < num_items; round += 64)
+        const int lmax = wave_max_small<TRIPS_MAX_LAYERS>(max_layer);
+        for (int layer = 0; layer < lmax; ++layer)
         {
-            if (round + lane < num_items)
+            if (layer >= max_layer) continue;
+            const long long pair = first + layer;
+            if (pair >= p.pair_capacity) continue;
+            // the pair's row: descriptor sums, then dL/dalpha of the four corners (zeros where no pixel retained the point)
+            const vf4* row = reinterpret_cast<const vf4*>(p.pair_sums + (size_t)pair * PRF);
+            vf4 tq[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) tq[q] = __builtin_nontemporal_load(row + q);
+            const vf4 gav = __builtin_nontemporal_load(row + NQ);
+            const float ga[4] = {gav.x, gav.y, gav.z, gav.w};
+            if (!(ga[0] != 0.f || ga[1] != 0.f || ga[2] != 0.f || ga[3] != 0.f))
             {
-                // one layer of one point: the four gathers are issued together, then consumed in corner order
-                const uint2 item    = s_item[wave][round + lane];
-                const int layer     = (int)(item.x >> 8);
-                const unsigned word = item.y;
-                const float* sp     = s_point[wave][item.x & 63u];
-                const float ipx = sp[0], ipy = sp[1], size_field = sp[2], conf = sp[3], size_px = sp[4], size_chain = sp[5];
-                const float mfac = 1.f / float(1 << layer);
-                const float ux = ipx * mfac, uy = ipy * mfac;
-                const float fx = floorf(ux), fy = floorf(uy);
-                const int px = (int)fx, py = (int)fy;
-                const float sx = ux - fx, sy = uy - fy;
-                float lfac = 1.f, J_lf = 0.f;
-                if (want_size) lfac = layer_factor_encoded_grad(size_field, size_px, layer, p.num_layers, &J_lf);
-                float2 e[4];
-                float4 gq[4][CPAD / 4];
-                // 64-byte rows: a footprint that starts at an odd pixel reads the copy in which its two pixels of a
-                // row share a line (not across the border of a tile, where they are not neighbours in memory)
-                const float* rows = (shifted_rows && (px & 1) && (px & (kTile - 1)) != kTile - 1)
-                                        ? p.entry_grad_shifted
-                                        : p.entry_grad;
+                bool t_any = false;
 #pragma unroll
-                for (int corner = 0; corner < 4; ++corner)
-                {
-                    const unsigned j = (word >> (8 * corner)) & 0xFFu;
-                    const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                    const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, gx, gy);
-                    const bool on      = j != 0xFFu;
-                    const float* row   = rows + (size_t)pix * entry_row_floats(CPAD);  // the pixel's row
-                    const unsigned jj  = j & 15u;
-                    const float2* src2 = jj < (unsigned)KIN ? reinterpret_cast<const float2*>(row + CPAD) + jj
-                                                            : reinterpret_cast<const float2*>(p.entry_over) + ((size_t)pix * (16 - KIN) + (jj - KIN));
-                    e[corner]          = on ? *src2 : make_float2(0.f, 0.f);
-                    const float4* src  = reinterpret_cast<const float4*>(row);
-#pragma unroll
-                    for (int q = 0; q < CPAD / 4; ++q) gq[corner][q] = on ? src[q] : make_float4(0.f, 0.f, 0.f, 0.f);
-                }
-                float i_conf = 0.f, i_d0 = 0.f, i_d1 = 0.f, i_size = 0.f;
-                float i_tex[CPAD];
-#pragma unroll
-                for (int c = 0; c < CPAD; ++c) i_tex[c] = 0.f;
-#pragma unroll
-                for (int corner = 0; corner < 4; ++corner)
-                {
-                    const unsigned j = (word >> (8 * corner)) & 0xFFu;
-                    if (j == 0xFFu) continue;
-                    const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                    float gv[CPAD];
-#pragma unroll
-                    for (int q = 0; q < CPAD / 4; ++q)
-                    {
-                        gv[4 * q]     = gq[corner][q].x;
-                        gv[4 * q + 1] = gq[corner][q].y;
-                        gv[4 * q + 2] = gq[corner][q].z;
-                        gv[4 * q + 3] = gq[corner][q].w;
-                    }
-                    const float grad_alpha = e[corner].x;
-                    const float ta         = e[corner].y;
-#pragma unroll
-                    for (int c = 0; c < C; ++c) i_tex[c] += ta * gv[c];
-                    // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
-                    // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
-                    const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
-                    const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
-                    float blend    = wx * wy;
-                    const float J0 = x_hi ? wy : -wy;
-                    const float J1 = y_hi ? wx : -wx;
-                    if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
-                    i_conf += blend * lfac * grad_alpha;
-                    const float gbs = conf * lfac * grad_alpha;
-                    i_d0 += J0 * gbs;
-                    i_d1 += J1 * gbs;
-                    if (want_size)
-                    {
-                        const float grad_layer_ps = size_chain * J_lf * grad_alpha;
-                        i_size += blend * conf * grad_layer_ps;
-                    }
-                }
-                float4* out = reinterpret_cast<float4*>(s_sums[wave][lane]);
-                out[0]      = make_float4(i_conf, i_d0, i_d1, i_size);
-#pragma unroll
-                for (int q = 0; q < CPAD / 4; ++q) out[1 + q] = make_float4(i_tex[4 * q], i_tex[4 * q + 1], i_tex[4 * q + 2], i_tex[4 * q + 3]);
+                for (int q = 0; q < NQ; ++q) t_any = t_any || tq[q].x != 0.f || tq[q].y != 0.f || tq[q].z != 0.f || tq[q].w != 0.f;
+                if (!t_any) continue;  // no pixel retained the point in this layer
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            // the point's items of this round, in layer order
-            const int j_end = min(first_item + my_items, round + 64);
-            for (int j = max(first_item, round); j < j_end; ++j)
-            {
-                const float4* in = reinterpret_cast<const float4*>(s_sums[wave][j - round]);
-                const float4 a   = in[0];
-                conf_grad += a.x;
-                d0 += a.y;
-                d1 += a.z;
-                size_grad += a.w;
+            any = true;
+            const float mfac = 1.f / float(1 << layer);
+            const float ux = ipx * mfac, uy = ipy * mfac;
+            const float fx = floorf(ux), fy = floorf(uy);
+            const int px = (int)fx, py = (int)fy;
+            const float sx = ux - fx, sy = uy - fy;
+            float lfac = 1.f, J_lf = 0.f;
+            if (want_size) lfac = layer_factor_encoded_grad(size_field, size_px, layer, p.num_layers, &J_lf);
+            float i_conf = 0.f, i_d0 = 0.f, i_d1 = 0.f, i_size = 0.f;
 #pragma unroll
-                for (int q = 0; q < CPAD / 4; ++q)
+            for (int corner = 0; corner < 4; ++corner)
+            {
+                const int gx = px + (corner & 1), gy = py + (corner >> 1);
+                const float grad_alpha = ga[corner];
+                // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
+                // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
+                const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
+                const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
+                float blend    = wx * wy;
+                const float J0 = x_hi ? wy : -wy;
+                const float J1 = y_hi ? wx : -wx;
+                if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
+                i_conf += blend * lfac * grad_alpha;
+                const float gbs = conf * lfac * grad_alpha;
+                i_d0 += J0 * gbs;
+                i_d1 += J1 * gbs;
+                if (want_size)
                 {
-                    const float4 t = in[1 + q];
-                    if (4 * q < C) tex_grad[4 * q] += t.x;
-                    if (4 * q + 1 < C) tex_grad[4 * q + 1] += t.y;
-                    if (4 * q + 2 < C) tex_grad[4 * q + 2] += t.z;
-                    if (4 * q + 3 < C) tex_grad[4 * q + 3] += t.w;
+                    const float grad_layer_ps = size_chain * J_lf * grad_alpha;
+                    i_size += blend * conf * grad_layer_ps;
                 }
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // the point's layers add up in layer order
+            conf_grad += i_conf;
+            d0 += i_d0;
+            d1 += i_d1;
+            size_grad += i_size;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                const vf4 t4 = tq[c / 4];
+                tex_grad[c] += (c & 3) == 0 ? t4.x : (c & 3) == 1 ? t4.y : (c & 3) == 2 ? t4.z : t4.w;
+            }
         }
         if (pid >= p.num_points || (!live && !overwrite)) continue;
         const int tex = identity ? pid : p.index[pid];  // (a column outside the table: the point was culled)
@@ -543,8 +504,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
         float g_point[3] = {0.f, 0.f, 0.f}, g_pose[6], g_k[5], g_dis[8];
         if (any)
         {
-            const float* sp = s_point[wave][lane];
-            project_backward(s_cam.cam, s_cam.R, sp[6], sp[7], sp[8], d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
+            project_backward(s_cam.cam, s_cam.R, view[0], view[1], view[2], d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
             if (want_pose)
             {
 #pragma unroll
@@ -624,16 +584,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(C <= 4 ? 4 
     }
 }
 
-// Before the two passes of the first view. Overwrite mode (`texels`): the descriptor and confidence gradients of the
-// columns that the point pass does not write itself. With the identity index (the forward noted it in the header)
-// those are the columns past the last point; otherwise all of them, the point pass then adds with atomics.
-// `clear_sums`: the block sums that both passes add to (background, every pose row, every intrinsics row).
-__global__ __launch_bounds__(256) void zero_texel_grads_kernel(const ViewHeader* __restrict__ header, float* __restrict__ d_texture,
-                                                               float* __restrict__ d_confidence, int channels, int num_texels,
-                                                               int num_points, int texels, int clear_sums,
-                                                               float* __restrict__ d_background, double* __restrict__ d_pose,
-                                                               int num_images, float* __restrict__ d_intrinsics, int num_cameras)
+// Before the two passes of a view: the rows of the view's pairs start as zeros (the tile pass writes the rows of the
+// pairs that some pixel retained, the point pass reads all rows of a point). On the first view of a call also, in
+// overwrite mode (`texels`): the descriptor and confidence gradients of the columns that the point pass does not write
+// itself. With the identity index (the forward noted it in the header) those are the columns past the last point;
+// otherwise all of them, the point pass then adds with atomics. `clear_sums`: the block sums that both passes add to
+// (background, every pose row, every intrinsics row).
+__global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader* __restrict__ header, float* __restrict__ pair_sums,
+                                                                int pair_row, long long pair_capacity, float* __restrict__ d_texture,
+                                                                float* __restrict__ d_confidence, int channels, int num_texels,
+                                                                int num_points, int texels, int clear_sums,
+                                                                float* __restrict__ d_background, double* __restrict__ d_pose,
+                                                                int num_images, float* __restrict__ d_intrinsics, int num_cameras)
 {
+    {
+        long long pairs = (long long)header->n_entries;
+        if (pairs > pair_capacity) pairs = pair_capacity;
+        const long long quads = pairs * pair_row / 4;  // (rows are a multiple of four floats)
+        vf4* dst              = reinterpret_cast<vf4*>(pair_sums);
+        for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < quads; i += (long long)gridDim.x * 256)
+            __builtin_nontemporal_store(vf4{0.f, 0.f, 0.f, 0.f}, dst + i);
+    }
     if (clear_sums && blockIdx.x == 0)
     {
         if (d_background)
@@ -656,6 +627,16 @@ __global__ __launch_bounds__(256) void zero_texel_grads_kernel(const ViewHeader*
     }
 }
 
+template <int C>
+hipError_t launch_tiles(const BackwardParams& p, int blocks, hipStream_t stream)
+{
+    const size_t lds = tiles_lds_bytes((C + 3) & ~3);
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&backward_tiles_kernel<C>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((backward_tiles_kernel<C>), dim3(blocks), dim3(256), lds, stream, p);
+    return hipSuccess;
+}
+
 #define TRIPS_BW_DISPATCH(KERNEL, BLOCKS)                                                                      \
     switch (channels)                                                                                          \
     {                                                                                                          \
@@ -669,20 +650,31 @@ __global__ __launch_bounds__(256) void zero_texel_grads_kernel(const ViewHeader*
 
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof)
 {
-    const int P           = p.geom.bin_off[p.num_layers] * kTilePixels;
-    const int N           = p.num_points;
-    // (no points: only the background receives gradient)
-    if (p.overwrite || p.clear_block_sums)
-        hipLaunchKernelGGL(zero_texel_grads_kernel, dim3(p.overwrite ? 1024 : 1), dim3(256), 0, stream, p.header, p.d_texture,
-                           p.d_confidence, channels, p.num_texels, N, p.overwrite, p.clear_block_sums, p.d_background, p.d_pose_all,
-                           p.num_images, p.d_intrinsics_all, p.num_cameras);
+    const int NB = p.geom.bin_off[p.num_layers];
+    const int N  = p.num_points;
     {
-        ProfScope ps(prof, "backward_pixels", stream);
-        const long long waves = ((long long)P + 3) / 4;
-        long long blocks_ll   = (waves + 3) / 4;
-        int blocks            = (int)(blocks_ll < 8192 ? (blocks_ll < 1 ? 1 : blocks_ll) : 8192);
-        blocks                = ((blocks + 4 * kNumXcd - 1) / (4 * kNumXcd)) * (4 * kNumXcd);  // whole groups of 8 tiles x 4
-        TRIPS_BW_DISPATCH(backward_pixels_kernel, blocks);
+        ProfScope ps(prof, "backward_prologue", stream);
+        hipLaunchKernelGGL(backward_prologue_kernel, dim3(2048), dim3(256), 0, stream, p.header, p.pair_sums,
+                           pair_row_floats((channels + 3) & ~3), p.pair_capacity, p.d_texture, p.d_confidence, channels, p.num_texels,
+                           N, p.overwrite, p.clear_block_sums, p.d_background, p.d_pose_all, p.num_images, p.d_intrinsics_all,
+                           p.num_cameras);
+    }
+    {
+        // (no points: only the background receives gradient)
+        ProfScope ps(prof, "backward_tiles", stream);
+        const long long tiles8 = (((long long)NB + kNumXcd - 1) / kNumXcd) * kNumXcd;  // tiles rounded up to 8
+        const int blocks       = (int)(tiles8 * 4);
+        hipError_t e           = hipErrorInvalidValue;
+        switch (channels)
+        {
+            case 3: e = launch_tiles<3>(p, blocks, stream); break;
+            case 4: e = launch_tiles<4>(p, blocks, stream); break;
+            case 6: e = launch_tiles<6>(p, blocks, stream); break;
+            case 8: e = launch_tiles<8>(p, blocks, stream); break;
+            case 16: e = launch_tiles<16>(p, blocks, stream); break;
+            default: break;
+        }
+        if (e != hipSuccess) return e;
     }
     if (N > 0)
     {

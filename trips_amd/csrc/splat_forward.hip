@@ -208,22 +208,22 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     constexpr int WAVES = kBinThreads / 64;
     extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
     __shared__ int s_valid[2][WAVES];  // valid points of every wavefront in this step (two steps in flight)
+    __shared__ int s_pairs[2][WAVES];  // (point, layer) pairs of every wavefront in this step
     __shared__ int s_flags;            // bit 0: not_identity, bit 1: bad_index, of any point of the chunk
-    __shared__ int s_same_tile;        // valid points in the finest-layer tile of the point before them
     const Camera cam  = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L       = p.num_layers;
     const int NB      = p.geom.bin_off[L];
     bool not_identity = false;  // some point's descriptor column differs from its own index
     bool bad_index    = false;
     for (int i = threadIdx.x; i < NB; i += kBinThreads) s_hist[i] = 0;
-    if (threadIdx.x == 0) s_flags = 0, s_same_tile = 0;
+    if (threadIdx.x == 0) s_flags = 0;
     __syncthreads();
-    int same_tile = 0;  // (wavefront-uniform)
 
     int begin, end;
     chunk_point_range(p, begin, end);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int next       = begin;  // workgroup-uniform: compact number of the chunk's next valid point
+    int next_pair  = 0;      // workgroup-uniform: pairs of the chunk's points so far
     int step       = 0;
     // the loads of the next step's points are in flight while this step's are projected
     PointInputs nxt;
@@ -247,27 +247,39 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
             for (int c = 0; c < C; ++c) d[c] = p.texture[(size_t)c * p.num_texels + in.tex];
         }
         PointProjection o;
-        o.valid = false;
+        o.valid  = false;
+        o.layers = 0;
         if (pid < end) o = project_point<TRAIN>(p, cam, pid, in, s_hist, not_identity, bad_index);
         const unsigned long long vm = __ballot(o.valid);
-        if (lane == 0) s_valid[step][wave] = (int)__popcll(vm);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        // pairs of the wavefront's points before this one, and of the wavefront: a point has 0..8 layers, one ballot per bit
+        int pairs_before = 0, pairs_wave = 0;
+        if (TRAIN)
         {
-            // how coherent the cloud's memory order is on the screen (lane 0 of a wavefront has no neighbour here)
-            const int tile      = o.valid ? (((int)o.ipy >> kTileShift) << 16) | ((int)o.ipx >> kTileShift) : -1;
-            const int tile_prev = __shfl_up(tile, 1);
-            same_tile += (int)__popcll(__ballot(o.valid && lane > 0 && tile == tile_prev));
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+            {
+                const unsigned long long m = __ballot((o.layers >> b) & 1);
+                pairs_before += (int)__popcll(m & below) << b;
+                pairs_wave += (int)__popcll(m) << b;
+            }
         }
+        if (lane == 0) s_valid[step][wave] = (int)__popcll(vm), s_pairs[step][wave] = pairs_wave;
         __syncthreads();
-        int before = 0, total = 0;
+        int before = 0, total = 0, pbefore = 0, ptotal = 0;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w)
         {
-            const int c = s_valid[step][w];
+            const int c = s_valid[step][w], q = s_pairs[step][w];
             before += w < wave ? c : 0;
             total += c;
+            pbefore += w < wave ? q : 0;
+            ptotal += q;
         }
-        const int cid = next + before + (int)__popcll(vm & ((1ull << lane) - 1ull));
+        const int cid        = next + before + (int)__popcll(vm & below);
+        const int first_pair = next_pair + pbefore + pairs_before;  // within the chunk; the scatter pass adds the chunk's first
         next += total;
+        next_pair += ptotal;
         if (pid >= end) continue;
         if (TRAIN) p.cid_of[pid] = o.valid ? cid : -1;
         if (!o.valid) continue;
@@ -286,19 +298,12 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         if (TRAIN)
         {
             __builtin_nontemporal_store(pid, p.pid_of + cid);
-            // The rank table of the backward (which of a point's (layer, corner) pixels retained it, and where in the
-            // pixel's list; filled by the blend kernels): a plane of 16 bytes per compact number for layers 0..3 and a second
-            // one for layers 4..7. Every valid point clears its row of the first, the few points that reach layer 4 and
-            // beyond their row of the second as well.
-            __builtin_nontemporal_store(vu4{~0u, ~0u, ~0u, ~0u}, reinterpret_cast<vu4*>(p.rank + (size_t)cid * 16));
-            if (o.layers > 4)
-                *reinterpret_cast<uint4*>(p.rank + (size_t)p.num_points * 16 + (size_t)cid * 16) = make_uint4(~0u, ~0u, ~0u, ~0u);
+            __builtin_nontemporal_store(first_pair, p.pair_first + cid);
         }
     }
     {
         const int flags = (__ballot(not_identity) != 0 ? 1 : 0) | (__ballot(bad_index) != 0 ? 2 : 0);
         if (flags && lane == 0) atomicOr(&s_flags, flags);
-        if (same_tile && lane == 0) atomicAdd(&s_same_tile, same_tile);
     }
 
     // this workgroup's row of the histogram matrix [workgroup][bin]; its valid points and flags for the scan kernel,
@@ -310,7 +315,8 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     {
         p.chunk_valid[blockIdx.x]                = next - begin;
         p.chunk_valid[p.bin_groups + blockIdx.x] = s_flags;
-        p.chunk_valid[2 * p.bin_groups + blockIdx.x] = s_same_tile;
+        p.chunk_valid[2 * p.bin_groups + blockIdx.x] = 0;
+        p.chunk_valid[3 * p.bin_groups + blockIdx.x] = next_pair;
     }
 }
 
@@ -327,7 +333,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
 // kernels), which saves a launch of its own.
 __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restrict__ bin_count, int32_t* __restrict__ bin_start,
                                                          int32_t* __restrict__ slice_start, int NB, long long capacity,
-                                                         const int32_t* __restrict__ chunk_valid, int G, ViewHeader* header,
+                                                         int32_t* __restrict__ chunk_valid, int G, ViewHeader* header,
                                                          ViewHeader* status, int first_view, int32_t* __restrict__ long_count,
                                                          uint4* __restrict__ clear, long long clear_n)
 {
@@ -359,6 +365,22 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
             v += (unsigned long long)(unsigned)chunk_valid[g];
             f |= chunk_valid[G + g];
             st += (unsigned long long)(unsigned)chunk_valid[2 * G + g];
+        }
+        // number of every chunk's first (point, layer) pair: exclusive prefix of the chunks' pair counts (G <= 1024)
+        {
+            const int mine = (int)threadIdx.x < G ? chunk_valid[3 * G + threadIdx.x] : 0;
+            int inc        = mine;
+            for (int o = 1; o < 64; o <<= 1)
+            {
+                const int t = __shfl_up(inc, o);
+                if (lane >= o) inc += t;
+            }
+            if (lane == 63) s_wave[0][wave] = inc;
+            __syncthreads();
+            int prefix = inc - mine;
+            for (int w = 0; w < wave; ++w) prefix += s_wave[0][w];
+            if ((int)threadIdx.x < G) chunk_valid[4 * G + threadIdx.x] = prefix;
+            __syncthreads();
         }
         for (int o = 32; o > 0; o >>= 1)
         {
@@ -542,6 +564,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
     int begin, end;
     chunk_point_range(p, begin, end);
     const int n      = p.chunk_valid[blockIdx.x];
+    const int pair_base = p.chunk_valid[4 * p.bin_groups + blockIdx.x];
     unsigned dropped = 0;
     constexpr int U  = 2;  // records of a thread in flight together
     for (int cid0 = begin + (int)threadIdx.x; cid0 < begin + n; cid0 += U * kBinThreads)
@@ -557,6 +580,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
                 const vf4 t = __builtin_nontemporal_load(reinterpret_cast<const vf4*>(p.prec) + cid);
                 tail[u]     = make_float4(t.x, t.y, t.z, t.w);
                 ip[u]   = *reinterpret_cast<const float2*>(p.rec + (size_t)cid * p.rec_floats);
+                // the point's first pair: the projection numbered it within the chunk, the scan found the chunk's first
+                if (p.pair_first) p.pair_first[cid] += pair_base;
             }
         }
 #pragma unroll
@@ -796,7 +821,6 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
 //                      sorts them with a network, any other merges the (sorted, cut) lists of its four cells; then the
 //                      alpha blend front to back (RenderForward.cu:820-1048).
 // A pixel's colour is summed in the order of a balanced binary tree over the list positions.
-constexpr int kCellKeep    = 16;  // keys of a cell that can reach a pixel's list (the largest list depth)
 constexpr int kLaneSortMax = 8;   // longest list that a lane sorts with a network
 constexpr int kStagedKeys  = 8;   // keys per cell that blend_kernel stages in LDS for the merging lanes
 
@@ -830,20 +854,6 @@ __device__ __forceinline__ int4 load_cell(const ForwardParams& p, const TileCtx&
     return r;
 }
 
-// alpha of a list entry at pixel (gx, gy) of `layer` and the entry's (layer, footprint corner) slot of its point
-__device__ __forceinline__ float entry_alpha(const float4& r0, int layer, int num_layers, int gx, int gy, int& slot)
-{
-    const float m  = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
-    const float ux = r0.x * m, uy = r0.y * m;
-    float w        = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
-    if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
-    float a = w * r0.w;
-    a *= layer_factor_encoded(r0.z, layer, num_layers);
-    const int cx = gx - (int)floorf(ux), cy = gy - (int)floorf(uy);
-    slot         = layer * 4 + ((cy & 1) << 1) + (cx & 1);
-    return a;
-}
-
 template <int C>
 __device__ __forceinline__ void store_pixel(const ForwardParams& p, float* img, int lw, int lh, int gx, int gy, const float (&col)[C])
 {
@@ -874,13 +884,28 @@ __device__ __forceinline__ void sort_pair(u64& a, u64& b)
     a = lo;
     b = hi;
 }
-__device__ __forceinline__ void lane_sort4(u64 (&k)[kLaneSortMax])
+// a key with a tag that travels with it
+struct TaggedKey
+{
+    u64 key;
+    int tag;
+};
+__device__ __forceinline__ void sort_pair(TaggedKey& a, TaggedKey& b)
+{
+    const bool sw = b.key < a.key;
+    const TaggedKey lo{sw ? b.key : a.key, sw ? b.tag : a.tag}, hi{sw ? a.key : b.key, sw ? a.tag : b.tag};
+    a = lo;
+    b = hi;
+}
+template <typename T>
+__device__ __forceinline__ void lane_sort4(T (&k)[kLaneSortMax])
 {
     sort_pair(k[0], k[1]), sort_pair(k[2], k[3]);
     sort_pair(k[0], k[2]), sort_pair(k[1], k[3]);
     sort_pair(k[1], k[2]);
 }
-__device__ __forceinline__ void lane_sort8(u64 (&k)[kLaneSortMax])
+template <typename T>
+__device__ __forceinline__ void lane_sort8(T (&k)[kLaneSortMax])
 {
     sort_pair(k[0], k[1]), sort_pair(k[2], k[3]), sort_pair(k[4], k[5]), sort_pair(k[6], k[7]);
     sort_pair(k[0], k[2]), sort_pair(k[1], k[3]), sort_pair(k[4], k[6]), sort_pair(k[5], k[7]);
@@ -890,7 +915,8 @@ __device__ __forceinline__ void lane_sort8(u64 (&k)[kLaneSortMax])
     sort_pair(k[1], k[2]), sort_pair(k[3], k[4]), sort_pair(k[5], k[6]);
 }
 // ascending sort of the first nmax (wave-uniform) of the lane's keys
-__device__ __forceinline__ void lane_sort(u64 (&k)[kLaneSortMax], int nmax)
+template <typename T>
+__device__ __forceinline__ void lane_sort(T (&k)[kLaneSortMax], int nmax)
 {
     if (nmax > 4)
         lane_sort8(k);
@@ -1157,6 +1183,9 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
     const bool merges = total > kLaneSortMax;
 
     unsigned id[16];  // compact numbers of the pixel's entries, nearest first
+    // where each entry came from, for the backward: which of the pixel's four cells (bits 4..5) and its place in that
+    // cell's sorted list (bits 0..3); one byte per list position, four positions per word
+    unsigned tagw[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int j = 0; j < 16; ++j) id[j] = ~0u;
 
@@ -1169,23 +1198,32 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
             // position i of the concatenation of the four cell lists lies in cell (i >= o1) + (i >= o2) + (i >= o3)
             // (sums of steps rather than a chain of selects: the compiler turns the chain into a table in memory);
             // none of these cells has a long list
-            u64 k[kLaneSortMax];
+            TaggedKey k[kLaneSortMax];
             const int o1 = c0.y, o2 = o1 + c1.y, o3 = o2 + c2.y;
             const int b0 = c0.x, b1 = c1.x - o1, b2 = c2.x - o2, b3 = c3.x - o3;
 #pragma unroll
             for (int i = 0; i < kLaneSortMax; ++i)
             {
-                k[i] = ~0ull;
+                k[i].key = ~0ull;
+                k[i].tag = 0;
                 if (i < nmax)
                 {
                     const int base = b0 + (i >= o1 ? b1 - b0 : 0) + (i >= o2 ? b2 - b1 : 0) + (i >= o3 ? b3 - b2 : 0);
-                    if (i < mine) k[i] = p.keys[(unsigned)(base + i)];
+                    if (i < mine) k[i].key = p.keys[(unsigned)(base + i)];
+                    // cell w, place i - (first position of cell w)
+                    if (TRAIN)
+                        k[i].tag = (((i >= o1) + (i >= o2) + (i >= o3)) << 4) |
+                                   (i - ((i >= o1 ? o1 : 0) + (i >= o2 ? o2 - o1 : 0) + (i >= o3 ? o3 - o2 : 0)));
                 }
             }
             lane_sort(k, nmax);
 #pragma unroll
             for (int i = 0; i < kLaneSortMax; ++i)
-                if (i < mine) id[i] = (unsigned)k[i];
+                if (i < mine)
+                {
+                    id[i] = (unsigned)k[i].key;
+                    tagw[i / 4] |= (unsigned)k[i].tag << (8 * (i & 3));
+                }
         }
     }
     // ---- more: merge the four sorted cell lists. The first kStagedKeys keys of the block's cells wait in LDS; a
@@ -1230,6 +1268,7 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
                     const bool hi = m23 < m01;
                     id[j]         = (unsigned)(hi ? m23 : m01);
                     const int w   = hi ? (b23 ? 3 : 2) : (b01 ? 1 : 0);  // the list that gave the key
+                    if (TRAIN) tagw[j / 4] |= (unsigned)((w << 4) | (w == 0 ? q0 : w == 1 ? q1 : w == 2 ? q2 : q3)) << (8 * (j & 3));
                     q0 += w == 0, q1 += w == 1, q2 += w == 2, q3 += w == 3;
                     if (j + 1 < n)
                     {
@@ -1258,9 +1297,8 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
         constexpr int j = decltype(jc)::value;
         constexpr int b = j % BATCH;
         const bool has  = j < n;
-        int slot        = 0;
         float a         = 0.f;
-        if (has) a = entry_alpha(r0[b], tc.layer, p.num_layers, gx, gy, slot);
+        if (has) a = entry_alpha(r0[b], tc.layer, p.num_layers, gx, gy);
         const float Tc  = (T >= kAlphaDestCutoff) ? T : 0.f;
         const bool kept = has && Tc >= kAlphaDestCutoff;
         run_open        = run_open && kept;
@@ -1277,12 +1315,6 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
         sum.template push<j>(pr);
         // background weight (RenderForward.cu:1002-1022): taken at the last list position
         if (j == n - 1) bgw = (p.background_mode == TRIPS_BG_REFERENCE) ? Tc : T * (1.f - a);
-        // rank of this entry in the pixel's list, into the point's table, for the entries the backward will visit
-        // (two planes of 16 bytes per point: layers 0..3, then layers 4..7)
-#ifndef EXP_NORANK
-        if (TRAIN && run_open)
-            p.rank[(tc.layer < 4 ? (size_t)0 : (size_t)p.num_points * 16 - 16) + ((size_t)id[j] << 4) + slot] = (unsigned char)j;
-#endif
         T = T * (1.f - a);
     };
     // the records of BATCH positions are requested together, then the positions are walked
@@ -1348,11 +1380,10 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
                                     p.retained + pix);
         const int kshift = p.list_depth == 16 ? 4 : 3;
         vi4* row         = reinterpret_cast<vi4*>(p.lists + ((size_t)(unsigned)pix << kshift));
-#ifndef EXP_NOLISTS
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             if (4 * q < n) __builtin_nontemporal_store(vi4{(int)id[4 * q], (int)id[4 * q + 1], (int)id[4 * q + 2], (int)id[4 * q + 3]}, row + q);
-#endif
+        if (n > 0) __builtin_nontemporal_store(vu4{tagw[0], tagw[1], tagw[2], tagw[3]}, reinterpret_cast<vu4*>(p.tags) + (unsigned)pix);
     }
 }
 

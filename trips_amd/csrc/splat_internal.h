@@ -127,6 +127,9 @@ constexpr int kSliceEntries = 8192;
 constexpr int kLongList    = 1024;
 constexpr int kLongSegment = 512;
 constexpr int kStageKeys  = 7168;   // keys of one tile staged in LDS before they are written (56 KB)
+// keys of a cell that can reach a pixel's list (the larger list depth): the forward sorts every cell's list and keeps
+// this many
+constexpr int kCellKeep = 16;
 
 struct PyramidGeom
 {
@@ -225,10 +228,6 @@ struct ViewHeader
     unsigned long long reserved;
 };
 
-// The backward keeps a second, shifted copy of its exchange rows (BackwardParams::entry_grad_shifted) when fewer than a
-// quarter of the valid points lie in the finest-layer tile of the point before them in memory.
-__host__ __device__ inline bool use_shifted_rows(const ViewHeader& h) { return 4 * h.same_tile_as_previous < h.n_valid; }
-
 // Layout of one view's saved state (all offsets in bytes, 256-aligned)
 struct SavedLayout
 {
@@ -237,31 +236,30 @@ struct SavedLayout
     size_t prec;      // float [N * kPointRecordFloats]
     size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded); a row's positions past its ids are undefined
     size_t retained;  // int32 [Pi]: retained entries in bits 0..4, list positions that hold an id (min(length, K)) in bits 5..9, list length from bit 10
-    size_t rank;      // uint8 [2][N, 16] rank of the point's retained entry in each of its (layer, corner) pixels, 0xFF = none:
-                      // plane 0 layers 0..3, plane 1 layers 4..7 (rows defined only for points written to those layers)
+    size_t tags;      // uint8 [Pi, 16]  where a list position came from: which of the pixel's four cells (bits 4..5) and its
+                      // place in that cell's sorted list (bits 0..3); a row's positions past its ids are undefined
     size_t cid_of;    // int32 [N] compact number of every point (-1 = culled)
     size_t pid_of;    // int32 [N] point of every compact number (the first n_valid are defined)
+    size_t pair_first;  // int32 [N] by compact number: the number of the point's first (point, layer) pair; its pairs are
+                        // numbered consecutively by layer, all pairs of a view densely in point order
     size_t bytes_per_view;
 };
 
-// A pixel's row of the backward's exchange table: the image gradient, then the entries that fit behind it: 64 bytes
-// with 6 entries at 4 channels and 4 at 8, 128 bytes with 8 entries at 16 channels (a list keeps at most 16; the
-// rest go to a table of their own). The 128-byte rows that hold 14 entries at 4 channels measured 5 % slower in the
-// pixel pass, which writes them, and no faster in the point pass, which gathers from them.
-__host__ __device__ constexpr int entry_row_floats(int cpad) { return cpad <= 8 ? 16 : 32; }
-__host__ __device__ constexpr int entry_row_entries(int cpad) { return (entry_row_floats(cpad) - cpad) / 2 < 16 ? (entry_row_floats(cpad) - cpad) / 2 : 16; }
+// The backward sums, per (point, layer) pair, what the four pixels of the footprint contribute before the projection
+// chain: the descriptor gradient sum_corners T alpha dL/dimage (Cpad floats) and dL/dalpha of each corner (4 floats).
+__host__ __device__ constexpr int pair_row_floats(int cpad) { return cpad + 4; }
 
 struct BackwardWorkspaceLayout
 {
-    size_t entry_grad;  // float [Pi, entry_row_floats]
-    size_t entry_grad_shifted;  // 64-byte rows only: float [1 + Pi + 1, 16], a second copy one row further on (0: none)
-    size_t entry_over;  // float2 [Pi, 16 - entry_row_entries]
+    size_t pair_sums;  // float [capacity, pair_row_floats] by pair number
+    size_t capacity;   // (point, layer) pairs
     size_t bytes;
 };
 
 struct WorkspaceLayout
 {
-    size_t chunk_valid;   // int32 [3 G]  valid points of every chunk of the binning kernels, the chunks' flags, their same-tile counts
+    size_t chunk_valid;   // int32 [5 G]  per chunk of the binning kernels: valid points, flags, same-tile counts, (point, layer)
+                          //              pairs, and (from the scan) the number of the chunk's first pair
     size_t prec;         // float4 [N]         point records, when there is no saved state to hold them
     size_t counts;       // int32 [Pi]   list length per cell (the points whose 2 x 2 footprint starts at that pixel)
     size_t cursor;       // int32 [Pi]   first key of each cell's list (-1 - first candidate row for a long list)
@@ -327,7 +325,8 @@ struct ForwardParams
     int32_t rec_floats;
     int32_t* lists;
     int32_t* retained;
-    unsigned char* rank;  // training only
+    unsigned char* tags;  // training only
+    int32_t* pair_first;  // training only
     ViewHeader* header;  // counters of this view
     ViewHeader* status;  // overflow flag of the whole forward call (start of the workspace)
     float* image[TRIPS_MAX_LAYERS];
@@ -355,17 +354,10 @@ struct BackwardParams
     const int32_t* cid_of;
     const ViewHeader* header;
     const float* grad_image[TRIPS_MAX_LAYERS];
-    float* entry_grad;    // [Pi, entry_row_floats] a row per pixel: dL/dimage[0..Cpad), then float2 {dL/dalpha, T alpha} of
-                          // the first entry_row_entries retained entries (workspace)
-    float* entry_over;    // [Pi, 16 - entry_row_entries] float2: the retained entries beyond those (workspace)
-    // Rows of 64 bytes: two pixels share a 128-byte line, the pairs (0,1), (2,3), ... of a tile row. A footprint that
-    // starts at an odd pixel would find its two pixels of a row in two lines; the rows are therefore written a second
-    // time, one row further on, where the pairs are (1,2), (3,4), ...: row of pixel pix at entry_grad_shifted + 16 pix
-    // (the pointer already includes the shift; null when a row is a line of its own). Written and read only for clouds
-    // whose memory order is not coherent on the screen (use_shifted_rows): in a coherent one the lines are shared
-    // by neighbouring lanes anyway, and the second copy costs the pixel pass more than it saves the point pass.
-    float* entry_grad_shifted;
-    const unsigned char* rank;  // [2][N, 16] (saved state) rank of the point's entry in each of its (layer, corner) pixels, 0xFF = none
+    const unsigned char* tags;  // [Pi, 16] (saved state) cell and place in the cell's list of every list position
+    const int32_t* pair_first;  // [N] (saved state) by compact number
+    float* pair_sums;  // [pairs, pair_row_floats] (workspace)
+    long long pair_capacity;
     float* d_texture;
     float* d_confidence;
     float* d_background;

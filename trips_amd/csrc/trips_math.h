@@ -126,6 +126,19 @@ __device__ __forceinline__ float layer_factor_encoded_grad(float field, float tr
     return layer_factor_interpolated(field, layer, max_layers, grad);
 }
 
+// alpha of a list entry (r0: the first four floats of its point's blend record) at pixel (gx, gy) of `layer`
+// (RenderForward.cu:875-899: bilinear weight x confidence x layer factor)
+__device__ __forceinline__ float entry_alpha(const float4& r0, int layer, int num_layers, int gx, int gy)
+{
+    const float m  = __uint_as_float((uint32_t)(127 - layer) << 23);  // 2^-layer
+    const float ux = r0.x * m, uy = r0.y * m;
+    float w        = (1.f - fabsf(ux - float(gx))) * (1.f - fabsf(uy - float(gy)));
+    if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) w = 0.f;
+    float a = w * r0.w;
+    a *= layer_factor_encoded(r0.z, layer, num_layers);
+    return a;
+}
+
 struct Pose
 {
     float qx, qy, qz, qw, tx, ty, tz;

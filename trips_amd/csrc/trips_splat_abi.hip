@@ -210,11 +210,13 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(P * K * sizeof(int32_t));
     s.retained = o;
     o += align256(P * sizeof(int32_t));
-    s.rank = o;
-    o += align256(N * 32);
+    s.tags = o;
+    o += align256(P * 16);
     s.cid_of = o;
     o += align256(N * sizeof(int32_t));
     s.pid_of = o;
+    o += align256(N * sizeof(int32_t));
+    s.pair_first = o;
     o += align256(N * sizeof(int32_t));
     s.bytes_per_view = o;
     return s;
@@ -272,18 +274,11 @@ namespace
 BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     BackwardWorkspaceLayout w;
-    const size_t P = (size_t)g.bin_off[d.num_layers] * kTilePixels;
-    size_t o       = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
-    w.entry_grad   = o;
-    o += align256(P * (size_t)entry_row_floats((d.num_channels + 3) & ~3) * sizeof(float));
-    w.entry_over = o;
-    o += align256(P * (size_t)(16 - entry_row_entries((d.num_channels + 3) & ~3)) * 2 * sizeof(float));
-    w.entry_grad_shifted = 0;
-    if (entry_row_floats((d.num_channels + 3) & ~3) == 16)
-    {
-        w.entry_grad_shifted = o;
-        o += align256((P + 2) * 16 * sizeof(float));
-    }
+    // a row per (point, layer) pair: as many as the forward can file
+    w.capacity  = d.max_list_entries > 0 ? ((size_t)d.max_list_entries + 3) / 4 : (size_t)d.num_points * (size_t)d.num_layers;
+    size_t o    = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
+    w.pair_sums = o;
+    o += align256(w.capacity * (size_t)pair_row_floats((d.num_channels + 3) & ~3) * sizeof(float));
     w.bytes = o;
     return w;
 }
@@ -451,7 +446,8 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
             p.rec_floats = record_floats(d.num_channels);
             p.lists      = reinterpret_cast<int32_t*>(sv + sl.lists);
             p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
-            p.rank       = reinterpret_cast<unsigned char*>(sv + sl.rank);
+            p.tags       = reinterpret_cast<unsigned char*>(sv + sl.tags);
+            p.pair_first = reinterpret_cast<int32_t*>(sv + sl.pair_first);
             p.cid_of     = reinterpret_cast<int32_t*>(sv + sl.cid_of);
             p.pid_of     = reinterpret_cast<int32_t*>(sv + sl.pid_of);
         }
@@ -553,10 +549,10 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.retained     = reinterpret_cast<const int32_t*>(sv + sl.retained);
         p.cid_of       = reinterpret_cast<const int32_t*>(sv + sl.cid_of);
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
-        p.entry_grad   = reinterpret_cast<float*>(ws + bl.entry_grad);
-        p.entry_over   = reinterpret_cast<float*>(ws + bl.entry_over);
-        p.entry_grad_shifted = bl.entry_grad_shifted ? reinterpret_cast<float*>(ws + bl.entry_grad_shifted) + 16 : nullptr;
-        p.rank         = reinterpret_cast<const unsigned char*>(sv + sl.rank);
+        p.tags         = reinterpret_cast<const unsigned char*>(sv + sl.tags);
+        p.pair_first   = reinterpret_cast<const int32_t*>(sv + sl.pair_first);
+        p.pair_sums    = reinterpret_cast<float*>(ws + bl.pair_sums);
+        p.pair_capacity = (long long)bl.capacity;
         for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
         p.d_texture    = grads->d_texture;
         p.d_confidence = grads->d_confidence;
