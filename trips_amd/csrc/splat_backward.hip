@@ -87,9 +87,9 @@ __device__ __forceinline__ int wave_max_small(int v)
 
 // ---------------------------------------------------------------------------------------------------------
 // Pass 1: per block of 16 x 16 cells.
-constexpr int kBlockCells  = 16;                       // cells per side of a workgroup's block
-constexpr int kBlockSide   = kBlockCells + 1;          // pixels per side that those cells' footprints cover
-constexpr int kBlockPixels = kBlockSide * kBlockSide;  // 289
+constexpr int kBlockSide   = 16;                       // pixels per side of a workgroup's block: one pixel per lane
+constexpr int kBlockCells  = kBlockSide - 1;           // cells per side whose footprints lie inside those pixels
+constexpr int kBlockPixels = kBlockSide * kBlockSide;  // 256
 constexpr int kListMax     = 16;                       // entries of a pixel's list (the larger list depth)
 
 // LDS of a block: {dL/dalpha, T alpha} per (pixel, list position); dL/dimage per pixel; per (cell, place in the cell's
@@ -106,7 +106,9 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     constexpr int RF    = 4 + CPAD;  // floats per blend record
     constexpr int NQ    = CPAD / 4;
     constexpr int PRF   = pair_row_floats(CPAD);
-    constexpr int BATCH = 4;  // list positions whose records are requested together
+    // list positions whose records are requested together (the LDS of a block bounds the wavefronts per SIMD before the
+    // registers do)
+    constexpr int BATCH = CPAD <= 4 ? 8 : 4;
     extern __shared__ __align__(16) unsigned char s_mem[];
     float2* const s_ex     = reinterpret_cast<float2*>(s_mem);
     float* const s_g       = reinterpret_cast<float*>(s_mem + (size_t)kBlockPixels * kListMax * 8);
@@ -115,15 +117,19 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     __shared__ double s_acc[4][C];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int NB   = p.geom.bin_off[p.num_layers];
-    // a quarter of a tile per workgroup, the four of a tile on one XCD
-    const long long lblock = xcd_tile_block(blockIdx.x, 4);
-    if (lblock >= (long long)NB * 4) return;
-    const int bin = (int)(lblock >> 2), quarter = (int)(lblock & 3);
-    const TileCtx tc = tile_ctx(p.geom, bin);
-    const int bx = (quarter & 1) * kBlockCells, by = (quarter >> 1) * kBlockCells;
-    if (tc.x0 + bx >= tc.w || tc.y0 + by >= tc.h) return;  // a block of padding
-    const float* const gi = p.grad_image[tc.layer];
+    // Blocks of 16 x 16 pixels that overlap by one row and one column (so that every cell's four pixels lie in one
+    // block): block (i, j) of a layer starts at pixel (15 i, 15 j). Runs of eight blocks of a block row share an XCD.
+    const long long lblock = xcd_tile_block(blockIdx.x, 8);
+    if (lblock >= p.blocks_off[p.num_layers]) return;
+    int layer = 0;
+#pragma unroll
+    for (int l = 1; l < TRIPS_MAX_LAYERS; ++l)
+        if (l < p.num_layers && lblock >= p.blocks_off[l]) layer = l;
+    const int in_layer = (int)lblock - p.blocks_off[layer];
+    const int byi = in_layer / p.blocks_x[layer], bxi = in_layer - byi * p.blocks_x[layer];
+    const int lw = p.geom.w[layer], lh = p.geom.h[layer];
+    const int x0 = bxi * kBlockCells, y0 = byi * kBlockCells;  // the block's first pixel
+    const float* const gi = p.grad_image[layer];
     const int kshift      = p.list_depth == 16 ? 4 : 3;
 
     // no entry yet under any (cell, place)
@@ -135,19 +141,33 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
 #pragma unroll
     for (int c = 0; c < C; ++c) acc_bg[c] = 0.f;
 
-    // ---- the block's pixels, one per lane: 256, then the 33 that are left (the first wavefront) ----
-    for (int round = 0; round < 2; ++round)
+    // ---- the block's pixels, one per lane, a wavefront taking 8 x 8 of them (the four pixels of a footprint then
+    // mostly sit in one wavefront and share their gathers) ----
     {
-        if (round == 1 && wave > 0) break;
-        const int t       = round * 256 + (int)threadIdx.x;
-        const bool active = t < kBlockPixels;
-        const int py = t / kBlockSide, px = t - py * kBlockSide;
-        const int gx = tc.x0 + bx + px, gy = tc.y0 + by + py;
-        const bool inside = active && gx < tc.w && gy < tc.h;
-        const bool owned  = inside && px < kBlockCells && py < kBlockCells;  // (the rest belongs to a neighbour's block)
-        const unsigned pix = inside ? (unsigned)pix_index_mul24(p.geom, tc.layer, gx, gy) : 0u;
-        const int m        = inside ? (p.retained[pix] & kRetainedMask) : 0;
-        const int mmax     = wave_max_small<kListMax>(m);
+        const int px = ((wave & 1) << 3) + (lane & 7), py = ((wave >> 1) << 3) + (lane >> 3);
+        const int t  = py * kBlockSide + px;
+        const int gx = x0 + px, gy = y0 + py;
+        const bool inside = gx < lw && gy < lh;
+        // (the last row and column are the first of the neighbours' blocks)
+        const bool owned   = inside && px < kBlockCells && py < kBlockCells;
+        const unsigned pix = inside ? (unsigned)pix_index_mul24(p.geom, layer, gx, gy) : 0u;
+        // the pixel's retained count, its list (compact numbers and where each entry came from) and dL/dimage are all
+        // requested before the first is looked at; list positions past the retained ones hold anything and are not used
+        int word = 0;
+        int id[kListMax];
+        unsigned tagw[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < kListMax; ++j) id[j] = 0;
+        if (inside)
+        {
+            word = p.retained[pix];
+            {
+                const vi4 v = __builtin_nontemporal_load(reinterpret_cast<const vi4*>(p.lists + ((size_t)pix << kshift)));
+                id[0] = v.x, id[1] = v.y, id[2] = v.z, id[3] = v.w;
+            }
+            const vu4 v = __builtin_nontemporal_load(reinterpret_cast<const vu4*>(p.tags) + pix);
+            tagw[0] = v.x, tagw[1] = v.y, tagw[2] = v.z, tagw[3] = v.w;
+        }
 
         float g[C];
 #pragma unroll
@@ -157,44 +177,37 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             // offsets inside one view's image stay far below 2^32 (the pyramid has at most kMaxBins tiles)
             if (p.layout == TRIPS_LAYOUT_CHW)
             {
-                const size_t plane = (size_t)tc.w * tc.h;
+                const size_t plane = (size_t)lw * lh;
                 const float* o     = gi + ((size_t)p.view_index * C) * plane;
-                const unsigned at  = __umul24((unsigned)gy, (unsigned)tc.w) + (unsigned)gx;
+                const unsigned at  = __umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx;
 #pragma unroll
                 for (int c = 0; c < C; ++c) g[c] = (o + c * plane)[at];
             }
             else
             {
-                const float* o    = gi + ((size_t)p.view_index * tc.h * tc.w) * C;
-                const unsigned at = (__umul24((unsigned)gy, (unsigned)tc.w) + (unsigned)gx) * C;
+                const float* o    = gi + ((size_t)p.view_index * lh * lw) * C;
+                const unsigned at = (__umul24((unsigned)gy, (unsigned)lw) + (unsigned)gx) * C;
 #pragma unroll
                 for (int c = 0; c < C; ++c) g[c] = o[at + c];
             }
         }
-        if (active)
-        {
+        const int m    = word & kRetainedMask;
+        const int mmax = wave_max_small<kListMax>(m);
+        // (two thirds of the pixels of a typical view retain at most four entries: the rest of a list only where needed)
 #pragma unroll
-            for (int c = 0; c < CPAD; ++c) s_g[t * CPAD + c] = c < C ? g[c] : 0.f;
+        for (int q = 1; q < 4; ++q)
+        {
+            if (4 * q < mmax && 4 * q < m)
+            {
+                const vi4 v = __builtin_nontemporal_load(reinterpret_cast<const vi4*>(p.lists + ((size_t)pix << kshift)) + q);
+                id[4 * q] = v.x, id[4 * q + 1] = v.y, id[4 * q + 2] = v.z, id[4 * q + 3] = v.w;
+            }
         }
+#pragma unroll
+        for (int c = 0; c < CPAD; ++c) s_g[t * CPAD + c] = c < C ? g[c] : 0.f;
         float sbg = 0.f;
 #pragma unroll
         for (int c = 0; c < C; ++c) sbg += p.background[c] * g[c];
-
-        // the pixel's list: compact numbers and where each entry came from
-        int id[kListMax];
-        unsigned tagw[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-        {
-            vi4 v = {0, 0, 0, 0};
-            if (4 * q < mmax && 4 * q < m) v = __builtin_nontemporal_load(reinterpret_cast<const vi4*>(p.lists + ((size_t)pix << kshift)) + q);
-            id[4 * q] = v.x, id[4 * q + 1] = v.y, id[4 * q + 2] = v.z, id[4 * q + 3] = v.w;
-        }
-        if (m > 0)
-        {
-            const vu4 v = __builtin_nontemporal_load(reinterpret_cast<const vu4*>(p.tags) + pix);
-            tagw[0] = v.x, tagw[1] = v.y, tagw[2] = v.z, tagw[3] = v.w;
-        }
 
         // front to back: alpha, transmittance (the forward's chain), descriptor . dL/dimage
         float A[kListMax], Tr[kListMax], S[kListMax];
@@ -208,7 +221,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             constexpr int b = j % BATCH;
             const bool has  = j < m;
             float a         = 0.f;
-            if (has) a = entry_alpha(r0[b], tc.layer, p.num_layers, gx, gy);
+            if (has) a = entry_alpha(r0[b], layer, p.num_layers, gx, gy);
             float s = 0.f;
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -231,7 +244,11 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 r0[b] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) rd[b][q] = make_float4(0.f, 0.f, 0.f, 0.f);
+#ifdef EXP_NOREC
+                if (false)
+#else
                 if (j0 + b < mmax && j0 + b < m)
+#endif
                 {
                     const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)id[j0 + b] * RF);
                     r0[b]             = rec[0];
@@ -243,11 +260,23 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             if (j0 + 1 < mmax) position(std::integral_constant<int, j0 + 1>{});
             if (j0 + 2 < mmax) position(std::integral_constant<int, j0 + 2>{});
             if (j0 + 3 < mmax) position(std::integral_constant<int, j0 + 3>{});
+            if constexpr (BATCH > 4)
+            {
+                if (j0 + 4 < mmax) position(std::integral_constant<int, j0 + 4>{});
+                if (j0 + 5 < mmax) position(std::integral_constant<int, j0 + 5>{});
+                if (j0 + 6 < mmax) position(std::integral_constant<int, j0 + 6>{});
+                if (j0 + 7 < mmax) position(std::integral_constant<int, j0 + 7>{});
+            }
         };
         if (mmax > 0) batch(std::integral_constant<int, 0>{});
-        if (mmax > 4) batch(std::integral_constant<int, 4>{});
-        if (mmax > 8) batch(std::integral_constant<int, 8>{});
-        if (mmax > 12) batch(std::integral_constant<int, 12>{});
+        if constexpr (BATCH == 4)
+        {
+            if (mmax > 4) batch(std::integral_constant<int, 4>{});
+            if (mmax > 8) batch(std::integral_constant<int, 8>{});
+            if (mmax > 12) batch(std::integral_constant<int, 12>{});
+        }
+        else if (mmax > 8)
+            batch(std::integral_constant<int, 8>{});
 
         // transmittance after the m retained entries decides whether the background is reached
         // (RenderBackward.cu:205-210,302-308); T is that product (1 for an empty list)
@@ -293,17 +322,36 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     __syncthreads();
 
     // ---- the block's cells, one per lane: a row per (point, layer) pair that some pixel retained ----
+#ifndef EXP_NOPHASE2
     {
-        const int cell = threadIdx.x;  // (cyl * 16 + cxl)
-        const int cyl = cell >> 4, cxl = cell & 15;
-#pragma unroll 1
+        const int cell = min((int)threadIdx.x, kBlockCells * kBlockCells - 1);  // (cyl * 15 + cxl; the lanes past the last cell idle)
+        const bool is_cell = (int)threadIdx.x < kBlockCells * kBlockCells;
+        const int cyl = cell / kBlockCells, cxl = cell - cyl * kBlockCells;
+        // the places of the cell that hold a point, and the numbers of those points' first pairs (all requested before
+        // the first row is formed)
+        unsigned words[kCellKeep];
+        int first_pair[kCellKeep];
+#pragma unroll
         for (int place = 0; place < kCellKeep; ++place)
         {
-            const unsigned word = s_rank[cell * kCellKeep + place];
+            words[place]      = is_cell ? s_rank[cell * kCellKeep + place] : ~0u;
+            first_pair[place] = 0;
+            if (__ballot(words[place] != ~0u))
+            {
+#ifdef EXP_NOPF
+                if (words[place] != ~0u) first_pair[place] = (int)s_cid[cell * kCellKeep + place];
+#else
+                if (words[place] != ~0u) first_pair[place] = p.pair_first[s_cid[cell * kCellKeep + place]];
+#endif
+            }
+        }
+#pragma unroll
+        for (int place = 0; place < kCellKeep; ++place)
+        {
+            const unsigned word = words[place];
             if (!__ballot(word != ~0u)) continue;
             if (word == ~0u) continue;
-            const unsigned cid = s_cid[cell * kCellKeep + place];
-            const long long pair = (long long)p.pair_first[cid] + tc.layer;
+            const long long pair = (long long)first_pair[place] + layer;
             float tex[CPAD], ga[4];
 #pragma unroll
             for (int c = 0; c < CPAD; ++c) tex[c] = 0.f;
@@ -328,6 +376,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             }
         }
     }
+#endif
 
 #pragma unroll
     for (int i = 0; i < C; ++i)
@@ -345,9 +394,14 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Pass 2: per point. The rows of a point's pairs follow each other (layer by layer), and those of consecutive valid
-// points as well: the loads below are dense. What does not change from point to point (camera, rotation matrix) waits
-// in LDS rather than in registers.
+// Pass 2: per point. A wavefront takes 64 consecutive points. The work of a point is one item per layer it was written
+// to; points differ in the layers they reach, so the items of the 64 points are dealt out to the lanes through LDS,
+// one item per lane and round (usually one or two rounds): the items of a round are consecutive (point, layer) pairs,
+// whose rows are consecutive in memory, and every lane works instead of all lanes walking the layers of the deepest
+// point. An item's sums return through LDS and each point adds its items up in layer order. What does not change from
+// point to point (camera, rotation matrix) waits in LDS rather than in registers.
+constexpr int kItemFloats(int cpad) { return 4 + cpad; }  // {confidence, ip.x, ip.y, size} sums, then the descriptor's
+
 struct PointPassCamera
 {
     Camera cam;
@@ -362,7 +416,9 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     constexpr int NQ   = CPAD / 4;
     constexpr int PRF  = pair_row_floats(CPAD);
     constexpr int NACC = 6 + 5 + 8;  // pose, K, distortion
+    constexpr int NIT  = kItemFloats(CPAD);
     const int lane     = threadIdx.x & 63;
+    const int wave     = threadIdx.x >> 6;
     const bool want_pose = p.d_pose != nullptr;
     const bool want_intr = p.d_intrinsics != nullptr;
     const bool want_size = p.d_point_size != nullptr;
@@ -373,6 +429,11 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     // the identity, were cleared by the prologue kernel.)
 
     __shared__ PointPassCamera s_cam;
+    // what an item needs of its point {ip.x, ip.y, size field, confidence, size_px, softplus' * d size_px / d size,
+    // number of its first pair}, then the point in view space, kept here for the point's own lane
+    __shared__ float s_point[4][64][10];
+    __shared__ unsigned short s_item[4][64 * TRIPS_MAX_LAYERS];  // lane of the point | layer << 8
+    __shared__ __align__(16) float s_sums[4][64][NIT];           // sums of the items of one round
     if (threadIdx.x == 0)
     {
         s_cam.cam = load_camera_bw(p.pose, p.intrinsics, p.view, p.dist_cutoff);
@@ -404,15 +465,12 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             cid_next             = pid2 < p.num_points ? p.cid_of[pid2] : -1;  // in flight during this step
         }
         // {softplus'(raw size), depth, layers written, size_px}
-        const float4 tail   = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
-        const int max_layer = live ? __float_as_int(tail.z) : 0;
-        float4 r0           = make_float4(0.f, 0.f, 0.f, 0.f);  // ip.x ip.y size field conf
-        float view[3]       = {0.f, 0.f, 1.f};
-        long long first     = 0;
+        const float4 tail = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
+        int max_layer     = live ? __float_as_int(tail.z) : 0;
         if (live)
         {
-            r0    = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
-            first = p.pair_first[cid];
+            const float4 r0 = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);  // ip.x ip.y size field conf
+            const int first = p.pair_first[cid];
             // the point in view space, exactly as the projection kernel computed it
             float4 pos = p.position[pid];
             if (p.displacement)
@@ -422,80 +480,128 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
                 pos.y += dsp[1];
                 pos.z += dsp[2];
             }
+            float view[3];
             transform_point(s_cam.cam.V, pos.x, pos.y, pos.z, view);
+            const float J_softmax_proj = s_cam.cam.fx * s_cam.cam.cfx / fmaxf(view[2], 0.f);
+            float* sp = s_point[wave][lane];
+            sp[0] = r0.x, sp[1] = r0.y, sp[2] = r0.z, sp[3] = r0.w, sp[4] = tail.w, sp[5] = tail.x * J_softmax_proj;
+            sp[6] = __int_as_float(first);
+            sp[7] = view[0], sp[8] = view[1], sp[9] = view[2];
+            // (rows past the capacity of the table do not exist: the forward reported the overflow)
+            if ((long long)first + max_layer > p.pair_capacity) max_layer = (int)max(0ll, p.pair_capacity - first);
         }
-        const float ipx = r0.x, ipy = r0.y, size_field = r0.z, conf = r0.w, size_px = tail.w;
-        const float size_chain = tail.x * (s_cam.cam.fx * s_cam.cam.cfx / fmaxf(view[2], 0.f));  // softplus' * d size_px / d size
+
+        // ---- the point's items: the layers it was written to ----
+        const int my_items = max_layer;
+        int first_item     = my_items;  // inclusive prefix over the wavefront, then made exclusive
+        for (int o = 1; o < 64; o <<= 1)
+        {
+            const int t = __shfl_up(first_item, o);
+            if (lane >= o) first_item += t;
+        }
+        const int num_items = __builtin_amdgcn_readlane(first_item, 63);  // <= 64 * 8
+        first_item -= my_items;
+        for (int l = 0; l < my_items; ++l) s_item[wave][first_item + l] = (unsigned short)(lane | (l << 8));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
         float conf_grad = 0.f, size_grad = 0.f, d0 = 0.f, d1 = 0.f;
         float tex_grad[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) tex_grad[c] = 0.f;
-        bool any = false;
+        bool any = false;  // some pixel retained the point
 
-        const int lmax = wave_max_small<TRIPS_MAX_LAYERS>(max_layer);
-        for (int layer = 0; layer < lmax; ++layer)
+        for (int round = 0; round < num_items; round += 64)
         {
-            if (layer >= max_layer) continue;
-            const long long pair = first + layer;
-            if (pair >= p.pair_capacity) continue;
-            // the pair's row: descriptor sums, then dL/dalpha of the four corners (zeros where no pixel retained the point)
-            const vf4* row = reinterpret_cast<const vf4*>(p.pair_sums + (size_t)pair * PRF);
-            vf4 tq[NQ];
-#pragma unroll
-            for (int q = 0; q < NQ; ++q) tq[q] = __builtin_nontemporal_load(row + q);
-            const vf4 gav = __builtin_nontemporal_load(row + NQ);
-            const float ga[4] = {gav.x, gav.y, gav.z, gav.w};
-            if (!(ga[0] != 0.f || ga[1] != 0.f || ga[2] != 0.f || ga[3] != 0.f))
-            {
-                bool t_any = false;
-#pragma unroll
-                for (int q = 0; q < NQ; ++q) t_any = t_any || tq[q].x != 0.f || tq[q].y != 0.f || tq[q].z != 0.f || tq[q].w != 0.f;
-                if (!t_any) continue;  // no pixel retained the point in this layer
-            }
-            any = true;
-            const float mfac = 1.f / float(1 << layer);
-            const float ux = ipx * mfac, uy = ipy * mfac;
-            const float fx = floorf(ux), fy = floorf(uy);
-            const int px = (int)fx, py = (int)fy;
-            const float sx = ux - fx, sy = uy - fy;
-            float lfac = 1.f, J_lf = 0.f;
-            if (want_size) lfac = layer_factor_encoded_grad(size_field, size_px, layer, p.num_layers, &J_lf);
             float i_conf = 0.f, i_d0 = 0.f, i_d1 = 0.f, i_size = 0.f;
+            float i_tex[CPAD];
 #pragma unroll
-            for (int corner = 0; corner < 4; ++corner)
+            for (int c = 0; c < CPAD; ++c) i_tex[c] = 0.f;
+            if (round + lane < num_items)
             {
-                const int gx = px + (corner & 1), gy = py + (corner >> 1);
-                const float grad_alpha = ga[corner];
-                // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
-                // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
-                const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
-                const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
-                float blend    = wx * wy;
-                const float J0 = x_hi ? wy : -wy;
-                const float J1 = y_hi ? wx : -wx;
-                if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
-                i_conf += blend * lfac * grad_alpha;
-                const float gbs = conf * lfac * grad_alpha;
-                i_d0 += J0 * gbs;
-                i_d1 += J1 * gbs;
-                if (want_size)
+                // one layer of one point: its row holds the descriptor sums, then dL/dalpha of the four corners (zeros
+                // where no pixel retained the point)
+                const unsigned item = s_item[wave][round + lane];
+                const int layer     = (int)(item >> 8);
+                const float* sp     = s_point[wave][item & 63u];
+                const float ipx = sp[0], ipy = sp[1], size_field = sp[2], conf = sp[3], size_px = sp[4], size_chain = sp[5];
+                const vf4* row = reinterpret_cast<const vf4*>(p.pair_sums + ((size_t)__float_as_int(sp[6]) + layer) * PRF);
+                vf4 tq[NQ];
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) tq[q] = __builtin_nontemporal_load(row + q);
+                const vf4 gav     = __builtin_nontemporal_load(row + NQ);
+                const float ga[4] = {gav.x, gav.y, gav.z, gav.w};
+                const float mfac = 1.f / float(1 << layer);
+                const float ux = ipx * mfac, uy = ipy * mfac;
+                const float fx = floorf(ux), fy = floorf(uy);
+                const int px = (int)fx, py = (int)fy;
+                const float sx = ux - fx, sy = uy - fy;
+                float lfac = 1.f, J_lf = 0.f;
+                if (want_size) lfac = layer_factor_encoded_grad(size_field, size_px, layer, p.num_layers, &J_lf);
+#pragma unroll
+                for (int corner = 0; corner < 4; ++corner)
                 {
-                    const float grad_layer_ps = size_chain * J_lf * grad_alpha;
-                    i_size += blend * conf * grad_layer_ps;
+                    const int gx = px + (corner & 1), gy = py + (corner >> 1);
+                    const float grad_alpha = ga[corner];
+                    // blend_fac_index / compute_blending_fac (PointBlending.h:216-264)
+                    // the four cases of the reference's switch on y_i + x_i as selects (same products, exact negations)
+                    const bool x_hi = !(float(gx) < ux), y_hi = !(float(gy) < uy);
+                    const float wx = x_hi ? sx : 1.f - sx, wy = y_hi ? sy : 1.f - sy;
+                    float blend    = wx * wy;
+                    const float J0 = x_hi ? wy : -wy;
+                    const float J1 = y_hi ? wx : -wx;
+                    if (fabsf(ux - float(gx)) > 1.f || fabsf(uy - float(gy)) > 1.f) blend *= 0.f;
+                    i_conf += blend * lfac * grad_alpha;
+                    const float gbs = conf * lfac * grad_alpha;
+                    i_d0 += J0 * gbs;
+                    i_d1 += J1 * gbs;
+                    if (want_size)
+                    {
+                        const float grad_layer_ps = size_chain * J_lf * grad_alpha;
+                        i_size += blend * conf * grad_layer_ps;
+                    }
                 }
-            }
-            // the point's layers add up in layer order
-            conf_grad += i_conf;
-            d0 += i_d0;
-            d1 += i_d1;
-            size_grad += i_size;
 #pragma unroll
-            for (int c = 0; c < C; ++c)
-            {
-                const vf4 t4 = tq[c / 4];
-                tex_grad[c] += (c & 3) == 0 ? t4.x : (c & 3) == 1 ? t4.y : (c & 3) == 2 ? t4.z : t4.w;
+                for (int c = 0; c < CPAD; ++c)
+                {
+                    const vf4 t4 = tq[c / 4];
+                    i_tex[c]     = (c & 3) == 0 ? t4.x : (c & 3) == 1 ? t4.y : (c & 3) == 2 ? t4.z : t4.w;
+                }
+                float4* out = reinterpret_cast<float4*>(s_sums[wave][lane]);
+                out[0]      = make_float4(i_conf, i_d0, i_d1, i_size);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) out[1 + q] = make_float4(i_tex[4 * q], i_tex[4 * q + 1], i_tex[4 * q + 2], i_tex[4 * q + 3]);
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // the point's items of this round, in layer order
+            const int j_end = min(first_item + my_items, round + 64);
+            for (int j = max(first_item, round); j < j_end; ++j)
+            {
+                const float4* in = reinterpret_cast<const float4*>(s_sums[wave][j - round]);
+                const float4 a   = in[0];
+                bool nz          = a.x != 0.f || a.y != 0.f || a.z != 0.f || a.w != 0.f;
+                conf_grad += a.x;
+                d0 += a.y;
+                d1 += a.z;
+                size_grad += a.w;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q)
+                {
+                    const float4 t = in[1 + q];
+                    nz             = nz || t.x != 0.f || t.y != 0.f || t.z != 0.f || t.w != 0.f;
+                    if (4 * q < C) tex_grad[4 * q] += t.x;
+                    if (4 * q + 1 < C) tex_grad[4 * q + 1] += t.y;
+                    if (4 * q + 2 < C) tex_grad[4 * q + 2] += t.z;
+                    if (4 * q + 3 < C) tex_grad[4 * q + 3] += t.w;
+                }
+                any = any || nz;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
         if (pid >= p.num_points || (!live && !overwrite)) continue;
         const int tex = identity ? pid : p.index[pid];  // (a column outside the table: the point was culled)
@@ -504,7 +610,8 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         float g_point[3] = {0.f, 0.f, 0.f}, g_pose[6], g_k[5], g_dis[8];
         if (any)
         {
-            project_backward(s_cam.cam, s_cam.R, view[0], view[1], view[2], d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
+            const float* sp = s_point[wave][lane];
+            project_backward(s_cam.cam, s_cam.R, sp[7], sp[8], sp[9], d0, d1, g_point, g_pose, g_k, g_dis, want_intr);
             if (want_pose)
             {
 #pragma unroll
@@ -650,8 +757,7 @@ hipError_t launch_tiles(const BackwardParams& p, int blocks, hipStream_t stream)
 
 hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream_t stream, Profiler* prof)
 {
-    const int NB = p.geom.bin_off[p.num_layers];
-    const int N  = p.num_points;
+    const int N = p.num_points;
     {
         ProfScope ps(prof, "backward_prologue", stream);
         hipLaunchKernelGGL(backward_prologue_kernel, dim3(2048), dim3(256), 0, stream, p.header, p.pair_sums,
@@ -662,9 +768,9 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
     {
         // (no points: only the background receives gradient)
         ProfScope ps(prof, "backward_tiles", stream);
-        const long long tiles8 = (((long long)NB + kNumXcd - 1) / kNumXcd) * kNumXcd;  // tiles rounded up to 8
-        const int blocks       = (int)(tiles8 * 4);
-        hipError_t e           = hipErrorInvalidValue;
+        const long long blocks8 = (((long long)p.blocks_off[p.num_layers] + 8 * kNumXcd - 1) / (8 * kNumXcd)) * (8 * kNumXcd);  // whole runs of 8 blocks x 8 XCDs
+        const int blocks        = (int)blocks8;
+        hipError_t e            = hipErrorInvalidValue;
         switch (channels)
         {
             case 3: e = launch_tiles<3>(p, blocks, stream); break;

@@ -357,6 +357,9 @@ struct BackwardParams
     const unsigned char* tags;  // [Pi, 16] (saved state) cell and place in the cell's list of every list position
     const int32_t* pair_first;  // [N] (saved state) by compact number
     float* pair_sums;  // [pairs, pair_row_floats] (workspace)
+    // blocks of the tile pass (16 x 16 pixels, 15 apart): first block of each layer, blocks per block row of each layer
+    int32_t blocks_off[TRIPS_MAX_LAYERS + 1];
+    int32_t blocks_x[TRIPS_MAX_LAYERS];
     long long pair_capacity;
     float* d_texture;
     float* d_confidence;

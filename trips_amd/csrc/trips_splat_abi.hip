@@ -553,6 +553,14 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.pair_first   = reinterpret_cast<const int32_t*>(sv + sl.pair_first);
         p.pair_sums    = reinterpret_cast<float*>(ws + bl.pair_sums);
         p.pair_capacity = (long long)bl.capacity;
+        p.blocks_off[0] = 0;
+        for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
+        {
+            // blocks of 16 x 16 pixels, 15 apart, so that every pixel is the first-15 part of exactly one block
+            const int nx = l < d.num_layers ? (g.w[l] + 14) / 15 : 0, ny = l < d.num_layers ? (g.h[l] + 14) / 15 : 0;
+            p.blocks_x[l]       = nx;
+            p.blocks_off[l + 1] = p.blocks_off[l] + nx * ny;
+        }
         for (int l = 0; l < d.num_layers; ++l) p.grad_image[l] = grad_image[l];
         p.d_texture    = grads->d_texture;
         p.d_confidence = grads->d_confidence;
