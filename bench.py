@@ -104,6 +104,87 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam
     }
 
 
+def measure_other_config(ctx, name, steps):
+    """One of the other BASELINE configurations (1, 2, 4) at its full size, beside the headline: wall time of the forward
+    and of forward + backward with inputs resident, per-kernel times, the run's counters, the algorithmic bytes of
+    SURVEY 8(d) from them and the fraction of the HBM peak they stand for. Configuration 1 is forward-only by definition."""
+    import numpy as np
+    import torch
+    from trips_amd import abi, scenes
+    from trips_amd.renderer import SplatContext
+    dev = ctx.device
+    sc = getattr(scenes, name)()
+    backward = name != "config1"
+    desc = abi.desc_for_scene(sc, train=backward)
+    f = lambda a, dt=torch.float32: torch.as_tensor(np.ascontiguousarray(a), dtype=dt).to(dev).contiguous()
+    t = dict(position=f(sc.position), point_size=f(sc.point_size), index=f(sc.index, torch.int32), texture=f(sc.texture),
+             confidence=f(sc.confidence), background=f(sc.background), poses_se3=f(sc.poses_se3, torch.float64),
+             intrinsics=f(sc.intrinsics), dropout=None)
+    tin = SplatContext.make_in(**t)
+    workspace = ctx.alloc_bytes(ctx.workspace_size(desc))
+    saved = ctx.alloc_bytes(ctx.saved_size(desc)) if backward else None
+    images = ctx.alloc_images(desc)
+    N, C, B = desc.num_points, desc.num_channels, desc.num_views
+    grads = grad_images = None
+    if backward:
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(4321)
+        grad_images = [torch.randn(im.shape, generator=gen, device=dev, dtype=torch.float32) for im in images]
+        grads = dict(d_texture=torch.zeros((C, N), device=dev), d_confidence=torch.zeros(N, device=dev),
+                     d_background=torch.zeros(C, device=dev), d_position=torch.zeros((N, 4), device=dev),
+                     d_point_size=torch.zeros(N, device=dev),
+                     d_pose=torch.zeros((desc.num_images, 6), dtype=torch.float64, device=dev),
+                     d_intrinsics=torch.zeros((desc.num_cameras, 13), device=dev))
+
+    def fwd():
+        ctx.forward(desc, tin, images, saved, workspace)
+
+    def both():
+        ctx.forward(desc, tin, images, saved, workspace)
+        ctx.backward(desc, tin, saved, grad_images, grads, workspace, overwrite_point_grads=True, clear_block_sums=True)
+
+    def wall(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    out = {"workload": sc.name + ": " + " ".join((getattr(scenes, name).__doc__ or "").split()),
+           "points": N, "views": B, "width": sc.width, "height": sc.height, "layers": desc.num_layers,
+           "list_depth": desc.list_depth, "ms_forward": round(wall(fwd), 4)}
+    if backward:
+        out["ms_forward_backward"] = round(wall(both), 4)
+        ctx.check(workspace)
+        per_view = [ctx.counters(desc, saved, b) for b in range(B)]
+        c = {k: sum(v[k] for v in per_view) for k in ("valid", "E", "R", "P")}
+        out["counters"] = c
+        ctx.profile_enable(True)
+        ctx.profile_read()
+        for _ in range(steps):
+            both()
+        torch.cuda.synchronize()
+        prof, _parts = merge_parts(ctx.profile_read())
+        ctx.profile_enable(False)
+        kern = {k: round(ms / steps, 4) for k, (ms, n) in prof.items()}  # per step: all views
+        out["kernels_ms_per_step"] = kern
+        alg = algorithmic_bytes(c, N * B, C)
+        alg_fb = sum(v for k, v in alg.items() if k != "adam_fused")
+        k_ms = sum(kern.values())
+        out["fwd_bwd_kernels_ms"] = round(k_ms, 4)
+        out["alg_bytes_fwd_bwd"] = int(alg_fb)
+        out["hbm_frac_fwd_bwd"] = round(alg_fb / (k_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if k_ms > 0 else None
+        out["points_per_s_fwd_bwd"] = round(N * B / (out["ms_forward_backward"] * 1e-3), 1)
+    else:
+        out["points_per_s_forward"] = round(N * B / (out["ms_forward"] * 1e-3), 1)
+    del workspace, saved, images, grads, grad_images, t, tin
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -120,6 +201,8 @@ def main():
     ap.add_argument("--no-net", action="store_true", help="skip the reconstruction-net forward that is reported beside the splat")
     ap.add_argument("--no-adam-variants", action="store_true",
                     help="skip the separate timing of the optimiser kernel with int32 and int64 step counters")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the block that measures BASELINE configurations 1, 2 and 4 beside the headline workload")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three plain 256 MiB device copies, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -417,6 +500,11 @@ def main():
             "net_backward_tflops": round(2 * flops / (net_bwd_ms * 1e-3) / 1e12, 1) if net_bwd_ms > 0 else None,
             "kernels": {k: round(ms / max(n, 1), 4) for k, (ms, n) in tprof.items() if k.startswith("unet_bwd")}}
 
+    # the other BASELINE configurations, each at its full size, outside the region that `value` is timed in
+    other_configs = None
+    if not args.no_other_configs:
+        other_configs = {name: measure_other_config(ctx, name, max(5, args.steps // 2)) for name in ("config1", "config2", "config4")}
+
     cpu = None
     if args.cpu_steps > 0:
         from tests import oracle_lib
@@ -482,6 +570,7 @@ def main():
             "alg_GBs_int64": round(alg_adam_i64 / (r["adam_ms"]["int64_counters"] * 1e-3) / 1e9, 1)},
         "kernels": kernels,
         "other_point_order": other_order,
+        "other_configs": other_configs,
         "unet": unet,
         "cpu_baseline": cpu,
     }

@@ -32,7 +32,10 @@ extern "C" {
 
 #define TRIPS_MAX_LAYERS 8 /* max_layers, src/lib/rendering/RenderConstants.h:38 */
 #define TRIPS_MAX_VIEWS 16
-#define TRIPS_ABI_VERSION 1
+/* 2: TripsSplatGrads gained clear_block_sums, TripsUnetDesc gained weights_packed, and the layouts of the saved state
+ * and the workspace changed (a saved state or workspace sized by a version-1 library does not fit). A caller built
+ * against another version is refused by every entry point that takes a descriptor. */
+#define TRIPS_ABI_VERSION 2
 
 /* status codes (the reference aborts through SAIGA_ASSERT instead) */
 enum {
@@ -167,7 +170,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
  * desc->max_list_entries lowers the need. The call allocates nothing on the host or the device and creates no
  * events (the per-kernel timer of trips_profile_enable does not cover it). All calls on one GPU share the one array:
  * calls that overlap on the same GPU (two streams, two threads, two contexts) race; calls on one stream are ordered
- * and each call clears the counters it relies on. trips_splat_check(ctx, NULL, stream) reports on the last such call.
+ * and each call clears the counters it relies on. trips_splat_check_static(ctx, stream) reports on the last such call.
  * The caller still passes the images and, with desc->train, the saved state. */
 #define TRIPS_STATIC_WORKSPACE_BYTES (64u << 20)
 int trips_splat_forward_static(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* in, const TripsSplatOut* out,
@@ -178,6 +181,9 @@ int trips_splat_forward_static(TripsCtx* ctx, const TripsSplatDesc* desc, const 
  * values of `index` outside [0, num_texels) (TRIPS_ERR_INVALID_ARG; such points are left out of the image, the
  * reference reads past its tables). */
 int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream);
+
+/* The same for the last trips_splat_forward_static on this context's GPU (its workspace is inside the library). */
+int trips_splat_check_static(TripsCtx* ctx, void* stream);
 
 /* Counters of the last forward of view `view` kept in the saved state: [0]=valid points, [1]=E list entries,
  * [2]=R retained entries, [3]=P pyramid pixels. Synchronises `stream`. */

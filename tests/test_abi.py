@@ -83,7 +83,7 @@ def test_ctypes_mirrors_have_c_sizes(tmp_path):
 def test_header_compiles_as_c_and_cpp(tmp_path):
     for comp, ext in (("gcc", "c"), ("g++", "cpp")):
         src = tmp_path / f"t.{ext}"
-        src.write_text('#include "trips_splat.h"\nint main(void){return TRIPS_ABI_VERSION - 1;}\n')
+        src.write_text('#include "trips_splat.h"\nint main(void){return TRIPS_ABI_VERSION - 2;}\n')
         subprocess.check_call([comp, "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src), "-o",
                                str(tmp_path / "t.o")])
 
@@ -193,15 +193,34 @@ def test_too_many_points_for_32_bit_offsets():
     lib = _lib.load()
     sc = scenes.tiny(n=10)
     d = abi.desc_for_scene(sc)
-    d.num_points = 100_000_000  # 4*N*L = 1.2e9*... exceeds 2^31-1 with 8 layers
+    d.num_points = 300_000_000  # N*L = 2.4e9 (point, layer) pairs exceed 2^31-1 with 8 layers
     d.num_layers = 8
     b = C.c_size_t(0)
     assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_UNSUPPORTED
-    # a granted capacity does not shorten the 32-bit prefix sums over the entries that could exist: still refused
+    # a granted capacity does not shorten the 32-bit prefix sums over the pairs that could exist: still refused
     d.max_list_entries = 1_000_000_000
     assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_UNSUPPORTED
-    d.num_points = 60_000_000  # 4*N*L = 1.92e9 fits
+    d.num_points = 250_000_000  # N*L = 2.0e9 fits: one key and one bin entry per pair, the four list entries of a
+    assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == 0  # pair are only counted (in 64 bits)
+
+
+def test_abi_version_mismatch_is_refused():
+    lib = _lib.load()
+    sc = scenes.tiny(n=10)
+    d = abi.desc_for_scene(sc)
+    b = C.c_size_t(0)
     assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == 0
+    d.abi_version = abi.TRIPS_ABI_VERSION - 1  # a caller built against the previous header
+    assert lib.trips_splat_workspace_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_INVALID_ARG
+    assert lib.trips_splat_saved_size(C.byref(d), C.byref(b)) == abi.TRIPS_ERR_INVALID_ARG
+    assert b"abi_version" in lib.trips_last_error_string()
+
+
+def test_check_needs_a_workspace():
+    lib = _lib.load()
+    # (no context is dereferenced before the arguments are looked at)
+    assert lib.trips_splat_check(None, None, None) == abi.TRIPS_ERR_INVALID_ARG
+    assert lib.trips_splat_check_static(None, None) == abi.TRIPS_ERR_INVALID_ARG
 
 
 def test_product_path_fails_loudly_without_gpu_or_library(monkeypatch, tmp_path):

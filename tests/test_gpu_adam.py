@@ -188,6 +188,39 @@ def test_packed_point_adam_equals_per_tensor_adam(oracle, n, c):
     assert packed.packed_state.shape[0] == m + 5 and int(packed.packed_state[m:].abs().sum()) == 0
 
 
+def test_packed_point_adam_state_dict_round_trip():
+    """A checkpoint of MyAdamPoints carries the rows of the four point parameters: an optimiser restored from
+    state_dict() continues bit for bit like the one that never stopped."""
+    from trips_amd.adam import MyAdamPoints
+    n, c = 4001, 4
+    rng = np.random.default_rng(12)
+    w0 = _point_params(n, c, rng)
+    mk = lambda: [torch.nn.Parameter(torch.as_tensor(x).cuda()) for x in w0]
+    groups = lambda ps: [{"params": [ps[0]], "lr": 1e-3}, {"params": [ps[1]], "lr": 2e-3, "adabound": True},
+                         {"params": [ps[2]], "lr": 5e-3}, {"params": [ps[3]], "lr": 1e-2}]
+    pa = mk()
+    a = MyAdamPoints(groups(pa), *pa)
+    grads = [_point_grads(n, c, rng, 0.4) for _ in range(4)]
+    for step in range(2):
+        for p, g in zip(pa, grads[step]):
+            p.grad = torch.as_tensor(g).cuda()
+        a.step()
+    sd = a.state_dict()
+    assert sd["packed_state"] is not None and sd["packed_state"].shape[0] == n
+    pb = [torch.nn.Parameter(p.detach().clone()) for p in pa]
+    b = MyAdamPoints(groups(pb), *pb)
+    b.load_state_dict(sd)
+    for step in range(2, 4):
+        for opt, ps in ((a, pa), (b, pb)):
+            for p, g in zip(ps, grads[step]):
+                p.grad = torch.as_tensor(g).cuda()
+            opt.step()
+    torch.cuda.synchronize()
+    for x, y in zip(pa, pb):
+        assert torch.equal(x.data, y.data)
+    assert torch.equal(a.packed_state, b.packed_state)
+
+
 def test_packed_point_adam_argument_checks():
     from trips_amd import _lib
     from trips_amd.renderer import get_context

@@ -32,7 +32,9 @@ def _both(sc, desc):
     rc = run.ctx.lib.trips_splat_forward_static(run.ctx.ctx, C.byref(desc), C.byref(run.tin), C.byref(out), stream)
     assert rc == abi.TRIPS_OK, run.ctx.lib.trips_last_error_string()
     torch.cuda.synchronize()
-    assert run.ctx.lib.trips_splat_check(run.ctx.ctx, None, stream) == abi.TRIPS_OK
+    assert run.ctx.lib.trips_splat_check_static(run.ctx.ctx, stream) == abi.TRIPS_OK
+    # a forgotten workspace is an error, not a silent look at the static one
+    assert run.ctx.lib.trips_splat_check(run.ctx.ctx, None, stream) == abi.TRIPS_ERR_INVALID_ARG
     for l, (a, b) in enumerate(zip(images, want)):
         np.testing.assert_array_equal(a.cpu().numpy(), b, err_msg=f"layer {l}")
     if desc.train:
@@ -49,6 +51,52 @@ def test_static_workspace_forward_twice_then_smaller():
     small = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=8, seed=78)
     _both(small, abi.desc_for_scene(small))
     _both(small, abi.desc_for_scene(small, train=False))  # no saved state: counters and records live in the workspace
+
+
+def test_static_workspace_call_allocates_nothing_and_replays_from_a_graph():
+    """The property the entry point exists for: no device memory is taken by the call, and it can be recorded into a
+    HIP graph and replayed."""
+    from tests.gpu_util import GpuRun
+    sc = scenes.tiny(n=3000, w=64, h=48, f=60.0, num_layers=3, list_depth=8, seed=79)
+    desc = abi.desc_for_scene(sc, train=False)
+    run = GpuRun(sc, desc)
+    want = run.forward()
+    images = run.ctx.alloc_images(desc, fill=float("nan"))
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    run.ctx.forward_static(desc, run.tin, images, None)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, "the call changed the free device memory"
+    for a, b in zip(images, want):
+        np.testing.assert_array_equal(a.cpu().numpy(), b)
+    # recorded once, replayed twice with eager work in between
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            run.ctx.forward_static(desc, run.tin, images, None)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        for im in images:
+            im.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(images, want):
+            np.testing.assert_array_equal(a.cpu().numpy(), b)
+
+
+def test_static_workspace_train_forward_is_gated_on_the_forward_share_only():
+    """In train mode trips_splat_workspace_size covers the backward's tables as well; the static entry point only runs
+    the forward and must not refuse a scene on their account."""
+    from trips_amd.renderer import get_context
+    ctx = get_context(0)
+    sc = scenes.tiny(n=3000, w=640, h=480, f=300.0, num_layers=6, list_depth=16, seed=80)
+    d = abi.desc_for_scene(sc, train=True, max_list_entries=200_000)
+    d_eval = abi.desc_for_scene(sc, train=False, max_list_entries=200_000)
+    assert ctx.workspace_size(d_eval) <= abi.TRIPS_STATIC_WORKSPACE_BYTES
+    _both(sc, d)
 
 
 def test_static_workspace_rejects_scenes_beyond_its_size():

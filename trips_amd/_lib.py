@@ -15,7 +15,7 @@ SYMBOLS = [
     "trips_version", "trips_last_error_string", "trips_ctx_create", "trips_ctx_destroy", "trips_splat_layer_sizes",
     "trips_splat_workspace_size", "trips_splat_saved_size", "trips_splat_forward", "trips_splat_forward_static",
     "trips_splat_backward",
-    "trips_splat_check", "trips_splat_counters", "trips_splat_export_lists", "trips_splat_export_points",
+    "trips_splat_check", "trips_splat_check_static", "trips_splat_counters", "trips_splat_export_lists", "trips_splat_export_points",
     "trips_adam_step_fused", "trips_adam_points_state_size", "trips_adam_step_points", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
 ]
 # every symbol include/trips_unet.h declares
@@ -56,6 +56,7 @@ def load():
     lib.trips_splat_backward.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), C.POINTER(abi.TripsSplatIn), vp,
                                          C.POINTER(vp), C.POINTER(abi.TripsSplatGrads), vp, C.c_size_t, vp]
     lib.trips_splat_check.argtypes = [vp, vp, vp]
+    lib.trips_splat_check_static.argtypes = [vp, vp]
     lib.trips_splat_counters.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), vp, i32, C.POINTER(i64), vp]
     lib.trips_splat_export_lists.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), vp, i32, vp, vp, vp, vp]
     lib.trips_splat_export_points.argtypes = [vp, C.POINTER(abi.TripsSplatDesc), vp, i32, vp, vp, vp, vp, vp]

@@ -7,7 +7,7 @@ import ctypes as C
 
 TRIPS_MAX_LAYERS = 8
 TRIPS_MAX_VIEWS = 16
-TRIPS_ABI_VERSION = 1
+TRIPS_ABI_VERSION = 2
 TRIPS_STATIC_WORKSPACE_BYTES = 64 << 20  # workspace inside the library, trips_splat_forward_static
 TRIPS_STEPS_I64, TRIPS_STEPS_I32 = 0, 1
 TRIPS_PROFILE_MAX_KERNELS = 32

@@ -144,6 +144,19 @@ class MyAdamPoints(MyAdam):
         self.packed_state = None
         self._zero_grads = {}
 
+    def state_dict(self):
+        """MyAdam's state dict plus the rows of the four point parameters (`packed_state`) and their step counts, which
+        live outside the per-parameter state."""
+        d = super().state_dict()
+        d["packed_state"] = None if self.packed_state is None else self.packed_state.clone()
+        return d
+
+    def load_state_dict(self, state_dict):
+        state_dict = dict(state_dict)
+        rows = state_dict.pop("packed_state", None)
+        super().load_state_dict(state_dict)
+        self.packed_state = None if rows is None else rows.to(self._packed[0].device).contiguous().clone()
+
     def _geometry(self):
         position, point_size, texture, confidence = self._packed
         n = int(position.shape[0])

@@ -406,6 +406,45 @@ bool MyAdam::describe(Tensor& p, OptimizerParamGroup& group, bool packed, TripsA
     return true;
 }
 
+void MyAdam::save(serialize::OutputArchive& archive) const
+{
+    int64_t index = 0;
+    for (const auto& group : param_groups_)
+        for (const auto& p : group.params())
+        {
+            const std::string key = std::to_string(index++);
+            auto it               = state_.find(p.unsafeGetTensorImpl());
+            if (it == state_.end()) continue;
+            const auto& st = static_cast<const MyAdamParamState&>(*it->second);
+            archive.write(key + "/first_moments", st.first_moments());
+            archive.write(key + "/second_moments", st.second_moments());
+            archive.write(key + "/param_steps", st.param_steps());
+            archive.write(key + "/current_step", torch::tensor(st.current_step(), torch::kInt64));
+        }
+}
+
+void MyAdam::load(serialize::InputArchive& archive)
+{
+    int64_t index = 0;
+    for (auto& group : param_groups_)
+        for (auto& p : group.params())
+        {
+            const std::string key = std::to_string(index++);
+            Tensor m, v, steps, current;
+            if (!archive.try_read(key + "/first_moments", m)) continue;
+            archive.read(key + "/second_moments", v);
+            archive.read(key + "/param_steps", steps);
+            archive.read(key + "/current_step", current);
+            TORCH_CHECK(m.sizes() == p.sizes(), "MyAdam::load: state of parameter ", key, " does not fit its shape");
+            auto st = std::make_unique<MyAdamParamState>();
+            st->first_moments(m.to(p.device()).contiguous());
+            st->second_moments(v.to(p.device()).contiguous());
+            st->param_steps(steps.to(p.device()).contiguous());
+            st->current_step(current.item<int64_t>());
+            state_[p.unsafeGetTensorImpl()] = std::move(st);
+        }
+}
+
 torch::Tensor MyAdam::step(LossClosure closure)
 {
     NoGradGuard no_grad;
@@ -528,6 +567,22 @@ torch::Tensor MyAdamPoints::step(LossClosure closure)
         check(trips_adam_step_fused(context_for(any), descs.data(), (int)descs.size(), current_stream(any)),
               "trips_adam_step_fused");
     return loss;
+}
+
+void MyAdamPoints::save(serialize::OutputArchive& archive) const
+{
+    MyAdam::save(archive);  // (the four packed parameters have no per-tensor state and are passed over)
+    if (packed_state.defined()) archive.write("points/packed_state", packed_state);
+    archive.write("points/steps", torch::tensor(std::vector<int64_t>(packed_steps_, packed_steps_ + 4), torch::kInt64));
+}
+
+void MyAdamPoints::load(serialize::InputArchive& archive)
+{
+    MyAdam::load(archive);
+    Tensor rows, steps;
+    if (archive.try_read("points/packed_state", rows)) packed_state = rows.to(packed_[0].device()).contiguous();
+    archive.read("points/steps", steps);
+    for (int i = 0; i < 4; ++i) packed_steps_[i] = steps[i].item<int64_t>();
 }
 
 void MyAdamPoints::shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep)

@@ -174,6 +174,10 @@ class MyAdam : public Optimizer
     torch::Tensor step(LossClosure closure = nullptr) override;
     virtual void shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep);
     virtual void appendToInternalState(int param_group_index, int new_size);
+    // The state of every parameter (moments, per-element step counters, step count) under "<index in group order>/...";
+    // the reference leaves both unimplemented (MyAdam.cu:417-425). A checkpoint resumes bit for bit.
+    void save(serialize::OutputArchive& archive) const override;
+    void load(serialize::InputArchive& archive) override;
 
    protected:
     // one parameter's step description for the library (creates its state on first use unless `packed`)
@@ -194,6 +198,9 @@ class MyAdamPoints : public MyAdam
     torch::Tensor step(LossClosure closure = nullptr) override;
     void shrinkInternalState(int param_group_index, torch::Tensor indices_to_keep) override;
     void appendToInternalState(int param_group_index, int new_size) override;
+    // the per-tensor state of the other parameters as MyAdam saves it, plus the rows and the step counts of the four
+    void save(serialize::OutputArchive& archive) const override;
+    void load(serialize::InputArchive& archive) override;
     torch::Tensor packed_state;  // [N, row bytes / 4] int32, defined after the first step
 
    private:

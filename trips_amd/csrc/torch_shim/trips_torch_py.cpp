@@ -210,5 +210,19 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
                                                                             tx.confidence_value_of_point,
                                                                             torch::optim::MyAdamOptions(lr));
              })
-        .def("adam_step", [](Session& s) { s.optimizer->step(); });
+        .def("adam_step", [](Session& s) { s.optimizer->step(); })
+        .def("adam_save",
+             [](Session& s, const std::string& path)
+             {
+                 torch::serialize::OutputArchive archive;
+                 s.optimizer->save(archive);
+                 archive.save_to(path);
+             })
+        .def("adam_load",
+             [](Session& s, const std::string& path)
+             {
+                 torch::serialize::InputArchive archive;
+                 archive.load_from(path);
+                 s.optimizer->load(archive);
+             });
 }

@@ -101,11 +101,13 @@ int check_desc(const TripsSplatDesc* d)
         if (v.camera_index < 0 || v.camera_index >= d->num_cameras)
             return fail(TRIPS_ERR_INVALID_ARG, "view %d: camera_index %d out of range", b, v.camera_index);
     }
-    // List entries and their prefix sums are 32-bit: no scan may exceed the worst case of 4 N L entries, whatever the
-    // capacity the caller grants (a smaller max_list_entries only drops entries, it does not shorten the scans).
-    if (4ll * d->num_points * d->num_layers > 0x7fffffffll)
-        return fail(TRIPS_ERR_UNSUPPORTED, "4*N*L = %lld list entries exceed 2^31-1", 4ll * d->num_points * d->num_layers);
-    if (d->max_list_entries > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "max_list_entries exceeds 2^31-1");
+    // A (point, layer) pair is filed once (one bin entry, one key, one row of the backward), and the prefix sums over
+    // the pairs are 32-bit: no scan may exceed the worst case of N L pairs, whatever the capacity the caller grants (a
+    // smaller max_list_entries only drops entries, it does not shorten the scans). The list entries that the counters
+    // report, four per pair, are counted in 64 bits.
+    if ((long long)d->num_points * d->num_layers > 0x7fffffffll)
+        return fail(TRIPS_ERR_UNSUPPORTED, "N*L = %lld (point, layer) pairs exceed 2^31-1", (long long)d->num_points * d->num_layers);
+    if (d->max_list_entries > 4ll * 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "max_list_entries exceeds 4 (2^31-1)");
     {
         // one LDS counter per 32 x 32 tile of the pyramid in the binning kernels
         long long bins = 0;
@@ -480,12 +482,17 @@ int trips_splat_forward_static(TripsCtx* ctx, const TripsSplatDesc* desc, const 
                                void* stream)
 {
     if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
-    size_t need = 0;
-    if (int e = trips_splat_workspace_size(desc, &need)) return e;
+    // what the forward itself carves out of a workspace (the backward's tables are not part of it: the backward takes a
+    // caller-owned workspace)
+    if (int e = check_desc(desc)) return e;
+    if (pyramid_pixels_checked(*desc) > 0x7fffffffll) return fail(TRIPS_ERR_UNSUPPORTED, "pyramid has more than 2^31-1 pixels");
+    PyramidGeom g;
+    make_geom(*desc, g);
+    const size_t need = workspace_layout(*desc, g).bytes;
     if (need > (size_t)TRIPS_STATIC_WORKSPACE_BYTES)
         return fail(TRIPS_ERR_WORKSPACE_SMALL,
-                    "this scene needs %zu bytes of workspace, the static one holds %zu: use trips_splat_forward with a "
-                    "caller-owned workspace, or lower max_list_entries",
+                    "the forward of this scene needs %zu bytes of workspace, the static one holds %zu: use trips_splat_forward "
+                    "with a caller-owned workspace, or lower max_list_entries",
                     need, (size_t)TRIPS_STATIC_WORKSPACE_BYTES);
     // no event creation either: the per-kernel timer is left out of this entry point
     return forward_impl(ctx, desc, in, out, ctx->static_scratch, (size_t)TRIPS_STATIC_WORKSPACE_BYTES, stream, false);
@@ -581,11 +588,12 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
     return TRIPS_OK;
 }
 
-int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
+}  // extern "C"
+
+namespace
 {
-    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
-    const void* header_owner = workspace ? workspace : ctx->static_scratch;  // NULL: the last trips_splat_forward_static
-    if (!header_owner) return fail(TRIPS_ERR_INVALID_ARG, "workspace is NULL");
+int check_status_block(const void* header_owner, void* stream_)
+{
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     ViewHeader h;
     hipError_t e = hipMemcpyAsync(&h, header_owner, sizeof(h), hipMemcpyDeviceToHost, stream);
@@ -595,6 +603,23 @@ int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
     if (h.bad_index) return fail(TRIPS_ERR_INVALID_ARG, "index holds values outside [0, num_texels): those points were left out");
     if (h.overflow) return fail(TRIPS_ERR_LIST_OVERFLOW, "%llu list entries dropped: max_list_entries too small", 4 * h.overflow);
     return TRIPS_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int trips_splat_check(TripsCtx* ctx, const void* workspace, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (!workspace) return fail(TRIPS_ERR_INVALID_ARG, "workspace is NULL (trips_splat_check_static reports on the static one)");
+    return check_status_block(workspace, stream_);
+}
+
+int trips_splat_check_static(TripsCtx* ctx, void* stream_)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (!ctx->static_scratch) return fail(TRIPS_ERR_INVALID_ARG, "this context has no static workspace");
+    return check_status_block(ctx->static_scratch, stream_);
 }
 
 int trips_splat_counters(TripsCtx* ctx, const TripsSplatDesc* desc, const void* saved, int view, int64_t counters[4],

@@ -129,8 +129,14 @@ class SplatContext:
                                                  _stream_ptr(self.device)))
 
     def check(self, workspace):
-        """workspace None: the library's static workspace (after forward_static)."""
+        """What the last forward on `workspace` found on the device (list overflow, bad descriptor columns); raises."""
+        if workspace is None:
+            raise ValueError("check(None): pass the workspace of the forward, or call check_static() after forward_static")
         _lib.check(self.lib.trips_splat_check(self.ctx, _ptr(workspace), _stream_ptr(self.device)))
+
+    def check_static(self):
+        """The same for the last forward_static on this GPU."""
+        _lib.check(self.lib.trips_splat_check_static(self.ctx, _stream_ptr(self.device)))
 
     def counters(self, desc, saved, view=0):
         c = (C.c_int64 * 4)()
