@@ -92,11 +92,11 @@ constexpr int kBlockCells  = kBlockSide - 1;           // cells per side whose f
 constexpr int kBlockPixels = kBlockSide * kBlockSide;  // 256
 constexpr int kListMax     = 16;                       // entries of a pixel's list (the larger list depth)
 
-// LDS of a block: {dL/dalpha, T alpha} per (pixel, list position); dL/dimage per pixel; per (cell, place in the cell's
-// sorted list) the list positions of that point's entry in its four corner pixels (0xFF: none) and its compact number
+// LDS of a block: {dL/dalpha, T alpha} per (list position, pixel); dL/dimage per (channel, pixel); per (place in the
+// cell's sorted list, cell) the list positions of that point's entry in its four corner pixels (0xFF: none). The pixel or the cell is the fastest index everywhere: neighbouring lanes, neighbouring banks.
 __host__ __device__ constexpr size_t tiles_lds_bytes(int cpad)
 {
-    return (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * cpad * 4 + (size_t)kBlockCells * kBlockCells * kCellKeep * 8;
+    return (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * cpad * 4 + (size_t)kBlockCells * kBlockCells * kCellKeep * 4;
 }
 
 template <int C>
@@ -113,7 +113,6 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     float2* const s_ex     = reinterpret_cast<float2*>(s_mem);
     float* const s_g       = reinterpret_cast<float*>(s_mem + (size_t)kBlockPixels * kListMax * 8);
     unsigned* const s_rank = reinterpret_cast<unsigned*>(s_mem + (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * CPAD * 4);
-    unsigned* const s_cid  = s_rank + kBlockCells * kBlockCells * kCellKeep;
     __shared__ double s_acc[4][C];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -204,7 +203,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             }
         }
 #pragma unroll
-        for (int c = 0; c < CPAD; ++c) s_g[t * CPAD + c] = c < C ? g[c] : 0.f;
+        for (int c = 0; c < CPAD; ++c) s_g[c * kBlockPixels + t] = c < C ? g[c] : 0.f;
         float sbg = 0.f;
 #pragma unroll
         for (int c = 0; c < C; ++c) sbg += p.background[c] * g[c];
@@ -302,7 +301,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 {
                     const float dem        = 1.f / (1.f - A[j] + 1e-9f);
                     const float grad_alpha = Tr[j] * S[j] - (later + bg_term) * dem;
-                    s_ex[t * kListMax + j] = make_float2(grad_alpha, ta);
+                    s_ex[j * kBlockPixels + t] = make_float2(grad_alpha, ta);
                     const unsigned tag     = (tagw[j / 4] >> (8 * (j & 3))) & 0xFFu;
                     const int w = (int)(tag >> 4) & 3, place = (int)(tag & 15u);
                     // the cell the entry came from: (x-1, y-1), (x, y-1), (x-1, y), (x, y) for w = 0..3; this pixel is corner
@@ -310,9 +309,8 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                     const int cxl = px - 1 + (w & 1), cyl = py - 1 + (w >> 1);
                     if ((unsigned)cxl < (unsigned)kBlockCells && (unsigned)cyl < (unsigned)kBlockCells)
                     {
-                        const int slot = (cyl * kBlockCells + cxl) * kCellKeep + place;
+                        const int slot = place * (kBlockCells * kBlockCells) + cyl * kBlockCells + cxl;
                         reinterpret_cast<unsigned char*>(s_rank)[slot * 4 + (3 - w)] = (unsigned char)j;
-                        s_cid[slot] = (unsigned)id[j];  // (the four corners write the same number)
                     }
                 }
                 later += ta * S[j];
@@ -334,15 +332,28 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
 #pragma unroll
         for (int place = 0; place < kCellKeep; ++place)
         {
-            words[place]      = is_cell ? s_rank[cell * kCellKeep + place] : ~0u;
+            words[place]      = is_cell ? s_rank[place * (kBlockCells * kBlockCells) + cell] : ~0u;
             first_pair[place] = 0;
             if (__ballot(words[place] != ~0u))
             {
-#ifdef EXP_NOPF
-                if (words[place] != ~0u) first_pair[place] = (int)s_cid[cell * kCellKeep + place];
-#else
-                if (words[place] != ~0u) first_pair[place] = p.pair_first[s_cid[cell * kCellKeep + place]];
-#endif
+                if (words[place] != ~0u)
+                {
+                    // the point's compact number: from the list of the first corner pixel that retained it
+                    const unsigned w4 = words[place];
+                    const int corner  = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
+                    const unsigned r  = (w4 >> (8 * corner)) & 0xFFu;
+                    const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, x0 + cxl + (corner & 1), y0 + cyl + (corner >> 1));
+                    first_pair[place]  = p.lists[((size_t)pix << kshift) + r];
+                }
+            }
+        }
+        // the numbers of those points' first pairs
+#pragma unroll
+        for (int place = 0; place < kCellKeep; ++place)
+        {
+            if (__ballot(words[place] != ~0u))
+            {
+                if (words[place] != ~0u) first_pair[place] = p.pair_first[first_pair[place]];
             }
         }
 #pragma unroll
@@ -362,10 +373,10 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 ga[corner]       = 0.f;
                 if (r == 0xFFu) continue;
                 const int tp   = (cyl + (corner >> 1)) * kBlockSide + cxl + (corner & 1);
-                const float2 e = s_ex[tp * kListMax + (int)r];
+                const float2 e = s_ex[(int)r * kBlockPixels + tp];
                 ga[corner]     = e.x;
 #pragma unroll
-                for (int c = 0; c < C; ++c) tex[c] += e.y * s_g[tp * CPAD + c];
+                for (int c = 0; c < C; ++c) tex[c] += e.y * s_g[c * kBlockPixels + tp];
             }
             if (pair < p.pair_capacity)
             {
@@ -737,7 +748,10 @@ __global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader
 template <int C>
 hipError_t launch_tiles(const BackwardParams& p, int blocks, hipStream_t stream)
 {
-    const size_t lds = tiles_lds_bytes((C + 3) & ~3);
+#ifndef EXP_LDS_EXTRA
+#define EXP_LDS_EXTRA 0
+#endif
+    const size_t lds = tiles_lds_bytes((C + 3) & ~3) + EXP_LDS_EXTRA;
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&backward_tiles_kernel<C>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((backward_tiles_kernel<C>), dim3(blocks), dim3(256), lds, stream, p);

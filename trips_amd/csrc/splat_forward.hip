@@ -992,41 +992,45 @@ __device__ __forceinline__ u64 shfl16(u64 v, int src)
 }
 
 // The 16 smallest of key_at(0 .. readable - 1) for each of the wavefront's four 16-lane rows, ascending over the row's
-// lanes (all-ones where the row has fewer keys).
+// lanes (all-ones where the row has fewer keys). A chunk of 16 further keys is sorted and merged only if one of them
+// beats the current 16th; most chunks of a long list are passed over, so the loop runs at the latency of its loads:
+// four chunks are requested together and the next four are in flight while these are looked at. The first 16 + 64
+// keys can be requested ahead of the call (row_top16_first), e.g. while the rows still work on other lists.
+struct RowKeys
+{
+    u64 k0;              // keys 0..15
+    u64 f0, f1, f2, f3;  // keys 16..79
+};
 template <typename KeyAt>
-__device__ __forceinline__ u64 row_top16(KeyAt&& key_at, int readable)
+__device__ __forceinline__ void row_load4(KeyAt&& key_at, int readable, int base, u64& f0, u64& f1, u64& f2, u64& f3)
+{
+    const int i = base + (int)(threadIdx.x & 15);
+    const u64 kInf = ~0ull;
+    f0 = i < readable ? key_at(i) : kInf;
+    f1 = i + 16 < readable ? key_at(i + 16) : kInf;
+    f2 = i + 32 < readable ? key_at(i + 32) : kInf;
+    f3 = i + 48 < readable ? key_at(i + 48) : kInf;
+}
+template <typename KeyAt>
+__device__ __forceinline__ RowKeys row_top16_first(KeyAt&& key_at, int readable)
+{
+    RowKeys r;
+    const int sub = threadIdx.x & 15;
+    r.k0 = sub < readable ? key_at(sub) : ~0ull;
+    row_load4(key_at, readable, 16, r.f0, r.f1, r.f2, r.f3);
+    return r;
+}
+template <typename KeyAt>
+__device__ __forceinline__ u64 row_top16(KeyAt&& key_at, int readable, const RowKeys& first)
 {
     const int lane = threadIdx.x & 63;
-    const int sub = lane & 15, grp = lane >> 4;
-    const u64 kInf = ~0ull;
-    u64 best;
+    const int grp  = lane >> 4;
     int maxlen = readable;
     maxlen     = max(maxlen, __shfl_xor(maxlen, 16));
     maxlen     = max(maxlen, __shfl_xor(maxlen, 32));
     const u64 grp_mask = 0xFFFFull << (grp * 16);
     maxlen             = __builtin_amdgcn_readfirstlane(maxlen);
-    {
-        u64 k = kInf;
-        if (sub < readable) k = key_at(sub);
-        best = row_sort16(k);
-    }
-    // A chunk of 16 further keys is sorted and merged only if one of them beats the current 16th; most chunks of a
-    // long list are passed over, so the loop runs at the latency of its loads: four chunks are requested together
-    // and the next four are in flight while these are looked at.
-    struct Four
-    {
-        u64 k0, k1, k2, k3;
-    };
-    auto load4 = [&](int base)
-    {
-        Four f;
-        const int i = base + sub;
-        f.k0        = i < readable ? key_at(i) : kInf;
-        f.k1        = i + 16 < readable ? key_at(i + 16) : kInf;
-        f.k2        = i + 32 < readable ? key_at(i + 32) : kInf;
-        f.k3        = i + 48 < readable ? key_at(i + 48) : kInf;
-        return f;
-    };
+    u64 best = row_sort16(first.k0);
     auto consider = [&](u64 k)
     {
         const u64 worst = shfl16(best, 15);
@@ -1041,18 +1045,24 @@ __device__ __forceinline__ u64 row_top16(KeyAt&& key_at, int readable)
     };
     if (maxlen > 16)
     {
-        Four cur = load4(16), nxt = cur;
+        u64 c0 = first.f0, c1 = first.f1, c2 = first.f2, c3 = first.f3;
+        u64 n0 = c0, n1 = c1, n2 = c2, n3 = c3;
         for (int base = 16; base < maxlen; base += 64)
         {
-            if (base + 64 < maxlen) nxt = load4(base + 64);
-            consider(cur.k0);
-            if (base + 16 < maxlen) consider(cur.k1);
-            if (base + 32 < maxlen) consider(cur.k2);
-            if (base + 48 < maxlen) consider(cur.k3);
-            cur = nxt;
+            if (base + 64 < maxlen) row_load4(key_at, readable, base + 64, n0, n1, n2, n3);
+            consider(c0);
+            if (base + 16 < maxlen) consider(c1);
+            if (base + 32 < maxlen) consider(c2);
+            if (base + 48 < maxlen) consider(c3);
+            c0 = n0, c1 = n1, c2 = n2, c3 = n3;
         }
     }
     return best;
+}
+template <typename KeyAt>
+__device__ __forceinline__ u64 row_top16(KeyAt&& key_at, int readable)
+{
+    return row_top16(key_at, readable, row_top16_first(key_at, readable));
 }
 
 // Reduction pass over the segments of long lists (tile_lists_kernel hands them out): a 16-lane row keeps the 16
@@ -1109,10 +1119,17 @@ __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
             }
         }
     }
-    // ---- longer lists: one cell per 16-lane row, four at a time ----
+    // ---- longer lists: one cell per 16-lane row, four at a time; the first keys of the next four are requested
+    // before these four are worked on ----
     u64 todo = __ballot(rd > kLaneSortMax);
     const int sub = lane & 15, grp = lane >> 4;
-    while (todo)
+    struct Pass
+    {
+        u64* base;
+        int readable;
+        RowKeys first;
+    };
+    auto next_pass = [&]()
     {
         int src = -1;  // the lane whose cell this row takes
 #pragma unroll
@@ -1129,10 +1146,25 @@ __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
         const int row_rd    = __shfl(rd, from);  // (by every lane: a source lane may sit in a row that has no cell)
         const unsigned b_lo = (unsigned)__shfl((int)(unsigned)(uintptr_t)base, from);
         const unsigned b_hi = (unsigned)__shfl((int)(unsigned)((uintptr_t)base >> 32), from);
-        u64* const row_base = reinterpret_cast<u64*>(((uintptr_t)b_hi << 32) | (uintptr_t)b_lo);
-        const int readable  = src >= 0 ? row_rd : 0;
-        const u64 best      = row_top16([&](int i) { return row_base[i]; }, readable);
-        if (sub < min(readable, kCellKeep)) row_base[sub] = best;
+        Pass ps;
+        ps.base     = reinterpret_cast<u64*>(((uintptr_t)b_hi << 32) | (uintptr_t)b_lo);
+        ps.readable = src >= 0 ? row_rd : 0;
+        u64* const rb = ps.base;
+        ps.first    = row_top16_first([&](int i) { return rb[i]; }, ps.readable);
+        return ps;
+    };
+    if (!todo) return;
+    Pass cur = next_pass();
+    for (;;)
+    {
+        const bool more = todo != 0;
+        Pass nxt        = cur;
+        if (more) nxt = next_pass();
+        u64* const rb  = cur.base;
+        const u64 best = row_top16([&](int i) { return rb[i]; }, cur.readable, cur.first);
+        if (sub < min(cur.readable, kCellKeep)) rb[sub] = best;
+        if (!more) break;
+        cur = nxt;
     }
 }
 
