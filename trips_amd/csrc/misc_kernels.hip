@@ -495,7 +495,7 @@ __global__ __launch_bounds__(256) void export_lists_kernel(const PyramidGeom g, 
     if (out_lists)
         for (int k = 0; k < K; ++k)
         {
-            const int cid                = k < filled ? lists[(size_t)ip * K + k] : -1;  // compact number of the point
+            const int cid                = k < filled ? lists[list_word((unsigned)ip, k, K)] : -1;  // compact number of the point
             out_lists[(size_t)r * K + k] = cid >= 0 ? pid_of[cid] : -1;
         }
 }

@@ -129,7 +129,6 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     const int lw = p.geom.w[layer], lh = p.geom.h[layer];
     const int x0 = bxi * kBlockCells, y0 = byi * kBlockCells;  // the block's first pixel
     const float* const gi = p.grad_image[layer];
-    const int kshift      = p.list_depth == 16 ? 4 : 3;
 
     // no entry yet under any (cell, place)
     for (int i = threadIdx.x; i < kBlockCells * kBlockCells * kCellKeep / 4; i += 256)
@@ -154,14 +153,16 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
         // requested before the first is looked at; list positions past the retained ones hold anything and are not used
         int word = 0;
         int id[kListMax];
+        const vi4* mine = nullptr;  // the pixel's list: positions 4q .. 4q + 3 at mine[64 q]
         unsigned tagw[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int j = 0; j < kListMax; ++j) id[j] = 0;
         if (inside)
         {
             word = p.retained[pix];
+            mine = reinterpret_cast<const vi4*>(p.lists + list_word(pix, 0, p.list_depth));
             {
-                const vi4 v = __builtin_nontemporal_load(reinterpret_cast<const vi4*>(p.lists + ((size_t)pix << kshift)));
+                const vi4 v = __builtin_nontemporal_load(mine);
                 id[0] = v.x, id[1] = v.y, id[2] = v.z, id[3] = v.w;
             }
             const vu4 v = __builtin_nontemporal_load(reinterpret_cast<const vu4*>(p.tags) + pix);
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
         {
             if (4 * q < mmax && 4 * q < m)
             {
-                const vi4 v = __builtin_nontemporal_load(reinterpret_cast<const vi4*>(p.lists + ((size_t)pix << kshift)) + q);
+                const vi4 v = __builtin_nontemporal_load(mine + (q << 6));
                 id[4 * q] = v.x, id[4 * q + 1] = v.y, id[4 * q + 2] = v.z, id[4 * q + 3] = v.w;
             }
         }
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                     const int corner  = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
                     const unsigned r  = (w4 >> (8 * corner)) & 0xFFu;
                     const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, x0 + cxl + (corner & 1), y0 + cyl + (corner >> 1));
-                    first_pair[place]  = p.lists[((size_t)pix << kshift) + r];
+                    first_pair[place]  = p.lists[list_word(pix, (int)r, p.list_depth)];
                 }
             }
         }

@@ -1410,11 +1410,12 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
                                                  ((unsigned)min(length, kMaxExportedLength) << (2 * kRetainedBits)))
                                          : 0,
                                     p.retained + pix);
-        const int kshift = p.list_depth == 16 ? 4 : 3;
-        vi4* row         = reinterpret_cast<vi4*>(p.lists + ((size_t)(unsigned)pix << kshift));
+        // four positions at a time, the block's 64 pixels side by side (list_word)
+        vi4* const mine = reinterpret_cast<vi4*>(p.lists + list_word((unsigned)pix, 0, p.list_depth));
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            if (4 * q < n) __builtin_nontemporal_store(vi4{(int)id[4 * q], (int)id[4 * q + 1], (int)id[4 * q + 2], (int)id[4 * q + 3]}, row + q);
+            if (4 * q < nmax && 4 * q < n)
+                __builtin_nontemporal_store(vi4{(int)id[4 * q], (int)id[4 * q + 1], (int)id[4 * q + 2], (int)id[4 * q + 3]}, mine + (q << 6));
         if (n > 0) __builtin_nontemporal_store(vu4{tagw[0], tagw[1], tagw[2], tagw[3]}, reinterpret_cast<vu4*>(p.tags) + (unsigned)pix);
     }
 }

@@ -171,6 +171,17 @@ __device__ inline int pix_index_mul24(const PyramidGeom& g, int layer, int x, in
     return (bin << (2 * kTileShift)) | ((y & (kTile - 1)) << kTileShift) | (x & (kTile - 1));
 }
 
+// The saved lists are stored by 8 x 8 blocks of pixels, four list positions at a time: the 64 pixels of a block (one
+// wavefront of the blend) keep positions 4q .. 4q + 3 of their lists in 64 consecutive 16-byte words, so that the
+// wavefront writes them as one kilobyte and the eight pixels of a row of the block share a line. Word of (pixel pix,
+// position j) of lists of depth K:
+__host__ __device__ inline size_t list_word(unsigned pix, int j, int K)
+{
+    const unsigned x = pix & (kTile - 1), y = (pix >> kTileShift) & (kTile - 1), bin = pix >> (2 * kTileShift);
+    const unsigned block = (bin << 4) | ((y >> 3) << 2) | (x >> 3), lane = ((y & 7) << 3) | (x & 7);
+    return ((((size_t)block * (unsigned)(K >> 2) + (unsigned)(j >> 2)) << 6) + lane) * 4 + (unsigned)(j & 3);
+}
+
 // What the pixels of one 32 x 32 tile share: its layer, that layer's size and the tile's first pixel.
 struct TileCtx
 {
@@ -234,7 +245,7 @@ struct SavedLayout
     size_t header;    // ViewHeader
     size_t rec;       // float [N * record_floats]
     size_t prec;      // float [N * kPointRecordFloats]
-    size_t lists;     // int32 [Pi, K]   Pi = number of bins * 1024 (tile-major, padded); a row's positions past its ids are undefined
+    size_t lists;     // int32 [Pi / 64, K / 4, 64, 4] (see list_word)  Pi = number of bins * 1024 (tile-major, padded); a pixel's positions past its ids are undefined
     size_t retained;  // int32 [Pi]: retained entries in bits 0..4, list positions that hold an id (min(length, K)) in bits 5..9, list length from bit 10
     size_t tags;      // uint8 [Pi, 16]  where a list position came from: which of the pixel's four cells (bits 4..5) and its
                       // place in that cell's sorted list (bits 0..3); a row's positions past its ids are undefined
