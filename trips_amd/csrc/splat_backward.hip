@@ -7,18 +7,19 @@
 // (3 position + 1 size + 1 confidence + C descriptor atomics per retained entry). Scattered atomics run at about
 // 2e10 per second on this GPU, and what bounds the kernels of this path is the number of scattered memory requests,
 // whatever their size. So the four pixels of a point's footprint meet in LDS, not in memory:
-//   1. tiles: a workgroup owns 16 x 16 cells of a tile (a cell = the footprints that start at that pixel) and walks
-//      the 17 x 17 pixels they cover, one pixel per lane (its right column and bottom row are walked again by the
-//      neighbours). A lane recomputes alpha and transmittance of its pixel's retained entries from the per-point
+//   1. tiles: a workgroup walks a block of 16 x 16 pixels, one pixel per lane, and owns the 15 x 15 cells whose four
+//      pixels lie inside it (a cell = the footprints that start at that pixel); blocks overlap by one row and one
+//      column, which the neighbours walk again. A lane recomputes alpha and transmittance of its pixel's retained entries from the per-point
 //      record exactly as the forward computed them, forms dL/dalpha (the "all later entries" sum of
 //      RenderBackward.cu:284-301 is a running sum from the back of the list) and leaves {dL/dalpha, T alpha} of every
 //      entry in LDS, together with the entry's rank under the (cell, place in the cell's list) that the forward noted
 //      for it. Then a lane per cell collects, for each of the cell's points, the four corner pixels' entries and
 //      writes ONE row per (point, layer) pair: sum over the corners of T alpha dL/dimage and the four dL/dalpha.
-//   2. points: one thread per point reads the rows of its pairs (consecutive in memory, numbered in point order),
+//      The rows of a point's first two layers sit at its compact number, further layers in an overflow table.
+//   2. points: the (point, layer) pairs of 64 consecutive points are dealt out to the lanes; a lane reads its pair's row,
 //      evaluates the bilinear weights' Jacobian and the layer factor per corner (PointBlending.h:216-264,
-//      RenderBackward.cu:366-438), sums the image-space gradient of all its entries and runs the projection chain
-//      ONCE (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then stores or adds its
+//      RenderBackward.cu:366-438); the point's own lane sums the image-space gradient of all its entries and runs the
+//      projection chain ONCE (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then stores or adds its
 //      gradients. Pose / intrinsics partials stay in registers over a grid-stride loop before one block-level
 //      reduction and one atomic per value and block (the reference keeps them in shared double arrays,
 //      :160-187,546-617).
@@ -244,11 +245,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 r0[b] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) rd[b][q] = make_float4(0.f, 0.f, 0.f, 0.f);
-#ifdef EXP_NOREC
-                if (false)
-#else
                 if (j0 + b < mmax && j0 + b < m)
-#endif
                 {
                     const float4* rec = reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)id[j0 + b] * RF);
                     r0[b]             = rec[0];
@@ -321,20 +318,20 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     __syncthreads();
 
     // ---- the block's cells, one per lane: a row per (point, layer) pair that some pixel retained ----
-#ifndef EXP_NOPHASE2
     {
         const int cell = min((int)threadIdx.x, kBlockCells * kBlockCells - 1);  // (cyl * 15 + cxl; the lanes past the last cell idle)
         const bool is_cell = (int)threadIdx.x < kBlockCells * kBlockCells;
         const int cyl = cell / kBlockCells, cxl = cell - cyl * kBlockCells;
-        // the places of the cell that hold a point, and the numbers of those points' first pairs (all requested before
-        // the first row is formed)
+        // the places of the cell that hold a point, and those points' compact numbers (all requested before the first
+        // row is formed)
+        const bool inline_row = layer < kInlineLayers;  // (the same for the whole block)
         unsigned words[kCellKeep];
-        int first_pair[kCellKeep];
+        int row_of[kCellKeep];
 #pragma unroll
         for (int place = 0; place < kCellKeep; ++place)
         {
-            words[place]      = is_cell ? s_rank[place * (kBlockCells * kBlockCells) + cell] : ~0u;
-            first_pair[place] = 0;
+            words[place]  = is_cell ? s_rank[place * (kBlockCells * kBlockCells) + cell] : ~0u;
+            row_of[place] = 0;
             if (__ballot(words[place] != ~0u))
             {
                 if (words[place] != ~0u)
@@ -344,17 +341,20 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                     const int corner  = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
                     const unsigned r  = (w4 >> (8 * corner)) & 0xFFu;
                     const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, x0 + cxl + (corner & 1), y0 + cyl + (corner >> 1));
-                    first_pair[place]  = p.lists[list_word(pix, (int)r, p.list_depth)];
+                    row_of[place]      = p.lists[list_word(pix, (int)r, p.list_depth)];
                 }
             }
         }
-        // the numbers of those points' first pairs
-#pragma unroll
-        for (int place = 0; place < kCellKeep; ++place)
+        // past the second layer: the number of the point's first row in the overflow table
+        if (!inline_row)
         {
-            if (__ballot(words[place] != ~0u))
+#pragma unroll
+            for (int place = 0; place < kCellKeep; ++place)
             {
-                if (words[place] != ~0u) first_pair[place] = p.pair_first[first_pair[place]];
+                if (__ballot(words[place] != ~0u))
+                {
+                    if (words[place] != ~0u) row_of[place] = p.over_first[row_of[place]];
+                }
             }
         }
 #pragma unroll
@@ -363,7 +363,6 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             const unsigned word = words[place];
             if (!__ballot(word != ~0u)) continue;
             if (word == ~0u) continue;
-            const long long pair = (long long)first_pair[place] + layer;
             float tex[CPAD], ga[4];
 #pragma unroll
             for (int c = 0; c < CPAD; ++c) tex[c] = 0.f;
@@ -379,16 +378,17 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
 #pragma unroll
                 for (int c = 0; c < C; ++c) tex[c] += e.y * s_g[c * kBlockPixels + tp];
             }
-            if (pair < p.pair_capacity)
+            const long long over = (long long)row_of[place] + (layer - kInlineLayers);
+            if (inline_row || over < p.over_capacity)
             {
-                vf4* row = reinterpret_cast<vf4*>(p.pair_sums + (size_t)pair * PRF);
+                vf4* row = reinterpret_cast<vf4*>(inline_row ? p.rows_inline + ((size_t)(unsigned)row_of[place] * kInlineLayers + layer) * PRF
+                                                             : p.rows_over + (size_t)over * PRF);
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) row[q] = vf4{tex[4 * q], tex[4 * q + 1], tex[4 * q + 2], tex[4 * q + 3]};
                 row[NQ] = vf4{ga[0], ga[1], ga[2], ga[3]};
             }
         }
     }
-#endif
 
 #pragma unroll
     for (int i = 0; i < C; ++i)
@@ -442,8 +442,8 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 
     __shared__ PointPassCamera s_cam;
     // what an item needs of its point {ip.x, ip.y, size field, confidence, size_px, softplus' * d size_px / d size,
-    // number of its first pair}, then the point in view space, kept here for the point's own lane
-    __shared__ float s_point[4][64][10];
+    // number of its first overflow row, compact number}, then the point in view space, kept here for the point's own lane
+    __shared__ float s_point[4][64][11];
     __shared__ unsigned short s_item[4][64 * TRIPS_MAX_LAYERS];  // lane of the point | layer << 8
     __shared__ __align__(16) float s_sums[4][64][NIT];           // sums of the items of one round
     if (threadIdx.x == 0)
@@ -482,7 +482,8 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         if (live)
         {
             const float4 r0 = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);  // ip.x ip.y size field conf
-            const int first = p.pair_first[cid];
+            // (a point of one or two layers has no overflow rows, and its number there is not looked at)
+            const int first = max_layer > kInlineLayers ? p.over_first[cid] : 0;
             // the point in view space, exactly as the projection kernel computed it
             float4 pos = p.position[pid];
             if (p.displacement)
@@ -499,8 +500,10 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             sp[0] = r0.x, sp[1] = r0.y, sp[2] = r0.z, sp[3] = r0.w, sp[4] = tail.w, sp[5] = tail.x * J_softmax_proj;
             sp[6] = __int_as_float(first);
             sp[7] = view[0], sp[8] = view[1], sp[9] = view[2];
-            // (rows past the capacity of the table do not exist: the forward reported the overflow)
-            if ((long long)first + max_layer > p.pair_capacity) max_layer = (int)max(0ll, p.pair_capacity - first);
+            sp[10] = __int_as_float(cid);
+            // (rows past the capacity of the overflow table do not exist: the forward reported the overflow)
+            if (max_layer > kInlineLayers && (long long)first + (max_layer - kInlineLayers) > p.over_capacity)
+                max_layer = kInlineLayers + (int)max(0ll, p.over_capacity - first);
         }
 
         // ---- the point's items: the layers it was written to ----
@@ -538,7 +541,9 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
                 const int layer     = (int)(item >> 8);
                 const float* sp     = s_point[wave][item & 63u];
                 const float ipx = sp[0], ipy = sp[1], size_field = sp[2], conf = sp[3], size_px = sp[4], size_chain = sp[5];
-                const vf4* row = reinterpret_cast<const vf4*>(p.pair_sums + ((size_t)__float_as_int(sp[6]) + layer) * PRF);
+                const vf4* row = reinterpret_cast<const vf4*>(
+                    layer < kInlineLayers ? p.rows_inline + ((size_t)(unsigned)__float_as_int(sp[10]) * kInlineLayers + layer) * PRF
+                                          : p.rows_over + ((size_t)__float_as_int(sp[6]) + (layer - kInlineLayers)) * PRF);
                 vf4 tq[NQ];
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) tq[q] = __builtin_nontemporal_load(row + q);
@@ -704,23 +709,36 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 }
 
 // Before the two passes of a view: the rows of the view's pairs start as zeros (the tile pass writes the rows of the
-// pairs that some pixel retained, the point pass reads all rows of a point). On the first view of a call also, in
+// pairs that some pixel retained, the point pass reads all rows of a point): the two inline rows of every valid point
+// (compact numbers are dense within each chunk of the binning kernels) and the overflow rows that the forward counted.
+// On the first view of a call also, in
 // overwrite mode (`texels`): the descriptor and confidence gradients of the columns that the point pass does not write
 // itself. With the identity index (the forward noted it in the header) those are the columns past the last point;
 // otherwise all of them, the point pass then adds with atomics. `clear_sums`: the block sums that both passes add to
 // (background, every pose row, every intrinsics row).
-__global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader* __restrict__ header, float* __restrict__ pair_sums,
-                                                                int pair_row, long long pair_capacity, float* __restrict__ d_texture,
+__global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader* __restrict__ header, const int32_t* __restrict__ chunk_valid,
+                                                                int bin_groups, int points_per_block, float* __restrict__ rows_inline,
+                                                                float* __restrict__ rows_over, int pair_row, long long over_capacity,
+                                                                float* __restrict__ d_texture,
                                                                 float* __restrict__ d_confidence, int channels, int num_texels,
                                                                 int num_points, int texels, int clear_sums,
                                                                 float* __restrict__ d_background, double* __restrict__ d_pose,
                                                                 int num_images, float* __restrict__ d_intrinsics, int num_cameras)
 {
     {
-        long long pairs = (long long)header->n_entries;
-        if (pairs > pair_capacity) pairs = pair_capacity;
-        const long long quads = pairs * pair_row / 4;  // (rows are a multiple of four floats)
-        vf4* dst              = reinterpret_cast<vf4*>(pair_sums);
+        // (rows are a multiple of four floats)
+        const int row_quads = kInlineLayers * pair_row / 4;
+        for (int chunk = blockIdx.x; chunk < bin_groups; chunk += gridDim.x)
+        {
+            const int begin = min(num_points, chunk * points_per_block);
+            const int quads = chunk_valid[chunk] * row_quads;
+            vf4* dst        = reinterpret_cast<vf4*>(rows_inline) + (size_t)begin * row_quads;
+            for (int i = threadIdx.x; i < quads; i += 256) __builtin_nontemporal_store(vf4{0.f, 0.f, 0.f, 0.f}, dst + i);
+        }
+        long long rows = (long long)header->overflow_rows;
+        if (rows > over_capacity) rows = over_capacity;
+        const long long quads = rows * pair_row / 4;
+        vf4* dst              = reinterpret_cast<vf4*>(rows_over);
         for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < quads; i += (long long)gridDim.x * 256)
             __builtin_nontemporal_store(vf4{0.f, 0.f, 0.f, 0.f}, dst + i);
     }
@@ -749,10 +767,7 @@ __global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader
 template <int C>
 hipError_t launch_tiles(const BackwardParams& p, int blocks, hipStream_t stream)
 {
-#ifndef EXP_LDS_EXTRA
-#define EXP_LDS_EXTRA 0
-#endif
-    const size_t lds = tiles_lds_bytes((C + 3) & ~3) + EXP_LDS_EXTRA;
+    const size_t lds = tiles_lds_bytes((C + 3) & ~3);
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&backward_tiles_kernel<C>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((backward_tiles_kernel<C>), dim3(blocks), dim3(256), lds, stream, p);
@@ -775,8 +790,8 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
     const int N = p.num_points;
     {
         ProfScope ps(prof, "backward_prologue", stream);
-        hipLaunchKernelGGL(backward_prologue_kernel, dim3(2048), dim3(256), 0, stream, p.header, p.pair_sums,
-                           pair_row_floats((channels + 3) & ~3), p.pair_capacity, p.d_texture, p.d_confidence, channels, p.num_texels,
+        hipLaunchKernelGGL(backward_prologue_kernel, dim3(2048), dim3(256), 0, stream, p.header, p.chunk_valid, p.bin_groups,
+                           p.points_per_block, p.rows_inline, p.rows_over, pair_row_floats((channels + 3) & ~3), p.over_capacity, p.d_texture, p.d_confidence, channels, p.num_texels,
                            N, p.overwrite, p.clear_block_sums, p.d_background, p.d_pose_all, p.num_images, p.d_intrinsics_all,
                            p.num_cameras);
     }

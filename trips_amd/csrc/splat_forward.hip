@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     constexpr int WAVES = kBinThreads / 64;
     extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
     __shared__ int s_valid[2][WAVES];  // valid points of every wavefront in this step (two steps in flight)
-    __shared__ int s_pairs[2][WAVES];  // (point, layer) pairs of every wavefront in this step
+    __shared__ int s_pairs[2][WAVES];  // overflow rows (layers past the second) of every wavefront's points in this step
     __shared__ int s_flags;            // bit 0: not_identity, bit 1: bad_index, of any point of the chunk
     const Camera cam  = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L       = p.num_layers;
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     chunk_point_range(p, begin, end);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int next       = begin;  // workgroup-uniform: compact number of the chunk's next valid point
-    int next_pair  = 0;      // workgroup-uniform: pairs of the chunk's points so far
+    int next_pair  = 0;      // workgroup-uniform: overflow rows of the chunk's points so far
     int step       = 0;
     // the loads of the next step's points are in flight while this step's are projected
     PointInputs nxt;
@@ -252,14 +252,16 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         if (pid < end) o = project_point<TRAIN>(p, cam, pid, in, s_hist, not_identity, bad_index);
         const unsigned long long vm = __ballot(o.valid);
         const unsigned long long below = (1ull << lane) - 1ull;
-        // pairs of the wavefront's points before this one, and of the wavefront: a point has 0..8 layers, one ballot per bit
+        // rows of the backward's overflow table (one per layer past the second) of the wavefront's points before this
+        // one, and of the wavefront: 0..6 per point, one ballot per bit
         int pairs_before = 0, pairs_wave = 0;
         if (TRAIN)
         {
+            const int extra = max(o.layers - kInlineLayers, 0);
 #pragma unroll
-            for (int b = 0; b < 4; ++b)
+            for (int b = 0; b < 3; ++b)
             {
-                const unsigned long long m = __ballot((o.layers >> b) & 1);
+                const unsigned long long m = __ballot((extra >> b) & 1);
                 pairs_before += (int)__popcll(m & below) << b;
                 pairs_wave += (int)__popcll(m) << b;
             }
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
         if (TRAIN)
         {
             __builtin_nontemporal_store(pid, p.pid_of + cid);
-            __builtin_nontemporal_store(first_pair, p.pair_first + cid);
+            __builtin_nontemporal_store(first_pair, p.over_first + cid);
         }
     }
     {
@@ -335,7 +337,7 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
                                                          int32_t* __restrict__ slice_start, int NB, long long capacity,
                                                          int32_t* __restrict__ chunk_valid, int G, ViewHeader* header,
                                                          ViewHeader* status, int first_view, int32_t* __restrict__ long_count,
-                                                         uint4* __restrict__ clear, long long clear_n)
+                                                         uint4* __restrict__ clear, long long clear_n, int32_t* __restrict__ saved_chunk_valid)
 {
     if (blockIdx.x > 0)
     {
@@ -347,8 +349,10 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
     __shared__ int s_carry[2];
     __shared__ unsigned long long s_valid_total, s_same_total;
     __shared__ int s_flags;
+    __shared__ int s_over_total;
     if (threadIdx.x == 0)
     {
+        s_over_total = 0;
         s_carry[0] = s_carry[1] = 0;
         s_valid_total = s_same_total = 0;
         s_flags                 = 0;
@@ -366,7 +370,7 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
             f |= chunk_valid[G + g];
             st += (unsigned long long)(unsigned)chunk_valid[2 * G + g];
         }
-        // number of every chunk's first (point, layer) pair: exclusive prefix of the chunks' pair counts (G <= 1024)
+        // number of every chunk's first overflow row: exclusive prefix of the chunks' row counts (G <= 1024)
         {
             const int mine = (int)threadIdx.x < G ? chunk_valid[3 * G + threadIdx.x] : 0;
             int inc        = mine;
@@ -380,6 +384,8 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
             int prefix = inc - mine;
             for (int w = 0; w < wave; ++w) prefix += s_wave[0][w];
             if ((int)threadIdx.x < G) chunk_valid[4 * G + threadIdx.x] = prefix;
+            if ((int)threadIdx.x == G - 1) s_over_total = prefix + mine;
+            if (saved_chunk_valid && (int)threadIdx.x < G) saved_chunk_valid[threadIdx.x] = chunk_valid[threadIdx.x];
             __syncthreads();
         }
         for (int o = 32; o > 0; o >>= 1)
@@ -454,12 +460,12 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
         header->not_identity = (unsigned long long)(s_flags & 1);
         header->bad_index    = 0;
         header->same_tile_as_previous = s_same_total;
-        header->reserved              = 0;
+        header->overflow_rows         = (unsigned long long)(unsigned)s_over_total;
         if (first_view)
         {
             status->n_valid = status->n_entries = status->overflow = status->retained = status->not_identity = 0;
             status->bad_index                                                       = bad;
-            status->same_tile_as_previous = status->reserved = 0;
+            status->same_tile_as_previous = status->overflow_rows = 0;
         }
         else if (bad)
             status->bad_index = 1;  // (the views of a call run one after the other on the stream)
@@ -580,8 +586,8 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
                 const vf4 t = __builtin_nontemporal_load(reinterpret_cast<const vf4*>(p.prec) + cid);
                 tail[u]     = make_float4(t.x, t.y, t.z, t.w);
                 ip[u]   = *reinterpret_cast<const float2*>(p.rec + (size_t)cid * p.rec_floats);
-                // the point's first pair: the projection numbered it within the chunk, the scan found the chunk's first
-                if (p.pair_first) p.pair_first[cid] += pair_base;
+                // the point's first overflow row: the projection numbered it within the chunk, the scan found the chunk's first
+                if (p.over_first) p.over_first[cid] += pair_base;
             }
         }
 #pragma unroll
@@ -1460,7 +1466,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
         const long long quads = 2ll * NB * kTilePixels / 4;
         hipLaunchKernelGGL(scan_plan_kernel, dim3(1 + (unsigned)std::min<long long>((quads + 1023) / 1024, 1024)), dim3(1024), 0, stream,
                            p.bin_count, p.bin_start, p.slice_start, NB, p.capacity, p.chunk_valid, G, p.header, p.status, first_view ? 1 : 0,
-                           p.long_count, reinterpret_cast<uint4*>(p.counts), quads);
+                           p.long_count, reinterpret_cast<uint4*>(p.counts), quads, p.saved_chunk_valid);
     }
     {
         ProfScope ps(prof, "bin_scatter", stream);

@@ -236,7 +236,8 @@ struct ViewHeader
     // stored along a space-filling curve, near zero for one in random order (the backward chooses its exchange layout
     // by it)
     unsigned long long same_tile_as_previous;
-    unsigned long long reserved;
+    // rows of the backward's overflow table that the view's points own: sum over the valid points of max(layers - 2, 0)
+    unsigned long long overflow_rows;
 };
 
 // Layout of one view's saved state (all offsets in bytes, 256-aligned)
@@ -251,26 +252,32 @@ struct SavedLayout
                       // place in that cell's sorted list (bits 0..3); a row's positions past its ids are undefined
     size_t cid_of;    // int32 [N] compact number of every point (-1 = culled)
     size_t pid_of;    // int32 [N] point of every compact number (the first n_valid are defined)
-    size_t pair_first;  // int32 [N] by compact number: the number of the point's first (point, layer) pair; its pairs are
-                        // numbered consecutively by layer, all pairs of a view densely in point order
+    size_t over_first;  // int32 [N] by compact number: for a point written to more than two layers, the number of its
+                        // first row in the backward's overflow table (rows numbered densely in point order)
+    size_t chunk_valid;  // int32 [kBinGroups] valid points of every chunk of the binning kernels (their compact numbers
+                         // start at the chunk's first point number)
     size_t bytes_per_view;
 };
 
 // The backward sums, per (point, layer) pair, what the four pixels of the footprint contribute before the projection
 // chain: the descriptor gradient sum_corners T alpha dL/dimage (Cpad floats) and dL/dalpha of each corner (4 floats).
+// The rows of a point's first two layers sit at its compact number (most points are written to one or two layers: the
+// tile pass then needs no look-up to place a row), those of further layers in an overflow table.
 __host__ __device__ constexpr int pair_row_floats(int cpad) { return cpad + 4; }
+constexpr int kInlineLayers = 2;
 
 struct BackwardWorkspaceLayout
 {
-    size_t pair_sums;  // float [capacity, pair_row_floats] by pair number
-    size_t capacity;   // (point, layer) pairs
+    size_t rows_inline;  // float [N, kInlineLayers, pair_row_floats] by compact number
+    size_t rows_over;    // float [over_capacity, pair_row_floats]
+    size_t over_capacity;
     size_t bytes;
 };
 
 struct WorkspaceLayout
 {
-    size_t chunk_valid;   // int32 [5 G]  per chunk of the binning kernels: valid points, flags, same-tile counts, (point, layer)
-                          //              pairs, and (from the scan) the number of the chunk's first pair
+    size_t chunk_valid;   // int32 [5 G]  per chunk of the binning kernels: valid points, flags, (unused), overflow rows of the
+                          //              backward, and (from the scan) the number of the chunk's first overflow row
     size_t prec;         // float4 [N]         point records, when there is no saved state to hold them
     size_t counts;       // int32 [Pi]   list length per cell (the points whose 2 x 2 footprint starts at that pixel)
     size_t cursor;       // int32 [Pi]   first key of each cell's list (-1 - first candidate row for a long list)
@@ -337,7 +344,8 @@ struct ForwardParams
     int32_t* lists;
     int32_t* retained;
     unsigned char* tags;  // training only
-    int32_t* pair_first;  // training only
+    int32_t* over_first;  // training only
+    int32_t* saved_chunk_valid;  // training only
     ViewHeader* header;  // counters of this view
     ViewHeader* status;  // overflow flag of the whole forward call (start of the workspace)
     float* image[TRIPS_MAX_LAYERS];
@@ -366,12 +374,15 @@ struct BackwardParams
     const ViewHeader* header;
     const float* grad_image[TRIPS_MAX_LAYERS];
     const unsigned char* tags;  // [Pi, 16] (saved state) cell and place in the cell's list of every list position
-    const int32_t* pair_first;  // [N] (saved state) by compact number
-    float* pair_sums;  // [pairs, pair_row_floats] (workspace)
+    const int32_t* over_first;   // [N] (saved state) by compact number
+    const int32_t* chunk_valid;  // [kBinGroups] (saved state)
+    int32_t bin_groups, points_per_block;
+    float* rows_inline;  // [N, kInlineLayers, pair_row_floats] (workspace)
+    float* rows_over;    // [over_capacity, pair_row_floats] (workspace)
     // blocks of the tile pass (16 x 16 pixels, 15 apart): first block of each layer, blocks per block row of each layer
     int32_t blocks_off[TRIPS_MAX_LAYERS + 1];
     int32_t blocks_x[TRIPS_MAX_LAYERS];
-    long long pair_capacity;
+    long long over_capacity;
     float* d_texture;
     float* d_confidence;
     float* d_background;

@@ -218,8 +218,10 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     o += align256(N * sizeof(int32_t));
     s.pid_of = o;
     o += align256(N * sizeof(int32_t));
-    s.pair_first = o;
+    s.over_first = o;
     o += align256(N * sizeof(int32_t));
+    s.chunk_valid = o;
+    o += align256((size_t)kBinGroups * sizeof(int32_t));
     s.bytes_per_view = o;
     return s;
 }
@@ -276,11 +278,16 @@ namespace
 BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const PyramidGeom& g)
 {
     BackwardWorkspaceLayout w;
-    // a row per (point, layer) pair: as many as the forward can file
-    w.capacity  = d.max_list_entries > 0 ? ((size_t)d.max_list_entries + 3) / 4 : (size_t)d.num_points * (size_t)d.num_layers;
-    size_t o    = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
-    w.pair_sums = o;
-    o += align256(w.capacity * (size_t)pair_row_floats((d.num_channels + 3) & ~3) * sizeof(float));
+    // a row per (point, layer) pair: two per point by its compact number, the rest as many as the forward can file
+    const size_t extra_layers = d.num_layers > kInlineLayers ? (size_t)(d.num_layers - kInlineLayers) : 0;
+    const size_t row          = (size_t)pair_row_floats((d.num_channels + 3) & ~3) * sizeof(float);
+    w.over_capacity = (size_t)d.num_points * extra_layers;
+    if (d.max_list_entries > 0) w.over_capacity = std::min(w.over_capacity, ((size_t)d.max_list_entries + 3) / 4);
+    size_t o      = align256(sizeof(ViewHeader));  // keeps the status block of the forward intact
+    w.rows_inline = o;
+    o += align256((size_t)d.num_points * kInlineLayers * row);
+    w.rows_over = o;
+    o += align256(w.over_capacity * row);
     w.bytes = o;
     return w;
 }
@@ -449,7 +456,8 @@ int forward_impl(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsSplatIn* 
             p.lists      = reinterpret_cast<int32_t*>(sv + sl.lists);
             p.retained   = reinterpret_cast<int32_t*>(sv + sl.retained);
             p.tags       = reinterpret_cast<unsigned char*>(sv + sl.tags);
-            p.pair_first = reinterpret_cast<int32_t*>(sv + sl.pair_first);
+            p.over_first = reinterpret_cast<int32_t*>(sv + sl.over_first);
+            p.saved_chunk_valid = reinterpret_cast<int32_t*>(sv + sl.chunk_valid);
             p.cid_of     = reinterpret_cast<int32_t*>(sv + sl.cid_of);
             p.pid_of     = reinterpret_cast<int32_t*>(sv + sl.pid_of);
         }
@@ -557,9 +565,13 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.cid_of       = reinterpret_cast<const int32_t*>(sv + sl.cid_of);
         p.header       = reinterpret_cast<const ViewHeader*>(sv + sl.header);
         p.tags         = reinterpret_cast<const unsigned char*>(sv + sl.tags);
-        p.pair_first   = reinterpret_cast<const int32_t*>(sv + sl.pair_first);
-        p.pair_sums    = reinterpret_cast<float*>(ws + bl.pair_sums);
-        p.pair_capacity = (long long)bl.capacity;
+        p.over_first   = reinterpret_cast<const int32_t*>(sv + sl.over_first);
+        p.chunk_valid  = reinterpret_cast<const int32_t*>(sv + sl.chunk_valid);
+        p.bin_groups   = kBinGroups;
+        p.points_per_block = (d.num_points + kBinGroups - 1) / kBinGroups;
+        p.rows_inline  = reinterpret_cast<float*>(ws + bl.rows_inline);
+        p.rows_over    = reinterpret_cast<float*>(ws + bl.rows_over);
+        p.over_capacity = (long long)bl.over_capacity;
         p.blocks_off[0] = 0;
         for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
         {
