@@ -38,7 +38,7 @@ PMC_KIB_DEFAULT_WORKLOAD = {
     "tile_count": (13142, 2296),
     "tile_scatter": (32640, 110285),
     "sort_blend": (333383, 350795),
-    "backward_pixels": (453556, 296281),
+    "backward_tiles": (453556, 296281),
     "backward_points": (866929, 234887),
     "adam_fused": (383862, 498420),
 }
@@ -57,7 +57,7 @@ def kernel_sources_sha256():
 
 
 # The sort + blend of the forward runs as two launches (the lists of the cells sorted and cut, then the pixels merged
-# and blended); the algorithmic bytes of SURVEY's row are those of the pair, so the two are reported as one kernel
+# and blended); the algorithmic bytes of the sort + blend are those of the pair, so the two are reported as one kernel
 # with parts.
 KERNEL_PARTS = {"sort_blend": ("cell_sort", "blend")}
 
@@ -95,10 +95,11 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam
         "project_bin": 24 * N,                                    # position 16 + size 4 + index 4
         "tile_scatter": 8 * E,                                    # one 64-bit key written per entry
         "sort_blend": 8 * E + (20 + 4 + 4 * C + 28) * R + 4 * C * P,  # keys read, record+conf+descriptor, saved, image
-        # the backward's bytes split as its two passes split the work: the compositing (pixel pass) reads dL/dimage, the
+        # the backward's bytes split as its two passes split the work: the compositing (tile pass) reads dL/dimage, the
         # saved entry, descriptor and confidence; the geometry (point pass) reads position + size again (20 B per entry)
-        # and makes the one write per accumulated gradient float
-        "backward_pixels": 4 * C * P + (28 + 4 * C + 4) * R,
+        # and makes the one write per accumulated gradient float. (The prologue that clears the exchange rows has no
+        # algorithmic bytes: its time counts, its bytes do not.)
+        "backward_tiles": 4 * C * P + (28 + 4 * C + 4) * R,
         "backward_points": (20 + 4 * C + 4 + 12 + 4) * R,
         "adam_fused": (28 + 2 * adam_step_bytes) * adam_nonzero + 8 * adam_zero,
     }
@@ -106,8 +107,8 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam
 
 def measure_other_config(ctx, name, steps):
     """One of the other BASELINE configurations (1, 2, 4) at its full size, beside the headline: wall time of the forward
-    and of forward + backward with inputs resident, per-kernel times, the run's counters, the algorithmic bytes of
-    SURVEY 8(d) from them and the fraction of the HBM peak they stand for. Configuration 1 is forward-only by definition."""
+    and of forward + backward with inputs resident, per-kernel times, the run's counters, the algorithmic bytes that
+    follow from them and the fraction of the HBM peak they stand for. Configuration 1 is forward-only by definition."""
     import numpy as np
     import torch
     from trips_amd import abi, scenes
@@ -317,6 +318,26 @@ def main():
         torch.cuda.synchronize()
         eval_ms = (time.perf_counter() - v0) * 1e3 / args.steps
         del ws_eval
+        # the same step with the optimiser state laid out as the reference lays it out (one array per tensor, int64 step
+        # counters): what a caller gets who keeps the reference's optimiser structure
+        ref_layout_ms = None
+        if not args.no_adam_variants:
+            o3 = MyAdam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, param_steps_dtype=torch.int64)
+
+            def step_ref_layout():
+                ctx.forward(desc, tin, images, saved, workspace)
+                ctx.backward(desc, tin, saved, grad_images, grads, workspace, overwrite_point_grads=True, clear_block_sums=True)
+                o3.step()
+
+            for _ in range(max(args.warmup, 2)):
+                step_ref_layout()
+            torch.cuda.synchronize()
+            r0 = time.perf_counter()
+            for _ in range(args.steps):
+                step_ref_layout()
+            torch.cuda.synchronize()
+            ref_layout_ms = (time.perf_counter() - r0) * 1e3 / args.steps
+            del o3
         # Adam on its own, with the step counters the product uses (int32) and with the reference's int64 state tensor
         adam_ms = {}
         for name, dt in (() if args.no_adam_variants else (("int32_counters", torch.int32), ("int64_counters", torch.int64))):
@@ -333,7 +354,7 @@ def main():
             ctx.profile_enable(False)
             adam_ms[name] = ms / max(launches, 1)
             del o2
-        return dict(graph_ms=graph_ms, events_ms=ms_per_step_events, eval_ms=eval_ms, adam_ms=adam_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
+        return dict(ref_layout_ms=ref_layout_ms, graph_ms=graph_ms, events_ms=ms_per_step_events, eval_ms=eval_ms, adam_ms=adam_ms, sc=sc, desc=desc, t=t, tin=tin, workspace=workspace, saved=saved, images=images, gen=gen,
                     grad_images=grad_images, grads=grads, opt=opt, counters=counters, nz=nz, total_el=total_el,
                     prof=prof, ms_per_step=ms_per_step)
 
@@ -528,6 +549,10 @@ def main():
         "unit": "points/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
+        # the same step with the reference's optimiser state layout (per-tensor arrays, int64 step counters) instead of
+        # the packed per-point rows that `value` is timed with
+        "ms_per_step_reference_adam_layout": None if r["ref_layout_ms"] is None else round(r["ref_layout_ms"], 4),
+        "value_reference_adam_layout": None if r["ref_layout_ms"] is None else round(N / (r["ref_layout_ms"] * 1e-3), 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config3: 6M points (80% noisy ground plane, 20% box), 1920x1080, 8 layers, K=16, "
