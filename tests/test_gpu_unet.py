@@ -137,19 +137,24 @@ def test_unet_refuses_cpu_tensors():
 GRAD_TOL = 2e-2
 
 
-@pytest.mark.parametrize("filters,levels,w,h,batch", [
-    ([16, 32, 64, 64], 4, 96, 72, 1),      # the benchmark's channel plan
-    ([32, 32, 32, 32, 32], 5, 100, 60, 2),  # shipped filters, odd sizes, two images
-    ([16, 24], 2, 37, 29, 1),               # partial tiles
-    ([32, 64, 64], 3, 70, 50, 1),           # 64 input channels at the finest level
-    ([16, 48, 32], 3, 70, 50, 2),           # 40 outputs on 32 inputs (the weight gradient's four-wavefront shape)
+@pytest.mark.parametrize("filters,levels,w,h,batch,cin", [
+    ([16, 32, 64, 64], 4, 96, 72, 1, 4),      # the benchmark's channel plan
+    ([32, 32, 32, 32, 32], 5, 100, 60, 2, 4),  # shipped filters, odd sizes, two images
+    ([16, 24], 2, 37, 29, 1, 4),               # partial tiles
+    ([32, 64, 64], 3, 70, 50, 1, 4),           # 64 input channels at the finest level
+    ([16, 48, 32], 3, 70, 50, 2, 4),           # 40 outputs on 32 inputs (the weight gradient's four-wavefront shape)
+    # fewer than four image channels: the coarser level's outputs then start at a position of the finer block's input
+    # that is not a multiple of eight
+    ([16, 32, 64, 64], 4, 96, 72, 1, 3),       # 58 outputs below 64 inputs: no spare position
+    ([16, 24, 32], 3, 37, 29, 2, 2),
+    ([12, 20], 2, 40, 24, 1, 1),
 ])
-def test_unet_backward_matches_torch_autograd(filters, levels, w, h, batch):
+def test_unet_backward_matches_torch_autograd(filters, levels, w, h, batch, cin):
     import copy
     from tests.ref_unet import unet_forward
-    net = _net(filters, levels, seed=20 + levels)
+    net = _net(filters, levels, seed=20 + levels, cin=cin)
     ref = copy.deepcopy(net)
-    inputs = _pyramid(w, h, levels, 4, batch=batch, seed=30 + levels)
+    inputs = _pyramid(w, h, levels, cin, batch=batch, seed=30 + levels)
     g = torch.Generator().manual_seed(7)
     upstream = torch.randn((batch, 3, h, w), generator=g) * 1e-3
 

@@ -115,6 +115,9 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     float* const s_g       = reinterpret_cast<float*>(s_mem + (size_t)kBlockPixels * kListMax * 8);
     unsigned* const s_rank = reinterpret_cast<unsigned*>(s_mem + (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * CPAD * 4);
     __shared__ double s_acc[4][C];
+    // (point, layer) pairs of a wavefront's cells that wait for a lane: place * 225 + cell; at most 63 are left over when
+    // a place adds its (at most 57) cells
+    __shared__ unsigned short s_queue[4][128];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // Blocks of 16 x 16 pixels that overlap by one row and one column (so that every cell's four pixels lie in one
@@ -130,11 +133,6 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     const int lw = p.geom.w[layer], lh = p.geom.h[layer];
     const int x0 = bxi * kBlockCells, y0 = byi * kBlockCells;  // the block's first pixel
     const float* const gi = p.grad_image[layer];
-
-    // no entry yet under any (cell, place)
-    for (int i = threadIdx.x; i < kBlockCells * kBlockCells * kCellKeep / 4; i += 256)
-        reinterpret_cast<uint4*>(s_rank)[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
-    __syncthreads();
 
     float acc_bg[C];  // a lane sees a few pixels: its own sums stay in single precision, everything across lanes is double
 #pragma unroll
@@ -192,6 +190,10 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 for (int c = 0; c < C; ++c) g[c] = o[at + c];
             }
         }
+        // no entry yet under any (cell, place): cleared while the loads above travel
+        for (int i = threadIdx.x; i < kBlockCells * kBlockCells * kCellKeep / 4; i += 256)
+            reinterpret_cast<uint4*>(s_rank)[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+        __syncthreads();
         const int m    = word & kRetainedMask;
         const int mmax = wave_max_small<kListMax>(m);
         // (two thirds of the pixels of a typical view retain at most four entries: the rest of a list only where needed)
@@ -317,77 +319,89 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     }
     __syncthreads();
 
-    // ---- the block's cells, one per lane: a row per (point, layer) pair that some pixel retained ----
+    // ---- a row per (point, layer) pair that some pixel retained. The pairs of a block are few and unevenly spread over
+    // its cells (most cells hold one or two, some sixteen), so they are dealt out: every wavefront scans its quarter of
+    // the cells place by place, queues the slots that hold a point, and whenever 64 wait, each lane forms one row. ----
     {
-        const int cell = min((int)threadIdx.x, kBlockCells * kBlockCells - 1);  // (cyl * 15 + cxl; the lanes past the last cell idle)
-        const bool is_cell = (int)threadIdx.x < kBlockCells * kBlockCells;
-        const int cyl = cell / kBlockCells, cxl = cell - cyl * kBlockCells;
-        // the places of the cell that hold a point, and those points' compact numbers (all requested before the first
-        // row is formed)
+        constexpr int kCells        = kBlockCells * kBlockCells;
+        constexpr int kCellsPerWave = (kCells + 3) / 4;
+        unsigned short* const queue = s_queue[wave];
+        const int cell       = wave * kCellsPerWave + lane;
+        const bool is_cell   = lane < kCellsPerWave && cell < kCells;
         const bool inline_row = layer < kInlineLayers;  // (the same for the whole block)
-        unsigned words[kCellKeep];
-        int row_of[kCellKeep];
-#pragma unroll
-        for (int place = 0; place < kCellKeep; ++place)
+        int waiting = 0;  // slots in the queue (the same in every lane)
+        // forms the rows of the first `n` slots of the queue (n <= 64)
+        auto form_rows = [&](int n)
         {
-            words[place]  = is_cell ? s_rank[place * (kBlockCells * kBlockCells) + cell] : ~0u;
-            row_of[place] = 0;
-            if (__ballot(words[place] != ~0u))
+            if (lane < n)
             {
-                if (words[place] != ~0u)
+                const int slot    = queue[lane];
+                const int place   = slot / kCells, c2 = slot - place * kCells;
+                const int cyl = c2 / kBlockCells, cxl = c2 - cyl * kBlockCells;
+                const unsigned w4 = s_rank[slot];
+                // the point's compact number: from the list of the first corner pixel that retained it
+                const int first   = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
+                const unsigned rf = (w4 >> (8 * first)) & 0xFFu;
+                const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, x0 + cxl + (first & 1), y0 + cyl + (first >> 1));
+                int row_of         = p.lists[list_word(pix, (int)rf, p.list_depth)];
+                // past the second layer: the number of the point's first row in the overflow table
+                if (!inline_row) row_of = p.over_first[row_of];
+                float tex[CPAD], ga[4];
+#pragma unroll
+                for (int c = 0; c < CPAD; ++c) tex[c] = 0.f;
+#pragma unroll
+                for (int corner = 0; corner < 4; ++corner)
                 {
-                    // the point's compact number: from the list of the first corner pixel that retained it
-                    const unsigned w4 = words[place];
-                    const int corner  = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
-                    const unsigned r  = (w4 >> (8 * corner)) & 0xFFu;
-                    const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, x0 + cxl + (corner & 1), y0 + cyl + (corner >> 1));
-                    row_of[place]      = p.lists[list_word(pix, (int)r, p.list_depth)];
+                    const unsigned r = (w4 >> (8 * corner)) & 0xFFu;
+                    ga[corner]       = 0.f;
+                    if (r == 0xFFu) continue;
+                    const int tp   = (cyl + (corner >> 1)) * kBlockSide + cxl + (corner & 1);
+                    const float2 e = s_ex[(int)r * kBlockPixels + tp];
+                    ga[corner]     = e.x;
+#pragma unroll
+                    for (int c = 0; c < C; ++c) tex[c] += e.y * s_g[c * kBlockPixels + tp];
+                }
+                const long long over = (long long)row_of + (layer - kInlineLayers);
+                if (inline_row || over < p.over_capacity)
+                {
+                    vf4* row = reinterpret_cast<vf4*>(inline_row ? p.rows_inline + ((size_t)(unsigned)row_of * kInlineLayers + layer) * PRF
+                                                                 : p.rows_over + (size_t)over * PRF);
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) row[q] = vf4{tex[4 * q], tex[4 * q + 1], tex[4 * q + 2], tex[4 * q + 3]};
+                    row[NQ] = vf4{ga[0], ga[1], ga[2], ga[3]};
                 }
             }
-        }
-        // past the second layer: the number of the point's first row in the overflow table
-        if (!inline_row)
+        };
+        // the first 64 slots leave the queue, the others move up
+        auto pop64 = [&]()
         {
-#pragma unroll
-            for (int place = 0; place < kCellKeep; ++place)
-            {
-                if (__ballot(words[place] != ~0u))
-                {
-                    if (words[place] != ~0u) row_of[place] = p.over_first[row_of[place]];
-                }
-            }
-        }
-#pragma unroll
+            form_rows(min(waiting, 64));
+            unsigned short moved = 0;
+            if (64 + lane < waiting) moved = queue[64 + lane];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (64 + lane < waiting) queue[lane] = moved;
+            waiting = max(waiting - 64, 0);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        };
+#pragma unroll 1
         for (int place = 0; place < kCellKeep; ++place)
         {
-            const unsigned word = words[place];
-            if (!__ballot(word != ~0u)) continue;
-            if (word == ~0u) continue;
-            float tex[CPAD], ga[4];
-#pragma unroll
-            for (int c = 0; c < CPAD; ++c) tex[c] = 0.f;
-#pragma unroll
-            for (int corner = 0; corner < 4; ++corner)
-            {
-                const unsigned r = (word >> (8 * corner)) & 0xFFu;
-                ga[corner]       = 0.f;
-                if (r == 0xFFu) continue;
-                const int tp   = (cyl + (corner >> 1)) * kBlockSide + cxl + (corner & 1);
-                const float2 e = s_ex[(int)r * kBlockPixels + tp];
-                ga[corner]     = e.x;
-#pragma unroll
-                for (int c = 0; c < C; ++c) tex[c] += e.y * s_g[c * kBlockPixels + tp];
-            }
-            const long long over = (long long)row_of[place] + (layer - kInlineLayers);
-            if (inline_row || over < p.over_capacity)
-            {
-                vf4* row = reinterpret_cast<vf4*>(inline_row ? p.rows_inline + ((size_t)(unsigned)row_of[place] * kInlineLayers + layer) * PRF
-                                                             : p.rows_over + (size_t)over * PRF);
-#pragma unroll
-                for (int q = 0; q < NQ; ++q) row[q] = vf4{tex[4 * q], tex[4 * q + 1], tex[4 * q + 2], tex[4 * q + 3]};
-                row[NQ] = vf4{ga[0], ga[1], ga[2], ga[3]};
-            }
+            const int slot  = place * kCells + cell;
+            const bool has  = is_cell && s_rank[slot] != ~0u;
+            const unsigned long long mask = __ballot(has);
+            if (!mask) continue;
+            if (has) queue[waiting + (int)__popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)slot;
+            waiting += (int)__popcll(mask);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (waiting >= 64) pop64();
         }
+        if (waiting > 0) pop64();
     }
 
 #pragma unroll

@@ -399,11 +399,15 @@ __device__ __forceinline__ float up2_weight(int dst, int fine_size, int src, int
     return (i0 == src ? 1.f - l : 0.f) + (i1 == src ? l : 0.f);
 }
 
+// SHIFT = (2 C) % 8: the block outputs of the coarser level start at position 2 C of the finer block's input, which is
+// a multiple of 8 halves only for C = 4; otherwise a group of eight outputs straddles two aligned groups of positions.
+template <int SHIFT>
 __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointParams p)
 {
     const int half   = p.npad / 2;
     const int groups = 1 + half / 8;  // group 0: the image below; group q: 8 block outputs
     const size_t pb  = (size_t)p.Hb * p.Wb;
+    const int base8  = (2 * p.c_feat) & ~7;  // aligned position at or before the first block output
     for (size_t item = (size_t)blockIdx.x * 256 + threadIdx.x; item < pb * groups; item += (size_t)gridDim.x * 256)
     {
         const int q     = (int)(item % groups);
@@ -419,19 +423,19 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
             f8 = *reinterpret_cast<const half8*>(p.pre + bp * p.npad + ch0);
             m8 = *reinterpret_cast<const half8*>(p.pre + bp * p.npad + half + ch0);
         }
-        float a[8];
+        float wy[4], wx[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) a[i] = 0.f;
-        const int pos = 8 * q;  // position in the finer block's input: [0, C) its own image, then x of this level
-        if (pos < p.cin_fine)
+        for (int k = 0; k < 4; ++k)
         {
-            float wy[4], wx[4];
+            wy[k] = up2_weight(2 * Y - 1 + k, p.H, Y, p.Hb);
+            wx[k] = up2_weight(2 * X - 1 + k, p.W, X, p.Wb);
+        }
+        // the adjoint of the upsampling for the eight positions from `pos` on (a multiple of 8)
+        auto gather = [&](int pos, float (&a)[8])
+        {
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-            {
-                wy[k] = up2_weight(2 * Y - 1 + k, p.H, Y, p.Hb);
-                wx[k] = up2_weight(2 * X - 1 + k, p.W, X, p.Wb);
-            }
+            for (int i = 0; i < 8; ++i) a[i] = 0.f;
+            if (pos >= p.cin_fine) return;
             // all 16 gathers are issued before the first one is used (a load inside a branch on its weight would be
             // waited for there: 16 memory round trips in a row); pixels outside the image have weight 0 and are read
             // at a clamped position instead
@@ -461,14 +465,33 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
                     }
                 }
             }
-        }
+        };
+        float a[8];
         if (q == 0)
         {
-            // positions [C, 2C) are this level's image (C = 4: a[4..7])
-            for (int c = 0; c < p.c_feat; ++c) p.d_feat[c * pb + bp] = a[p.c_feat + c] * p.scale_inv;
+            // positions [0, C) are the finer level's own image, [C, 2C) this level's
+            gather(0, a);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+            {
+                // (a[c_feat + c] with compile-time indices: a run-time index would put the array into scratch memory)
+                float v = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v = (i == p.c_feat + c) ? a[i] : v;
+                if (c < p.c_feat) p.d_feat[c * pb + bp] = v * p.scale_inv;
+            }
         }
         else
         {
+            // output ch0 + i of this level sits at position 2 C + ch0 + i = base8 + ch0 + SHIFT + i
+            gather(base8 + ch0, a);
+            if (SHIFT != 0)
+            {
+                float hi[8];
+                gather(base8 + ch0 + 8, hi);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a[i] = SHIFT + i < 8 ? a[(SHIFT + i) & 7] : hi[(SHIFT + i) & 7];
+            }
             _Float16* dp = p.dpre + bp * p.npad;
             half8 of, om;
 #pragma unroll
@@ -667,7 +690,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
     // flight together), and written to LDS one tile later, so that the loads of tile t + 1 travel while tile t is
     // upsampled and multiplied ----
     constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + THREADS - 1) / THREADS;
-    constexpr int kMaxPerPix  = 1 + (CIN - 8) / 8;  // image below + groups of 8 block outputs (C = 4)
+    constexpr int kMaxPerPix  = 1 + CIN / 8;  // image below + groups of 8 block outputs
     constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + THREADS - 1) / THREADS;
     constexpr int kDpreGroups = NPAD / 8;  // 16-byte groups of a pixel's gradient row
     constexpr int kDpreItems  = (kConvTileH * kConvTileW * kDpreGroups + THREADS - 1) / THREADS;
@@ -762,6 +785,22 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
         }
         for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
     };
+    // eight block outputs of the level below (group q >= 1) into positions 2 C + 8 (q - 1) .. of a below-patch pixel
+    auto put_below_act = [&](int bp, int q, const uint4& v)
+    {
+        _Float16* row = s_below + (size_t)bp * ROW;
+        const int pos = 2 * C + 8 * (q - 1);
+        if (C == 4)
+            *reinterpret_cast<uint4*>(row + pos) = v;
+        else
+        {
+            // (positions that are not a multiple of 8: element by element; outputs past the padded input are padding)
+            const half8 a = __builtin_bit_cast(half8, v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (pos + i < CIN) row[pos + i] = a[i];
+        }
+    };
     auto commit_loads = [&](const TileLoads& r)
     {
 #pragma unroll
@@ -786,7 +825,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                         put_below_image(bp, f);
                     }
                     else
-                        *reinterpret_cast<uint4*>(s_below + (size_t)bp * ROW + 2 * C + 8 * (q - 1)) = r.below[k];
+                        put_below_act(bp, q, r.below[k]);
                 }
             }
         }
@@ -832,8 +871,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                 }
                 else
                 {
-                    *reinterpret_cast<half8*>(s_below + (size_t)bp * ROW + 2 * C + 8 * (q - 1)) =
-                        *reinterpret_cast<const half8*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+                    put_below_act(bp, q, *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1)));
                 }
             }
         }
@@ -1158,7 +1196,6 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
     if (!weights || !inputs || !saved || !d_output || !grads || !workspace) return set_error(TRIPS_ERR_INVALID_ARG, "NULL argument");
     const TripsUnetDesc& d = *desc;
     const int C = d.num_input_channels, L = d.num_levels;
-    if (C != 4) return set_error(TRIPS_ERR_UNSUPPORTED, "the backward is built for num_input_channels = 4 (got %d)", C);
     if (!(grad_scale > 0.f) || !std::isfinite(grad_scale)) return set_error(TRIPS_ERR_INVALID_ARG, "grad_scale must be positive");
     for (int i = 0; i < L; ++i)
     {
@@ -1346,7 +1383,13 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
                     up.dpre      = dpre_ptr(i + 1, b);
                     const size_t items = (size_t)lb.H * lb.W * (1 + lb.npad / 16);
                     const int blocks   = (int)std::min<size_t>((items + 255) / 256, 1u << 20);
-                    hipLaunchKernelGGL(up2_adjoint_gate_kernel, dim3(blocks), dim3(256), 0, stream, up);
+                    switch ((2 * C) & 7)
+                    {
+                        case 0: hipLaunchKernelGGL(up2_adjoint_gate_kernel<0>, dim3(blocks), dim3(256), 0, stream, up); break;
+                        case 2: hipLaunchKernelGGL(up2_adjoint_gate_kernel<2>, dim3(blocks), dim3(256), 0, stream, up); break;
+                        case 4: hipLaunchKernelGGL(up2_adjoint_gate_kernel<4>, dim3(blocks), dim3(256), 0, stream, up); break;
+                        default: hipLaunchKernelGGL(up2_adjoint_gate_kernel<6>, dim3(blocks), dim3(256), 0, stream, up); break;
+                    }
                 }
             }
         }

@@ -242,8 +242,6 @@ class MultiScaleUnet2dDecOnlySmallFixed(torch.nn.Module):
         params = [q.to(dev, torch.float32).contiguous() for q in self.ordered_parameters()]
         needs_grad = torch.is_grad_enabled() and (any(t.requires_grad for t in ins) or any(q.requires_grad for q in params))
         if needs_grad:
-            if p.num_input_channels != 4:
-                raise NotImplementedError("the device backward is built for num_input_channels = 4")
             return _UnetFunction.apply(self, L, *ins, *params)
         return self._run_forward([t.detach() for t in ins], [q.detach() for q in params], None)
 
