@@ -115,9 +115,11 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
     float* const s_g       = reinterpret_cast<float*>(s_mem + (size_t)kBlockPixels * kListMax * 8);
     unsigned* const s_rank = reinterpret_cast<unsigned*>(s_mem + (size_t)kBlockPixels * kListMax * 8 + (size_t)kBlockPixels * CPAD * 4);
     __shared__ double s_acc[4][C];
-    // (point, layer) pairs of a wavefront's cells that wait for a lane: place * 225 + cell; at most 63 are left over when
-    // a place adds its (at most 57) cells
-    __shared__ unsigned short s_queue[4][128];
+    // (point, layer) pairs that wait for a lane of their wavefront: slot = place * 225 + cell, and the point's compact
+    // number. The queue is emptied down to fewer than kQueueSlack pairs before a list position adds up to 64.
+    constexpr int kQueueSlack = 32, kQueue = kQueueSlack + 64;
+    __shared__ unsigned short s_qslot[4][kQueue];
+    __shared__ int s_qcid[4][kQueue];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // Blocks of 16 x 16 pixels that overlap by one row and one column (so that every cell's four pixels lie in one
@@ -316,34 +318,28 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 later += ta * S[j];
             }
         }
-    }
-    __syncthreads();
+        __syncthreads();
 
-    // ---- a row per (point, layer) pair that some pixel retained. The pairs of a block are few and unevenly spread over
-    // its cells (most cells hold one or two, some sixteen), so they are dealt out: every wavefront scans its quarter of
-    // the cells place by place, queues the slots that hold a point, and whenever 64 wait, each lane forms one row. ----
-    {
-        constexpr int kCells        = kBlockCells * kBlockCells;
-        constexpr int kCellsPerWave = (kCells + 3) / 4;
-        unsigned short* const queue = s_queue[wave];
-        const int cell       = wave * kCellsPerWave + lane;
-        const bool is_cell   = lane < kCellsPerWave && cell < kCells;
-        const bool inline_row = layer < kInlineLayers;  // (the same for the whole block)
-        int waiting = 0;  // slots in the queue (the same in every lane)
-        // forms the rows of the first `n` slots of the queue (n <= 64)
+        // ---- a row per (point, layer) pair that some pixel retained. Each pair is formed once: by the wavefront of
+        // the first of its four corner pixels that retained it, whose lane still holds the point's compact number.
+        // The pairs are unevenly spread over the pixels, so a wavefront queues {slot, compact number} of the pairs its
+        // pixels are first for, position by position, and whenever enough wait, each lane forms one row. ----
+        constexpr int kCells           = kBlockCells * kBlockCells;
+        unsigned short* const qslot    = s_qslot[wave];
+        int* const qcid                = s_qcid[wave];
+        const bool inline_row          = layer < kInlineLayers;  // (the same for the whole block)
+        const unsigned long long below = (1ull << lane) - 1ull;
+        int waiting = 0;  // pairs in the queue (the same in every lane)
+        // forms the rows of the first `n` pairs of the queue (n <= 64)
         auto form_rows = [&](int n)
         {
             if (lane < n)
             {
-                const int slot    = queue[lane];
-                const int place   = slot / kCells, c2 = slot - place * kCells;
+                const int slot  = qslot[lane];
+                int row_of      = qcid[lane];
+                const int place = slot / kCells, c2 = slot - place * kCells;
                 const int cyl = c2 / kBlockCells, cxl = c2 - cyl * kBlockCells;
                 const unsigned w4 = s_rank[slot];
-                // the point's compact number: from the list of the first corner pixel that retained it
-                const int first   = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
-                const unsigned rf = (w4 >> (8 * first)) & 0xFFu;
-                const unsigned pix = (unsigned)pix_index_mul24(p.geom, layer, x0 + cxl + (first & 1), y0 + cyl + (first >> 1));
-                int row_of         = p.lists[list_word(pix, (int)rf, p.list_depth)];
                 // past the second layer: the number of the point's first row in the overflow table
                 if (!inline_row) row_of = p.over_first[row_of];
                 float tex[CPAD], ga[4];
@@ -372,36 +368,69 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
                 }
             }
         };
-        // the first 64 slots leave the queue, the others move up
+        // the first 64 pairs leave the queue, the others move up
         auto pop64 = [&]()
         {
             form_rows(min(waiting, 64));
-            unsigned short moved = 0;
-            if (64 + lane < waiting) moved = queue[64 + lane];
+            unsigned short mslot = 0;
+            int mcid             = 0;
+            if (64 + lane < waiting) mslot = qslot[64 + lane], mcid = qcid[64 + lane];
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if (64 + lane < waiting) queue[lane] = moved;
+            if (64 + lane < waiting) qslot[lane] = mslot, qcid[lane] = mcid;
             waiting = max(waiting - 64, 0);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         };
+        // four list positions at a time (a loop over all sixteen, unrolled, would repeat the row code sixteen times;
+        // one that is not unrolled would index the registers that hold the list)
 #pragma unroll 1
-        for (int place = 0; place < kCellKeep; ++place)
+        for (int q4 = 0; q4 < kListMax / 4; ++q4)
         {
-            const int slot  = place * kCells + cell;
-            const bool has  = is_cell && s_rank[slot] != ~0u;
-            const unsigned long long mask = __ballot(has);
-            if (!mask) continue;
-            if (has) queue[waiting + (int)__popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)slot;
-            waiting += (int)__popcll(mask);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if (waiting >= 64) pop64();
+            if (4 * q4 >= mmax) break;
+            const unsigned tw = q4 == 0 ? tagw[0] : q4 == 1 ? tagw[1] : q4 == 2 ? tagw[2] : tagw[3];
+            int idq[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) idq[i] = q4 == 0 ? id[i] : q4 == 1 ? id[4 + i] : q4 == 2 ? id[8 + i] : id[12 + i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                const int j = 4 * q4 + i;
+                if (j >= mmax) break;
+                bool own = false;
+                int slot = 0;
+                if (j < m)
+                {
+                    const unsigned tag = (tw >> (8 * i)) & 0xFFu;
+                    const int w = (int)(tag >> 4) & 3, place = (int)(tag & 15u);
+                    const int cxl = px - 1 + (w & 1), cyl = py - 1 + (w >> 1);
+                    if ((unsigned)cxl < (unsigned)kBlockCells && (unsigned)cyl < (unsigned)kBlockCells)
+                    {
+                        slot              = place * kCells + cyl * kBlockCells + cxl;
+                        const unsigned w4 = s_rank[slot];
+                        // this pixel is corner 3 - w of the footprint: it forms the row if no corner before it retained the point
+                        const int first = (w4 & 0xFFu) != 0xFFu ? 0 : ((w4 >> 8) & 0xFFu) != 0xFFu ? 1 : ((w4 >> 16) & 0xFFu) != 0xFFu ? 2 : 3;
+                        own             = first == 3 - w;
+                    }
+                }
+                const unsigned long long mask = __ballot(own);
+                if (!mask) continue;
+                if (own)
+                {
+                    const int at = waiting + (int)__popcll(mask & below);
+                    qslot[at]    = (unsigned short)slot;
+                    qcid[at]     = idq[i];
+                }
+                waiting += (int)__popcll(mask);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                if (waiting >= kQueueSlack) pop64();
+            }
         }
-        if (waiting > 0) pop64();
+        while (waiting > 0) pop64();
     }
 
 #pragma unroll
