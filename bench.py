@@ -204,6 +204,8 @@ def main():
                     help="skip the separate timing of the optimiser kernel with int32 and int64 step counters")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the block that measures BASELINE configurations 1, 2 and 4 beside the headline workload")
+    ap.add_argument("--only-config", choices=("config1", "config2", "config4"), default=None,
+                    help="measure that BASELINE configuration alone and print its block (for profiler runs; no headline line)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three plain 256 MiB device copies, the yardstick for rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -223,6 +225,10 @@ def main():
         sys.exit(1)
     ctx = get_context(0)
     dev = ctx.device
+    if args.only_config:
+        print(json.dumps({args.only_config: measure_other_config(ctx, args.only_config, args.steps)}))
+        return
+
     def splat_run(order):
         """Builds config 3 with the given memory order of the points and times warm-up + steps of the splat step."""
         sc = scenes.config3(n=args.points, order=order)

@@ -328,6 +328,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
         unsigned short* const qslot    = s_qslot[wave];
         int* const qcid                = s_qcid[wave];
         const bool inline_row          = layer < kInlineLayers;  // (the same for the whole block)
+        const bool sparse              = *p.mode != 0;  // (the same for the whole view)
         const unsigned long long below = (1ull << lane) - 1ull;
         int waiting = 0;  // pairs in the queue (the same in every lane)
         // forms the rows of the first `n` pairs of the queue (n <= 64)
@@ -336,7 +337,8 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
             if (lane < n)
             {
                 const int slot  = qslot[lane];
-                int row_of      = qcid[lane];
+                const int cid   = qcid[lane];
+                int row_of      = cid;
                 const int place = slot / kCells, c2 = slot - place * kCells;
                 const int cyl = c2 / kBlockCells, cxl = c2 - cyl * kBlockCells;
                 const unsigned w4 = s_rank[slot];
@@ -365,6 +367,7 @@ __global__ __launch_bounds__(256) void backward_tiles_kernel(const BackwardParam
 #pragma unroll
                     for (int q = 0; q < NQ; ++q) row[q] = vf4{tex[4 * q], tex[4 * q + 1], tex[4 * q + 2], tex[4 * q + 3]};
                     row[NQ] = vf4{ga[0], ga[1], ga[2], ga[3]};
+                    if (sparse) p.flags[(size_t)(unsigned)cid * TRIPS_MAX_LAYERS + layer] = 1;
                 }
             }
         };
@@ -479,6 +482,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     const bool want_size = p.d_point_size != nullptr;
     const bool identity  = p.header->not_identity == 0;  // index[pid] == pid for every point
     const bool overwrite = p.overwrite != 0;             // outputs are written, not added to
+    const bool sparse    = *p.mode != 0;  // only the flagged rows exist
     // In that mode every point stores all its outputs (zeros where it has no gradient), all lanes at one place, so that
     // whole lines are written. (Descriptor columns other than the points' own, and all of them when the index is not
     // the identity, were cleared by the prologue kernel.)
@@ -521,14 +525,13 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         }
         // {softplus'(raw size), depth, layers written, size_px}
         const float4 tail = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
-        int max_layer     = live ? __float_as_int(tail.z) : 0;
-        if (live)
+        // {ip.x, ip.y, size field, confidence} of the blend record and the position: requested here, beside the point
+        // record, unless the flags decide first whether the point has any row at all
+        float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), pos = make_float4(0.f, 0.f, 0.f, 0.f);
+        auto load_point_inputs = [&]()
         {
-            const float4 r0 = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);  // ip.x ip.y size field conf
-            // (a point of one or two layers has no overflow rows, and its number there is not looked at)
-            const int first = max_layer > kInlineLayers ? p.over_first[cid] : 0;
-            // the point in view space, exactly as the projection kernel computed it
-            float4 pos = p.position[pid];
+            r0  = *reinterpret_cast<const float4*>(p.rec + (size_t)(unsigned)cid * RF);
+            pos = p.position[pid];
             if (p.displacement)
             {
                 const float* dsp = p.displacement + (size_t)pid * 3;
@@ -536,6 +539,30 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
                 pos.y += dsp[1];
                 pos.z += dsp[2];
             }
+        };
+        if (live && !sparse) load_point_inputs();
+        int max_layer = live ? __float_as_int(tail.z) : 0;
+        // (a point of one or two layers has no overflow rows, and its number there is not looked at)
+        const int first = max_layer > kInlineLayers ? p.over_first[cid] : 0;
+        // (rows past the capacity of the overflow table do not exist: the forward reported the overflow)
+        if (max_layer > kInlineLayers && (long long)first + (max_layer - kInlineLayers) > p.over_capacity)
+            max_layer = kInlineLayers + (int)max(0ll, p.over_capacity - first);
+        // the layers whose rows the point's items read: all it was written to, or those whose flag the tile pass set
+        unsigned layer_mask = (1u << max_layer) - 1u;
+        if (sparse && live)
+        {
+            // (one byte per layer at the point's compact number)
+            const unsigned long long eight = *reinterpret_cast<const unsigned long long*>(p.flags + (size_t)(unsigned)cid * TRIPS_MAX_LAYERS);
+            unsigned flagged = 0;
+#pragma unroll
+            for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
+                if ((eight >> (8 * l)) & 0xFFull) flagged |= 1u << l;
+            layer_mask &= flagged;
+            if (layer_mask) load_point_inputs();
+        }
+        if (live && layer_mask)
+        {
+            // the point in view space, exactly as the projection kernel computed it
             float view[3];
             transform_point(s_cam.cam.V, pos.x, pos.y, pos.z, view);
             const float J_softmax_proj = s_cam.cam.fx * s_cam.cam.cfx / fmaxf(view[2], 0.f);
@@ -544,13 +571,10 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
             sp[6] = __int_as_float(first);
             sp[7] = view[0], sp[8] = view[1], sp[9] = view[2];
             sp[10] = __int_as_float(cid);
-            // (rows past the capacity of the overflow table do not exist: the forward reported the overflow)
-            if (max_layer > kInlineLayers && (long long)first + (max_layer - kInlineLayers) > p.over_capacity)
-                max_layer = kInlineLayers + (int)max(0ll, p.over_capacity - first);
         }
 
         // ---- the point's items: the layers it was written to ----
-        const int my_items = max_layer;
+        const int my_items = (int)__popc(layer_mask);
         int first_item     = my_items;  // inclusive prefix over the wavefront, then made exclusive
         for (int o = 1; o < 64; o <<= 1)
         {
@@ -559,7 +583,11 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         }
         const int num_items = __builtin_amdgcn_readlane(first_item, 63);  // <= 64 * 8
         first_item -= my_items;
-        for (int l = 0; l < my_items; ++l) s_item[wave][first_item + l] = (unsigned short)(lane | (l << 8));
+        {
+            int at = first_item;
+            for (int l = 0; l < max_layer; ++l)
+                if ((layer_mask >> l) & 1u) s_item[wave][at++] = (unsigned short)(lane | (l << 8));
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -754,6 +782,8 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 // Before the two passes of a view: the rows of the view's pairs start as zeros (the tile pass writes the rows of the
 // pairs that some pixel retained, the point pass reads all rows of a point): the two inline rows of every valid point
 // (compact numbers are dense within each chunk of the binning kernels) and the overflow rows that the forward counted.
+// For a view in which few pairs are retained (sparse_pair_rows) the flag bytes of the rows are cleared instead; the choice
+// is left in the workspace for the two passes.
 // On the first view of a call also, in
 // overwrite mode (`texels`): the descriptor and confidence gradients of the columns that the point pass does not write
 // itself. With the identity index (the forward noted it in the header) those are the columns past the last point;
@@ -761,13 +791,33 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 // (background, every pose row, every intrinsics row).
 __global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader* __restrict__ header, const int32_t* __restrict__ chunk_valid,
                                                                 int bin_groups, int points_per_block, float* __restrict__ rows_inline,
-                                                                float* __restrict__ rows_over, int pair_row, long long over_capacity,
+                                                                float* __restrict__ rows_over, unsigned char* __restrict__ flags, int32_t* __restrict__ mode, int pair_row, long long over_capacity,
                                                                 float* __restrict__ d_texture,
                                                                 float* __restrict__ d_confidence, int channels, int num_texels,
                                                                 int num_points, int texels, int clear_sums,
                                                                 float* __restrict__ d_background, double* __restrict__ d_pose,
                                                                 int num_images, float* __restrict__ d_intrinsics, int num_cameras)
 {
+    long long over_rows = (long long)header->overflow_rows;
+    if (over_rows > over_capacity) over_rows = over_capacity;
+    // the view's retained entries: every workgroup adds the blend kernel's partial sums up for itself
+    __shared__ unsigned long long s_retained[4];
+    {
+        unsigned long long r = (unsigned long long)(unsigned)chunk_valid[bin_groups + threadIdx.x];  // (kRetainedParts = 256 threads)
+        for (int o = 32; o > 0; o >>= 1) r += __shfl_xor(r, o);
+        if ((threadIdx.x & 63) == 0) s_retained[threadIdx.x >> 6] = r;
+        __syncthreads();
+    }
+    const bool sparse = sparse_pair_rows((s_retained[0] + s_retained[1] + s_retained[2] + s_retained[3]) * kRetainedSample, header->n_entries);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *mode = sparse ? 1 : 0;
+    if (sparse)
+    {
+        // (the table ends on a multiple of 256 bytes: whole 16-byte words are cleared)
+        const long long words = ((long long)num_points * TRIPS_MAX_LAYERS + 15) / 16;
+        for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < words; i += (long long)gridDim.x * 256)
+            reinterpret_cast<vu4*>(flags)[i] = vu4{0u, 0u, 0u, 0u};
+    }
+    else
     {
         // (rows are a multiple of four floats)
         const int row_quads = kInlineLayers * pair_row / 4;
@@ -778,9 +828,7 @@ __global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader
             vf4* dst        = reinterpret_cast<vf4*>(rows_inline) + (size_t)begin * row_quads;
             for (int i = threadIdx.x; i < quads; i += 256) __builtin_nontemporal_store(vf4{0.f, 0.f, 0.f, 0.f}, dst + i);
         }
-        long long rows = (long long)header->overflow_rows;
-        if (rows > over_capacity) rows = over_capacity;
-        const long long quads = rows * pair_row / 4;
+        const long long quads = over_rows * pair_row / 4;
         vf4* dst              = reinterpret_cast<vf4*>(rows_over);
         for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < quads; i += (long long)gridDim.x * 256)
             __builtin_nontemporal_store(vf4{0.f, 0.f, 0.f, 0.f}, dst + i);
@@ -834,7 +882,8 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
     {
         ProfScope ps(prof, "backward_prologue", stream);
         hipLaunchKernelGGL(backward_prologue_kernel, dim3(2048), dim3(256), 0, stream, p.header, p.chunk_valid, p.bin_groups,
-                           p.points_per_block, p.rows_inline, p.rows_over, pair_row_floats((channels + 3) & ~3), p.over_capacity, p.d_texture, p.d_confidence, channels, p.num_texels,
+                           p.points_per_block, p.rows_inline, p.rows_over, p.flags, p.mode, pair_row_floats((channels + 3) & ~3),
+                           p.over_capacity, p.d_texture, p.d_confidence, channels, p.num_texels,
                            N, p.overwrite, p.clear_block_sums, p.d_background, p.d_pose_all, p.num_images, p.d_intrinsics_all,
                            p.num_cameras);
     }
@@ -858,7 +907,9 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
     if (N > 0)
     {
         ProfScope ps(prof, "backward_points", stream);
-        const int blocks = min((N + 255) / 256, 4096);
+        // (four workgroups per CU, each walking its share of the points: every further workgroup adds its atomics on the
+        // pose and intrinsics sums)
+        const int blocks = min((N + 255) / 256, 1024);
         TRIPS_BW_DISPATCH(backward_points_kernel, blocks);
     }
     return hipGetLastError();

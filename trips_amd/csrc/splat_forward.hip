@@ -386,6 +386,7 @@ __global__ __launch_bounds__(1024) void scan_plan_kernel(const int32_t* __restri
             if ((int)threadIdx.x < G) chunk_valid[4 * G + threadIdx.x] = prefix;
             if ((int)threadIdx.x == G - 1) s_over_total = prefix + mine;
             if (saved_chunk_valid && (int)threadIdx.x < G) saved_chunk_valid[threadIdx.x] = chunk_valid[threadIdx.x];
+            if (saved_chunk_valid && (int)threadIdx.x < kRetainedParts) saved_chunk_valid[G + threadIdx.x] = 0;  // (the blend adds)
             __syncthreads();
         }
         for (int o = 32; o > 0; o >>= 1)
@@ -1423,6 +1424,17 @@ __global__ __launch_bounds__(256) void blend_kernel(const ForwardParams p)
             if (4 * q < nmax && 4 * q < n)
                 __builtin_nontemporal_store(vi4{(int)id[4 * q], (int)id[4 * q + 1], (int)id[4 * q + 2], (int)id[4 * q + 3]}, mine + (q << 6));
         if (n > 0) __builtin_nontemporal_store(vu4{tagw[0], tagw[1], tagw[2], tagw[3]}, reinterpret_cast<vu4*>(p.tags) + (unsigned)pix);
+        // the view's retained entries, for the backward's choice of how it keeps its pair rows: estimated from every
+        // kRetainedSample-th workgroup, one atomic per wavefront (the sum of 64 values of at most 16, a ballot per bit),
+        // spread over kRetainedParts counters
+        unsigned wave_ret = 0;
+        if (blockIdx.x % (unsigned)kRetainedSample == 0)
+        {
+#pragma unroll
+            for (int b = 0; b < 5; ++b) wave_ret += (unsigned)__popcll(__ballot(live && ((ret >> b) & 1))) << b;
+        }
+        if (lane == 0 && wave_ret)
+            atomicAdd(p.saved_chunk_valid + p.bin_groups + (int)((blockIdx.x / (unsigned)kRetainedSample * 4u + (unsigned)wave) % (unsigned)kRetainedParts), (int)wave_ret);
     }
 }
 

@@ -240,6 +240,18 @@ struct ViewHeader
     unsigned long long overflow_rows;
 };
 
+// Most (point, layer) pairs of a usual view are retained by some pixel, and the backward then clears and reads the rows
+// of all pairs. In a view whose lists are mostly hidden behind their first entries only a few pairs are: the backward
+// then keeps a flag byte per row instead, clears only those, and its point pass reads only the rows whose flag the tile
+// pass has set. The blend kernel adds the view's retained entries up in kRetainedParts counters (one atomic per
+// wavefront; on a single counter they would queue up for longer than the kernel runs), the backward's first kernel
+// sums them and leaves the choice in the workspace for the two passes.
+constexpr int kRetainedParts = 256;
+// (An estimate is enough for that choice, both ways of keeping the rows give the same gradients: every
+// kRetainedSample-th workgroup of the blend kernel contributes.)
+constexpr int kRetainedSample = 16;
+__host__ __device__ inline bool sparse_pair_rows(unsigned long long retained, unsigned long long pairs) { return 4ull * retained < pairs; }
+
 // Layout of one view's saved state (all offsets in bytes, 256-aligned)
 struct SavedLayout
 {
@@ -255,7 +267,8 @@ struct SavedLayout
     size_t over_first;  // int32 [N] by compact number: for a point written to more than two layers, the number of its
                         // first row in the backward's overflow table (rows numbered densely in point order)
     size_t chunk_valid;  // int32 [kBinGroups] valid points of every chunk of the binning kernels (their compact numbers
-                         // start at the chunk's first point number)
+                         // start at the chunk's first point number), then [kRetainedParts] partial sums of the view's
+                         // retained entries
     size_t bytes_per_view;
 };
 
@@ -270,6 +283,9 @@ struct BackwardWorkspaceLayout
 {
     size_t rows_inline;  // float [N, kInlineLayers, pair_row_floats] by compact number
     size_t rows_over;    // float [over_capacity, pair_row_floats]
+    size_t flags;         // uint8 [N, TRIPS_MAX_LAYERS] by compact number: 1 where the tile pass wrote the pair's row
+                          // (only for views in which few pairs are retained)
+    size_t mode;          // int32: 1 = only flagged rows exist (written by the prologue kernel)
     size_t over_capacity;
     size_t bytes;
 };
@@ -345,7 +361,7 @@ struct ForwardParams
     int32_t* retained;
     unsigned char* tags;  // training only
     int32_t* over_first;  // training only
-    int32_t* saved_chunk_valid;  // training only
+    int32_t* saved_chunk_valid;  // training only: [kBinGroups + kRetainedParts]
     ViewHeader* header;  // counters of this view
     ViewHeader* status;  // overflow flag of the whole forward call (start of the workspace)
     float* image[TRIPS_MAX_LAYERS];
@@ -375,10 +391,12 @@ struct BackwardParams
     const float* grad_image[TRIPS_MAX_LAYERS];
     const unsigned char* tags;  // [Pi, 16] (saved state) cell and place in the cell's list of every list position
     const int32_t* over_first;   // [N] (saved state) by compact number
-    const int32_t* chunk_valid;  // [kBinGroups] (saved state)
+    const int32_t* chunk_valid;  // [kBinGroups + kRetainedParts] (saved state)
+    int32_t* mode;               // (workspace) 1 = only flagged rows exist
     int32_t bin_groups, points_per_block;
     float* rows_inline;  // [N, kInlineLayers, pair_row_floats] (workspace)
     float* rows_over;    // [over_capacity, pair_row_floats] (workspace)
+    unsigned char* flags;  // [N, TRIPS_MAX_LAYERS] (workspace) by compact number
     // blocks of the tile pass (16 x 16 pixels, 15 apart): first block of each layer, blocks per block row of each layer
     int32_t blocks_off[TRIPS_MAX_LAYERS + 1];
     int32_t blocks_x[TRIPS_MAX_LAYERS];

@@ -221,7 +221,7 @@ SavedLayout saved_layout(const TripsSplatDesc& d, const PyramidGeom& g)
     s.over_first = o;
     o += align256(N * sizeof(int32_t));
     s.chunk_valid = o;
-    o += align256((size_t)kBinGroups * sizeof(int32_t));
+    o += align256((size_t)(kBinGroups + kRetainedParts) * sizeof(int32_t));
     s.bytes_per_view = o;
     return s;
 }
@@ -288,6 +288,10 @@ BackwardWorkspaceLayout backward_workspace_layout(const TripsSplatDesc& d, const
     o += align256((size_t)d.num_points * kInlineLayers * row);
     w.rows_over = o;
     o += align256(w.over_capacity * row);
+    w.flags = o;
+    o += align256((size_t)d.num_points * TRIPS_MAX_LAYERS);
+    w.mode = o;
+    o += 256;
     w.bytes = o;
     return w;
 }
@@ -571,6 +575,8 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.points_per_block = (d.num_points + kBinGroups - 1) / kBinGroups;
         p.rows_inline  = reinterpret_cast<float*>(ws + bl.rows_inline);
         p.rows_over    = reinterpret_cast<float*>(ws + bl.rows_over);
+        p.flags        = reinterpret_cast<unsigned char*>(ws + bl.flags);
+        p.mode         = reinterpret_cast<int32_t*>(ws + bl.mode);
         p.over_capacity = (long long)bl.over_capacity;
         p.blocks_off[0] = 0;
         for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
