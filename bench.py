@@ -31,16 +31,18 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "5b71e9a27a10fa76f013affe06541409e80f7e317b3c265497fefd3d6d0a417f"
+PMC_SOURCES_SHA256 = "0262f38ac2fe1907fde5da1bf2956b9f3ee31bd250d6a742519c11a75c3e3fc4"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129125, 292728),
-    "bin_scatter": (88876, 152867),
-    "tile_count": (13142, 2296),
-    "tile_scatter": (32640, 110285),
-    "sort_blend": (333383, 350795),
-    "backward_tiles": (453556, 296281),
-    "backward_points": (866929, 234887),
-    "adam_fused": (383862, 498420),
+    "project_bin": (129116, 251278),
+    "bin_scatter": (95990, 166508),
+    "tile_count": (13141, 2296),
+    "tile_scatter": (32593, 110316),
+    "cell_sort": (35543, 42964),
+    "blend": (318216, 196234),
+    "backward_prologue": (55, 265145),
+    "backward_tiles": (425952, 121583),
+    "backward_points": (297269, 234503),
+    "adam_fused": (383877, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
@@ -79,10 +81,12 @@ def merge_parts(prof):
 
 
 def measured_traffic_bytes(kernel, usable=True):
-    if not usable or kernel not in PMC_KIB_DEFAULT_WORKLOAD:
+    """HBM bytes per launch from the committed counter profile; a kernel reported with parts is the sum of its parts."""
+    parts = KERNEL_PARTS.get(kernel, (kernel,))
+    if not usable or any(k not in PMC_KIB_DEFAULT_WORKLOAD for k in parts):
         return None
-    f, w = PMC_KIB_DEFAULT_WORKLOAD[kernel]
-    return int((f * PMC_FETCH_SCALE + w * PMC_WRITE_SCALE) * 1024)
+    return sum(int((PMC_KIB_DEFAULT_WORKLOAD[k][0] * PMC_FETCH_SCALE + PMC_KIB_DEFAULT_WORKLOAD[k][1] * PMC_WRITE_SCALE) * 1024)
+               for k in parts)
 
 
 def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam_step_bytes=4):

@@ -466,11 +466,12 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
                 }
             }
         };
+        // (one gather for all lanes of a wavefront, whatever their group: lanes of both kinds sit side by side)
         float a[8];
+        gather(q == 0 ? 0 : base8 + ch0, a);
         if (q == 0)
         {
             // positions [0, C) are the finer level's own image, [C, 2C) this level's
-            gather(0, a);
 #pragma unroll
             for (int c = 0; c < 4; ++c)
             {
@@ -484,7 +485,6 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
         else
         {
             // output ch0 + i of this level sits at position 2 C + ch0 + i = base8 + ch0 + SHIFT + i
-            gather(base8 + ch0, a);
             if (SHIFT != 0)
             {
                 float hi[8];
