@@ -43,7 +43,8 @@ __device__ __forceinline__ bool adam_element(const AdamScalars& h, float gradien
                                              float& v, long long& step, float& new_weight, uint32_t lr_step = 0,
                                              float lr_of_step = 0.f)
 {
-    float gradient = gradient_raw / h.loss_scale;
+    float gradient = gradient_raw;
+    if (h.loss_scale != 1.f) gradient = gradient_raw / h.loss_scale;  // (a division by 1 changes nothing: skipped)
     if (gradient == 0.f) return false;  // parameter not seen in this step (MyAdam.cu:57-61)
     const float gradient_sq   = gradient * gradient;
     const float first_moment  = h.beta1 * m + (1 - h.beta1) * gradient;
@@ -100,11 +101,16 @@ __device__ __forceinline__ void adam_block(const AdamTable& tab, int ti)
         else
             *reinterpret_cast<int4*>(&s[0]) = *reinterpret_cast<const int4*>(st + i0);
         long long s0 = s[0], s1 = s[1], s2 = s[2], s3 = s[3];
+        // The four elements are mostly updated together, so their counters agree: the bias correction (two powf, a square
+        // root, a division) of the run's largest counter is computed once and taken by every element whose new counter
+        // equals it.
+        const uint32_t top = (uint32_t)max(max(s0, s1), max(s2, s3)) + 1u;
+        const float top_lr = adam_corrected_lr(h, top);
         float nw;
-        if (adam_element(h, g4.x, w4.x, m4.x, v4.x, s0, nw)) w4.x = nw;
-        if (adam_element(h, g4.y, w4.y, m4.y, v4.y, s1, nw)) w4.y = nw;
-        if (adam_element(h, g4.z, w4.z, m4.z, v4.z, s2, nw)) w4.z = nw;
-        if (adam_element(h, g4.w, w4.w, m4.w, v4.w, s3, nw)) w4.w = nw;
+        if (adam_element(h, g4.x, w4.x, m4.x, v4.x, s0, nw, top, top_lr)) w4.x = nw;
+        if (adam_element(h, g4.y, w4.y, m4.y, v4.y, s1, nw, top, top_lr)) w4.y = nw;
+        if (adam_element(h, g4.z, w4.z, m4.z, v4.z, s2, nw, top, top_lr)) w4.z = nw;
+        if (adam_element(h, g4.w, w4.w, m4.w, v4.w, s3, nw, top, top_lr)) w4.w = nw;
         s[0] = (STEP)s0, s[1] = (STEP)s1, s[2] = (STEP)s2, s[3] = (STEP)s3;
         *reinterpret_cast<float4*>(w + i0)  = w4;
         *reinterpret_cast<float4*>(mo + i0) = m4;
@@ -295,9 +301,20 @@ __global__ __launch_bounds__(256) void adam_points_kernel(const AdamPointsParams
             const int t = e < 4 ? 0 : e == 4 ? 1 : e < 5 + C ? 2 : 3;
             top[t]      = max(top[t], (int)row[3 * e + 2]);
         }
+        // (and tensors with the same learning rate and betas whose largest counters agree share it: usually all four)
         float top_lr[4];
+        top_lr[0] = adam_corrected_lr(p.h[0], (uint32_t)(top[0] + 1));
 #pragma unroll
-        for (int t = 0; t < 4; ++t) top_lr[t] = adam_corrected_lr(p.h[t], (uint32_t)(top[t] + 1));
+        for (int t = 1; t < 4; ++t)
+        {
+            const bool same_scalars = p.h[t].lr == p.h[0].lr && p.h[t].beta1 == p.h[0].beta1 && p.h[t].beta2 == p.h[0].beta2;
+            const bool shares       = same_scalars && top[t] == top[0];
+            top_lr[t]               = top_lr[0];
+            if (__ballot(!shares))  // (skipped by the whole wavefront in the usual case)
+            {
+                if (!shares) top_lr[t] = adam_corrected_lr(p.h[t], (uint32_t)(top[t] + 1));
+            }
+        }
 #pragma unroll
         for (int e = 0; e < E; ++e)
         {
