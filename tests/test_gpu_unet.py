@@ -68,6 +68,21 @@ def test_unet_forward_three_input_channels():
     _compare(net, inputs)
 
 
+@pytest.mark.parametrize("cin,filters,levels,w,h", [
+    (6, [24, 32, 64], 3, 70, 50),        # the coarser level's outputs start at position 12 of the finer block's input
+    (8, [32, 48, 64, 64], 4, 96, 72),    # ... at 16
+    (16, [48, 64, 64], 3, 70, 50),       # ... at 32: the image fills the first two groups of eight
+    (16, [40], 1, 40, 24),               # start block only
+])
+def test_unet_forward_more_input_channels(cin, filters, levels, w, h):
+    """The descriptor widths of the splat beyond four (6, 8, 16 channels per image)."""
+    net = _net(filters, levels, seed=40 + cin, cin=cin)
+    inputs = _pyramid(w, h, levels, cin, batch=2, seed=50 + cin)
+    if levels == 1:
+        net.final = torch.nn.Sequential(torch.nn.Conv2d(filters[0] - cin, 3, 1), torch.nn.Identity())
+    _compare(net, inputs)
+
+
 def test_unet_packed_weights_are_reused_on_request():
     """A viewer's frames: with reuse_packed_weights the fp16 weights are packed by the first no-grad forward only
     (TripsUnetDesc.weights_packed); the later frames give the same bits, and a changed weight takes effect after

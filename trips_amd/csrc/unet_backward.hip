@@ -1196,6 +1196,7 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
     if (!weights || !inputs || !saved || !d_output || !grads || !workspace) return set_error(TRIPS_ERR_INVALID_ARG, "NULL argument");
     const TripsUnetDesc& d = *desc;
     const int C = d.num_input_channels, L = d.num_levels;
+    if (C > 4) return set_error(TRIPS_ERR_UNSUPPORTED, "the backward is built for num_input_channels 1..4 (got %d)", C);
     if (!(grad_scale > 0.f) || !std::isfinite(grad_scale)) return set_error(TRIPS_ERR_INVALID_ARG, "grad_scale must be positive");
     for (int i = 0; i < L; ++i)
     {

@@ -19,7 +19,8 @@ constexpr int kConvPatchW  = kConvTileW + 2;
 constexpr int kBelowH      = kConvTileH / 2 + 2;  // rows / columns of the level below that an upsampled patch touches
 constexpr int kBelowW      = kConvTileW / 2 + 2;
 constexpr int kFinalPixelsPerBlock = 512;   // pixels a workgroup of the 1x1 convolution's backward takes at a time
-constexpr int kFinalPartFloats     = 4 * (4 + 64) + 4;  // its partial sums: [4 outputs][4 image + <= 64 block channels], 4 biases
+constexpr int kUnetMaxImageChannels = 16;  // channels of the splat images (the descriptor widths of the splat: 3, 4, 6, 8, 16)
+constexpr int kFinalPartFloats     = 4 * (kUnetMaxImageChannels + 64) + 4;  // its partial sums: [4 outputs][<= 16 image + <= 64 block channels], 4 biases
 constexpr int kLdsChanPad  = 8;  // halves added to every LDS row so that 16 lanes reading 16 bytes hit 64 distinct banks
 
 // source row / column and weight of torch's bilinear upsampling with scale_factor 2, align_corners = false
@@ -207,8 +208,8 @@ inline int check_unet_desc(const TripsUnetDesc* d)
         return set_error(TRIPS_ERR_INVALID_ARG, "abi_version %d, library has %d", d->abi_version, TRIPS_ABI_VERSION);
     if (d->num_levels < 1 || d->num_levels > TRIPS_UNET_MAX_LEVELS)
         return set_error(TRIPS_ERR_INVALID_ARG, "num_levels %d not in 1..%d", d->num_levels, TRIPS_UNET_MAX_LEVELS);
-    if (d->num_input_channels < 1 || d->num_input_channels > 4)
-        return set_error(TRIPS_ERR_UNSUPPORTED, "num_input_channels %d not in 1..4", d->num_input_channels);
+    if (d->num_input_channels < 1 || d->num_input_channels > kUnetMaxImageChannels)
+        return set_error(TRIPS_ERR_UNSUPPORTED, "num_input_channels %d not in 1..%d", d->num_input_channels, kUnetMaxImageChannels);
     if (d->num_output_channels < 1 || d->num_output_channels > 4)
         return set_error(TRIPS_ERR_UNSUPPORTED, "num_output_channels %d not in 1..4", d->num_output_channels);
     if (d->batch < 1) return set_error(TRIPS_ERR_INVALID_ARG, "batch < 1");

@@ -47,9 +47,11 @@ struct ConvParams
     int final_cout;
 };
 
-template <int CIN, int NPAD, int THREADS>
+// CI: image channels the kernel has room for (4, 8 or 16; C <= CI)
+template <int CIN, int NPAD, int THREADS, int CI>
 __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams p)
 {
+    constexpr int IQ = CI / 4;  // 16-byte items that carry the image of a pixel of the level below
     constexpr int MB = 16 / (THREADS / 64);  // 16-pixel row blocks of a wavefront: two rows of the tile, or one
     constexpr int ROW  = CIN + kLdsChanPad;  // halves per patch pixel in LDS
     constexpr int NB   = NPAD / 16;          // 16-column blocks; the first half are feature outputs
@@ -62,12 +64,13 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     ConvTapStage<CIN, NPAD, THREADS> taps;
     conv_tap_fetch(taps, p.wpack, 0);  // in flight while the patch is assembled
     // weights and biases of the 1x1 output convolution, rounded to fp16 like every other operand
-    __shared__ float s_fw[4 * (4 + 64) + 4];
+    constexpr int kFwBias = 4 * (CI + 64);  // [final_cout <= 4][C + cout <= CI + 64] weights, then the biases
+    __shared__ float s_fw[kFwBias + 4];
     if (p.final_out)
     {
         const int cin = p.c_feat + p.cout;
         for (int i = threadIdx.x; i < p.final_cout * cin; i += THREADS) s_fw[i] = float(_Float16(p.final_w[i]));
-        if ((int)threadIdx.x < p.final_cout) s_fw[4 * (4 + 64) + threadIdx.x] = p.final_b[threadIdx.x];
+        if ((int)threadIdx.x < p.final_cout) s_fw[kFwBias + threadIdx.x] = p.final_b[threadIdx.x];
     }
 
     // ---- stage 1: everything the patch needs from memory, all loads of a thread in flight together ----
@@ -81,12 +84,12 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     // item by item, a thread's five round trips to memory ran one after the other and stage 1 was 39 % of a
     // workgroup's life)
     constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + THREADS - 1) / THREADS;
-    constexpr int kMaxPerPix  = 1 + CIN / 8;  // image below + groups of 8 block outputs
+    constexpr int kMaxPerPix  = IQ + CIN / 8;  // image below (four channels per item) + groups of 8 block outputs
     constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + THREADS - 1) / THREADS;
-    float feat_v[kFeatItems][4];
+    float feat_v[kFeatItems][CI];
     uint4 below_v[kBelowItems];
     const int act_groups = has_below ? p.cb_store / 8 : 0;
-    const int per_pixel  = 1 + act_groups;  // item 0 of a pixel: the image below; others: 8 activations each
+    const int per_pixel  = IQ + act_groups;  // items 0 .. IQ - 1 of a pixel: the image below; others: 8 activations each
     {
         const size_t plane = (size_t)p.H * p.W;
 #pragma unroll
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
             const int y = y0 + py - 1, x = x0 + px - 1;
             const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) feat_v[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+            for (int c = 0; c < CI; ++c) feat_v[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
         }
     }
     if (has_below)
@@ -113,16 +116,16 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
                 const int q = item % per_pixel, bp = item / per_pixel;
                 const int r = bp / kBelowW, c0 = bp - r * kBelowW;
                 const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
-                if (q == 0)
+                if (q < IQ)
                 {
                     const float* src = p.feat_below + (size_t)yy * p.Wb + xx;
                     float f[4];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) f[c] = c < C ? src[c * pb] : 0.f;
+                    for (int c = 0; c < 4; ++c) f[c] = 4 * q + c < C ? src[(size_t)(4 * q + c) * pb] : 0.f;
                     below_v[k] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
                 }
                 else
-                    below_v[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+                    below_v[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - IQ));
             }
         }
     }
@@ -133,13 +136,13 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
         if (item < kConvPatchH * kConvPatchW)
         {
             _Float16* row = s_patch + (size_t)item * ROW;
-            if (C == 4)  // one 8-byte LDS store instead of four 2-byte ones
+            if (CI == 4 && C == 4)  // one 8-byte LDS store instead of four 2-byte ones
                 *reinterpret_cast<half4*>(row) =
                     half4{_Float16(feat_v[k][0]), _Float16(feat_v[k][1]), _Float16(feat_v[k][2]), _Float16(feat_v[k][3])};
             else
             {
 #pragma unroll
-                for (int c = 0; c < 4; ++c)  // (a run-time bound would put the register array into scratch memory)
+                for (int c = 0; c < CI; ++c)  // (a run-time bound would put the register array into scratch memory)
                     if (c < C) row[c] = _Float16(feat_v[k][c]);
             }
             if (!has_below)
@@ -159,23 +162,24 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
             {
                 const int q = item % per_pixel, bp = item / per_pixel;
                 _Float16* row = s_below + (size_t)bp * ROW;
-                if (q == 0)
+                if (q < IQ)
                 {
                     const float f[4] = {__uint_as_float(below_v[k].x), __uint_as_float(below_v[k].y), __uint_as_float(below_v[k].z),
                                         __uint_as_float(below_v[k].w)};
-                    if (C == 4)
+                    if (CI == 4 && C == 4)
                         *reinterpret_cast<half4*>(row + 4) = half4{_Float16(f[0]), _Float16(f[1]), _Float16(f[2]), _Float16(f[3])};
                     else
                     {
 #pragma unroll
                         for (int c = 0; c < 4; ++c)
-                            if (c < C) row[C + c] = _Float16(f[c]);
+                            if (4 * q + c < C) row[C + 4 * q + c] = _Float16(f[c]);
                     }
-                    for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);  // padding channels
+                    if (q == 0)
+                        for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);  // padding channels
                 }
                 else
                 {
-                    const int pos = 2 * C + 8 * (q - 1);
+                    const int pos = 2 * C + 8 * (q - IQ);
                     if (C == 4)
                         *reinterpret_cast<uint4*>(row + pos) = below_v[k];
                     else
@@ -217,13 +221,17 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
                 h = __builtin_elementwise_fma(d, W11, __builtin_elementwise_fma(c, W10, __builtin_elementwise_fma(b, W01, a * W00)));
             }
             _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
-            if (g == 0)
+            if (8 * g < C)
             {
                 // [0, C) holds this level's image
-                if (C == 4)
+                if (CI == 4 && C == 4)
                     *reinterpret_cast<half4*>(dst + 4) = half4{h[4], h[5], h[6], h[7]};
                 else
-                    for (int i = C; i < 8; ++i) dst[i] = h[i];
+                {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        if (8 * g + i >= C) dst[i] = h[i];
+                }
             }
             else
                 *reinterpret_cast<half8*>(dst) = h;
@@ -242,15 +250,20 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
 
     // ---- epilogue: elu(feature) * sigmoid(mask) in fp16, staged in LDS (the patch is no longer needed) and
     // written channels innermost with full-line stores; the pre-activations too when the backward needs them ----
-    constexpr int AS = NPAD / 2 + kLdsChanPad, PS = NPAD + kLdsChanPad;
+    constexpr int IPAD = CI > kLdsChanPad ? CI : kLdsChanPad;  // padding columns of a staged row: room for the image
+    constexpr int AS = NPAD / 2 + IPAD, PS = NPAD + kLdsChanPad;
     _Float16* s_act = smem;                                      // [256][AS]
     _Float16* s_pre = smem + kConvTileH * kConvTileW * AS;       // [256][PS]
-    float my_feat[4] = {0.f, 0.f, 0.f, 0.f};  // this thread's pixel of the image, as the convolution saw it (fp16)
+    float my_feat[CI];  // this thread's pixel of the image, as the convolution saw it (fp16)
+#pragma unroll
+    for (int c = 0; c < CI; ++c) my_feat[c] = 0.f;
     const bool owns_pixel = THREADS == kConvTileH * kConvTileW || (int)threadIdx.x < kConvTileH * kConvTileW;  // one thread per pixel
     if (p.final_out && owns_pixel)
     {
         const _Float16* row = s_patch + (size_t)((threadIdx.x / kConvTileW + 1) * kConvPatchW + threadIdx.x % kConvTileW + 1) * ROW;
-        for (int c = 0; c < C; ++c) my_feat[c] = float(row[c]);
+#pragma unroll
+        for (int c = 0; c < CI; ++c)
+            if (c < C) my_feat[c] = float(row[c]);
     }
     __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
@@ -290,15 +303,15 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
         // `final` of the net (Networks.h:1129-1131) on the matrix cores: per 16 pixels one MFMA per 32 input channels,
         // A = the staged tile rows (block outputs, then the image in the row's padding columns), B = the 1x1 weights,
         // rounded to fp16 like every other operand, outputs in the first columns.
-        constexpr int KF  = NPAD / 2 + kLdsChanPad;  // block outputs (padded) | image | zeros
+        constexpr int KF  = NPAD / 2 + IPAD;  // block outputs (padded) | image | zeros
         constexpr int KFB = (KF + 31) / 32;
         const int cin     = C + p.cout;
-        // the image joins the staged rows (columns NPAD/2 .. NPAD/2 + 7; nobody has read them yet)
+        // the image joins the staged rows (columns NPAD/2 .. NPAD/2 + IPAD - 1; nobody has read them yet)
         if (owns_pixel)
         {
             _Float16* row = s_act + (size_t)threadIdx.x * AS + NPAD / 2;
 #pragma unroll
-            for (int c = 0; c < kLdsChanPad; ++c) row[c] = c < C ? _Float16(my_feat[c]) : _Float16(0.f);
+            for (int c = 0; c < IPAD; ++c) row[c] = (c < CI && c < C) ? _Float16(my_feat[c < CI ? c : 0]) : _Float16(0.f);
         }
         half8 bfin[KFB];
 #pragma unroll
@@ -319,7 +332,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
             }
         __syncthreads();  // image columns in place
         const size_t plane = (size_t)p.H * p.W;
-        const float fb     = lrow < p.final_cout ? s_fw[4 * (4 + 64) + lrow] : 0.f;
+        const float fb     = lrow < p.final_cout ? s_fw[kFwBias + lrow] : 0.f;
 #pragma unroll
         for (int m = 0; m < MB; ++m)
         {
@@ -400,42 +413,52 @@ __global__ __launch_bounds__(256) void pack_conv_weights_kernel(const PackTable 
 // ---------------------------------------------------------------------------------------------------------
 namespace
 {
-template <int CIN, int NPAD>
+template <int CIN, int NPAD, int CI>
 hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
 {
     constexpr int ROW  = CIN + kLdsChanPad;
+    constexpr int IPAD = CI > kLdsChanPad ? CI : kLdsChanPad;
     // the patch, then the patch of the level below or (later) two tap buffers of the weights, whichever is larger
     const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW * ROW + std::max(kBelowH * kBelowW * ROW, 2 * NPAD * ROW)) * sizeof(_Float16);
-    const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NPAD / 2 + kLdsChanPad) + (p.pre ? NPAD + kLdsChanPad : 0)) * sizeof(_Float16);
+    const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NPAD / 2 + IPAD) + (p.pre ? NPAD + kLdsChanPad : 0)) * sizeof(_Float16);
     const size_t lds     = std::max(lds_in, lds_out);  // up to 104 KB when the largest block saves its pre-activations
     // eight wavefronts per tile (one row each): the phases around the tap loop run at the latency of their loads and LDS
     // round trips, and twice the wavefronts per tile hide twice as much of it
     constexpr int THREADS = 512;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD, THREADS>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gated_conv3x3_kernel<CIN, NPAD, THREADS, CI>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     dim3 grid((p.W + kConvTileW - 1) / kConvTileW, (p.H + kConvTileH - 1) / kConvTileH);
-    hipLaunchKernelGGL((gated_conv3x3_kernel<CIN, NPAD, THREADS>), grid, dim3(THREADS), lds, stream, p);
+    hipLaunchKernelGGL((gated_conv3x3_kernel<CIN, NPAD, THREADS, CI>), grid, dim3(THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
-hipError_t dispatch_conv(const ConvParams& p, int cin_pad, int npad, hipStream_t stream)
+template <int CI>
+hipError_t dispatch_conv_ci(const ConvParams& p, int cin_pad, int npad, hipStream_t stream)
 {
     if (cin_pad == 32)
     {
-        if (npad == 32) return launch_conv<32, 32>(p, stream);
-        if (npad == 64) return launch_conv<32, 64>(p, stream);
-        if (npad == 96) return launch_conv<32, 96>(p, stream);
-        if (npad == 128) return launch_conv<32, 128>(p, stream);
+        if (npad == 32) return launch_conv<32, 32, CI>(p, stream);
+        if (npad == 64) return launch_conv<32, 64, CI>(p, stream);
+        if (npad == 96) return launch_conv<32, 96, CI>(p, stream);
+        if (npad == 128) return launch_conv<32, 128, CI>(p, stream);
     }
     else
     {
-        if (npad == 32) return launch_conv<64, 32>(p, stream);
-        if (npad == 64) return launch_conv<64, 64>(p, stream);
-        if (npad == 96) return launch_conv<64, 96>(p, stream);
-        if (npad == 128) return launch_conv<64, 128>(p, stream);
+        if (npad == 32) return launch_conv<64, 32, CI>(p, stream);
+        if (npad == 64) return launch_conv<64, 64, CI>(p, stream);
+        if (npad == 96) return launch_conv<64, 96, CI>(p, stream);
+        if (npad == 128) return launch_conv<64, 128, CI>(p, stream);
     }
     return hipErrorInvalidValue;
+}
+
+// (the kernel is built for 4, 8 and 16 image channels; fewer use the next size up)
+hipError_t dispatch_conv(const ConvParams& p, int cin_pad, int npad, hipStream_t stream)
+{
+    if (p.c_feat <= 4) return dispatch_conv_ci<4>(p, cin_pad, npad, stream);
+    if (p.c_feat <= 8) return dispatch_conv_ci<8>(p, cin_pad, npad, stream);
+    return dispatch_conv_ci<16>(p, cin_pad, npad, stream);
 }
 }  // namespace
 }  // namespace trips
