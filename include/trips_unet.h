@@ -36,7 +36,7 @@ extern "C" {
 typedef struct TripsUnetDesc {
     int32_t abi_version;          /* TRIPS_ABI_VERSION */
     int32_t num_levels;           /* L, 1..8: in[0..L-1] are consumed (MultiScaleUnet2dParams::num_layers) */
-    int32_t num_input_channels;   /* C, 1..4 (4 in every shipped config) */
+    int32_t num_input_channels;   /* C, 1..16 (4 in every shipped config; the kernels are built with room for 4, 8, 16) */
     int32_t num_output_channels;  /* 1..4 (3) */
     int32_t batch;                /* images per call */
     int32_t filters[TRIPS_UNET_MAX_LEVELS];  /* F[0..L-1] (filters_network); conv outputs must be >= 1 and <= 64 */
@@ -91,7 +91,7 @@ int trips_unet_forward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnet
  * Intermediate gradients are fp16: they are carried multiplied by grad_scale (a power of two such as 65536 keeps
  * dL/doutput ~ 1e-7 of a mean loss over millions of pixels in range) and every fp32 result is divided by it again.
  * Replaces what autograd does for MultiScaleUnet2dDecOnlySmallFixedImpl::forward in the reference
- * (src/lib/models/Networks.h:1139-1191). num_input_channels 1..4, as the forward. Stream-ordered, allocates nothing. */
+ * (src/lib/models/Networks.h:1139-1191). Stream-ordered, allocates nothing. */
 int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUnetWeights* weights,
                         const float* const inputs[TRIPS_UNET_MAX_LEVELS], const void* saved, const float* d_output,
                         float grad_scale, const TripsUnetGrads* grads, void* workspace, size_t workspace_bytes,

@@ -21,9 +21,10 @@ NET_GRAD_TOL = 2e-2
 ADAM_TOL = 2e-6
 
 
-def _make_net(num_input_layers, seed):
+def _make_net(num_input_layers, seed, channels=4, filters=(16, 32, 64, 64)):
     from trips_amd.unet import MultiScaleUnet2dDecOnlySmallFixed, MultiScaleUnet2dParams
-    p = MultiScaleUnet2dParams(num_input_layers=num_input_layers, num_layers=4, filters_network=[16, 32, 64, 64])
+    p = MultiScaleUnet2dParams(num_input_layers=num_input_layers, num_layers=4, num_input_channels=channels,
+                               filters_network=list(filters))
     g = torch.Generator().manual_seed(seed)
     net = MultiScaleUnet2dDecOnlySmallFixed(p).he_normal_(g)
     with torch.no_grad():
@@ -53,17 +54,19 @@ def _oracle_adam(oracle, w, g, lr=1e-3):
     return w, steps
 
 
-def test_config5_chain_small(oracle):
+@pytest.mark.parametrize("channels,filters", [(4, (16, 32, 64, 64)), (8, (32, 48, 64, 64))])
+def test_config5_chain_small(oracle, channels, filters):
     from tests.gpu_util import assert_grads_close
     from tests.ref_unet import unet_forward
     from tests.test_gpu_operator import _info
     from trips_amd.adam import MyAdam
     from trips_amd.renderer import BlendPointCloud, NeuralScene
 
-    sc = scenes.tiny(n=20000, w=160, h=120, f=120.0, num_layers=8, list_depth=16, seed=55, radius=(0.004, 0.3))
+    sc = scenes.tiny(n=20000, w=160, h=120, f=120.0, num_layers=8, list_depth=16, seed=55, radius=(0.004, 0.3),
+                     channels=channels)
     d = abi.desc_for_scene(sc)
     ns = NeuralScene.from_arrays(sc, requires_grad=True)
-    net_cpu = _make_net(8, seed=11)
+    net_cpu = _make_net(8, seed=11, channels=channels, filters=filters)
     net = copy.deepcopy(net_cpu).cuda()
     target = torch.rand((1, 3, sc.height, sc.width), generator=torch.Generator().manual_seed(12))
 

@@ -163,6 +163,11 @@ GRAD_TOL = 2e-2
     ([16, 32, 64, 64], 4, 96, 72, 1, 3),       # 58 outputs below 64 inputs: no spare position
     ([16, 24, 32], 3, 37, 29, 2, 2),
     ([12, 20], 2, 40, 24, 1, 1),
+    # the splat's other descriptor widths: the image then spans up to two groups of eight positions
+    ([24, 32, 64], 3, 70, 50, 1, 6),
+    ([32, 48, 64, 64], 4, 96, 72, 2, 8),
+    ([48, 64, 64], 3, 70, 50, 1, 16),
+    ([40, 56], 2, 37, 29, 1, 12),               # (a width the splat does not have: 24 positions of image)
 ])
 def test_unet_backward_matches_torch_autograd(filters, levels, w, h, batch, cin):
     import copy

@@ -101,10 +101,11 @@ struct FinalBwdParams
 // pixels in registers, a workgroup folds them through LDS and writes its sums once (final_reduce_kernel adds the
 // workgroups up: atomics of a thousand workgroups on these few addresses would serialise in one L2 channel).
 // CS = halves per pixel of the block output.
-template <int CS, bool WGRAD>
+// CI = image channels the kernel has room for (4, 8 or 16).
+template <int CS, bool WGRAD, int CI>
 __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParams p)
 {
-    constexpr int MAXC = 4 + CS;
+    constexpr int MAXC = CI + CS;
     // LPP lanes share a pixel, one per 16 bytes of its pre-activation row (feature groups first, then mask groups),
     // so that a wavefront reads and writes whole lines of the channels-innermost arrays. The feature and the mask
     // lane of a channel group exchange their values with one cross-lane read.
@@ -113,11 +114,11 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
     __shared__ float s_w[4 * MAXC];
     __shared__ float s_sum[4 * MAXC + 4];
     const int cin = p.c_feat + p.cact;
-    // weights as the forward used them (fp16), laid out [k][4 image channels | CS block outputs], zero where unused
+    // weights as the forward used them (fp16), laid out [k][CI image channels | CS block outputs], zero where unused
     for (int i = threadIdx.x; i < 4 * MAXC; i += 256)
     {
         const int k = i / MAXC, r = i - k * MAXC;
-        const int c = r < 4 ? (r < p.c_feat ? r : -1) : (r - 4 < p.cact ? p.c_feat + r - 4 : -1);
+        const int c = r < CI ? (r < p.c_feat ? r : -1) : (r - CI < p.cact ? p.c_feat + r - CI : -1);
         s_w[i]      = (k < p.cout && c >= 0) ? float(_Float16(p.weight[k * cin + c])) : 0.f;
     }
     for (int i = threadIdx.x; i < 4 * MAXC + 4; i += 256) s_sum[i] = 0.f;
@@ -131,17 +132,26 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
     const int ch0      = 8 * (is_f ? g : g - hg);        // first of this lane's 8 channels
     const int partner  = is_f ? lane + hg : lane - hg;   // the lane with the other half of the same channels
     const bool has_act = is_f && ch0 < CS;               // this lane also reads the block output of its channels
-    const bool has_img = g < p.c_feat;                   // ... and image channel g
-    float wj[4][8], wimg[4];
+    // ... and the image channels g, g + LPP, ... (one each for up to LPP image channels)
+    constexpr int NI = (CI + LPP - 1) / LPP;
+    bool has_img[NI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) has_img[j] = g + LPP * j < p.c_feat;
+    float wj[4][8], wimg[4][NI];
 #pragma unroll
     for (int k = 0; k < 4; ++k)
     {
-        wimg[k] = has_img ? s_w[k * MAXC + g] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) wj[k][i] = (in_row && ch0 + i < CS) ? s_w[k * MAXC + 4 + ch0 + i] : 0.f;
+        for (int j = 0; j < NI; ++j) wimg[k][j] = has_img[j] ? s_w[k * MAXC + g + LPP * j] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wj[k][i] = (in_row && ch0 + i < CS) ? s_w[k * MAXC + CI + ch0 + i] : 0.f;
     }
     float acc[4][8];
-    float acc_img[4] = {0.f, 0.f, 0.f, 0.f}, accb[4] = {0.f, 0.f, 0.f, 0.f};
+    float acc_img[4][NI], accb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc_img[k][j] = 0.f;
 #pragma unroll
     for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -149,7 +159,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
 
     struct Loaded
     {
-        float g[4], x;
+        float g[4], x[NI];
         half8 mine;
     };
     auto load = [&](size_t pix, bool valid)
@@ -157,7 +167,8 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
         Loaded l;
 #pragma unroll
         for (int k = 0; k < 4; ++k) l.g[k] = (valid && k < p.cout) ? p.d_out[k * plane + pix] : 0.f;
-        l.x = (WGRAD && valid && has_img) ? p.feat[g * plane + pix] : 0.f;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) l.x[j] = (WGRAD && valid && has_img[j]) ? p.feat[(size_t)(g + LPP * j) * plane + pix] : 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) l.mine[i] = _Float16(0.f);
         if (valid && in_row) l.mine = *reinterpret_cast<const half8*>(p.pre + pix * p.npad + 8 * g);
@@ -196,21 +207,28 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
                 v[i]   = (valid && has_act && ch0 + i < p.cact) ? float(_Float16(a)) : 0.f;
             }
             if (valid && in_row) *reinterpret_cast<half8*>(p.dpre + pix * p.npad + 8 * g) = out;
-            if (valid && has_img)
-            {
-                float d = 0.f;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) d += wimg[k] * cur.g[k];
-                p.d_feat[g * plane + pix] = d;
+            for (int j = 0; j < NI; ++j)
+            {
+                if (valid && has_img[j])
+                {
+                    float d = 0.f;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) d += wimg[k][j] * cur.g[k];
+                    p.d_feat[(size_t)(g + LPP * j) * plane + pix] = d;
+                }
             }
             if (WGRAD)
             {
-                const float xr = float(_Float16(cur.x));
+                float xr[NI];
+#pragma unroll
+                for (int j = 0; j < NI; ++j) xr[j] = float(_Float16(cur.x[j]));
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
                 {
                     accb[k] += cur.g[k];
-                    acc_img[k] += cur.g[k] * xr;
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) acc_img[k][j] += cur.g[k] * xr[j];
 #pragma unroll
                     for (int i = 0; i < 8; ++i) acc[k][i] += cur.g[k] * v[i];
                 }
@@ -231,13 +249,17 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
     {
         const float b = fold(accb[k]);
         if (lane == 0) atomicAdd(&s_sum[4 * MAXC + k], b);
-        const float im = fold(acc_img[k]);
-        if (lane < LPP && has_img) atomicAdd(&s_sum[k * MAXC + g], im);
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+        {
+            const float im = fold(acc_img[k][j]);
+            if (lane < LPP && has_img[j]) atomicAdd(&s_sum[k * MAXC + g + LPP * j], im);
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i)
         {
             const float v = fold(acc[k][i]);
-            if (lane < LPP && has_act && ch0 + i < CS) atomicAdd(&s_sum[k * MAXC + 4 + ch0 + i], v);
+            if (lane < LPP && has_act && ch0 + i < CS) atomicAdd(&s_sum[k * MAXC + CI + ch0 + i], v);
         }
     }
     __syncthreads();
@@ -259,8 +281,8 @@ __device__ __forceinline__ float block_column_sum(const float* __restrict__ part
 }
 
 // d_weight [cout][c_feat + cact] and d_bias [cout] of the 1x1 convolution from final_backward_kernel's partial sums
-// (row layout [k][4 image channels | CS block outputs], then 4 biases); one workgroup per result
-__global__ __launch_bounds__(256) void final_reduce_kernel(const float* __restrict__ part, int rows, int maxc, int c_feat, int cact,
+// (row layout [k][ci image channels | CS block outputs], then 4 biases; maxc = ci + CS); one workgroup per result
+__global__ __launch_bounds__(256) void final_reduce_kernel(const float* __restrict__ part, int rows, int maxc, int ci, int c_feat, int cact,
                                                            int cout, float* __restrict__ d_weight, float* __restrict__ d_bias)
 {
     const int cin = c_feat + cact;
@@ -270,7 +292,7 @@ __global__ __launch_bounds__(256) void final_reduce_kernel(const float* __restri
     if (t < cout * cin)
     {
         const int k = t / cin, c = t - k * cin;
-        col = k * maxc + (c < c_feat ? c : 4 + (c - c_feat));
+        col = k * maxc + (c < c_feat ? c : ci + (c - c_feat));
         dst = d_weight + t;
     }
     else
@@ -294,7 +316,8 @@ struct BwdDataParams
     _Float16* d_in;        // [H][W][NN] or nullptr (start block: nothing below)
 };
 
-template <int KC, int NN, int THREADS>
+// CI = image channels the kernel has room for (4, 8 or 16): positions [0, C) of the block input are the level's image.
+template <int KC, int NN, int THREADS, int CI>
 __global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataParams p)
 {
     constexpr int MB = 16 / (THREADS / 64);  // 16-pixel row blocks of a wavefront: two rows of the tile, or one
@@ -341,7 +364,7 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataPar
     // 16-byte stores, whole lines at a time; the image channels' share kept in fp32 beside it ----
     constexpr int OS   = NN + kLdsChanPad;
     _Float16* s_out    = smem;                                                                   // [256][OS]
-    float* s_img       = reinterpret_cast<float*>(smem + kConvTileH * kConvTileW * OS);          // [4][256]
+    float* s_img       = reinterpret_cast<float*>(smem + kConvTileH * kConvTileW * OS);          // [CI][256]
     __syncthreads();  // every wavefront is done reading the patch
 #pragma unroll
     for (int m = 0; m < MB; ++m)
@@ -353,10 +376,10 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataPar
             const int c0 = 16 * n + (lane >> 4) * 4;  // this lane's four channels
             *reinterpret_cast<half4*>(s_out + tp * OS + c0) =
                 half4{_Float16(acc[m][n][0]), _Float16(acc[m][n][1]), _Float16(acc[m][n][2]), _Float16(acc[m][n][3])};
-            if (n == 0 && c0 == 0)
+            if (n == 0 && c0 < CI)
             {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) s_img[i * (kConvTileH * kConvTileW) + tp] = acc[m][0][i];
+                for (int i = 0; i < 4; ++i) s_img[(c0 + i) * (kConvTileH * kConvTileW) + tp] = acc[m][0][i];
             }
         }
     }
@@ -367,10 +390,12 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataPar
         const int y = y0 + threadIdx.x / kConvTileW, x = x0 + threadIdx.x % kConvTileW;
         if ((int)threadIdx.x < kConvTileH * kConvTileW && y < p.H && x < p.W)
         {
-            float old[4];
-            for (int c = 0; c < p.c_feat; ++c) old[c] = p.d_feat[c * plane + (size_t)y * p.W + x];
-            for (int c = 0; c < p.c_feat; ++c)
-                p.d_feat[c * plane + (size_t)y * p.W + x] = old[c] + s_img[c * (kConvTileH * kConvTileW) + threadIdx.x] * p.scale_inv;
+            float old[CI];
+#pragma unroll
+            for (int c = 0; c < CI; ++c) old[c] = c < p.c_feat ? p.d_feat[c * plane + (size_t)y * p.W + x] : 0.f;
+#pragma unroll
+            for (int c = 0; c < CI; ++c)
+                if (c < p.c_feat) p.d_feat[c * plane + (size_t)y * p.W + x] = old[c] + s_img[c * (kConvTileH * kConvTileW) + threadIdx.x] * p.scale_inv;
         }
     }
 }
@@ -405,20 +430,24 @@ template <int SHIFT>
 __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointParams p)
 {
     const int half   = p.npad / 2;
-    const int groups = 1 + half / 8;  // group 0: the image below; group q: 8 block outputs
+    const int C      = p.c_feat;
+    // the coarser level's image sits at positions [C, 2C) of the finer block's input: the aligned groups of eight
+    // positions g0 .. g0 + ig - 1 (one group up to C = 4 and for C = 8, two for 6 and 16)
+    const int g0 = C / 8, ig = (2 * C - 1) / 8 - g0 + 1;
+    const int groups = ig + half / 8;  // groups 0 .. ig - 1: the image below; then 8 block outputs each
     const size_t pb  = (size_t)p.Hb * p.Wb;
-    const int base8  = (2 * p.c_feat) & ~7;  // aligned position at or before the first block output
+    const int base8  = (2 * C) & ~7;  // aligned position at or before the first block output
     for (size_t item = (size_t)blockIdx.x * 256 + threadIdx.x; item < pb * groups; item += (size_t)gridDim.x * 256)
     {
         const int q     = (int)(item % groups);
         const size_t bp = item / groups;
         const int Y = (int)(bp / p.Wb), X = (int)(bp - (size_t)Y * p.Wb);
         // the pre-activations first: in flight during the gather
-        const int ch0 = 8 * (q - 1);
+        const int ch0 = 8 * (q - ig);
         half8 f8, m8;
 #pragma unroll
         for (int i = 0; i < 8; ++i) f8[i] = m8[i] = _Float16(0.f);
-        if (q > 0)
+        if (q >= ig)
         {
             f8 = *reinterpret_cast<const half8*>(p.pre + bp * p.npad + ch0);
             m8 = *reinterpret_cast<const half8*>(p.pre + bp * p.npad + half + ch0);
@@ -468,18 +497,16 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
         };
         // (one gather for all lanes of a wavefront, whatever their group: lanes of both kinds sit side by side)
         float a[8];
-        gather(q == 0 ? 0 : base8 + ch0, a);
-        if (q == 0)
+        const int first = q < ig ? 8 * (g0 + q) : base8 + ch0;  // first of the eight positions this item gathers
+        gather(first, a);
+        if (q < ig)
         {
             // positions [0, C) are the finer level's own image, [C, 2C) this level's
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
+            for (int i = 0; i < 8; ++i)
             {
-                // (a[c_feat + c] with compile-time indices: a run-time index would put the array into scratch memory)
-                float v = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v = (i == p.c_feat + c) ? a[i] : v;
-                if (c < p.c_feat) p.d_feat[c * pb + bp] = v * p.scale_inv;
+                const int c = first + i - C;  // (a[] only with compile-time indices: else the array goes to scratch memory)
+                if (c >= 0 && c < C) p.d_feat[(size_t)c * pb + bp] = a[i] * p.scale_inv;
             }
         }
         else
@@ -634,9 +661,11 @@ __device__ __forceinline__ void lds_read_pixel_windows(const _Float16* tile, int
 }
 
 // THREADS: 256, or 512 for the largest shape, whose 9 x NPAD x CIN sums are 288 registers per lane of four wavefronts.
-template <int CIN, int NPAD, bool BIAS, int THREADS>
+// CI: image channels the kernel has room for (4, 8 or 16; C <= CI)
+template <int CIN, int NPAD, bool BIAS, int THREADS, int CI>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 32 && NPAD == 32 ? 4 : 1))) void conv_bwd_weight_kernel(const BwdWeightParams p)
 {
+    constexpr int IQ = CI / 4;  // 16-byte items that carry the image of a pixel of the level below
     constexpr int ROW    = CIN + kLdsChanPad;   // halves per pixel of the input patch
     constexpr int DS     = NPAD + kLdsChanPad;  // halves per pixel of the gradient tile
     constexpr int GROUPS = CIN / 8;
@@ -690,18 +719,18 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
     // flight together), and written to LDS one tile later, so that the loads of tile t + 1 travel while tile t is
     // upsampled and multiplied ----
     constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + THREADS - 1) / THREADS;
-    constexpr int kMaxPerPix  = 1 + CIN / 8;  // image below + groups of 8 block outputs
+    constexpr int kMaxPerPix  = IQ + CIN / 8;  // image below (four channels per item) + groups of 8 block outputs
     constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + THREADS - 1) / THREADS;
     constexpr int kDpreGroups = NPAD / 8;  // 16-byte groups of a pixel's gradient row
     constexpr int kDpreItems  = (kConvTileH * kConvTileW * kDpreGroups + THREADS - 1) / THREADS;
     struct TileLoads
     {
-        float feat[kFeatItems][4];
+        float feat[kFeatItems][CI];
         uint4 below[kBelowItems];
         half8 dpre[kDpreItems];
     };
     const int act_groups = p.cb_store / 8;
-    const int per_pixel  = 1 + act_groups;
+    const int per_pixel  = IQ + act_groups;
     auto issue_loads = [&](int tile, TileLoads& r)
     {
         const int ty = tile / p.tiles_x, tx = tile - ty * p.tiles_x;
@@ -716,7 +745,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
             const int y = y0 + py - 1, x = x0 + px - 1;
             const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) r.feat[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+            for (int c = 0; c < CI; ++c) r.feat[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
         }
         if (has_below)
         {
@@ -731,15 +760,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                     const int q = item % per_pixel, bp = item / per_pixel;
                     const int rr = bp / kBelowW, c0 = bp - rr * kBelowW;
                     const int yy = min(max(by0 + rr, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
-                    if (q == 0)
+                    if (q < IQ)
                     {
                         float f[4];
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) f[c] = c < C ? p.feat_below[c * pb + (size_t)yy * p.Wb + xx] : 0.f;
+                        for (int c = 0; c < 4; ++c) f[c] = 4 * q + c < C ? p.feat_below[(size_t)(4 * q + c) * pb + (size_t)yy * p.Wb + xx] : 0.f;
                         r.below[k] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
                     }
                     else
-                        r.below[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1));
+                        r.below[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - IQ));
                 }
             }
         }
@@ -757,39 +786,50 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
     };
     // this level's image into channels [0, C) of a patch pixel (the channels [C, 8) follow from the upsampling, or are
     // zero for the start block, whose other channels are cleared once, below)
-    auto put_image = [&](int item, const float (&v)[4])
+    auto put_image = [&](int item, const float (&v)[CI])
     {
         _Float16* row = s_patch + (size_t)item * ROW;
-        if (has_below && C == 4)
+        if (CI == 4 && has_below && C == 4)
             *reinterpret_cast<half4*>(row) = half4{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3])};
         else if (has_below)
         {
 #pragma unroll
-            for (int c = 0; c < 4; ++c)  // a run-time bound would put the register array into scratch memory
+            for (int c = 0; c < CI; ++c)  // a run-time bound would put the register array into scratch memory
                 if (c < C) row[c] = _Float16(v[c]);
         }
         else
-            *reinterpret_cast<half8*>(row) = half8{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3]),
-                                                   _Float16(0.f), _Float16(0.f), _Float16(0.f), _Float16(0.f)};
+        {
+            // start block: the image is the whole input; the first groups of eight written whole (v is zero past C)
+#pragma unroll
+            for (int g8 = 0; g8 < (CI + 7) / 8; ++g8)
+            {
+                half8 h;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = 8 * g8 + i < CI ? _Float16(v[8 * g8 + i < CI ? 8 * g8 + i : 0]) : _Float16(0.f);
+                *reinterpret_cast<half8*>(row + 8 * g8) = h;
+            }
+        }
     };
-    auto put_below_image = [&](int bp, const float (&v)[4])
+    // four channels 4 qi .. 4 qi + 3 of the image of the level below into positions C + 4 qi .. of a below-patch pixel
+    auto put_below_image = [&](int bp, int qi, const float (&v)[4])
     {
         _Float16* row = s_below + (size_t)bp * ROW;
-        if (C == 4)
+        if (CI == 4 && C == 4)
             *reinterpret_cast<half4*>(row + 4) = half4{_Float16(v[0]), _Float16(v[1]), _Float16(v[2]), _Float16(v[3])};
         else
         {
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                if (c < C) row[C + c] = _Float16(v[c]);
+                if (4 * qi + c < C) row[C + 4 * qi + c] = _Float16(v[c]);
         }
-        for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
+        if (qi == 0)
+            for (int c = 2 * C + p.cb_store; c < CIN; ++c) row[c] = _Float16(0.f);
     };
-    // eight block outputs of the level below (group q >= 1) into positions 2 C + 8 (q - 1) .. of a below-patch pixel
+    // eight block outputs of the level below (item q >= IQ) into positions 2 C + 8 (q - IQ) .. of a below-patch pixel
     auto put_below_act = [&](int bp, int q, const uint4& v)
     {
         _Float16* row = s_below + (size_t)bp * ROW;
-        const int pos = 2 * C + 8 * (q - 1);
+        const int pos = 2 * C + 8 * (q - IQ);
         if (C == 4)
             *reinterpret_cast<uint4*>(row + pos) = v;
         else
@@ -818,11 +858,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                 if (item < kBelowH * kBelowW * per_pixel)
                 {
                     const int q = item % per_pixel, bp = item / per_pixel;
-                    if (q == 0)
+                    if (q < IQ)
                     {
                         const float f[4] = {__uint_as_float(r.below[k].x), __uint_as_float(r.below[k].y), __uint_as_float(r.below[k].z),
                                             __uint_as_float(r.below[k].w)};
-                        put_below_image(bp, f);
+                        put_below_image(bp, q, f);
                     }
                     else
                         put_below_act(bp, q, r.below[k]);
@@ -848,9 +888,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                 const int py = item / kConvPatchW, px = item - py * kConvPatchW;
                 const int y = y0 + py - 1, x = x0 + px - 1;
                 const bool in = y >= 0 && y < p.H && x >= 0 && x < p.W;
-                float v[4];
+                float v[CI];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) v[c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+                for (int c = 0; c < CI; ++c) v[c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
                 put_image(item, v);
             }
         }
@@ -862,16 +902,16 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                 const int q = item % per_pixel, bp = item / per_pixel;
                 const int r = bp / kBelowW, c0 = bp - r * kBelowW;
                 const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
-                if (q == 0)
+                if (q < IQ)
                 {
                     float v[4];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) v[c] = c < C ? p.feat_below[c * pb + (size_t)yy * p.Wb + xx] : 0.f;
-                    put_below_image(bp, v);
+                    for (int c = 0; c < 4; ++c) v[c] = 4 * q + c < C ? p.feat_below[(size_t)(4 * q + c) * pb + (size_t)yy * p.Wb + xx] : 0.f;
+                    put_below_image(bp, q, v);
                 }
                 else
                 {
-                    put_below_act(bp, q, *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - 1)));
+                    put_below_act(bp, q, *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - IQ)));
                 }
             }
         }
@@ -887,14 +927,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
         }
     };
 
-    // start block: the channels beyond the first eight of a patch pixel are never written and stay zero
+    // start block: the channels beyond the image's groups of eight of a patch pixel are never written and stay zero
+    constexpr int kImageGroups = (CI + 7) / 8;
     if (!has_below)
-        for (int i = threadIdx.x; i < kConvPatchH * kConvPatchW * (GROUPS - 1); i += THREADS)
+        for (int i = threadIdx.x; i < kConvPatchH * kConvPatchW * (GROUPS - kImageGroups); i += THREADS)
         {
             half8 z;
 #pragma unroll
             for (int k = 0; k < 8; ++k) z[k] = _Float16(0.f);
-            *reinterpret_cast<half8*>(s_patch + (size_t)(i / (GROUPS - 1)) * ROW + 8 * (1 + i % (GROUPS - 1))) = z;
+            *reinterpret_cast<half8*>(s_patch + (size_t)(i / (GROUPS - kImageGroups)) * ROW + 8 * (kImageGroups + i % (GROUPS - kImageGroups))) = z;
         }
 
     // with 64 input channels and more than 64 pre-activations the accumulators leave no registers for a tile in flight
@@ -942,13 +983,17 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(CIN == 
                     h = __builtin_elementwise_fma(d, W11, __builtin_elementwise_fma(c, W10, __builtin_elementwise_fma(b, W01, a * W00)));
                 }
                 _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
-                if (g == 0)
+                if (8 * g < C)
                 {
                     // [0, C) holds this level's image
-                    if (C == 4)
+                    if (CI == 4 && C == 4)
                         *reinterpret_cast<half4*>(dst + 4) = half4{h[4], h[5], h[6], h[7]};
                     else
-                        for (int i = C; i < 8; ++i) dst[i] = h[i];
+                    {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            if (8 * g + i >= C) dst[i] = h[i];
+                    }
                 }
                 else
                     *reinterpret_cast<half8*>(dst) = h;
@@ -1120,56 +1165,66 @@ __global__ __launch_bounds__(256) void reduce_weight_grad_kernel(const ReduceTab
 // ---------------------------------------------------------------------------------------------------------
 namespace
 {
-template <int KC, int NN>
+template <int KC, int NN, int CI>
 hipError_t launch_bwd_data(const BwdDataParams& p, hipStream_t stream)
 {
     // the patch and two tap buffers of the weights: up to 92 + 35 KB
     const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW + 2 * NN) * (KC + kLdsChanPad) * sizeof(_Float16);
-    const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NN + kLdsChanPad) * sizeof(_Float16) + 4 * sizeof(float));
+    const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NN + kLdsChanPad) * sizeof(_Float16) + CI * sizeof(float));
     const size_t lds     = std::max(lds_in, lds_out);
     constexpr int THREADS = 512;  // eight wavefronts per tile, as in the forward convolution
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN, THREADS>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_data_kernel<KC, NN, THREADS, CI>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     dim3 grid((p.W + kConvTileW - 1) / kConvTileW, (p.H + kConvTileH - 1) / kConvTileH);
-    hipLaunchKernelGGL((conv_bwd_data_kernel<KC, NN, THREADS>), grid, dim3(THREADS), lds, stream, p);
+    hipLaunchKernelGGL((conv_bwd_data_kernel<KC, NN, THREADS, CI>), grid, dim3(THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
 hipError_t dispatch_bwd_data(const BwdDataParams& p, int npad, int cin_pad, hipStream_t stream)
 {
-#define TRIPS_BD(KC_, NN_) \
-    if (npad == KC_ && cin_pad == NN_) return launch_bwd_data<KC_, NN_>(p, stream);
+#define TRIPS_BD(KC_, NN_)                                                                   \
+    if (npad == KC_ && cin_pad == NN_)                                                       \
+        return p.c_feat <= 4 ? launch_bwd_data<KC_, NN_, 4>(p, stream)                       \
+                             : p.c_feat <= 8 ? launch_bwd_data<KC_, NN_, 8>(p, stream) : launch_bwd_data<KC_, NN_, 16>(p, stream);
     TRIPS_BD(32, 32) TRIPS_BD(64, 32) TRIPS_BD(96, 32) TRIPS_BD(128, 32)
     TRIPS_BD(32, 64) TRIPS_BD(64, 64) TRIPS_BD(96, 64) TRIPS_BD(128, 64)
 #undef TRIPS_BD
     return hipErrorInvalidValue;
 }
 
-template <int CIN, int NPAD, bool BIAS>
+template <int CIN, int NPAD, bool BIAS, int CI>
 hipError_t launch_bwd_weight(const BwdWeightParams& p, int groups, hipStream_t stream)
 {
     constexpr int THREADS = wgrad_threads(CIN, NPAD);
     const size_t lds = ((size_t)(kConvPatchH * kConvPatchW + kBelowH * kBelowW) * (CIN + kLdsChanPad) +
                         (size_t)kConvTileH * kConvTileW * (NPAD + kLdsChanPad)) *
                        sizeof(_Float16);  // up to 133 KB
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD, BIAS, THREADS>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bwd_weight_kernel<CIN, NPAD, BIAS, THREADS, CI>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD, BIAS, THREADS>), dim3(groups), dim3(THREADS), lds, stream, p);
+    hipLaunchKernelGGL((conv_bwd_weight_kernel<CIN, NPAD, BIAS, THREADS, CI>), dim3(groups), dim3(THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
-hipError_t dispatch_bwd_weight(const BwdWeightParams& p, int cin_pad, int npad, int groups, hipStream_t stream)
+template <int CI>
+hipError_t dispatch_bwd_weight_ci(const BwdWeightParams& p, int cin_pad, int npad, int groups, hipStream_t stream)
 {
 #define TRIPS_BW(CIN_, NPAD_)                                                                  \
     if (cin_pad == CIN_ && npad == NPAD_)                                                      \
-        return p.bias_part ? launch_bwd_weight<CIN_, NPAD_, true>(p, groups, stream) \
-                                          : launch_bwd_weight<CIN_, NPAD_, false>(p, groups, stream);
+        return p.bias_part ? launch_bwd_weight<CIN_, NPAD_, true, CI>(p, groups, stream) \
+                                          : launch_bwd_weight<CIN_, NPAD_, false, CI>(p, groups, stream);
     TRIPS_BW(32, 32) TRIPS_BW(32, 64) TRIPS_BW(32, 96) TRIPS_BW(32, 128)
     TRIPS_BW(64, 32) TRIPS_BW(64, 64) TRIPS_BW(64, 96) TRIPS_BW(64, 128)
 #undef TRIPS_BW
     return hipErrorInvalidValue;
+}
+
+hipError_t dispatch_bwd_weight(const BwdWeightParams& p, int cin_pad, int npad, int groups, hipStream_t stream)
+{
+    if (p.c_feat <= 4) return dispatch_bwd_weight_ci<4>(p, cin_pad, npad, groups, stream);
+    if (p.c_feat <= 8) return dispatch_bwd_weight_ci<8>(p, cin_pad, npad, groups, stream);
+    return dispatch_bwd_weight_ci<16>(p, cin_pad, npad, groups, stream);
 }
 }  // namespace
 }  // namespace trips
@@ -1196,7 +1251,6 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
     if (!weights || !inputs || !saved || !d_output || !grads || !workspace) return set_error(TRIPS_ERR_INVALID_ARG, "NULL argument");
     const TripsUnetDesc& d = *desc;
     const int C = d.num_input_channels, L = d.num_levels;
-    if (C > 4) return set_error(TRIPS_ERR_UNSUPPORTED, "the backward is built for num_input_channels 1..4 (got %d)", C);
     if (!(grad_scale > 0.f) || !std::isfinite(grad_scale)) return set_error(TRIPS_ERR_INVALID_ARG, "grad_scale must be positive");
     for (int i = 0; i < L; ++i)
     {
@@ -1217,6 +1271,7 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
     Profiler* prof     = ctx->prof.enabled ? &ctx->prof : nullptr;
     const float scale_inv = 1.f / grad_scale;
     const int K           = d.num_output_channels;
+    const int ci          = C <= 4 ? 4 : C <= 8 ? 8 : 16;  // image channels the kernels are built with room for
 
     auto act_ptr = [&](int level, int b)
     {
@@ -1282,27 +1337,41 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
             p.d_feat   = grads->inputs[0] + (size_t)b * C * plane;
             p.dpre     = dpre_ptr(0, b);
             p.chunks   = (int)((plane + kFinalPixelsPerBlock - 1) / kFinalPixelsPerBlock);
-            p.part     = reinterpret_cast<float*>(ws + np.final_part_off) + (size_t)b * np.final_groups * (4 * (4 + lv.cout_store) + 4);
+            p.part     = reinterpret_cast<float*>(ws + np.final_part_off) + (size_t)b * np.final_groups * (4 * (ci + lv.cout_store) + 4);
             const bool wgrad = grads->final_weight || grads->final_bias;
             const int chunks = wgrad ? np.final_groups : p.chunks;
             switch (lv.cout_store)
             {
-#define TRIPS_FW(CS_)                                                                                         \
-    case CS_:                                                                                                 \
-        if (wgrad)                                                                                            \
-            hipLaunchKernelGGL((final_backward_kernel<CS_, true>), dim3(chunks), dim3(256), 0, stream, p);    \
-        else                                                                                                  \
-            hipLaunchKernelGGL((final_backward_kernel<CS_, false>), dim3(chunks), dim3(256), 0, stream, p);   \
+#define TRIPS_FW_CI(CS_, CI_)                                                                                     \
+    if (wgrad)                                                                                                    \
+        hipLaunchKernelGGL((final_backward_kernel<CS_, true, CI_>), dim3(chunks), dim3(256), 0, stream, p);       \
+    else                                                                                                          \
+        hipLaunchKernelGGL((final_backward_kernel<CS_, false, CI_>), dim3(chunks), dim3(256), 0, stream, p);
+#define TRIPS_FW(CS_)                \
+    case CS_:                        \
+        if (ci == 4)                 \
+        {                            \
+            TRIPS_FW_CI(CS_, 4)      \
+        }                            \
+        else if (ci == 8)            \
+        {                            \
+            TRIPS_FW_CI(CS_, 8)      \
+        }                            \
+        else                         \
+        {                            \
+            TRIPS_FW_CI(CS_, 16)     \
+        }                            \
         break;
                 TRIPS_FW(8) TRIPS_FW(16) TRIPS_FW(24) TRIPS_FW(32) TRIPS_FW(40) TRIPS_FW(48) TRIPS_FW(56) TRIPS_FW(64)
 #undef TRIPS_FW
+#undef TRIPS_FW_CI
                 default: return set_error(TRIPS_ERR_UNSUPPORTED, "block output stride %d", lv.cout_store);
             }
         }
         if (grads->final_weight || grads->final_bias)
         {
             hipLaunchKernelGGL(final_reduce_kernel, dim3(K * (C + lv.cout) + K), dim3(256), 0, stream,
-                               reinterpret_cast<const float*>(ws + np.final_part_off), d.batch * np.final_groups, 4 + lv.cout_store, C,
+                               reinterpret_cast<const float*>(ws + np.final_part_off), d.batch * np.final_groups, ci + lv.cout_store, ci, C,
                                lv.cout, K, grads->final_weight, grads->final_bias);
         }
     }
@@ -1382,7 +1451,7 @@ int trips_unet_backward(TripsCtx* ctx, const TripsUnetDesc* desc, const TripsUne
                     up.pre       = pre_ptr(i + 1, b);
                     up.d_feat    = grads->inputs[i + 1] + (size_t)b * C * lb.H * lb.W;
                     up.dpre      = dpre_ptr(i + 1, b);
-                    const size_t items = (size_t)lb.H * lb.W * (1 + lb.npad / 16);
+                    const size_t items = (size_t)lb.H * lb.W * ((2 * C - 1) / 8 - C / 8 + 1 + lb.npad / 16);
                     const int blocks   = (int)std::min<size_t>((items + 255) / 256, 1u << 20);
                     switch ((2 * C) & 7)
                     {
