@@ -29,11 +29,26 @@ struct AdamScalars
     float lr, beta1, beta2, eps, rel_wd, abs_wd, clip, lo, hi, loss_scale;
 };
 
+// beta^t for a step count t: by squaring in double precision, rounded to float once. (The library powf is some 400
+// instructions, and two of them per point were half of the packed kernel's work. The squarings' error doubles per
+// squaring from 2^-53: below a float's for any t < 2^28, and beta^t of a beta < 1 is zero long before that.)
+__device__ __forceinline__ float pow_step(float beta, uint32_t t)
+{
+    double r = 1.0, b = (double)beta;
+    while (t)
+    {
+        if (t & 1u) r *= b;
+        b *= b;
+        t >>= 1;
+    }
+    return (float)r;
+}
+
 // learning rate with the bias correction of step `current_step` (MyAdam.cu:66-68)
 __device__ __forceinline__ float adam_corrected_lr(const AdamScalars& h, uint32_t current_step)
 {
     float learning_rate = h.lr;
-    learning_rate *= sqrtf(1 - powf(h.beta2, (float)current_step)) / (1 - powf(h.beta1, (float)current_step));
+    learning_rate *= sqrtf(1 - pow_step(h.beta2, current_step)) / (1 - pow_step(h.beta1, current_step));
     return learning_rate;
 }
 
