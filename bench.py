@@ -31,18 +31,18 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "0262f38ac2fe1907fde5da1bf2956b9f3ee31bd250d6a742519c11a75c3e3fc4"
+PMC_SOURCES_SHA256 = "125852cb436ca51971bf9050f399f94a43c5176b526fae49c1f0fbb8c58a82dc"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129116, 251278),
-    "bin_scatter": (95990, 166508),
-    "tile_count": (13141, 2296),
-    "tile_scatter": (32593, 110316),
-    "cell_sort": (35543, 42964),
-    "blend": (318216, 196234),
-    "backward_prologue": (55, 265145),
-    "backward_tiles": (425952, 121583),
-    "backward_points": (297269, 234503),
-    "adam_fused": (383877, 498420),
+    "project_bin": (129116, 254462),
+    "bin_scatter": (95982, 166664),
+    "tile_count": (13142, 2296),
+    "tile_scatter": (32801, 110488),
+    "cell_sort": (35541, 42963),
+    "blend": (319622, 195756),
+    "backward_prologue": (50, 265182),
+    "backward_tiles": (425515, 121577),
+    "backward_points": (297114, 234503),
+    "adam_fused": (383789, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
                         "splat_internal.h", "trips_math.h", "row16.h")
