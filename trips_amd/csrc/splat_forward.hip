@@ -208,7 +208,6 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
     constexpr int WAVES = kBinThreads / 64;
     extern __shared__ int s_hist[];  // bin entries of this workgroup's points, one counter per tile
     __shared__ int s_valid[2][WAVES];  // valid points of every wavefront in this step (two steps in flight)
-    __shared__ int s_pairs[2][WAVES];  // overflow rows (layers past the second) of every wavefront's points in this step
     __shared__ int s_flags;            // bit 0: not_identity, bit 1: bad_index, of any point of the chunk
     const Camera cam  = load_camera(p.pose, p.intrinsics, p.view, p.dist_cutoff);
     const int L       = p.num_layers;
@@ -266,18 +265,22 @@ __global__ __launch_bounds__(kBinThreads) void project_bin_kernel(const ForwardP
                 pairs_wave += (int)__popcll(m) << b;
             }
         }
-        if (lane == 0) s_valid[step][wave] = (int)__popcll(vm), s_pairs[step][wave] = pairs_wave;
+        // both counts of a wavefront in one word (at most 64 valid points and 384 rows per wavefront, 1024 and 6144 per
+        // step: 16 bits each); every wavefront then takes the prefix over the 16 words in its first 16 lanes
+        if (lane == 0) s_valid[step][wave] = (int)__popcll(vm) | (pairs_wave << 16);
         __syncthreads();
-        int before = 0, total = 0, pbefore = 0, ptotal = 0;
+        static_assert(WAVES == 16, "the prefix below runs over one 16-lane row");
+        const int word = lane < WAVES ? s_valid[step][lane] : 0;  // the counts of wavefront w in lane w
+        int inc        = word;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w)
+        for (int o = 1; o < WAVES; o <<= 1)
         {
-            const int c = s_valid[step][w], q = s_pairs[step][w];
-            before += w < wave ? c : 0;
-            total += c;
-            pbefore += w < wave ? q : 0;
-            ptotal += q;
+            const int t = __shfl_up(inc, o);
+            if (lane >= o) inc += t;
         }
+        const int upto = __shfl(inc, WAVES - 1);     // the step's totals
+        const int excl = __shfl(inc - word, wave);   // the wavefronts before this one
+        const int before = excl & 0xFFFF, pbefore = excl >> 16, total = upto & 0xFFFF, ptotal = upto >> 16;
         const int cid        = next + before + (int)__popcll(vm & below);
         const int first_pair = next_pair + pbefore + pairs_before;  // within the chunk; the scatter pass adds the chunk's first
         next += total;
