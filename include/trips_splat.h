@@ -256,6 +256,13 @@ int trips_profile_enable(TripsCtx* ctx, int enabled);
 int trips_profile_read(TripsCtx* ctx, int* n, const char* names[TRIPS_PROFILE_MAX_KERNELS],
                        float ms[TRIPS_PROFILE_MAX_KERNELS], int launches[TRIPS_PROFILE_MAX_KERNELS]);
 
+/* ---- a knob for tests (no counterpart in the reference) ----
+ * The backward keeps the (point, layer) rows between its two passes in one of two forms and chooses per view on the
+ * device: rows of all pairs cleared beforehand, or a flag byte per row for views in which few pairs are retained by a
+ * pixel. Both give the same gradients bit for bit. mode: 0 = choose per view (default), 1 = always the first form,
+ * 2 = always the second. Applies to the backward calls made through `ctx` from then on. */
+int trips_splat_pair_rows_mode(TripsCtx* ctx, int mode);
+
 #ifdef __cplusplus
 }
 #endif

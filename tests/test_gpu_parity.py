@@ -202,6 +202,44 @@ def test_backward_small(oracle, L, K, bg):
     assert np.abs(g["d_pose"]).max() > 0 and np.abs(g["d_intrinsics"]).max() > 0
 
 
+@pytest.mark.parametrize("scene", ["ordinary", "tight_cluster", "many_layers_two_views"])
+def test_backward_pair_row_forms_agree(oracle, scene):
+    """Between its two passes the backward keeps a row per (point, layer) pair, either all rows cleared beforehand or a
+    flag byte per row (chosen per view on the device from the share of retained entries). Forced either way and left
+    to choose, the gradients are the same bits, and they are the oracle's."""
+    from tests.gpu_util import GpuRun, assert_grads_close
+    if scene == "ordinary":
+        sc = scenes.tiny(n=6000, w=90, h=70, f=70.0, num_layers=4, list_depth=16, seed=301, radius=(0.004, 0.3))
+    elif scene == "tight_cluster":
+        sc = scenes.tiny(n=20000, w=96, h=64, f=80.0, num_layers=4, list_depth=16, seed=302, radius=(0.004, 0.2))
+        rng = np.random.default_rng(5)
+        sc.position[:, :3] = (rng.normal(0, 0.01, (20000, 3)) + np.array([0.05, -0.02, 0.0])).astype(np.float32)
+    else:
+        sc = scenes.tiny(n=3000, w=128, h=96, f=110.0, num_layers=8, list_depth=16, seed=303, views=2, radius=(0.05, 0.6))
+    d = abi.desc_for_scene(sc)
+    ref = oracle.forward(sc, d)
+    rng = np.random.default_rng(9)
+    grads = [rng.normal(0, 1, (d.num_views, d.num_channels, h, w)).astype(np.float32) for (w, h) in ref["sizes"]]
+    g_ref = oracle.backward(sc, d, ref, grads)
+    run = GpuRun(sc, d)
+    run.forward()
+    got = {}
+    try:
+        for mode in (1, 2, 0):
+            run.ctx.pair_rows_mode(mode)
+            got[mode] = {k: np.array(v, copy=True) for k, v in run.backward(grads).items()}
+    finally:
+        run.ctx.pair_rows_mode(0)
+    assert_grads_close(got[1], g_ref)
+    from tests.gpu_util import rel_err
+    for k in got[1]:
+        if k in ("d_texture", "d_confidence", "d_position", "d_point_size"):
+            np.testing.assert_array_equal(got[2][k], got[1][k], err_msg=f"{k}: flagged rows against rows of all pairs")
+            np.testing.assert_array_equal(got[0][k], got[1][k], err_msg=f"{k}: the device's own choice")
+        else:  # sums over workgroups, added with atomics: the same terms in an order that varies from launch to launch
+            assert rel_err(got[2][k], got[1][k]) < 1e-6 and rel_err(got[0][k], got[1][k]) < 1e-6, k
+
+
 @pytest.mark.parametrize("channels", [4, 16])
 def test_backward_points_written_to_many_layers(oracle, channels):
     """Every point is large enough for four to eight layers: a wavefront of the point pass then has several hundred

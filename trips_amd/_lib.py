@@ -17,6 +17,7 @@ SYMBOLS = [
     "trips_splat_backward",
     "trips_splat_check", "trips_splat_check_static", "trips_splat_counters", "trips_splat_export_lists", "trips_splat_export_points",
     "trips_adam_step_fused", "trips_adam_points_state_size", "trips_adam_step_points", "trips_apply_tangent", "trips_profile_enable", "trips_profile_read",
+    "trips_splat_pair_rows_mode",
 ]
 # every symbol include/trips_unet.h declares
 UNET_SYMBOLS = ["trips_unet_workspace_size", "trips_unet_saved_size", "trips_unet_backward_workspace_size",
@@ -74,6 +75,7 @@ def load():
                                         C.POINTER(vp), vp, vp, C.c_float, C.POINTER(abi.TripsUnetGrads), vp,
                                         C.c_size_t, vp]
     lib.trips_profile_enable.argtypes = [vp, i32]
+    lib.trips_splat_pair_rows_mode.argtypes = [vp, i32]
     lib.trips_profile_read.argtypes = [vp, C.POINTER(i32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
                                        C.POINTER(i32)]
     for name in SYMBOLS:

@@ -791,7 +791,7 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
 // (background, every pose row, every intrinsics row).
 __global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader* __restrict__ header, const int32_t* __restrict__ chunk_valid,
                                                                 int bin_groups, int points_per_block, float* __restrict__ rows_inline,
-                                                                float* __restrict__ rows_over, unsigned char* __restrict__ flags, int32_t* __restrict__ mode, int pair_row, long long over_capacity,
+                                                                float* __restrict__ rows_over, unsigned char* __restrict__ flags, int32_t* __restrict__ mode, int force_mode, int pair_row, long long over_capacity,
                                                                 float* __restrict__ d_texture,
                                                                 float* __restrict__ d_confidence, int channels, int num_texels,
                                                                 int num_points, int texels, int clear_sums,
@@ -808,7 +808,8 @@ __global__ __launch_bounds__(256) void backward_prologue_kernel(const ViewHeader
         if ((threadIdx.x & 63) == 0) s_retained[threadIdx.x >> 6] = r;
         __syncthreads();
     }
-    const bool sparse = sparse_pair_rows((s_retained[0] + s_retained[1] + s_retained[2] + s_retained[3]) * kRetainedSample, header->n_entries);
+    const bool sparse = force_mode == 0 ? sparse_pair_rows((s_retained[0] + s_retained[1] + s_retained[2] + s_retained[3]) * kRetainedSample, header->n_entries)
+                                        : force_mode == 2;
     if (blockIdx.x == 0 && threadIdx.x == 0) *mode = sparse ? 1 : 0;
     if (sparse)
     {
@@ -882,7 +883,7 @@ hipError_t launch_backward_view(const BackwardParams& p, int channels, hipStream
     {
         ProfScope ps(prof, "backward_prologue", stream);
         hipLaunchKernelGGL(backward_prologue_kernel, dim3(2048), dim3(256), 0, stream, p.header, p.chunk_valid, p.bin_groups,
-                           p.points_per_block, p.rows_inline, p.rows_over, p.flags, p.mode, pair_row_floats((channels + 3) & ~3),
+                           p.points_per_block, p.rows_inline, p.rows_over, p.flags, p.mode, p.force_mode, pair_row_floats((channels + 3) & ~3),
                            p.over_capacity, p.d_texture, p.d_confidence, channels, p.num_texels,
                            N, p.overwrite, p.clear_block_sums, p.d_background, p.d_pose_all, p.num_images, p.d_intrinsics_all,
                            p.num_cameras);

@@ -85,6 +85,7 @@ struct TripsCtx
     // this device's copy of the library's static scratch array (trips_splat_forward_static), resolved when the
     // context is created
     void* static_scratch = nullptr;
+    int pair_rows_mode = 0;  // trips_splat_pair_rows_mode: 0 = the backward chooses per view
 };
 
 namespace trips
@@ -393,6 +394,7 @@ struct BackwardParams
     const int32_t* over_first;   // [N] (saved state) by compact number
     const int32_t* chunk_valid;  // [kBinGroups + kRetainedParts] (saved state)
     int32_t* mode;               // (workspace) 1 = only flagged rows exist
+    int32_t force_mode;          // 0 = chosen per view from the retained entries, 1 = rows of all pairs, 2 = flagged rows
     int32_t bin_groups, points_per_block;
     float* rows_inline;  // [N, kInlineLayers, pair_row_floats] (workspace)
     float* rows_over;    // [over_capacity, pair_row_floats] (workspace)

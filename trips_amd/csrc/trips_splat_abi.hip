@@ -577,6 +577,7 @@ int trips_splat_backward(TripsCtx* ctx, const TripsSplatDesc* desc, const TripsS
         p.rows_over    = reinterpret_cast<float*>(ws + bl.rows_over);
         p.flags        = reinterpret_cast<unsigned char*>(ws + bl.flags);
         p.mode         = reinterpret_cast<int32_t*>(ws + bl.mode);
+        p.force_mode   = ctx->pair_rows_mode;
         p.over_capacity = (long long)bl.over_capacity;
         p.blocks_off[0] = 0;
         for (int l = 0; l < TRIPS_MAX_LAYERS; ++l)
@@ -774,6 +775,14 @@ int trips_apply_tangent(TripsCtx* ctx, double* tangent, double* poses_se3, int n
     if (n < 0 || (n > 0 && (!tangent || !poses_se3))) return fail(TRIPS_ERR_INVALID_ARG, "tangent / poses_se3");
     hipError_t e = launch_apply_tangent(tangent, poses_se3, n, reinterpret_cast<hipStream_t>(stream_));
     if (e != hipSuccess) return hip_fail(e, "apply_tangent launch");
+    return TRIPS_OK;
+}
+
+int trips_splat_pair_rows_mode(TripsCtx* ctx, int mode)
+{
+    if (!ctx) return fail(TRIPS_ERR_INVALID_ARG, "ctx is NULL");
+    if (mode < 0 || mode > 2) return fail(TRIPS_ERR_INVALID_ARG, "mode must be 0, 1 or 2");
+    ctx->pair_rows_mode = mode;
     return TRIPS_OK;
 }
 

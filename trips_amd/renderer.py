@@ -164,6 +164,11 @@ class SplatContext:
                                                       _stream_ptr(self.device)))
         return ip, depth, size_px, max_layer
 
+    def pair_rows_mode(self, mode):
+        """For tests: 0 = the backward chooses per view how it keeps its (point, layer) rows, 1 = rows of all pairs
+        cleared beforehand, 2 = a flag byte per row. Same gradients either way."""
+        _lib.check(self.lib.trips_splat_pair_rows_mode(self.ctx, int(mode)))
+
     # ---- per-kernel timing ----
     def profile_enable(self, on=True):
         _lib.check(self.lib.trips_profile_enable(self.ctx, int(bool(on))))
