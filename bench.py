@@ -101,7 +101,7 @@ def algorithmic_bytes(c, n_points, channels=4, adam_nonzero=0, adam_zero=0, adam
         "sort_blend": 8 * E + (20 + 4 + 4 * C + 28) * R + 4 * C * P,  # keys read, record+conf+descriptor, saved, image
         # the backward's bytes split as its two passes split the work: the compositing (tile pass) reads dL/dimage, the
         # saved entry, descriptor and confidence; the geometry (point pass) reads position + size again (20 B per entry)
-        # and makes the one write per accumulated gradient float. (The prologue that clears the exchange rows has no
+        # and makes the one write per accumulated gradient float. (The prologue that clears the pair rows has no
         # algorithmic bytes: its time counts, its bytes do not.)
         "backward_tiles": 4 * C * P + (28 + 4 * C + 4) * R,
         "backward_points": (20 + 4 * C + 4 + 12 + 4) * R,

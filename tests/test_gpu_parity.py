@@ -138,8 +138,8 @@ def test_medium_views_other_channel_counts(oracle, channels, K, layout, views):
 
 @pytest.mark.parametrize("order", ["random", "by_screen_tile"])
 def test_medium_view_memory_order_of_the_points(oracle, order):
-    """The backward lays its exchange rows out differently for clouds whose memory order is coherent on the screen
-    (neighbouring points in the same tile) and for randomly ordered ones: the same view with the points in both orders."""
+    """The same view with its points in random order and sorted by screen tile (neighbouring points in the same tile:
+    neighbouring lanes of the point pass then share their rows' lines, and the chunks' compact numbers follow the screen)."""
     sc = scenes.tiny(n=200_000, w=640, h=480, f=520.0, num_layers=6, list_depth=16, seed=61, radius=(0.0005, 0.05))
     if order == "by_screen_tile":
         d0 = abi.desc_for_scene(sc)
