@@ -1095,20 +1095,31 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
 }
 
 // Every cell's list in ascending order, in place; of a list longer than kCellKeep its kCellKeep smallest keys, at its
-// start. A wavefront takes 64 consecutive cells (their lists follow each other in the key array), a workgroup a
-// quarter of a tile; the four workgroups of a tile run on the XCD that blends the tile.
+// start. A workgroup takes 64 consecutive cells (their lists follow each other in the key array); the sixteen
+// workgroups of a tile run on the XCD that blends the tile. The first wavefront sorts the lists of up to kLaneSortMax
+// keys, one cell per lane, with a network; the longer lists are dealt to the sixteen 16-lane rows of the workgroup's
+// four wavefronts, which stream them (a wavefront that kept all 64 cells to itself walked up to 64 long lists one
+// after the other, four at a time: in a crowded tile that chain of memory round trips was the kernel's duration).
 __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
 {
-    const int lane = threadIdx.x & 63;
+    __shared__ int s_start[64], s_rd[64];
+    __shared__ unsigned char s_long[64];  // lanes of the cells with a longer list
+    __shared__ int s_num_long;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int NB   = p.geom.bin_off[p.num_layers];
-    const long long lblock = xcd_tile_block(blockIdx.x, 4);
-    if (lblock >= (long long)NB * 4) return;
-    const int cell  = ((int)lblock * 4 + (int)(threadIdx.x >> 6)) * 64 + lane;
-    const int4 info = cell_info(p, cell);
-    const int rd    = info.y;
-    u64* const base = cell_keys(p, info.x);
-    // ---- up to kLaneSortMax keys: one cell per lane ----
+    const long long lblock = xcd_tile_block(blockIdx.x, 16);
+    if (lblock >= (long long)NB * 16) return;
+    if (wave == 0)
     {
+        const int cell  = (int)lblock * 64 + lane;
+        const int4 info = cell_info(p, cell);
+        const int rd    = info.y;
+        u64* const base = cell_keys(p, info.x);
+        const u64 longer = __ballot(rd > kLaneSortMax);
+        s_start[lane] = info.x, s_rd[lane] = rd;
+        if (rd > kLaneSortMax) s_long[__popcll(longer & ((1ull << lane) - 1ull))] = (unsigned char)lane;
+        if (lane == 0) s_num_long = (int)__popcll(longer);
+        // ---- up to kLaneSortMax keys: one cell per lane ----
         const int mine = rd <= kLaneSortMax ? rd : 0;
         const int nmax = wave_max_small<kLaneSortMax>(mine);
         if (nmax > 1)
@@ -1129,51 +1140,40 @@ __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
             }
         }
     }
-    // ---- longer lists: one cell per 16-lane row, four at a time; the first keys of the next four are requested
-    // before these four are worked on ----
-    u64 todo = __ballot(rd > kLaneSortMax);
-    const int sub = lane & 15, grp = lane >> 4;
+    __syncthreads();
+    // ---- longer lists: one cell per 16-lane row, row r of the workgroup takes the lists r, r + 16, ...; the first keys
+    // of a row's next list are requested before it works on this one ----
+    const int num_long = s_num_long;
+    if (num_long == 0) return;
+    const int sub = lane & 15, row = wave * 4 + (lane >> 4);
     struct Pass
     {
         u64* base;
         int readable;
         RowKeys first;
     };
-    auto next_pass = [&]()
+    auto pass_of = [&](int index)
     {
-        int src = -1;  // the lane whose cell this row takes
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-        {
-            if (todo)
-            {
-                const int l = (int)__builtin_ctzll(todo);
-                todo &= todo - 1;
-                if (grp == r) src = l;
-            }
-        }
-        const int from      = max(src, 0);
-        const int row_rd    = __shfl(rd, from);  // (by every lane: a source lane may sit in a row that has no cell)
-        const unsigned b_lo = (unsigned)__shfl((int)(unsigned)(uintptr_t)base, from);
-        const unsigned b_hi = (unsigned)__shfl((int)(unsigned)((uintptr_t)base >> 32), from);
         Pass ps;
-        ps.base     = reinterpret_cast<u64*>(((uintptr_t)b_hi << 32) | (uintptr_t)b_lo);
-        ps.readable = src >= 0 ? row_rd : 0;
-        u64* const rb = ps.base;
-        ps.first    = row_top16_first([&](int i) { return rb[i]; }, ps.readable);
+        const bool has = index < num_long;
+        const int src  = has ? (int)s_long[index] : 0;
+        ps.base        = cell_keys(p, s_start[src]);
+        ps.readable    = has ? s_rd[src] : 0;
+        u64* const rb  = ps.base;
+        ps.first       = row_top16_first([&](int i) { return rb[i]; }, ps.readable);
         return ps;
     };
-    if (!todo) return;
-    Pass cur = next_pass();
-    for (;;)
+    // (the rows of a wavefront walk in step: as many passes as the wavefront's first row has lists)
+    const int passes = (num_long - wave * 4 + 15) / 16;
+    if (passes <= 0) return;
+    Pass cur = pass_of(row);
+    for (int j = 0; j < passes; ++j)
     {
-        const bool more = todo != 0;
-        Pass nxt        = cur;
-        if (more) nxt = next_pass();
+        Pass nxt = cur;
+        if (j + 1 < passes) nxt = pass_of(row + 16 * (j + 1));
         u64* const rb  = cur.base;
         const u64 best = row_top16([&](int i) { return rb[i]; }, cur.readable, cur.first);
         if (sub < min(cur.readable, kCellKeep)) rb[sub] = best;
-        if (!more) break;
         cur = nxt;
     }
 }
@@ -1523,7 +1523,7 @@ hipError_t launch_forward_view(const ForwardParams& p, int channels, bool train,
     const int quarter_tiles = (int)(tiles8 * 4);                                   // a quarter tile per workgroup
     {
         ProfScope ps(prof, "cell_sort", stream);
-        hipLaunchKernelGGL(cell_sort_kernel, dim3(quarter_tiles), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL(cell_sort_kernel, dim3((unsigned)(tiles8 * 16)), dim3(256), 0, stream, p);  // 64 cells per workgroup
     }
     {
         ProfScope ps(prof, "blend", stream);
