@@ -506,10 +506,16 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
     for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
 
     const int stride = (int)gridDim.x * 256;
-    int cid_next     = -1;
+    // The compact number of a point is requested two steps ahead and its point record one step ahead, so that a step
+    // starts with both in hand (a step otherwise begins with two dependent round trips to memory).
+    const float4 kNoRecord = make_float4(0.f, -1.f, 0.f, 0.f);
+    int cid_cur = -1, cid_next = -1;
+    float4 tail_cur = kNoRecord;
     {
-        const int pid0 = (int)blockIdx.x * 256 + (int)threadIdx.x;
-        if (pid0 < p.num_points) cid_next = p.cid_of[pid0];
+        const long long pid0 = (long long)blockIdx.x * 256 + (int)threadIdx.x;
+        if (pid0 < p.num_points) cid_cur = p.cid_of[pid0];
+        if (pid0 + stride < p.num_points) cid_next = p.cid_of[pid0 + stride];
+        if (cid_cur >= 0) tail_cur = reinterpret_cast<const float4*>(p.prec)[cid_cur];
     }
     for (int base = blockIdx.x * 256; base < p.num_points; base += stride)
     {
@@ -517,14 +523,17 @@ __global__ __launch_bounds__(256) void backward_points_kernel(const BackwardPara
         const int pid = base + (int)threadIdx.x;
         // the records of a valid point sit at its compact number (valid points numbered in point order: lanes that are
         // neighbours here are neighbours there)
-        const int cid   = cid_next;
+        const int cid   = cid_cur;
         const bool live = cid >= 0;
-        {
-            const long long pid2 = (long long)pid + stride;
-            cid_next             = pid2 < p.num_points ? p.cid_of[pid2] : -1;  // in flight during this step
-        }
         // {softplus'(raw size), depth, layers written, size_px}
-        const float4 tail = live ? reinterpret_cast<const float4*>(p.prec)[cid] : make_float4(0.f, -1.f, 0.f, 0.f);
+        const float4 tail = tail_cur;
+        {
+            // in flight during this step: the next step's point record, the compact number of the step after it
+            cid_cur              = cid_next;
+            tail_cur             = cid_cur >= 0 ? reinterpret_cast<const float4*>(p.prec)[cid_cur] : kNoRecord;
+            const long long pid3 = (long long)pid + 2ll * stride;
+            cid_next             = pid3 < p.num_points ? p.cid_of[pid3] : -1;
+        }
         // {ip.x, ip.y, size field, confidence} of the blend record and the position: requested here, beside the point
         // record, unless the flags decide first whether the point has any row at all
         float4 r0 = make_float4(0.f, 0.f, 0.f, 0.f), pos = make_float4(0.f, 0.f, 0.f, 0.f);
