@@ -9,21 +9,25 @@
 // whatever their size. So the four pixels of a point's footprint meet in LDS, not in memory:
 //   1. tiles: a workgroup walks a block of 16 x 16 pixels, one pixel per lane, and owns the 15 x 15 cells whose four
 //      pixels lie inside it (a cell = the footprints that start at that pixel); blocks overlap by one row and one
-//      column, which the neighbours walk again. A lane recomputes alpha and transmittance of its pixel's retained entries from the per-point
-//      record exactly as the forward computed them, forms dL/dalpha (the "all later entries" sum of
-//      RenderBackward.cu:284-301 is a running sum from the back of the list) and leaves {dL/dalpha, T alpha} of every
-//      entry in LDS, together with the entry's rank under the (cell, place in the cell's list) that the forward noted
-//      for it. Then a lane per cell collects, for each of the cell's points, the four corner pixels' entries and
-//      writes ONE row per (point, layer) pair: sum over the corners of T alpha dL/dimage and the four dL/dalpha.
-//      The rows of a point's first two layers sit at its compact number, further layers in an overflow table.
-//   2. points: the (point, layer) pairs of 64 consecutive points are dealt out to the lanes; a lane reads its pair's row,
-//      evaluates the bilinear weights' Jacobian and the layer factor per corner (PointBlending.h:216-264,
+//      column, which the neighbours walk again. A lane recomputes alpha and transmittance of its pixel's retained
+//      entries from the per-point record exactly as the forward computed them, forms dL/dalpha (the "all later
+//      entries" sum of RenderBackward.cu:284-301 is a running sum from the back of the list) and leaves
+//      {dL/dalpha, T alpha} of every entry in LDS, together with the entry's list position under the (cell, place in
+//      the cell's list, corner) that the forward noted for it. After a barrier every (point, layer) pair is formed
+//      once, by the wavefront of the first of its corner pixels that retained it: the pairs are queued and dealt to
+//      the lanes, a lane collects the four corner pixels' entries and writes ONE row per pair: sum over the corners of
+//      T alpha dL/dimage and the four dL/dalpha. The rows of a point's first two layers sit at its compact number,
+//      further layers in an overflow table.
+//   2. points: the (point, layer) pairs of 64 consecutive points are dealt out to the lanes; a lane reads its pair's
+//      row, evaluates the bilinear weights' Jacobian and the layer factor per corner (PointBlending.h:216-264,
 //      RenderBackward.cu:366-438); the point's own lane sums the image-space gradient of all its entries and runs the
-//      projection chain ONCE (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then stores or adds its
-//      gradients. Pose / intrinsics partials stay in registers over a grid-stride loop before one block-level
-//      reduction and one atomic per value and block (the reference keeps them in shared double arrays,
+//      projection chain ONCE (the chain is linear in the image-space gradient, RenderBackward.cu:385-417), then stores
+//      or adds its gradients. Pose / intrinsics partials stay in registers over a grid-stride loop before one
+//      block-level reduction and one atomic per value and block (the reference keeps them in shared double arrays,
 //      :160-187,546-617).
-// Gradients are summed in a fixed order and are bit-reproducible from run to run.
+// A prologue kernel clears the rows (or, for a view in which few pairs are retained, one flag byte per row) beforehand.
+// The per-point gradients are summed in a fixed order and are bit-reproducible from run to run; the few block sums
+// (background, pose, intrinsics) are added with one atomic per workgroup, in an order that varies.
 #include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"
