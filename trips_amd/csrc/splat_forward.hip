@@ -15,9 +15,10 @@
 // and a column scan: no global atomics); a workgroup per tile then counts, scans and places the keys of its 1024
 // cells with LDS atomics, one key per pair, and the blend gathers a pixel's list from the four cells whose
 // footprints cover it. The sort is done per cell (each serves four pixels); a pixel is one lane of a wavefront that
-// owns 8 x 8 of them, merges its four cell lists and blends front to back, instead of two lists per 32-lane warp; the per-point record gathered by the blend carries position, size,
-// confidence and descriptor together; what is kept for the backward is the sorted id list per pixel (64 B) instead
-// of 16 x 7 floats.
+// owns 8 x 8 of them, merges its four cell lists and blends front to back, instead of two lists per 32-lane warp; the
+// per-point record gathered by the blend carries position, size, confidence and descriptor together; what is kept
+// for the backward is the sorted id list per pixel (64 B) and a byte per list position that says which cell the
+// entry came from and where it stood in that cell's list, instead of 16 x 7 floats.
 #include "row16.h"
 #include "splat_internal.h"
 #include "trips_math.h"
