@@ -706,16 +706,29 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         return;
     }
 
+    // This workgroup files at most kSliceEntries entries: a thread reads its share once, all loads in flight together,
+    // and keeps it in registers from the count to the placement.
+    constexpr int MAXE = (kSliceEntries + THREADS - 1) / THREADS;
+    ET mine_e[MAXE];
+    const int n_filed = split && slice < 0 ? 0 : n;  // (the workgroup of a split tile files nothing itself)
+#pragma unroll
+    for (int j = 0; j < MAXE; ++j)
+        if ((int)threadIdx.x + j * THREADS < n_filed) mine_e[j] = entries[(int)threadIdx.x + j * THREADS];
+    auto for_mine = [&](auto&& f)
+    {
+#pragma unroll
+        for (int j = 0; j < MAXE; ++j)
+            if ((int)threadIdx.x + j * THREADS < n_filed) f(mine_e[j]);
+    };
     // exclusive scan of the tile's 1024 lengths: PER consecutive pixels per thread
     constexpr int PER = kTilePixels / THREADS;
     const int base4   = threadIdx.x * PER;
     int v[PER], sum = 0;
     if (!split)
     {
-        // count here (the entries come from the L2 when they are read again for the placement)
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
-        for_entries<THREADS>(entries, n, [&](const ET& e) { atomicAdd(&s_cnt[E::cell(e)], 1); });
+        for_mine([&](const ET& e) { atomicAdd(&s_cnt[E::cell(e)], 1); });
         __syncthreads();
     }
 #pragma unroll
@@ -772,7 +785,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     {
         // this slice's share of every cell's list: count, then claim the slots with one atomic per cell
         int32_t* run = p.run + (size_t)bin * kTilePixels;
-        for_entries<THREADS>(entries, n, [&](const ET& e) { atomicAdd(&mine(E::cell(e)), 1); });
+        for_mine([&](const ET& e) { atomicAdd(&mine(E::cell(e)), 1); });
         __syncthreads();
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
@@ -780,7 +793,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
             if (c) s_cnt[i] += atomicAdd(&run[i], c);  // cleared before the counting kernel
         }
         __syncthreads();
-        for_entries<THREADS>(entries, n,
+        for_mine(
                     [&](const ET& e)
                     {
                         const u64 key  = E::key(e);
@@ -798,7 +811,7 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
     extern __shared__ u64 s_keys[];
     const int tile_total = p.bin_start[bin + 1] - key_start;
     const bool staged    = tile_total <= kStageKeys && (long long)key_start + tile_total <= p.capacity;
-    for_entries<THREADS>(entries, n,
+    for_mine(
                 [&](const ET& e)
                 {
                     const u64 key  = E::key(e);
