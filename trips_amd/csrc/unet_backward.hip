@@ -329,7 +329,7 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataPar
     const int x0 = blockIdx.x * kConvTileW, y0 = blockIdx.y * kConvTileH;
     ConvTapStage<KC, NN, THREADS> taps;
     conv_tap_fetch(taps, p.wt, 0);  // in flight while the patch is loaded
-    _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;  // two tap buffers of the weights
+    _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;  // the staged taps of the weights
     // the patch of pre-activation gradients, four 16-byte loads of a thread in flight together
     constexpr int kItems = kConvPatchH * kConvPatchW * GROUPS;
     for (int item0 = threadIdx.x; item0 < kItems; item0 += 4 * THREADS)
@@ -1168,8 +1168,8 @@ namespace
 template <int KC, int NN, int CI>
 hipError_t launch_bwd_data(const BwdDataParams& p, hipStream_t stream)
 {
-    // the patch and two tap buffers of the weights: up to 92 + 35 KB
-    const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW + 2 * NN) * (KC + kLdsChanPad) * sizeof(_Float16);
+    // the patch and the staged taps of the weights
+    const size_t lds_in  = ((size_t)kConvPatchH * kConvPatchW * (KC + kLdsChanPad) + ConvTapStage<KC, NN, 512>::LDS_HALVES) * sizeof(_Float16);
     const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NN + kLdsChanPad) * sizeof(_Float16) + CI * sizeof(float));
     const size_t lds     = std::max(lds_in, lds_out);
     constexpr int THREADS = 512;  // eight wavefronts per tile, as in the forward convolution

@@ -41,13 +41,16 @@ __device__ __forceinline__ void up2_source(int dst, int in_size, int& i0, int& i
 // weights [tap][NOUT][KIN]) reach the matrix cores through LDS as well: with every wavefront loading its own
 // fragments from memory, each of a tile's four wavefronts pulled the level's whole weight set (18 - 147 KB) out of
 // the L2 again, 0.6 GB per launch at the two finest levels, and that traffic, not the MFMAs, set the length of the
-// tap loop. Now the workgroup copies one tap's weights at a time into LDS (the next tap's words travel in registers
-// while the current tap is multiplied, then go to the other of two buffers; one barrier per tap) and every wavefront
-// reads its fragments from there: a quarter of the L2 traffic, the same bank-conflict-free row layout as the patch.
+// tap loop. Now the workgroup copies the weights into LDS and every wavefront reads its fragments from there: a
+// quarter of the L2 traffic, the same bank-conflict-free row layout as the patch. A tap's MFMAs take far less time
+// than a round trip to the L2, so as many taps as the LDS has room for are staged together: all nine (requested when
+// the kernel starts; the tap loop then has neither loads nor barriers), or three (the next three travel in
+// registers while these are multiplied; two barriers per three taps), or one (two buffers, one barrier per tap).
 // A wavefront owns two rows of the 8 x 32 output tile = four 16-pixel row blocks; acc[m][n] is the 16 x 16 block of
 // pixels m, outputs 16n .. 16n+15.
 // THREADS = threads of the workgroup: 256 (a wavefront owns two rows of the tile = four 16-pixel row blocks) or 512 (one
 // row = two row blocks).
+constexpr int kTapLdsBytes = 28 * 1024;  // LDS that the staged taps of a workgroup may take
 template <int KIN, int NOUT, int THREADS = 256>
 struct ConvTapStage
 {
@@ -55,13 +58,18 @@ struct ConvTapStage
     static constexpr int KB    = KIN / 32;
     static constexpr int ROW   = KIN + kLdsChanPad;   // halves per output row of a tap in LDS
     static constexpr int ITEMS = NOUT * KIN / 8;      // 16-byte words per tap
-    static constexpr int PER   = (ITEMS + THREADS - 1) / THREADS;  // per thread
     static constexpr int MB    = 16 / (THREADS / 64);  // 16-pixel row blocks of a wavefront
-    static constexpr int BUF   = NOUT * ROW;           // halves per tap buffer; the kernel provides two
+    static constexpr int BUF   = NOUT * ROW;           // halves per tap in LDS
+    // taps staged together
+    static constexpr int T = 9 * BUF * 2 <= kTapLdsBytes ? 9 : 3 * BUF * 2 <= kTapLdsBytes ? 3 : 1;
+    static constexpr int STAGE_ITEMS = T * ITEMS;      // 16-byte words per stage
+    static constexpr int PER   = (STAGE_ITEMS + THREADS - 1) / THREADS;  // per thread
+    static constexpr int LDS_HALVES = (T == 1 ? 2 : T) * BUF;  // what the kernel provides at s_taps
     half8 r[PER];
 };
 
-// this thread's share of tap `tap` from memory into registers
+// this thread's share of taps `tap` .. `tap` + T - 1 from memory into registers (the packed weights are dense:
+// [tap][NOUT][KIN])
 template <int KIN, int NOUT, int THREADS>
 __device__ __forceinline__ void conv_tap_fetch(ConvTapStage<KIN, NOUT, THREADS>& st, const _Float16* __restrict__ wpack, int tap)
 {
@@ -71,11 +79,11 @@ __device__ __forceinline__ void conv_tap_fetch(ConvTapStage<KIN, NOUT, THREADS>&
     for (int j = 0; j < S::PER; ++j)
     {
         const int item = threadIdx.x + THREADS * j;
-        if (S::ITEMS % THREADS == 0 || item < S::ITEMS) st.r[j] = src[item];
+        if (S::STAGE_ITEMS % THREADS == 0 || item < S::STAGE_ITEMS) st.r[j] = src[item];
     }
 }
 
-// ... and from the registers into a tap buffer
+// ... and from the registers into the tap buffers at s_tap (T of them, one after the other)
 template <int KIN, int NOUT, int THREADS>
 __device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT, THREADS>& st, _Float16* s_tap)
 {
@@ -84,13 +92,16 @@ __device__ __forceinline__ void conv_tap_stage(const ConvTapStage<KIN, NOUT, THR
     for (int j = 0; j < S::PER; ++j)
     {
         const int item = threadIdx.x + THREADS * j;
-        if (S::ITEMS % THREADS == 0 || item < S::ITEMS)
-            *reinterpret_cast<half8*>(s_tap + (item / (KIN / 8)) * S::ROW + (item % (KIN / 8)) * 8) = st.r[j];
+        if (S::STAGE_ITEMS % THREADS == 0 || item < S::STAGE_ITEMS)
+        {
+            const int t = item / S::ITEMS, w = item - t * S::ITEMS;
+            *reinterpret_cast<half8*>(s_tap + t * S::BUF + (w / (KIN / 8)) * S::ROW + (w % (KIN / 8)) * 8) = st.r[j];
+        }
     }
 }
 
-// Precondition: tap 0 sits in s_taps[0 .. BUF) (conv_tap_fetch + conv_tap_stage) and a barrier has passed since.
-// Every thread of the workgroup must call this (it contains barriers).
+// Precondition: the first T taps sit at s_taps (conv_tap_fetch(.., 0) + conv_tap_stage) and a barrier has passed since.
+// Every thread of the workgroup must call this (it contains barriers unless all nine taps are staged).
 // Result layout: lane l holds, of the 16 x 16 block acc[m][n], pixels (l / 16) * 4 .. + 3 of output 16n + l % 16; with
 // OUTPUTS_IN_ROWS (the operands of the MFMA exchanged) outputs 16n + (l / 16) * 4 .. + 3 of pixel l % 16, four
 // neighbouring channels of one pixel, which an epilogue can store as one 8-byte word.
@@ -104,6 +115,7 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
     constexpr int ROW = KIN + kLdsChanPad;
     constexpr int NB  = S::NB;
     constexpr int KB  = S::KB;
+    constexpr int T   = S::T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 #pragma unroll
@@ -114,8 +126,9 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
     for (int tap = 0; tap < 9; ++tap)
     {
         const int dy = tap / 3, dx = tap - dy * 3;  // patch coordinates already include the halo
-        if (tap + 1 < 9) conv_tap_fetch(st, wpack, tap + 1);
-        const _Float16* sb = s_taps + (tap & 1) * S::BUF;
+        // the next stage's weights: requested before this stage's first tap is multiplied
+        if (T < 9 && tap % T == 0 && tap + T < 9) conv_tap_fetch(st, wpack, tap + T);
+        const _Float16* sb = s_taps + (T == 1 ? tap & 1 : tap % T) * S::BUF;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
         {
@@ -133,9 +146,19 @@ __device__ __forceinline__ void conv_taps_mfma(const _Float16* s_patch, _Float16
                                                 : __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[n], acc[m][n], 0, 0, 0);
             }
         }
-        if (tap + 1 < 9) conv_tap_stage(st, s_taps + ((tap + 1) & 1) * S::BUF);
-        __syncthreads();  // the next tap is in place; nobody reads this tap's buffer any more
+        if (T == 1)
+        {
+            if (tap + 1 < 9) conv_tap_stage(st, s_taps + ((tap + 1) & 1) * S::BUF);
+            __syncthreads();  // the next tap is in place; nobody reads this tap's buffer any more
+        }
+        else if (T < 9 && tap % T == T - 1 && tap + 1 < 9)
+        {
+            __syncthreads();  // nobody reads this stage's taps any more
+            conv_tap_stage(st, s_taps);
+            __syncthreads();  // the next stage is in place
+        }
     }
+    if (T != 1) __syncthreads();  // (as after the last tap of the one-tap form: patch and taps may be overwritten now)
 }
 
 // Copies `groups` x 8 halves per pixel of an 8 x 32 tile staged in LDS ([256][lds_stride]) to a channels-innermost

@@ -69,8 +69,8 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     if (p.final_out)
     {
         const int cin = p.c_feat + p.cout;
-        for (int i = threadIdx.x; i < p.final_cout * cin; i += THREADS) s_fw[i] = float(_Float16(p.final_w[i]));
-        if ((int)threadIdx.x < p.final_cout) s_fw[kFwBias + threadIdx.x] = p.final_b[threadIdx.x];
+        for (int i = (int)threadIdx.x; i < p.final_cout * cin; i += THREADS) s_fw[i] = float(_Float16(p.final_w[i]));
+        if ((int)threadIdx.x < p.final_cout) s_fw[kFwBias + (int)threadIdx.x] = p.final_b[(int)threadIdx.x];
     }
 
     // ---- stage 1: everything the patch needs from memory, all loads of a thread in flight together ----
@@ -90,12 +90,16 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     uint4 below_v[kBelowItems];
     const int act_groups = has_below ? p.cb_store / 8 : 0;
     const int per_pixel  = IQ + act_groups;  // items 0 .. IQ - 1 of a pixel: the image below; others: 8 activations each
+    // item / per_pixel without an integer division: items stay below 2^11 and per_pixel below 2^5, so the quotient of
+    // item + 1/2 is at least 1/64 away from every integer, far more than the rounding of the product
+    const float inv_per_pixel = 1.f / float(per_pixel);
+    auto pixel_of_item        = [&](int item) { return (int)((float(item) + 0.5f) * inv_per_pixel); };
     {
         const size_t plane = (size_t)p.H * p.W;
 #pragma unroll
         for (int k = 0; k < kFeatItems; ++k)
         {
-            const int item = threadIdx.x + THREADS * k;
+            const int item = (int)threadIdx.x + THREADS * k;
             const int py = item / kConvPatchW, px = item - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
             const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
@@ -109,11 +113,11 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
 #pragma unroll
         for (int k = 0; k < kBelowItems; ++k)
         {
-            const int item = threadIdx.x + THREADS * k;
+            const int item = (int)threadIdx.x + THREADS * k;
             below_v[k]     = make_uint4(0u, 0u, 0u, 0u);
             if (item < kBelowH * kBelowW * per_pixel)
             {
-                const int q = item % per_pixel, bp = item / per_pixel;
+                const int bp = pixel_of_item(item), q = item - bp * per_pixel;
                 const int r = bp / kBelowW, c0 = bp - r * kBelowW;
                 const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
                 if (q < IQ)
@@ -132,7 +136,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
 #pragma unroll
     for (int k = 0; k < kFeatItems; ++k)
     {
-        const int item = threadIdx.x + THREADS * k;
+        const int item = (int)threadIdx.x + THREADS * k;
         if (item < kConvPatchH * kConvPatchW)
         {
             _Float16* row = s_patch + (size_t)item * ROW;
@@ -157,10 +161,10 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
 #pragma unroll
         for (int k = 0; k < kBelowItems; ++k)
         {
-            const int item = threadIdx.x + THREADS * k;
+            const int item = (int)threadIdx.x + THREADS * k;
             if (item < kBelowH * kBelowW * per_pixel)
             {
-                const int q = item % per_pixel, bp = item / per_pixel;
+                const int bp = pixel_of_item(item), q = item - bp * per_pixel;
                 _Float16* row = s_below + (size_t)bp * ROW;
                 if (q < IQ)
                 {
@@ -193,59 +197,73 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
         }
         __syncthreads();
         // ---- stage 2: bilinear 2x upsampling from the below patch into channels [C, CIN) of the patch ----
-        for (int item = threadIdx.x; item < kConvPatchH * kConvPatchW * GROUPS; item += THREADS)
+        // A thread takes a pixel of the patch and walks its groups of 8 channels: the pixel's position, sources and
+        // weights are worked out once (with an item per (pixel, group) that arithmetic was most of the stage).
+        for (int pp = (int)threadIdx.x; pp < kConvPatchH * kConvPatchW; pp += THREADS)
         {
-            const int g = item % GROUPS, pp = item / GROUPS;
             const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
+            const bool inside = y >= 0 && y < p.H && x >= 0 && x < p.W;
             // The interpolation runs in packed fp16: the weights are products of 0, 1/4, 3/4 and 1 (exact in fp16), the
             // operands are fp16 already and the result is stored as fp16; three fused multiply-adds per pair of channels
             // instead of eight conversions and four fp32 operations per channel.
-            half8 h;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) h[i] = _Float16(0.f);
-            if (y >= 0 && y < p.H && x >= 0 && x < p.W)
+            int ya = by0, yb = by0, xa = bx0, xb = bx0;
+            float ly = 0.f, lx = 0.f;
+            if (inside)
             {
-                int ya, yb, xa, xb;
-                float ly, lx;
                 up2_source(y, p.Hb, ya, yb, ly);
                 up2_source(x, p.Wb, xa, xb, lx);
-                const _Float16 w00 = _Float16((1.f - ly) * (1.f - lx)), w01 = _Float16((1.f - ly) * lx);
-                const _Float16 w10 = _Float16(ly * (1.f - lx)), w11 = _Float16(ly * lx);
-                const half8 a = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
-                const half8 b = *reinterpret_cast<const half8*>(s_below + ((ya - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
-                const half8 c = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xa - bx0)) * ROW + 8 * g);
-                const half8 d = *reinterpret_cast<const half8*>(s_below + ((yb - by0) * kBelowW + (xb - bx0)) * ROW + 8 * g);
-                const half8 W00 = {w00, w00, w00, w00, w00, w00, w00, w00}, W01 = {w01, w01, w01, w01, w01, w01, w01, w01};
-                const half8 W10 = {w10, w10, w10, w10, w10, w10, w10, w10}, W11 = {w11, w11, w11, w11, w11, w11, w11, w11};
-                h = __builtin_elementwise_fma(d, W11, __builtin_elementwise_fma(c, W10, __builtin_elementwise_fma(b, W01, a * W00)));
             }
-            _Float16* dst = s_patch + (size_t)pp * ROW + 8 * g;
-            if (8 * g < C)
-            {
-                // [0, C) holds this level's image
-                if (CI == 4 && C == 4)
-                    *reinterpret_cast<half4*>(dst + 4) = half4{h[4], h[5], h[6], h[7]};
-                else
-                {
+            const _Float16 w00 = _Float16((1.f - ly) * (1.f - lx)), w01 = _Float16((1.f - ly) * lx);
+            const _Float16 w10 = _Float16(ly * (1.f - lx)), w11 = _Float16(ly * lx);
+            const half8 W00 = {w00, w00, w00, w00, w00, w00, w00, w00}, W01 = {w01, w01, w01, w01, w01, w01, w01, w01};
+            const half8 W10 = {w10, w10, w10, w10, w10, w10, w10, w10}, W11 = {w11, w11, w11, w11, w11, w11, w11, w11};
+            const _Float16* sa = s_below + ((ya - by0) * kBelowW + (xa - bx0)) * ROW;
+            const _Float16* sb = s_below + ((ya - by0) * kBelowW + (xb - bx0)) * ROW;
+            const _Float16* sc = s_below + ((yb - by0) * kBelowW + (xa - bx0)) * ROW;
+            const _Float16* sd = s_below + ((yb - by0) * kBelowW + (xb - bx0)) * ROW;
+            _Float16* drow     = s_patch + (size_t)pp * ROW;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i)
-                        if (8 * g + i >= C) dst[i] = h[i];
+            for (int g = 0; g < GROUPS; ++g)
+            {
+                half8 h;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = _Float16(0.f);
+                if (inside)
+                {
+                    const half8 a = *reinterpret_cast<const half8*>(sa + 8 * g);
+                    const half8 b = *reinterpret_cast<const half8*>(sb + 8 * g);
+                    const half8 c = *reinterpret_cast<const half8*>(sc + 8 * g);
+                    const half8 d = *reinterpret_cast<const half8*>(sd + 8 * g);
+                    h = __builtin_elementwise_fma(d, W11, __builtin_elementwise_fma(c, W10, __builtin_elementwise_fma(b, W01, a * W00)));
                 }
+                _Float16* dst = drow + 8 * g;
+                if (8 * g < C)
+                {
+                    // [0, C) holds this level's image
+                    if (CI == 4 && C == 4)
+                        *reinterpret_cast<half4*>(dst + 4) = half4{h[4], h[5], h[6], h[7]};
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            if (8 * g + i >= C) dst[i] = h[i];
+                    }
+                }
+                else
+                    *reinterpret_cast<half8*>(dst) = h;
             }
-            else
-                *reinterpret_cast<half8*>(dst) = h;
         }
     }
 
     __syncthreads();  // patch complete; the patch of the level below is no longer needed
-    // two tap buffers for the weights, in place of the patch of the level below
+    // the staged taps of the weights, in place of the patch of the level below
     _Float16* s_taps = s_patch + kConvPatchH * kConvPatchW * ROW;
     conv_tap_stage(taps, s_taps);
     __syncthreads();
     floatx4 acc[MB][NB];
     conv_taps_mfma<CIN, NPAD, true, THREADS>(s_patch, s_taps, p.wpack, taps, acc);  // a lane: four channels of one pixel
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
     const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
     // ---- epilogue: elu(feature) * sigmoid(mask) in fp16, staged in LDS (the patch is no longer needed) and
@@ -260,7 +278,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     const bool owns_pixel = THREADS == kConvTileH * kConvTileW || (int)threadIdx.x < kConvTileH * kConvTileW;  // one thread per pixel
     if (p.final_out && owns_pixel)
     {
-        const _Float16* row = s_patch + (size_t)((threadIdx.x / kConvTileW + 1) * kConvPatchW + threadIdx.x % kConvTileW + 1) * ROW;
+        const _Float16* row = s_patch + (size_t)(((int)threadIdx.x / kConvTileW + 1) * kConvPatchW + (int)threadIdx.x % kConvTileW + 1) * ROW;
 #pragma unroll
         for (int c = 0; c < CI; ++c)
             if (c < C) my_feat[c] = float(row[c]);
@@ -309,7 +327,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
         // the image joins the staged rows (columns NPAD/2 .. NPAD/2 + IPAD - 1; nobody has read them yet)
         if (owns_pixel)
         {
-            _Float16* row = s_act + (size_t)threadIdx.x * AS + NPAD / 2;
+            _Float16* row = s_act + (size_t)(int)threadIdx.x * AS + NPAD / 2;
 #pragma unroll
             for (int c = 0; c < IPAD; ++c) row[c] = (c < CI && c < C) ? _Float16(my_feat[c < CI ? c : 0]) : _Float16(0.f);
         }
@@ -418,8 +436,8 @@ hipError_t launch_conv(const ConvParams& p, hipStream_t stream)
 {
     constexpr int ROW  = CIN + kLdsChanPad;
     constexpr int IPAD = CI > kLdsChanPad ? CI : kLdsChanPad;
-    // the patch, then the patch of the level below or (later) two tap buffers of the weights, whichever is larger
-    const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW * ROW + std::max(kBelowH * kBelowW * ROW, 2 * NPAD * ROW)) * sizeof(_Float16);
+    // the patch, then the patch of the level below or (later) the staged taps of the weights, whichever is larger
+    const size_t lds_in  = (size_t)(kConvPatchH * kConvPatchW * ROW + std::max(kBelowH * kBelowW * ROW, ConvTapStage<CIN, NPAD, 512>::LDS_HALVES)) * sizeof(_Float16);
     const size_t lds_out = (size_t)kConvTileH * kConvTileW * ((NPAD / 2 + IPAD) + (p.pre ? NPAD + kLdsChanPad : 0)) * sizeof(_Float16);
     const size_t lds     = std::max(lds_in, lds_out);  // up to 104 KB when the largest block saves its pre-activations
     // eight wavefronts per tile (one row each): the phases around the tap loop run at the latency of their loads and LDS
