@@ -31,17 +31,17 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "a4c5a59755d3f423c9a4196a558f58819c956e1262c1df3f5d8f9539c451c331"
+PMC_SOURCES_SHA256 = "88e7d2760502716c0120058a721ce33c9f304c6865feb49a652b349e683180e8"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129116, 243308),
-    "bin_scatter": (95989, 166616),
+    "project_bin": (129114, 243885),
+    "bin_scatter": (95985, 166456),
     "tile_count": (13142, 2296),
-    "tile_scatter": (32664, 109463),
-    "cell_sort": (35353, 42128),
-    "blend": (318476, 195715),
-    "backward_prologue": (50, 265161),
-    "backward_tiles": (425230, 121558),
-    "backward_points": (297431, 234503),
+    "tile_scatter": (26677, 105408),
+    "cell_sort": (35350, 42131),
+    "blend": (318236, 195795),
+    "backward_prologue": (50, 265115),
+    "backward_tiles": (425765, 121589),
+    "backward_points": (297573, 234503),
     "adam_fused": (383789, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
