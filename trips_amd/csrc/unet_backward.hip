@@ -131,22 +131,25 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
     const bool in_row  = g < 2 * hg;                     // lanes past the row idle (rows of 96 halves on 16 lanes)
     const int ch0      = 8 * (is_f ? g : g - hg);        // first of this lane's 8 channels
     const int partner  = is_f ? lane + hg : lane - hg;   // the lane with the other half of the same channels
-    const bool has_act = is_f && ch0 < CS;               // this lane also reads the block output of its channels
     // ... and the image channels g, g + LPP, ... (one each for up to LPP image channels)
     constexpr int NI = (CI + LPP - 1) / LPP;
     bool has_img[NI];
 #pragma unroll
     for (int j = 0; j < NI; ++j) has_img[j] = g + LPP * j < p.c_feat;
-    float wj[4][8], wimg[4][NI];
+    // The feature lane and the mask lane of a group hold the same eight channels once they have exchanged their values:
+    // the feature lane works out the first four (gradients of both pre-activations, the block's output), the mask lane
+    // the other four, and they exchange what the other one stores.
+    const int c0 = ch0 + (is_f ? 0 : 4);  // first of the four channels this lane works out
+    float wj[4][4], wimg[4][NI];
 #pragma unroll
     for (int k = 0; k < 4; ++k)
     {
 #pragma unroll
         for (int j = 0; j < NI; ++j) wimg[k][j] = has_img[j] ? s_w[k * MAXC + g + LPP * j] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) wj[k][i] = (in_row && ch0 + i < CS) ? s_w[k * MAXC + CI + ch0 + i] : 0.f;
+        for (int i = 0; i < 4; ++i) wj[k][i] = (in_row && c0 + i < CS) ? s_w[k * MAXC + CI + c0 + i] : 0.f;
     }
-    float acc[4][8];
+    float acc[4][4];
     float acc_img[4][NI], accb[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < 4; ++k)
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
 #pragma unroll
     for (int k = 0; k < 4; ++k)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[k][i] = 0.f;
+        for (int i = 0; i < 4; ++i) acc[k][i] = 0.f;
 
     struct Loaded
     {
@@ -193,19 +196,29 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
             for (int q = 0; q < 4; ++q) oth[q] = __shfl(raw[q], partner);
             const half8 other = __builtin_bit_cast(half8, oth);
             const half8 f8 = is_f ? cur.mine : other, m8 = is_f ? other : cur.mine;
-            half8 out;
-            float v[8];  // the block's output as the forward's 1x1 convolution read it (fp16), on the feature lanes
+            half4 keep, give;  // what this lane stores of its four channels, and what its partner stores of them
+            float v[4];        // the block's output as the forward's 1x1 convolution read it (fp16)
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < 4; ++i)
             {
                 float da = 0.f;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) da += wj[k][i] * cur.g[k];
                 float df, dm, a;
-                gate_backward(da * p.scale, float(f8[i]), float(m8[i]), df, dm, a);
-                out[i] = _Float16(is_f ? df : dm);
-                v[i]   = (valid && has_act && ch0 + i < p.cact) ? float(_Float16(a)) : 0.f;
+                gate_backward(da * p.scale, float(is_f ? f8[i] : f8[4 + i]), float(is_f ? m8[i] : m8[4 + i]), df, dm, a);
+                keep[i] = _Float16(is_f ? df : dm);
+                give[i] = _Float16(is_f ? dm : df);
+                v[i]    = (valid && in_row && c0 + i < p.cact) ? float(_Float16(a)) : 0.f;
             }
+            typedef int intx2 __attribute__((ext_vector_type(2)));
+            const intx2 give_raw = __builtin_bit_cast(intx2, give);
+            intx2 got_raw;
+            got_raw[0] = __shfl(give_raw[0], partner);
+            got_raw[1] = __shfl(give_raw[1], partner);
+            const half4 got = __builtin_bit_cast(half4, got_raw);
+            // a feature lane stores the feature gradients of the eight channels: its own four, then the partner's
+            const half8 out = is_f ? half8{keep[0], keep[1], keep[2], keep[3], got[0], got[1], got[2], got[3]}
+                                   : half8{got[0], got[1], got[2], got[3], keep[0], keep[1], keep[2], keep[3]};
             if (valid && in_row) *reinterpret_cast<half8*>(p.dpre + pix * p.npad + 8 * g) = out;
 #pragma unroll
             for (int j = 0; j < NI; ++j)
@@ -230,7 +243,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
 #pragma unroll
                     for (int j = 0; j < NI; ++j) acc_img[k][j] += cur.g[k] * xr[j];
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc[k][i] += cur.g[k] * v[i];
+                    for (int i = 0; i < 4; ++i) acc[k][i] += cur.g[k] * v[i];
                 }
             }
         }
@@ -256,10 +269,10 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
             if (lane < LPP && has_img[j]) atomicAdd(&s_sum[k * MAXC + g + LPP * j], im);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 4; ++i)
         {
             const float v = fold(acc[k][i]);
-            if (lane < LPP && has_act && ch0 + i < CS) atomicAdd(&s_sum[k * MAXC + CI + ch0 + i], v);
+            if (lane < LPP && in_row && c0 + i < CS) atomicAdd(&s_sum[k * MAXC + CI + c0 + i], v);
         }
     }
     __syncthreads();
