@@ -100,6 +100,8 @@ struct FinalBwdParams
 // WGRAD, the weight and bias gradients of the 1x1 convolution. Every thread keeps the cout x cin products of its
 // pixels in registers, a workgroup folds them through LDS and writes its sums once (final_reduce_kernel adds the
 // workgroups up: atomics of a thousand workgroups on these few addresses would serialise in one L2 channel).
+// (The library is compiled without contraction of products and sums; this kernel is bound by its arithmetic
+// instructions, and its sums are written as fused multiply-adds.)
 // CS = halves per pixel of the block output.
 // CI = image channels the kernel has room for (4, 8 or 16).
 template <int CS, bool WGRAD, int CI>
@@ -203,7 +205,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
             {
                 float da = 0.f;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) da += wj[k][i] * cur.g[k];
+                for (int k = 0; k < 4; ++k) da = __builtin_fmaf(wj[k][i], cur.g[k], da);
                 float df, dm, a;
                 gate_backward(da * p.scale, float(is_f ? f8[i] : f8[4 + i]), float(is_f ? m8[i] : m8[4 + i]), df, dm, a);
                 keep[i] = _Float16(is_f ? df : dm);
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
                 {
                     float d = 0.f;
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) d += wimg[k][j] * cur.g[k];
+                    for (int k = 0; k < 4; ++k) d = __builtin_fmaf(wimg[k][j], cur.g[k], d);
                     p.d_feat[(size_t)(g + LPP * j) * plane + pix] = d;
                 }
             }
@@ -241,9 +243,9 @@ __global__ __launch_bounds__(256) void final_backward_kernel(const FinalBwdParam
                 {
                     accb[k] += cur.g[k];
 #pragma unroll
-                    for (int j = 0; j < NI; ++j) acc_img[k][j] += cur.g[k] * xr[j];
+                    for (int j = 0; j < NI; ++j) acc_img[k][j] = __builtin_fmaf(cur.g[k], xr[j], acc_img[k][j]);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[k][i] += cur.g[k] * v[i];
+                    for (int i = 0; i < 4; ++i) acc[k][i] = __builtin_fmaf(cur.g[k], v[i], acc[k][i]);
                 }
             }
         }
@@ -482,16 +484,16 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
             // waited for there: 16 memory round trips in a row); pixels outside the image have weight 0 and are read
             // at a clamped position instead
             half8 v[4][4];
+            int xoff[4];  // (a row of the finer level stays below 2^31 halves)
+#pragma unroll
+            for (int kx = 0; kx < 4; ++kx) xoff[kx] = min(max(2 * X - 1 + kx, 0), p.W - 1) * p.cin_fine + pos;
 #pragma unroll
             for (int ky = 0; ky < 4; ++ky)
             {
-                const int y = min(max(2 * Y - 1 + ky, 0), p.H - 1);
+                const int y         = min(max(2 * Y - 1 + ky, 0), p.H - 1);
+                const _Float16* row = p.d_in + (size_t)y * p.W * p.cin_fine;
 #pragma unroll
-                for (int kx = 0; kx < 4; ++kx)
-                {
-                    const int x = min(max(2 * X - 1 + kx, 0), p.W - 1);
-                    v[ky][kx]   = *reinterpret_cast<const half8*>(p.d_in + ((size_t)y * p.W + x) * p.cin_fine + pos);
-                }
+                for (int kx = 0; kx < 4; ++kx) v[ky][kx] = *reinterpret_cast<const half8*>(row + xoff[kx]);
             }
 #pragma unroll
             for (int ky = 0; ky < 4; ++ky)
@@ -502,8 +504,9 @@ __global__ __launch_bounds__(256) void up2_adjoint_gate_kernel(const UpAdjointPa
                     const float w = wy[ky] * wx[kx];
                     if (w != 0.f)
                     {
+                        // (one fused multiply-add that reads the fp16 value, instead of a conversion, a product and a sum)
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) a[i] += w * float(v[ky][kx][i]);
+                        for (int i = 0; i < 8; ++i) a[i] = __builtin_fmaf(w, float(v[ky][kx][i]), a[i]);
                     }
                 }
             }
