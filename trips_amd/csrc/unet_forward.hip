@@ -47,6 +47,12 @@ struct ConvParams
     int final_cout;
 };
 
+// A loaded value that is only needed under a condition is otherwise loaded under that condition by the compiler, in a
+// branch that waits for it before it ends. Values passed through here exist where this is called, whatever they are
+// used for later: called for all loads of a stage after the last of them, it keeps them in flight together.
+__device__ __forceinline__ void loaded(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void loaded(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+
 // CI: image channels the kernel has room for (4, 8 or 16; C <= CI)
 template <int CIN, int NPAD, int THREADS, int CI>
 __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams p)
@@ -66,34 +72,41 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
     // weights and biases of the 1x1 output convolution, rounded to fp16 like every other operand
     constexpr int kFwBias = 4 * (CI + 64);  // [final_cout <= 4][C + cout <= CI + 64] weights, then the biases
     __shared__ float s_fw[kFwBias + 4];
-    if (p.final_out)
-    {
-        const int cin = p.c_feat + p.cout;
-        for (int i = (int)threadIdx.x; i < p.final_cout * cin; i += THREADS) s_fw[i] = float(_Float16(p.final_w[i]));
-        if ((int)threadIdx.x < p.final_cout) s_fw[kFwBias + (int)threadIdx.x] = p.final_b[(int)threadIdx.x];
-    }
 
     // ---- stage 1: everything the patch needs from memory, all loads of a thread in flight together ----
     // (a) this level's image -> channels [0, C) of the patch; (b) the level below, x_{i+1} = cat(image, activations),
     // as a (TILE/2 + 2)^2 patch in the same row format, channel k of the concatenated input at row position k.
+    // Every load below is unconditional, at an address clamped into its array, and what a thread does not need is
+    // replaced by zero afterwards: a load inside a branch is waited for before the branch is left, and the eight or
+    // nine round trips to memory of a thread then ran one after the other (72 % of a tile's life at the finest level).
     constexpr int GROUPS = CIN / 8;
     _Float16* s_below    = s_patch + kConvPatchH * kConvPatchW * ROW;  // [kBelowH * kBelowW][ROW]
     const int by0 = y0 / 2 - 1, bx0 = x0 / 2 - 1;
     const int C   = p.c_feat;
-    // (first every load into registers, then the conversions and LDS stores: written as loops that load and store
-    // item by item, a thread's five round trips to memory ran one after the other and stage 1 was 39 % of a
-    // workgroup's life)
     constexpr int kFeatItems  = (kConvPatchH * kConvPatchW + THREADS - 1) / THREADS;
     constexpr int kMaxPerPix  = IQ + CIN / 8;  // image below (four channels per item) + groups of 8 block outputs
     constexpr int kBelowItems = (kBelowH * kBelowW * kMaxPerPix + THREADS - 1) / THREADS;
     float feat_v[kFeatItems][CI];
+    bool feat_in[kFeatItems];
     uint4 below_v[kBelowItems];
+    float below_f[kBelowItems][4];
+    bool below_have[kBelowItems], below_img[kBelowItems];
     const int act_groups = has_below ? p.cb_store / 8 : 0;
     const int per_pixel  = IQ + act_groups;  // items 0 .. IQ - 1 of a pixel: the image below; others: 8 activations each
     // item / per_pixel without an integer division: items stay below 2^11 and per_pixel below 2^5, so the quotient of
     // item + 1/2 is at least 1/64 away from every integer, far more than the rounding of the product
     const float inv_per_pixel = 1.f / float(per_pixel);
     auto pixel_of_item        = [&](int item) { return (int)((float(item) + 0.5f) * inv_per_pixel); };
+    // the 1x1's weights and biases: requested here, stored to LDS with the patch
+    constexpr int kFwItems = (kFwBias + THREADS - 1) / THREADS;
+    float fw_v[kFwItems], fb_v = 0.f;
+    const int fw_n = p.final_out ? p.final_cout * (p.c_feat + p.cout) : 0;
+    if (p.final_out)
+    {
+#pragma unroll
+        for (int k = 0; k < kFwItems; ++k) fw_v[k] = p.final_w[min((int)threadIdx.x + THREADS * k, fw_n - 1)];
+        fb_v = p.final_b[min((int)threadIdx.x, p.final_cout - 1)];
+    }
     {
         const size_t plane = (size_t)p.H * p.W;
 #pragma unroll
@@ -103,8 +116,10 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
             const int py = item / kConvPatchW, px = item - py * kConvPatchW;
             const int y = y0 + py - 1, x = x0 + px - 1;
             const bool in = item < kConvPatchH * kConvPatchW && y >= 0 && y < p.H && x >= 0 && x < p.W;
+            const float* src = p.feat + (size_t)min(max(y, 0), p.H - 1) * p.W + min(max(x, 0), p.W - 1);
+            feat_in[k] = in;
 #pragma unroll
-            for (int c = 0; c < CI; ++c) feat_v[k][c] = (in && c < C) ? p.feat[c * plane + (size_t)y * p.W + x] : 0.f;
+            for (int c = 0; c < CI; ++c) feat_v[k][c] = src[(c < C ? c : 0) * plane];
         }
     }
     if (has_below)
@@ -114,24 +129,68 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
         for (int k = 0; k < kBelowItems; ++k)
         {
             const int item = (int)threadIdx.x + THREADS * k;
-            below_v[k]     = make_uint4(0u, 0u, 0u, 0u);
-            if (item < kBelowH * kBelowW * per_pixel)
-            {
-                const int bp = pixel_of_item(item), q = item - bp * per_pixel;
-                const int r = bp / kBelowW, c0 = bp - r * kBelowW;
-                const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
-                if (q < IQ)
-                {
-                    const float* src = p.feat_below + (size_t)yy * p.Wb + xx;
-                    float f[4];
+            // (kBelowItems is sized for the widest level below; a round in which no thread has an item is skipped as a
+            // whole: the finest level of the usual plan has 432 items for its 512 threads)
+            if (THREADS * k >= kBelowH * kBelowW * per_pixel) break;
+            const bool have = item < kBelowH * kBelowW * per_pixel;
+            const int it    = have ? item : 0;
+            const int bp = pixel_of_item(it), q = it - bp * per_pixel;
+            const int r = bp / kBelowW, c0 = bp - r * kBelowW;
+            const int yy = min(max(by0 + r, 0), p.Hb - 1), xx = min(max(bx0 + c0, 0), p.Wb - 1);
+            const bool img = q < IQ;
+            // an image item: four planes of the image below; any other item reads plane 0 four times and drops it
+            const float* src = p.feat_below + (size_t)yy * p.Wb + xx;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) f[c] = 4 * q + c < C ? src[(size_t)(4 * q + c) * pb] : 0.f;
-                    below_v[k] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
-                }
-                else
-                    below_v[k] = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (q - IQ));
-            }
+            for (int c = 0; c < 4; ++c) below_f[k][c] = src[(size_t)(img && 4 * q + c < C ? 4 * q + c : 0) * pb];
+            // an item of block outputs: eight of them; an image item reads the pixel's first eight and drops them
+            below_v[k]    = *reinterpret_cast<const uint4*>(p.act_below + ((size_t)yy * p.Wb + xx) * p.cb_store + 8 * (img ? 0 : q - IQ));
+            below_have[k] = have;
+            below_img[k]  = img;
         }
+    }
+    // ---- all loads are on their way: from here on their values are used ----
+    if (p.final_out)
+    {
+#pragma unroll
+        for (int k = 0; k < kFwItems; ++k) loaded(fw_v[k]);
+        loaded(fb_v);
+    }
+#pragma unroll
+    for (int k = 0; k < kFeatItems; ++k)
+#pragma unroll
+        for (int c = 0; c < CI; ++c)
+        {
+            loaded(feat_v[k][c]);
+            if (!(feat_in[k] && c < C)) feat_v[k][c] = 0.f;
+        }
+    if (has_below)
+    {
+#pragma unroll
+        for (int k = 0; k < kBelowItems; ++k)
+        {
+            if (THREADS * k >= kBelowH * kBelowW * per_pixel) break;
+            const int item = (int)threadIdx.x + THREADS * k;
+            const int it   = below_have[k] ? item : 0;
+            const int q    = it - pixel_of_item(it) * per_pixel;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+            {
+                loaded(below_f[k][c]);
+                if (!(below_img[k] && 4 * q + c < C)) below_f[k][c] = 0.f;
+            }
+            loaded(below_v[k]);
+            if (below_img[k])
+                below_v[k] = make_uint4(__float_as_uint(below_f[k][0]), __float_as_uint(below_f[k][1]), __float_as_uint(below_f[k][2]),
+                                        __float_as_uint(below_f[k][3]));
+            if (!below_have[k]) below_v[k] = make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+    if (p.final_out)
+    {
+#pragma unroll
+        for (int k = 0; k < kFwItems; ++k)
+            if ((int)threadIdx.x + THREADS * k < fw_n) s_fw[(int)threadIdx.x + THREADS * k] = float(_Float16(fw_v[k]));
+        if ((int)threadIdx.x < p.final_cout) s_fw[kFwBias + (int)threadIdx.x] = fb_v;
     }
 #pragma unroll
     for (int k = 0; k < kFeatItems; ++k)
@@ -162,6 +221,7 @@ __global__ __launch_bounds__(THREADS) void gated_conv3x3_kernel(const ConvParams
         for (int k = 0; k < kBelowItems; ++k)
         {
             const int item = (int)threadIdx.x + THREADS * k;
+            if (THREADS * k >= kBelowH * kBelowW * per_pixel) break;
             if (item < kBelowH * kBelowW * per_pixel)
             {
                 const int bp = pixel_of_item(item), q = item - bp * per_pixel;
