@@ -33,15 +33,15 @@ DEFAULT_POINTS = 6_000_000
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_SOURCES_SHA256 = "88e7d2760502716c0120058a721ce33c9f304c6865feb49a652b349e683180e8"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129116, 243119),
-    "bin_scatter": (95993, 166646),
-    "tile_count": (13142, 2296),
-    "tile_scatter": (26691, 106076),
-    "cell_sort": (35349, 42134),
-    "blend": (318290, 196130),
-    "backward_prologue": (50, 265163),
-    "backward_tiles": (426348, 121587),
-    "backward_points": (297327, 234503),
+    "project_bin": (129115, 243748),
+    "bin_scatter": (95998, 167080),
+    "tile_count": (13143, 2296),
+    "tile_scatter": (26681, 106180),
+    "cell_sort": (36176, 42128),
+    "blend": (318137, 196154),
+    "backward_prologue": (50, 265178),
+    "backward_tiles": (425839, 121584),
+    "backward_points": (297411, 234503),
     "adam_fused": (383789, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
