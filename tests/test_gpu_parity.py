@@ -366,7 +366,7 @@ def test_index_outside_the_descriptor_table_is_left_out_and_reported(oracle):
 
 def test_tight_cluster_long_lists_and_split_tiles(oracle):
     """Thousands of points on a handful of pixels: lists far longer than the segment length of the long-list
-    reduction (1024 / 512 keys) and tiles with more bin entries than a slice (8192), with exact depth ties."""
+    reduction (512 / 256 keys) and tiles with more bin entries than a slice (8192), with exact depth ties."""
     sc = scenes.tiny(n=30000, w=96, h=64, f=80.0, num_layers=4, list_depth=16, seed=91, radius=(0.004, 0.2))
     rng = np.random.default_rng(3)
     sc.position[:, :3] = (rng.normal(0, 0.004, (30000, 3)) + np.array([0.05, -0.02, 0.0])).astype(np.float32)

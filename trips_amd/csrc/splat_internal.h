@@ -125,8 +125,8 @@ constexpr int kMaxBins    = 15360;  // one LDS counter per tile in the binning k
 constexpr int kSliceEntries = 8192;
 // A pixel list longer than kLongList keys is cut into segments of kLongSegment keys; a pass of its own keeps the 16
 // smallest keys of every segment (a 16-lane row each), and the blend kernel then sorts those instead of the list.
-constexpr int kLongList    = 1024;
-constexpr int kLongSegment = 512;
+constexpr int kLongList    = 512;
+constexpr int kLongSegment = 256;
 constexpr int kStageKeys  = 7168;   // keys of one tile staged in LDS before they are written (56 KB)
 // keys of a cell that can reach a pixel's list (the larger list depth): the forward sorts every cell's list and keeps
 // this many
