@@ -1111,29 +1111,38 @@ __global__ __launch_bounds__(256) void long_list_reduce_kernel(const ForwardPara
 // Every cell's list in ascending order, in place; of a list longer than kCellKeep its kCellKeep smallest keys, at its
 // start. A workgroup takes 64 consecutive cells (their lists follow each other in the key array); the sixteen
 // workgroups of a tile run on the XCD that blends the tile. The first wavefront sorts the lists of up to kLaneSortMax
-// keys, one cell per lane, with a network; the longer lists are dealt to the sixteen 16-lane rows of the workgroup's
-// four wavefronts, which stream them (a wavefront that kept all 64 cells to itself walked up to 64 long lists one
-// after the other, four at a time: in a crowded tile that chain of memory round trips was the kernel's duration).
+// keys, one cell per lane, with a network; the longer lists are taken, one after the other, by whichever of the
+// sixteen 16-lane rows of the workgroup's four wavefronts is free, and streamed (a wavefront that kept all 64 cells to
+// itself walked up to 64 long lists one after the other, four at a time: in a crowded tile that chain of memory round
+// trips was the kernel's duration). The other three wavefronts start on the long lists while the first sorts the
+// short ones.
 __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
 {
     __shared__ int s_start[64], s_rd[64];
     __shared__ unsigned char s_long[64];  // lanes of the cells with a longer list
-    __shared__ int s_num_long;
+    __shared__ int s_num_long, s_next;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int NB   = p.geom.bin_off[p.num_layers];
     const long long lblock = xcd_tile_block(blockIdx.x, 16);
     if (lblock >= (long long)NB * 16) return;
+    int4 info = make_int4(0, 0, 0, 0);
     if (wave == 0)
     {
-        const int cell  = (int)lblock * 64 + lane;
-        const int4 info = cell_info(p, cell);
-        const int rd    = info.y;
-        u64* const base = cell_keys(p, info.x);
+        const int cell = (int)lblock * 64 + lane;
+        info           = cell_info(p, cell);
+        const int rd   = info.y;
         const u64 longer = __ballot(rd > kLaneSortMax);
         s_start[lane] = info.x, s_rd[lane] = rd;
         if (rd > kLaneSortMax) s_long[__popcll(longer & ((1ull << lane) - 1ull))] = (unsigned char)lane;
-        if (lane == 0) s_num_long = (int)__popcll(longer);
-        // ---- up to kLaneSortMax keys: one cell per lane ----
+        if (lane == 0) s_num_long = (int)__popcll(longer), s_next = 0;
+    }
+    __syncthreads();
+    // ---- up to kLaneSortMax keys: one cell per lane of the first wavefront, while the other wavefronts start on the
+    // longer lists ----
+    if (wave == 0)
+    {
+        const int rd    = info.y;
+        u64* const base = cell_keys(p, info.x);
         const int mine = rd <= kLaneSortMax ? rd : 0;
         const int nmax = wave_max_small<kLaneSortMax>(mine);
         if (nmax > 1)
@@ -1154,17 +1163,23 @@ __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
             }
         }
     }
-    __syncthreads();
-    // ---- longer lists: one cell per 16-lane row, row r of the workgroup takes the lists r, r + 16, ...; the first keys
-    // of a row's next list are requested before it works on this one ----
+    // ---- longer lists: one cell per 16-lane row; a row takes the next list that nobody has taken yet (the first
+    // wavefront's rows join when its short lists are done), and the first keys of a row's next list are requested
+    // before it works on this one ----
     const int num_long = s_num_long;
     if (num_long == 0) return;
-    const int sub = lane & 15, row = wave * 4 + (lane >> 4);
+    const int sub = lane & 15;
     struct Pass
     {
         u64* base;
         int readable;
         RowKeys first;
+    };
+    auto take = [&]()
+    {
+        int index = 0;
+        if (sub == 0) index = atomicAdd(&s_next, 1);
+        return __shfl(index, lane & ~15);
     };
     auto pass_of = [&](int index)
     {
@@ -1177,18 +1192,18 @@ __global__ __launch_bounds__(256) void cell_sort_kernel(const ForwardParams p)
         ps.first       = row_top16_first([&](int i) { return rb[i]; }, ps.readable);
         return ps;
     };
-    // (the rows of a wavefront walk in step: as many passes as the wavefront's first row has lists)
-    const int passes = (num_long - wave * 4 + 15) / 16;
-    if (passes <= 0) return;
-    Pass cur = pass_of(row);
-    for (int j = 0; j < passes; ++j)
+    int index = take();
+    Pass cur  = pass_of(index);
+    // (the rows of a wavefront walk in step: until none of them has a list)
+    while (__ballot(index < num_long) != 0ull)
     {
-        Pass nxt = cur;
-        if (j + 1 < passes) nxt = pass_of(row + 16 * (j + 1));
+        const int next_index = take();
+        Pass nxt             = pass_of(next_index);
         u64* const rb  = cur.base;
         const u64 best = row_top16([&](int i) { return rb[i]; }, cur.readable, cur.first);
         if (sub < min(cur.readable, kCellKeep)) rb[sub] = best;
-        cur = nxt;
+        cur   = nxt;
+        index = next_index;
     }
 }
 
