@@ -620,18 +620,18 @@ __global__ __launch_bounds__(kBinThreads) void bin_scatter_kernel(const ForwardP
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Walks entries [0, n) with the workgroup, four loads of a thread in flight together.
-template <int THREADS, typename T, typename F>
+// Walks entries [0, n) with the workgroup, U loads of a thread in flight together.
+template <int THREADS, int U, typename T, typename F>
 __device__ __forceinline__ void for_entries(const T* __restrict__ entries, int n, F&& f)
 {
-    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * THREADS)
+    for (int i0 = threadIdx.x; i0 < n; i0 += U * THREADS)
     {
-        T e[4];
+        T e[U];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < U; ++j)
             if (i0 + THREADS * j < n) e[j] = entries[i0 + THREADS * j];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < U; ++j)
             if (i0 + THREADS * j < n) f(e[j]);
     }
 }
@@ -696,7 +696,9 @@ __global__ __launch_bounds__(THREADS) void tile_lists_kernel(const ForwardParams
         if (slice < 0) return;  // the slices count for a split tile; any other tile is counted where its keys are placed
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS) s_cnt[i] = 0;
         __syncthreads();
-        for_entries<THREADS>(entries, n, [&](const ET& e) { atomicAdd(&s_cnt[E::cell(e)], 1); });
+        // (sixteen loads of a thread in flight: the slices of a view are few, and the kernel lasts as long as one slice's
+        // round trips to memory, one after the other)
+        for_entries<THREADS, 16>(entries, n, [&](const ET& e) { atomicAdd(&s_cnt[E::cell(e)], 1); });
         __syncthreads();
         for (int i = threadIdx.x; i < kTilePixels; i += THREADS)
         {
