@@ -31,17 +31,17 @@ DEFAULT_POINTS = 6_000_000
 # sources whose digest is PMC_SOURCES_SHA256 (kernel_sources_sha256 below): when the sources have changed since the
 # profile, no traffic figure is reported.
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
-PMC_SOURCES_SHA256 = "3c17a9a1d38c670316fc7bb15f44d723444a0751621e37f6ddea78dd7c717101"
+PMC_SOURCES_SHA256 = "d9c026c0d3e07d77b1959417be03cf789c9f51952ba1a1782b13b9803885a19b"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129116, 242776),
-    "bin_scatter": (95954, 166993),
-    "tile_count": (13142, 2296),
-    "tile_scatter": (26680, 105866),
-    "cell_sort": (35350, 42129),
-    "blend": (318190, 196308),
-    "backward_prologue": (55, 265188),
-    "backward_tiles": (425928, 121560),
-    "backward_points": (297413, 234503),
+    "project_bin": (129115, 243754),
+    "bin_scatter": (95992, 166669),
+    "tile_count": (13152, 2296),
+    "tile_scatter": (26659, 105391),
+    "cell_sort": (35349, 42140),
+    "blend": (318281, 195401),
+    "backward_prologue": (55, 265126),
+    "backward_tiles": (426225, 121577),
+    "backward_points": (297346, 234503),
     "adam_fused": (383789, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
