@@ -349,18 +349,27 @@ __global__ __launch_bounds__(THREADS) void conv_bwd_data_kernel(const BwdDataPar
     constexpr int kItems = kConvPatchH * kConvPatchW * GROUPS;
     for (int item0 = threadIdx.x; item0 < kItems; item0 += 4 * THREADS)
     {
+        // (every load unconditional, at a position clamped into the image, and all four requested before the first is
+        // used: a load under a condition is waited for where the condition ends)
+        uint4 raw[4];
+        bool in[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const int item = min(item0 + THREADS * j, kItems - 1);
+            const int g = item % GROUPS, pp = item / GROUPS;
+            const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
+            const int y = y0 + py - 1, x = x0 + px - 1;
+            in[j]  = y >= 0 && y < p.H && x >= 0 && x < p.W;
+            raw[j] = *reinterpret_cast<const uint4*>(p.dpre + ((size_t)min(max(y, 0), p.H - 1) * p.W + min(max(x, 0), p.W - 1)) * KC + 8 * g);
+        }
         half8 v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
         {
-            const int item = item0 + THREADS * j;
-            const int g = item % GROUPS, pp = item / GROUPS;
-            const int py = pp / kConvPatchW, px = pp - py * kConvPatchW;
-            const int y = y0 + py - 1, x = x0 + px - 1;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[j][i] = _Float16(0.f);
-            if (item < kItems && y >= 0 && y < p.H && x >= 0 && x < p.W)
-                v[j] = *reinterpret_cast<const half8*>(p.dpre + ((size_t)y * p.W + x) * KC + 8 * g);
+            asm volatile("" : "+v"(raw[j].x), "+v"(raw[j].y), "+v"(raw[j].z), "+v"(raw[j].w));
+            if (!in[j]) raw[j] = make_uint4(0u, 0u, 0u, 0u);
+            v[j] = __builtin_bit_cast(half8, raw[j]);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
