@@ -33,15 +33,15 @@ DEFAULT_POINTS = 6_000_000
 PMC_FETCH_SCALE, PMC_WRITE_SCALE = 2.0, 1.0
 PMC_SOURCES_SHA256 = "d9c026c0d3e07d77b1959417be03cf789c9f51952ba1a1782b13b9803885a19b"
 PMC_KIB_DEFAULT_WORKLOAD = {
-    "project_bin": (129115, 243754),
-    "bin_scatter": (95992, 166669),
+    "project_bin": (129117, 244115),
+    "bin_scatter": (96028, 166743),
     "tile_count": (13152, 2296),
-    "tile_scatter": (26659, 105391),
-    "cell_sort": (35349, 42140),
-    "blend": (318281, 195401),
-    "backward_prologue": (55, 265126),
-    "backward_tiles": (426225, 121577),
-    "backward_points": (297346, 234503),
+    "tile_scatter": (26691, 108508),
+    "cell_sort": (35350, 42126),
+    "blend": (317781, 195746),
+    "backward_prologue": (55, 265170),
+    "backward_tiles": (426000, 121572),
+    "backward_points": (297376, 234503),
     "adam_fused": (383789, 498420),
 }
 SPLAT_KERNEL_SOURCES = ("splat_forward.hip", "splat_backward.hip", "misc_kernels.hip", "trips_splat_abi.hip",
